@@ -1,0 +1,343 @@
+// C ABI of libgomlx_hipq.so: argument validation, device selection, dispatch to the kernel
+// families, HIP-graph recording and per-kernel timing.  See include/gomlx_hipq.h for the
+// contract of every entry point and the reference interface it replaces.
+#include "common.hpp"
+
+#include <atomic>
+#include <cstring>
+#include <mutex>
+
+namespace gq {
+
+namespace {
+thread_local char g_error[512] = "";
+std::atomic<int> g_device{-1};
+std::atomic<int> g_cu_count{256};
+std::mutex g_init_mutex;
+}  // namespace
+
+int fail(int status, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    std::vsnprintf(g_error, sizeof g_error, fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+int hip_fail(hipError_t e, const char *what) {
+    if (e == hipErrorOutOfMemory) return fail(GQ_ERR_OOM, "%s: %s", what, hipGetErrorString(e));
+    if (e == hipErrorNoDevice || e == hipErrorInvalidDevice)
+        return fail(GQ_ERR_NO_DEVICE, "%s: %s", what, hipGetErrorString(e));
+    return fail(GQ_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+int use_device() {
+    const int dev = g_device.load(std::memory_order_acquire);
+    if (dev < 0) return fail(GQ_ERR_NO_DEVICE, "gq_init() has not been called (or failed)");
+    int cur = -1;
+    if (hipGetDevice(&cur) != hipSuccess || cur != dev) GQ_HIP(hipSetDevice(dev));
+    return GQ_OK;
+}
+
+int device_cu_count() { return g_cu_count.load(std::memory_order_relaxed); }
+
+ProfileState &profile_state() {
+    thread_local ProfileState ps;
+    return ps;
+}
+
+namespace {
+
+struct TypeInfo { int bpb, vpb; };
+
+bool type_info(int type, TypeInfo &ti) {
+    switch (type) {
+    case GQ_Q4_0: ti = {18, 32}; return true;
+    case GQ_Q8_0: ti = {34, 32}; return true;
+    case GQ_Q4_K: ti = {144, 256}; return true;
+    case GQ_IQ4_NL: ti = {18, 32}; return true;
+    default: return false;
+    }
+}
+
+bool aligned_to(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// Run-time argument checks shared by the dense entry points.
+int check_dense_args(const char *fn, int type, const void *x, int64_t M, int64_t K, const void *W, int64_t N,
+                     const float *bias, int act, const float *y, size_t x_align) {
+    TypeInfo ti;
+    if (!type_info(type, ti)) return fail(GQ_ERR_NOT_IMPLEMENTED, "%s: ggml type %d is not implemented", fn, type);
+    if (M < 0 || N < 0) return fail(GQ_ERR_INVALID, "%s: negative dimension (M=%lld, N=%lld)", fn, (long long)M, (long long)N);
+    if (K <= 0 || K % ti.vpb != 0)
+        return fail(GQ_ERR_INVALID, "%s: K=%lld is not a positive multiple of the block size %d", fn, (long long)K, ti.vpb);
+    if (act < GQ_ACT_NONE || act > GQ_ACT_TANH) return fail(GQ_ERR_INVALID, "%s: unknown activation %d", fn, act);
+    if (M == 0 || N == 0) return GQ_OK;
+    if (!x || !W || !y) return fail(GQ_ERR_INVALID, "%s: null device pointer", fn);
+    if (!aligned_to(x, x_align)) return fail(GQ_ERR_INVALID, "%s: x must be %zu-byte aligned", fn, x_align);
+    if (!aligned_to(W, 16)) return fail(GQ_ERR_INVALID, "%s: weights must be 16-byte aligned", fn);
+    if (!aligned_to(y, 4) || (bias && !aligned_to(bias, 4))) return fail(GQ_ERR_INVALID, "%s: y / bias must be 4-byte aligned", fn);
+    return GQ_OK;
+}
+
+}  // namespace
+}  // namespace gq
+
+using namespace gq;
+
+extern "C" {
+
+int gq_abi_version(void) { return 1; }
+
+int gq_bytes_per_block(int type) {
+    TypeInfo ti;
+    return type_info(type, ti) ? ti.bpb : 0;
+}
+
+int gq_values_per_block(int type) {
+    TypeInfo ti;
+    return type_info(type, ti) ? ti.vpb : 0;
+}
+
+size_t gq_row_bytes(int type, int64_t K) {
+    TypeInfo ti;
+    if (!type_info(type, ti) || K <= 0 || K % ti.vpb != 0) return 0;
+    return (size_t)(K / ti.vpb) * (size_t)ti.bpb;
+}
+
+int gq_qdense_check(int type, int x_dtype, int64_t M, int64_t x_last_dim, int64_t N, int64_t w_row_bytes,
+                    int64_t bias_len, int act, int64_t *K_out) {
+    TypeInfo ti;
+    if (!type_info(type, ti)) return fail(GQ_ERR_NOT_IMPLEMENTED, "FusedQuantizedDense: ggml type %d is not implemented", type);
+    if (x_dtype != GQ_F32 && x_dtype != GQ_BF16)
+        return fail(GQ_ERR_NOT_IMPLEMENTED, "FusedQuantizedDense: activation dtype %d is not implemented", x_dtype);
+    if (M < 0 || N < 0) return fail(GQ_ERR_INVALID, "FusedQuantizedDense: negative dimension");
+    if (w_row_bytes <= 0 || w_row_bytes % ti.bpb != 0)
+        return fail(GQ_ERR_INVALID, "FusedQuantizedDense: weight row of %lld bytes is not a whole number of %d-byte blocks",
+                    (long long)w_row_bytes, ti.bpb);
+    const int64_t K = w_row_bytes / ti.bpb * ti.vpb;
+    if (x_last_dim != K)  // ml/ggml/dense.go:38-41
+        return fail(GQ_ERR_INVALID, "FusedQuantizedDense: x has %lld features but the weights decode to K=%lld",
+                    (long long)x_last_dim, (long long)K);
+    if (bias_len >= 0 && bias_len != N)
+        return fail(GQ_ERR_INVALID, "FusedQuantizedDense: bias has %lld elements, expected N=%lld", (long long)bias_len, (long long)N);
+    if (act < GQ_ACT_NONE || act > GQ_ACT_TANH) return fail(GQ_ERR_INVALID, "FusedQuantizedDense: unknown activation %d", act);
+    if (K_out) *K_out = K;
+    return GQ_OK;
+}
+
+int gq_device_count(int *count) {
+    if (!count) return fail(GQ_ERR_INVALID, "gq_device_count: null argument");
+    int n = 0;
+    const hipError_t e = hipGetDeviceCount(&n);
+    if (e == hipErrorNoDevice) { *count = 0; return GQ_OK; }
+    if (e != hipSuccess) { *count = 0; return hip_fail(e, "hipGetDeviceCount"); }
+    *count = n;
+    return GQ_OK;
+}
+
+int gq_init(int device) {
+    std::lock_guard<std::mutex> lock(g_init_mutex);
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n == 0) return fail(GQ_ERR_NO_DEVICE, "gq_init: no HIP device (%s)", hipGetErrorString(e));
+    if (device < 0 || device >= n) return fail(GQ_ERR_NO_DEVICE, "gq_init: device %d out of range (found %d)", device, n);
+    const int cur = g_device.load();
+    if (cur >= 0 && cur != device)
+        return fail(GQ_ERR_INVALID, "gq_init: already initialised on device %d (one device per process)", cur);
+    hipDeviceProp_t prop;
+    GQ_HIP(hipGetDeviceProperties(&prop, device));
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(GQ_ERR_NO_DEVICE, "gq_init: device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName);
+    GQ_HIP(hipSetDevice(device));
+    g_cu_count.store(prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256);
+    g_device.store(device, std::memory_order_release);
+    return GQ_OK;
+}
+
+int gq_device_name(char *buf, size_t n) {
+    if (!buf || n == 0) return fail(GQ_ERR_INVALID, "gq_device_name: null buffer");
+    if (int rc = use_device()) return rc;
+    hipDeviceProp_t prop;
+    GQ_HIP(hipGetDeviceProperties(&prop, g_device.load()));
+    std::snprintf(buf, n, "%s (%s, %d CUs)", prop.name, prop.gcnArchName, prop.multiProcessorCount);
+    return GQ_OK;
+}
+
+int gq_malloc(void **dptr, size_t bytes) {
+    if (!dptr) return fail(GQ_ERR_INVALID, "gq_malloc: null argument");
+    *dptr = nullptr;
+    if (int rc = use_device()) return rc;
+    if (bytes == 0) return GQ_OK;
+    GQ_HIP(hipMalloc(dptr, bytes));
+    return GQ_OK;
+}
+
+int gq_free(void *dptr) {
+    if (!dptr) return GQ_OK;
+    if (int rc = use_device()) return rc;
+    GQ_HIP(hipFree(dptr));
+    return GQ_OK;
+}
+
+int gq_h2d(void *d, const void *h, size_t bytes, void *stream) {
+    if (bytes == 0) return GQ_OK;
+    if (!d || !h) return fail(GQ_ERR_INVALID, "gq_h2d: null pointer");
+    if (int rc = use_device()) return rc;
+    GQ_HIP(hipMemcpyAsync(d, h, bytes, hipMemcpyHostToDevice, (hipStream_t)stream));
+    GQ_HIP(hipStreamSynchronize((hipStream_t)stream));
+    return GQ_OK;
+}
+
+int gq_d2h(void *h, const void *d, size_t bytes, void *stream) {
+    if (bytes == 0) return GQ_OK;
+    if (!d || !h) return fail(GQ_ERR_INVALID, "gq_d2h: null pointer");
+    if (int rc = use_device()) return rc;
+    GQ_HIP(hipMemcpyAsync(h, d, bytes, hipMemcpyDeviceToHost, (hipStream_t)stream));
+    GQ_HIP(hipStreamSynchronize((hipStream_t)stream));
+    return GQ_OK;
+}
+
+int gq_stream_create(void **stream) {
+    if (!stream) return fail(GQ_ERR_INVALID, "gq_stream_create: null argument");
+    if (int rc = use_device()) return rc;
+    hipStream_t s;
+    GQ_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *stream = s;
+    return GQ_OK;
+}
+
+int gq_stream_destroy(void *stream) {
+    if (!stream) return GQ_OK;
+    if (int rc = use_device()) return rc;
+    GQ_HIP(hipStreamDestroy((hipStream_t)stream));
+    return GQ_OK;
+}
+
+int gq_sync(void *stream) {
+    if (int rc = use_device()) return rc;
+    GQ_HIP(hipStreamSynchronize((hipStream_t)stream));
+    return GQ_OK;
+}
+
+int gq_dequantize(int type, const void *dW, int64_t N, int64_t K, float *dOut, void *stream) {
+    TypeInfo ti;
+    if (!type_info(type, ti)) return fail(GQ_ERR_NOT_IMPLEMENTED, "gq_dequantize: ggml type %d is not implemented", type);
+    if (N < 0) return fail(GQ_ERR_INVALID, "gq_dequantize: negative N");
+    if (K <= 0 || K % ti.vpb != 0)
+        return fail(GQ_ERR_INVALID, "gq_dequantize: K=%lld is not a positive multiple of the block size %d", (long long)K, ti.vpb);
+    if (N == 0) return GQ_OK;
+    if (!dW || !dOut) return fail(GQ_ERR_INVALID, "gq_dequantize: null device pointer");
+    if (!aligned_to(dW, 16) || !aligned_to(dOut, 16))
+        return fail(GQ_ERR_INVALID, "gq_dequantize: weights and output must be 16-byte aligned");
+    if (int rc = use_device()) return rc;
+    return launch_dequantize(type, (const uint8_t *)dW, N, K, dOut, (hipStream_t)stream);
+}
+
+int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *dW, int64_t N, const float *dBias,
+                  int act, float *dY, void *stream) {
+    if (int rc = check_dense_args("gq_qdense_f32", type, dX, M, K, dW, N, dBias, act, dY, 4)) return rc;
+    if (M == 0 || N == 0) return GQ_OK;
+    if (int rc = use_device()) return rc;
+    // Up to four activation rows: one bandwidth-bound pass over W per row, fp32 throughout.
+    // More rows: W is read once per 128-row tile and contracted on the matrix cores.
+    if (M <= 4) return launch_gemv(type, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
+    return launch_gemm(type, false, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
+}
+
+int gq_qdense_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, const void *dW, int64_t N,
+                   const float *dBias, int act, float *dY, void *stream) {
+    if (int rc = check_dense_args("gq_qdense_bf16", type, dX, M, K, dW, N, dBias, act, dY, 2)) return rc;
+    if (M == 0 || N == 0) return GQ_OK;
+    if (int rc = use_device()) return rc;
+    return launch_gemm(type, true, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
+}
+
+int gq_embedding_lookup(int type, const void *dTable, int64_t vocab, int64_t K, const int32_t *dIndices,
+                        int64_t count, float *dOut, int32_t *dErrFlag, void *stream) {
+    TypeInfo ti;
+    if (!type_info(type, ti)) return fail(GQ_ERR_NOT_IMPLEMENTED, "gq_embedding_lookup: ggml type %d is not implemented", type);
+    if (vocab < 0 || count < 0) return fail(GQ_ERR_INVALID, "gq_embedding_lookup: negative size");
+    if (K <= 0 || K % ti.vpb != 0)
+        return fail(GQ_ERR_INVALID, "gq_embedding_lookup: K=%lld is not a positive multiple of the block size %d", (long long)K, ti.vpb);
+    if (count == 0) return GQ_OK;
+    if (vocab == 0) return fail(GQ_ERR_INVALID, "gq_embedding_lookup: empty table with %lld indices", (long long)count);
+    if (!dTable || !dIndices || !dOut) return fail(GQ_ERR_INVALID, "gq_embedding_lookup: null device pointer");
+    if (!aligned_to(dTable, 16) || !aligned_to(dOut, 16) || !aligned_to(dIndices, 4))
+        return fail(GQ_ERR_INVALID, "gq_embedding_lookup: table and output must be 16-byte aligned");
+    if (int rc = use_device()) return rc;
+    return launch_embedding_lookup(type, (const uint8_t *)dTable, vocab, K, dIndices, count, dOut, dErrFlag,
+                                   (hipStream_t)stream);
+}
+
+int gq_graph_begin(void *stream) {
+    if (!stream) return fail(GQ_ERR_INVALID, "gq_graph_begin: recording needs an explicit stream");
+    if (profile_state().active) return fail(GQ_ERR_INVALID, "gq_graph_begin: kernel timing is active on this thread");
+    if (int rc = use_device()) return rc;
+    GQ_HIP(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
+    return GQ_OK;
+}
+
+int gq_graph_end(void *stream, void **graph_exec) {
+    if (!stream || !graph_exec) return fail(GQ_ERR_INVALID, "gq_graph_end: null argument");
+    *graph_exec = nullptr;
+    if (int rc = use_device()) return rc;
+    hipGraph_t graph = nullptr;
+    GQ_HIP(hipStreamEndCapture((hipStream_t)stream, &graph));
+    hipGraphExec_t exec = nullptr;
+    const hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (e != hipSuccess) return hip_fail(e, "hipGraphInstantiate");
+    *graph_exec = exec;
+    return GQ_OK;
+}
+
+int gq_graph_launch(void *graph_exec, void *stream) {
+    if (!graph_exec) return fail(GQ_ERR_INVALID, "gq_graph_launch: null graph");
+    if (int rc = use_device()) return rc;
+    GQ_HIP(hipGraphLaunch((hipGraphExec_t)graph_exec, (hipStream_t)stream));
+    return GQ_OK;
+}
+
+int gq_graph_destroy(void *graph_exec) {
+    if (!graph_exec) return GQ_OK;
+    if (int rc = use_device()) return rc;
+    GQ_HIP(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
+    return GQ_OK;
+}
+
+int gq_profile_begin(void) {
+    ProfileState &ps = profile_state();
+    if (ps.active) return fail(GQ_ERR_INVALID, "gq_profile_begin: already active on this thread");
+    if (int rc = use_device()) return rc;
+    ps.active = true;
+    ps.events.clear();
+    return GQ_OK;
+}
+
+int gq_profile_end(int *launches, double *total_us) {
+    ProfileState &ps = profile_state();
+    if (!ps.active) return fail(GQ_ERR_INVALID, "gq_profile_end: timing is not active on this thread");
+    ps.active = false;
+    int rc = use_device();
+    double total = 0.0;
+    int n = 0;
+    for (size_t i = 0; i + 1 < ps.events.size(); i += 2) {
+        if (rc == GQ_OK) {
+            float ms = 0.f;
+            hipError_t e = hipEventSynchronize(ps.events[i + 1]);
+            if (e == hipSuccess) e = hipEventElapsedTime(&ms, ps.events[i], ps.events[i + 1]);
+            if (e != hipSuccess) rc = hip_fail(e, "hipEventElapsedTime");
+            else { total += (double)ms * 1000.0; n++; }
+        }
+        (void)hipEventDestroy(ps.events[i]);
+        (void)hipEventDestroy(ps.events[i + 1]);
+    }
+    ps.events.clear();
+    if (launches) *launches = n;
+    if (total_us) *total_us = total;
+    return rc;
+}
+
+const char *gq_last_error(void) { return g_error; }
+
+}  // extern "C"

@@ -1,0 +1,177 @@
+// Device-side decoding of GGML blocks (Q8_0, Q4_0, IQ4_NL, Q4_K) for gfx950.
+//
+// Arithmetic follows ml/ggml/dequant.go:58-136 of the reference (Q8_0, Q4_0, IQ4_NL) and
+// the public GGML block_q4_K layout (Q4_K): every fp32 multiply / subtract is a separate,
+// individually rounded operation.  This translation unit family is compiled with
+// -ffp-contract=off, so `a * b - c` below never becomes a fused multiply-add.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace gq {
+
+constexpr int kQ4_0 = 2, kQ8_0 = 8, kQ4_K = 12, kIQ4_NL = 20;
+constexpr int kActNone = 0, kActGelu = 1, kActRelu = 2, kActSilu = 3, kActHardSwish = 4, kActTanh = 5;
+
+template <int T> struct Geom;
+template <> struct Geom<kQ4_0> { static constexpr int bpb = 18, vpb = 32; };
+template <> struct Geom<kQ8_0> { static constexpr int bpb = 34, vpb = 32; };
+template <> struct Geom<kIQ4_NL> { static constexpr int bpb = 18, vpb = 32; };
+template <> struct Geom<kQ4_K> { static constexpr int bpb = 144, vpb = 256; };
+
+// 16 bytes that are only guaranteed to be 2-byte aligned (Q4_0 / Q8_0 payloads start two
+// bytes into an 18- or 34-byte block).  gfx950 global loads accept unaligned addresses, so
+// this still compiles to a single global_load_dwordx4.
+struct __attribute__((packed, aligned(2))) u128_a2 { uint32_t v[4]; };
+
+__device__ __forceinline__ float half_bits_to_float(uint32_t h) {
+    const uint16_t b = (uint16_t)h;
+    _Float16 v;
+    __builtin_memcpy(&v, &b, 2);
+    return (float)v;  // v_cvt_f32_f16: exact, subnormals included
+}
+
+__device__ __forceinline__ uint32_t load_u16(const uint8_t *p) {
+    return *reinterpret_cast<const uint16_t *>(p);
+}
+
+// Byte j of v as an fp32 number (v_cvt_f32_ubyteN).  Inline asm keeps the compiler from
+// re-deriving the byte with a separate bit-field extract.
+__device__ __forceinline__ float ubyte0(uint32_t v) { float f; asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(v)); return f; }
+__device__ __forceinline__ float ubyte1(uint32_t v) { float f; asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(v)); return f; }
+__device__ __forceinline__ float ubyte2(uint32_t v) { float f; asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(v)); return f; }
+__device__ __forceinline__ float ubyte3(uint32_t v) { float f; asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(v)); return f; }
+
+// Public GGML IQ4_NL code book (compute.IQ4NLLookupTable, ml/ggml/dequant.go:130).
+__device__ __forceinline__ float iq4nl_value(uint32_t nib) {
+    // Packed as int8 in four dwords; selected with a byte permute instead of a memory table.
+    const uint32_t t0 = 0xBFAD9881u;  // -127 -104 -83 -65
+    const uint32_t t1 = 0xF6EADDCFu;  // -49 -35 -22 -10
+    const uint32_t t2 = 0x26190D01u;  // 1 13 25 38
+    const uint32_t t3 = 0x71594535u;  // 53 69 89 113
+    const uint32_t lo = (nib & 4) ? t1 : t0;
+    const uint32_t hi = (nib & 4) ? t3 : t2;
+    const uint32_t w = (nib & 8) ? hi : lo;
+    const int32_t b = (int32_t)(int8_t)(w >> ((nib & 3) * 8));
+    return (float)b;
+}
+
+// The 6-bit (scale, min) pair of sub-block j (0..7) of a Q4_K super-block whose twelve
+// packed bytes are given as three little-endian dwords a = s[0..3], b = s[4..7], c = s[8..11].
+__device__ __forceinline__ void q4k_scale_min(uint32_t a, uint32_t b, uint32_t c, int j, uint32_t &sc, uint32_t &mn) {
+    const int sh = (j & 3) * 8;
+    const uint32_t aj = a >> sh, bj = b >> sh, cj = c >> sh;
+    if (j < 4) {
+        sc = aj & 63u;
+        mn = bj & 63u;
+    } else {
+        sc = (cj & 0x0Fu) | (((aj >> 6) & 3u) << 4);
+        mn = ((cj >> 4) & 0x0Fu) | (((bj >> 6) & 3u) << 4);
+    }
+}
+
+// Exact dequantisation of 16 consecutive values of one weight row:
+// out[0..15] = w[16*i .. 16*i+15].  Bit-exact with the reference arithmetic.
+template <int T>
+__device__ __forceinline__ void dequant16(const uint8_t *__restrict__ row, int64_t i, float *out);
+
+template <>
+__device__ __forceinline__ void dequant16<kQ8_0>(const uint8_t *__restrict__ row, int64_t i, float *out) {
+    const uint8_t *blk = row + (i >> 1) * 34;
+    const float d = half_bits_to_float(load_u16(blk));
+    const u128_a2 q = *reinterpret_cast<const u128_a2 *>(blk + 2 + 16 * (i & 1));
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int32_t v = (int32_t)(int8_t)(q.v[w] >> (8 * j));
+            out[4 * w + j] = (float)v * d;  // ml/ggml/dequant.go:74
+        }
+    }
+}
+
+template <>
+__device__ __forceinline__ void dequant16<kQ4_0>(const uint8_t *__restrict__ row, int64_t i, float *out) {
+    const uint8_t *blk = row + (i >> 1) * 18;
+    const float d = half_bits_to_float(load_u16(blk));
+    const u128_a2 q = *reinterpret_cast<const u128_a2 *>(blk + 2);
+    const int sh = (int)(i & 1) * 4;  // values 0..15: low nibbles, 16..31: high nibbles
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t nib = (q.v[w] >> (8 * j + sh)) & 0x0Fu;
+            out[4 * w + j] = ((float)nib - 8.0f) * d;  // ml/ggml/dequant.go:108-112
+        }
+    }
+}
+
+template <>
+__device__ __forceinline__ void dequant16<kIQ4_NL>(const uint8_t *__restrict__ row, int64_t i, float *out) {
+    const uint8_t *blk = row + (i >> 1) * 18;
+    const float d = half_bits_to_float(load_u16(blk));
+    const u128_a2 q = *reinterpret_cast<const u128_a2 *>(blk + 2);
+    const int sh = (int)(i & 1) * 4;
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t nib = (q.v[w] >> (8 * j + sh)) & 0x0Fu;
+            out[4 * w + j] = iq4nl_value(nib) * d;  // ml/ggml/dequant.go:130-133
+        }
+    }
+}
+
+template <>
+__device__ __forceinline__ void dequant16<kQ4_K>(const uint8_t *__restrict__ row, int64_t i, float *out) {
+    const uint8_t *sb = row + (i >> 4) * 144;  // 16 runs of 16 values per super-block
+    const int idx = (int)(i & 15);
+    const int g = idx >> 2;         // group of 64 values sharing 32 code bytes
+    const int h = (idx >> 1) & 1;   // 0: low nibbles (sub-block 2g), 1: high nibbles (2g+1)
+    const int p = idx & 1;          // which 16 of the 32 code bytes
+    const uint4 hd = *reinterpret_cast<const uint4 *>(sb);
+    const float d = half_bits_to_float(hd.x & 0xFFFFu);
+    const float dmin = half_bits_to_float(hd.x >> 16);
+    uint32_t sc, mn;
+    q4k_scale_min(hd.y, hd.z, hd.w, 2 * g + h, sc, mn);
+    const float ds = d * (float)sc;
+    const float dm = dmin * (float)mn;
+    const uint4 q = *reinterpret_cast<const uint4 *>(sb + 16 + 32 * g + 16 * p);
+    const uint32_t qq[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t nib = (qq[w] >> (8 * j + 4 * h)) & 0x0Fu;
+            out[4 * w + j] = ds * (float)nib - dm;
+        }
+    }
+}
+
+// Epilogue of the fused op: activation.Apply formulas
+// (ml/layers/activation/activation.go:161,195,222-243,274-286); Gelu is the exact erf form.
+__device__ __forceinline__ float apply_act(int act, float v) {
+    switch (act) {
+    case kActRelu: return fmaxf(v, 0.0f);
+    case kActSilu: return v / (1.0f + __expf(-v));
+    case kActHardSwish: return v * fminf(fmaxf(v * (1.0f / 6.0f) + 0.5f, 0.0f), 1.0f);
+    case kActTanh: return tanhf(v);
+    case kActGelu: return v * 0.5f * (1.0f + erff(v * 0.70710678118654752f));
+    default: return v;
+    }
+}
+
+// Sum over the 64 lanes of a wavefront; every lane receives the total.  The first four
+// steps are DPP moves inside a row of 16 lanes, the last two cross rows.
+__device__ __forceinline__ float wave_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // row_half_mirror
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));  // row_mirror
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    return v;
+}
+
+}  // namespace gq

@@ -1,0 +1,69 @@
+// Host-side plumbing shared by the translation units of libgomlx_hipq.so: status codes,
+// thread-local error text, the active device, and the single kernel-launch path (which is
+// where per-kernel event timing hooks in).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <vector>
+
+#include "../../include/gomlx_hipq.h"
+
+namespace gq {
+
+// ---- error text -----------------------------------------------------------------------
+int fail(int status, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+int hip_fail(hipError_t e, const char *what);
+
+#define GQ_HIP(call)                                          \
+    do {                                                      \
+        hipError_t e__ = (call);                              \
+        if (e__ != hipSuccess) return ::gq::hip_fail(e__, #call); \
+    } while (0)
+
+// ---- device ---------------------------------------------------------------------------
+// Makes the device chosen by gq_init() current on this thread; fails if gq_init() has not
+// succeeded yet.
+int use_device();
+int device_cu_count();
+
+// ---- launch ---------------------------------------------------------------------------
+struct ProfileState {
+    bool active = false;
+    std::vector<hipEvent_t> events;  // start/stop pairs of the launches made while active
+};
+ProfileState &profile_state();
+
+// Launches `kernel`; while profiling is active on this thread the launch carries a
+// start/stop event pair whose timestamps are the kernel's own begin and end.
+template <typename... KArgs, typename... Args>
+int launch(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t shmem, hipStream_t stream, Args... args) {
+    ProfileState &ps = profile_state();
+    if (ps.active) {
+        hipEvent_t a, b;
+        GQ_HIP(hipEventCreate(&a));
+        GQ_HIP(hipEventCreate(&b));
+        hipExtLaunchKernelGGL(kernel, grid, block, (unsigned)shmem, stream, a, b, 0, static_cast<KArgs>(args)...);
+        ps.events.push_back(a);
+        ps.events.push_back(b);
+    } else {
+        hipLaunchKernelGGL(kernel, grid, block, (unsigned)shmem, stream, static_cast<KArgs>(args)...);
+    }
+    GQ_HIP(hipGetLastError());
+    return GQ_OK;
+}
+
+// ---- kernel families (one translation unit each) -----------------------------------------
+int launch_dequantize(int type, const uint8_t *W, int64_t N, int64_t K, float *out, hipStream_t s);
+int launch_embedding_lookup(int type, const uint8_t *table, int64_t vocab, int64_t K, const int32_t *idx,
+                            int64_t count, float *out, int32_t *err_flag, hipStream_t s);
+int launch_gemv(int type, const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N,
+                const float *bias, int act, float *y, hipStream_t s);
+int launch_gemm(int type, bool x_is_bf16, const void *x, int64_t M, int64_t K, const uint8_t *W, int64_t N,
+                const float *bias, int act, float *y, hipStream_t s);
+
+}  // namespace gq

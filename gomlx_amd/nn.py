@@ -1,0 +1,167 @@
+"""Host-side mirror of the reference's quantized-Dense operator interface over torch
+device tensors.  Names, argument meaning and error behaviour follow
+
+* ``nn.QuantizedDense``   ml/nn/quantized_dense.go:31-57
+* ``nn.QuantizedGather``  ml/nn/quantized_gather.go:30-43
+* ``ggml.Dequantize``     ml/ggml/dequant.go:39-54
+* ``graph.Quantization``  core/graph/fused_ops.go:18-48
+* ``activation.Type.ToBackend``  ml/layers/activation/activation.go:58-75
+
+torch only supplies device memory and the current stream; all arithmetic runs in
+libgomlx_hipq.so.  There is no CPU path: tensors must live on the GPU.
+"""
+from __future__ import annotations
+
+import enum
+from dataclasses import dataclass
+
+import torch
+
+from . import _lib, ggml
+
+
+class QuantizationScheme(enum.IntEnum):
+    """compute.QuantizationScheme; only GGML is on this path."""
+    LINEAR = 0
+    NF4 = 1
+    GGML = 2
+
+
+class Activation(enum.IntEnum):
+    """activation.Type of the reference (ml/layers/activation/activation.go:30-54)."""
+    NONE = 0
+    RELU = 1
+    SIGMOID = 2
+    HARD_SIGMOID = 3
+    LEAKY_RELU = 4
+    SELU = 5
+    SWISH = 6
+    HARD_SWISH = 7
+    SILU = 8
+    TANH = 9
+    GELU = 10
+    GELU_APPROX = 11
+    SWIGLU = 12
+
+    def to_backend(self) -> int:
+        """activation.Type.ToBackend: types without a backend enum map to NONE, and both
+        GELU flavours map to the single backend Gelu (activation.go:58-75)."""
+        return {
+            Activation.NONE: 0, Activation.GELU: 1, Activation.GELU_APPROX: 1, Activation.RELU: 2,
+            Activation.SWISH: 3, Activation.SILU: 3, Activation.HARD_SWISH: 4, Activation.TANH: 5,
+        }.get(self, 0)
+
+
+@dataclass
+class Quantization:
+    """graph.Quantization (core/graph/fused_ops.go:18-48).  For GGML only scheme and
+    ggml_type are used; the scales live inside the blocks."""
+    scheme: QuantizationScheme = QuantizationScheme.GGML
+    ggml_type: int = ggml.Q8_0
+    scale: object = None
+    zero_point: object = None
+    block_axis: int = 0
+    block_size: int = 0
+
+
+def _stream_ptr(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _require_cuda(name: str, t: torch.Tensor) -> None:
+    if not t.is_cuda:
+        raise ValueError(f"{name} must be a GPU tensor: this backend has no CPU path")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+
+
+def _weights_2d(weights: torch.Tensor) -> None:
+    if weights.dtype != torch.uint8 or weights.dim() != 2:
+        raise ValueError("weights must be a Uint8 [N, bytesPerRow] tensor of native GGML blocks")
+
+
+def dequantize(weights: torch.Tensor, ggml_type: int) -> torch.Tensor:
+    """ggml.Dequantize: [N, bytesPerRow] uint8 -> [N, K] float32, bit-exact."""
+    _require_cuda("weights", weights)
+    _weights_2d(weights)
+    _lib.init(weights.device.index or 0)
+    N, rb = weights.shape
+    bpb = ggml.bytes_per_block(ggml_type)
+    if rb % bpb:
+        raise ValueError(f"row of {rb} bytes is not a whole number of {bpb}-byte blocks")
+    K = rb // bpb * ggml.values_per_block(ggml_type)
+    out = torch.empty((N, K), dtype=torch.float32, device=weights.device)
+    _lib.check(_lib.lib().gq_dequantize(ggml_type, weights.data_ptr(), N, K, out.data_ptr(), _stream_ptr(weights)))
+    return out
+
+
+def quantized_dense(x: torch.Tensor, weights: torch.Tensor, quant: Quantization, bias: torch.Tensor | None = None,
+                    *optional_activation: Activation) -> torch.Tensor:
+    """nn.QuantizedDense for the GGML scheme: y = activation(x @ dequant(weights)^T + bias).
+
+    x: [batch..., K] float32 or bfloat16; weights: [N, bytesPerRow] uint8; bias: [N] float32.
+    Returns [batch..., N] float32.
+    """
+    if len(optional_activation) > 1:
+        raise ValueError(f"quantized_dense can only take one optional activation, got {optional_activation}")
+    act = optional_activation[0] if optional_activation else Activation.NONE
+    if quant is None:
+        raise ValueError("quant must not be None")  # core/graph/fused_ops.go:198-200
+    if quant.scheme != QuantizationScheme.GGML:
+        raise _lib.NotImplementedByBackend(_lib.ERR_NOT_IMPLEMENTED,
+                                           f"scheme {quant.scheme.name} is outside this backend (GGML only)")
+    _require_cuda("x", x)
+    _require_cuda("weights", weights)
+    _weights_2d(weights)
+    if x.dtype == torch.float32:
+        xd = _lib.F32
+    elif x.dtype == torch.bfloat16:
+        xd = _lib.BF16
+    else:
+        raise _lib.NotImplementedByBackend(_lib.ERR_NOT_IMPLEMENTED, f"activation dtype {x.dtype} is not implemented")
+    L = _lib.lib()
+    N, rb = weights.shape
+    K_in = x.shape[-1]
+    M = x.numel() // K_in if K_in else 0
+    blen = -1
+    if bias is not None:
+        _require_cuda("bias", bias)
+        if bias.dtype != torch.float32 or bias.dim() != 1:
+            raise ValueError("bias must be a float32 [N] tensor")
+        blen = bias.shape[0]
+    import ctypes
+    K = ctypes.c_int64(0)
+    _lib.check(L.gq_qdense_check(quant.ggml_type, xd, M, K_in, N, rb, blen, act.to_backend(), ctypes.byref(K)))
+    _lib.init(x.device.index or 0)
+    y = torch.empty(x.shape[:-1] + (N,), dtype=torch.float32, device=x.device)
+    fn = L.gq_qdense_f32 if xd == _lib.F32 else L.gq_qdense_bf16
+    _lib.check(fn(quant.ggml_type, x.data_ptr(), M, K.value, weights.data_ptr(), N,
+                  None if bias is None else bias.data_ptr(), act.to_backend(), y.data_ptr(), _stream_ptr(x)))
+    return y
+
+
+def quantized_gather(table: torch.Tensor, indices: torch.Tensor, quant: Quantization) -> torch.Tensor:
+    """nn.QuantizedGather: indices [batch..., 1] (int32) -> [batch..., K] float32 rows of the
+    dequantised table.  An out-of-range index raises IndexError."""
+    if quant.scheme != QuantizationScheme.GGML:
+        raise ValueError("quantized_gather: only the GGML scheme is supported")  # quantized_gather.go:31-33
+    _require_cuda("table", table)
+    _require_cuda("indices", indices)
+    _weights_2d(table)
+    if indices.dim() < 1 or indices.shape[-1] != 1:
+        raise ValueError("indices must have last dimension 1")
+    idx = indices.to(torch.int32).contiguous()
+    _lib.init(table.device.index or 0)
+    vocab, rb = table.shape
+    bpb = ggml.bytes_per_block(quant.ggml_type)
+    if rb % bpb:
+        raise ValueError(f"row of {rb} bytes is not a whole number of {bpb}-byte blocks")
+    K = rb // bpb * ggml.values_per_block(quant.ggml_type)
+    count = idx.numel()
+    out = torch.empty(tuple(indices.shape[:-1]) + (K,), dtype=torch.float32, device=table.device)
+    flag = torch.zeros(1, dtype=torch.int32, device=table.device)
+    _lib.check(_lib.lib().gq_embedding_lookup(quant.ggml_type, table.data_ptr(), vocab, K, idx.data_ptr(), count,
+                                              out.data_ptr(), flag.data_ptr(), _stream_ptr(table)))
+    if count and int(flag.item()):
+        raise IndexError("quantized_gather: index out of range")
+    return out

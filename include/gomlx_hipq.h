@@ -1,0 +1,134 @@
+/*
+ * gomlx_hipq - MI355X (gfx950) implementation of GoMLX's quantized Dense hot path.
+ *
+ * C ABI of libgomlx_hipq.so.  A Go backend reaches it through cgo; every entry point
+ * below names the interface of the reference (gomlx/gomlx, file:line) it stands in for.
+ *
+ * Conventions
+ *   - Every function returns a gq_status (0 = success) unless stated otherwise; nothing
+ *     throws or aborts across this boundary.  gq_last_error() returns the message of the
+ *     last failure on the calling thread.
+ *   - GQ_ERR_NOT_IMPLEMENTED is the analogue of compute.ErrNotImplemented: the caller may
+ *     fall back to the decomposed graph (core/graph/fused_ops.go:357-363).  Any other
+ *     error is a hard failure (core/graph/fused_ops.go:365).
+ *   - All pointers named d* are device pointers owned by the caller; the library keeps no
+ *     reference to them after the call returns (launches are asynchronous on `stream`, so
+ *     the memory must stay valid until the stream has been synchronised).
+ *   - stream == NULL selects the null stream of the active device.  Otherwise it is a
+ *     hipStream_t.  The active device is the one given to gq_init(); every entry point
+ *     makes it current on the calling thread itself (cgo may move a goroutine to another
+ *     OS thread between calls).
+ *   - Weights are native GGML blocks, row-major [N, gq_row_bytes(type, K)] bytes: one row
+ *     per output feature, blocks running along K (ml/ggml/dense.go:19).
+ *   - Activations x are row-major [M, K]; outputs y are row-major [M, N] fp32.
+ */
+#ifndef GOMLX_HIPQ_H
+#define GOMLX_HIPQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    GQ_OK = 0,
+    GQ_ERR_INVALID = 1,         /* malformed arguments: hard error */
+    GQ_ERR_NOT_IMPLEMENTED = 2, /* valid but unsupported: caller may fall back */
+    GQ_ERR_HIP = 3,             /* a HIP runtime call failed */
+    GQ_ERR_NO_DEVICE = 4,       /* no usable gfx950 device / gq_init not called */
+    GQ_ERR_OOM = 5
+} gq_status;
+
+/* compute.GGMLQuantType (core/graph/fused_ops.go:46-47); numeric values follow the public
+ * GGML type ids. */
+typedef enum { GQ_Q4_0 = 2, GQ_Q8_0 = 8, GQ_Q4_K = 12, GQ_IQ4_NL = 20 } gq_type;
+
+/* compute.ActivationType as produced by activation.Type.ToBackend
+ * (ml/layers/activation/activation.go:58-75). */
+typedef enum {
+    GQ_ACT_NONE = 0, GQ_ACT_GELU = 1, GQ_ACT_RELU = 2, GQ_ACT_SILU = 3,
+    GQ_ACT_HARDSWISH = 4, GQ_ACT_TANH = 5
+} gq_act;
+
+/* Activation element types accepted by the dense entry points. */
+typedef enum { GQ_F32 = 0, GQ_BF16 = 1 } gq_dtype;
+
+/* ABI version: bumped on any incompatible change. */
+int gq_abi_version(void);
+
+/* ---- geometry: GGMLQuantType.BytesPerBlock / ValuesPerBlock (ml/ggml/dequant.go:41,
+ * ml/ggml/gather.go:24-25).  Pure host functions; return 0 for an unknown type. ---- */
+int gq_bytes_per_block(int type);
+int gq_values_per_block(int type);
+/* (K / valuesPerBlock) * bytesPerBlock; 0 if the type is unknown or K is not a positive
+ * whole number of blocks. */
+size_t gq_row_bytes(int type, int64_t K);
+
+/* ---- build-time validation: what Function.FusedQuantizedDense checks when the graph
+ * is built (core/graph/fused_ops.go:195-245) and what Builder.OpShape then reports
+ * (core/graph/fused_ops.go:238).  Needs no GPU.  On success *K_out receives the logical
+ * feature count derived from w_row_bytes; the output shape is [M, N]. ---- */
+int gq_qdense_check(int type, int x_dtype, int64_t M, int64_t x_last_dim, int64_t N,
+                    int64_t w_row_bytes, int64_t bias_len /* -1: no bias */, int act,
+                    int64_t *K_out);
+
+/* ---- device, memory, streams: compute.Backend buffer plumbing
+ * (BufferFromFlatData / ToFlatData, core/tensors/ondevice.go:273-285,462). ---- */
+int gq_device_count(int *count);
+int gq_init(int device);                 /* idempotent, thread-safe; requires gfx950 */
+int gq_device_name(char *buf, size_t n);
+int gq_malloc(void **dptr, size_t bytes);
+int gq_free(void *dptr);
+int gq_h2d(void *d, const void *h, size_t bytes, void *stream);  /* returns after the copy is done */
+int gq_d2h(void *h, const void *d, size_t bytes, void *stream);  /* returns after the copy is done */
+int gq_stream_create(void **stream);     /* default priority */
+int gq_stream_destroy(void *stream);
+int gq_sync(void *stream);
+
+/* ---- ggml.Dequantize (ml/ggml/dequant.go:39-54): dW [N, row_bytes] -> dOut [N, K] fp32,
+ * bit-exact with the reference arithmetic (one fp32 rounding per operation, no FMA). ---- */
+int gq_dequantize(int type, const void *dW, int64_t N, int64_t K, float *dOut, void *stream);
+
+/* ---- compute.Function.FusedQuantizedDense (core/graph/fused_ops.go:231-232), run time:
+ * y = act(x . dequant(W)^T + bias), the contract of nn.QuantizedDense
+ * (ml/nn/quantized_dense.go:31-57) and ggml.DenseDecomposed (ml/ggml/dense.go:23-62).
+ * dBias may be NULL.  fp32 activations: fp32 accumulation. ---- */
+int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *dW, int64_t N,
+                  const float *dBias, int act, float *dY, void *stream);
+/* bf16 activations (raw 16-bit patterns): weights are dequantised to bf16 tiles in LDS and
+ * contracted on bf16 MFMA with fp32 accumulation; fp32 output. */
+int gq_qdense_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, const void *dW,
+                   int64_t N, const float *dBias, int act, float *dY, void *stream);
+
+/* ---- compute.Function.QuantizedEmbeddingLookup (core/graph/fused_ops.go:295-296;
+ * nn.QuantizedGather ml/nn/quantized_gather.go:30-43; ml/ggml/gather.go:21-49):
+ * dOut[i, :] = dequant(dTable[dIndices[i], :]), bit-exact.  An index outside [0, vocab)
+ * yields a row of NaN and sets *dErrFlag (a device int32, may be NULL) to 1. ---- */
+int gq_embedding_lookup(int type, const void *dTable, int64_t vocab, int64_t K,
+                        const int32_t *dIndices, int64_t count, float *dOut,
+                        int32_t *dErrFlag, void *stream);
+
+/* ---- Executable.Execute of a compiled graph (core/graph/graph.go:669): a sequence of
+ * launches recorded once and replayed with one submission (HIP graph).  Between begin
+ * and end, entry points called with this stream are recorded, not run. ---- */
+int gq_graph_begin(void *stream);
+int gq_graph_end(void *stream, void **graph_exec);
+int gq_graph_launch(void *graph_exec, void *stream);
+int gq_graph_destroy(void *graph_exec);
+
+/* ---- kernel timing (the counterpart of the klog -v=1 wall clock around Execute,
+ * core/graph/graph.go:667-671): while enabled on the calling thread, every kernel launch
+ * is bracketed by HIP events on its own stream.  gq_profile_end waits for them and
+ * reports the launch count and the summed kernel time. ---- */
+int gq_profile_begin(void);
+int gq_profile_end(int *launches, double *total_us);
+
+/* Message of the last error on this thread; valid until the next failing call. */
+const char *gq_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

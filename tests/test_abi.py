@@ -1,0 +1,116 @@
+"""CPU-side checks of the C ABI: the library loads, exports every symbol the header declares,
+and its host-only entry points (geometry, build-time validation, error reporting) behave
+like the reference's graph-build checks.  No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from gomlx_amd import _lib, ggml
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "gomlx_hipq.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(gq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_all_exported_and_bound():
+    syms = declared_symbols()
+    assert len(syms) >= 20
+    L = ctypes.CDLL(_lib.LIB_PATH)
+    for s in syms:
+        assert hasattr(L, s), f"{s} is declared in the header but not exported"
+    bound = {name for name, _, _ in _lib.SIGNATURES}
+    assert bound == set(syms)
+
+
+def test_no_oracle_or_torch_linked_into_the_library():
+    import subprocess
+    out = subprocess.run(["ldd", _lib.LIB_PATH], capture_output=True, text=True).stdout
+    assert "libamdhip64" in out
+    assert "ggml_oracle" not in out and "torch" not in out
+
+
+def test_geometry_matches_reference_block_formats():
+    L = _lib.lib()
+    assert L.gq_abi_version() == 1
+    for t, bpb, vpb in [(ggml.Q4_0, 18, 32), (ggml.Q8_0, 34, 32), (ggml.Q4_K, 144, 256), (ggml.IQ4_NL, 18, 32)]:
+        assert L.gq_bytes_per_block(t) == bpb == ggml.bytes_per_block(t)
+        assert L.gq_values_per_block(t) == vpb == ggml.values_per_block(t)
+    assert L.gq_row_bytes(ggml.Q8_0, 4096) == 4352
+    assert L.gq_row_bytes(ggml.Q4_0, 4096) == 2304
+    assert L.gq_row_bytes(ggml.Q4_K, 14336) == 8064
+    assert L.gq_row_bytes(ggml.Q4_K, 4096) == 2304
+    assert L.gq_row_bytes(ggml.Q4_K, 4128) == 0      # not a whole number of super-blocks
+    assert L.gq_row_bytes(ggml.Q8_0, 0) == 0
+    assert L.gq_row_bytes(99, 4096) == 0
+    assert L.gq_bytes_per_block(99) == 0
+    assert ggml.can_decompose(ggml.Q8_0) and ggml.can_decompose(ggml.Q4_0) and ggml.can_decompose(ggml.IQ4_NL)
+    assert not ggml.can_decompose(ggml.Q4_K)   # ml/ggml/dequant.go:20-27
+
+
+def check(*args):
+    K = ctypes.c_int64(-1)
+    rc = _lib.lib().gq_qdense_check(*args, ctypes.byref(K))
+    return rc, K.value, _lib.lib().gq_last_error().decode()
+
+
+def test_build_time_validation():
+    # (type, x_dtype, M, x_last_dim, N, w_row_bytes, bias_len, act)
+    assert check(ggml.Q8_0, _lib.F32, 1, 4096, 4096, 4352, -1, 0)[:2] == (_lib.OK, 4096)
+    assert check(ggml.Q4_K, _lib.F32, 32, 14336, 4096, 8064, 4096, 3)[:2] == (_lib.OK, 14336)
+    assert check(ggml.Q8_0, _lib.BF16, 2048, 4096, 4096, 4352, -1, 0)[:2] == (_lib.OK, 4096)
+    assert check(ggml.Q4_0, _lib.F32, 0, 32, 2, 18, -1, 0)[0] == _lib.OK          # empty batch is fine
+    # malformed -> hard error (the graph layer panics, core/graph/fused_ops.go:233-235)
+    rc, _, msg = check(ggml.Q8_0, _lib.F32, 1, 4096, 4096, 4353, -1, 0)
+    assert rc == _lib.ERR_INVALID and "whole number" in msg
+    rc, _, msg = check(ggml.Q8_0, _lib.F32, 1, 4000, 4096, 4352, -1, 0)           # ml/ggml/dense.go:38-41
+    assert rc == _lib.ERR_INVALID and "K=4096" in msg
+    assert check(ggml.Q8_0, _lib.F32, 1, 4096, 4096, 4352, 4095, 0)[0] == _lib.ERR_INVALID
+    assert check(ggml.Q8_0, _lib.F32, 1, 4096, 4096, 4352, -1, 6)[0] == _lib.ERR_INVALID
+    assert check(ggml.Q8_0, _lib.F32, 1, 4096, 4096, 0, -1, 0)[0] == _lib.ERR_INVALID
+    # valid but unsupported -> NotImplemented (caller falls back, core/graph/fused_ops.go:357-363)
+    assert check(14, _lib.F32, 1, 256, 4, 210, -1, 0)[0] == _lib.ERR_NOT_IMPLEMENTED   # Q6_K
+    assert check(ggml.Q8_0, 7, 1, 4096, 4096, 4352, -1, 0)[0] == _lib.ERR_NOT_IMPLEMENTED
+
+
+def test_argument_errors_are_reported_before_any_device_work():
+    L = _lib.lib()
+    # bad K / type are diagnosed from the arguments alone, with or without a GPU
+    assert L.gq_qdense_f32(ggml.Q8_0, 16, 1, 33, 16, 1, None, 0, 16, None) == _lib.ERR_INVALID
+    assert b"multiple of the block size" in L.gq_last_error()
+    assert L.gq_qdense_f32(99, 16, 1, 32, 16, 1, None, 0, 16, None) == _lib.ERR_NOT_IMPLEMENTED
+    assert L.gq_qdense_bf16(ggml.Q4_K, 16, 1, 255, 16, 1, None, 0, 16, None) == _lib.ERR_INVALID
+    assert L.gq_qdense_f32(ggml.Q8_0, 16, 1, 32, 16, 1, None, 9, 16, None) == _lib.ERR_INVALID
+    assert L.gq_qdense_f32(ggml.Q8_0, None, 1, 32, 16, 1, None, 0, 16, None) == _lib.ERR_INVALID
+    assert L.gq_qdense_f32(ggml.Q8_0, 16, 1, 32, 24, 1, None, 0, 16, None) == _lib.ERR_INVALID   # W not 16-B aligned
+    assert L.gq_dequantize(ggml.Q4_0, 16, 2, 48, 16, None) == _lib.ERR_INVALID
+    assert L.gq_dequantize(ggml.Q4_0, 16, -1, 32, 16, None) == _lib.ERR_INVALID
+    assert L.gq_embedding_lookup(ggml.Q4_0, 16, 0, 32, 16, 3, 16, None, None) == _lib.ERR_INVALID
+    assert L.gq_graph_begin(None) == _lib.ERR_INVALID
+    assert L.gq_profile_end(None, None) == _lib.ERR_INVALID
+    # empty problems succeed without touching a device
+    assert L.gq_qdense_f32(ggml.Q8_0, None, 0, 32, None, 5, None, 0, None, None) == _lib.OK
+    assert L.gq_dequantize(ggml.Q8_0, None, 0, 32, None, None) == _lib.OK
+
+
+def test_python_wrapper_maps_statuses_to_exceptions():
+    with pytest.raises(_lib.HipqError) as e:
+        _lib.check(_lib.lib().gq_qdense_f32(ggml.Q8_0, 16, 1, 33, 16, 1, None, 0, 16, None))
+    assert e.value.status == _lib.ERR_INVALID and not isinstance(e.value, _lib.NotImplementedByBackend)
+    with pytest.raises(_lib.NotImplementedByBackend):
+        _lib.check(_lib.lib().gq_qdense_f32(99, 16, 1, 32, 16, 1, None, 0, 16, None))
+
+
+def test_activation_mapping_quirks():
+    from gomlx_amd.nn import Activation
+    # activation.Type.ToBackend, ml/layers/activation/activation.go:58-75
+    assert Activation.GELU.to_backend() == Activation.GELU_APPROX.to_backend() == 1
+    assert Activation.SWISH.to_backend() == Activation.SILU.to_backend() == 3
+    assert Activation.RELU.to_backend() == 2 and Activation.HARD_SWISH.to_backend() == 4 and Activation.TANH.to_backend() == 5
+    for dropped in (Activation.SIGMOID, Activation.HARD_SIGMOID, Activation.LEAKY_RELU, Activation.SELU, Activation.SWIGLU):
+        assert dropped.to_backend() == 0

@@ -1,0 +1,336 @@
+"""GPU parity: the HIP path (through the C ABI) against the CPU oracle on identical inputs.
+
+Bars (from the task statement): dequantised weights bit-exact; fp32-activation outputs within
+1e-3, bf16-MFMA outputs within 2e-2, both measured as max|got - want| / max|want| over the
+output (per-element relative error is meaningless for near-cancelling sums of thousands of
+N(0,1) terms).
+"""
+import numpy as np
+import pytest
+
+from gomlx_amd import ggml, nn, synth
+from gomlx_amd.nn import Activation, Quantization
+
+pytestmark = pytest.mark.gpu
+
+Q4_0, Q8_0, Q4_K, IQ4_NL = ggml.Q4_0, ggml.Q8_0, ggml.Q4_K, ggml.IQ4_NL
+ALL_TYPES = [Q4_0, Q8_0, Q4_K, IQ4_NL]
+TOL_F32 = 1e-3
+TOL_BF16 = 2e-2
+
+BACKEND_ACT = {0: Activation.NONE, 1: Activation.GELU, 2: Activation.RELU, 3: Activation.SILU,
+               4: Activation.HARD_SWISH, 5: Activation.TANH}
+
+
+def dev(torch, a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def rel_err(got, want):
+    scale = float(np.max(np.abs(want))) or 1.0
+    return float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)))) / scale
+
+
+def run_dense(torch, t, x, W, bias=None, act=0, bf16=False):
+    xd = dev(torch, x)
+    if bf16:
+        xd = xd.to(torch.bfloat16)
+    y = nn.quantized_dense(xd, dev(torch, W), Quantization(ggml_type=t), None if bias is None else dev(torch, bias),
+                           BACKEND_ACT[act])
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+def bf16_round(x):
+    import torch
+    return torch.from_numpy(x).to(torch.bfloat16).to(torch.float32).numpy()
+
+
+# ------------------------------------------------------------------------------ reference KATs
+
+def test_reference_dense_kats(gpu, kats):
+    for k in kats["dense"]:
+        got = run_dense(gpu, k["type"], np.array(k["x"], np.float32), np.array(k["w"], np.uint8),
+                        None if k["bias"] is None else np.array(k["bias"], np.float32), k["act"])
+        np.testing.assert_allclose(got, np.array(k["want"], np.float32), rtol=0, atol=k["tol"], err_msg=k["name"])
+
+
+def test_reference_gather_kats(gpu, kats):
+    for k in kats["gather"]:
+        out = nn.quantized_gather(dev(gpu, np.array(k["table"], np.uint8)), dev(gpu, np.array(k["indices"], np.int32)),
+                                  Quantization(ggml_type=k["type"]))
+        np.testing.assert_allclose(out.cpu().numpy(), np.array(k["want"], np.float32), rtol=0, atol=k["tol"],
+                                   err_msg=k["name"])
+
+
+# ------------------------------------------------------------------------------ dequantisation (bit-exact)
+
+@pytest.mark.parametrize("t", ALL_TYPES)
+@pytest.mark.parametrize("N,K", [(1, 256), (37, 512), (300, 4096)])
+def test_dequantize_bit_exact(gpu, oracle, t, N, K):
+    W = synth.weights(t, 10 + t, N, K)
+    got = nn.dequantize(dev(gpu, W), t).cpu().numpy()
+    want = oracle.c_dequantize(t, W, K)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("t", ALL_TYPES)
+def test_dequantize_bit_exact_on_extreme_scales(gpu, oracle, t):
+    """Random bytes everywhere, including the fp16 scale fields (subnormals, large values)."""
+    K, N = 1024, 64
+    rb = ggml.row_bytes(t, K)
+    raw = (synth.bits64(77, t, N * rb) >> np.uint64(20)).astype(np.uint8).reshape(N, rb)
+    blk = raw.reshape(N, -1, ggml.bytes_per_block(t))
+    # keep the fp16 fields finite (exponent != 31): inf/NaN scales are outside the contract
+    for off in ([1] if t != Q4_K else [1, 3]):
+        hi = blk[:, :, off]
+        hi[(hi & 0x7C) == 0x7C] &= 0xBF
+    got = nn.dequantize(dev(gpu, raw), t).cpu().numpy()
+    want = oracle.c_dequantize(t, raw, K)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_dequantize_full_size_config0(gpu, oracle):
+    W = synth.weights(Q8_0, 1000, 4096, 4096)
+    got = nn.dequantize(dev(gpu, W), Q8_0).cpu().numpy()
+    want = oracle.c_dequantize(Q8_0, W, 4096)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+# ------------------------------------------------------------------------------ decode GEMV (fp32)
+
+@pytest.mark.parametrize("t", ALL_TYPES)
+@pytest.mark.parametrize("M,K,N", [(1, 256, 1), (1, 512, 7), (2, 1024, 33), (3, 4096, 130), (4, 2048, 257), (1, 14336, 64)])
+def test_gemv_parity(gpu, oracle, t, M, K, N):
+    W = synth.weights(t, 20 + t, N, K)
+    x = synth.activations(21 + t, M, K)
+    bias = synth.normal(22 + t, 0, N).astype(np.float32) * 0.1
+    for act in (0, 3):
+        got = run_dense(gpu, t, x, W, bias, act)
+        want = oracle.c_qdense(t, x, W, bias, act)
+        assert got.shape == (M, N)
+        assert rel_err(got, want) < TOL_F32, (t, M, K, N, act)
+
+
+@pytest.mark.parametrize("t", ALL_TYPES)
+def test_gemv_long_k_is_chunked(gpu, oracle, t):
+    """K above the 16384 values one LDS pass holds."""
+    K, N = 16384 + 4096, 19
+    W = synth.weights(t, 30 + t, N, K)
+    x = synth.activations(31 + t, 1, K)
+    assert rel_err(run_dense(gpu, t, x, W), oracle.c_qdense(t, x, W)) < TOL_F32
+
+
+@pytest.mark.parametrize("t", ALL_TYPES)
+def test_gemv_all_activations_and_no_bias(gpu, oracle, t):
+    K, N = 512, 96
+    W = synth.weights(t, 40 + t, N, K)
+    x = synth.activations(41 + t, 1, K)
+    # scale so pre-activations spread over roughly [-4, 4]
+    pre = oracle.c_qdense(t, x, W)
+    x = (x * (2.0 / (np.std(pre) + 1e-9))).astype(np.float32)
+    for act in range(6):
+        got = run_dense(gpu, t, x, W, None, act)
+        want = oracle.c_qdense(t, x, W, None, act)
+        assert rel_err(got, want) < TOL_F32, (t, act)
+
+
+@pytest.mark.parametrize("t", ALL_TYPES)
+def test_gemv_unit_vectors_return_dequantised_columns(gpu, oracle, t):
+    K, N = 512, 40
+    W = synth.weights(t, 50 + t, N, K)
+    Wd = oracle.c_dequantize(t, W, K)
+    for k in [0, 15, 16, 31, 32, 63, 255, 256, 300, 511]:
+        x = np.zeros((1, K), np.float32)
+        x[0, k] = 1.0
+        got = run_dense(gpu, t, x, W)[0]
+        np.testing.assert_allclose(got, Wd[:, k], rtol=2e-6, atol=1e-9)
+
+
+def test_gemv_unaligned_activation_pointer(gpu, oracle):
+    K, N = 1024, 50
+    W = synth.weights(Q4_0, 60, N, K)
+    x = synth.activations(61, 1, K)
+    buf = gpu.zeros(K + 1, dtype=gpu.float32, device="cuda")
+    buf[1:] = dev(gpu, x[0])
+    xv = buf[1:].view(1, K)  # 4-byte aligned only
+    y = nn.quantized_dense(xv, dev(gpu, W), Quantization(ggml_type=Q4_0))
+    assert rel_err(y.cpu().numpy(), oracle.c_qdense(Q4_0, x, W)) < TOL_F32
+
+
+def test_leading_batch_axes_and_empty_batch(gpu, oracle):
+    K, N = 256, 12
+    W = synth.weights(Q8_0, 70, N, K)
+    x = synth.activations(71, 6, K).reshape(2, 3, K)
+    y = nn.quantized_dense(dev(gpu, x), dev(gpu, W), Quantization(ggml_type=Q8_0))
+    assert tuple(y.shape) == (2, 3, N)
+    assert rel_err(y.cpu().numpy().reshape(6, N), oracle.c_qdense(Q8_0, x.reshape(6, K), W)) < TOL_F32
+    y0 = nn.quantized_dense(gpu.zeros((0, K), device="cuda"), dev(gpu, W), Quantization(ggml_type=Q8_0))
+    assert tuple(y0.shape) == (0, N)
+
+
+# ------------------------------------------------------------------------------ batched (MFMA) paths
+
+@pytest.mark.parametrize("t", ALL_TYPES)
+@pytest.mark.parametrize("M,K,N", [(5, 256, 7), (32, 1024, 130), (130, 512, 257), (64, 4096, 96)])
+def test_batched_f32_parity(gpu, oracle, t, M, K, N):
+    W = synth.weights(t, 80 + t, N, K)
+    x = synth.activations(81 + t, M, K)
+    bias = synth.normal(82 + t, 0, N).astype(np.float32) * 0.1
+    for act in (0, 2):
+        got = run_dense(gpu, t, x, W, bias, act)
+        want = oracle.c_qdense(t, x, W, bias, act)
+        assert rel_err(got, want) < TOL_F32, (t, M, K, N, act)
+
+
+@pytest.mark.parametrize("t", ALL_TYPES)
+@pytest.mark.parametrize("M,K,N", [(1, 256, 5), (64, 1024, 130), (200, 512, 300)])
+def test_bf16_prefill_parity(gpu, oracle, t, M, K, N):
+    W = synth.weights(t, 90 + t, N, K)
+    x = bf16_round(synth.activations(91 + t, M, K))
+    bias = synth.normal(92 + t, 0, N).astype(np.float32) * 0.1
+    got = run_dense(gpu, t, x, W, bias, 3, bf16=True)
+    want = oracle.c_qdense(t, x, W, bias, 3)
+    assert rel_err(got, want) < TOL_BF16, (t, M, K, N)
+
+
+# ------------------------------------------------------------------------------ benchmark configurations, full size
+
+def test_config0_q8_0_gemv_4096(gpu, oracle):
+    W = synth.weights(Q8_0, 1000, 4096, 4096)
+    x = synth.activations(1000, 1, 4096)
+    assert rel_err(run_dense(gpu, Q8_0, x, W), oracle.c_qdense(Q8_0, x, W)) < TOL_F32
+
+
+def test_config1_q4_0_gemv_14336(gpu, oracle):
+    W = synth.weights(Q4_0, 1001, 14336, 4096)
+    x = synth.activations(1001, 1, 4096)
+    assert rel_err(run_dense(gpu, Q4_0, x, W), oracle.c_qdense(Q4_0, x, W)) < TOL_F32
+
+
+def test_config2_q4_k_batch32(gpu, oracle):
+    W = synth.weights(Q4_K, 1002, 4096, 14336)
+    x = synth.activations(1002, 32, 14336)
+    assert rel_err(run_dense(gpu, Q4_K, x, W), oracle.c_qdense(Q4_K, x, W)) < TOL_F32
+
+
+def test_config3_q8_0_prefill_bf16(gpu, oracle):
+    W = synth.weights(Q8_0, 1000, 4096, 4096)
+    x = bf16_round(synth.activations(1003, 2048, 4096))
+    got = run_dense(gpu, Q8_0, x, W, bf16=True)
+    rows = np.array([0, 1, 31, 32, 127, 128, 1000, 2047])
+    want = oracle.c_qdense(Q8_0, x[rows], W)
+    assert got.shape == (2048, 4096)
+    assert rel_err(got[rows], want) < TOL_BF16
+    # size-independent property on the whole output: duplicated activation rows give identical rows
+    x2 = x.copy()
+    x2[1024:] = x2[:1024]
+    got2 = run_dense(gpu, Q8_0, x2, W, bf16=True)
+    assert np.array_equal(got2[:1024], got2[1024:])
+    assert np.array_equal(got2[:1024], got[:1024])
+
+
+def test_config4_llama_layer_projections(gpu, oracle):
+    shapes = [(4096, 4096), (4096, 1024), (4096, 1024), (4096, 4096), (4096, 14336), (4096, 14336), (14336, 4096)]
+    for i, (K, N) in enumerate(shapes):
+        W = synth.weights(Q4_K, 1004 + i, N, K)
+        x = synth.activations(1104 + i, 1, K)
+        assert rel_err(run_dense(gpu, Q4_K, x, W), oracle.c_qdense(Q4_K, x, W)) < TOL_F32, (K, N)
+
+
+# ------------------------------------------------------------------------------ gather
+
+@pytest.mark.parametrize("t", ALL_TYPES)
+def test_gather_random_rows_bit_exact(gpu, oracle, t):
+    vocab, K = 1000, 512
+    table = synth.weights(t, 110 + t, vocab, K)
+    idx = synth.randint(111, t, 2 * 77, 0, vocab - 1).astype(np.int32).reshape(2, 77, 1)
+    out = nn.quantized_gather(dev(gpu, table), dev(gpu, idx), Quantization(ggml_type=t)).cpu().numpy()
+    want = oracle.c_embedding_lookup(t, table, K, idx)
+    assert out.shape == (2, 77, K)
+    assert np.array_equal(out.view(np.uint32), want.view(np.uint32))
+
+
+def test_gather_out_of_range_index_raises(gpu):
+    table = synth.weights(Q8_0, 120, 10, 64)
+    for bad in (10, -1):
+        with pytest.raises(IndexError):
+            nn.quantized_gather(dev(gpu, table), dev(gpu, np.array([[3], [bad]], np.int32)), Quantization(ggml_type=Q8_0))
+
+
+# ------------------------------------------------------------------------------ recorded replays and timing hooks
+
+def test_recorded_chain_replays_match_eager(gpu, oracle):
+    """Seven projections recorded once (HIP graph) and replayed; every replay must equal the
+    eager result, with eager work and synchronisations in between."""
+    from gomlx_amd import _lib
+    torch = gpu
+    L = _lib.lib()
+    shapes = [(1024, 512), (1024, 256), (1024, 256), (1024, 512), (1024, 1536), (1024, 1536), (1536, 1024)]
+    Ws = [dev(torch, synth.weights(Q4_K, 130 + i, N, K)) for i, (K, N) in enumerate(shapes)]
+    xs = [dev(torch, synth.activations(140 + i, 1, K)) for i, (K, N) in enumerate(shapes)]
+    ys = [torch.zeros(1, N, device="cuda") for (K, N) in shapes]
+    eager = [nn.quantized_dense(x, W, Quantization(ggml_type=Q4_K)).clone() for x, W in zip(xs, Ws)]
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    sp = stream.cuda_stream
+    _lib.check(L.gq_graph_begin(sp))
+    for (K, N), x, W, y in zip(shapes, xs, Ws, ys):
+        _lib.check(L.gq_qdense_f32(Q4_K, x.data_ptr(), 1, K, W.data_ptr(), N, None, 0, y.data_ptr(), sp))
+    import ctypes
+    g = ctypes.c_void_p()
+    _lib.check(L.gq_graph_end(sp, ctypes.byref(g)))
+    for rep in range(4):
+        for y in ys:
+            y.fill_(float("nan"))
+        torch.cuda.synchronize()
+        _lib.check(L.gq_graph_launch(g, sp))
+        _lib.check(L.gq_sync(sp))
+        for y, e in zip(ys, eager):
+            assert torch.equal(y, e), rep
+        # eager work between replays
+        again = nn.quantized_dense(xs[0], Ws[0], Quantization(ggml_type=Q4_K))
+        torch.cuda.synchronize()
+        assert torch.equal(again, eager[0])
+    _lib.check(L.gq_graph_destroy(g))
+
+
+def test_kernel_timing_hook_counts_launches(gpu):
+    from gomlx_amd import _lib
+    import ctypes
+    L = _lib.lib()
+    W = dev(gpu, synth.weights(Q8_0, 150, 512, 1024))
+    x = dev(gpu, synth.activations(151, 1, 1024))
+    ref = nn.quantized_dense(x, W, Quantization(ggml_type=Q8_0))
+    _lib.check(L.gq_profile_begin())
+    outs = [nn.quantized_dense(x, W, Quantization(ggml_type=Q8_0)) for _ in range(5)]
+    n, us = ctypes.c_int(0), ctypes.c_double(0.0)
+    _lib.check(L.gq_profile_end(ctypes.byref(n), ctypes.byref(us)))
+    assert n.value == 5 and 0.0 < us.value < 5e4
+    for o in outs:
+        assert gpu.equal(o, ref)
+
+
+# ------------------------------------------------------------------------------ operator-level error behaviour
+
+def test_operator_rejects_bad_arguments(gpu):
+    from gomlx_amd import _lib
+    W = dev(gpu, synth.weights(Q8_0, 160, 8, 64))
+    x = gpu.zeros((1, 64), device="cuda")
+    q = Quantization(ggml_type=Q8_0)
+    with pytest.raises(_lib.HipqError):            # x features != K (ml/ggml/dense.go:38-41)
+        nn.quantized_dense(gpu.zeros((1, 96), device="cuda"), W, q)
+    with pytest.raises(_lib.HipqError):            # bias length
+        nn.quantized_dense(x, W, q, gpu.zeros(7, device="cuda"))
+    with pytest.raises(ValueError):                # more than one activation (quantized_dense.go:35-38)
+        nn.quantized_dense(x, W, q, None, Activation.RELU, Activation.TANH)
+    with pytest.raises(_lib.NotImplementedByBackend):
+        nn.quantized_dense(x, W, Quantization(scheme=nn.QuantizationScheme.NF4))
+    with pytest.raises(_lib.NotImplementedByBackend):
+        nn.quantized_dense(x.to(gpu.float16), W, q)
+    with pytest.raises(ValueError):                # CPU tensors: there is no CPU path
+        nn.quantized_dense(x.cpu(), W, q)
+    # activations without a backend enum are dropped on the fused route (activation.go:72-73)
+    y0 = nn.quantized_dense(x + 1.0, W, q)
+    y1 = nn.quantized_dense(x + 1.0, W, q, None, Activation.SIGMOID)
+    assert gpu.equal(y0, y1)
