@@ -1,0 +1,267 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized Dense hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1] [--others]
+
+A "step" is one quantized Dense call (one pass over one weight matrix) on synthetic data that
+is already resident in HBM.  The headline workload is BASELINE.json configs[1]: Q4_0 decode
+GEMV, batch 1, K=4096 -> N=14336.  Steps rotate over enough distinct weight copies (> 512 MB)
+that every pass streams its weights from HBM rather than from the 256 MB Infinity Cache.
+
+Prints ONE JSON line.  `value` is weight-GB/s over the wall clock of the K timed steps
+(submitted as one recorded HIP graph unless --no-graph).  `roofline` is the dominant kernel's
+own rate: algorithmic weight bytes per launch / mean kernel duration from start/stop HIP
+events attached to each launch on its stream (a second pass over the same K steps).
+`cpu_baseline` times the CPU oracle's fused fp32 restatement on the host cores (rank 0, N=1).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+# name -> (ggml type name, M, K, N, activation dtype, bound)
+CONFIGS = {
+    "c0": ("Q8_0", 1, 4096, 4096, "f32", "hbm"),
+    "c1": ("Q4_0", 1, 4096, 14336, "f32", "hbm"),
+    "c2": ("Q4_K", 32, 14336, 4096, "f32", "hbm"),
+    "c3": ("Q8_0", 2048, 4096, 4096, "bf16", "mfma"),
+}
+C4_SHAPES = [(4096, 4096), (4096, 1024), (4096, 1024), (4096, 4096), (4096, 14336), (4096, 14336), (14336, 4096)]
+WORKLOAD_TEXT = {
+    "c0": "configs[0]: Q8_0 dense GEMV, x f32 [1,4096], W [4096,4096]",
+    "c1": "configs[1]: Q4_0 dense GEMV, batch 1, K=4096 -> N=14336",
+    "c2": "configs[2]: Q4_K dense, decode batch M=32, K=14336 -> N=4096",
+    "c3": "configs[3]: Q8_0 prefill GEMM, M=2048 bf16, K=4096, N=4096",
+    "c4": "configs[4]: seven Q4_K projections of a Llama-3-8B layer, batch 1",
+}
+
+
+def parse_args():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=200)
+    p.add_argument("--warmup", type=int, default=20)
+    p.add_argument("--config", default="c1", choices=sorted(list(CONFIGS) + ["c4"]))
+    p.add_argument("--others", action="store_true", help="also measure the other configurations (reported under 'others')")
+    p.add_argument("--no-graph", action="store_true", help="submit the timed steps one call at a time")
+    p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    p.add_argument("--hot", action="store_true", help="single weight buffer (Infinity-Cache resident) instead of the cold rotation")
+    return p.parse_args()
+
+
+class Problem:
+    """One (x, W-rotation, y) set resident on the GPU plus the launch closure."""
+
+    def __init__(self, torch, name, hot=False):
+        from gomlx_amd import _lib, ggml, synth
+        import numpy as np
+        self.torch, self.name = torch, name
+        self.L = _lib.lib()
+        self.check = _lib.check
+        if name == "c4":
+            shapes = [("Q4_K", 1, K, N) for K, N in C4_SHAPES]
+            self.dtype, self.bound = "f32", "hbm"
+        else:
+            tn, M, K, N, self.dtype, self.bound = CONFIGS[name]
+            shapes = [(tn, M, K, N)]
+        self.parts = []
+        seed = 1000 + int(name[1])
+        total_w = 0
+        for i, (tn, M, K, N) in enumerate(shapes):
+            t = getattr(ggml, tn)
+            W = torch.from_numpy(synth.weights(t, seed + i, N, K)).cuda()
+            x = torch.from_numpy(synth.activations(seed + 100 + i, M, K)).cuda()
+            if self.dtype == "bf16":
+                x = x.to(torch.bfloat16)
+            y = torch.empty((M, N), dtype=torch.float32, device="cuda")
+            self.parts.append(dict(t=t, M=M, K=K, N=N, W=[W], x=x, y=y, wbytes=W.numel()))
+            total_w += W.numel()
+        self.weight_bytes = total_w
+        self.flops = sum(2 * p["M"] * p["K"] * p["N"] for p in self.parts)
+        # cold rotation: distinct copies (rows rolled) until the set exceeds 2 x Infinity Cache
+        self.copies = 1 if hot else max(2, -(-(512 << 20) // total_w) + 1)
+        for p in self.parts:
+            for c in range(1, self.copies):
+                p["W"].append(torch.roll(p["W"][0], shifts=c, dims=0).contiguous())
+        self.stream = torch.cuda.current_stream().cuda_stream
+        torch.cuda.synchronize()
+
+    def launch(self, step):
+        c = step % self.copies
+        for p in self.parts:
+            fn = self.L.gq_qdense_bf16 if self.dtype == "bf16" else self.L.gq_qdense_f32
+            self.check(fn(p["t"], p["x"].data_ptr(), p["M"], p["K"], p["W"][c].data_ptr(), p["N"], None, 0,
+                          p["y"].data_ptr(), self.stream))
+
+    def run(self, steps, warmup, use_graph):
+        torch, L = self.torch, self.L
+        for s in range(warmup):
+            self.launch(s)
+        torch.cuda.synchronize()
+        graph = None
+        if use_graph:
+            side = torch.cuda.Stream()
+            sp = side.cuda_stream
+            saved, self.stream = self.stream, sp
+            self.check(L.gq_graph_begin(sp))
+            for s in range(steps):
+                self.launch(warmup + s)
+            g = ctypes.c_void_p()
+            self.check(L.gq_graph_end(sp, ctypes.byref(g)))
+            self.stream = saved
+            graph = g
+            if warmup > 0:  # untimed first replay: uploads the graph
+                self.check(L.gq_graph_launch(graph, self.stream))
+            torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        if graph is not None:
+            self.check(L.gq_graph_launch(graph, self.stream))
+        else:
+            for s in range(steps):
+                self.launch(warmup + s)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        if graph is not None:
+            self.check(L.gq_graph_destroy(graph))
+        # second pass over the same steps: per-launch start/stop events on the launch stream
+        self.check(L.gq_profile_begin())
+        for s in range(steps):
+            self.launch(warmup + s)
+        n, us = ctypes.c_int(0), ctypes.c_double(0.0)
+        self.check(L.gq_profile_end(ctypes.byref(n), ctypes.byref(us)))
+        kernel_us_per_step = us.value / steps
+        return wall, kernel_us_per_step, n.value // steps
+
+    def report(self, wall, kernel_us, steps):
+        out = {}
+        if self.bound == "hbm":
+            out["metric"], out["unit"] = "dense GEMV weight-GB/s", "GB/s"
+            out["value"] = self.weight_bytes * steps / wall / 1e9
+            ach = self.weight_bytes / (kernel_us * 1e-6) / 1e9
+            out["roofline"] = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                               "frac": ach / HBM_PEAK_GBS, "traffic": None,
+                               "algorithmic_bytes_per_launch": self.weight_bytes, "kernel_us": kernel_us}
+        else:
+            out["metric"], out["unit"] = "prefill GEMM TFLOP/s", "TFLOP/s"
+            out["value"] = self.flops * steps / wall / 1e12
+            ach = self.flops / (kernel_us * 1e-6) / 1e12
+            out["roofline"] = {"bound": "mfma", "achieved": ach, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                               "frac": ach / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                               "algorithmic_flops_per_launch": self.flops, "kernel_us": kernel_us}
+        out["ms_per_step"] = wall / steps * 1e3
+        return out
+
+
+def cpu_baseline(name):
+    """The CPU oracle's fused fp32 restatement on the host cores (checker code used as a
+    reported baseline only): >= 2 warm-ups, then >= 5 runs and >= 3 s, like the reference's own
+    timing protocol (internal/perf/dotgeneral_perf_test.go:366-381), capped at ~25 s."""
+    import numpy as np
+    from gomlx_amd import ggml, synth
+    from oracle import ggml_oracle as oracle
+    cores = min(os.cpu_count() or 1, 16)
+    if name == "c4":
+        shapes = [("Q4_K", 1, K, N) for K, N in C4_SHAPES]
+    else:
+        tn, M, K, N, _, _ = CONFIGS[name]
+        shapes = [(tn, M, K, N)]
+    sample = "full workload"
+    if name == "c3":  # 34 GMAC per pass is minutes of CPU time: a 64-row slice of the 2048 activations
+        shapes = [("Q8_0", 64, 4096, 4096)]
+        sample = "64 of the 2048 activation rows (1/32 of the FLOPs), all of W"
+    probs = []
+    for i, (tn, M, K, N) in enumerate(shapes):
+        t = getattr(ggml, tn)
+        probs.append((t, synth.activations(5 + i, M, K), synth.weights(t, 6 + i, N, K)))
+    wbytes = sum(p[2].size for p in probs)
+    flops = sum(2 * p[1].shape[0] * p[1].shape[1] * p[2].shape[0] for p in probs)
+
+    def once():
+        for t, x, W in probs:
+            oracle.c_qdense(t, x, W, None, 0, f32acc_threads=cores)
+
+    once(); once()
+    runs, t0 = 0, time.perf_counter()
+    while True:
+        once()
+        runs += 1
+        el = time.perf_counter() - t0
+        if (runs >= 5 and el >= 3.0) or el >= 25.0:
+            break
+    per = el / runs
+    if name == "c3":
+        return {"value": flops / per / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+                "sample": f"{sample}; {runs} runs, {per * 1e3:.2f} ms each"}
+    return {"value": wbytes / per / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"{sample}; {runs} runs, {per * 1e3:.2f} ms each"}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path is a single-GPU kernel; see DESIGN.md "
+              "for how it would shard); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; there is no CPU fallback for the product path", file=sys.stderr)
+        sys.exit(3)
+    from gomlx_amd import _lib
+    _lib.init(0)
+    torch.cuda.set_device(0)
+
+    def measure(name):
+        prob = Problem(torch, name, hot=args.hot)
+        wall, kus, launches = prob.run(args.steps, args.warmup, not args.no_graph)
+        rep = prob.report(wall, kus, args.steps)
+        rep["weight_copies"] = prob.copies
+        rep["launches_per_step"] = launches
+        del prob
+        torch.cuda.empty_cache()
+        return rep
+
+    rep = measure(args.config)
+    tn = "Q4_K" if args.config == "c4" else CONFIGS[args.config][0]
+    line = {
+        "metric": rep["metric"], "value": rep["value"], "unit": rep["unit"], "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": rep["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.config == "c3" else "f32", "data": "synthetic",
+        "config": {"workload": WORKLOAD_TEXT[args.config], "ggml_type": tn,
+                   "weights": "cache-resident single buffer" if args.hot else
+                   f"cold: rotation over {rep['weight_copies']} distinct weight copies",
+                   "submission": "eager" if args.no_graph else "one recorded HIP graph of all timed steps",
+                   "launches_per_step": rep["launches_per_step"]},
+        "roofline": rep["roofline"],
+    }
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(args.config)
+    if args.others:
+        others = {}
+        for name in ["c0", "c1", "c2", "c3", "c4"]:
+            if name == args.config:
+                continue
+            steps = args.steps if name != "c3" else max(10, args.steps // 10)
+            saved = args.steps
+            args.steps = steps
+            r = measure(name)
+            args.steps = saved
+            others[name] = {"workload": WORKLOAD_TEXT[name], "metric": r["metric"], "value": r["value"], "unit": r["unit"],
+                            "ms_per_step": r["ms_per_step"], "roofline": r["roofline"], "steps": steps}
+        line["others"] = others
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
