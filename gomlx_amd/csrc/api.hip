@@ -240,7 +240,11 @@ int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *d
     if (int rc = use_device()) return rc;
     // Up to four activation rows: one bandwidth-bound pass over W per row, fp32 throughout.
     // More rows: W is read once per 128-row tile and contracted on the matrix cores.
-    if (M <= 4) return launch_gemv(type, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
+    if (M <= 4) {
+        if (gemv_xs_supported(type, K, N, dX))
+            return launch_gemv_xs(type, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
+        return launch_gemv(type, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
+    }
     return launch_gemm(type, false, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
 }
 

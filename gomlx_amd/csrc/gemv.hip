@@ -171,6 +171,184 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_b32_kernel(const float *__res
     }
 }
 
+// ---- 32-value block formats, two blocks per lane ---------------------------------------
+//
+// The fast path whenever K is a multiple of 64.  A pair of consecutive blocks (36 bytes for
+// Q4_0 / IQ4_NL, 68 bytes for Q8_0) starts on a 4-byte boundary, so a lane fetches its pair
+// as whole dwords (dwordx4 ... + dword) and realigns the first block's payload in registers
+// with v_alignbit.  Measured on MI355X this pattern streams as fast as perfectly aligned
+// 16-byte loads, while one 18-byte block per lane (2-byte aligned loads) costs ~30 %.
+// The weight loads of the first step are issued before the activations are staged, so the
+// HBM latency overlaps the LDS fill and its barrier.
+template <int T> struct LanePair;
+
+template <> struct LanePair<kQ4_0> {
+    struct __attribute__((packed, aligned(4))) Raw { uint32_t v[9]; };
+    Raw raw;
+    __device__ __forceinline__ void load(const uint8_t *p) { raw = *reinterpret_cast<const Raw *>(p); }
+    __device__ __forceinline__ float dot(const float *xv, float xsum0, float xsum1) const {
+        const uint32_t *v = raw.v;
+        float r0, r1;
+        {
+            float lo = 0.f, hi = 0.f;
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                const uint32_t q = __builtin_amdgcn_alignbit(v[w + 1], v[w], 16);
+                const uint32_t l = q & 0x0F0F0F0Fu, h = q & 0xF0F0F0F0u;
+                lo = fmaf(ubyte0(l), xv[4 * w + 0], lo);
+                lo = fmaf(ubyte1(l), xv[4 * w + 1], lo);
+                lo = fmaf(ubyte2(l), xv[4 * w + 2], lo);
+                lo = fmaf(ubyte3(l), xv[4 * w + 3], lo);
+                hi = fmaf(ubyte0(h), xv[16 + 4 * w + 0], hi);
+                hi = fmaf(ubyte1(h), xv[16 + 4 * w + 1], hi);
+                hi = fmaf(ubyte2(h), xv[16 + 4 * w + 2], hi);
+                hi = fmaf(ubyte3(h), xv[16 + 4 * w + 3], hi);
+            }
+            r0 = half_bits_to_float(v[0] & 0xFFFFu) * (fmaf(hi, 0.0625f, lo) - 8.0f * xsum0);
+        }
+        {
+            float lo = 0.f, hi = 0.f;
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                const uint32_t q = v[5 + w];
+                const uint32_t l = q & 0x0F0F0F0Fu, h = q & 0xF0F0F0F0u;
+                lo = fmaf(ubyte0(l), xv[32 + 4 * w + 0], lo);
+                lo = fmaf(ubyte1(l), xv[32 + 4 * w + 1], lo);
+                lo = fmaf(ubyte2(l), xv[32 + 4 * w + 2], lo);
+                lo = fmaf(ubyte3(l), xv[32 + 4 * w + 3], lo);
+                hi = fmaf(ubyte0(h), xv[48 + 4 * w + 0], hi);
+                hi = fmaf(ubyte1(h), xv[48 + 4 * w + 1], hi);
+                hi = fmaf(ubyte2(h), xv[48 + 4 * w + 2], hi);
+                hi = fmaf(ubyte3(h), xv[48 + 4 * w + 3], hi);
+            }
+            r1 = half_bits_to_float(v[4] >> 16) * (fmaf(hi, 0.0625f, lo) - 8.0f * xsum1);
+        }
+        return r0 + r1;
+    }
+};
+
+template <> struct LanePair<kIQ4_NL> {
+    struct __attribute__((packed, aligned(4))) Raw { uint32_t v[9]; };
+    Raw raw;
+    __device__ __forceinline__ void load(const uint8_t *p) { raw = *reinterpret_cast<const Raw *>(p); }
+    __device__ __forceinline__ float dot(const float *xv, float, float) const {
+        const uint32_t *v = raw.v;
+        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const uint32_t qa = __builtin_amdgcn_alignbit(v[w + 1], v[w], 16), qb = v[5 + w];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint32_t a = (qa >> (8 * j)) & 0xFFu, b = (qb >> (8 * j)) & 0xFFu;
+                s0 = fmaf(iq4nl_value(a & 15u), xv[4 * w + j], s0);
+                s0 = fmaf(iq4nl_value(a >> 4), xv[16 + 4 * w + j], s0);
+                s1 = fmaf(iq4nl_value(b & 15u), xv[32 + 4 * w + j], s1);
+                s1 = fmaf(iq4nl_value(b >> 4), xv[48 + 4 * w + j], s1);
+            }
+        }
+        return half_bits_to_float(v[0] & 0xFFFFu) * s0 + half_bits_to_float(v[4] >> 16) * s1;
+    }
+};
+
+template <> struct LanePair<kQ8_0> {
+    struct __attribute__((packed, aligned(4))) Raw { uint32_t v[17]; };
+    Raw raw;
+    __device__ __forceinline__ void load(const uint8_t *p) { raw = *reinterpret_cast<const Raw *>(p); }
+    __device__ __forceinline__ float dot(const float *xv, float xsum0, float xsum1) const {
+        const uint32_t *v = raw.v;
+        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+            const uint32_t a = __builtin_amdgcn_alignbit(v[w + 1], v[w], 16) ^ 0x80808080u;
+            const uint32_t b = v[9 + w] ^ 0x80808080u;
+            s0 = fmaf(ubyte0(a), xv[4 * w + 0], s0);
+            s0 = fmaf(ubyte1(a), xv[4 * w + 1], s0);
+            s0 = fmaf(ubyte2(a), xv[4 * w + 2], s0);
+            s0 = fmaf(ubyte3(a), xv[4 * w + 3], s0);
+            s1 = fmaf(ubyte0(b), xv[32 + 4 * w + 0], s1);
+            s1 = fmaf(ubyte1(b), xv[32 + 4 * w + 1], s1);
+            s1 = fmaf(ubyte2(b), xv[32 + 4 * w + 2], s1);
+            s1 = fmaf(ubyte3(b), xv[32 + 4 * w + 3], s1);
+        }
+        return half_bits_to_float(v[0] & 0xFFFFu) * (s0 - 128.0f * xsum0) +
+               half_bits_to_float(v[8] >> 16) * (s1 - 128.0f * xsum1);
+    }
+};
+
+// LDS layout of the activation chunk: float4 #j (0..15) of pair p lives at xs[j * npc + p].
+template <int T, int R, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gemv_pair_kernel(const float *__restrict__ X, const uint8_t *__restrict__ W,
+                                                               const float *__restrict__ bias, float *__restrict__ Y,
+                                                               int K, int N, int64_t row_bytes, int kchunk, int act) {
+    extern __shared__ float4 xs[];
+    constexpr int pair_bytes = 2 * Geom<T>::bpb;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const float *x = X + (int64_t)blockIdx.y * K;
+    float *y = Y + (int64_t)blockIdx.y * N;
+    const bool aligned = (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+    const int ngroups = (N + R - 1) / R;
+    const int grp = blockIdx.x * WAVES + wave;
+    const bool live = grp < ngroups;
+    const int row0 = grp * R;
+    const uint8_t *wrow[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) wrow[r] = W + (int64_t)min(row0 + r, N - 1) * row_bytes;
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.f;
+
+    LanePair<T> cur[R];
+    const int np_total = K >> 6;
+    if (live && lane < np_total) {
+#pragma unroll
+        for (int r = 0; r < R; r++) cur[r].load(wrow[r] + (int64_t)lane * pair_bytes);
+    }
+    for (int k0 = 0; k0 < K; k0 += kchunk) {
+        const int kc = min(kchunk, K - k0);
+        const int npc = kc >> 6;
+        if (k0 > 0) __syncthreads();
+        for (int i = tid; i < (kc >> 2); i += WAVES * 64) xs[(i & 15) * npc + (i >> 4)] = load_x4(x + k0, i, aligned);
+        __syncthreads();
+        if (!live) continue;
+        for (int p0 = 0; p0 < npc; p0 += 64) {
+            const int p = p0 + lane;
+            // prefetch the next step's pairs (next 64 pairs of the row, possibly in the next chunk)
+            LanePair<T> nxt[R];
+            const int pn = (k0 >> 6) + p0 + 64 + lane;
+            const bool more = pn < np_total;
+            if (more) {
+#pragma unroll
+                for (int r = 0; r < R; r++) nxt[r].load(wrow[r] + (int64_t)pn * pair_bytes);
+            }
+            if (p < npc) {
+                float xv[64];
+#pragma unroll
+                for (int j = 0; j < 16; j++) {
+                    const float4 t = xs[j * npc + p];
+                    xv[4 * j] = t.x; xv[4 * j + 1] = t.y; xv[4 * j + 2] = t.z; xv[4 * j + 3] = t.w;
+                }
+                const float xsum0 = sum32(xv), xsum1 = sum32(xv + 32);
+#pragma unroll
+                for (int r = 0; r < R; r++) acc[r] += cur[r].dot(xv, xsum0, xsum1);
+            }
+            if (more) {
+#pragma unroll
+                for (int r = 0; r < R; r++) cur[r] = nxt[r];
+            }
+        }
+    }
+    if (!live) return;
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = wave_sum(acc[r]);
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int row = row0 + r;
+            if (row < N) y[row] = apply_act(act, acc[r] + (bias ? bias[row] : 0.f));
+        }
+    }
+}
+
 // ---- Q4_K -----------------------------------------------------------------------------
 //
 // Eight lanes share one 144-byte super-block: lane part i (0..7) takes code bytes
@@ -304,6 +482,9 @@ int launch_one(const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N
         return launch(gemv_q4k_kernel<R, WAVES>, grid, dim3(WAVES * 64), shmem, s, x, W, bias, y, (int)K, (int)N,
                       row_bytes, kchunk, act);
     } else {
+        if (K % 64 == 0)
+            return launch(gemv_pair_kernel<T, R, WAVES>, grid, dim3(WAVES * 64), shmem, s, x, W, bias, y, (int)K, (int)N,
+                          row_bytes, kchunk, act);
         return launch(gemv_b32_kernel<T, R, WAVES>, grid, dim3(WAVES * 64), shmem, s, x, W, bias, y, (int)K, (int)N,
                       row_bytes, kchunk, act);
     }
