@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "csrc", "build")
 LIB = os.path.join(HERE, "libgomlx_hipq.so")
 
-SOURCES = ["api.hip", "dequant.hip", "gemv.hip", "gemv_xs.hip", "gemm.hip"]
+SOURCES = ["api.hip", "dequant.hip", "gemv.hip", "gemv_xs.hip", "mmq.hip", "gemm.hip"]
 
 # -packed-fp32-ops (note the minus): keep hipcc from forming v_pk_*_f32 instructions.
 # -ffp-contract=off: dequantisation must round every fp32 operation on its own; fused
