@@ -245,7 +245,7 @@ int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *d
             return launch_gemv_xs(type, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
         return launch_gemv(type, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
     }
-    if (mmq_supported(type, M, K, N, dX))
+    if (mmq_supported(type, M, K, N, dX, dBias, dY))
         return launch_mmq(type, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
     return launch_gemm(type, false, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
 }

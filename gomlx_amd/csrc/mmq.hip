@@ -33,14 +33,15 @@ namespace {
 
 typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
-typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f16v __attribute__((ext_vector_type(16)));
 
 constexpr int kSliceSB = 8;                 // super-blocks per K-slice
 constexpr int kSliceK = kSliceSB * 256;     // 2048 values
-constexpr int kRowsPerWG = 128;             // 8 wavefronts x 16 rows
+constexpr int kRowsPerWG = 128;             // 4 row tiles of 32; kParts wavefronts (interleaved super-blocks) per tile
+constexpr int kParts = 2;                   // wavefronts sharing a row tile
 constexpr int kMT = 32;                     // batch columns per pass
 constexpr int kXFBytes = kSliceK * kMT * 2;          // 131072: fp16 activations, fragment order
-constexpr int kXSBytes = kSliceSB * 2 * kMT * 8;     // 4096: sub-block sums, fragment order
+constexpr int kXSBytes = kSliceSB * kMT * 16;        // 4096: eight sub-block sums per (super-block, column)
 constexpr int kLdsBytes = kXFBytes + kXSBytes;
 
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
@@ -52,8 +53,11 @@ __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
 
 __device__ __forceinline__ h2 as_h2(uint32_t u) { return __builtin_bit_cast(h2, u); }
 
-// (u & mask) | 0x64006400 as an fp16 pair: 1024 + n (mask 0x000F000F) or 1024 + 16 n (0x00F000F0)
-__device__ __forceinline__ h2 magic_pair(uint32_t u, uint32_t mask) { return as_h2((u & mask) | 0x64006400u); }
+// (u & mask) | 0x64006400 as an fp16 pair: 1024 + n (mask 0x000F000F), 1024 + 16 n (0x00F000F0)
+// or 1024 + byte (0x00FF00FF)
+// The 0x64006400 operand is passed in a register: with two literals the compiler has to split the
+// operation into v_and + v_or, with one it is a single v_and_or_b32.
+__device__ __forceinline__ h2 magic_pair(uint32_t u, uint32_t mask, uint32_t magic) { return as_h2((u & mask) | magic); }
 
 __device__ __forceinline__ float dpp_quad_sum(float v) {
     v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
@@ -65,173 +69,225 @@ __device__ __forceinline__ float dpp_quad_sum(float v) {
 //
 // One item = 8 consecutive activations of one batch column ("octet").  Inside a super-block the
 // value index v = 64 g' + 32 high + idx: byte idx of group g', low (high = 0) or high nibble.
-// A lane of the main loop loads the 16-byte chunk c = 2 g' + idx / 16 and turns it into four
-// octets q = 2 high + (idx % 16) / 8; chunk c is handled at step t = c / 4 by lane group
-// g = c % 4.  Within an octet the code bytes come out in the order (0, 2, 1, 3, 4, 6, 5, 7).
-__device__ __forceinline__ void stage_x(const float *__restrict__ X, int M, int K, int m0, int k0, uint8_t *lds, int tid) {
-    constexpr int kItems = kMT * (kSliceK / 8);  // 8192
-    constexpr int kBatch = 4;
-    for (int base = 0; base < kItems; base += 512 * kBatch) {
-        float4 lo[kBatch], hi[kBatch];
+// The main loop loads the 16-byte chunk c = 2 g' + idx / 16 and turns it into four octets
+// q = 2 high + (idx % 16) / 8, the code bytes inside an octet coming out in the order
+// (0, 2, 1, 3, 4, 6, 5, 7).  Octet (sbl, c, q) of column m lives in slot (8 sbl + c) * 4 + q at
+// column position m ^ (slot & 15): consecutive threads hold consecutive octets of ONE column,
+// i.e. different slots with the same m, and the xor spreads their 16-byte stores (and the 32
+// columns a half-wave later reads from one slot) over all LDS banks.
+// The eight sub-block sums of (sbl, m) are stored in the order (0, 2, 1, 3, 4, 6, 5, 7) too.
+template <int ROUNDS>
+__device__ __forceinline__ void stage_x(const float *__restrict__ X, int M, int K, int m0, int k0, uint8_t *__restrict__ lds, int tid,
+                                        int round0) {
+    const int oct = tid & 255;  // fixed per thread; its items are columns (tid >> 8) + 2 r
+    const int k = k0 + 8 * oct;
+    const int sbl = oct >> 5, v8 = oct & 31;
+    const int gp = v8 >> 3, w8 = v8 & 7, high = w8 >> 2, idx8 = w8 & 3;
+    const int q = high * 2 + (idx8 & 1), c = 2 * gp + (idx8 >> 1);
+    const int slot = (sbl * 8 + c) * 4 + q, swz = slot & 15;
+    const int j = 2 * gp + high;
+    const int jpos = (j & 4) | ((j & 1) << 1) | ((j >> 1) & 1);
+    uint8_t *xf_base = lds + slot * (kMT * 16);
+    uint8_t *xs_base = lds + kXFBytes + sbl * (kMT * 16) + jpos * 2;
+    const bool k_ok = k < K;
+    const float *src = X + min(k, K - 8);
+    float4 lo[ROUNDS], hi[ROUNDS];
 #pragma unroll
-        for (int r = 0; r < kBatch; r++) {
-            const int i = base + r * 512 + tid;
-            const int m = i >> 8, oct = i & 255;
-            const int k = k0 + 8 * oct;
-            const bool ok = (m0 + m < M) && (k < K);
-            const float4 *p = reinterpret_cast<const float4 *>(X + (int64_t)min(m0 + m, M - 1) * K + min(k, K - 8));
-            const float4 a = p[0], b = p[1];
-            lo[r] = ok ? a : make_float4(0.f, 0.f, 0.f, 0.f);
-            hi[r] = ok ? b : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
+    for (int r = 0; r < ROUNDS; r++) {
+        const int m = (tid >> 8) + 2 * (round0 + r);
+        const float4 *p = reinterpret_cast<const float4 *>(src + (int64_t)min(m0 + m, M - 1) * K);
+        lo[r] = p[0];
+        hi[r] = p[1];
+    }
 #pragma unroll
-        for (int r = 0; r < kBatch; r++) {
-            const int i = base + r * 512 + tid;
-            const int m = i >> 8, oct = i & 255;
-            const int sbl = oct >> 5, v8 = oct & 31;
-            const int gp = v8 >> 3, w8 = v8 & 7, high = w8 >> 2, idx8 = w8 & 3;
-            const int q = high * 2 + (idx8 & 1);
-            const int c = 2 * gp + (idx8 >> 1);
-            const int t = c >> 2, g = c & 3;
-            const float4 a = lo[r], b = hi[r];
-            uint4 o;  // bytes (0,2,1,3,4,6,5,7)
-            o.x = pack_h2(a.x, a.z);
-            o.y = pack_h2(a.y, a.w);
-            o.z = pack_h2(b.x, b.z);
-            o.w = pack_h2(b.y, b.w);
-            *reinterpret_cast<uint4 *>(lds + ((((sbl * 2 + t) * 4 + q) * 4 + g) * kMT + m) * 16) = o;
-            float s = ((a.x + a.y) + (a.z + a.w)) + ((b.x + b.y) + (b.z + b.w));
-            s = dpp_quad_sum(s);  // the four octets of one 32-value sub-block sit in one quad
-            if ((oct & 3) == 0) {
-                const int j = 2 * gp + high;
-                const int gsel = (j >> 1) & 1, pos = (j & 1) + 2 * (j >> 2);
-                *reinterpret_cast<_Float16 *>(lds + kXFBytes + (((sbl * 2 + gsel) * kMT + m) * 4 + pos) * 2) = (_Float16)s;
-            }
-        }
+    for (int r = 0; r < ROUNDS; r++) {
+        const int m = (tid >> 8) + 2 * (round0 + r);
+        const bool ok = k_ok && (m0 + m < M);
+        const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+        const float4 a = ok ? lo[r] : z, b = ok ? hi[r] : z;
+        uint4 o;  // bytes (0,2,1,3,4,6,5,7)
+        o.x = pack_h2(a.x, a.z);
+        o.y = pack_h2(a.y, a.w);
+        o.z = pack_h2(b.x, b.z);
+        o.w = pack_h2(b.y, b.w);
+        *reinterpret_cast<uint4 *>(xf_base + (m ^ swz) * 16) = o;
+        float sum = ((a.x + a.y) + (a.z + a.w)) + ((b.x + b.y) + (b.z + b.w));
+        sum = dpp_quad_sum(sum);  // the four octets of one 32-value sub-block sit in one quad
+        if (idx8 == 0) *reinterpret_cast<_Float16 *>(xs_base + m * 16) = (_Float16)sum;
     }
 }
 
-struct RawSB { uint4 hd, c0, c1; };  // header + this lane's chunk at step 0 and step 1
+struct RawSB { uint4 hd, c[4]; };  // header + this lane's four chunks (steps 0..3)
 
-__device__ __forceinline__ void load_sb(RawSB &r, const uint8_t *sb, int g) {
+__device__ __forceinline__ void load_sb(RawSB &r, const uint8_t *sb, int kg) {
     r.hd = *reinterpret_cast<const uint4 *>(sb);
-    r.c0 = *reinterpret_cast<const uint4 *>(sb + 16 + 16 * g);
-    r.c1 = *reinterpret_cast<const uint4 *>(sb + 16 + 64 + 16 * g);
+#pragma unroll
+    for (int st = 0; st < 4; st++) r.c[st] = *reinterpret_cast<const uint4 *>(sb + 16 + 32 * st + 16 * kg);
+}
+
+#ifdef GQ_MMQ_TRACE
+__device__ unsigned long long g_mmq_trace[4096 * 8];
+#define MMQ_TRACE(k) do { if (lane == 0) g_mmq_trace[(((size_t)blockIdx.y * gridDim.x + blockIdx.x) * (4 * kParts) + wave) % 4096 * 8 + (k)] = (k) >= 6 ? __builtin_amdgcn_s_memrealtime() : __builtin_readcyclecounter(); } while (0)
+#else
+#define MMQ_TRACE(k) do { } while (0)
+#endif
+
+// Activation pre-pass: writes each (K-slice, column tile)'s LDS image (fragment-ordered fp16
+// activations + sub-block sums) to global memory once; the row-range workgroups of the main
+// kernel then only copy 132 KiB each instead of converting it again.  grid = (slices, column
+// tiles, 8): each workgroup converts four of the tile's 32 columns.
+__global__ __launch_bounds__(512) void mmq_xprep_kernel(const float *__restrict__ X, uint8_t *__restrict__ ximg, int M, int K) {
+    const int slice = blockIdx.x, mt = blockIdx.y;
+    stage_x<2>(X, M, K, mt * kMT, slice * kSliceK, ximg + ((size_t)mt * gridDim.x + slice) * kLdsBytes, threadIdx.x,
+               2 * blockIdx.z);
 }
 
 // partial[slice][m][n] = sum over the slice's k of x[m][k] * w[n][k]
-__global__ __launch_bounds__(512) void mmq_q4k_kernel(const float *__restrict__ X, const uint8_t *__restrict__ W,
+//
+// 4 * kParts wavefronts: wavefront w contracts row tile (w & 3) (32 rows of W) over the
+// super-blocks (w >> 2), (w >> 2) + kParts, ... of the slice; the partial tiles meet in LDS at the end.  v_mfma_f32_32x32x16_f16 with
+// A = activations (32 batch columns x 16 k) and B = weights (16 k x 32 rows): one 16-byte LDS
+// read per lane feeds 16384 multiply-adds, and a lane's 16 results all belong to its own row.
+__global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__restrict__ ximg, const uint8_t *__restrict__ W,
                                                       float *__restrict__ partial, int M, int K, int N,
                                                       int64_t row_bytes, int m0) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int g = lane >> 4, col = lane & 15;
+    const int kg = lane >> 5, col = lane & 31;
+    const int rt = wave & 3, par = wave >> 2;  // par = 0 .. kParts-1
     const int slice = blockIdx.y;
     const int k0 = slice * kSliceK;
     const int nsb = min(kSliceSB, (K - k0) >> 8);
-    const int n = blockIdx.x * kRowsPerWG + wave * 16 + col;  // this lane's weight row
+    const int n = blockIdx.x * kRowsPerWG + rt * 32 + col;  // this lane's weight row
     const uint8_t *wrow = W + (int64_t)min(n, N - 1) * row_bytes + (int64_t)(k0 >> 8) * 144;
 
-    RawSB cur, nxt;
-    load_sb(cur, wrow, g);
-    stage_x(X, M, K, m0, k0, lds, tid);
+    MMQ_TRACE(0);
+    MMQ_TRACE(6);
+    // the slice's activation image goes straight from global memory into LDS (no registers)
+    {
+        const uint8_t *img = ximg + ((size_t)(m0 / kMT) * gridDim.y + slice) * kLdsBytes;
+        for (int i = wave; i < kLdsBytes / 1024; i += 4 * kParts)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(img + i * 1024 + lane * 16),
+                                             (__attribute__((address_space(3))) void *)(lds + i * 1024), 16, 0, 0);
+    }
+    RawSB cur;
+    load_sb(cur, wrow + (int64_t)min(par, nsb - 1) * 144, kg);
+    MMQ_TRACE(1);
     __syncthreads();
+    MMQ_TRACE(2);
 
-    f4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-    const uint8_t *xf = lds + (g * kMT + col) * 16;   // + ((sbl*2+t)*4+q) * (4*kMT*16) + half*256
-    const uint8_t *xs = lds + kXFBytes + ((g >> 1) * kMT + col) * 8;  // + sbl * (2*kMT*8) + half*128
+    f16v acc, acc2;
+#pragma unroll
+    for (int r = 0; r < 16; r++) { acc[r] = 0.f; acc2[r] = 0.f; }
+    uint32_t magic;
+    asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));
 
-    for (int sbl = 0; sbl < nsb; sbl++) {
-        load_sb(nxt, wrow + (int64_t)min(sbl + 1, nsb - 1) * 144, g);
+    for (int sbl = par; sbl < nsb; sbl += kParts) {
+        RawSB nxt;
+        load_sb(nxt, wrow + (int64_t)min(sbl + kParts, nsb - 1) * 144, kg);
         const float d = half_bits_to_float(cur.hd.x & 0xFFFFu), dmin = half_bits_to_float(cur.hd.x >> 16);
         // all eight 6-bit scales / minima as bytes: sc0..3, sc4..7, m0..3, m4..7
         const uint32_t a = cur.hd.y, b = cur.hd.z, c = cur.hd.w;
         const uint32_t sc_lo = a & 0x3F3F3F3Fu, mn_lo = b & 0x3F3F3F3Fu;
         const uint32_t sc_hi = (c & 0x0F0F0F0Fu) | ((a >> 2) & 0x30303030u);
         const uint32_t mn_hi = ((c >> 4) & 0x0F0F0F0Fu) | ((b >> 2) & 0x30303030u);
-        f4 p1[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+        f16v p1;
 #pragma unroll
-        for (int t = 0; t < 2; t++) {
-            // chunk 4t+g: group g' = 2t + g/2, sub-blocks j0 = 2g' (low nibbles), j0+1 (high nibbles)
-            const uint32_t scw = (t == 0 ? sc_lo : sc_hi) >> (16 * (g >> 1));
+        for (int r = 0; r < 16; r++) p1[r] = 0.f;
+        // all sixteen activation fragments of this super-block are requested up front so that the
+        // LDS latency hides behind the code conversion below
+        h8 xfr[16];
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const int slot = (sbl * 8 + 2 * (i >> 2) + kg) * 4 + (i & 3);
+            xfr[i] = *reinterpret_cast<const h8 *>(lds + (slot * kMT + (col ^ (slot & 15))) * 16);
+        }
+#pragma unroll
+        for (int st = 0; st < 4; st++) {
+            // chunk 2 st + kg lies in group st: sub-block 2 st in the low nibbles, 2 st + 1 in the high ones
+            const uint32_t scw = (st < 2 ? sc_lo : sc_hi) >> (16 * (st & 1));
             const float s0f = (float)(scw & 0xFFu), s1f = (float)((scw >> 8) & 0xFFu);
             const h2 s0 = as_h2(pack_h2(s0f, s0f));
             const h2 s1 = as_h2(pack_h2(s1f * 0.0625f, s1f * 0.0625f));  // high-nibble pairs arrive as 1024 + 16 n
             const h2 k0h = as_h2(pack_h2(-1024.f * s0f, -1024.f * s0f));
             const h2 k1h = as_h2(pack_h2(-64.f * s1f, -64.f * s1f));
-            const uint4 ch = t == 0 ? cur.c0 : cur.c1;
-            const uint32_t dw[4] = {ch.x, ch.y, ch.z, ch.w};
+            const uint32_t dw[4] = {cur.c[st].x, cur.c[st].y, cur.c[st].z, cur.c[st].w};
             uint32_t wl[8], wh[8];
 #pragma unroll
             for (int w = 0; w < 4; w++) {
                 const uint32_t u = dw[w], v = dw[w] >> 8;
-                wl[2 * w] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(u, 0x000F000Fu), s0, k0h));
-                wl[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(v, 0x000F000Fu), s0, k0h));
-                wh[2 * w] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(u, 0x00F000F0u), s1, k1h));
-                wh[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(v, 0x00F000F0u), s1, k1h));
+                wl[2 * w] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(u, 0x000F000Fu, magic), s0, k0h));
+                wl[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(v, 0x000F000Fu, magic), s0, k0h));
+                wh[2 * w] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(u, 0x00F000F0u, magic), s1, k1h));
+                wh[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(v, 0x00F000F0u, magic), s1, k1h));
             }
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 const uint32_t *src = (q < 2 ? wl : wh) + 4 * (q & 1);
-                const uint4 wv = make_uint4(src[0], src[1], src[2], src[3]);
-                const h8 wfrag = __builtin_bit_cast(h8, wv);
-                const uint8_t *xp = xf + ((sbl * 2 + t) * 4 + q) * (4 * kMT * 16);
-#pragma unroll
-                for (int h = 0; h < 2; h++) {
-                    const h8 xfrag = *reinterpret_cast<const h8 *>(xp + h * 256);
-                    p1[h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xfrag, wfrag, p1[h], 0, 0, 0);
-                }
+                const h8 wfrag = __builtin_bit_cast(h8, make_uint4(src[0], src[1], src[2], src[3]));
+                p1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xfr[4 * st + q], wfrag, p1, 0, 0, 0);
             }
         }
-        // minima: lane groups 0 and 2 carry (m0,m1,m4,m5) and (m2,m3,m6,m7) against the matching sums
-        uint4 mv = make_uint4(0u, 0u, 0u, 0u);
-        if ((g & 1) == 0) {
-            const int sh = 16 * (g >> 1);
-            const uint32_t lo2 = mn_lo >> sh, hi2 = mn_hi >> sh;
-            mv.x = pack_h2((float)(lo2 & 0xFFu), (float)((lo2 >> 8) & 0xFFu));
-            mv.y = pack_h2((float)(hi2 & 0xFFu), (float)((hi2 >> 8) & 0xFFu));
+        // minima: k-group 0 carries dmin * (m0, m2, m1, m3, m4, m6, m5, m7) against the sums in the same order
+        uint4 mv = make_uint4(0u, 0u, 0u, 0u), sv = make_uint4(0u, 0u, 0u, 0u);
+        if (kg == 0) {
+            const h2 off = as_h2(0xE400E400u);  // (-1024, -1024)
+            const _Float16 dmh = (_Float16)dmin;
+            h2 dm2;
+            dm2.x = dmh;
+            dm2.y = dmh;
+            mv.x = __builtin_bit_cast(uint32_t, (magic_pair(mn_lo, 0x00FF00FFu, magic) + off) * dm2);
+            mv.y = __builtin_bit_cast(uint32_t, (magic_pair(mn_lo >> 8, 0x00FF00FFu, magic) + off) * dm2);
+            mv.z = __builtin_bit_cast(uint32_t, (magic_pair(mn_hi, 0x00FF00FFu, magic) + off) * dm2);
+            mv.w = __builtin_bit_cast(uint32_t, (magic_pair(mn_hi >> 8, 0x00FF00FFu, magic) + off) * dm2);
+            sv = *reinterpret_cast<const uint4 *>(lds + kXFBytes + (sbl * kMT + col) * 16);
         }
-        const h8 mfrag = __builtin_bit_cast(h8, mv);
-        f4 p2[2];
+        acc2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, sv), __builtin_bit_cast(h8, mv), acc2, 0, 0, 0);
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
-            uint4 sv = make_uint4(0u, 0u, 0u, 0u);
-            if ((g & 1) == 0) {
-                const uint2 s2 = *reinterpret_cast<const uint2 *>(xs + sbl * (2 * kMT * 8) + h * 128);
-                sv.x = s2.x;
-                sv.y = s2.y;
-            }
-            const f4 zero = {0.f, 0.f, 0.f, 0.f};
-            p2[h] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, sv), mfrag, zero, 0, 0, 0);
-        }
-#pragma unroll
-        for (int h = 0; h < 2; h++)
-#pragma unroll
-            for (int r = 0; r < 4; r++) acc[h][r] = fmaf(d, p1[h][r], fmaf(-dmin, p2[h][r], acc[h][r]));
+        for (int r = 0; r < 16; r++) acc[r] = fmaf(d, p1[r], acc[r]);
         cur = nxt;
     }
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] -= acc2[r];
+    MMQ_TRACE(3);
 
-    // lane holds y[m = 16 h + 4 g + r][n] for its K-slice
-    if (n < N) {
+    // wavefronts 1..kParts-1 of a row tile hand their 32 x 32 partial tiles to wavefront 0 through LDS
+    __syncthreads();
+    float *xch = reinterpret_cast<float *>(lds) + rt * ((kParts - 1) * 16 * 64);
+    if (par > 0) {
 #pragma unroll
-        for (int h = 0; h < 2; h++)
+        for (int r = 0; r < 16; r++) xch[((par - 1) * 16 + r) * 64 + lane] = acc[r];
+    }
+    __syncthreads();
+    MMQ_TRACE(7);
+    if (par == 0 && n < N) {
+        // lane holds y[m = 8 (r / 4) + 4 kg + r % 4][n] for its K-slice
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int m = m0 + 16 * h + 4 * g + r;
-                if (m < M) partial[((int64_t)slice * M + m) * N + n] = acc[h][r];
-            }
+        for (int r = 0; r < 16; r++) {
+            const int m = m0 + 8 * (r >> 2) + 4 * kg + (r & 3);
+            float v = acc[r];
+#pragma unroll
+            for (int p = 0; p < kParts - 1; p++) v += xch[(p * 16 + r) * 64 + lane];
+            if (m < M) partial[((int64_t)slice * M + m) * N + n] = v;
+        }
     }
 }
 
-// y[m][n] = act(sum_s partial[s][m][n] + bias[n])
+// y[m][n] = act(sum_s partial[s][m][n] + bias[n]); N % 4 == 0 is guaranteed by the caller
 __global__ __launch_bounds__(256) void mmq_reduce_kernel(const float *__restrict__ partial, int nslices, int64_t MN, int N,
                                                          const float *__restrict__ bias, int act, float *__restrict__ Y) {
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < MN; i += (int64_t)gridDim.x * 256) {
-        float s = 0.f;
-        for (int k = 0; k < nslices; k++) s += partial[(int64_t)k * MN + i];
-        if (bias) s += bias[i % N];
-        Y[i] = apply_act(act, s);
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= MN) return;
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int k = 0; k < nslices; k++) {
+        const float4 p = *reinterpret_cast<const float4 *>(partial + (int64_t)k * MN + i);
+        s.x += p.x; s.y += p.y; s.z += p.z; s.w += p.w;
     }
+    if (bias) {
+        const float4 b = *reinterpret_cast<const float4 *>(bias + (int)(i % N));
+        s.x += b.x; s.y += b.y; s.z += b.z; s.w += b.w;
+    }
+    *reinterpret_cast<float4 *>(Y + i) = make_float4(apply_act(act, s.x), apply_act(act, s.y), apply_act(act, s.z), apply_act(act, s.w));
 }
 
 // ---- per-stream workspace for the K-slice partial sums -----------------------------------
@@ -259,9 +315,9 @@ int workspace_for(hipStream_t s, size_t bytes, float **out) {
 
 }  // namespace
 
-bool mmq_supported(int type, int64_t M, int64_t K, int64_t N, const void *x) {
-    return type == kQ4_K && M >= 2 && M <= 256 && K % 256 == 0 && N <= (int64_t)INT32_MAX / 2 && K <= INT32_MAX &&
-           (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+bool mmq_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, const void *bias, const void *y) {
+    return type == kQ4_K && M >= 2 && M <= 256 && K % 256 == 0 && N % 4 == 0 && N <= (int64_t)INT32_MAX / 2 && K <= INT32_MAX &&
+           ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(bias) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
 }
 
 int launch_mmq(int type, const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act,
@@ -273,20 +329,26 @@ int launch_mmq(int type, const float *x, int64_t M, int64_t K, const uint8_t *W,
     }();
     if (!lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", kLdsBytes);
     const int nslices = (int)((K + kSliceK - 1) / kSliceK);
-    float *partial = nullptr;
-    if (int rc = workspace_for(s, (size_t)nslices * M * N * sizeof(float), &partial)) return rc;
+    const int mtiles = (int)((M + kMT - 1) / kMT);
+    // workspace: [activation images: mtiles x nslices x kLdsBytes][partial sums: nslices x M x N fp32]
+    const size_t img_bytes = (size_t)mtiles * nslices * kLdsBytes;
+    const size_t part_bytes = (size_t)nslices * M * N * sizeof(float);
+    float *ws = nullptr;
+    if (int rc = workspace_for(s, img_bytes + part_bytes, &ws)) return rc;
+    uint8_t *ximg = reinterpret_cast<uint8_t *>(ws);
+    float *partial = reinterpret_cast<float *>(ximg + img_bytes);
     const int64_t row_bytes = (K / 256) * 144;
+    if (int rc = launch(mmq_xprep_kernel, dim3((unsigned)nslices, (unsigned)mtiles, 8), dim3(512), 0, s, x, ximg, (int)M, (int)K))
+        return rc;
     const dim3 grid((unsigned)((N + kRowsPerWG - 1) / kRowsPerWG), (unsigned)nslices);
     for (int64_t m0 = 0; m0 < M; m0 += kMT) {
-        if (int rc = launch(mmq_q4k_kernel, grid, dim3(512), (size_t)kLdsBytes, s, x, W, partial, (int)M, (int)K, (int)N,
-                            row_bytes, (int)m0))
+        if (int rc = launch(mmq_q4k_kernel, grid, dim3(256 * kParts), (size_t)kLdsBytes, s, (const uint8_t *)ximg, W, partial, (int)M,
+                            (int)K, (int)N, row_bytes, (int)m0))
             return rc;
     }
     const int64_t MN = M * N;
-    int64_t blocks = (MN + 255) / 256;
-    if (blocks > 4096) blocks = 4096;
-    return launch(mmq_reduce_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (const float *)partial, nslices, MN, (int)N, bias,
-                  act, y);
+    return launch(mmq_reduce_kernel, dim3((unsigned)((MN / 4 + 255) / 256)), dim3(256), 0, s, (const float *)partial, nslices, MN,
+                  (int)N, bias, act, y);
 }
 
 }  // namespace gq
