@@ -94,11 +94,22 @@ class Problem:
         for p in self.parts:
             for c in range(1, self.copies):
                 p["W"].append(torch.roll(p["W"][0], shifts=c, dims=0).contiguous())
-        self.stream = torch.cuda.current_stream().cuda_stream
+        # one explicit stream for everything: warm-up, the recorded graph and the timed launches
+        # (per-stream workspaces of the library must exist before a recording starts)
+        self.tstream = torch.cuda.Stream()
+        self.stream = self.tstream.cuda_stream
         torch.cuda.synchronize()
 
     def launch(self, step):
         c = step % self.copies
+        if self.name == "c4":  # the seven independent projections go out as one batched submission
+            from gomlx_amd import _lib
+            descs = (_lib.DenseDesc * len(self.parts))()
+            for d, p in zip(descs, self.parts):
+                d.type, d.act, d.dX, d.M, d.K = p["t"], 0, p["x"].data_ptr(), p["M"], p["K"]
+                d.dW, d.N, d.dBias, d.dY = p["W"][c].data_ptr(), p["N"], None, p["y"].data_ptr()
+            self.check(self.L.gq_qdense_f32_batch(len(self.parts), descs, self.stream))
+            return
         for p in self.parts:
             fn = self.L.gq_qdense_bf16 if self.dtype == "bf16" else self.L.gq_qdense_f32
             self.check(fn(p["t"], p["x"].data_ptr(), p["M"], p["K"], p["W"][c].data_ptr(), p["N"], None, 0,
@@ -111,15 +122,14 @@ class Problem:
         torch.cuda.synchronize()
         graph = None
         if use_graph:
-            side = torch.cuda.Stream()
-            sp = side.cuda_stream
-            saved, self.stream = self.stream, sp
-            self.check(L.gq_graph_begin(sp))
+            if warmup == 0:
+                self.launch(0)  # creates the stream's workspace, if the path needs one
+                torch.cuda.synchronize()
+            self.check(L.gq_graph_begin(self.stream))
             for s in range(steps):
                 self.launch(warmup + s)
             g = ctypes.c_void_p()
-            self.check(L.gq_graph_end(sp, ctypes.byref(g)))
-            self.stream = saved
+            self.check(L.gq_graph_end(self.stream, ctypes.byref(g)))
             graph = g
             if warmup > 0:  # untimed first replay: uploads the graph
                 self.check(L.gq_graph_launch(graph, self.stream))

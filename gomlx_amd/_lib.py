@@ -35,6 +35,7 @@ SIGNATURES = [
     ("gq_sync", _int, [_vp]),
     ("gq_dequantize", _int, [_int, _vp, _i64, _i64, _vp, _vp]),
     ("gq_qdense_f32", _int, [_int, _vp, _i64, _i64, _vp, _i64, _vp, _int, _vp, _vp]),
+    ("gq_qdense_f32_batch", _int, [_int, _vp, _vp]),
     ("gq_qdense_bf16", _int, [_int, _vp, _i64, _i64, _vp, _i64, _vp, _int, _vp, _vp]),
     ("gq_embedding_lookup", _int, [_int, _vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp]),
     ("gq_graph_begin", _int, [_vp]),
@@ -45,6 +46,12 @@ SIGNATURES = [
     ("gq_profile_end", _int, [_pint, ctypes.POINTER(ctypes.c_double)]),
     ("gq_last_error", ctypes.c_char_p, []),
 ]
+
+
+class DenseDesc(ctypes.Structure):
+    """gq_dense_desc of include/gomlx_hipq.h."""
+    _fields_ = [("type", _int), ("act", _int), ("dX", _vp), ("M", _i64), ("K", _i64), ("dW", _vp), ("N", _i64),
+                ("dBias", _vp), ("dY", _vp)]
 
 
 class HipqError(RuntimeError):

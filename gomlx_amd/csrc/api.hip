@@ -250,6 +250,37 @@ int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *d
     return launch_gemm(type, false, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
 }
 
+int gq_qdense_f32_batch(int count, const gq_dense_desc *descs, void *stream) {
+    if (count < 0 || (count > 0 && !descs)) return fail(GQ_ERR_INVALID, "gq_qdense_f32_batch: bad descriptor list");
+    for (int i = 0; i < count; i++) {
+        const gq_dense_desc &d = descs[i];
+        if (int rc = check_dense_args("gq_qdense_f32_batch", d.type, d.dX, d.M, d.K, d.dW, d.N, d.dBias, d.act, d.dY, 4)) return rc;
+    }
+    if (count == 0) return GQ_OK;
+    if (int rc = use_device()) return rc;
+    // merge runs of batch-1 problems of one type that the streaming GEMV handles; the rest go one by one
+    int i = 0;
+    while (i < count) {
+        int j = i;
+        XsBatchItem items[8];
+        while (j < count && j - i < 8 && descs[j].type == descs[i].type && descs[j].M == 1 && descs[j].N > 0 &&
+               gemv_xs_supported(descs[j].type, descs[j].K, descs[j].N, descs[j].dX)) {
+            const gq_dense_desc &d = descs[j];
+            items[j - i] = XsBatchItem{d.dX, (const uint8_t *)d.dW, d.dBias, d.dY, d.K, d.N, d.act};
+            j++;
+        }
+        if (j - i >= 2) {
+            if (int rc = launch_gemv_xs_batch(descs[i].type, j - i, items, (hipStream_t)stream)) return rc;
+            i = j;
+            continue;
+        }
+        const gq_dense_desc &d = descs[i];
+        if (int rc = gq_qdense_f32(d.type, d.dX, d.M, d.K, d.dW, d.N, d.dBias, d.act, d.dY, stream)) return rc;
+        i++;
+    }
+    return GQ_OK;
+}
+
 int gq_qdense_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, const void *dW, int64_t N,
                    const float *dBias, int act, float *dY, void *stream) {
     if (int rc = check_dense_args("gq_qdense_bf16", type, dX, M, K, dW, N, dBias, act, dY, 2)) return rc;

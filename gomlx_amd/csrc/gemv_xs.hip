@@ -336,18 +336,17 @@ template <> struct JointSum<2> {
 // activations then leaves the code loads in flight while the digit planes are being built.
 #ifdef GQ_XS_TRACE
 __device__ unsigned long long g_xs_trace[4096 * 16];
-#define XS_TRACE(k) do { if (lane == 0) g_xs_trace[((size_t)blockIdx.x * (blockDim.x >> 6) + wave) % 4096 * 16 + (k)] = __builtin_readcyclecounter(); } while (0)
-#define XS_TRACE_WALL(k) do { if (lane == 0) g_xs_trace[((size_t)blockIdx.x * (blockDim.x >> 6) + wave) % 4096 * 16 + (k)] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#define XS_TRACE(k) do { if (lane == 0) g_xs_trace[((size_t)wg * (blockDim.x >> 6) + wave) % 4096 * 16 + (k)] = __builtin_readcyclecounter(); } while (0)
+#define XS_TRACE_WALL(k) do { if (lane == 0) g_xs_trace[((size_t)wg * (blockDim.x >> 6) + wave) % 4096 * 16 + (k)] = __builtin_amdgcn_s_memrealtime(); } while (0)
 #else
 #define XS_TRACE(k) do { } while (0)
 #define XS_TRACE_WALL(k) do { } while (0)
 #endif
 
-template <int T, int PF, int MAXT>
-__global__ __launch_bounds__(MAXT) void gemv_xs_kernel(const float *__restrict__ X, const uint8_t *__restrict__ W,
-                                                       const float *__restrict__ bias, float *__restrict__ Y, int K,
-                                                       int N, int64_t row_bytes, int S, int iters, int act) {
-    extern __shared__ uint32_t lds[];
+template <int T, int PF>
+__device__ __forceinline__ void gemv_xs_body(const float *__restrict__ x, const uint8_t *__restrict__ W,
+                                             const float *__restrict__ bias, float *__restrict__ y, int K, int N,
+                                             int64_t row_bytes, int S, int iters, int act, int wg, uint32_t *lds) {
     typedef typename XS<T>::Raw Raw;
     typedef typename XS<T>::Item Item;
     constexpr int NX = XS<T>::kX;
@@ -358,9 +357,7 @@ __global__ __launch_bounds__(MAXT) void gemv_xs_kernel(const float *__restrict__
     const int nunits = K >> 6;
     const int u = slice * 64 + lane;
     const bool have_unit = u < nunits;
-    const int first = (blockIdx.x * G + g) * iters;  // this wavefront's rows: first .. first + iters - 1
-    const float *x = X + (int64_t)blockIdx.y * K;
-    float *y = Y + (int64_t)blockIdx.y * N;
+    const int first = (wg * G + g) * iters;  // this wavefront's rows: first .. first + iters - 1
     constexpr bool aligned = true;
     const int nitems = K >> XS<T>::kItemShift;
 
@@ -476,6 +473,43 @@ __global__ __launch_bounds__(MAXT) void gemv_xs_kernel(const float *__restrict__
     }
 }
 
+template <int T, int PF, int MAXT>
+__global__ __launch_bounds__(MAXT) void gemv_xs_kernel(const float *__restrict__ X, const uint8_t *__restrict__ W,
+                                                       const float *__restrict__ bias, float *__restrict__ Y, int K,
+                                                       int N, int64_t row_bytes, int S, int iters, int act) {
+    extern __shared__ uint32_t lds[];
+    gemv_xs_body<T, PF>(X + (int64_t)blockIdx.y * K, W, bias, Y + (int64_t)blockIdx.y * N, K, N, row_bytes, S, iters, act,
+                        (int)blockIdx.x, lds);
+}
+
+// Several independent batch-1 problems of one format in a single launch: workgroups
+// [wg_begin, next wg_begin) belong to problem i.  This is how the projections of a decoder
+// layer that do not depend on each other (q/k/v, gate/up) share one submission.
+constexpr int kMaxBatch = 8;
+struct XsProblem {
+    const float *x;
+    const uint8_t *W;
+    const float *bias;
+    float *y;
+    int64_t row_bytes;
+    int K, N, S, iters, act, wg_begin;
+};
+struct XsBatch {
+    int count;
+    XsProblem p[kMaxBatch];
+};
+
+template <int T, int PF, int MAXT>
+__global__ __launch_bounds__(MAXT) void gemv_xs_batch_kernel(const XsBatch b) {
+    extern __shared__ uint32_t lds[];
+    int i = 0;
+#pragma unroll
+    for (int j = 1; j < kMaxBatch; j++)
+        if (j < b.count && (int)blockIdx.x >= b.p[j].wg_begin) i = j;
+    const XsProblem &q = b.p[i];
+    gemv_xs_body<T, PF>(q.x, q.W, q.bias, q.y, q.K, q.N, q.row_bytes, q.S, q.iters, q.act, (int)blockIdx.x - q.wg_begin, lds);
+}
+
 struct Plan { int waves, S, G, wgs, iters; };
 
 // Picks workgroup size, slices and grid.  GOMLX_HIPQ_GEMV_XS="wgs_per_cu,waves" overrides the
@@ -494,7 +528,7 @@ Plan make_plan(int64_t K, int64_t N, int max_waves) {
     while ((int64_t)p.waves * 64 * 32 < K) p.waves <<= 1;  // staging: at most K / 32 threads' worth of items
     p.G = p.waves / S;
     const int cus = device_cu_count();
-    const int64_t target_wgs = (int64_t)cus * (env_wgs ? env_wgs : (16 / p.waves > 0 ? 16 / p.waves : 1));
+    const int64_t target_wgs = (int64_t)cus * (env_wgs ? env_wgs : 1);  // one workgroup per CU measured best
     int64_t slots = target_wgs * p.G;
     int64_t iters = (N + slots - 1) / slots;
     if (iters < 1) iters = 1;
@@ -528,7 +562,64 @@ int launch_depth(const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t
     return launch_xs<T, PFMAX, 512>(p, x, M, K, W, N, bias, act, y, s);
 }
 
+template <int T>
+size_t xs_lds_bytes(int64_t K, int waves) {
+    size_t shmem = (size_t)(T == kQ4_0 ? kNibDwords : kLimbDwords) * (size_t)(K >> 6) * sizeof(uint32_t);
+    const size_t part_bytes = (size_t)waves * 64 * sizeof(float);
+    return shmem < part_bytes ? part_bytes : shmem;
+}
+
+// One launch for `count` batch-1 problems: the chip's workgroup slots are shared out in proportion
+// to each problem's weight bytes, so every CU streams for about the same time.
+template <int T>
+int launch_xs_batch(int count, const XsProblem *in, hipStream_t s) {
+    XsBatch b;
+    b.count = count;
+    const int cus = device_cu_count();
+    double total = 0.0;
+    for (int i = 0; i < count; i++) total += (double)in[i].row_bytes * in[i].N;
+    size_t shmem = 0;
+    int wg = 0;
+    for (int i = 0; i < count; i++) {
+        XsProblem q = in[i];
+        int S = 1;
+        while (S * 64 < (q.K >> 6)) S <<= 1;
+        const int waves = 8, G = waves / S;
+        int64_t share = (int64_t)((double)cus * ((double)q.row_bytes * q.N) / total + 0.5);
+        if (share < 1) share = 1;
+        int64_t iters = (q.N + share * G - 1) / (share * G);
+        if (iters < 1) iters = 1;
+        if (iters > 64) iters = 64;
+        q.S = S;
+        q.iters = (int)iters;
+        q.wg_begin = wg;
+        wg += (int)((q.N + iters * G - 1) / (iters * G));
+        b.p[i] = q;
+        const size_t need = xs_lds_bytes<T>(q.K, waves);
+        if (need > shmem) shmem = need;
+    }
+    return launch(gemv_xs_batch_kernel<T, 4, 512>, dim3((unsigned)wg), dim3(512), shmem, s, b);
+}
+
 }  // namespace
+
+int launch_gemv_xs_batch(int type, int count, const XsBatchItem *items, hipStream_t s) {
+    if (count < 1 || count > kMaxBatch) return fail(GQ_ERR_INVALID, "gemv batch: %d problems (1..%d supported per launch)", count, kMaxBatch);
+    XsProblem p[kMaxBatch];
+    for (int i = 0; i < count; i++) {
+        const XsBatchItem &it = items[i];
+        p[i].x = it.x; p[i].W = it.W; p[i].bias = it.bias; p[i].y = it.y;
+        p[i].K = (int)it.K; p[i].N = (int)it.N; p[i].act = it.act;
+        p[i].row_bytes = (int64_t)gq_row_bytes(type, it.K);
+        p[i].S = p[i].iters = p[i].wg_begin = 0;
+    }
+    switch (type) {
+    case kQ4_0: return launch_xs_batch<kQ4_0>(count, p, s);
+    case kQ8_0: return launch_xs_batch<kQ8_0>(count, p, s);
+    case kQ4_K: return launch_xs_batch<kQ4_K>(count, p, s);
+    default: return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv batch: ggml type %d is not implemented", type);
+    }
+}
 
 bool gemv_xs_supported(int type, int64_t K, int64_t N, const void *x) {
     if (reinterpret_cast<uintptr_t>(x) & 15) return false;

@@ -165,3 +165,43 @@ def quantized_gather(table: torch.Tensor, indices: torch.Tensor, quant: Quantiza
     if count and int(flag.item()):
         raise IndexError("quantized_gather: index out of range")
     return out
+
+
+def quantized_dense_batch(problems) -> list:
+    """Several independent nn.QuantizedDense calls submitted together (gq_qdense_f32_batch).
+
+    ``problems`` is a sequence of ``(x, weights, quant, bias, activation)`` tuples with float32
+    activations; returns the list of outputs.  Results equal those of separate calls; batch-1
+    problems of one GGML type share a single kernel launch.
+    """
+    import ctypes
+    L = _lib.lib()
+    descs = (_lib.DenseDesc * len(problems))()
+    outs = []
+    for i, (x, weights, quant, bias, act) in enumerate(problems):
+        act = Activation.NONE if act is None else act
+        if quant is None or quant.scheme != QuantizationScheme.GGML:
+            raise _lib.NotImplementedByBackend(_lib.ERR_NOT_IMPLEMENTED, "only the GGML scheme is on this path")
+        _require_cuda("x", x)
+        _require_cuda("weights", weights)
+        _weights_2d(weights)
+        if x.dtype != torch.float32:
+            raise _lib.NotImplementedByBackend(_lib.ERR_NOT_IMPLEMENTED, "batched submission takes float32 activations")
+        N, rb = weights.shape
+        K_in = x.shape[-1]
+        M = x.numel() // K_in if K_in else 0
+        blen = -1
+        if bias is not None:
+            _require_cuda("bias", bias)
+            blen = bias.shape[0]
+        K = ctypes.c_int64(0)
+        _lib.check(L.gq_qdense_check(quant.ggml_type, _lib.F32, M, K_in, N, rb, blen, act.to_backend(), ctypes.byref(K)))
+        y = torch.empty(x.shape[:-1] + (N,), dtype=torch.float32, device=x.device)
+        outs.append(y)
+        d = descs[i]
+        d.type, d.act, d.dX, d.M, d.K = quant.ggml_type, act.to_backend(), x.data_ptr(), M, K.value
+        d.dW, d.N, d.dBias, d.dY = weights.data_ptr(), N, (None if bias is None else bias.data_ptr()), y.data_ptr()
+    if problems:
+        _lib.init(problems[0][0].device.index or 0)
+        _lib.check(L.gq_qdense_f32_batch(len(problems), descs, _stream_ptr(problems[0][0])))
+    return outs

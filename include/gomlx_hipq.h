@@ -102,6 +102,23 @@ int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *d
 int gq_qdense_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, const void *dW,
                    int64_t N, const float *dBias, int act, float *dY, void *stream);
 
+/* ---- Several FusedQuantizedDense nodes of one compiled graph that do not depend on each other
+ * (e.g. the q/k/v or gate/up projections of a decoder layer) submitted together: the work an
+ * Executable.Execute (core/graph/graph.go:669) is free to overlap.  Equivalent to calling
+ * gq_qdense_f32 once per descriptor, in any order; outputs must not alias any input.  Batch-1
+ * problems of one GGML type are merged into a single launch. ---- */
+typedef struct {
+    int type;            /* gq_type */
+    int act;             /* gq_act */
+    const float *dX;     /* [M, K] */
+    int64_t M, K;
+    const void *dW;      /* [N, gq_row_bytes(type, K)] */
+    int64_t N;
+    const float *dBias;  /* [N] or NULL */
+    float *dY;           /* [M, N] */
+} gq_dense_desc;
+int gq_qdense_f32_batch(int count, const gq_dense_desc *descs, void *stream);
+
 /* ---- compute.Function.QuantizedEmbeddingLookup (core/graph/fused_ops.go:295-296;
  * nn.QuantizedGather ml/nn/quantized_gather.go:30-43; ml/ggml/gather.go:21-49):
  * dOut[i, :] = dequant(dTable[dIndices[i], :]), bit-exact.  An index outside [0, vocab)

@@ -239,6 +239,32 @@ def test_config4_llama_layer_projections(gpu, oracle):
         assert rel_err(run_dense(gpu, Q4_K, x, W), oracle.c_qdense(Q4_K, x, W)) < TOL_F32, (K, N)
 
 
+def test_batched_submission_equals_separate_calls(gpu, oracle):
+    """gq_qdense_f32_batch: the seven projections of a decoder layer (scaled down), mixed with a
+    batch-5 problem and another format, against one call each and against the oracle."""
+    torch = gpu
+    shapes = [(1024, 1024), (1024, 256), (1024, 256), (1024, 1024), (1024, 3584), (1024, 3584), (3584, 1024)]
+    probs, hosts = [], []
+    for i, (K, N) in enumerate(shapes):
+        W = synth.weights(Q4_K, 170 + i, N, K)
+        x = synth.activations(180 + i, 1, K)
+        b = synth.normal(190 + i, 0, N).astype(np.float32) * 0.1 if i % 2 else None
+        act = Activation.SILU if i == 4 else Activation.NONE
+        hosts.append((Q4_K, x, W, b, act))
+    hosts.append((Q4_K, synth.activations(200, 5, 512), synth.weights(Q4_K, 201, 64, 512), None, Activation.NONE))
+    hosts.append((Q8_0, synth.activations(202, 1, 2048), synth.weights(Q8_0, 203, 300, 2048), None, Activation.RELU))
+    hosts.append((Q8_0, synth.activations(204, 1, 2048), synth.weights(Q8_0, 205, 77, 2048), None, Activation.NONE))
+    for t, x, W, b, act in hosts:
+        probs.append((dev(torch, x), dev(torch, W), Quantization(ggml_type=t), None if b is None else dev(torch, b), act))
+    outs = nn.quantized_dense_batch(probs)
+    torch.cuda.synchronize()
+    for (t, x, W, b, act), p, y in zip(hosts, probs, outs):
+        single = nn.quantized_dense(p[0], p[1], p[2], p[3], act)
+        assert torch.equal(single, y)
+        want = oracle.c_qdense(t, x, W, b, act.to_backend())
+        assert rel_err(y.cpu().numpy(), want) < TOL_F32
+
+
 # ------------------------------------------------------------------------------ gather
 
 @pytest.mark.parametrize("t", ALL_TYPES)
