@@ -1,14 +1,19 @@
 // Batched / prefill quantised Dense on the gfx950 matrix cores:
 //   Y[m,n] = act(sum_k X[m,k] * w[n,k] + b[n]),  X [M,K],  W GGML blocks [N, row_bytes].
 //
-// Each workgroup owns a BM x BN tile of Y.  Per 32-wide K step it dequantises its BN x 32
-// slab of W (exact fp32 values, then rounded once to the 16-bit MFMA operand type) into
-// LDS, stages the BM x 32 slab of X beside it, and the wavefronts contract the two slabs
-// with v_mfma_f32_32x32x16 (fp32 accumulation).  Both operands are K-contiguous, which is
-// exactly the A / B fragment shape the instruction wants (8 consecutive k per lane).
+// A workgroup of 8 wavefronts owns a 256 x 128 tile of Y (256 activation rows, 128 weight
+// rows); each wavefront a 64 x 64 sub-tile = 2 x 2 v_mfma_f32_32x32x16 accumulators.  Per
+// 128-wide K step the workgroup dequantises its 128 x 128 slab of W (exact fp32 values, then one
+// rounding to the 16-bit MFMA operand type) and stages the 256 x 128 slab of X next to it in
+// LDS.  Both operands are K-contiguous, which is exactly the A / B fragment shape the
+// instruction wants (8 consecutive k per lane), so fragments are single 16-byte LDS reads from
+// rows padded to 272 bytes (conflict-free).
+//
+// The global loads of step k+1 are issued right after the barrier that publishes step k and
+// wait in registers through the 32 MFMAs per wavefront of step k.
 //
 //   bf16 activations -> bf16 MFMA (the prefill path);
-//   fp32 activations -> rounded to fp16, fp16 MFMA (11-bit operands, small-batch path).
+//   fp32 activations -> rounded to fp16, fp16 MFMA (11-bit operands; generic batched path).
 #include "blocks.hpp"
 #include "common.hpp"
 
@@ -20,15 +25,19 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 128, BN = 128, BK = 32;
-constexpr int LDS_STRIDE = 40;  // 16-bit elements per LDS row: 64 B of data + 16 B pad (conflict-free ds_read_b128)
+constexpr int BM = 256, BN = 128, BK = 128;
+constexpr int LDS_STRIDE = BK + 8;  // 16-bit elements per LDS row: 256 B of data + 16 B pad
+constexpr int LDS_BYTES = (BM + BN) * LDS_STRIDE * 2;
 
 template <bool BF16> struct Operand;
 template <> struct Operand<true> {
     typedef bf16x8 vec8;
-    static __device__ __forceinline__ uint16_t from_float(float f) {
-        const __bf16 b = (__bf16)f;
-        return __builtin_bit_cast(uint16_t, b);
+    static __device__ __forceinline__ uint32_t pack(float a, float b) {
+        typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+        bf2 v;
+        v.x = (__bf16)a;
+        v.y = (__bf16)b;
+        return __builtin_bit_cast(uint32_t, v);
     }
     static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
@@ -36,24 +45,117 @@ template <> struct Operand<true> {
 };
 template <> struct Operand<false> {
     typedef f16x8 vec8;
-    static __device__ __forceinline__ uint16_t from_float(float f) {
-        const _Float16 h = (_Float16)f;
-        return __builtin_bit_cast(uint16_t, h);
+    static __device__ __forceinline__ uint32_t pack(float a, float b) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        h2 v;
+        v.x = (_Float16)a;
+        v.y = (_Float16)b;
+        return __builtin_bit_cast(uint32_t, v);
     }
     static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
     }
 };
 
-__device__ __forceinline__ uint32_t pack2(uint16_t lo, uint16_t hi) { return (uint32_t)lo | ((uint32_t)hi << 16); }
+// ---- raw (still packed) share of one thread in the W slab: one 32-value run of one row ---------
+// Thread (row = t / 4, blk = t % 4) owns weights k0 + 32 blk .. + 31 of its row.
+template <int T> struct WRaw;
 
+template <> struct WRaw<kQ8_0> {
+    uint32_t d;
+    u128_a2 q0, q1;
+    __device__ __forceinline__ void load(const uint8_t *row, int64_t kblk) {
+        const uint8_t *blk = row + kblk * 34;
+        d = load_u16(blk);
+        q0 = *reinterpret_cast<const u128_a2 *>(blk + 2);
+        q1 = *reinterpret_cast<const u128_a2 *>(blk + 18);
+    }
+    // int8 q = (q ^ 0x80) - 128 with the xor-ed byte read as unsigned; fma(u, d, -128 d) = d * q
+    // exactly (the product has at most 18 significant bits), i.e. the reference's f32(d) * f32(q).
+    __device__ __forceinline__ void values(float *w) const {
+        const float df = half_bits_to_float(d), off = -128.0f * df;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const uint32_t a = (i < 4 ? q0.v[i] : q1.v[i - 4]) ^ 0x80808080u;
+            w[4 * i + 0] = fmaf(ubyte0(a), df, off);
+            w[4 * i + 1] = fmaf(ubyte1(a), df, off);
+            w[4 * i + 2] = fmaf(ubyte2(a), df, off);
+            w[4 * i + 3] = fmaf(ubyte3(a), df, off);
+        }
+    }
+};
+
+// Other formats: keep the position and decode through the exact 16-value helper at store time.
+template <int T> struct WRaw {
+    const uint8_t *row;
+    int64_t i16;
+    __device__ __forceinline__ void load(const uint8_t *r, int64_t kblk) {
+        row = r;
+        i16 = kblk * 2;
+    }
+    __device__ __forceinline__ void values(float *w) const {
+        dequant16<T>(row, i16, w);
+        dequant16<T>(row, i16 + 1, w + 16);
+    }
+};
+
+// The 256 x 128 activation slab as 16-byte chunks, chunk-major over the 512 threads: chunk
+// g = 512 j + t (j-th load of thread t) is chunk g % CPR of row g / CPR, so consecutive lanes read
+// consecutive 16 bytes of one row (a wavefront covers 4 full rows = 8 cache lines per load
+// instead of 64 lines with a row-per-lane assignment, which leaves the kernel bound by the
+// texture addresser).
+template <bool BF16> struct XRaw;
+template <> struct XRaw<true> {
+    static constexpr int CPR = 16, NCH = 8;  // chunks per row (8 bf16 each), chunks per thread
+    uint4 v[NCH];
+    __device__ __forceinline__ void load(const void *X, int bm, int M, int k0, int K, int tid) {
+        const uint16_t *p = reinterpret_cast<const uint16_t *>(X);
+#pragma unroll
+        for (int j = 0; j < NCH; j++) {
+            const int g = 512 * j + tid, row = g / CPR, k = k0 + (g % CPR) * 8;
+            v[j] = *reinterpret_cast<const uint4 *>(p + (int64_t)min(bm + row, M - 1) * K + (k < K ? k : 0));
+        }
+    }
+    __device__ __forceinline__ void store(uint16_t *xs, int bm, int M, int k0, int K, int tid) const {
+#pragma unroll
+        for (int j = 0; j < NCH; j++) {
+            const int g = 512 * j + tid, row = g / CPR, c = g % CPR;
+            const bool ok = bm + row < M && k0 + c * 8 < K;
+            *reinterpret_cast<uint4 *>(xs + row * LDS_STRIDE + c * 8) = ok ? v[j] : make_uint4(0, 0, 0, 0);
+        }
+    }
+};
+template <> struct XRaw<false> {
+    static constexpr int CPR = 32, NCH = 16;  // chunks per row (4 fp32 each), chunks per thread
+    float4 v[NCH];
+    __device__ __forceinline__ void load(const void *X, int bm, int M, int k0, int K, int tid) {
+        const float *p = reinterpret_cast<const float *>(X);
+#pragma unroll
+        for (int j = 0; j < NCH; j++) {
+            const int g = 512 * j + tid, row = g / CPR, k = k0 + (g % CPR) * 4;
+            v[j] = *reinterpret_cast<const float4 *>(p + (int64_t)min(bm + row, M - 1) * K + (k < K ? k : 0));
+        }
+    }
+    __device__ __forceinline__ void store(uint16_t *xs, int bm, int M, int k0, int K, int tid) const {
+#pragma unroll
+        for (int j = 0; j < NCH; j++) {
+            const int g = 512 * j + tid, row = g / CPR, c = g % CPR;
+            const bool ok = bm + row < M && k0 + c * 4 < K;
+            const uint2 h = make_uint2(Operand<false>::pack(v[j].x, v[j].y), Operand<false>::pack(v[j].z, v[j].w));
+            *reinterpret_cast<uint2 *>(xs + row * LDS_STRIDE + c * 4) = ok ? h : make_uint2(0, 0);
+        }
+    }
+};
+
+// X must be 16-byte aligned; K % 32 == 0.  One LDS stage of BK = 128: the MFMA phase of a step
+// (32 MFMAs per wavefront) is long enough to cover the global-memory latency of the next
+// step's loads, which wait in registers and are converted and stored between two barriers.
 template <int T, bool BF16>
-__global__ __launch_bounds__(256) void gemm_kernel(const void *__restrict__ Xv, const uint8_t *__restrict__ W,
+__global__ __launch_bounds__(512) void gemm_kernel(const void *__restrict__ Xv, const uint8_t *__restrict__ W,
                                                    const float *__restrict__ bias, float *__restrict__ Y, int M, int K,
                                                    int N, int64_t row_bytes, int act) {
     typedef Operand<BF16> Op;
-    __shared__ __attribute__((aligned(16))) uint16_t xs[BM * LDS_STRIDE];
-    __shared__ __attribute__((aligned(16))) uint16_t ws[BN * LDS_STRIDE];
+    extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int bm = blockIdx.y * BM, bn = blockIdx.x * BN;
@@ -67,47 +169,37 @@ __global__ __launch_bounds__(256) void gemm_kernel(const void *__restrict__ Xv, 
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-    // staging role of this thread: row (tid / 2) of the slab, 16-element half (tid % 2)
-    const int srow = tid >> 1, shalf = tid & 1;
-    const int xm = bm + srow, wn_row = bn + srow;
-    const uint8_t *wrow = W + (int64_t)min(wn_row, N - 1) * row_bytes;
+    // staging role for W: 128 rows x 4 runs of 32 weights
+    const int wrow_i = tid >> 2, wblk = tid & 3;
+    const uint8_t *wrow = W + (int64_t)min(bn + wrow_i, N - 1) * row_bytes;
+    uint16_t *wdst = lds + (BM + wrow_i) * LDS_STRIDE + 32 * wblk;
 
-    for (int k0 = 0; k0 < K; k0 += BK) {
-        // ---- X slab -> LDS
-        uint32_t xp[8];
-        if (xm < M) {
-            if constexpr (BF16) {
-                const uint16_t *xr = reinterpret_cast<const uint16_t *>(Xv) + (int64_t)xm * K + k0 + 16 * shalf;
+    XRaw<BF16> xr[1];
+    WRaw<T> wr[1];
+    const int nk = (K + BK - 1) / BK;
+    const int64_t nblk32 = K >> 5;
+    auto fetch = [&](int kt, XRaw<BF16> &x, WRaw<T> &w) {
+        const int k0 = kt * BK;
+        x.load(Xv, bm, M, k0, K, tid);
+        w.load(wrow, min((int64_t)(k0 >> 5) + wblk, nblk32 - 1));
+    };
+    auto stage = [&](int kt, const XRaw<BF16> &x, const WRaw<T> &wq) {
+        const int k0 = kt * BK;
+        x.store(lds, bm, M, k0, K, tid);
+        float w[32];
+        wq.values(w);
+        const bool w_ok = k0 + 32 * wblk < K;
+        uint4 *d = reinterpret_cast<uint4 *>(wdst);
 #pragma unroll
-                for (int j = 0; j < 8; j++) xp[j] = pack2(xr[2 * j], xr[2 * j + 1]);
-            } else {
-                const float *xr = reinterpret_cast<const float *>(Xv) + (int64_t)xm * K + k0 + 16 * shalf;
+        for (int j = 0; j < 4; j++)
+            d[j] = w_ok ? make_uint4(Op::pack(w[8 * j], w[8 * j + 1]), Op::pack(w[8 * j + 2], w[8 * j + 3]),
+                                     Op::pack(w[8 * j + 4], w[8 * j + 5]), Op::pack(w[8 * j + 6], w[8 * j + 7]))
+                        : make_uint4(0, 0, 0, 0);
+    };
+    const uint16_t *xs = lds, *ws = lds + BM * LDS_STRIDE;
+    auto contract = [&]() {
 #pragma unroll
-                for (int j = 0; j < 8; j++) xp[j] = pack2(Op::from_float(xr[2 * j]), Op::from_float(xr[2 * j + 1]));
-            }
-        } else {
-#pragma unroll
-            for (int j = 0; j < 8; j++) xp[j] = 0u;
-        }
-        // ---- W slab: exact fp32 dequantisation, one rounding to the operand type
-        float wv[16];
-        dequant16<T>(wrow, (int64_t)(k0 >> 4) + shalf, wv);
-        uint32_t wp[8];
-#pragma unroll
-        for (int j = 0; j < 8; j++) wp[j] = pack2(Op::from_float(wv[2 * j]), Op::from_float(wv[2 * j + 1]));
-
-        if (k0 > 0) __syncthreads();
-        uint4 *xd = reinterpret_cast<uint4 *>(&xs[srow * LDS_STRIDE + 16 * shalf]);
-        xd[0] = make_uint4(xp[0], xp[1], xp[2], xp[3]);
-        xd[1] = make_uint4(xp[4], xp[5], xp[6], xp[7]);
-        uint4 *wd = reinterpret_cast<uint4 *>(&ws[srow * LDS_STRIDE + 16 * shalf]);
-        wd[0] = make_uint4(wp[0], wp[1], wp[2], wp[3]);
-        wd[1] = make_uint4(wp[4], wp[5], wp[6], wp[7]);
-        __syncthreads();
-
-        // ---- contract: two K=16 MFMA steps over the 32-wide slab
-#pragma unroll
-        for (int kk = 0; kk < 2; kk++) {
+        for (int kk = 0; kk < BK / 16; kk++) {
             const int koff = kk * 16 + (lane >> 5) * 8;
             typename Op::vec8 a[2], b[2];
 #pragma unroll
@@ -121,6 +213,15 @@ __global__ __launch_bounds__(256) void gemm_kernel(const void *__restrict__ Xv, 
 #pragma unroll
                 for (int j = 0; j < 2; j++) acc[i][j] = Op::mfma(a[i], b[j], acc[i][j]);
         }
+    };
+
+    fetch(0, xr[0], wr[0]);
+    for (int kt = 0; kt < nk; kt++) {
+        stage(kt, xr[0], wr[0]);
+        __syncthreads();
+        fetch(min(kt + 1, nk - 1), xr[0], wr[0]);  // unconditional (clamped): in flight during the MFMA phase
+        contract();
+        __syncthreads();
     }
 
     // ---- epilogue: acc[i][j][r] is Y[m, n] with n = lane % 32, m = 8*(r/4) + 4*(lane/32) + r%4
@@ -143,9 +244,15 @@ __global__ __launch_bounds__(256) void gemm_kernel(const void *__restrict__ Xv, 
 template <int T, bool BF16>
 int launch_one(const void *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y,
                hipStream_t s) {
+    static const bool lds_ok = [] {
+        return hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kernel<T, BF16>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) == hipSuccess;
+    }();
+    if (!lds_ok) return fail(GQ_ERR_HIP, "gemm: cannot reserve %d bytes of LDS", LDS_BYTES);
     const int64_t row_bytes = (K / Geom<T>::vpb) * Geom<T>::bpb;
     const dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM));
-    return launch(gemm_kernel<T, BF16>, grid, dim3(256), 0, s, x, W, bias, y, (int)M, (int)K, (int)N, row_bytes, act);
+    return launch(gemm_kernel<T, BF16>, grid, dim3(512), (size_t)LDS_BYTES, s, x, W, bias, y, (int)M, (int)K, (int)N, row_bytes,
+                  act);
 }
 
 template <int T>
@@ -163,6 +270,8 @@ int launch_gemm(int type, bool x_is_bf16, const void *x, int64_t M, int64_t K, c
     if (N > INT32_MAX || K > INT32_MAX || M > INT32_MAX || (M + BM - 1) / BM > 65535)
         return fail(GQ_ERR_NOT_IMPLEMENTED, "gemm: dimensions M=%lld K=%lld N=%lld exceed the kernel's index range",
                     (long long)M, (long long)K, (long long)N);
+    if (reinterpret_cast<uintptr_t>(x) & 15)
+        return fail(GQ_ERR_NOT_IMPLEMENTED, "qdense: batched activations that are not 16-byte aligned are not implemented");
     switch (type) {
     case kQ4_0: return launch_type<kQ4_0>(x_is_bf16, x, M, K, W, N, bias, act, y, s);
     case kQ8_0: return launch_type<kQ8_0>(x_is_bf16, x, M, K, W, N, bias, act, y, s);

@@ -159,6 +159,20 @@ def test_gemv_unaligned_activation_pointer(gpu, oracle):
     assert rel_err(y.cpu().numpy(), oracle.c_qdense(Q4_0, x, W)) < TOL_F32
 
 
+@pytest.mark.parametrize("t", [Q4_0, Q8_0, IQ4_NL])
+@pytest.mark.parametrize("K", [32, 96, 160])
+def test_batched_ragged_k_steps(gpu, oracle, t, K):
+    """K that is not a multiple of the kernels' K step (32-value blocks only)."""
+    M, N = 9, 21
+    W = synth.weights(t, 300 + K, N, K)
+    x = synth.activations(301 + K, M, K)
+    assert rel_err(run_dense(gpu, t, x, W), oracle.c_qdense(t, x, W)) < TOL_F32
+    xb = bf16_round(x)
+    assert rel_err(run_dense(gpu, t, xb, W, bf16=True), oracle.c_qdense(t, xb, W)) < TOL_BF16
+    x1 = x[:1]
+    assert rel_err(run_dense(gpu, t, x1, W), oracle.c_qdense(t, x1, W)) < TOL_F32
+
+
 def test_leading_batch_axes_and_empty_batch(gpu, oracle):
     K, N = 256, 12
     W = synth.weights(Q8_0, 70, N, K)
@@ -173,7 +187,7 @@ def test_leading_batch_axes_and_empty_batch(gpu, oracle):
 # ------------------------------------------------------------------------------ batched (MFMA) paths
 
 @pytest.mark.parametrize("t", ALL_TYPES)
-@pytest.mark.parametrize("M,K,N", [(5, 256, 7), (32, 1024, 130), (130, 512, 257), (64, 4096, 96)])
+@pytest.mark.parametrize("M,K,N", [(5, 256, 7), (32, 1024, 130), (130, 512, 257), (64, 4096, 96), (300, 768, 40)])
 def test_batched_f32_parity(gpu, oracle, t, M, K, N):
     W = synth.weights(t, 80 + t, N, K)
     x = synth.activations(81 + t, M, K)
@@ -185,7 +199,7 @@ def test_batched_f32_parity(gpu, oracle, t, M, K, N):
 
 
 @pytest.mark.parametrize("t", ALL_TYPES)
-@pytest.mark.parametrize("M,K,N", [(1, 256, 5), (64, 1024, 130), (200, 512, 300)])
+@pytest.mark.parametrize("M,K,N", [(1, 256, 5), (64, 1024, 130), (200, 512, 300), (260, 768, 129)])
 def test_bf16_prefill_parity(gpu, oracle, t, M, K, N):
     W = synth.weights(t, 90 + t, N, K)
     x = bf16_round(synth.activations(91 + t, M, K))
