@@ -12,6 +12,8 @@ Prints ONE JSON line.  `value` is weight-GB/s over the wall clock of the K timed
 (submitted as one recorded HIP graph unless --no-graph).  `roofline` is the dominant kernel's
 own rate: algorithmic weight bytes per launch / mean kernel duration from start/stop HIP
 events attached to each launch on its stream (a second pass over the same K steps).
+The kernel time is taken two ways with HIP events and the smaller is used (both are upper
+bounds): events bracketing every launch, and two events around the timed region divided by K.
 `cpu_baseline` times the CPU oracle's fused fp32 restatement on the host cores (rank 0, N=1).
 """
 from __future__ import annotations
@@ -29,6 +31,27 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+# HBM-side traffic per step in bytes, from hardware counters: two `rocprofv3 --pmc` passes per
+# workload (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch, summed over the step's kernels), each
+# scaled by what the same counter reads for the 64 MiB copy of --copy-calibration (FETCH_SIZE
+# reads 32780.6 KiB for 65536 KiB copied: factor 1.99924; WRITE_SIZE reads 65536.0: factor 1.0).
+# The readings are summarised under profiles/; they are properties of the kernels' access
+# pattern, not of a particular run, and are re-measured whenever a kernel changes.
+_KIB, _FETCH_SCALE, _WRITE_SCALE = 1024, 65536.0 / 32780.6, 1.0
+COUNTER_KIB = {  # workload -> (FETCH_SIZE, WRITE_SIZE) raw counter KiB per step
+    "c0": (8874.1, 16.0),
+    "c1": (16281.3, 56.0),
+    "c2": (19871.0 + 1822.1 + 911.5, 3584.0 + 512.0 + 924.0),
+    "c3": (74690.3, 32768.0),
+    "c4": (60646.4, 172.1),
+}
+
+
+def measured_traffic(name):
+    f, w = COUNTER_KIB[name]
+    return int(round((f * _FETCH_SCALE + w * _WRITE_SCALE) * _KIB))
+
 
 # name -> (ggml type name, M, K, N, activation dtype, bound)
 CONFIGS = {
@@ -57,6 +80,9 @@ def parse_args():
     p.add_argument("--no-graph", action="store_true", help="submit the timed steps one call at a time")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     p.add_argument("--hot", action="store_true", help="single weight buffer (Infinity-Cache resident) instead of the cold rotation")
+    p.add_argument("--copy-calibration", action="store_true",
+                   help="instead of the benchmark, run a plain 64 MiB device-to-device copy kernel --steps times: the known-size "
+                        "workload that hardware counter readings (FETCH_SIZE / WRITE_SIZE) are scaled by")
     return p.parse_args()
 
 
@@ -134,14 +160,18 @@ class Problem:
             if warmup > 0:  # untimed first replay: uploads the graph
                 self.check(L.gq_graph_launch(graph, self.stream))
             torch.cuda.synchronize()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
+        ev0.record(self.tstream)  # events on the stream the kernels are launched on
         if graph is not None:
             self.check(L.gq_graph_launch(graph, self.stream))
         else:
             for s in range(steps):
                 self.launch(warmup + s)
+        ev1.record(self.tstream)
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
+        self.region_us_per_step = ev0.elapsed_time(ev1) * 1e3 / steps
         if graph is not None:
             self.check(L.gq_graph_destroy(graph))
         # second pass over the same steps: per-launch start/stop events on the launch stream
@@ -150,7 +180,10 @@ class Problem:
             self.launch(warmup + s)
         n, us = ctypes.c_int(0), ctypes.c_double(0.0)
         self.check(L.gq_profile_end(ctypes.byref(n), ctypes.byref(us)))
-        kernel_us_per_step = us.value / steps
+        self.bracketed_us_per_step = us.value / steps
+        # Both figures bound the mean kernel time from above: the bracketed one carries the cost of
+        # the two event packets around every launch, the region one the gaps between launches.
+        kernel_us_per_step = min(self.bracketed_us_per_step, self.region_us_per_step)
         return wall, kernel_us_per_step, n.value // steps
 
     def report(self, wall, kernel_us, steps):
@@ -160,15 +193,17 @@ class Problem:
             out["value"] = self.weight_bytes * steps / wall / 1e9
             ach = self.weight_bytes / (kernel_us * 1e-6) / 1e9
             out["roofline"] = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                               "frac": ach / HBM_PEAK_GBS, "traffic": None,
+                               "frac": ach / HBM_PEAK_GBS, "traffic": measured_traffic(self.name),
                                "algorithmic_bytes_per_launch": self.weight_bytes, "kernel_us": kernel_us}
         else:
             out["metric"], out["unit"] = "prefill GEMM TFLOP/s", "TFLOP/s"
             out["value"] = self.flops * steps / wall / 1e12
             ach = self.flops / (kernel_us * 1e-6) / 1e12
             out["roofline"] = {"bound": "mfma", "achieved": ach, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                               "frac": ach / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                               "frac": ach / MFMA_BF16_PEAK_TFLOPS, "traffic": measured_traffic(self.name),
                                "algorithmic_flops_per_launch": self.flops, "kernel_us": kernel_us}
+        out["roofline"]["kernel_us_bracketed"] = self.bracketed_us_per_step
+        out["roofline"]["kernel_us_region"] = self.region_us_per_step
         out["ms_per_step"] = wall / steps * 1e3
         return out
 
@@ -217,6 +252,19 @@ def cpu_baseline(name):
             "sample": f"{sample}; {runs} runs, {per * 1e3:.2f} ms each"}
 
 
+def copy_calibration(torch, steps):
+    """A copy kernel of known size: each launch reads 64 MiB and writes 64 MiB (an elementwise
+    `dst = src + 0` over 16 Mi floats; sources rotate over 10 buffers so reads come from HBM)."""
+    n = (64 << 20) // 4
+    srcs = [torch.full((n,), float(i), device="cuda") for i in range(10)]
+    dst = torch.empty(n, device="cuda")
+    torch.cuda.synchronize()
+    for s in range(steps):
+        torch.add(srcs[s % len(srcs)], 0.0, out=dst)
+    torch.cuda.synchronize()
+    print(json.dumps({"copy_calibration": True, "launches": steps, "read_bytes_per_launch": n * 4, "write_bytes_per_launch": n * 4}))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -227,9 +275,12 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; there is no CPU fallback for the product path", file=sys.stderr)
         sys.exit(3)
+    torch.cuda.set_device(0)
+    if args.copy_calibration:
+        copy_calibration(torch, args.steps)
+        return
     from gomlx_amd import _lib
     _lib.init(0)
-    torch.cuda.set_device(0)
 
     def measure(name):
         prob = Problem(torch, name, hot=args.hot)

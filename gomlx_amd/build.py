@@ -15,6 +15,9 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "csrc", "build")
 LIB = os.path.join(HERE, "libgomlx_hipq.so")
 
+HOST = os.path.join(HERE, "host")
+HOST_TEST = os.path.join(HOST, "build", "hipq_backend_test")
+
 SOURCES = ["api.hip", "dequant.hip", "gemv.hip", "gemv_xs.hip", "mmq.hip", "gemm.hip"]
 
 # -packed-fp32-ops (note the minus): keep hipcc from forming v_pk_*_f32 instructions.
@@ -57,7 +60,23 @@ def build(verbose: bool = True) -> str:
         raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
     if verbose:
         print(f"built {LIB}")
+    build_host_test(verbose)
     return LIB
+
+
+def build_host_test(verbose: bool = True) -> str:
+    """Compiles the C++ host layer's test program (host code only) against the library."""
+    os.makedirs(os.path.dirname(HOST_TEST), exist_ok=True)
+    cmd = ["g++", "-O1", "-std=c++17", "-Wall", "-Wextra", os.path.join(HOST, "hipq_backend_test.cpp"), "-o", HOST_TEST,
+           "-L" + HERE, "-lgomlx_hipq", "-Wl,-rpath,$ORIGIN/../..", "-Wl,-rpath,/opt/rocm/lib"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"host test build failed:\n{r.stdout}\n{r.stderr}")
+    if r.stderr.strip():
+        sys.stderr.write(r.stderr)
+    if verbose:
+        print(f"built {HOST_TEST}")
+    return HOST_TEST
 
 
 if __name__ == "__main__":

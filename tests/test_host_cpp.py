@@ -1,0 +1,40 @@
+"""Runs the C++ host layer's own test program (gomlx_amd/host/hipq_backend_test.cpp), which
+mirrors the reference's Go tests of nn.QuantizedDense / nn.QuantizedGather
+(ml/nn/quantized_dense_test.go:272-452, ml/nn/quantized_gather_test.go:17-169) above the C ABI."""
+import os
+import subprocess
+
+import pytest
+
+from gomlx_amd import build
+
+
+def _binary():
+    if not os.path.exists(build.HOST_TEST):
+        if not os.path.exists(build.LIB):
+            build.build(verbose=False)
+        else:
+            build.build_host_test(verbose=False)
+    return build.HOST_TEST
+
+
+def _run(*args):
+    r = subprocess.run([_binary(), *args], capture_output=True, text=True, timeout=100)
+    print(r.stdout)
+    print(r.stderr)
+    return r
+
+
+def test_host_layer_build_time_rules():
+    """Graph-build validation, ErrNotImplemented vs hard errors, GOMLX_FUSION: no GPU needed."""
+    r = _run("--build-only")
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "0 failed" in r.stdout and "FAIL" not in r.stdout
+
+
+@pytest.mark.gpu
+def test_host_layer_reference_cases_on_gpu():
+    r = _run()
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "0 failed" in r.stdout and "FAIL" not in r.stdout
+    assert "QuantizedDense_GGML_IQ4NL/basic" in r.stdout and "LayerGraph/independent_and_chained" in r.stdout
