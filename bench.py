@@ -40,11 +40,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # pattern, not of a particular run, and are re-measured whenever a kernel changes.
 _KIB, _FETCH_SCALE, _WRITE_SCALE = 1024, 65536.0 / 32780.6, 1.0
 COUNTER_KIB = {  # workload -> (FETCH_SIZE, WRITE_SIZE) raw counter KiB per step
-    "c0": (8874.1, 16.0),
-    "c1": (16281.3, 56.0),
+    "c0": (8804.6, 16.0),
+    "c1": (16256.7, 56.0),
     "c2": (19871.0 + 1822.1 + 911.5, 3584.0 + 512.0 + 924.0),
     "c3": (74690.3, 32768.0),
-    "c4": (60646.4, 172.1),
+    "c4": (60616.3, 168.0),
 }
 
 

@@ -241,6 +241,8 @@ int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *d
     // Up to four activation rows: one bandwidth-bound pass over W per row, fp32 throughout.
     // More rows: W is read once per 128-row tile and contracted on the matrix cores.
     if (M <= 4) {
+        if (gemv_ks_supported(type, K, N, dX))
+            return launch_gemv_ks(type, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
         if (gemv_xs_supported(type, K, N, dX))
             return launch_gemv_xs(type, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
         return launch_gemv(type, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
@@ -263,14 +265,18 @@ int gq_qdense_f32_batch(int count, const gq_dense_desc *descs, void *stream) {
     while (i < count) {
         int j = i;
         XsBatchItem items[8];
+        bool all_ks = true;
         while (j < count && j - i < 8 && descs[j].type == descs[i].type && descs[j].M == 1 && descs[j].N > 0 &&
                gemv_xs_supported(descs[j].type, descs[j].K, descs[j].N, descs[j].dX)) {
             const gq_dense_desc &d = descs[j];
             items[j - i] = XsBatchItem{d.dX, (const uint8_t *)d.dW, d.dBias, d.dY, d.K, d.N, d.act};
+            all_ks = all_ks && gemv_ks_supported(d.type, d.K, d.N, d.dX);
             j++;
         }
         if (j - i >= 2) {
-            if (int rc = launch_gemv_xs_batch(descs[i].type, j - i, items, (hipStream_t)stream)) return rc;
+            if (int rc = all_ks ? launch_gemv_ks_batch(descs[i].type, j - i, items, (hipStream_t)stream)
+                                : launch_gemv_xs_batch(descs[i].type, j - i, items, (hipStream_t)stream))
+                return rc;
             i = j;
             continue;
         }

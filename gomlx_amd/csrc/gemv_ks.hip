@@ -1,0 +1,544 @@
+// Decode GEMV, K-sliced integer-dot kernels with wavefront-local activation staging
+// (Q4_0, Q8_0, Q4_K; K % 512 == 0).
+//
+// The activation-stationary kernel of gemv_xs.hip lets every wavefront see all of K, so its
+// workgroup has to convert the whole activation vector together and meet at a barrier before the
+// first code byte can be used; on a 5-10 us kernel that prologue is a quarter of the run time.
+// Here a wavefront owns one 512-value slice of K (16 blocks of 32) instead: its 64 lanes convert
+// 8 activations each, exchange the fixed-point planes through a private piece of LDS (no
+// barrier: LDS operations of one wavefront execute in order) and start on the codes as soon as
+// their own 2 KB of x have arrived.  The wavefronts of a workgroup cover the slices of the same
+// rows and add their partial sums in LDS once, at the very end.
+//
+// Lane l = 8 * rg + c works on row (8 * it + rg) of the workgroup and on 64 values of the slice:
+//   Q4_0: blocks 2c, 2c+1: 36 bytes at a 4-byte-aligned address;
+//   Q8_0: blocks 2c, 2c+1: 68 bytes at a 4-byte-aligned address;
+//   Q4_K: super-block c / 4 of the slice, 64-value group c % 4: the 16-byte header and 32 code bytes.
+// A load instruction therefore covers 8 rows x one contiguous slice (288 or 544 bytes).
+//
+// Activation fixed point: 16 bits per 32 values.  Q4_0 uses four balanced base-16 digits (digit
+// planes in the nibble order of a weight dword, one v_dot8_i32_i4 per plane); Q8_0 and Q4_K use
+// two signed base-256 limbs (one v_dot4_i32_i8 per limb).  The rounding is at most 2^-16 of the
+// 32 values' largest magnitude per element; over K = 4096 random terms that is a relative output
+// error of a few 1e-5, well inside the 1e-3 bound of this path.
+#include "blocks.hpp"
+#include "common.hpp"
+
+#include <cstdlib>
+
+namespace gq {
+
+namespace {
+
+constexpr float kQmax4 = 30500.0f;                   // |q| <= 30583 fits four balanced hex digits
+constexpr float kMagic4 = 12582912.0f + 34952.0f;    // 1.5 * 2^23 + 0x8888
+constexpr float kQmaxL = 32500.0f;                   // |q| <= 32639 fits two balanced base-256 limbs
+constexpr float kMagicL = 12582912.0f + 32896.0f;    // 1.5 * 2^23 + 0x8080
+constexpr int kSliceValues = 512;
+constexpr int kMaxItersKs = 64;                      // rows per workgroup <= 512
+
+__device__ __forceinline__ float ks_quad_max(float v) {
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true)));
+    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true)));
+    return v;
+}
+// sum over the 8 lanes of an aligned group of 8 (every lane ends up with the total)
+__device__ __forceinline__ float ks_oct_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // row_half_mirror
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+    return v;
+}
+
+// sum over the 4 lanes of a quad (integer)
+__device__ __forceinline__ int ks_quad_sum(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true);
+    v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true);
+    return v;
+}
+
+struct XPair { float4 lo, hi; };
+
+// Scale of 32 activations for a fixed-point range of +-qmax.  All-zero groups quantise to zero; a
+// non-finite group poisons its scale so that the affected outputs come out as NaN.
+__device__ __forceinline__ void ks_scale(const float *e, float qmax, float &inv, float &scale) {
+    float amax = 0.f;
+    bool nan = false;
+#pragma unroll
+    for (int p = 0; p < 8; p++) { amax = fmaxf(amax, fabsf(e[p])); nan |= e[p] != e[p]; }
+    if (nan) amax = __builtin_inff();  // fmaxf would drop a NaN in the cross-lane maximum
+    amax = ks_quad_max(amax);          // the four lanes that hold 32 consecutive values form a quad
+    if (!(amax >= 0x1p-100f)) { inv = 0.f; scale = 0.f; }
+    else if (amax > 3.0e38f) { inv = 0.f; scale = __builtin_nanf(""); }
+    else { inv = qmax / amax; scale = amax / qmax; }
+}
+
+// What a lane publishes for the 8 activations it converts: four plane dwords, the scale of their
+// 32-value group and (limb formats) scale * sum of the group's fixed-point values.
+struct Staged { uint4 planes; float scale, sum; };
+
+// ---- per-format traits -----------------------------------------------------------------------------
+template <int T> struct KS;
+
+template <> struct KS<kQ4_0> {
+    static constexpr int kSliceBytes = 288;
+    struct __attribute__((packed, aligned(4))) Raw { uint32_t v[9]; };
+    static __device__ __forceinline__ int lane_offset(int c) { return c * 36; }
+    static __device__ __forceinline__ void load(Raw &r, const uint8_t *p) { r = *reinterpret_cast<const Raw *>(p); }
+    // the 8 activations that face weight dword (lane & 3) of block (lane >> 2) of the slice
+    static __device__ __forceinline__ XPair x_load(const float *__restrict__ xs, int lane) {
+        const float4 *x4 = reinterpret_cast<const float4 *>(xs) + (lane >> 2) * 8 + (lane & 3);
+        XPair p;
+        p.lo = x4[0];  // values 4w .. 4w+3 of the block (low nibbles of code bytes 4w .. 4w+3)
+        p.hi = x4[4];  // values 16+4w .. (high nibbles)
+        return p;
+    }
+    // nibble p of plane d = digit d of the activation facing nibble p of the weight dword
+    static __device__ __forceinline__ Staged stage(const XPair &xp) {
+        const float e[8] = {xp.lo.x, xp.hi.x, xp.lo.y, xp.hi.y, xp.lo.z, xp.hi.z, xp.lo.w, xp.hi.w};  // nibble order
+        Staged st;
+        float inv;
+        ks_scale(e, kQmax4, inv, st.scale);
+        st.sum = 0.f;
+        uint32_t z[8];
+#pragma unroll
+        for (int p = 0; p < 8; p++) z[p] = __builtin_bit_cast(uint32_t, fmaf(e[p], inv, kMagic4));  // low 16 bits: q + 0x8888
+        // byte 0 of z = digits 0,1; byte 1 = digits 2,3.  Gather the bytes of the even and of the
+        // odd nibble positions, then interleave nibbles.
+        const uint32_t ga = __builtin_amdgcn_perm(z[2], z[0], 0x05010400u), gb = __builtin_amdgcn_perm(z[6], z[4], 0x05010400u);
+        const uint32_t gc = __builtin_amdgcn_perm(z[3], z[1], 0x05010400u), gd = __builtin_amdgcn_perm(z[7], z[5], 0x05010400u);
+        const uint32_t e0 = __builtin_amdgcn_perm(gb, ga, 0x05040100u) ^ 0x88888888u, e1 = __builtin_amdgcn_perm(gb, ga, 0x07060302u) ^ 0x88888888u;
+        const uint32_t o0 = __builtin_amdgcn_perm(gd, gc, 0x05040100u) ^ 0x88888888u, o1 = __builtin_amdgcn_perm(gd, gc, 0x07060302u) ^ 0x88888888u;
+        constexpr uint32_t m = 0x0F0F0F0Fu;
+        st.planes.x = (e0 & m) | ((o0 & m) << 4);
+        st.planes.y = ((e0 >> 4) & m) | (o0 & ~m);
+        st.planes.z = (e1 & m) | ((o1 & m) << 4);
+        st.planes.w = ((e1 >> 4) & m) | (o1 & ~m);
+        return st;
+    }
+    // xq[4 h + w] = planes facing dword w of block h
+    static __device__ __forceinline__ float dot(const Raw &r, const uint4 *xq, const float *xsc, const float *, int) {
+        const uint32_t *v = r.v;
+#ifdef GQ_KS_NODOT  // tuning builds only: consume the loads without the arithmetic
+        { uint32_t a = xq[0].x; for (int i = 0; i < 9; i++) a ^= v[i]; return __builtin_bit_cast(float, a) * xsc[0]; }
+#endif
+        float out = 0.f;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            int s0 = 0, s1 = 0, s2 = 0, s3 = 0;
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                const int q = (int)((h == 0 ? __builtin_amdgcn_alignbit(v[w + 1], v[w], 16) : v[5 + w]) ^ 0x88888888u);
+                const uint4 &pl = xq[h * 4 + w];
+                s0 = __builtin_amdgcn_sdot8(q, (int)pl.x, s0, false);
+                s1 = __builtin_amdgcn_sdot8(q, (int)pl.y, s1, false);
+                s2 = __builtin_amdgcn_sdot8(q, (int)pl.z, s2, false);
+                s3 = __builtin_amdgcn_sdot8(q, (int)pl.w, s3, false);
+            }
+            uint32_t t = (uint32_t)s3;
+            t = (t << 4) + (uint32_t)s2;  // v_lshl_add_u32
+            t = (t << 4) + (uint32_t)s1;
+            t = (t << 4) + (uint32_t)s0;
+            const float d = half_bits_to_float(h == 0 ? (v[0] & 0xFFFFu) : (v[4] >> 16));
+            out = fmaf((float)(int)t, d * xsc[h], out);
+        }
+        return out;
+    }
+};
+
+// Q8_0 and Q4_K: lane l converts activations 8l .. 8l+7 of the slice, i.e. the values facing dwords
+// 2j, 2j+1 (j = l & 3) of 32-value group l >> 2.  planes = {limb0, limb1 of dword 2j, limb0, limb1 of
+// dword 2j+1}, byte i of a plane = limb of value 4 * dword + i.
+__device__ __forceinline__ XPair limb_x_load(const float *__restrict__ xs, int lane) {
+    const float4 *x4 = reinterpret_cast<const float4 *>(xs) + 2 * lane;
+    XPair p;
+    p.lo = x4[0];
+    p.hi = x4[1];
+    return p;
+}
+__device__ __forceinline__ Staged limb_stage(const XPair &xp) {
+    const float e[8] = {xp.lo.x, xp.lo.y, xp.lo.z, xp.lo.w, xp.hi.x, xp.hi.y, xp.hi.z, xp.hi.w};
+    Staged st;
+    float inv;
+    ks_scale(e, kQmaxL, inv, st.scale);
+    uint32_t z[8];
+    int xsum = 0;
+#pragma unroll
+    for (int p = 0; p < 8; p++) {
+        const int zs = (int)(__builtin_bit_cast(uint32_t, fmaf(e[p], inv, kMagicL)) - 0x4B400000u);  // q + 0x8080
+        xsum += zs - 0x8080;
+        z[p] = (uint32_t)zs;
+    }
+    xsum = ks_quad_sum(xsum);
+    st.sum = st.scale * (float)xsum;
+    const uint32_t a01 = __builtin_amdgcn_perm(z[1], z[0], 0x05010400u), a23 = __builtin_amdgcn_perm(z[3], z[2], 0x05010400u);
+    const uint32_t b01 = __builtin_amdgcn_perm(z[5], z[4], 0x05010400u), b23 = __builtin_amdgcn_perm(z[7], z[6], 0x05010400u);
+    st.planes.x = __builtin_amdgcn_perm(a23, a01, 0x05040100u) ^ 0x80808080u;
+    st.planes.y = __builtin_amdgcn_perm(a23, a01, 0x07060302u) ^ 0x80808080u;
+    st.planes.z = __builtin_amdgcn_perm(b23, b01, 0x05040100u) ^ 0x80808080u;
+    st.planes.w = __builtin_amdgcn_perm(b23, b01, 0x07060302u) ^ 0x80808080u;
+    return st;
+}
+// planes of dword w (0..7) of group h: limb 0 and limb 1
+__device__ __forceinline__ void limb_planes(const uint4 *xq, int h, int w, int &p0, int &p1) {
+    const uint4 &pl = xq[h * 4 + (w >> 1)];
+    p0 = (int)((w & 1) ? pl.z : pl.x);
+    p1 = (int)((w & 1) ? pl.w : pl.y);
+}
+
+template <> struct KS<kQ8_0> {
+    static constexpr int kSliceBytes = 544;
+    struct __attribute__((packed, aligned(4))) Raw { uint32_t v[17]; };
+    static __device__ __forceinline__ int lane_offset(int c) { return c * 68; }
+    static __device__ __forceinline__ void load(Raw &r, const uint8_t *p) { r = *reinterpret_cast<const Raw *>(p); }
+    static __device__ __forceinline__ XPair x_load(const float *__restrict__ xs, int lane) { return limb_x_load(xs, lane); }
+    static __device__ __forceinline__ Staged stage(const XPair &xp) { return limb_stage(xp); }
+    static __device__ __forceinline__ float dot(const Raw &r, const uint4 *xq, const float *xsc, const float *, int) {
+        const uint32_t *v = r.v;
+        float out = 0.f;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            int s0 = 0, s1 = 0;
+#pragma unroll
+            for (int w = 0; w < 8; w++) {
+                const int q = (int)(h == 0 ? __builtin_amdgcn_alignbit(v[w + 1], v[w], 16) : v[9 + w]);
+                int p0, p1;
+                limb_planes(xq, h, w, p0, p1);
+                s0 = __builtin_amdgcn_sdot4(q, p0, s0, false);
+                s1 = __builtin_amdgcn_sdot4(q, p1, s1, false);
+            }
+            const int t = (s1 << 8) + s0;
+            const float d = half_bits_to_float(h == 0 ? (v[0] & 0xFFFFu) : (v[8] >> 16));
+            out = fmaf((float)t, d * xsc[h], out);
+        }
+        return out;
+    }
+};
+
+template <> struct KS<kQ4_K> {
+    static constexpr int kSliceBytes = 288;  // two super-blocks
+    struct Raw { uint4 hd, q0, q1; };
+    static __device__ __forceinline__ int lane_offset(int c) { return (c >> 2) * 144; }
+    static __device__ __forceinline__ void load(Raw &r, const uint8_t *sb, int c) {
+        r.hd = *reinterpret_cast<const uint4 *>(sb);
+        const uint4 *q = reinterpret_cast<const uint4 *>(sb + 16 + 32 * (c & 3));
+        r.q0 = q[0];
+        r.q1 = q[1];
+    }
+    static __device__ __forceinline__ XPair x_load(const float *__restrict__ xs, int lane) { return limb_x_load(xs, lane); }
+    static __device__ __forceinline__ Staged stage(const XPair &xp) { return limb_stage(xp); }
+    static __device__ __forceinline__ float dot(const Raw &r, const uint4 *xq, const float *xsc, const float *xsm, int c) {
+        const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+        const float d = half_bits_to_float(r.hd.x & 0xFFFFu), dmin = half_bits_to_float(r.hd.x >> 16);
+        const int g = c & 3;
+        float out = 0.f;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            int s0 = 0, s1 = 0;
+#pragma unroll
+            for (int w = 0; w < 8; w++) {
+                const int cw = (int)((h == 0 ? q[w] : (q[w] >> 4)) & 0x0F0F0F0Fu);  // four codes as bytes 0..15
+                int p0, p1;
+                limb_planes(xq, h, w, p0, p1);
+                s0 = __builtin_amdgcn_sdot4(cw, p0, s0, false);
+                s1 = __builtin_amdgcn_sdot4(cw, p1, s1, false);
+            }
+            const int t = (s1 << 8) + s0;
+            uint32_t sc, mn;
+            q4k_scale_min(r.hd.y, r.hd.z, r.hd.w, 2 * g + h, sc, mn);
+            out = fmaf((float)t, (d * (float)sc) * xsc[h], out);
+            out = fmaf(-(dmin * (float)mn), xsm[h], out);
+        }
+        return out;
+    }
+};
+
+template <int T>
+__device__ __forceinline__ void ks_load(typename KS<T>::Raw &r, const uint8_t *p, int c) {
+    if constexpr (T == kQ4_K) KS<T>::load(r, p, c);
+    else KS<T>::load(r, p);
+}
+
+#ifdef GQ_KS_TRACE
+__device__ unsigned long long g_ks_trace[4096 * 16];
+#define KS_TRACE(k) do { if (lane == 0) g_ks_trace[((size_t)wg * waves + wave) % 4096 * 16 + (k)] = __builtin_readcyclecounter(); } while (0)
+#define KS_TRACE_WALL(k) do { if (lane == 0) g_ks_trace[((size_t)wg * waves + wave) % 4096 * 16 + (k)] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#else
+#define KS_TRACE(k) do { } while (0)
+#define KS_TRACE_WALL(k) do { } while (0)
+#endif
+
+constexpr int kWaveLdsDwords = 72 * 4;  // per wavefront: 64 uint4 of planes, 16 scales, 16 sums
+
+// Workgroup `wg` of a problem: `waves` wavefronts work (threads beyond them only join the final
+// barrier); wavefront w handles slices w, w + waves, ... (spw of them) of the 8 * iters rows
+// starting at wg * 8 * iters.  PF divides iters: rows are consumed in groups of PF, buffer j of a
+// group always holding the row-step with (it % PF == j).
+// WIN <= PF row-steps are kept in flight: WIN go out before the activations are converted, and
+// each consumed step is followed by the load of the step WIN ahead, so that load issue (which
+// blocks while the memory pipeline is full) and arithmetic alternate instead of forming two
+// phases.
+template <int T, int PF, int WIN>
+__device__ __forceinline__ void ks_body(const float *__restrict__ x, const uint8_t *__restrict__ W, const float *__restrict__ bias,
+                                        float *__restrict__ y, int N, int64_t row_bytes, int iters, int spw, int act, int waves,
+                                        int wg, uint32_t *lds) {
+    typedef typename KS<T>::Raw Raw;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int rg = lane >> 3, c = lane & 7;
+    const int rows_wg = iters * 8;
+    const int row0 = wg * rows_wg;
+    float *all = reinterpret_cast<float *>(lds + waves * kWaveLdsDwords);  // partial sums [waves][rows_wg]
+    if (wave < waves) {
+        uint4 *my_planes = reinterpret_cast<uint4 *>(lds + wave * kWaveLdsDwords);
+        float *my_scales = reinterpret_cast<float *>(my_planes + 64);
+        float *my_sums = my_scales + 16;
+        float *part = all + wave * rows_wg;
+
+        KS_TRACE(0);
+        KS_TRACE_WALL(12);
+        XPair xp = KS<T>::x_load(x + wave * kSliceValues, lane);
+        const int last_row = N - 1;
+        auto addr = [&](int j, int it) -> const uint8_t * {
+            const int row = min(row0 + it * 8 + rg, last_row);
+            return W + (int64_t)row * row_bytes + (int64_t)(wave + j * waves) * KS<T>::kSliceBytes + KS<T>::lane_offset(c);
+        };
+        Raw buf[PF];
+#pragma unroll
+        for (int j = 0; j < WIN; j++) ks_load<T>(buf[j], addr(0, j), c);
+        KS_TRACE(1);
+
+        uint4 xq[8];
+        float xsc[2], xsm[2] = {0.f, 0.f};
+        auto stage = [&](const XPair &p) {
+            const Staged st = KS<T>::stage(p);
+            my_planes[lane] = st.planes;
+            if ((lane & 3) == 0) {
+                my_scales[lane >> 2] = st.scale;
+                if constexpr (T == kQ4_K) my_sums[lane >> 2] = st.sum;
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int i = 0; i < 8; i++) xq[i] = my_planes[8 * c + i];
+            xsc[0] = my_scales[2 * c];
+            xsc[1] = my_scales[2 * c + 1];
+            if constexpr (T == kQ4_K) { xsm[0] = my_sums[2 * c]; xsm[1] = my_sums[2 * c + 1]; }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        };
+        stage(xp);
+        KS_TRACE(2);
+        if (spw > 1) xp = KS<T>::x_load(x + (wave + waves) * kSliceValues, lane);
+        KS_TRACE(3);
+
+        const int ngroups = spw * (iters / PF);
+        int j = 0, i0 = 0;  // slice index and first row-step of the current group
+        for (int g = 0; g < ngroups; g++) {
+            const bool last_group = g == ngroups - 1;
+            // where the buffers of this group are refilled from: same slice PF steps on, or the next slice
+            const bool wrap = i0 + PF >= iters;
+            const int nj = wrap ? j + 1 : j, ni0 = wrap ? 0 : i0 + PF;
+#pragma unroll
+            for (int jj = 0; jj < PF; jj++) {
+                float d = KS<T>::dot(buf[jj], xq, xsc, xsm, c);
+                if (jj + WIN < PF) ks_load<T>(buf[jj + WIN], addr(j, i0 + jj + WIN), c);
+                else if (!last_group) ks_load<T>(buf[jj + WIN - PF], addr(nj, ni0 + jj + WIN - PF), c);
+                d = ks_oct_sum(d);
+                if (c == 0) {
+                    float *slot = part + (i0 + jj) * 8 + rg;
+                    *slot = j == 0 ? d : *slot + d;
+                }
+            }
+            if (wrap && !last_group) {  // next group starts a new slice: convert its activations
+                stage(xp);
+                if (nj + 1 < spw) xp = KS<T>::x_load(x + (wave + (nj + 1) * waves) * kSliceValues, lane);
+            }
+            j = nj;
+            i0 = ni0;
+        }
+        KS_TRACE(14);
+        KS_TRACE_WALL(13);
+    }
+    __syncthreads();
+    for (int r = tid; r < rows_wg; r += blockDim.x) {
+        const int row = row0 + r;
+        if (row < N) {
+            float t = 0.f;
+            for (int w = 0; w < waves; w++) t += all[w * rows_wg + r];
+            y[row] = apply_act(act, t + (bias ? bias[row] : 0.f));
+        }
+    }
+}
+
+template <int T, int PF, int WIN>
+__global__ __launch_bounds__(512) void gemv_ks_kernel(const float *__restrict__ X, const uint8_t *__restrict__ W,
+                                                      const float *__restrict__ bias, float *__restrict__ Y, int K, int N,
+                                                      int64_t row_bytes, int iters, int spw, int act) {
+    extern __shared__ uint32_t lds[];
+    ks_body<T, PF, WIN>(X + (int64_t)blockIdx.y * K, W, bias, Y + (int64_t)blockIdx.y * N, N, row_bytes, iters, spw, act,
+                        (int)(blockDim.x >> 6), (int)blockIdx.x, lds);
+}
+
+// Several independent batch-1 problems of one format in a single launch: workgroups
+// [wg_begin, next wg_begin) belong to problem i.  This is how the projections of a decoder layer
+// that do not depend on each other (q/k/v, gate/up) share one submission.  Every problem runs in
+// groups of four row-steps (its iters is a multiple of 4).
+constexpr int kMaxBatchKs = 8;
+struct KsProblem {
+    const float *x;
+    const uint8_t *W;
+    const float *bias;
+    float *y;
+    int64_t row_bytes;
+    int N, iters, spw, waves, act, wg_begin;
+};
+struct KsBatch {
+    int count;
+    KsProblem p[kMaxBatchKs];
+};
+
+template <int T>
+__global__ __launch_bounds__(512) void gemv_ks_batch_kernel(const KsBatch b) {
+    extern __shared__ uint32_t lds[];
+    int i = 0;
+#pragma unroll
+    for (int j = 1; j < kMaxBatchKs; j++)
+        if (j < b.count && (int)blockIdx.x >= b.p[j].wg_begin) i = j;
+    const KsProblem &q = b.p[i];
+    ks_body<T, 4, 3>(q.x, q.W, q.bias, q.y, q.N, q.row_bytes, q.iters, q.spw, q.act, q.waves, (int)blockIdx.x - q.wg_begin, lds);
+}
+
+struct KsPlan { int waves, spw, iters, pf, wgs; size_t shmem; };
+
+// GOMLX_HIPQ_GEMV_KS="waves_per_cu" overrides the built-in choice (tuning runs only).
+int ks_env_waves() {
+    static const int v = [] { const char *e = std::getenv("GOMLX_HIPQ_GEMV_KS"); return e ? std::atoi(e) : 0; }();
+    return v;
+}
+
+// wavefronts per workgroup (a divisor of the slice count, at most 8) and slices per wavefront
+bool ks_split(int64_t K, int &waves, int &spw) {
+    if (K % kSliceValues != 0 || K <= 0) return false;
+    const int nslices = (int)(K / kSliceValues);
+    waves = 0;
+    for (int w = 8; w >= 1; w--)
+        if (nslices % w == 0) { waves = w; break; }
+    if (waves < 4 && nslices > 8) return false;  // awkward K (e.g. a large prime number of slices)
+    spw = nslices / waves;
+    return true;
+}
+
+size_t ks_lds_bytes(int waves, int iters) { return (size_t)waves * kWaveLdsDwords * 4 + (size_t)waves * iters * 8 * sizeof(float); }
+
+bool ks_plan(int64_t K, int64_t N, KsPlan &p) {
+    if (N <= 0 || !ks_split(K, p.waves, p.spw)) return false;
+    const int cus = device_cu_count();
+    // One 8-wavefront workgroup per CU streams best; problems that would leave a wavefront with
+    // only one or two row-steps are launch- and latency-bound and do better with twice the
+    // wavefronts (more independent prologues in flight).
+    auto iters_for = [&](int waves_per_cu) {
+        int64_t wgs = (int64_t)cus * waves_per_cu / p.waves;
+        if (wgs < 1) wgs = 1;
+        const int64_t it = (N + wgs * 8 - 1) / (wgs * 8);
+        return it < 1 ? (int64_t)1 : it;
+    };
+    int64_t iters = ks_env_waves() > 0 ? iters_for(ks_env_waves()) : iters_for(8);
+    if (ks_env_waves() <= 0 && iters <= 2) iters = iters_for(16);
+    if (iters > 8) iters = (iters + 3) / 4 * 4;  // deep problems run in groups of 4 rows
+    if (iters > kMaxItersKs) iters = kMaxItersKs;
+    p.iters = (int)iters;
+    p.pf = iters <= 8 ? (int)iters : 4;
+    p.wgs = (int)((N + iters * 8 - 1) / (iters * 8));
+    p.shmem = ks_lds_bytes(p.waves, p.iters);
+    return true;
+}
+
+template <int T, int PF>
+int launch_ks_pf(const KsPlan &p, const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act,
+                 float *y, hipStream_t s) {
+    const int64_t row_bytes = (K / Geom<T>::vpb) * Geom<T>::bpb;
+    const dim3 grid((unsigned)p.wgs, (unsigned)M), block((unsigned)p.waves * 64);
+    constexpr int WIN = PF < 3 ? PF : 3;
+    return launch(gemv_ks_kernel<T, PF, WIN>, grid, block, p.shmem, s, x, W, bias, y, (int)K, (int)N, row_bytes, p.iters, p.spw, act);
+}
+
+template <int T>
+int launch_ks(const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y, hipStream_t s) {
+    KsPlan p;
+    if (!ks_plan(K, N, p)) return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv_ks: unsupported problem");
+    switch (p.pf) {
+    case 1: return launch_ks_pf<T, 1>(p, x, M, K, W, N, bias, act, y, s);
+    case 2: return launch_ks_pf<T, 2>(p, x, M, K, W, N, bias, act, y, s);
+    case 3: return launch_ks_pf<T, 3>(p, x, M, K, W, N, bias, act, y, s);
+    case 4: return launch_ks_pf<T, 4>(p, x, M, K, W, N, bias, act, y, s);
+    case 5: return launch_ks_pf<T, 5>(p, x, M, K, W, N, bias, act, y, s);
+    case 6: return launch_ks_pf<T, 6>(p, x, M, K, W, N, bias, act, y, s);
+    case 7: return launch_ks_pf<T, 7>(p, x, M, K, W, N, bias, act, y, s);
+    default: return launch_ks_pf<T, 8>(p, x, M, K, W, N, bias, act, y, s);
+    }
+}
+
+// One launch for `count` batch-1 problems: the chip's workgroup slots are shared out in proportion
+// to each problem's weight bytes, so every CU streams for about the same time.
+template <int T>
+int launch_ks_batch(int count, const XsBatchItem *items, hipStream_t s) {
+    KsBatch b;
+    b.count = count;
+    const int cus = device_cu_count();
+    double total = 0.0;
+    for (int i = 0; i < count; i++) total += (double)gq_row_bytes(T, items[i].K) * (double)items[i].N;
+    size_t shmem = 0;
+    int wg = 0;
+    for (int i = 0; i < count; i++) {
+        const XsBatchItem &it = items[i];
+        KsProblem q;
+        q.x = it.x; q.W = it.W; q.bias = it.bias; q.y = it.y; q.N = (int)it.N; q.act = it.act;
+        q.row_bytes = (int64_t)gq_row_bytes(T, it.K);
+        if (!ks_split(it.K, q.waves, q.spw)) return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv_ks batch: unsupported K");
+        int64_t share = (int64_t)((double)cus * ((double)q.row_bytes * (double)it.N) / total + 0.5);
+        if (share < 1) share = 1;
+        int64_t iters = (it.N + share * 8 - 1) / (share * 8);
+        iters = (iters + 3) / 4 * 4;
+        if (iters > kMaxItersKs) iters = kMaxItersKs;
+        q.iters = (int)iters;
+        q.wg_begin = wg;
+        wg += (int)((it.N + iters * 8 - 1) / (iters * 8));
+        b.p[i] = q;
+        const size_t need = ks_lds_bytes(q.waves, q.iters);
+        if (need > shmem) shmem = need;
+    }
+    return launch(gemv_ks_batch_kernel<T>, dim3((unsigned)wg), dim3(512), shmem, s, b);
+}
+
+}  // namespace
+
+bool gemv_ks_supported(int type, int64_t K, int64_t N, const void *x) {
+    if (reinterpret_cast<uintptr_t>(x) & 15) return false;
+    if (type != kQ4_0 && type != kQ8_0 && type != kQ4_K) return false;
+    if (N <= 0 || N > (int64_t)INT32_MAX / 2) return false;
+    int waves, spw;
+    return ks_split(K, waves, spw);
+}
+
+int launch_gemv_ks(int type, const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act,
+                   float *y, hipStream_t s) {
+    switch (type) {
+    case kQ4_0: return launch_ks<kQ4_0>(x, M, K, W, N, bias, act, y, s);
+    case kQ8_0: return launch_ks<kQ8_0>(x, M, K, W, N, bias, act, y, s);
+    case kQ4_K: return launch_ks<kQ4_K>(x, M, K, W, N, bias, act, y, s);
+    default: return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv_ks: ggml type %d is not implemented", type);
+    }
+}
+
+int launch_gemv_ks_batch(int type, int count, const XsBatchItem *items, hipStream_t s) {
+    if (count < 1 || count > kMaxBatchKs) return fail(GQ_ERR_INVALID, "gemv batch: %d problems (1..%d supported per launch)", count, kMaxBatchKs);
+    switch (type) {
+    case kQ4_0: return launch_ks_batch<kQ4_0>(count, items, s);
+    case kQ8_0: return launch_ks_batch<kQ8_0>(count, items, s);
+    case kQ4_K: return launch_ks_batch<kQ4_K>(count, items, s);
+    default: return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv batch: ggml type %d is not implemented", type);
+    }
+}
+
+}  // namespace gq
