@@ -2,15 +2,15 @@
 //   Y[m,n] = act(sum_k X[m,k] * w[n,k] + b[n]),  X [M,K],  W GGML blocks [N, row_bytes].
 //
 // A workgroup of 8 wavefronts owns a 256 x 128 tile of Y (256 activation rows, 128 weight
-// rows); each wavefront a 64 x 64 sub-tile = 2 x 2 v_mfma_f32_32x32x16 accumulators.  Per
-// 128-wide K step the workgroup dequantises its 128 x 128 slab of W (exact fp32 values, then one
-// rounding to the 16-bit MFMA operand type) and stages the 256 x 128 slab of X next to it in
-// LDS.  Both operands are K-contiguous, which is exactly the A / B fragment shape the
-// instruction wants (8 consecutive k per lane), so fragments are single 16-byte LDS reads from
-// rows padded to 272 bytes (conflict-free).
-//
-// The global loads of step k+1 are issued right after the barrier that publishes step k and
-// wait in registers through the 32 MFMAs per wavefront of step k.
+// rows); each wavefront a 64 x 64 sub-tile = 2 x 2 v_mfma_f32_32x32x16 accumulators.  K advances
+// in steps of 64 through two LDS buffers: while the matrix cores contract step k out of one
+// buffer, the same wavefronts dequantise the 128 x 64 slab of W of step k+1 (exact fp32 values,
+// then one rounding to the 16-bit MFMA operand type) and copy the 256 x 64 slab of X into the
+// other buffer, so the vector ALU work hides in the shadow of the MFMAs and one barrier per step
+// suffices.  The global loads run two steps ahead of the staging, in two register sets.
+// Both operands are K-contiguous, which is exactly the A / B fragment shape the instruction
+// wants (8 consecutive k per lane), so fragments are single 16-byte LDS reads from rows padded
+// to 144 bytes (conflict-free).
 //
 //   bf16 activations -> bf16 MFMA (the prefill path);
 //   fp32 activations -> rounded to fp16, fp16 MFMA (11-bit operands; generic batched path).
@@ -25,9 +25,10 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 256, BN = 128, BK = 128;
-constexpr int LDS_STRIDE = BK + 8;  // 16-bit elements per LDS row: 256 B of data + 16 B pad
-constexpr int LDS_BYTES = (BM + BN) * LDS_STRIDE * 2;
+constexpr int BM = 256, BN = 128, BK = 64;
+constexpr int LDS_STRIDE = BK + 8;  // 16-bit elements per LDS row: 128 B of data + 16 B pad
+constexpr int LDS_BUF = (BM + BN) * LDS_STRIDE;  // elements per buffer
+constexpr int LDS_BYTES = 2 * LDS_BUF * 2;
 
 template <bool BF16> struct Operand;
 template <> struct Operand<true> {
@@ -57,31 +58,31 @@ template <> struct Operand<false> {
     }
 };
 
-// ---- raw (still packed) share of one thread in the W slab: one 32-value run of one row ---------
-// Thread (row = t / 4, blk = t % 4) owns weights k0 + 32 blk .. + 31 of its row.
+// ---- raw (still packed) share of one thread in the W slab: one 16-value run of one row ---------
+// Thread (row = t / 4, run = t % 4) owns weights k0 + 16 run .. + 15 of its row.
 template <int T> struct WRaw;
 
 template <> struct WRaw<kQ8_0> {
     uint32_t d;
-    u128_a2 q0, q1;
-    __device__ __forceinline__ void load(const uint8_t *row, int64_t kblk) {
-        const uint8_t *blk = row + kblk * 34;
+    u128_a2 q;
+    // `base` is uniform (first row of the tile, block column of the K step); `off` is this thread's
+    // constant byte offset of its block within the tile.
+    __device__ __forceinline__ void set_row(const uint8_t *) {}
+    __device__ __forceinline__ void load(const uint8_t *base, uint32_t off, uint32_t run, int64_t) {
+        const uint8_t *blk = base + off;
         d = load_u16(blk);
-        q0 = *reinterpret_cast<const u128_a2 *>(blk + 2);
-        q1 = *reinterpret_cast<const u128_a2 *>(blk + 18);
+        q = *reinterpret_cast<const u128_a2 *>(blk + 2 + 16 * (run & 1));
     }
-    // int8 q = (q ^ 0x80) - 128 with the xor-ed byte read as unsigned; fma(u, d, -128 d) = d * q
-    // exactly (the product has at most 18 significant bits), i.e. the reference's f32(d) * f32(q).
-    __device__ __forceinline__ void values(float *w) const {
+    // Values 4 part .. 4 part + 3 of the run.  int8 q = (q ^ 0x80) - 128 with the xor-ed byte read
+    // as unsigned; fma(u, d, -128 d) = d * q exactly (the product has at most 18 significant
+    // bits), i.e. the reference's f32(d) * f32(q).
+    __device__ __forceinline__ void part(int i, float *w) const {
         const float df = half_bits_to_float(d), off = -128.0f * df;
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const uint32_t a = (i < 4 ? q0.v[i] : q1.v[i - 4]) ^ 0x80808080u;
-            w[4 * i + 0] = fmaf(ubyte0(a), df, off);
-            w[4 * i + 1] = fmaf(ubyte1(a), df, off);
-            w[4 * i + 2] = fmaf(ubyte2(a), df, off);
-            w[4 * i + 3] = fmaf(ubyte3(a), df, off);
-        }
+        const uint32_t a = q.v[i] ^ 0x80808080u;
+        w[4 * i + 0] = fmaf(ubyte0(a), df, off);
+        w[4 * i + 1] = fmaf(ubyte1(a), df, off);
+        w[4 * i + 2] = fmaf(ubyte2(a), df, off);
+        w[4 * i + 3] = fmaf(ubyte3(a), df, off);
     }
 };
 
@@ -89,69 +90,88 @@ template <> struct WRaw<kQ8_0> {
 template <int T> struct WRaw {
     const uint8_t *row;
     int64_t i16;
-    __device__ __forceinline__ void load(const uint8_t *r, int64_t kblk) {
-        row = r;
-        i16 = kblk * 2;
-    }
-    __device__ __forceinline__ void values(float *w) const {
-        dequant16<T>(row, i16, w);
-        dequant16<T>(row, i16 + 1, w + 16);
+    __device__ __forceinline__ void set_row(const uint8_t *r) { row = r; }
+    __device__ __forceinline__ void load(const uint8_t *, uint32_t, uint32_t, int64_t i) { i16 = i; }
+    __device__ __forceinline__ void part(int i, float *w) const {
+        if (i == 0) dequant16<T>(row, i16, w);
     }
 };
 
-// The 256 x 128 activation slab as 16-byte chunks, chunk-major over the 512 threads: chunk
+// The 256 x 64 activation slab as 16-byte chunks, chunk-major over the 512 threads: chunk
 // g = 512 j + t (j-th load of thread t) is chunk g % CPR of row g / CPR, so consecutive lanes read
-// consecutive 16 bytes of one row (a wavefront covers 4 full rows = 8 cache lines per load
-// instead of 64 lines with a row-per-lane assignment, which leaves the kernel bound by the
-// texture addresser).
+// consecutive 16 bytes of one row (a row-per-lane assignment touches 64 cache lines per load
+// and leaves the kernel bound by the texture addresser).
 template <bool BF16> struct XRaw;
+__device__ __forceinline__ uint32_t all_ones_if(bool c) { return c ? 0xFFFFFFFFu : 0u; }
+// Addressing: a uniform base pointer (tile row 0, column of the K step) advances on the scalar unit;
+// each thread adds constant 32-bit byte offsets (its row, clamped to M - 1, and its chunk).  In a
+// last step that covers only 32 columns the chunks of the missing half re-read the first half;
+// store_part zeroes them.
 template <> struct XRaw<true> {
-    static constexpr int CPR = 16, NCH = 8;  // chunks per row (8 bf16 each), chunks per thread
+    static constexpr int CPR = 8, NCH = 4;  // chunks per row (8 bf16 each), chunks per thread
+    static constexpr int ESIZE = 2;
     uint4 v[NCH];
-    __device__ __forceinline__ void load(const void *X, int bm, int M, int k0, int K, int tid) {
-        const uint16_t *p = reinterpret_cast<const uint16_t *>(X);
-#pragma unroll
-        for (int j = 0; j < NCH; j++) {
-            const int g = 512 * j + tid, row = g / CPR, k = k0 + (g % CPR) * 8;
-            v[j] = *reinterpret_cast<const uint4 *>(p + (int64_t)min(bm + row, M - 1) * K + (k < K ? k : 0));
-        }
+    static __device__ __forceinline__ uint32_t offset(int j, int bm, int M, int K, int tid, bool tail) {
+        const int g = 512 * j + tid, row = g / CPR;
+        int c = g % CPR;
+        if (tail && c >= CPR / 2) c -= CPR / 2;
+        return (uint32_t)(min(row, M - 1 - bm) * K + c * 8) * ESIZE;
     }
-    __device__ __forceinline__ void store(uint16_t *xs, int bm, int M, int k0, int K, int tid) const {
+    __device__ __forceinline__ void load(const uint8_t *base, const uint32_t *off) {
 #pragma unroll
-        for (int j = 0; j < NCH; j++) {
-            const int g = 512 * j + tid, row = g / CPR, c = g % CPR;
-            const bool ok = bm + row < M && k0 + c * 8 < K;
-            *reinterpret_cast<uint4 *>(xs + row * LDS_STRIDE + c * 8) = ok ? v[j] : make_uint4(0, 0, 0, 0);
-        }
+        for (int j = 0; j < NCH; j++) v[j] = *reinterpret_cast<const uint4 *>(base + off[j]);
+    }
+    // the loads that refill what store_part(i) has just consumed
+    __device__ __forceinline__ void load_part(int i, const uint8_t *base, const uint32_t *off) {
+        v[i] = *reinterpret_cast<const uint4 *>(base + off[i]);
+    }
+    // Part i of 4 of the copy into LDS.  Columns at or beyond K become zero; rows beyond M hold a
+    // copy of row M - 1 and only feed outputs that are never written.
+    __device__ __forceinline__ void store_part(int i, uint16_t *xs, int k0, int K, int tid) const {
+        const int g = 512 * i + tid, row = g / CPR, c = g % CPR;
+        const uint32_t m = all_ones_if(k0 + c * 8 < K);
+        *reinterpret_cast<uint4 *>(xs + row * LDS_STRIDE + c * 8) = make_uint4(v[i].x & m, v[i].y & m, v[i].z & m, v[i].w & m);
     }
 };
 template <> struct XRaw<false> {
-    static constexpr int CPR = 32, NCH = 16;  // chunks per row (4 fp32 each), chunks per thread
+    static constexpr int CPR = 16, NCH = 8;  // chunks per row (4 fp32 each), chunks per thread
+    static constexpr int ESIZE = 4;
     float4 v[NCH];
-    __device__ __forceinline__ void load(const void *X, int bm, int M, int k0, int K, int tid) {
-        const float *p = reinterpret_cast<const float *>(X);
-#pragma unroll
-        for (int j = 0; j < NCH; j++) {
-            const int g = 512 * j + tid, row = g / CPR, k = k0 + (g % CPR) * 4;
-            v[j] = *reinterpret_cast<const float4 *>(p + (int64_t)min(bm + row, M - 1) * K + (k < K ? k : 0));
-        }
+    static __device__ __forceinline__ uint32_t offset(int j, int bm, int M, int K, int tid, bool tail) {
+        const int g = 512 * j + tid, row = g / CPR;
+        int c = g % CPR;
+        if (tail && c >= CPR / 2) c -= CPR / 2;
+        return (uint32_t)(min(row, M - 1 - bm) * K + c * 4) * ESIZE;
     }
-    __device__ __forceinline__ void store(uint16_t *xs, int bm, int M, int k0, int K, int tid) const {
+    __device__ __forceinline__ void load(const uint8_t *base, const uint32_t *off) {
 #pragma unroll
-        for (int j = 0; j < NCH; j++) {
+        for (int j = 0; j < NCH; j++) v[j] = *reinterpret_cast<const float4 *>(base + off[j]);
+    }
+    __device__ __forceinline__ void load_part(int i, const uint8_t *base, const uint32_t *off) {
+        v[2 * i] = *reinterpret_cast<const float4 *>(base + off[2 * i]);
+        v[2 * i + 1] = *reinterpret_cast<const float4 *>(base + off[2 * i + 1]);
+    }
+    __device__ __forceinline__ void store_part(int i, uint16_t *xs, int k0, int K, int tid) const {
+#pragma unroll
+        for (int j = 2 * i; j < 2 * i + 2; j++) {
             const int g = 512 * j + tid, row = g / CPR, c = g % CPR;
-            const bool ok = bm + row < M && k0 + c * 4 < K;
-            const uint2 h = make_uint2(Operand<false>::pack(v[j].x, v[j].y), Operand<false>::pack(v[j].z, v[j].w));
-            *reinterpret_cast<uint2 *>(xs + row * LDS_STRIDE + c * 4) = ok ? h : make_uint2(0, 0);
+            const uint32_t m = all_ones_if(k0 + c * 4 < K);
+            *reinterpret_cast<uint2 *>(xs + row * LDS_STRIDE + c * 4) =
+                make_uint2(Operand<false>::pack(v[j].x, v[j].y) & m, Operand<false>::pack(v[j].z, v[j].w) & m);
         }
     }
 };
 
-// X must be 16-byte aligned; K % 32 == 0.  One LDS stage of BK = 128: the MFMA phase of a step
-// (32 MFMAs per wavefront) is long enough to cover the global-memory latency of the next
-// step's loads, which wait in registers and are converted and stored between two barriers.
+#ifdef GQ_GEMM_TRACE
+__device__ unsigned long long g_gemm_trace[4 * 8 * 8];
+#endif
+
+// X must be 16-byte aligned; K % 32 == 0.
 template <int T, bool BF16>
-__global__ __launch_bounds__(512) void gemm_kernel(const void *__restrict__ Xv, const uint8_t *__restrict__ W,
+// (Xv and W are deliberately not __restrict__: loads through restrict-qualified read-only pointers
+// may be moved across the workgroup barriers, away from the place that gives them two steps of
+// latency cover.)
+__global__ __launch_bounds__(512) void gemm_kernel(const void *Xv, const uint8_t *W,
                                                    const float *__restrict__ bias, float *__restrict__ Y, int M, int K,
                                                    int N, int64_t row_bytes, int act) {
     typedef Operand<BF16> Op;
@@ -169,60 +189,162 @@ __global__ __launch_bounds__(512) void gemm_kernel(const void *__restrict__ Xv, 
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-    // staging role for W: 128 rows x 4 runs of 32 weights
-    const int wrow_i = tid >> 2, wblk = tid & 3;
-    const uint8_t *wrow = W + (int64_t)min(bn + wrow_i, N - 1) * row_bytes;
-    uint16_t *wdst = lds + (BM + wrow_i) * LDS_STRIDE + 32 * wblk;
+    // staging role for W: 128 rows x 4 runs of 16 weights
+    const int wrow_i = tid >> 2, wrun = tid & 3;
+    const int wrow_c = min(wrow_i, N - 1 - bn);  // clamped row within the tile
+    const int wdst_off = (BM + wrow_i) * LDS_STRIDE + 16 * wrun;
 
-    XRaw<BF16> xr[1];
-    WRaw<T> wr[1];
+    XRaw<BF16> xr[2];
+    WRaw<T> wr[2];
+    wr[0].set_row(W + (int64_t)(bn + wrow_c) * row_bytes);
+    wr[1].set_row(W + (int64_t)(bn + wrow_c) * row_bytes);
     const int nk = (K + BK - 1) / BK;
-    const int64_t nblk32 = K >> 5;
-    auto fetch = [&](int kt, XRaw<BF16> &x, WRaw<T> &w) {
-        const int k0 = kt * BK;
-        x.load(Xv, bm, M, k0, K, tid);
-        w.load(wrow, min((int64_t)(k0 >> 5) + wblk, nblk32 - 1));
-    };
-    auto stage = [&](int kt, const XRaw<BF16> &x, const WRaw<T> &wq) {
-        const int k0 = kt * BK;
-        x.store(lds, bm, M, k0, K, tid);
-        float w[32];
-        wq.values(w);
-        const bool w_ok = k0 + 32 * wblk < K;
-        uint4 *d = reinterpret_cast<uint4 *>(wdst);
+    const int64_t n16 = K >> 4;
+    const bool ktail = (K % BK) != 0;  // the last step covers 32 columns only
+    // constant per-thread byte offsets, for full steps and for a half last step
+    uint32_t xoff[XRaw<BF16>::NCH], xoff_t[XRaw<BF16>::NCH];
 #pragma unroll
-        for (int j = 0; j < 4; j++)
-            d[j] = w_ok ? make_uint4(Op::pack(w[8 * j], w[8 * j + 1]), Op::pack(w[8 * j + 2], w[8 * j + 3]),
-                                     Op::pack(w[8 * j + 4], w[8 * j + 5]), Op::pack(w[8 * j + 6], w[8 * j + 7]))
-                        : make_uint4(0, 0, 0, 0);
-    };
-    const uint16_t *xs = lds, *ws = lds + BM * LDS_STRIDE;
-    auto contract = [&]() {
+    for (int j = 0; j < XRaw<BF16>::NCH; j++) {
+        xoff[j] = XRaw<BF16>::offset(j, bm, M, K, tid, false);
+        xoff_t[j] = XRaw<BF16>::offset(j, bm, M, K, tid, true);
+    }
+    const uint32_t woff = (uint32_t)(wrow_c * row_bytes) + (uint32_t)(wrun >> 1) * 34u;
+    const uint32_t woff_t = (uint32_t)(wrow_c * row_bytes);  // half last step: runs 2, 3 re-read block 0
+    const uint8_t *xtile = reinterpret_cast<const uint8_t *>(Xv) + (int64_t)bm * K * XRaw<BF16>::ESIZE;
+    const uint8_t *wtile = W + (int64_t)bn * row_bytes;
+    auto fetch = [&](int kt, XRaw<BF16> &x, WRaw<T> &w) {  // unconditional: steps past the end re-read the last one
+#ifdef GQ_GEMM_NOFETCH  // tuning builds only
+        if (kt > 2) return;
+#endif
+#ifdef GQ_GEMM_HOTFETCH  // tuning builds only: every step re-reads step 0
+        const int kc = min(kt, 0);
+#else
+        const int kc = min(kt, nk - 1);  // uniform
+#endif
+        const bool tail = ktail && kc == nk - 1;
+        const uint8_t *xb = xtile + (int64_t)kc * (BK * XRaw<BF16>::ESIZE);
+        uint32_t o[XRaw<BF16>::NCH];
 #pragma unroll
-        for (int kk = 0; kk < BK / 16; kk++) {
+        for (int j = 0; j < XRaw<BF16>::NCH; j++) o[j] = tail ? xoff_t[j] : xoff[j];
+        x.load(xb, o);
+        w.load(wtile + (int64_t)kc * (BK / 32 * 34), tail ? woff_t : woff, (uint32_t)wrun,
+               min((int64_t)kc * (BK / 16) + wrun, n16 - 1));
+    };
+#ifdef GQ_GEMM_TRACE  // tuning builds only: cycle stamps of one pair of steps per wavefront
+#define GEMM_TRACE(slot) do { if (kt == 16 && lane == 0 && blockIdx.x < 4 && blockIdx.y == 0) g_gemm_trace[(blockIdx.x * 8 + wave) * 8 + (slot)] = __builtin_readcyclecounter(); } while (0)
+#else
+#define GEMM_TRACE(slot) do { } while (0)
+#endif
+    // One K step: the 16 MFMAs of step kt out of `cur`, in four groups of four, each group followed
+    // in program order by a quarter of the staging of step kt + 1 into `nxt` (MFMAs are issued
+    // asynchronously, so the vector ALU work that follows them runs in their shadow).  Fragments
+    // are read one group ahead.  The scheduling barriers keep the compiler from regrouping this.
+    auto step = [&](int kt, const uint16_t *cur, uint16_t *nxt, XRaw<BF16> &x, WRaw<T> &wq) {
+        const uint16_t *xs = cur, *ws = cur + BM * LDS_STRIDE;
+        const int k1 = (kt + 1) * BK;
+        // the register set staged here is refilled, piece by piece, with step kt + 3
+#ifdef GQ_GEMM_HOTFETCH  // tuning builds only: every step re-reads step 0
+        const int kc = 0;
+#else
+        const int kc = min(kt + 3, nk - 1);  // uniform; steps past the end re-read the last one
+#endif
+        const bool ftail = ktail && kc == nk - 1;
+        const uint8_t *xb = xtile + (int64_t)kc * (BK * XRaw<BF16>::ESIZE);
+        uint32_t fo[XRaw<BF16>::NCH];
+#pragma unroll
+        for (int j = 0; j < XRaw<BF16>::NCH; j++) fo[j] = ftail ? xoff_t[j] : xoff[j];
+        const uint32_t wmask = all_ones_if(k1 + 16 * wrun < K);
+        uint4 *wd = reinterpret_cast<uint4 *>(nxt + wdst_off);
+        typename Op::vec8 a[2][2], b[2][2];
+        auto frags = [&](int kk, typename Op::vec8 *fa, typename Op::vec8 *fb) {
             const int koff = kk * 16 + (lane >> 5) * 8;
-            typename Op::vec8 a[2], b[2];
 #pragma unroll
             for (int i = 0; i < 2; i++)
-                a[i] = *reinterpret_cast<const typename Op::vec8 *>(&xs[(wm + i * 32 + (lane & 31)) * LDS_STRIDE + koff]);
+                fa[i] = *reinterpret_cast<const typename Op::vec8 *>(&xs[(wm + i * 32 + (lane & 31)) * LDS_STRIDE + koff]);
 #pragma unroll
             for (int j = 0; j < 2; j++)
-                b[j] = *reinterpret_cast<const typename Op::vec8 *>(&ws[(wn + j * 32 + (lane & 31)) * LDS_STRIDE + koff]);
+                fb[j] = *reinterpret_cast<const typename Op::vec8 *>(&ws[(wn + j * 32 + (lane & 31)) * LDS_STRIDE + koff]);
+        };
+        float w[16];
+        frags(0, a[0], b[0]);
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+            if (kk < 3) frags(kk + 1, a[(kk + 1) & 1], b[(kk + 1) & 1]);
 #pragma unroll
             for (int i = 0; i < 2; i++)
 #pragma unroll
-                for (int j = 0; j < 2; j++) acc[i][j] = Op::mfma(a[i], b[j], acc[i][j]);
+                for (int j = 0; j < 2; j++) {
+#ifndef GQ_GEMM_NOMFMA  // tuning builds only
+                    acc[i][j] = Op::mfma(a[kk & 1][i], b[kk & 1][j], acc[i][j]);
+#endif
+                }
+#ifndef GQ_GEMM_NOSTAGE  // tuning builds only
+            x.store_part(kk, nxt, k1, K, tid);
+            wq.part(kk, w);
+#endif
+#ifndef GQ_GEMM_NOFETCH
+            x.load_part(kk, xb, fo);
+#endif
+            if (kk == 1 || kk == 3) {
+                const int o = (kk >> 1) * 8;
+                wd[kk >> 1] = make_uint4(Op::pack(w[o], w[o + 1]) & wmask, Op::pack(w[o + 2], w[o + 3]) & wmask,
+                                         Op::pack(w[o + 4], w[o + 5]) & wmask, Op::pack(w[o + 6], w[o + 7]) & wmask);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (cur == lds) GEMM_TRACE(1 + kk);
         }
+#ifndef GQ_GEMM_NOFETCH
+        wq.load(wtile + (int64_t)kc * (BK / 32 * 34), ftail ? woff_t : woff, (uint32_t)wrun,
+                min((int64_t)kc * (BK / 16) + wrun, n16 - 1));
+#endif
+    };
+    auto stage_first = [&](uint16_t *buf, const XRaw<BF16> &x, const WRaw<T> &wq) {
+        float w[16];
+        const uint32_t wmask = all_ones_if(16 * wrun < K);
+        uint4 *wd = reinterpret_cast<uint4 *>(buf + wdst_off);
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+            x.store_part(kk, buf, 0, K, tid);
+            wq.part(kk, w);
+        }
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+            wd[h] = make_uint4(Op::pack(w[8 * h], w[8 * h + 1]) & wmask, Op::pack(w[8 * h + 2], w[8 * h + 3]) & wmask,
+                               Op::pack(w[8 * h + 4], w[8 * h + 5]) & wmask, Op::pack(w[8 * h + 6], w[8 * h + 7]) & wmask);
     };
 
+    // Step s is staged (registers -> LDS buffer s % 2) during step s - 1 out of register set s % 2,
+    // which was filled by fetch(s) during step s - 3.  Steps come in pairs so that every pass of
+    // the loop body issues the same loads (the wait counters then stay exact); a step past the end
+    // of K stages zeros.
+    // (the scheduling barriers pin the order of issue, which is what the wait counts in the loop
+    // are derived from)
     fetch(0, xr[0], wr[0]);
-    for (int kt = 0; kt < nk; kt++) {
-        stage(kt, xr[0], wr[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    fetch(1, xr[1], wr[1]);
+    __builtin_amdgcn_sched_barrier(0);
+    stage_first(lds, xr[0], wr[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    fetch(2, xr[0], wr[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    auto pair = [&](int kt) {
+        GEMM_TRACE(0);
+        step(kt, lds, lds + LDS_BUF, xr[1], wr[1]);
+        __builtin_amdgcn_sched_barrier(0);
+        GEMM_TRACE(5);
         __syncthreads();
-        fetch(min(kt + 1, nk - 1), xr[0], wr[0]);  // unconditional (clamped): in flight during the MFMA phase
-        contract();
+        GEMM_TRACE(6);
+        step(kt + 1, lds + LDS_BUF, lds, xr[0], wr[0]);
+        __builtin_amdgcn_sched_barrier(0);
+        GEMM_TRACE(7);
         __syncthreads();
-    }
+    };
+    // The first pair runs outside the loop so that the loop is entered with exactly the loads in
+    // flight that its own back edge leaves (otherwise the wait counts at the loop head are derived
+    // from the prologue's different order and over-wait).
+    pair(0);
+    for (int kt = 2; kt < nk; kt += 2) pair(kt);
 
     // ---- epilogue: acc[i][j][r] is Y[m, n] with n = lane % 32, m = 8*(r/4) + 4*(lane/32) + r%4
 #pragma unroll
