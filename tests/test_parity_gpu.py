@@ -112,6 +112,28 @@ def test_gemv_parity(gpu, oracle, t, M, K, N):
         assert rel_err(got, want) < TOL_F32, (t, M, K, N, act)
 
 
+@pytest.mark.parametrize("t", [Q4_0, Q8_0, Q4_K])
+@pytest.mark.parametrize("M,K,N", [
+    (1, 1536, 100),     # 3 slices of 512: three wavefronts per workgroup
+    (2, 3584, 513),     # 7 slices, rows not a multiple of 8
+    (1, 4608, 40),      # 9 slices: no usable split, activation-stationary fallback
+    (1, 8192, 2100),    # two slices per wavefront
+    (3, 2048, 20000),   # five row-steps per wavefront, all in flight
+    (1, 512, 300000),   # one wavefront per workgroup, many groups of four row-steps
+    (1, 8192, 40000),   # groups of four row-steps wrapping from one slice to the next
+])
+def test_gemv_k_sliced_plans(gpu, oracle, t, M, K, N):
+    """Shapes that walk through the planner of the K-sliced decode kernel (wavefronts per
+    workgroup, slices per wavefront, prefetch groups) and its fallback."""
+    W = synth.weights(t, 40 + t, N, K)
+    x = synth.activations(41 + t, M, K)
+    bias = synth.normal(42 + t, 0, N).astype(np.float32) * 0.1
+    got = run_dense(gpu, t, x, W, bias, 0)
+    want = oracle.c_qdense(t, x, W, bias, 0)
+    assert got.shape == (M, N)
+    assert rel_err(got, want) < TOL_F32, (t, M, K, N)
+
+
 @pytest.mark.parametrize("t", ALL_TYPES)
 def test_gemv_long_k_is_chunked(gpu, oracle, t):
     """K above the 16384 values one LDS pass holds."""
