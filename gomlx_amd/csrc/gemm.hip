@@ -17,6 +17,8 @@
 #include "blocks.hpp"
 #include "common.hpp"
 
+#include <type_traits>
+
 namespace gq {
 
 namespace {
@@ -127,9 +129,11 @@ template <> struct XRaw<true> {
     }
     // Part i of 4 of the copy into LDS.  Columns at or beyond K become zero; rows beyond M hold a
     // copy of row M - 1 and only feed outputs that are never written.
+    // MASKED = false is for steps that lie entirely inside K.
+    template <bool MASKED>
     __device__ __forceinline__ void store_part(int i, uint16_t *xs, int k0, int K, int tid) const {
         const int g = 512 * i + tid, row = g / CPR, c = g % CPR;
-        const uint32_t m = all_ones_if(k0 + c * 8 < K);
+        const uint32_t m = MASKED ? all_ones_if(k0 + c * 8 < K) : 0xFFFFFFFFu;
         *reinterpret_cast<uint4 *>(xs + row * LDS_STRIDE + c * 8) = make_uint4(v[i].x & m, v[i].y & m, v[i].z & m, v[i].w & m);
     }
 };
@@ -151,11 +155,12 @@ template <> struct XRaw<false> {
         v[2 * i] = *reinterpret_cast<const float4 *>(base + off[2 * i]);
         v[2 * i + 1] = *reinterpret_cast<const float4 *>(base + off[2 * i + 1]);
     }
+    template <bool MASKED>
     __device__ __forceinline__ void store_part(int i, uint16_t *xs, int k0, int K, int tid) const {
 #pragma unroll
         for (int j = 2 * i; j < 2 * i + 2; j++) {
             const int g = 512 * j + tid, row = g / CPR, c = g % CPR;
-            const uint32_t m = all_ones_if(k0 + c * 4 < K);
+            const uint32_t m = MASKED ? all_ones_if(k0 + c * 4 < K) : 0xFFFFFFFFu;
             *reinterpret_cast<uint2 *>(xs + row * LDS_STRIDE + c * 4) =
                 make_uint2(Operand<false>::pack(v[j].x, v[j].y) & m, Operand<false>::pack(v[j].z, v[j].w) & m);
         }
@@ -239,7 +244,8 @@ __global__ __launch_bounds__(512) void gemm_kernel(const void *Xv, const uint8_t
     // in program order by a quarter of the staging of step kt + 1 into `nxt` (MFMAs are issued
     // asynchronously, so the vector ALU work that follows them runs in their shadow).  Fragments
     // are read one group ahead.  The scheduling barriers keep the compiler from regrouping this.
-    auto step = [&](int kt, const uint16_t *cur, uint16_t *nxt, XRaw<BF16> &x, WRaw<T> &wq) {
+    auto step = [&](int kt, const uint16_t *cur, uint16_t *nxt, XRaw<BF16> &x, WRaw<T> &wq, auto masked) {
+        constexpr bool MASKED = decltype(masked)::value;
         const uint16_t *xs = cur, *ws = cur + BM * LDS_STRIDE;
         const int k1 = (kt + 1) * BK;
         // the register set staged here is refilled, piece by piece, with step kt + 3
@@ -253,7 +259,7 @@ __global__ __launch_bounds__(512) void gemm_kernel(const void *Xv, const uint8_t
         uint32_t fo[XRaw<BF16>::NCH];
 #pragma unroll
         for (int j = 0; j < XRaw<BF16>::NCH; j++) fo[j] = ftail ? xoff_t[j] : xoff[j];
-        const uint32_t wmask = all_ones_if(k1 + 16 * wrun < K);
+        const uint32_t wmask = MASKED ? all_ones_if(k1 + 16 * wrun < K) : 0xFFFFFFFFu;
         uint4 *wd = reinterpret_cast<uint4 *>(nxt + wdst_off);
         typename Op::vec8 a[2][2], b[2][2];
         auto frags = [&](int kk, typename Op::vec8 *fa, typename Op::vec8 *fb) {
@@ -279,7 +285,7 @@ __global__ __launch_bounds__(512) void gemm_kernel(const void *Xv, const uint8_t
 #endif
                 }
 #ifndef GQ_GEMM_NOSTAGE  // tuning builds only
-            x.store_part(kk, nxt, k1, K, tid);
+            x.template store_part<MASKED>(kk, nxt, k1, K, tid);
             wq.part(kk, w);
 #endif
 #ifndef GQ_GEMM_NOFETCH
@@ -304,7 +310,7 @@ __global__ __launch_bounds__(512) void gemm_kernel(const void *Xv, const uint8_t
         uint4 *wd = reinterpret_cast<uint4 *>(buf + wdst_off);
 #pragma unroll
         for (int kk = 0; kk < 4; kk++) {
-            x.store_part(kk, buf, 0, K, tid);
+            x.template store_part<true>(kk, buf, 0, K, tid);
             wq.part(kk, w);
         }
 #pragma unroll
@@ -328,23 +334,27 @@ __global__ __launch_bounds__(512) void gemm_kernel(const void *Xv, const uint8_t
     fetch(2, xr[0], wr[0]);
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
-    auto pair = [&](int kt) {
+    auto pair = [&](int kt, auto masked) {
         GEMM_TRACE(0);
-        step(kt, lds, lds + LDS_BUF, xr[1], wr[1]);
+        step(kt, lds, lds + LDS_BUF, xr[1], wr[1], masked);
         __builtin_amdgcn_sched_barrier(0);
         GEMM_TRACE(5);
         __syncthreads();
         GEMM_TRACE(6);
-        step(kt + 1, lds + LDS_BUF, lds, xr[0], wr[0]);
+        step(kt + 1, lds + LDS_BUF, lds, xr[0], wr[0], masked);
         __builtin_amdgcn_sched_barrier(0);
         GEMM_TRACE(7);
         __syncthreads();
     };
     // The first pair runs outside the loop so that the loop is entered with exactly the loads in
     // flight that its own back edge leaves (otherwise the wait counts at the loop head are derived
-    // from the prologue's different order and over-wait).
-    pair(0);
-    for (int kt = 2; kt < nk; kt += 2) pair(kt);
+    // from the prologue's different order and over-wait).  Pairs whose staged steps (kt + 1, kt + 2)
+    // lie entirely inside K skip the zero-fill masks.
+    const int nk_full = K / BK;
+    pair(0, std::true_type());
+    int kt = 2;
+    for (; kt + 2 < nk_full; kt += 2) pair(kt, std::false_type());
+    for (; kt < nk; kt += 2) pair(kt, std::true_type());
 
     // ---- epilogue: acc[i][j][r] is Y[m, n] with n = lane % 32, m = 8*(r/4) + 4*(lane/32) + r%4
 #pragma unroll
