@@ -55,6 +55,7 @@ bool type_info(int type, TypeInfo &ti) {
     case GQ_Q4_0: ti = {18, 32}; return true;
     case GQ_Q8_0: ti = {34, 32}; return true;
     case GQ_Q4_K: ti = {144, 256}; return true;
+    case GQ_Q6_K: ti = {210, 256}; return true;
     case GQ_IQ4_NL: ti = {18, 32}; return true;
     default: return false;
     }

@@ -11,7 +11,7 @@
 
 namespace gq {
 
-constexpr int kQ4_0 = 2, kQ8_0 = 8, kQ4_K = 12, kIQ4_NL = 20;
+constexpr int kQ4_0 = 2, kQ8_0 = 8, kQ4_K = 12, kQ6_K = 14, kIQ4_NL = 20;
 constexpr int kActNone = 0, kActGelu = 1, kActRelu = 2, kActSilu = 3, kActHardSwish = 4, kActTanh = 5;
 
 template <int T> struct Geom;
@@ -19,6 +19,7 @@ template <> struct Geom<kQ4_0> { static constexpr int bpb = 18, vpb = 32; };
 template <> struct Geom<kQ8_0> { static constexpr int bpb = 34, vpb = 32; };
 template <> struct Geom<kIQ4_NL> { static constexpr int bpb = 18, vpb = 32; };
 template <> struct Geom<kQ4_K> { static constexpr int bpb = 144, vpb = 256; };
+template <> struct Geom<kQ6_K> { static constexpr int bpb = 210, vpb = 256; };
 
 // 16 bytes that are only guaranteed to be 2-byte aligned (Q4_0 / Q8_0 payloads start two
 // bytes into an 18- or 34-byte block).  gfx950 global loads accept unaligned addresses, so
@@ -145,6 +146,32 @@ __device__ __forceinline__ void dequant16<kQ4_K>(const uint8_t *__restrict__ row
         for (int j = 0; j < 4; j++) {
             const uint32_t nib = (qq[w] >> (8 * j + 4 * h)) & 0x0Fu;
             out[4 * w + j] = ds * (float)nib - dm;
+        }
+    }
+}
+
+// Q6_K super-block: 128 bytes ql (low 4 bits), 64 bytes qh (high 2 bits), 16 int8 scales, fp16 d
+// (210 bytes, 2-byte aligned).  Run i of 16 values lies in half h = i / 8 of the block, quadrant
+// qd = (i / 2) % 4 (which selects 32 of the 64 ql bytes, the nibble, and the 2-bit field of qh)
+// and covers l = 16 (i % 2) .. + 15, i.e. one scale.  w = (d * scale) * (q - 32): the exact product
+// has at most 24 significant bits, so the order of the multiplications does not matter.
+template <>
+__device__ __forceinline__ void dequant16<kQ6_K>(const uint8_t *__restrict__ row, int64_t i, float *out) {
+    const uint8_t *sb = row + (i >> 4) * 210;
+    const int r = (int)(i & 15);
+    const int h = r >> 3, qd = (r >> 1) & 3, l0 = (r & 1) * 16;
+    const u128_a2 ql = *reinterpret_cast<const u128_a2 *>(sb + 64 * h + 32 * (qd & 1) + l0);
+    const u128_a2 qh = *reinterpret_cast<const u128_a2 *>(sb + 128 + 32 * h + l0);
+    const int sc = (int)(int8_t)sb[192 + 8 * h + 2 * qd + (r & 1)];
+    const float ds = half_bits_to_float(load_u16(sb + 208)) * (float)sc;
+    const int nsh = (qd >> 1) * 4, hsh = 2 * qd;
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t lo = (ql.v[w] >> (8 * j + nsh)) & 0x0Fu;
+            const uint32_t hi = (qh.v[w] >> (8 * j + hsh)) & 0x03u;
+            out[4 * w + j] = ds * (float)((int)(lo | (hi << 4)) - 32);
         }
     }
 }

@@ -59,6 +59,7 @@ static int dispatch_rows(int type, const uint8_t *W, float *out, int64_t N, int6
     case kQ4_0: return launch_rows<kQ4_0>(W, out, N, K, indices, vocab, err_flag, s);
     case kIQ4_NL: return launch_rows<kIQ4_NL>(W, out, N, K, indices, vocab, err_flag, s);
     case kQ4_K: return launch_rows<kQ4_K>(W, out, N, K, indices, vocab, err_flag, s);
+    case kQ6_K: return launch_rows<kQ6_K>(W, out, N, K, indices, vocab, err_flag, s);
     default: return fail(GQ_ERR_NOT_IMPLEMENTED, "dequantize: ggml type %d is not implemented", type);
     }
 }

@@ -409,6 +409,7 @@ int launch_gemm(int type, bool x_is_bf16, const void *x, int64_t M, int64_t K, c
     case kQ8_0: return launch_type<kQ8_0>(x_is_bf16, x, M, K, W, N, bias, act, y, s);
     case kIQ4_NL: return launch_type<kIQ4_NL>(x_is_bf16, x, M, K, W, N, bias, act, y, s);
     case kQ4_K: return launch_type<kQ4_K>(x_is_bf16, x, M, K, W, N, bias, act, y, s);
+    case kQ6_K: return launch_type<kQ6_K>(x_is_bf16, x, M, K, W, N, bias, act, y, s);
     default: return fail(GQ_ERR_NOT_IMPLEMENTED, "qdense: ggml type %d is not implemented", type);
     }
 }

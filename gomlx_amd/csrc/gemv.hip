@@ -448,6 +448,49 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_q4k_kernel(const float *__res
     }
 }
 
+// ---- formats that only provide the 16-value decoder (Q6_K): one wavefront per row, lanes stride
+// over the runs of 16 weights, activations straight from global memory (they stay in L2).
+template <int T, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gemv_run16_kernel(const float *__restrict__ X, const uint8_t *__restrict__ W,
+                                                                const float *__restrict__ bias, float *__restrict__ Y, int K, int N,
+                                                                int64_t row_bytes, int act, int x_aligned) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int row = blockIdx.x * WAVES + wave;
+    if (row >= N) return;
+    const float *x = X + (int64_t)blockIdx.y * K;
+    const uint8_t *wrow = W + (int64_t)row * row_bytes;
+    const int runs = K >> 4;
+    float acc = 0.f;
+    for (int i = lane; i < runs; i += 64) {
+        float w[16], xv[16];
+        dequant16<T>(wrow, i, w);
+        if (x_aligned) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float4 t = reinterpret_cast<const float4 *>(x)[4 * i + j];
+                xv[4 * j] = t.x; xv[4 * j + 1] = t.y; xv[4 * j + 2] = t.z; xv[4 * j + 3] = t.w;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 16; j++) xv[j] = x[16 * i + j];
+        }
+#pragma unroll
+        for (int j = 0; j < 16; j++) acc = fmaf(w[j], xv[j], acc);
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) Y[(int64_t)blockIdx.y * N + row] = apply_act(act, acc + (bias ? bias[row] : 0.f));
+}
+
+template <int T>
+int launch_run16(const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y,
+                 hipStream_t s) {
+    constexpr int WAVES = 4;
+    const int64_t row_bytes = (K / Geom<T>::vpb) * Geom<T>::bpb;
+    const dim3 grid((unsigned)((N + WAVES - 1) / WAVES), (unsigned)M);
+    const int aligned = (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (K % 4) == 0;
+    return launch(gemv_run16_kernel<T, WAVES>, grid, dim3(WAVES * 64), 0, s, x, W, bias, y, (int)K, (int)N, row_bytes, act, aligned);
+}
+
 // ---- host side --------------------------------------------------------------------------
 
 struct Tuning { int rows_per_wave; int waves; };
@@ -524,6 +567,7 @@ int launch_gemv(int type, const float *x, int64_t M, int64_t K, const uint8_t *W
     case kQ8_0: return launch_type<kQ8_0>(x, M, K, W, N, bias, act, y, s);
     case kIQ4_NL: return launch_type<kIQ4_NL>(x, M, K, W, N, bias, act, y, s);
     case kQ4_K: return launch_type<kQ4_K>(x, M, K, W, N, bias, act, y, s);
+    case kQ6_K: return launch_run16<kQ6_K>(x, M, K, W, N, bias, act, y, s);
     default: return fail(GQ_ERR_NOT_IMPLEMENTED, "qdense: ggml type %d is not implemented", type);
     }
 }

@@ -9,10 +9,11 @@ from __future__ import annotations
 Q4_0 = 2
 Q8_0 = 8
 Q4_K = 12
+Q6_K = 14
 IQ4_NL = 20
 
-_GEOM = {Q4_0: (18, 32), Q8_0: (34, 32), Q4_K: (144, 256), IQ4_NL: (18, 32)}
-_NAMES = {Q4_0: "Q4_0", Q8_0: "Q8_0", Q4_K: "Q4_K", IQ4_NL: "IQ4_NL"}
+_GEOM = {Q4_0: (18, 32), Q8_0: (34, 32), Q4_K: (144, 256), Q6_K: (210, 256), IQ4_NL: (18, 32)}
+_NAMES = {Q4_0: "Q4_0", Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K", IQ4_NL: "IQ4_NL"}
 
 
 def name(t: int) -> str:

@@ -56,7 +56,7 @@ struct Shape {
 
 // compute.QuantizationScheme / GGMLQuantType / ActivationType
 enum class QuantScheme { Linear, NF4, GGML };
-enum class GGMLQuantType { Q4_0 = GQ_Q4_0, Q8_0 = GQ_Q8_0, Q4_K = GQ_Q4_K, IQ4NL = GQ_IQ4_NL, Q6_K = 14 };
+enum class GGMLQuantType { Q4_0 = GQ_Q4_0, Q8_0 = GQ_Q8_0, Q4_K = GQ_Q4_K, Q6_K = GQ_Q6_K, IQ4NL = GQ_IQ4_NL };
 inline int BytesPerBlock(GGMLQuantType t) { return gq_bytes_per_block((int)t); }
 inline int ValuesPerBlock(GGMLQuantType t) { return gq_values_per_block((int)t); }
 enum class ActivationType { None = GQ_ACT_NONE, Gelu = GQ_ACT_GELU, Relu = GQ_ACT_RELU, Silu = GQ_ACT_SILU,

@@ -271,7 +271,7 @@ static void TestBuildTimeErrors() {
     auto wf = f.Parameter("wf", Shape{DType::Float32, {2, 34}}).first;
     auto bias3 = f.Parameter("b", Shape{DType::Float32, {3}}).first;
     auto xi = f.Parameter("xi", Shape{DType::Int32, {1, 32}}).first;
-    Quantization q8 = GGML(GGMLQuantType::Q8_0), q4 = GGML(GGMLQuantType::Q4_0), q6k = GGML(GGMLQuantType::Q6_K), q4k = GGML(GGMLQuantType::Q4_K);
+    Quantization q8 = GGML(GGMLQuantType::Q8_0), q4 = GGML(GGMLQuantType::Q4_0), q5k = GGML(GGMLQuantType(13)), q4k = GGML(GGMLQuantType::Q4_K);
     Quantization lin; lin.scheme = QuantScheme::Linear;
     // nil wq is a hard error (core/graph/fused_ops.go:198-200)
     auto r = f.FusedQuantizedDense(x, w, Value(), nullptr, ActivationType::None);
@@ -279,8 +279,8 @@ static void TestBuildTimeErrors() {
     // schemes and types outside the backend are "not implemented": the caller may fall back
     r = f.FusedQuantizedDense(x, w, Value(), &lin, ActivationType::None);
     CHECK(IsNotImplemented(r.second), "Linear scheme: status %d", r.second.status);
-    r = f.FusedQuantizedDense(x, w, Value(), &q6k, ActivationType::None);
-    CHECK(IsNotImplemented(r.second), "Q6_K: status %d", r.second.status);
+    r = f.FusedQuantizedDense(x, w, Value(), &q5k, ActivationType::None);
+    CHECK(IsNotImplemented(r.second), "GGML type 13 (Q5_K): status %d", r.second.status);
     r = f.FusedQuantizedDense(xi, w, Value(), &q8, ActivationType::None);
     CHECK(IsNotImplemented(r.second), "Int32 activations: status %d", r.second.status);
     // malformed operands are hard errors

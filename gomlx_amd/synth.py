@@ -79,6 +79,10 @@ def weights(ggml_type: int, seed: int, N: int, K: int) -> np.ndarray:
         out[:, 2:4] = _f16_bytes(np.abs(normal(seed, 3, nb)) * 0.001)
         out[:, 4:16] = (bits64(seed, 4, nb * 12) >> np.uint64(24)).astype(np.uint8).reshape(nb, 12)
         out[:, 16:144] = (bits64(seed, 2, nb * 128) >> np.uint64(24)).astype(np.uint8).reshape(nb, 128)
+    elif ggml_type == ggml.Q6_K:  # d = fp16(|N(0, 2e-5)|), int8 scales and all code bits uniform
+        out[:, 0:192] = (bits64(seed, 2, nb * 192) >> np.uint64(24)).astype(np.uint8).reshape(nb, 192)
+        out[:, 192:208] = (bits64(seed, 4, nb * 16) >> np.uint64(24)).astype(np.uint8).reshape(nb, 16)
+        out[:, 208:210] = _f16_bytes(np.abs(normal(seed, 1, nb)) * 2e-5)
     else:
         raise ValueError(f"unsupported ggml type {ggml_type}")
     return out.reshape(N, (K // vpb) * bpb)

@@ -43,7 +43,7 @@ typedef enum {
 
 /* compute.GGMLQuantType (core/graph/fused_ops.go:46-47); numeric values follow the public
  * GGML type ids. */
-typedef enum { GQ_Q4_0 = 2, GQ_Q8_0 = 8, GQ_Q4_K = 12, GQ_IQ4_NL = 20 } gq_type;
+typedef enum { GQ_Q4_0 = 2, GQ_Q8_0 = 8, GQ_Q4_K = 12, GQ_Q6_K = 14, GQ_IQ4_NL = 20 } gq_type;
 
 /* compute.ActivationType as produced by activation.Type.ToBackend
  * (ml/layers/activation/activation.go:58-75). */

@@ -51,6 +51,7 @@ int gqo_bytes_per_block(int type) {
     case GQO_Q4_0: return 18;
     case GQO_Q8_0: return 34;
     case GQO_Q4_K: return 144;
+    case GQO_Q6_K: return 210;
     case GQO_IQ4_NL: return 18;
     default: return 0;
     }
@@ -59,7 +60,7 @@ int gqo_bytes_per_block(int type) {
 int gqo_values_per_block(int type) {
     switch (type) {
     case GQO_Q4_0: case GQO_Q8_0: case GQO_IQ4_NL: return 32;
-    case GQO_Q4_K: return 256;
+    case GQO_Q4_K: case GQO_Q6_K: return 256;
     default: return 0;
     }
 }
@@ -145,6 +146,36 @@ static void dequant_block_q4_k(const uint8_t *b, float *out) {
     }
 }
 
+/* Q6_K super-block (public GGML block_q6_K; listed by the reference among the GGMLQuantType values,
+ * docs/CHANGELOG.md:251-252, and reached from ml/nn/quantized_dense.go:56; arithmetic in the
+ * un-vendored github.com/gomlx/compute v0.1.2 - PARITY UNPINNED):
+ *   bytes 0-127 ql (low 4 bits), 128-191 qh (high 2 bits), 192-207 int8 scales x 16, 208-209 fp16 d.
+ *   For each half h of 128 values and l = 0..31:
+ *     value 128h + l      : ql[64h + l] & 15      | ((qh[32h + l] >> 0) & 3) << 4, scale 8h + l/16
+ *     value 128h + 32 + l : ql[64h + 32 + l] & 15 | ((qh[32h + l] >> 2) & 3) << 4, scale 8h + 2 + l/16
+ *     value 128h + 64 + l : ql[64h + l] >> 4      | ((qh[32h + l] >> 4) & 3) << 4, scale 8h + 4 + l/16
+ *     value 128h + 96 + l : ql[64h + 32 + l] >> 4 | ((qh[32h + l] >> 6) & 3) << 4, scale 8h + 6 + l/16
+ *   w = (f32(d) * scale) * (q - 32).  The exact product has at most 11 + 7 + 6 = 24 significant
+ *   bits, so every evaluation order gives the same fp32 value (denormal results aside). */
+static void dequant_block_q6_k(const uint8_t *b, float *out) {
+    const uint8_t *ql = b, *qh = b + 128;
+    const int8_t *sc = (const int8_t *)(b + 192);
+    const float d = gqo_fp16_to_fp32(load_u16le(b + 208));
+    for (int h = 0; h < 2; h++) {
+        for (int l = 0; l < 32; l++) {
+            const int is = l / 16;
+            const int q1 = (int)((ql[64 * h + l] & 0x0F) | (((qh[32 * h + l] >> 0) & 3) << 4)) - 32;
+            const int q2 = (int)((ql[64 * h + 32 + l] & 0x0F) | (((qh[32 * h + l] >> 2) & 3) << 4)) - 32;
+            const int q3 = (int)((ql[64 * h + l] >> 4) | (((qh[32 * h + l] >> 4) & 3) << 4)) - 32;
+            const int q4 = (int)((ql[64 * h + 32 + l] >> 4) | (((qh[32 * h + l] >> 6) & 3) << 4)) - 32;
+            out[128 * h + l] = (d * (float)sc[8 * h + is]) * (float)q1;
+            out[128 * h + 32 + l] = (d * (float)sc[8 * h + 2 + is]) * (float)q2;
+            out[128 * h + 64 + l] = (d * (float)sc[8 * h + 4 + is]) * (float)q3;
+            out[128 * h + 96 + l] = (d * (float)sc[8 * h + 6 + is]) * (float)q4;
+        }
+    }
+}
+
 typedef void (*block_fn)(const uint8_t *, float *);
 
 static block_fn block_dequantizer(int type) {
@@ -152,6 +183,7 @@ static block_fn block_dequantizer(int type) {
     case GQO_Q8_0: return dequant_block_q8_0;
     case GQO_Q4_0: return dequant_block_q4_0;
     case GQO_Q4_K: return dequant_block_q4_k;
+    case GQO_Q6_K: return dequant_block_q6_k;
     case GQO_IQ4_NL: return dequant_block_iq4_nl;
     default: return NULL;
     }

@@ -16,6 +16,10 @@
  *                         third-party module github.com/gomlx/compute v0.1.2 (package gobackend),
  *                         which is not vendored.  Restated from the public GGML block_q4_K
  *                         specification; self-consistency checks only.
+ *   Q6_K dequant          PARITY UNPINNED at the reference, for the same reason (the reference names
+ *                         the type, docs/CHANGELOG.md:251-252, but holds neither its arithmetic nor a
+ *                         test vector).  Restated from the public GGML block_q6_K specification;
+ *                         exact-arithmetic and structural checks only.
  */
 #ifndef GGML_ORACLE_H
 #define GGML_ORACLE_H
@@ -28,7 +32,7 @@ extern "C" {
 #endif
 
 /* GGML type ids (public ggml numbering). */
-enum { GQO_Q4_0 = 2, GQO_Q8_0 = 8, GQO_Q4_K = 12, GQO_IQ4_NL = 20 };
+enum { GQO_Q4_0 = 2, GQO_Q8_0 = 8, GQO_Q4_K = 12, GQO_Q6_K = 14, GQO_IQ4_NL = 20 };
 
 /* compute.ActivationType as used by activation.Type.ToBackend
  * (ml/layers/activation/activation.go:58-75). */

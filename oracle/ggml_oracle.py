@@ -17,6 +17,8 @@ pinned (reference KATs + closed forms + brute force, see tests/test_oracle.py).
 **Q4_K is PARITY UNPINNED at the reference**: its only implementation is in the
 un-vendored module github.com/gomlx/compute v0.1.2 (reached from
 ml/nn/quantized_dense.go:56); it is restated from the public GGML block_q4_K layout.
+**Q6_K is PARITY UNPINNED** for the same reason (the reference only names the type,
+docs/CHANGELOG.md:251-252); it is restated from the public GGML block_q6_K layout.
 """
 from __future__ import annotations
 
@@ -26,10 +28,10 @@ import subprocess
 
 import numpy as np
 
-Q4_0, Q8_0, Q4_K, IQ4_NL = 2, 8, 12, 20
+Q4_0, Q8_0, Q4_K, Q6_K, IQ4_NL = 2, 8, 12, 14, 20
 ACT_NONE, ACT_GELU, ACT_RELU, ACT_SILU, ACT_HARDSWISH, ACT_TANH = range(6)
 
-_GEOM = {Q4_0: (18, 32), Q8_0: (34, 32), Q4_K: (144, 256), IQ4_NL: (18, 32)}
+_GEOM = {Q4_0: (18, 32), Q8_0: (34, 32), Q4_K: (144, 256), Q6_K: (210, 256), IQ4_NL: (18, 32)}
 
 # Public GGML IQ4_NL table (compute.IQ4NLLookupTable, ml/ggml/dequant.go:130).
 IQ4NL_LUT = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113],
@@ -98,6 +100,19 @@ def np_dequantize(t: int, W: np.ndarray, K: int | None = None) -> np.ndarray:
         dsc = (d[:, :, None] * sc.astype(np.float32))[:, :, :, None]
         dm = (dmin[:, :, None] * mn.astype(np.float32))[:, :, :, None]
         return (dsc * codes - dm).astype(np.float32).reshape(N, nb * 256)
+    if t == Q6_K:  # public GGML block_q6_K (parity unpinned at the reference)
+        ql = w[:, :, 0:128].reshape(N, nb, 2, 2, 32)     # [half][which 32 bytes][l]
+        qh = w[:, :, 128:192].reshape(N, nb, 2, 1, 32)   # [half][.][l]
+        sc = w[:, :, 192:208].view(np.int8).astype(np.float32).reshape(N, nb, 2, 4, 2)  # [half][quadrant][l / 16]
+        d = _f16(w[:, :, 208:210])
+        lo = np.stack([ql & 0x0F, ql >> 4], axis=3)       # [N, nb, half, nibble, which, l]
+        lo = lo.reshape(N, nb, 2, 4, 32)                  # quadrant = 2 * nibble + which
+        shifts = np.array([0, 2, 4, 6], np.uint8).reshape(1, 1, 1, 4, 1)
+        hi = (qh >> shifts) & 3                           # [N, nb, half, quadrant, l]
+        q = (lo | (hi << 4)).astype(np.int32) - 32
+        scale = np.repeat(sc, 16, axis=4)                 # [N, nb, half, quadrant, 32]
+        ds = d[:, :, None, None, None] * scale
+        return (ds * q.astype(np.float32)).astype(np.float32).reshape(N, nb * 256)
     raise ValueError(f"unsupported ggml type {t}")
 
 

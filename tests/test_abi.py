@@ -38,7 +38,7 @@ def test_no_oracle_or_torch_linked_into_the_library():
 def test_geometry_matches_reference_block_formats():
     L = _lib.lib()
     assert L.gq_abi_version() == 1
-    for t, bpb, vpb in [(ggml.Q4_0, 18, 32), (ggml.Q8_0, 34, 32), (ggml.Q4_K, 144, 256), (ggml.IQ4_NL, 18, 32)]:
+    for t, bpb, vpb in [(ggml.Q4_0, 18, 32), (ggml.Q8_0, 34, 32), (ggml.Q4_K, 144, 256), (ggml.Q6_K, 210, 256), (ggml.IQ4_NL, 18, 32)]:
         assert L.gq_bytes_per_block(t) == bpb == ggml.bytes_per_block(t)
         assert L.gq_values_per_block(t) == vpb == ggml.values_per_block(t)
     assert L.gq_row_bytes(ggml.Q8_0, 4096) == 4352
@@ -50,7 +50,7 @@ def test_geometry_matches_reference_block_formats():
     assert L.gq_row_bytes(99, 4096) == 0
     assert L.gq_bytes_per_block(99) == 0
     assert ggml.can_decompose(ggml.Q8_0) and ggml.can_decompose(ggml.Q4_0) and ggml.can_decompose(ggml.IQ4_NL)
-    assert not ggml.can_decompose(ggml.Q4_K)   # ml/ggml/dequant.go:20-27
+    assert not ggml.can_decompose(ggml.Q4_K) and not ggml.can_decompose(ggml.Q6_K)   # ml/ggml/dequant.go:20-27
 
 
 def check(*args):
@@ -74,7 +74,8 @@ def test_build_time_validation():
     assert check(ggml.Q8_0, _lib.F32, 1, 4096, 4096, 4352, -1, 6)[0] == _lib.ERR_INVALID
     assert check(ggml.Q8_0, _lib.F32, 1, 4096, 4096, 0, -1, 0)[0] == _lib.ERR_INVALID
     # valid but unsupported -> NotImplemented (caller falls back, core/graph/fused_ops.go:357-363)
-    assert check(14, _lib.F32, 1, 256, 4, 210, -1, 0)[0] == _lib.ERR_NOT_IMPLEMENTED   # Q6_K
+    assert check(ggml.Q6_K, _lib.F32, 1, 256, 4, 210, -1, 0)[:2] == (_lib.OK, 256)
+    assert check(13, _lib.F32, 1, 256, 4, 176, -1, 0)[0] == _lib.ERR_NOT_IMPLEMENTED   # Q5_K is not built
     assert check(ggml.Q8_0, 7, 1, 4096, 4096, 4352, -1, 0)[0] == _lib.ERR_NOT_IMPLEMENTED
 
 

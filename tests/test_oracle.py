@@ -8,7 +8,7 @@ Sources of truth used here, none of which is the oracle's own formula retyped:
   * structural probes: single non-zero code / scale / min / byte, so that a wrong index,
     nibble order, sign or dropped term fails;
   * the two restatements (numpy, C) against each other on random blocks.
-Q4_K has no reference vector (parity unpinned); it gets the structural checks only.
+Q4_K and Q6_K have no reference vector (parity unpinned); they get the structural checks only.
 """
 import math
 import struct
@@ -17,8 +17,8 @@ from fractions import Fraction
 import numpy as np
 import pytest
 
-Q4_0, Q8_0, Q4_K, IQ4_NL = 2, 8, 12, 20
-ALL_TYPES = [Q4_0, Q8_0, Q4_K, IQ4_NL]
+Q4_0, Q8_0, Q4_K, Q6_K, IQ4_NL = 2, 8, 12, 14, 20
+ALL_TYPES = [Q4_0, Q8_0, Q4_K, Q6_K, IQ4_NL]
 
 
 def f32(x) -> np.float32:
@@ -241,6 +241,86 @@ def test_q4_k_byte_footprint(oracle):
         assert changed == {64 * g + l, 64 * g + 32 + l}, b
 
 
+# ------------------------------------------------------------------------------ Q6_K structure
+
+def make_q6k_block(dbits, scales, codes):
+    """codes: 256 ints in [0,63] in logical order; scales: 16 ints in [-128,127].  Written from the
+    public GGML layout: for half h and l = 0..31 the values 128h + l, + 32 + l, + 64 + l, + 96 + l
+    share byte 32h + l of qh (2 bits each, low to high) and use the low / high nibbles of
+    ql[64h + l] and ql[64h + 32 + l]."""
+    b = np.zeros(210, np.uint8)
+    for h in range(2):
+        for l in range(32):
+            q = [codes[128 * h + 32 * k + l] for k in range(4)]
+            b[64 * h + l] = (q[0] & 15) | ((q[2] & 15) << 4)
+            b[64 * h + 32 + l] = (q[1] & 15) | ((q[3] & 15) << 4)
+            b[128 + 32 * h + l] = (q[0] >> 4) | ((q[1] >> 4) << 2) | ((q[2] >> 4) << 4) | ((q[3] >> 4) << 6)
+    for j in range(16):
+        b[192 + j] = scales[j] & 0xFF
+    b[208], b[209] = dbits & 0xFF, dbits >> 8
+    return b
+
+
+@pytest.mark.parametrize("impl", ["np", "c"])
+def test_q6_k_full_block_against_exact_arithmetic(oracle, impl):
+    """w = d * scale * (q - 32) is exactly representable in fp32 (11 + 7 + 6 bits), so the expected
+    value is the exact rational product."""
+    rng = np.random.default_rng(17)
+    for trial, dbits in enumerate([0x2E66, 0x1A00, 0x3C00, 0x0155, 0x3555, 0xAE66]):
+        scales = [int(v) for v in rng.integers(-128, 128, 16)]
+        codes = [int(v) for v in rng.integers(0, 64, 256)]
+        W = make_q6k_block(dbits, scales, codes)[None, :]
+        got = oracle.np_dequantize(Q6_K, W) if impl == "np" else oracle.c_dequantize(Q6_K, W, 256)
+        d = half_value(dbits)
+        for i in range(256):
+            want = d * scales[i // 16] * (codes[i] - 32)
+            assert Fraction(float(got[0, i])) == want, (trial, i)
+
+
+@pytest.mark.parametrize("impl", ["np", "c"])
+def test_q6_k_single_field_probes(oracle, impl):
+    deq = (lambda W: oracle.np_dequantize(Q6_K, W)) if impl == "np" else (lambda W: oracle.c_dequantize(Q6_K, W, 256))
+    # (a) one scale, all codes 33 (q - 32 = 1): exactly that scale's 16 values light up
+    for j in range(16):
+        scales = [0] * 16
+        scales[j] = 5 + j if j % 2 else -(5 + j)
+        out = deq(make_q6k_block(0x3C00, scales, [33] * 256)[None, :])[0]
+        want = np.zeros(256, np.float32)
+        want[16 * j:16 * j + 16] = scales[j]
+        assert np.array_equal(out, want), j
+    # (b) one code: exactly one value, over the whole 6-bit range incl. the high two bits
+    for i, c in [(0, 63), (1, 0), (31, 47), (32, 16), (95, 32 + 17), (96, 1), (127, 62), (128, 63), (200, 48), (255, 15)]:
+        codes = [32] * 256
+        codes[i] = c
+        out = deq(make_q6k_block(0x4000, [1] * 16, codes)[None, :])[0]
+        want = np.zeros(256, np.float32)
+        want[i] = 2.0 * (c - 32)
+        assert np.array_equal(out, want), (i, c)
+
+
+def test_q6_k_byte_footprint(oracle):
+    """Flipping a byte of ql changes exactly two values, a byte of qh exactly four, a scale sixteen."""
+    rng = np.random.default_rng(5)
+    codes = [int(v) if v != 32 else 7 for v in rng.integers(0, 64, 256)]  # code 32 decodes to 0 whatever the scale
+    base = make_q6k_block(0x3C00, [int(v) for v in rng.integers(1, 100, 16)], codes)
+    ref = oracle.c_dequantize(Q6_K, base[None, :], 256)[0]
+
+    def changed(byte):
+        mod = base.copy()
+        mod[byte] ^= 0xFF
+        return set(np.nonzero(oracle.c_dequantize(Q6_K, mod[None, :], 256)[0] != ref)[0].tolist())
+
+    for b in range(128):
+        h, r = divmod(b, 64)
+        which, l = divmod(r, 32)
+        assert changed(b) == {128 * h + 32 * which + l, 128 * h + 64 + 32 * which + l}, b
+    for b in range(64):
+        h, l = divmod(b, 32)
+        assert changed(128 + b) == {128 * h + 32 * k + l for k in range(4)}, b
+    for j in range(16):
+        assert changed(192 + j) == set(range(16 * j, 16 * j + 16)), j
+
+
 # ------------------------------------------------------------------------------ numpy vs C
 
 def random_blocks(t, N, K, seed):
@@ -345,6 +425,7 @@ def test_oracle_rejects_ragged_and_unknown(oracle):
         oracle.c_dequantize(99, np.zeros((2, 34), np.uint8), 32)
     assert oracle.row_bytes(Q4_K, 255) == 0 and oracle.lib().gqo_row_bytes(Q4_K, 255) == 0
     assert oracle.row_bytes(Q4_K, 14336) == 8064 == oracle.lib().gqo_row_bytes(Q4_K, 14336)
+    assert oracle.row_bytes(Q6_K, 14336) == 11760 == oracle.lib().gqo_row_bytes(Q6_K, 14336)
     assert oracle.row_bytes(Q8_0, 4096) == 4352 and oracle.row_bytes(Q4_0, 4096) == 2304
 
 

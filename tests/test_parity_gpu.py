@@ -13,8 +13,8 @@ from gomlx_amd.nn import Activation, Quantization
 
 pytestmark = pytest.mark.gpu
 
-Q4_0, Q8_0, Q4_K, IQ4_NL = ggml.Q4_0, ggml.Q8_0, ggml.Q4_K, ggml.IQ4_NL
-ALL_TYPES = [Q4_0, Q8_0, Q4_K, IQ4_NL]
+Q4_0, Q8_0, Q4_K, Q6_K, IQ4_NL = ggml.Q4_0, ggml.Q8_0, ggml.Q4_K, ggml.Q6_K, ggml.IQ4_NL
+ALL_TYPES = [Q4_0, Q8_0, Q4_K, Q6_K, IQ4_NL]
 TOL_F32 = 1e-3
 TOL_BF16 = 2e-2
 
@@ -82,7 +82,7 @@ def test_dequantize_bit_exact_on_extreme_scales(gpu, oracle, t):
     raw = (synth.bits64(77, t, N * rb) >> np.uint64(20)).astype(np.uint8).reshape(N, rb)
     blk = raw.reshape(N, -1, ggml.bytes_per_block(t))
     # keep the fp16 fields finite (exponent != 31): inf/NaN scales are outside the contract
-    for off in ([1] if t != Q4_K else [1, 3]):
+    for off in {Q4_K: [1, 3], Q6_K: [209]}.get(t, [1]):
         hi = blk[:, :, off]
         hi[(hi & 0x7C) == 0x7C] &= 0xBF
     got = nn.dequantize(dev(gpu, raw), t).cpu().numpy()
