@@ -43,7 +43,7 @@ COUNTER_KIB = {  # workload -> (FETCH_SIZE, WRITE_SIZE) raw counter KiB per step
     "c0": (8804.6, 16.0),
     "c1": (16256.7, 56.0),
     "c2": (19871.0 + 1822.1 + 911.5, 3584.0 + 512.0 + 924.0),
-    "c3": (74690.3, 32768.0),
+    "c3": (74724.6, 32768.0),
     "c4": (60616.3, 168.0),
 }
 
