@@ -67,7 +67,7 @@ bool gemv_xs_supported(int type, int64_t K, int64_t N, const void *x);
 int launch_gemv_xs(int type, const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N,
                    const float *bias, int act, float *y, hipStream_t s);
 bool gemv_ks_supported(int type, int64_t K, int64_t N, const void *x);
-int launch_gemv_ks(int type, const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N,
+int launch_gemv_ks(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N,
                    const float *bias, int act, float *y, hipStream_t s);
 bool mmq_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, const void *bias, const void *y);
 int launch_mmq(int type, const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act,

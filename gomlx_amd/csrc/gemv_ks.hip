@@ -59,6 +59,10 @@ __device__ __forceinline__ int ks_quad_sum(int v) {
 
 struct XPair { float4 lo, hi; };
 
+// bf16 -> fp32 is a shift; two values per dword
+__device__ __forceinline__ float bf16_lo(uint32_t u) { return __builtin_bit_cast(float, u << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t u) { return __builtin_bit_cast(float, u & 0xFFFF0000u); }
+
 // Scale of 32 activations for a fixed-point range of +-qmax.  All-zero groups quantise to zero; a
 // non-finite group poisons its scale so that the affected outputs come out as NaN.
 __device__ __forceinline__ void ks_scale(const float *e, float qmax, float &inv, float &scale) {
@@ -91,6 +95,14 @@ template <> struct KS<kQ4_0> {
         XPair p;
         p.lo = x4[0];  // values 4w .. 4w+3 of the block (low nibbles of code bytes 4w .. 4w+3)
         p.hi = x4[4];  // values 16+4w .. (high nibbles)
+        return p;
+    }
+    static __device__ __forceinline__ XPair x_load_bf16(const uint16_t *__restrict__ xs, int lane) {
+        const uint2 *x2 = reinterpret_cast<const uint2 *>(xs) + (lane >> 2) * 8 + (lane & 3);
+        const uint2 a = x2[0], b = x2[4];
+        XPair p;
+        p.lo = make_float4(bf16_lo(a.x), bf16_hi(a.x), bf16_lo(a.y), bf16_hi(a.y));
+        p.hi = make_float4(bf16_lo(b.x), bf16_hi(b.x), bf16_lo(b.y), bf16_hi(b.y));
         return p;
     }
     // nibble p of plane d = digit d of the activation facing nibble p of the weight dword
@@ -156,6 +168,13 @@ __device__ __forceinline__ XPair limb_x_load(const float *__restrict__ xs, int l
     p.hi = x4[1];
     return p;
 }
+__device__ __forceinline__ XPair limb_x_load_bf16(const uint16_t *__restrict__ xs, int lane) {
+    const uint4 a = reinterpret_cast<const uint4 *>(xs)[lane];
+    XPair p;
+    p.lo = make_float4(bf16_lo(a.x), bf16_hi(a.x), bf16_lo(a.y), bf16_hi(a.y));
+    p.hi = make_float4(bf16_lo(a.z), bf16_hi(a.z), bf16_lo(a.w), bf16_hi(a.w));
+    return p;
+}
 __device__ __forceinline__ Staged limb_stage(const XPair &xp) {
     const float e[8] = {xp.lo.x, xp.lo.y, xp.lo.z, xp.lo.w, xp.hi.x, xp.hi.y, xp.hi.z, xp.hi.w};
     Staged st;
@@ -192,6 +211,7 @@ template <> struct KS<kQ8_0> {
     static __device__ __forceinline__ int lane_offset(int c) { return c * 68; }
     static __device__ __forceinline__ void load(Raw &r, const uint8_t *p) { r = *reinterpret_cast<const Raw *>(p); }
     static __device__ __forceinline__ XPair x_load(const float *__restrict__ xs, int lane) { return limb_x_load(xs, lane); }
+    static __device__ __forceinline__ XPair x_load_bf16(const uint16_t *__restrict__ xs, int lane) { return limb_x_load_bf16(xs, lane); }
     static __device__ __forceinline__ Staged stage(const XPair &xp) { return limb_stage(xp); }
     static __device__ __forceinline__ float dot(const Raw &r, const uint4 *xq, const float *xsc, const float *, int) {
         const uint32_t *v = r.v;
@@ -226,6 +246,7 @@ template <> struct KS<kQ4_K> {
         r.q1 = q[1];
     }
     static __device__ __forceinline__ XPair x_load(const float *__restrict__ xs, int lane) { return limb_x_load(xs, lane); }
+    static __device__ __forceinline__ XPair x_load_bf16(const uint16_t *__restrict__ xs, int lane) { return limb_x_load_bf16(xs, lane); }
     static __device__ __forceinline__ Staged stage(const XPair &xp) { return limb_stage(xp); }
     static __device__ __forceinline__ float dot(const Raw &r, const uint4 *xq, const float *xsc, const float *xsm, int c) {
         const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
@@ -279,15 +300,20 @@ constexpr int kWaveLdsDwords = 72 * 4;  // per wavefront: 64 uint4 of planes, 16
 // blocks while the memory pipeline is full) and arithmetic alternate instead of forming two
 // phases.
 template <int T, int PF, int WIN>
-__device__ __forceinline__ void ks_body(const float *__restrict__ x, const uint8_t *__restrict__ W, const float *__restrict__ bias,
-                                        float *__restrict__ y, int N, int64_t row_bytes, int iters, int spw, int act, int waves,
-                                        int wg, uint32_t *lds) {
+__device__ __forceinline__ void ks_body(const void *__restrict__ xv, int x_bf16, const uint8_t *__restrict__ W,
+                                        const float *__restrict__ bias, float *__restrict__ y, int N, int64_t row_bytes, int iters,
+                                        int spw, int act, int waves, int wg, uint32_t *lds) {
     typedef typename KS<T>::Raw Raw;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int rg = lane >> 3, c = lane & 7;
     const int rows_wg = iters * 8;
     const int row0 = wg * rows_wg;
     float *all = reinterpret_cast<float *>(lds + waves * kWaveLdsDwords);  // partial sums [waves][rows_wg]
+    // activations of slice sl for this lane (fp32, or bf16 widened on the fly; x_bf16 is uniform)
+    auto x_slice = [&](int sl) -> XPair {
+        if (x_bf16) return KS<T>::x_load_bf16(reinterpret_cast<const uint16_t *>(xv) + sl * kSliceValues, lane);
+        return KS<T>::x_load(reinterpret_cast<const float *>(xv) + sl * kSliceValues, lane);
+    };
     if (wave < waves) {
         uint4 *my_planes = reinterpret_cast<uint4 *>(lds + wave * kWaveLdsDwords);
         float *my_scales = reinterpret_cast<float *>(my_planes + 64);
@@ -296,7 +322,7 @@ __device__ __forceinline__ void ks_body(const float *__restrict__ x, const uint8
 
         KS_TRACE(0);
         KS_TRACE_WALL(12);
-        XPair xp = KS<T>::x_load(x + wave * kSliceValues, lane);
+        XPair xp = x_slice(wave);
         const int last_row = N - 1;
         auto addr = [&](int j, int it) -> const uint8_t * {
             const int row = min(row0 + it * 8 + rg, last_row);
@@ -329,7 +355,7 @@ __device__ __forceinline__ void ks_body(const float *__restrict__ x, const uint8
         };
         stage(xp);
         KS_TRACE(2);
-        if (spw > 1) xp = KS<T>::x_load(x + (wave + waves) * kSliceValues, lane);
+        if (spw > 1) xp = x_slice(wave + waves);
         KS_TRACE(3);
 
         const int ngroups = spw * (iters / PF);
@@ -352,7 +378,7 @@ __device__ __forceinline__ void ks_body(const float *__restrict__ x, const uint8
             }
             if (wrap && !last_group) {  // next group starts a new slice: convert its activations
                 stage(xp);
-                if (nj + 1 < spw) xp = KS<T>::x_load(x + (wave + (nj + 1) * waves) * kSliceValues, lane);
+                if (nj + 1 < spw) xp = x_slice(wave + (nj + 1) * waves);
             }
             j = nj;
             i0 = ni0;
@@ -372,12 +398,13 @@ __device__ __forceinline__ void ks_body(const float *__restrict__ x, const uint8
 }
 
 template <int T, int PF, int WIN>
-__global__ __launch_bounds__(512) void gemv_ks_kernel(const float *__restrict__ X, const uint8_t *__restrict__ W,
+__global__ __launch_bounds__(512) void gemv_ks_kernel(const void *__restrict__ X, int x_bf16, const uint8_t *__restrict__ W,
                                                       const float *__restrict__ bias, float *__restrict__ Y, int K, int N,
                                                       int64_t row_bytes, int iters, int spw, int act) {
     extern __shared__ uint32_t lds[];
-    ks_body<T, PF, WIN>(X + (int64_t)blockIdx.y * K, W, bias, Y + (int64_t)blockIdx.y * N, N, row_bytes, iters, spw, act,
-                        (int)(blockDim.x >> 6), (int)blockIdx.x, lds);
+    const uint8_t *x = reinterpret_cast<const uint8_t *>(X) + (int64_t)blockIdx.y * K * (x_bf16 ? 2 : 4);
+    ks_body<T, PF, WIN>(x, x_bf16, W, bias, Y + (int64_t)blockIdx.y * N, N, row_bytes, iters, spw, act, (int)(blockDim.x >> 6),
+                        (int)blockIdx.x, lds);
 }
 
 // Several independent batch-1 problems of one format in a single launch: workgroups
@@ -406,7 +433,7 @@ __global__ __launch_bounds__(512) void gemv_ks_batch_kernel(const KsBatch b) {
     for (int j = 1; j < kMaxBatchKs; j++)
         if (j < b.count && (int)blockIdx.x >= b.p[j].wg_begin) i = j;
     const KsProblem &q = b.p[i];
-    ks_body<T, 4, 3>(q.x, q.W, q.bias, q.y, q.N, q.row_bytes, q.iters, q.spw, q.act, q.waves, (int)blockIdx.x - q.wg_begin, lds);
+    ks_body<T, 4, 3>(q.x, 0, q.W, q.bias, q.y, q.N, q.row_bytes, q.iters, q.spw, q.act, q.waves, (int)blockIdx.x - q.wg_begin, lds);
 }
 
 struct KsPlan { int waves, spw, iters, pf, wgs; size_t shmem; };
@@ -455,27 +482,29 @@ bool ks_plan(int64_t K, int64_t N, KsPlan &p) {
 }
 
 template <int T, int PF>
-int launch_ks_pf(const KsPlan &p, const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act,
+int launch_ks_pf(const KsPlan &p, const void *x, int x_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act,
                  float *y, hipStream_t s) {
     const int64_t row_bytes = (K / Geom<T>::vpb) * Geom<T>::bpb;
     const dim3 grid((unsigned)p.wgs, (unsigned)M), block((unsigned)p.waves * 64);
     constexpr int WIN = PF < 3 ? PF : 3;
-    return launch(gemv_ks_kernel<T, PF, WIN>, grid, block, p.shmem, s, x, W, bias, y, (int)K, (int)N, row_bytes, p.iters, p.spw, act);
+    return launch(gemv_ks_kernel<T, PF, WIN>, grid, block, p.shmem, s, x, x_bf16, W, bias, y, (int)K, (int)N, row_bytes, p.iters, p.spw,
+                  act);
 }
 
 template <int T>
-int launch_ks(const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y, hipStream_t s) {
+int launch_ks(const void *x, int x_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y,
+              hipStream_t s) {
     KsPlan p;
     if (!ks_plan(K, N, p)) return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv_ks: unsupported problem");
     switch (p.pf) {
-    case 1: return launch_ks_pf<T, 1>(p, x, M, K, W, N, bias, act, y, s);
-    case 2: return launch_ks_pf<T, 2>(p, x, M, K, W, N, bias, act, y, s);
-    case 3: return launch_ks_pf<T, 3>(p, x, M, K, W, N, bias, act, y, s);
-    case 4: return launch_ks_pf<T, 4>(p, x, M, K, W, N, bias, act, y, s);
-    case 5: return launch_ks_pf<T, 5>(p, x, M, K, W, N, bias, act, y, s);
-    case 6: return launch_ks_pf<T, 6>(p, x, M, K, W, N, bias, act, y, s);
-    case 7: return launch_ks_pf<T, 7>(p, x, M, K, W, N, bias, act, y, s);
-    default: return launch_ks_pf<T, 8>(p, x, M, K, W, N, bias, act, y, s);
+    case 1: return launch_ks_pf<T, 1>(p, x, x_bf16, M, K, W, N, bias, act, y, s);
+    case 2: return launch_ks_pf<T, 2>(p, x, x_bf16, M, K, W, N, bias, act, y, s);
+    case 3: return launch_ks_pf<T, 3>(p, x, x_bf16, M, K, W, N, bias, act, y, s);
+    case 4: return launch_ks_pf<T, 4>(p, x, x_bf16, M, K, W, N, bias, act, y, s);
+    case 5: return launch_ks_pf<T, 5>(p, x, x_bf16, M, K, W, N, bias, act, y, s);
+    case 6: return launch_ks_pf<T, 6>(p, x, x_bf16, M, K, W, N, bias, act, y, s);
+    case 7: return launch_ks_pf<T, 7>(p, x, x_bf16, M, K, W, N, bias, act, y, s);
+    default: return launch_ks_pf<T, 8>(p, x, x_bf16, M, K, W, N, bias, act, y, s);
     }
 }
 
@@ -521,12 +550,13 @@ bool gemv_ks_supported(int type, int64_t K, int64_t N, const void *x) {
     return ks_split(K, waves, spw);
 }
 
-int launch_gemv_ks(int type, const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act,
-                   float *y, hipStream_t s) {
+int launch_gemv_ks(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias,
+                   int act, float *y, hipStream_t s) {
+    const int x_bf16 = x_is_bf16 ? 1 : 0;
     switch (type) {
-    case kQ4_0: return launch_ks<kQ4_0>(x, M, K, W, N, bias, act, y, s);
-    case kQ8_0: return launch_ks<kQ8_0>(x, M, K, W, N, bias, act, y, s);
-    case kQ4_K: return launch_ks<kQ4_K>(x, M, K, W, N, bias, act, y, s);
+    case kQ4_0: return launch_ks<kQ4_0>(x, x_bf16, M, K, W, N, bias, act, y, s);
+    case kQ8_0: return launch_ks<kQ8_0>(x, x_bf16, M, K, W, N, bias, act, y, s);
+    case kQ4_K: return launch_ks<kQ4_K>(x, x_bf16, M, K, W, N, bias, act, y, s);
     default: return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv_ks: ggml type %d is not implemented", type);
     }
 }

@@ -134,6 +134,30 @@ def test_gemv_k_sliced_plans(gpu, oracle, t, M, K, N):
     assert rel_err(got, want) < TOL_F32, (t, M, K, N)
 
 
+@pytest.mark.parametrize("t", [Q4_0, Q8_0, Q4_K])
+@pytest.mark.parametrize("M,K,N", [(1, 4096, 300), (3, 1024, 257), (16, 2048, 130)])
+def test_bf16_decode_batches_are_exact_widenings(gpu, oracle, t, M, K, N):
+    """bf16 activations of a decode batch run through the fp32 GEMV (bf16 -> fp32 is exact), so
+    they meet the fp32 tolerance against the oracle on the same bf16-valued inputs."""
+    W = synth.weights(t, 50 + t, N, K)
+    x = bf16_round(synth.activations(51 + t, M, K))
+    bias = synth.normal(52 + t, 0, N).astype(np.float32) * 0.1
+    got = run_dense(gpu, t, x, W, bias, 3, bf16=True)
+    assert rel_err(got, oracle.c_qdense(t, x, W, bias, 3)) < TOL_F32, (t, M, K, N)
+
+
+@pytest.mark.parametrize("t", [Q4_0, Q8_0, IQ4_NL])
+@pytest.mark.parametrize("M", [5, 9, 16, 17])
+def test_small_batches_f32(gpu, oracle, t, M):
+    """Batches just above the decode sizes: GEMV passes up to 16 rows where the format has no
+    small-batch MFMA kernel, the tiled kernel beyond (and for IQ4_NL)."""
+    K, N = 1024, 300
+    W = synth.weights(t, 60 + t, N, K)
+    x = synth.activations(61 + t, M, K)
+    got = run_dense(gpu, t, x, W, None, 0)
+    assert rel_err(got, oracle.c_qdense(t, x, W, None, 0)) < TOL_F32, (t, M)
+
+
 @pytest.mark.parametrize("t", ALL_TYPES)
 def test_gemv_long_k_is_chunked(gpu, oracle, t):
     """K above the 16384 values one LDS pass holds."""
