@@ -1,5 +1,5 @@
 // Decode GEMV, K-sliced integer-dot kernels with wavefront-local activation staging
-// (Q4_0, Q8_0, Q4_K; K % 512 == 0).
+// (Q4_0, Q8_0, Q4_K, Q6_K; K % 512 == 0).
 //
 // The activation-stationary kernel of gemv_xs.hip lets every wavefront see all of K, so its
 // workgroup has to convert the whole activation vector together and meet at a barrier before the
@@ -13,8 +13,11 @@
 // Lane l = 8 * rg + c works on row (8 * it + rg) of the workgroup and on 64 values of the slice:
 //   Q4_0: blocks 2c, 2c+1: 36 bytes at a 4-byte-aligned address;
 //   Q8_0: blocks 2c, 2c+1: 68 bytes at a 4-byte-aligned address;
-//   Q4_K: super-block c / 4 of the slice, 64-value group c % 4: the 16-byte header and 32 code bytes.
-// A load instruction therefore covers 8 rows x one contiguous slice (288 or 544 bytes).
+//   Q4_K: super-block c / 4 of the slice, 64-value group c % 4: the 16-byte header and 32 code bytes;
+//   Q6_K: super-block c / 4, half (c / 2) % 2, and of each of the half's four 32-value quadrants
+//         the 16 values (c % 2) * 16 ..: 16 + 16 bytes of low nibbles, 16 bytes of high bit pairs,
+//         the half's 8 scales and d.
+// A load instruction therefore covers 8 rows x one contiguous slice (288, 544 or 420 bytes).
 //
 // Activation fixed point: 16 bits per 32 values.  Q4_0 uses four balanced base-16 digits (digit
 // planes in the nibble order of a weight dword, one v_dot8_i32_i4 per plane); Q8_0 and Q4_K use
@@ -86,6 +89,11 @@ template <int T> struct KS;
 
 template <> struct KS<kQ4_0> {
     static constexpr int kSliceBytes = 288;
+    // where a lane finds what it needs of the staged slice: plane vector i (0..7), scale i, sum i
+    static constexpr int kScales = 2, kSumSpan = 0;
+    static __device__ __forceinline__ int plane_idx(int c, int i) { return 8 * c + i; }
+    static __device__ __forceinline__ int scale_idx(int c, int i) { return 2 * c + i; }
+    static __device__ __forceinline__ int sum_idx(int c, int i) { return 2 * c + i; }
     struct __attribute__((packed, aligned(4))) Raw { uint32_t v[9]; };
     static __device__ __forceinline__ int lane_offset(int c) { return c * 36; }
     static __device__ __forceinline__ void load(Raw &r, const uint8_t *p) { r = *reinterpret_cast<const Raw *>(p); }
@@ -175,6 +183,9 @@ __device__ __forceinline__ XPair limb_x_load_bf16(const uint16_t *__restrict__ x
     p.hi = make_float4(bf16_lo(a.z), bf16_hi(a.z), bf16_lo(a.w), bf16_hi(a.w));
     return p;
 }
+// SUM16: the published sum covers the 16 values of a lane pair and is pre-multiplied by -32 (the
+// offset of a Q6_K code); otherwise it covers the 32 values of the quad.
+template <bool SUM16 = false>
 __device__ __forceinline__ Staged limb_stage(const XPair &xp) {
     const float e[8] = {xp.lo.x, xp.lo.y, xp.lo.z, xp.lo.w, xp.hi.x, xp.hi.y, xp.hi.z, xp.hi.w};
     Staged st;
@@ -188,8 +199,13 @@ __device__ __forceinline__ Staged limb_stage(const XPair &xp) {
         xsum += zs - 0x8080;
         z[p] = (uint32_t)zs;
     }
-    xsum = ks_quad_sum(xsum);
-    st.sum = st.scale * (float)xsum;
+    if constexpr (SUM16) {
+        xsum += __builtin_amdgcn_update_dpp(0, xsum, 0xB1, 0xF, 0xF, true);
+        st.sum = -32.f * st.scale * (float)xsum;
+    } else {
+        xsum = ks_quad_sum(xsum);
+        st.sum = st.scale * (float)xsum;
+    }
     const uint32_t a01 = __builtin_amdgcn_perm(z[1], z[0], 0x05010400u), a23 = __builtin_amdgcn_perm(z[3], z[2], 0x05010400u);
     const uint32_t b01 = __builtin_amdgcn_perm(z[5], z[4], 0x05010400u), b23 = __builtin_amdgcn_perm(z[7], z[6], 0x05010400u);
     st.planes.x = __builtin_amdgcn_perm(a23, a01, 0x05040100u) ^ 0x80808080u;
@@ -207,6 +223,11 @@ __device__ __forceinline__ void limb_planes(const uint4 *xq, int h, int w, int &
 
 template <> struct KS<kQ8_0> {
     static constexpr int kSliceBytes = 544;
+    // where a lane finds what it needs of the staged slice: plane vector i (0..7), scale i, sum i
+    static constexpr int kScales = 2, kSumSpan = 0;
+    static __device__ __forceinline__ int plane_idx(int c, int i) { return 8 * c + i; }
+    static __device__ __forceinline__ int scale_idx(int c, int i) { return 2 * c + i; }
+    static __device__ __forceinline__ int sum_idx(int c, int i) { return 2 * c + i; }
     struct __attribute__((packed, aligned(4))) Raw { uint32_t v[17]; };
     static __device__ __forceinline__ int lane_offset(int c) { return c * 68; }
     static __device__ __forceinline__ void load(Raw &r, const uint8_t *p) { r = *reinterpret_cast<const Raw *>(p); }
@@ -237,6 +258,11 @@ template <> struct KS<kQ8_0> {
 
 template <> struct KS<kQ4_K> {
     static constexpr int kSliceBytes = 288;  // two super-blocks
+    // where a lane finds what it needs of the staged slice: plane vector i (0..7), scale i, sum i
+    static constexpr int kScales = 2, kSumSpan = 32;
+    static __device__ __forceinline__ int plane_idx(int c, int i) { return 8 * c + i; }
+    static __device__ __forceinline__ int scale_idx(int c, int i) { return 2 * c + i; }
+    static __device__ __forceinline__ int sum_idx(int c, int i) { return 2 * c + i; }
     struct Raw { uint4 hd, q0, q1; };
     static __device__ __forceinline__ int lane_offset(int c) { return (c >> 2) * 144; }
     static __device__ __forceinline__ void load(Raw &r, const uint8_t *sb, int c) {
@@ -274,9 +300,62 @@ template <> struct KS<kQ4_K> {
     }
 };
 
+
+// Q6_K: w = d * sc[16-value run] * (code - 32), code = low nibble | two high bits << 4.  The
+// -32 is applied through the activation sums of the run, so the codes stay unsigned bytes.
+template <> struct KS<kQ6_K> {
+    static constexpr int kSliceBytes = 420;  // two super-blocks
+    static constexpr int kScales = 4, kSumSpan = 16;
+    // c = 4 * sb + 2 * half + pp; quadrant qd's run is values 32 * qd + 16 * pp .. of the half
+    static __device__ __forceinline__ int plane_idx(int c, int i) { return 8 * (c & ~1) + 2 * (c & 1) + 4 * (i >> 1) + (i & 1); }
+    static __device__ __forceinline__ int scale_idx(int c, int i) { return 2 * (c & ~1) + i; }
+    static __device__ __forceinline__ int sum_idx(int c, int i) { return 4 * (c & ~1) + 2 * i + (c & 1); }
+    struct __attribute__((packed, aligned(2))) U4 { uint32_t v[4]; };
+    struct __attribute__((packed, aligned(2))) U2 { uint32_t v[2]; };
+    struct Raw { U4 a, b, h; U2 sc; uint32_t d; };
+    static __device__ __forceinline__ int lane_offset(int c) { return (c >> 2) * 210; }
+    static __device__ __forceinline__ void load(Raw &r, const uint8_t *sb, int c) {
+        const int half = (c >> 1) & 1, pp = c & 1;
+        const uint8_t *ql = sb + 64 * half + 16 * pp;
+        r.a = *reinterpret_cast<const U4 *>(ql);
+        r.b = *reinterpret_cast<const U4 *>(ql + 32);
+        r.h = *reinterpret_cast<const U4 *>(sb + 128 + 32 * half + 16 * pp);
+        r.sc = *reinterpret_cast<const U2 *>(sb + 192 + 8 * half);
+        r.d = *reinterpret_cast<const uint16_t *>(sb + 208);
+    }
+    static __device__ __forceinline__ XPair x_load(const float *__restrict__ xs, int lane) { return limb_x_load(xs, lane); }
+    static __device__ __forceinline__ XPair x_load_bf16(const uint16_t *__restrict__ xs, int lane) { return limb_x_load_bf16(xs, lane); }
+    static __device__ __forceinline__ Staged stage(const XPair &xp) { return limb_stage<true>(xp); }
+    // xq[2 qd + e] = planes of values 8 e .. 8 e + 7 of quadrant qd's run; xsc[qd] the scale of the
+    // quadrant's activations, xsm[qd] = -32 * (sum of the run's activations as quantised)
+    static __device__ __forceinline__ float dot(const Raw &r, const uint4 *xq, const float *xsc, const float *xsm, int c) {
+        const int sc_shift = 8 * (c & 1);
+        float out = 0.f;
+#pragma unroll
+        for (int qd = 0; qd < 4; qd++) {
+            int s0 = 0, s1 = 0;
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                const uint32_t src = (qd & 1) ? r.b.v[w] : r.a.v[w];
+                const uint32_t lo = ((qd >> 1) ? (src >> 4) : src) & 0x0F0F0F0Fu;
+                const uint32_t hv = r.h.v[w];
+                const uint32_t hs = qd == 0 ? (hv << 4) : qd == 1 ? (hv << 2) : qd == 2 ? hv : (hv >> 2);
+                const int code = (int)((hs & 0x30303030u) | lo);
+                const uint4 &pl = xq[2 * qd + (w >> 1)];
+                s0 = __builtin_amdgcn_sdot4(code, (int)((w & 1) ? pl.z : pl.x), s0, false);
+                s1 = __builtin_amdgcn_sdot4(code, (int)((w & 1) ? pl.w : pl.y), s1, false);
+            }
+            const int t = (s1 << 8) + s0;
+            const int sc = __builtin_amdgcn_sbfe((int)r.sc.v[qd >> 1], 16 * (qd & 1) + sc_shift, 8);
+            out = fmaf((float)sc, fmaf((float)t, xsc[qd], xsm[qd]), out);
+        }
+        return out * half_bits_to_float(r.d & 0xFFFFu);
+    }
+};
+
 template <int T>
 __device__ __forceinline__ void ks_load(typename KS<T>::Raw &r, const uint8_t *p, int c) {
-    if constexpr (T == kQ4_K) KS<T>::load(r, p, c);
+    if constexpr (T == kQ4_K || T == kQ6_K) KS<T>::load(r, p, c);
     else KS<T>::load(r, p);
 }
 
@@ -289,7 +368,7 @@ __device__ unsigned long long g_ks_trace[4096 * 16];
 #define KS_TRACE_WALL(k) do { } while (0)
 #endif
 
-constexpr int kWaveLdsDwords = 72 * 4;  // per wavefront: 64 uint4 of planes, 16 scales, 16 sums
+constexpr int kWaveLdsDwords = 76 * 4;  // per wavefront: 64 uint4 of planes, 16 scales, up to 32 sums
 
 // Workgroup `wg` of a problem: `waves` wavefronts work (threads beyond them only join the final
 // barrier); wavefront w handles slices w, w + waves, ... (spw of them) of the 8 * iters rows
@@ -334,22 +413,26 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, int x_bf16,
         KS_TRACE(1);
 
         uint4 xq[8];
-        float xsc[2], xsm[2] = {0.f, 0.f};
+        constexpr int NS = KS<T>::kScales, SPAN = KS<T>::kSumSpan;
+        float xsc[NS], xsm[NS];
+#pragma unroll
+        for (int i = 0; i < NS; i++) xsm[i] = 0.f;
         auto stage = [&](const XPair &p) {
             const Staged st = KS<T>::stage(p);
             my_planes[lane] = st.planes;
-            if ((lane & 3) == 0) {
-                my_scales[lane >> 2] = st.scale;
-                if constexpr (T == kQ4_K) my_sums[lane >> 2] = st.sum;
-            }
+            if ((lane & 3) == 0) my_scales[lane >> 2] = st.scale;
+            if constexpr (SPAN == 32) { if ((lane & 3) == 0) my_sums[lane >> 2] = st.sum; }
+            if constexpr (SPAN == 16) { if ((lane & 1) == 0) my_sums[lane >> 1] = st.sum; }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-            for (int i = 0; i < 8; i++) xq[i] = my_planes[8 * c + i];
-            xsc[0] = my_scales[2 * c];
-            xsc[1] = my_scales[2 * c + 1];
-            if constexpr (T == kQ4_K) { xsm[0] = my_sums[2 * c]; xsm[1] = my_sums[2 * c + 1]; }
+            for (int i = 0; i < 8; i++) xq[i] = my_planes[KS<T>::plane_idx(c, i)];
+#pragma unroll
+            for (int i = 0; i < NS; i++) {
+                xsc[i] = my_scales[KS<T>::scale_idx(c, i)];
+                if constexpr (SPAN != 0) xsm[i] = my_sums[KS<T>::sum_idx(c, i)];
+            }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
             __builtin_amdgcn_wave_barrier();
         };
@@ -544,7 +627,7 @@ int launch_ks_batch(int count, const XsBatchItem *items, hipStream_t s) {
 
 bool gemv_ks_supported(int type, int64_t K, int64_t N, const void *x) {
     if (reinterpret_cast<uintptr_t>(x) & 15) return false;
-    if (type != kQ4_0 && type != kQ8_0 && type != kQ4_K) return false;
+    if (type != kQ4_0 && type != kQ8_0 && type != kQ4_K && type != kQ6_K) return false;
     if (N <= 0 || N > (int64_t)INT32_MAX / 2) return false;
     int waves, spw;
     return ks_split(K, waves, spw);
@@ -557,6 +640,7 @@ int launch_gemv_ks(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K
     case kQ4_0: return launch_ks<kQ4_0>(x, x_bf16, M, K, W, N, bias, act, y, s);
     case kQ8_0: return launch_ks<kQ8_0>(x, x_bf16, M, K, W, N, bias, act, y, s);
     case kQ4_K: return launch_ks<kQ4_K>(x, x_bf16, M, K, W, N, bias, act, y, s);
+    case kQ6_K: return launch_ks<kQ6_K>(x, x_bf16, M, K, W, N, bias, act, y, s);
     default: return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv_ks: ggml type %d is not implemented", type);
     }
 }
@@ -567,6 +651,7 @@ int launch_gemv_ks_batch(int type, int count, const XsBatchItem *items, hipStrea
     case kQ4_0: return launch_ks_batch<kQ4_0>(count, items, s);
     case kQ8_0: return launch_ks_batch<kQ8_0>(count, items, s);
     case kQ4_K: return launch_ks_batch<kQ4_K>(count, items, s);
+    case kQ6_K: return launch_ks_batch<kQ6_K>(count, items, s);
     default: return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv batch: ggml type %d is not implemented", type);
     }
 }
