@@ -5,7 +5,9 @@ them into ``gomlx_amd/libgomlx_hipq.so``.  Cross-compiles without a GPU.
 """
 from __future__ import annotations
 
+import json
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -18,7 +20,7 @@ LIB = os.path.join(HERE, "libgomlx_hipq.so")
 HOST = os.path.join(HERE, "host")
 HOST_TEST = os.path.join(HOST, "build", "hipq_backend_test")
 
-SOURCES = ["api.hip", "dequant.hip", "gemv.hip", "gemv_xs.hip", "gemv_ks.hip", "mmq.hip", "gemm.hip"]
+SOURCES = ["api.hip", "dequant.hip", "gemv.hip", "gemv_xs.hip", "gemv_ks.hip", "mmq.hip", "gemm.hip", "gemm_dma.hip"]
 
 # -packed-fp32-ops (note the minus): keep hipcc from forming v_pk_*_f32 instructions.
 # -ffp-contract=off: dequantisation must round every fp32 operation on its own; fused
@@ -27,6 +29,7 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-command-line-argument", "-Wno-unknown-attributes",
+    "-Rpass-analysis=kernel-resource-usage",
 ]
 
 
@@ -37,23 +40,53 @@ def hipcc() -> str:
     raise RuntimeError("hipcc not found")
 
 
-def _compile(src: str) -> str:
+def _kernel_resources(stderr: str) -> dict:
+    """Per-kernel register and scratch use from the compiler's resource-usage remarks."""
+    out, name = {}, None
+    for line in stderr.splitlines():
+        m = re.search(r"remark: .*Function Name: (\S+)", line)
+        if m:
+            name = m.group(1)
+            out[name] = {}
+            continue
+        m = re.search(r"remark: .*?\s(VGPRs|AGPRs|ScratchSize \[bytes/lane\]|Occupancy \[waves/SIMD\]|LDS Size \[bytes/block\]): (\d+)", line)
+        if m and name:
+            out[name][m.group(1).split(" ")[0]] = int(m.group(2))
+    return out
+
+
+def _compile(src: str):
     obj = os.path.join(OBJ, os.path.splitext(src)[0] + ".o")
     cmd = [hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{r.stdout}\n{r.stderr}")
-    noise = ("packed-fp32-ops", "target feature")
-    warn = "\n".join(l for l in r.stderr.splitlines() if l.strip() and not any(n in l for n in noise))
+    noise = ("packed-fp32-ops", "target feature", "remark:")
+    lines = r.stderr.splitlines()
+    warn = "\n".join(l for i, l in enumerate(lines) if l.strip() and not any(n in l for n in noise)
+                     and not (i > 0 and "remark:" in lines[i - 1]) and not (i > 1 and "remark:" in lines[i - 2]))
     if "warning" in warn:
         sys.stderr.write(warn + "\n")
-    return obj
+    res = _kernel_resources(r.stderr)
+    # A kernel that spills registers to scratch memory runs one to two orders of magnitude slower
+    # than intended (it has happened when the compiler stopped inlining a kernel's lambdas): treat
+    # it as a build error rather than ship it.
+    spilled = {k: v["ScratchSize"] for k, v in res.items() if v.get("ScratchSize", 0) > 0}
+    if spilled:
+        raise RuntimeError(f"{src}: kernels use scratch memory (bytes per lane): {spilled}")
+    return obj, res
 
 
 def build(verbose: bool = True) -> str:
     os.makedirs(OBJ, exist_ok=True)
     with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as ex:
-        objs = list(ex.map(_compile, SOURCES))
+        results = list(ex.map(_compile, SOURCES))
+    objs = [o for o, _ in results]
+    resources = {}
+    for _, res in results:
+        resources.update(res)
+    with open(os.path.join(OBJ, "kernel_resources.json"), "w") as f:
+        json.dump(resources, f, indent=1, sort_keys=True)
     cmd = [hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:

@@ -31,6 +31,9 @@ int hip_fail(hipError_t e, const char *what);
 int use_device();
 int device_cu_count();
 
+// ---- per-stream scratch memory (grows on demand; must exist before a graph recording uses it) ----
+int stream_workspace(hipStream_t s, size_t bytes, void **out);
+
 // ---- launch ---------------------------------------------------------------------------
 struct ProfileState {
     bool active = false;
@@ -75,6 +78,12 @@ int launch_mmq(int type, const float *x, int64_t M, int64_t K, const uint8_t *W,
 struct XsBatchItem { const float *x; const uint8_t *W; const float *bias; float *y; int64_t K, N; int act; };
 int launch_gemv_xs_batch(int type, int count, const XsBatchItem *items, hipStream_t s);
 int launch_gemv_ks_batch(int type, int count, const XsBatchItem *items, hipStream_t s);
+// Large batches: dequantise W once into a 16-bit image (in `workspace`, gemm_two_pass_workspace()
+// bytes), then a plain 16-bit MFMA GEMM.
+bool gemm_two_pass_supported(int type, bool x_is_bf16, int64_t M, int64_t K, int64_t N, const void *x);
+size_t gemm_two_pass_workspace(bool x_is_bf16, int64_t M, int64_t K, int64_t N);
+int launch_gemm_two_pass(int type, bool x_is_bf16, const void *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias,
+                         int act, float *y, void *workspace, hipStream_t s);
 int launch_gemm(int type, bool x_is_bf16, const void *x, int64_t M, int64_t K, const uint8_t *W, int64_t N,
                 const float *bias, int act, float *y, hipStream_t s);
 

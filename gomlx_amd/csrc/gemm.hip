@@ -217,7 +217,7 @@ __global__ __launch_bounds__(512) void gemm_kernel(const void *Xv, const uint8_t
     const uint32_t woff_t = (uint32_t)(wrow_c * row_bytes);  // half last step: runs 2, 3 re-read block 0
     const uint8_t *xtile = reinterpret_cast<const uint8_t *>(Xv) + (int64_t)bm * K * XRaw<BF16>::ESIZE;
     const uint8_t *wtile = W + (int64_t)bn * row_bytes;
-    auto fetch = [&](int kt, XRaw<BF16> &x, WRaw<T> &w) {  // unconditional: steps past the end re-read the last one
+    auto fetch = [&](int kt, XRaw<BF16> &x, WRaw<T> &w) __attribute__((always_inline)) {  // unconditional: steps past the end re-read the last one
 #ifdef GQ_GEMM_NOFETCH  // tuning builds only
         if (kt > 2) return;
 #endif
@@ -240,12 +240,27 @@ __global__ __launch_bounds__(512) void gemm_kernel(const void *Xv, const uint8_t
 #else
 #define GEMM_TRACE(slot) do { } while (0)
 #endif
-    // One K step: the 16 MFMAs of step kt out of `cur`, in four groups of four, each group followed
-    // in program order by a quarter of the staging of step kt + 1 into `nxt` (MFMAs are issued
-    // asynchronously, so the vector ALU work that follows them runs in their shadow).  Fragments
-    // are read one group ahead.  The scheduling barriers keep the compiler from regrouping this.
-    auto step = [&](int kt, const uint16_t *cur, uint16_t *nxt, XRaw<BF16> &x, WRaw<T> &wq, auto masked) {
-        constexpr bool MASKED = decltype(masked)::value;
+    // One K step.  The MFMAs run in four groups of four, each group followed in program order by a
+    // quarter of the staging of step kt + 1 into `nxt` (MFMAs are issued asynchronously, so the
+    // vector ALU work that follows them runs in their shadow).  Fragments are read one group ahead,
+    // and the groups are skewed by one against the barriers: a step opens with the reads of its
+    // own group 0 and the MFMAs of the previous step's group 3, whose fragments were read before
+    // the barrier, so the matrix cores have work while the first LDS reads after a barrier are in
+    // flight.  The scheduling barriers keep the compiler from regrouping this.
+    // (The fp32-activation variants hold twice the activation registers and keep the plain order:
+    // carrying fragments across the barrier pushes some of them over the register budget.)
+    constexpr bool SKEW = BF16;
+    typename Op::vec8 fa[2][2], fb[2][2];  // [set][tile]; with SKEW set 1 carries group 3 across the barrier
+    auto mfma_group = [&](int set) __attribute__((always_inline)) {
+#ifndef GQ_GEMM_NOMFMA  // tuning builds only
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++) acc[i][j] = Op::mfma(fa[set][i], fb[set][j], acc[i][j]);
+#endif
+    };
+    auto step = [&](int kt, const uint16_t *cur, uint16_t *nxt, XRaw<BF16> &x, WRaw<T> &wq, auto masked, auto first) __attribute__((always_inline)) {
+        constexpr bool MASKED = decltype(masked)::value, FIRST = decltype(first)::value;
         const uint16_t *xs = cur, *ws = cur + BM * LDS_STRIDE;
         const int k1 = (kt + 1) * BK;
         // the register set staged here is refilled, piece by piece, with step kt + 3
@@ -261,29 +276,26 @@ __global__ __launch_bounds__(512) void gemm_kernel(const void *Xv, const uint8_t
         for (int j = 0; j < XRaw<BF16>::NCH; j++) fo[j] = ftail ? xoff_t[j] : xoff[j];
         const uint32_t wmask = MASKED ? all_ones_if(k1 + 16 * wrun < K) : 0xFFFFFFFFu;
         uint4 *wd = reinterpret_cast<uint4 *>(nxt + wdst_off);
-        typename Op::vec8 a[2][2], b[2][2];
-        auto frags = [&](int kk, typename Op::vec8 *fa, typename Op::vec8 *fb) {
-            const int koff = kk * 16 + (lane >> 5) * 8;
+        auto frags = [&](int kk) __attribute__((always_inline)) {
+            const int koff = kk * 16 + (lane >> 5) * 8, set = kk & 1;
 #pragma unroll
             for (int i = 0; i < 2; i++)
-                fa[i] = *reinterpret_cast<const typename Op::vec8 *>(&xs[(wm + i * 32 + (lane & 31)) * LDS_STRIDE + koff]);
+                fa[set][i] = *reinterpret_cast<const typename Op::vec8 *>(&xs[(wm + i * 32 + (lane & 31)) * LDS_STRIDE + koff]);
 #pragma unroll
             for (int j = 0; j < 2; j++)
-                fb[j] = *reinterpret_cast<const typename Op::vec8 *>(&ws[(wn + j * 32 + (lane & 31)) * LDS_STRIDE + koff]);
+                fb[set][j] = *reinterpret_cast<const typename Op::vec8 *>(&ws[(wn + j * 32 + (lane & 31)) * LDS_STRIDE + koff]);
         };
         float w[16];
-        frags(0, a[0], b[0]);
+        if (!SKEW) frags(0);
 #pragma unroll
         for (int kk = 0; kk < 4; kk++) {
-            if (kk < 3) frags(kk + 1, a[(kk + 1) & 1], b[(kk + 1) & 1]);
-#pragma unroll
-            for (int i = 0; i < 2; i++)
-#pragma unroll
-                for (int j = 0; j < 2; j++) {
-#ifndef GQ_GEMM_NOMFMA  // tuning builds only
-                    acc[i][j] = Op::mfma(a[kk & 1][i], b[kk & 1][j], acc[i][j]);
-#endif
-                }
+            if (SKEW) {
+                frags(kk);
+                if (kk > 0 || !FIRST) mfma_group((kk + 1) & 1);  // group kk - 1 (kk = 0: group 3 of the step before)
+            } else {
+                if (kk < 3) frags(kk + 1);
+                mfma_group(kk & 1);
+            }
 #ifndef GQ_GEMM_NOSTAGE  // tuning builds only
             x.template store_part<MASKED>(kk, nxt, k1, K, tid);
             wq.part(kk, w);
@@ -304,7 +316,7 @@ __global__ __launch_bounds__(512) void gemm_kernel(const void *Xv, const uint8_t
                 min((int64_t)kc * (BK / 16) + wrun, n16 - 1));
 #endif
     };
-    auto stage_first = [&](uint16_t *buf, const XRaw<BF16> &x, const WRaw<T> &wq) {
+    auto stage_first = [&](uint16_t *buf, const XRaw<BF16> &x, const WRaw<T> &wq) __attribute__((always_inline)) {
         float w[16];
         const uint32_t wmask = all_ones_if(16 * wrun < K);
         uint4 *wd = reinterpret_cast<uint4 *>(buf + wdst_off);
@@ -334,14 +346,14 @@ __global__ __launch_bounds__(512) void gemm_kernel(const void *Xv, const uint8_t
     fetch(2, xr[0], wr[0]);
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
-    auto pair = [&](int kt, auto masked) {
+    auto pair = [&](int kt, auto masked, auto first) __attribute__((always_inline)) {
         GEMM_TRACE(0);
-        step(kt, lds, lds + LDS_BUF, xr[1], wr[1], masked);
+        step(kt, lds, lds + LDS_BUF, xr[1], wr[1], masked, first);
         __builtin_amdgcn_sched_barrier(0);
         GEMM_TRACE(5);
         __syncthreads();
         GEMM_TRACE(6);
-        step(kt + 1, lds + LDS_BUF, lds, xr[0], wr[0], masked);
+        step(kt + 1, lds + LDS_BUF, lds, xr[0], wr[0], masked, std::false_type());
         __builtin_amdgcn_sched_barrier(0);
         GEMM_TRACE(7);
         __syncthreads();
@@ -351,10 +363,11 @@ __global__ __launch_bounds__(512) void gemm_kernel(const void *Xv, const uint8_t
     // from the prologue's different order and over-wait).  Pairs whose staged steps (kt + 1, kt + 2)
     // lie entirely inside K skip the zero-fill masks.
     const int nk_full = K / BK;
-    pair(0, std::true_type());
+    pair(0, std::true_type(), std::true_type());
     int kt = 2;
-    for (; kt + 2 < nk_full; kt += 2) pair(kt, std::false_type());
-    for (; kt < nk; kt += 2) pair(kt, std::true_type());
+    for (; kt + 2 < nk_full; kt += 2) pair(kt, std::false_type(), std::false_type());
+    for (; kt < nk; kt += 2) pair(kt, std::true_type(), std::false_type());
+    if (SKEW) mfma_group(1);  // group 3 of the last step
 
     // ---- epilogue: acc[i][j][r] is Y[m, n] with n = lane % 32, m = 8*(r/4) + 4*(lane/32) + r%4
 #pragma unroll

@@ -1,0 +1,353 @@
+// Large-batch quantised Dense in two passes:
+//   1. the weight matrix is dequantised once into a 16-bit [N, K] image in a workspace (exact
+//      fp32 values, one rounding to the MFMA operand type: the same operand values the fused
+//      kernel of gemm.hip builds tile by tile);
+//   2. a plain 16-bit x 16-bit -> fp32 MFMA GEMM contracts it with the activations.
+//
+// The fused kernel converts a 128-row slab of W again for every 256 rows of activations, and on a
+// SIMD those vector-ALU instructions do not overlap with its MFMAs; from a few hundred rows on it
+// is cheaper to convert once and let the matrix cores run without vector work.  The GEMM moves
+// both operands from global memory straight into LDS (buffer loads with the LDS modifier: no
+// registers, no vector-ALU instructions) three K steps ahead through a ring of three stages.
+//
+// Tile: 256 x 128 per workgroup, 8 wavefronts x (64 x 64 = 2 x 2 v_mfma_f32_32x32x16), or 128 x 128
+// and 128 x 64 when the problem has too few large tiles to fill the chip; K in steps of 64.  LDS rows are 128 bytes, unpadded (the DMA writes 1 KB = 8 rows per wavefront
+// instruction, lane l -> bytes 16 l ..), and 16-byte chunk c of row r is kept in slot
+// c ^ ((r >> 1) & 7): 16 consecutive lanes of a fragment read then cover all 64 banks once.  The
+// swizzle is applied on the global side: lane l of a DMA fetches chunk (l & 7) ^ ((r >> 1) & 7) of
+// row r = 8 * block + (l >> 3), so every 128-byte row is still read as one full line.
+#include "blocks.hpp"
+#include "common.hpp"
+
+#include <cstdlib>
+
+namespace gq {
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int DK = 64;
+constexpr int ROWB = 128;  // bytes per LDS row
+constexpr int NSTAGE = 3;
+
+template <bool BF16> struct Op16;
+template <> struct Op16<true> {
+    typedef bf16x8 vec8;
+    static __device__ __forceinline__ uint32_t pack(float a, float b) {
+        typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+        bf2 v;
+        v.x = (__bf16)a;
+        v.y = (__bf16)b;
+        return __builtin_bit_cast(uint32_t, v);
+    }
+    static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+};
+template <> struct Op16<false> {
+    typedef f16x8 vec8;
+    static __device__ __forceinline__ uint32_t pack(float a, float b) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        h2 v;
+        v.x = (_Float16)a;
+        v.y = (_Float16)b;
+        return __builtin_bit_cast(uint32_t, v);
+    }
+    static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+};
+
+// ---- pass 1: GGML blocks -> 16-bit [N, K] -------------------------------------------------------
+// One thread per run of 16 weights (32 output bytes).
+template <int T, bool BF16>
+__global__ __launch_bounds__(256) void dequant16bit_kernel(const uint8_t *__restrict__ W, uint16_t *__restrict__ out, int64_t runs_per_row,
+                                                          int64_t total_runs, int64_t row_bytes) {
+    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (g >= total_runs) return;
+    const int64_t row = g / runs_per_row, run = g % runs_per_row;
+    float w[16];
+    dequant16<T>(W + row * row_bytes, run, w);
+    uint4 *dst = reinterpret_cast<uint4 *>(out + g * 16);
+    dst[0] = make_uint4(Op16<BF16>::pack(w[0], w[1]), Op16<BF16>::pack(w[2], w[3]), Op16<BF16>::pack(w[4], w[5]), Op16<BF16>::pack(w[6], w[7]));
+    dst[1] = make_uint4(Op16<BF16>::pack(w[8], w[9]), Op16<BF16>::pack(w[10], w[11]), Op16<BF16>::pack(w[12], w[13]),
+                        Op16<BF16>::pack(w[14], w[15]));
+}
+
+// fp32 activations -> fp16 [M, K] (the generic batched path rounds activations to fp16 operands)
+__global__ __launch_bounds__(256) void x_to_f16_kernel(const float *__restrict__ x, uint16_t *__restrict__ out, int64_t total8) {
+    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (g >= total8) return;
+    const float4 a = reinterpret_cast<const float4 *>(x)[2 * g], b = reinterpret_cast<const float4 *>(x)[2 * g + 1];
+    reinterpret_cast<uint4 *>(out)[g] =
+        make_uint4(Op16<false>::pack(a.x, a.y), Op16<false>::pack(a.z, a.w), Op16<false>::pack(b.x, b.y), Op16<false>::pack(b.z, b.w));
+}
+
+// ---- pass 2: 16-bit GEMM with global -> LDS DMA --------------------------------------------------
+// One 16-byte-per-lane buffer load whose data goes to LDS at lds_addr + 16 * lane.  The compiler
+// does not see that the instruction writes LDS or that it is counted by vmcnt: the kernel orders
+// these loads against its LDS reads with explicit waits and barriers.  (The s_nop is the wait
+// state the hardware wants between a write of M0 and an LDS DMA; the assembler does not add it
+// inside inline assembly.)
+__device__ __forceinline__ void dma16(uint32_t lds_addr, i32x4 rsrc, uint32_t voff, uint32_t soff) {
+    lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);  // both are uniform by construction
+    soff = __builtin_amdgcn_readfirstlane(soff);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds" ::"s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+}
+
+__device__ __forceinline__ i32x4 make_rsrc(const void *base, uint64_t bytes) {
+    const uint64_t b = reinterpret_cast<uint64_t>(base);
+    i32x4 r;
+    r.x = __builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+    r.y = __builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32));  // stride 0: raw buffer, byte offsets
+    r.z = __builtin_amdgcn_readfirstlane((int)(uint32_t)(bytes > 0xFFFFFFFFull ? 0xFFFFFFFFull : bytes));
+    r.w = 0x00020000;  // 32-bit data format, no swizzle
+    return r;
+}
+
+// X [M, K] and Wh [N, K] 16-bit, K % 64 == 0, both 16-byte aligned.  The workgroup tile is
+// (128 TM) x (64 TN): 4 x 2 wavefronts of (32 TM) x (32 TN) each.  TM = TN = 2 is the tile for
+// large problems; the smaller ones keep the chip full when M x N yields too few big tiles.
+template <int TM, int TN> struct DmaTile {
+    static constexpr int DM = 128 * TM, DN = 64 * TN;
+    static constexpr int XI = 2 * TM, WI = TN;                 // DMAs per wavefront and step: X, W
+    static constexpr int kStageBytes = (DM + DN) * ROWB;
+    static constexpr int kLdsBytes = NSTAGE * kStageBytes;
+};
+
+template <bool BF16, int TM, int TN>
+__global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const uint16_t *Wh, const float *__restrict__ bias,
+                                                       float *__restrict__ Y, int M, int K, int N, int act) {
+    typedef Op16<BF16> Op;
+    typedef DmaTile<TM, TN> G;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int bm = blockIdx.y * G::DM, bn = blockIdx.x * G::DN;
+    const int wm = (wave >> 1) * (32 * TM), wn = (wave & 1) * (32 * TN);
+    const int nk = K / DK;
+
+    // ---- DMA roles: per step a wavefront moves XI row blocks (8 rows each) of X and WI of W
+    const i32x4 xrsrc = make_rsrc(X + (int64_t)bm * K, (uint64_t)(M - bm) * (uint64_t)K * 2);
+    const i32x4 wrsrc = make_rsrc(Wh + (int64_t)bn * K, (uint64_t)(N - bn) * (uint64_t)K * 2);
+    uint32_t xvoff[G::XI], wvoff[G::WI];
+#pragma unroll
+    for (int j = 0; j < G::XI; j++) {
+        const int row = 8 * (G::XI * wave + j) + (lane >> 3);
+        const int c = (lane & 7) ^ ((row >> 1) & 7);
+        xvoff[j] = (uint32_t)min(row, M - 1 - bm) * (uint32_t)(K * 2) + (uint32_t)c * 16u;
+    }
+#pragma unroll
+    for (int j = 0; j < G::WI; j++) {
+        const int row = 8 * (G::WI * wave + j) + (lane >> 3);
+        const int c = (lane & 7) ^ ((row >> 1) & 7);
+        wvoff[j] = (uint32_t)min(row, N - 1 - bn) * (uint32_t)(K * 2) + (uint32_t)c * 16u;
+    }
+    const uint32_t lds0 = (uint32_t)reinterpret_cast<uintptr_t>(lds);
+    const uint32_t xdst = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)(G::XI * wave) * 1024u);
+    const uint32_t wdst = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)(G::DM * ROWB) + (uint32_t)(G::WI * wave) * 1024u);
+    auto issue = [&](int kt, int stage) __attribute__((always_inline)) {  // steps past the end re-read the last one (the data is never used)
+#ifdef GQ_DMA_NOISSUE  // tuning builds only: nothing is loaded after the prologue
+        if (kt > 1) return;
+#endif
+#ifdef GQ_DMA_HOT  // tuning builds only: every step re-reads step 0
+        const uint32_t soff = 0;
+#else
+        const uint32_t soff = (uint32_t)min(kt, nk - 1) * (uint32_t)(DK * 2);
+#endif
+        const uint32_t sb = (uint32_t)stage * (uint32_t)G::kStageBytes;
+#pragma unroll
+        for (int j = 0; j < G::XI; j++) dma16(xdst + sb + (uint32_t)j * 1024u, xrsrc, xvoff[j], soff);
+#pragma unroll
+        for (int j = 0; j < G::WI; j++) dma16(wdst + sb + (uint32_t)j * 1024u, wrsrc, wvoff[j], soff);
+    };
+
+    // ---- fragment addresses: row (w? + 32 t + lane % 32), chunk 2 kk + lane / 32, swizzled
+    uint32_t aoff[4], boff[4];
+    {
+        const int l = lane & 31, sw = (l >> 1) & 7, hi = lane >> 5;  // wm, wn, 32 t are multiples of 16
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+            const uint32_t slot = (uint32_t)((2 * kk + hi) ^ sw);
+            aoff[kk] = (uint32_t)(wm + l) * ROWB + slot * 16u;
+            boff[kk] = (uint32_t)(G::DM * ROWB) + (uint32_t)(wn + l) * ROWB + slot * 16u;
+        }
+    }
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    typename Op::vec8 fa[2][TM], fb[2][TN];  // [set][tile]
+    auto frags = [&](int stage, int kk) __attribute__((always_inline)) {
+        const uint8_t *base = lds + stage * G::kStageBytes;
+        const int set = kk & 1;
+#pragma unroll
+        for (int t = 0; t < TM; t++) fa[set][t] = *reinterpret_cast<const typename Op::vec8 *>(base + aoff[kk] + t * 32 * ROWB);
+#pragma unroll
+        for (int t = 0; t < TN; t++) fb[set][t] = *reinterpret_cast<const typename Op::vec8 *>(base + boff[kk] + t * 32 * ROWB);
+    };
+    auto mfma_group = [&](int set) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) acc[i][j] = Op::mfma(fa[set][i], fb[set][j], acc[i][j]);
+    };
+    // Waits until this wavefront's DMAs of the next step have landed (those of the step after it may
+    // stay in flight) and its own LDS reads are done, then meets the other wavefronts.
+    auto publish = [&]() __attribute__((always_inline)) {
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(G::XI + G::WI) : "memory");
+    };
+
+    issue(0, 0);
+    issue(1, 1);
+    publish();
+    // Step kt computes out of stage kt % 3 while the DMAs of step kt + 2 fill stage (kt + 2) % 3,
+    // which every wavefront finished reading before the barrier that ended step kt - 1.  The MFMA
+    // groups are skewed by one against the barriers (group 3 of a step issues after the barrier,
+    // behind the first fragment reads of the next step).
+    auto step = [&](int kt, int stage, bool first) __attribute__((always_inline)) {
+        issue(kt + 2, (stage + 2) % NSTAGE);
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+            frags(stage, kk);
+            if (kk > 0 || !first) mfma_group((kk + 1) & 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        publish();
+    };
+    step(0, 0, true);
+    int kt = 1;
+    for (; kt + 2 < nk; kt += 3) {
+        step(kt, 1, false);
+        step(kt + 1, 2, false);
+        step(kt + 2, 0, false);
+    }
+    if (kt < nk) { step(kt, 1, false); kt++; }
+    if (kt < nk) { step(kt, 2, false); kt++; }
+    mfma_group(1);  // group 3 of the last step
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the re-read DMAs of the last two steps
+
+    // ---- epilogue: acc[i][j][r] is Y[m, n] with n = lane % 32, m = 8*(r/4) + 4*(lane/32) + r%4
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const int n = bn + wn + j * 32 + (lane & 31);
+        if (n >= N) continue;
+        const float bv = bias ? bias[n] : 0.f;
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = bm + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (m < M) Y[(int64_t)m * N + n] = apply_act(act, acc[i][j][r] + bv);
+            }
+        }
+    }
+}
+
+template <int T, bool BF16>
+int launch_dequant16bit(const uint8_t *W, int64_t N, int64_t K, uint16_t *out, hipStream_t s) {
+    const int64_t runs_per_row = K / 16, total = N * runs_per_row;
+    const int64_t row_bytes = (K / Geom<T>::vpb) * Geom<T>::bpb;
+    return launch(dequant16bit_kernel<T, BF16>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, W, out, runs_per_row, total, row_bytes);
+}
+
+template <bool BF16>
+int launch_dequant16bit_type(int type, const uint8_t *W, int64_t N, int64_t K, uint16_t *out, hipStream_t s) {
+    switch (type) {
+    case kQ4_0: return launch_dequant16bit<kQ4_0, BF16>(W, N, K, out, s);
+    case kQ8_0: return launch_dequant16bit<kQ8_0, BF16>(W, N, K, out, s);
+    case kIQ4_NL: return launch_dequant16bit<kIQ4_NL, BF16>(W, N, K, out, s);
+    case kQ4_K: return launch_dequant16bit<kQ4_K, BF16>(W, N, K, out, s);
+    case kQ6_K: return launch_dequant16bit<kQ6_K, BF16>(W, N, K, out, s);
+    default: return fail(GQ_ERR_NOT_IMPLEMENTED, "qdense: ggml type %d is not implemented", type);
+    }
+}
+
+template <bool BF16, int TM, int TN>
+int launch_gemm16_tile(const uint16_t *x, int64_t M, int64_t K, const uint16_t *Wh, int64_t N, const float *bias, int act, float *y,
+                       hipStream_t s) {
+    typedef DmaTile<TM, TN> G;
+    static const bool lds_ok = [] {
+        return hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_dma_kernel<BF16, TM, TN>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, G::kLdsBytes) == hipSuccess;
+    }();
+    if (!lds_ok) return fail(GQ_ERR_HIP, "gemm: cannot reserve %d bytes of LDS", G::kLdsBytes);
+    const dim3 grid((unsigned)((N + G::DN - 1) / G::DN), (unsigned)((M + G::DM - 1) / G::DM));
+    return launch(gemm_dma_kernel<BF16, TM, TN>, grid, dim3(512), (size_t)G::kLdsBytes, s, x, Wh, bias, y, (int)M, (int)K, (int)N, act);
+}
+
+// GOMLX_HIPQ_GEMM_TILE=0|1|2 forces the 256x128 / 128x128 / 128x64 tile (tuning runs only).
+int tile_env() {
+    static const int v = [] { const char *e = std::getenv("GOMLX_HIPQ_GEMM_TILE"); return e ? std::atoi(e) : -1; }();
+    return v;
+}
+
+// The largest tile that still gives the chip about one workgroup per CU.
+template <bool BF16>
+int launch_gemm16(const uint16_t *x, int64_t M, int64_t K, const uint16_t *Wh, int64_t N, const float *bias, int act, float *y, hipStream_t s) {
+    const int64_t want = (int64_t)device_cu_count() * 3 / 4;
+    auto tiles = [&](int64_t dm, int64_t dn) { return ((M + dm - 1) / dm) * ((N + dn - 1) / dn); };
+    int choice = tiles(256, 128) >= want ? 0 : tiles(128, 128) >= want ? 1 : 2;
+    if (tile_env() >= 0 && tile_env() <= 2) choice = tile_env();
+    switch (choice) {
+    case 0: return launch_gemm16_tile<BF16, 2, 2>(x, M, K, Wh, N, bias, act, y, s);
+    case 1: return launch_gemm16_tile<BF16, 1, 2>(x, M, K, Wh, N, bias, act, y, s);
+    default: return launch_gemm16_tile<BF16, 1, 1>(x, M, K, Wh, N, bias, act, y, s);
+    }
+}
+
+// Measured against the fused kernel (K = 4096, N = 4096 .. 14336): the two passes win from the
+// first batch size the GEMV passes do not take (17 rows: 33 against 60 us for Q8_0 at 64 rows, 37
+// against 66 .. 102 us at 512 rows) up to the largest; the fused kernel is within 5 % only for
+// Q8_0 with bf16 activations, whose conversion is the cheapest: there it stays ahead between
+// about 1300 and 4000 rows (2048 rows: 85 .. 88 us against 81 .. 95 us for the two passes).
+constexpr int64_t kMinRowsTwoPass = 17;
+constexpr int64_t kFusedQ8Bf16From = 1281, kFusedQ8Bf16Below = 4096;
+constexpr uint64_t kMaxImageBytes = (uint64_t)4 << 30;   // largest 16-bit weight image kept in a workspace
+
+// GOMLX_HIPQ_TWO_PASS_MIN_ROWS=<rows> overrides the threshold (tuning runs only).
+int64_t two_pass_env_rows() {
+    static const int64_t v = [] { const char *e = std::getenv("GOMLX_HIPQ_TWO_PASS_MIN_ROWS"); return e ? (int64_t)std::atoll(e) : (int64_t)0; }();
+    return v;
+}
+
+}  // namespace
+
+// K a multiple of 64 (whole LDS rows; also whole blocks of every format), per-thread byte offsets of
+// a 256-row tile within 32 bits, 16-byte aligned activations.
+bool gemm_two_pass_supported(int type, bool x_is_bf16, int64_t M, int64_t K, int64_t N, const void *x) {
+    if (type != kQ4_0 && type != kQ8_0 && type != kIQ4_NL && type != kQ4_K && type != kQ6_K) return false;
+    if (type == kQ8_0 && x_is_bf16 && M >= kFusedQ8Bf16From && M < kFusedQ8Bf16Below && two_pass_env_rows() <= 0) return false;
+    const int64_t min_rows = two_pass_env_rows() > 0 ? two_pass_env_rows() : kMinRowsTwoPass;
+    if (M < min_rows || K % 64 != 0) return false;
+    if (K > (1 << 22) || N > INT32_MAX || M > INT32_MAX || (M + 127) / 128 > 65535) return false;
+    if ((uint64_t)N * (uint64_t)K * 2 > kMaxImageBytes) return false;
+    return (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+}
+
+size_t gemm_two_pass_workspace(bool x_is_bf16, int64_t M, int64_t K, int64_t N) {
+    const size_t w = ((size_t)N * K * 2 + 255) & ~(size_t)255;
+    return w + (x_is_bf16 ? 0 : (size_t)M * K * 2);
+}
+
+int launch_gemm_two_pass(int type, bool x_is_bf16, const void *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias,
+                         int act, float *y, void *workspace, hipStream_t s) {
+    uint16_t *wh = static_cast<uint16_t *>(workspace);
+    if (x_is_bf16) {
+        if (int rc = launch_dequant16bit_type<true>(type, W, N, K, wh, s)) return rc;
+        return launch_gemm16<true>(static_cast<const uint16_t *>(x), M, K, wh, N, bias, act, y, s);
+    }
+    uint16_t *xh = wh + (((size_t)N * K * 2 + 255) & ~(size_t)255) / 2;
+    if (int rc = launch_dequant16bit_type<false>(type, W, N, K, wh, s)) return rc;
+    const int64_t total8 = M * K / 8;
+    if (int rc = launch(x_to_f16_kernel, dim3((unsigned)((total8 + 255) / 256)), dim3(256), 0, s, static_cast<const float *>(x), xh, total8))
+        return rc;
+    return launch_gemm16<false>(xh, M, K, wh, N, bias, act, y, s);
+}
+
+}  // namespace gq

@@ -12,8 +12,6 @@
 #include "blocks.hpp"
 #include "common.hpp"
 
-#include <cstdlib>
-
 namespace gq {
 
 namespace {
@@ -493,23 +491,8 @@ int launch_run16(const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t
 
 // ---- host side --------------------------------------------------------------------------
 
-struct Tuning { int rows_per_wave; int waves; };
-
-// Rows per wavefront and wavefronts per workgroup.  GOMLX_HIPQ_GEMV="R,WAVES" overrides the
-// built-in choice (R in {1,2,4}, WAVES in {4,8,16}); it exists for tuning runs.
-Tuning tuning_for(int64_t N) {
-    static const Tuning env = [] {
-        Tuning t{0, 0};
-        if (const char *e = std::getenv("GOMLX_HIPQ_GEMV")) {
-            int r = 0, w = 0;
-            if (std::sscanf(e, "%d,%d", &r, &w) == 2 && (r == 1 || r == 2 || r == 4) && (w == 4 || w == 8 || w == 16)) t = {r, w};
-        }
-        return t;
-    }();
-    if (env.rows_per_wave) return env;
-    (void)N;
-    return {2, 8};
-}
+// Two rows per wavefront, eight wavefronts per workgroup (the best of the combinations measured).
+constexpr int kRowsPerWave = 2, kWavesPerWG = 8;
 
 constexpr int kMaxChunk = 16384;  // fp32 activations staged in LDS per pass: 64 KiB
 
@@ -533,25 +516,10 @@ int launch_one(const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N
     }
 }
 
-template <int T, int R>
-int launch_waves(int waves, const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias,
-                 int act, float *y, hipStream_t s) {
-    switch (waves) {
-    case 4: return launch_one<T, R, 4>(x, M, K, W, N, bias, act, y, s);
-    case 16: return launch_one<T, R, 16>(x, M, K, W, N, bias, act, y, s);
-    default: return launch_one<T, R, 8>(x, M, K, W, N, bias, act, y, s);
-    }
-}
-
 template <int T>
 int launch_type(const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y,
                 hipStream_t s) {
-    const Tuning t = tuning_for(N);
-    switch (t.rows_per_wave) {
-    case 1: return launch_waves<T, 1>(t.waves, x, M, K, W, N, bias, act, y, s);
-    case 4: return launch_waves<T, 4>(t.waves, x, M, K, W, N, bias, act, y, s);
-    default: return launch_waves<T, 2>(t.waves, x, M, K, W, N, bias, act, y, s);
-    }
+    return launch_one<T, kRowsPerWave, kWavesPerWG>(x, M, K, W, N, bias, act, y, s);
 }
 
 }  // namespace

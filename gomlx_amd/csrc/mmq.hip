@@ -24,8 +24,6 @@
 #include "blocks.hpp"
 #include "common.hpp"
 
-#include <map>
-#include <mutex>
 
 namespace gq {
 
@@ -290,29 +288,6 @@ __global__ __launch_bounds__(256) void mmq_reduce_kernel(const float *__restrict
     *reinterpret_cast<float4 *>(Y + i) = make_float4(apply_act(act, s.x), apply_act(act, s.y), apply_act(act, s.z), apply_act(act, s.w));
 }
 
-// ---- per-stream workspace for the K-slice partial sums -----------------------------------
-struct Workspace { void *ptr = nullptr; size_t bytes = 0; };
-std::mutex g_ws_mutex;
-std::map<hipStream_t, Workspace> g_ws;
-
-int workspace_for(hipStream_t s, size_t bytes, float **out) {
-    std::lock_guard<std::mutex> lock(g_ws_mutex);
-    Workspace &w = g_ws[s];
-    if (w.bytes < bytes) {
-        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
-        if (s != nullptr && hipStreamIsCapturing(s, &st) == hipSuccess && st != hipStreamCaptureStatusNone)
-            return fail(GQ_ERR_INVALID, "qdense: the %zu-byte split-K workspace of this stream must exist before a graph is "
-                        "recorded; run the same call once outside the recording first", bytes);
-        // An outgrown buffer is retired, not freed: a recorded graph may still point at it.
-        w = Workspace();
-        size_t want = bytes < (size_t)(4u << 20) ? (size_t)(4u << 20) : bytes;
-        GQ_HIP(hipMalloc(&w.ptr, want));
-        w.bytes = want;
-    }
-    *out = static_cast<float *>(w.ptr);
-    return GQ_OK;
-}
-
 }  // namespace
 
 bool mmq_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, const void *bias, const void *y) {
@@ -333,8 +308,8 @@ int launch_mmq(int type, const float *x, int64_t M, int64_t K, const uint8_t *W,
     // workspace: [activation images: mtiles x nslices x kLdsBytes][partial sums: nslices x M x N fp32]
     const size_t img_bytes = (size_t)mtiles * nslices * kLdsBytes;
     const size_t part_bytes = (size_t)nslices * M * N * sizeof(float);
-    float *ws = nullptr;
-    if (int rc = workspace_for(s, img_bytes + part_bytes, &ws)) return rc;
+    void *ws = nullptr;
+    if (int rc = stream_workspace(s, img_bytes + part_bytes, &ws)) return rc;
     uint8_t *ximg = reinterpret_cast<uint8_t *>(ws);
     float *partial = reinterpret_cast<float *>(ximg + img_bytes);
     const int64_t row_bytes = (K / 256) * 144;

@@ -35,6 +35,20 @@ def test_no_oracle_or_torch_linked_into_the_library():
     assert "ggml_oracle" not in out and "torch" not in out
 
 
+def test_no_kernel_spills_registers():
+    """The build records every kernel's resource use; a kernel that needs scratch memory (register
+    spills) runs far slower than designed, and the build refuses it."""
+    import json
+    path = os.path.join(os.path.dirname(_lib.__file__), "csrc", "build", "kernel_resources.json")
+    if not os.path.exists(path):
+        pytest.skip("library was not built in this tree")
+    res = json.load(open(path))
+    assert len(res) > 20
+    for name, r in res.items():
+        assert r.get("ScratchSize", 0) == 0, name
+        assert r.get("VGPRs", 0) + r.get("AGPRs", 0) <= 512, name
+
+
 def test_geometry_matches_reference_block_formats():
     L = _lib.lib()
     assert L.gq_abi_version() == 1

@@ -255,6 +255,59 @@ def test_bf16_prefill_parity(gpu, oracle, t, M, K, N):
     assert rel_err(got, want) < TOL_BF16, (t, M, K, N)
 
 
+@pytest.mark.parametrize("t", ALL_TYPES)
+@pytest.mark.parametrize("M,K,N", [
+    (512, 256, 130),    # smallest batch of the two-pass path; four K steps; ragged last weight tile
+    (513, 512, 128),    # one row into a third activation tile
+    (700, 768, 300),    # twelve K steps: the stage ring wraps four times
+    (1024, 1280, 64),   # twenty steps, half a weight tile
+])
+def test_large_batches_two_pass(gpu, oracle, t, M, K, N):
+    """Batches of 512 rows and more dequantise W once into a 16-bit image and run a plain MFMA
+    GEMM whose operands go from global memory straight into LDS."""
+    W = synth.weights(t, 95 + t, N, K)
+    bias = synth.normal(96 + t, 0, N).astype(np.float32) * 0.1
+    x = synth.activations(97 + t, M, K)
+    want = oracle.c_qdense(t, x, W, bias, 2)
+    assert rel_err(run_dense(gpu, t, x, W, bias, 2), want) < TOL_F32, (t, M, K, N, "f32")
+    xb = bf16_round(x)
+    want = oracle.c_qdense(t, xb, W, None, 0)
+    assert rel_err(run_dense(gpu, t, xb, W, None, 0, bf16=True), want) < TOL_BF16, (t, M, K, N, "bf16")
+
+
+@pytest.mark.parametrize("t", [Q4_0, Q8_0, IQ4_NL])
+@pytest.mark.parametrize("M,K,N", [
+    (17, 64, 40),       # one K step, less than one weight tile
+    (33, 128, 64),      # two K steps, exactly one 64-row weight tile
+    (64, 192, 130),     # three K steps, ragged last weight tile
+    (100, 1024, 300),   # sixteen K steps
+    (128, 4096, 257),   # a full tile of activation rows
+    (20, 256, 40000),   # enough weight tiles for the largest tile
+])
+def test_batches_of_17_to_128_rows(gpu, oracle, t, M, K, N):
+    """The batch sizes between the GEMV passes and a full tile of activation rows, where the small
+    tiles of the 16-bit GEMM are chosen; few K steps, ragged weight tiles, both activation types."""
+    W = synth.weights(t, 85 + t, N, K)
+    bias = synth.normal(86 + t, 0, N).astype(np.float32) * 0.1
+    x = synth.activations(87 + t, M, K)
+    want = oracle.c_qdense(t, x, W, bias, 3)
+    assert rel_err(run_dense(gpu, t, x, W, bias, 3), want) < TOL_F32, (t, M, K, N, "f32")
+    xb = bf16_round(x)
+    want = oracle.c_qdense(t, xb, W, None, 0)
+    assert rel_err(run_dense(gpu, t, xb, W, None, 0, bf16=True), want) < TOL_BF16, (t, M, K, N, "bf16")
+
+
+@pytest.mark.parametrize("K", [64, 128, 192, 96])
+def test_large_batches_few_k_steps(gpu, oracle, K):
+    """One, two and three K steps (shorter than the stage ring) and a K that is not a multiple of
+    64, which stays on the fused kernel."""
+    M, N = 600, 200
+    W = synth.weights(Q8_0, 98, N, K)
+    x = bf16_round(synth.activations(99, M, K))
+    want = oracle.c_qdense(Q8_0, x, W, None, 0)
+    assert rel_err(run_dense(gpu, Q8_0, x, W, None, 0, bf16=True), want) < TOL_BF16, K
+
+
 # ------------------------------------------------------------------------------ benchmark configurations, full size
 
 def test_config0_q8_0_gemv_4096(gpu, oracle):
