@@ -8,7 +8,7 @@
 // SIMD those vector-ALU instructions do not overlap with its MFMAs; from a few hundred rows on it
 // is cheaper to convert once and let the matrix cores run without vector work.  The GEMM moves
 // both operands from global memory straight into LDS (buffer loads with the LDS modifier: no
-// registers, no vector-ALU instructions) three K steps ahead through a ring of three stages.
+// registers, no vector-ALU instructions) two K steps ahead through a ring of three LDS stages.
 //
 // Tile: 256 x 128 per workgroup, 8 wavefronts x (64 x 64 = 2 x 2 v_mfma_f32_32x32x16), or 128 x 128
 // and 128 x 64 when the problem has too few large tiles to fill the chip; K in steps of 64.  LDS rows are 128 bytes, unpadded (the DMA writes 1 KB = 8 rows per wavefront
@@ -32,7 +32,6 @@ typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int DK = 64;
 constexpr int ROWB = 128;  // bytes per LDS row
-constexpr int NSTAGE = 3;
 
 template <bool BF16> struct Op16;
 template <> struct Op16<true> {
@@ -112,7 +111,10 @@ template <int TM, int TN> struct DmaTile {
     static constexpr int DM = 128 * TM, DN = 64 * TN;
     static constexpr int XI = 2 * TM, WI = TN;                 // DMAs per wavefront and step: X, W
     static constexpr int kStageBytes = (DM + DN) * ROWB;
-    static constexpr int kLdsBytes = NSTAGE * kStageBytes;
+    // Three stages: deeper rings for the small tiles (4 and 6 stages fit) measured slightly slower,
+    // because they leave room for one workgroup per CU instead of two.
+    static constexpr int NS = 3;
+    static constexpr int kLdsBytes = NS * kStageBytes;
 };
 
 template <bool BF16, int TM, int TN>
@@ -197,21 +199,21 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const 
 #pragma unroll
             for (int j = 0; j < TN; j++) acc[i][j] = Op::mfma(fa[set][i], fb[set][j], acc[i][j]);
     };
-    // Waits until this wavefront's DMAs of the next step have landed (those of the step after it may
-    // stay in flight) and its own LDS reads are done, then meets the other wavefronts.
+    // Waits until this wavefront's DMAs of the next step have landed (those of the NS - 2 steps after
+    // it may stay in flight) and its own LDS reads are done, then meets the other wavefronts.
     auto publish = [&]() __attribute__((always_inline)) {
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(G::XI + G::WI) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((G::NS - 2) * (G::XI + G::WI)) : "memory");
     };
 
-    issue(0, 0);
-    issue(1, 1);
+#pragma unroll
+    for (int p = 0; p < G::NS - 1; p++) issue(p, p);
     publish();
-    // Step kt computes out of stage kt % 3 while the DMAs of step kt + 2 fill stage (kt + 2) % 3,
-    // which every wavefront finished reading before the barrier that ended step kt - 1.  The MFMA
-    // groups are skewed by one against the barriers (group 3 of a step issues after the barrier,
-    // behind the first fragment reads of the next step).
+    // Step kt computes out of stage kt % NS while the DMAs of step kt + NS - 1 fill the stage that
+    // every wavefront finished reading before the barrier that ended step kt - 1.  The MFMA groups
+    // are skewed by one against the barriers (group 3 of a step issues after the barrier, behind
+    // the first fragment reads of the next step).
     auto step = [&](int kt, int stage, bool first) __attribute__((always_inline)) {
-        issue(kt + 2, (stage + 2) % NSTAGE);
+        issue(kt + G::NS - 1, (stage + G::NS - 1) % G::NS);
 #pragma unroll
         for (int kk = 0; kk < 4; kk++) {
             frags(stage, kk);
@@ -222,15 +224,15 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const 
     };
     step(0, 0, true);
     int kt = 1;
-    for (; kt + 2 < nk; kt += 3) {
-        step(kt, 1, false);
-        step(kt + 1, 2, false);
-        step(kt + 2, 0, false);
+    for (; kt + G::NS - 1 < nk; kt += G::NS) {  // stages 1, 2, .., NS - 1, 0: compile-time LDS offsets
+#pragma unroll
+        for (int p = 0; p < G::NS; p++) step(kt + p, (1 + p) % G::NS, false);
     }
-    if (kt < nk) { step(kt, 1, false); kt++; }
-    if (kt < nk) { step(kt, 2, false); kt++; }
+#pragma unroll
+    for (int p = 0; p < G::NS - 1; p++)
+        if (kt < nk) { step(kt, 1 + p, false); kt++; }
     mfma_group(1);  // group 3 of the last step
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the re-read DMAs of the last two steps
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the re-read DMAs of the last steps
 
     // ---- epilogue: acc[i][j][r] is Y[m, n] with n = lane % 32, m = 8*(r/4) + 4*(lane/32) + r%4
 #pragma unroll
