@@ -93,7 +93,6 @@ bool type_info(int type, TypeInfo &ti) {
 }
 
 constexpr int64_t kGemvMaxRows = 16;  // above this many activation rows the tiled MFMA kernels win
-constexpr int64_t kMmqPreferredRows = 96;  // Q4_K: the split-K small-batch kernel up to here, two passes beyond
 
 bool aligned_to(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
@@ -293,13 +292,18 @@ int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *d
             return launch_gemv_xs(type, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
         return launch_gemv(type, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
     }
-    // Q4_K has its own small-batch kernel; beyond about a hundred rows (one launch per 32) the two
-    // passes are faster (K = 4096, N = 14336: 60 against 63 us at 128 rows, 113 against 78 at 256).
+    // Small batches: GEMV passes cost about one third of the first pass per extra row; the split-K
+    // MFMA kernels cost 20 .. 37 us (Q8_0 / Q4_0, K = 4096, N = 4096 .. 14336) for up to 32 rows and as
+    // much again per further 32; the two passes 33 .. 62 us for anything up to 128 rows.  Measured
+    // crossovers: GEMV below 10 rows (Q4_K: below 5), split-K up to 64 rows (Q4_K: 96), then two passes.
     const bool tp = gemm_two_pass_supported(type, false, M, K, N, dX);
-    if (mmq_supported(type, M, K, N, dX, dBias, dY) && (M <= kMmqPreferredRows || !tp))
-        return launch_mmq(type, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
-    if (M <= kGemvMaxRows && gemv_ks_supported(type, K, N, dX))
+    const bool ks = M <= kGemvMaxRows && gemv_ks_supported(type, K, N, dX);
+    const int64_t mmq_from = type == GQ_Q4_K ? 5 : 10, mmq_to = type == GQ_Q4_K ? 96 : 64;
+    if (ks && M < mmq_from)
         return launch_gemv_ks(type, dX, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
+    if (mmq_supported(type, M, K, N, dX, dBias, dY) && (M <= mmq_to || !tp))
+        return launch_mmq(type, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
+    if (ks) return launch_gemv_ks(type, dX, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
     if (tp) return two_pass(type, false, dX, M, K, dW, N, dBias, act, dY, (hipStream_t)stream);
     return launch_gemm(type, false, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
 }

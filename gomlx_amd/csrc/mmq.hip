@@ -1,4 +1,5 @@
-// Small-batch (decode batch 5..~128) quantised Dense for Q4_K on the gfx950 matrix cores.
+// Small-batch (decode batch 5..~128) quantised Dense on the gfx950 matrix cores: Q4_K, and further
+// down Q8_0 / Q4_0.
 //
 // At batch 32 the contraction is 228 flop per weight byte: far beyond the vector ALUs, still
 // below the MFMA machine balance, so the kernel should run at the speed the packed weights
@@ -23,7 +24,6 @@
 // lane's four results belong to ONE weight row, the one whose header it has already loaded.
 #include "blocks.hpp"
 #include "common.hpp"
-
 
 namespace gq {
 
@@ -288,15 +288,210 @@ __global__ __launch_bounds__(256) void mmq_reduce_kernel(const float *__restrict
     *reinterpret_cast<float4 *>(Y + i) = make_float4(apply_act(act, s.x), apply_act(act, s.y), apply_act(act, s.z), apply_act(act, s.w));
 }
 
+
+// ---- small batches of the 32-value-block formats (Q8_0, Q4_0) --------------------------------------
+//
+// Same plan as the Q4_K kernel above, simpler arithmetic: K is split in slices of S = 512, 1024 or
+// 2048 values (the smallest count of slices that still gives the chip a few hundred workgroups); a
+// workgroup keeps the slice of x for 32 batch columns in LDS as fp16 octets in natural order
+// ([octet][column][8 values], copied global -> LDS from an image a pre-pass wrote) and streams
+// 128 rows of W past it: 8 wavefronts = 4 row tiles of 32 x 2 interleaved block sequences.  Lane
+// (col = lane % 32, kg = lane / 32) owns W row `col` of its tile and half the codes of every block:
+//   Q8_0: bytes 16 kg .. 16 kg + 15 -> octets 4 b + 2 kg + j, j = 0, 1;
+//   Q4_0: bytes 8 kg .. 8 kg + 7: low nibbles -> octet 4 b + kg, high nibbles -> octet 4 b + 2 + kg.
+// Codes become exact fp16 integers (magic number 1024 + code, one packed add), two MFMAs contract
+// a block against the activations, and the block's partial tile is scaled by d in fp32:
+// x -> fp16 is the only rounding that is not fp32.  All of a wavefront's blocks of a 512-value
+// stretch are requested before the first is used.
+template <int T> struct B32;
+template <> struct B32<kQ8_0> {
+    static constexpr int kBlockBytes = 34;
+    struct Raw { uint32_t d; u128_a2 q; };
+    static __device__ __forceinline__ void load(Raw &r, const uint8_t *blk, int kg) {
+        r.d = load_u16(blk);
+        r.q = *reinterpret_cast<const u128_a2 *>(blk + 2 + 16 * kg);
+    }
+    static __device__ __forceinline__ int octet(int b, int kg, int j) { return 4 * b + 2 * kg + j; }
+    // fragment j: values 8 j .. 8 j + 7 of the lane's sixteen, as fp16 pairs (0,2) (1,3) (4,6) (5,7)
+    static __device__ __forceinline__ h8 frag(const Raw &r, int j, uint32_t magic) {
+        const uint32_t a = r.q.v[2 * j] ^ 0x80808080u, b = r.q.v[2 * j + 1] ^ 0x80808080u;  // code + 128, unsigned
+        const h2 off = as_h2(0xE480E480u);  // (-1152, -1152) = -(1024 + 128)
+        uint4 o;
+        o.x = __builtin_bit_cast(uint32_t, as_h2(__builtin_amdgcn_perm(magic, a, 0x07020700u)) + off);  // bytes (a0, 0x64, a2, 0x64)
+        o.y = __builtin_bit_cast(uint32_t, as_h2(__builtin_amdgcn_perm(magic, a, 0x07030701u)) + off);
+        o.z = __builtin_bit_cast(uint32_t, as_h2(__builtin_amdgcn_perm(magic, b, 0x07020700u)) + off);
+        o.w = __builtin_bit_cast(uint32_t, as_h2(__builtin_amdgcn_perm(magic, b, 0x07030701u)) + off);
+        return __builtin_bit_cast(h8, o);
+    }
+};
+template <> struct B32<kQ4_0> {
+    static constexpr int kBlockBytes = 18;
+    struct __attribute__((packed, aligned(2))) U2 { uint32_t v[2]; };
+    struct Raw { uint32_t d; U2 q; };
+    static __device__ __forceinline__ void load(Raw &r, const uint8_t *blk, int kg) {
+        r.d = load_u16(blk);
+        r.q = *reinterpret_cast<const U2 *>(blk + 2 + 8 * kg);
+    }
+    static __device__ __forceinline__ int octet(int b, int kg, int j) { return 4 * b + 2 * j + kg; }
+    // fragment 0: low nibbles, fragment 1: high nibbles of the lane's eight bytes, minus 8
+    static __device__ __forceinline__ h8 frag(const Raw &r, int j, uint32_t magic) {
+        const uint32_t a = r.q.v[0] >> (4 * j), b = r.q.v[1] >> (4 * j);
+        const h2 off = as_h2(0xE408E408u);  // (-1032, -1032) = -(1024 + 8)
+        uint4 o;
+        o.x = __builtin_bit_cast(uint32_t, magic_pair(a, 0x000F000Fu, magic) + off);       // nibbles of bytes (0, 2)
+        o.y = __builtin_bit_cast(uint32_t, magic_pair(a >> 8, 0x000F000Fu, magic) + off);  // (1, 3)
+        o.z = __builtin_bit_cast(uint32_t, magic_pair(b, 0x000F000Fu, magic) + off);
+        o.w = __builtin_bit_cast(uint32_t, magic_pair(b >> 8, 0x000F000Fu, magic) + off);
+        return __builtin_bit_cast(h8, o);
+    }
+};
+
+constexpr int kB32Stretch = 8;    // blocks a wavefront requests at once (a 512-value stretch, every other block)
+
+// Image of x for the main kernel: [column tile][slice][octet of the slice][32 columns][8 fp16 in the
+// order (0,2,1,3,4,6,5,7)]; columns beyond M and values beyond K are zero.
+__global__ __launch_bounds__(256) void mmq_b32_xprep_kernel(const float *__restrict__ X, uint8_t *__restrict__ ximg, int M, int K, int S,
+                                                            int nslices) {
+    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;  // (column tile, slice, octet, column)
+    const int m = (int)(g & 31);
+    const int64_t o = g >> 5;  // octet index over (column tile, slice, octet of slice)
+    const int opers = S / 8;
+    const int64_t ts = o / opers;
+    const int oct = (int)(o % opers), slice = (int)(ts % nslices), mt = (int)(ts / nslices);
+    if (mt * kMT >= M) return;
+    const int k = slice * S + oct * 8, row = mt * kMT + m;
+    float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+    if (row < M && k < K) {  // K is a multiple of 32: an octet is inside or outside as a whole
+        const float4 *p = reinterpret_cast<const float4 *>(X + (int64_t)row * K + k);
+        a = p[0];
+        b = p[1];
+    }
+    reinterpret_cast<uint4 *>(ximg)[g] = make_uint4(pack_h2(a.x, a.z), pack_h2(a.y, a.w), pack_h2(b.x, b.z), pack_h2(b.y, b.w));
+}
+
+// partial[slice][m][n] = sum over the slice's k of x[m][k] * w[n][k];  grid (row ranges, slices, column tiles)
+// RT row tiles of 32 W rows per workgroup, two wavefronts each.
+template <int T, int RT>
+__global__ __launch_bounds__(RT * 128) void mmq_b32_kernel(const uint8_t *__restrict__ ximg, const uint8_t *__restrict__ W,
+                                                      float *__restrict__ partial, int M, int K, int N, int64_t row_bytes, int S) {
+    typedef B32<T> F;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kg = lane >> 5, col = lane & 31;
+    const int rt = wave % RT, par = wave / RT;
+    const int slice = blockIdx.y, nslices = gridDim.y, mt = blockIdx.z;
+    const int img_bytes = S * 64;
+    const int kblocks = K >> 5, b0 = slice * (S >> 5);       // blocks of a row; first block of the slice
+    const int n = (blockIdx.x * RT + rt) * 32 + col;          // this lane's weight row
+    const uint8_t *wrow = W + (int64_t)min(n, N - 1) * row_bytes;
+
+    // the slice's activation image goes straight from global memory into LDS (no registers)
+    {
+        const uint8_t *img = ximg + ((size_t)mt * nslices + slice) * img_bytes;
+        for (int i = wave; i < img_bytes / 1024; i += 2 * RT)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(img + i * 1024 + lane * 16),
+                                             (__attribute__((address_space(3))) void *)(lds + i * 1024), 16, 0, 0);
+    }
+    // Wavefront `par` takes blocks par, par + 2, ...; blocks beyond K re-read the row's last block
+    // (their activations are zero in the image).
+    auto blk_ptr = [&](int i) { return wrow + (int64_t)min(b0 + 2 * i + par, kblocks - 1) * F::kBlockBytes; };
+    typename F::Raw buf[kB32Stretch];
+#pragma unroll
+    for (int j = 0; j < kB32Stretch; j++) F::load(buf[j], blk_ptr(j), kg);
+    __syncthreads();
+
+    f16v acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+    uint32_t magic;
+    asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));
+    const int nb = S >> 6;  // blocks per wavefront: 8, 16 or 32
+    for (int g = 0; g < nb; g += kB32Stretch) {
+        const bool more = g + kB32Stretch < nb;
+#pragma unroll
+        for (int j = 0; j < kB32Stretch; j++) {
+            const int b = 2 * (g + j) + par;  // block within the slice
+            const h8 x0 = *reinterpret_cast<const h8 *>(lds + (F::octet(b, kg, 0) * kMT + col) * 16);
+            const h8 x1 = *reinterpret_cast<const h8 *>(lds + (F::octet(b, kg, 1) * kMT + col) * 16);
+            const float d = half_bits_to_float(buf[j].d);
+            f16v p;
+#pragma unroll
+            for (int r = 0; r < 16; r++) p[r] = 0.f;
+            p = __builtin_amdgcn_mfma_f32_32x32x16_f16(x0, F::frag(buf[j], 0, magic), p, 0, 0, 0);
+            p = __builtin_amdgcn_mfma_f32_32x32x16_f16(x1, F::frag(buf[j], 1, magic), p, 0, 0, 0);
+            if (more) F::load(buf[j], blk_ptr(g + kB32Stretch + j), kg);
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[r] = fmaf(d, p[r], acc[r]);
+        }
+    }
+
+    // the second wavefront of a row tile hands its 32 x 32 partial tile to the first through LDS
+    __syncthreads();
+    float *xch = reinterpret_cast<float *>(lds) + rt * (16 * 64);
+    if (par > 0) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) xch[r * 64 + lane] = acc[r];
+    }
+    __syncthreads();
+    if (par == 0 && n < N) {
+        // lane holds y[m = 8 (r / 4) + 4 kg + r % 4][n] for its K-slice
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int m = mt * kMT + 8 * (r >> 2) + 4 * kg + (r & 3);
+            if (m < M) partial[((int64_t)slice * M + m) * N + n] = acc[r] + xch[r * 64 + lane];
+        }
+    }
+}
+
+template <int T, int RT>
+int launch_mmq_b32(const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y, hipStream_t s) {
+    const int cus = device_cu_count();
+    const int mtiles = (int)((M + kMT - 1) / kMT);
+    const int64_t rowwgs = (N + 32 * RT - 1) / (32 * RT);
+    int S = 512;
+    for (int cand : {2048, 1024})
+        if (rowwgs * ((K + cand - 1) / cand) * mtiles >= (int64_t)cus * 3 / 2) { S = cand; break; }
+    const int nslices = (int)((K + S - 1) / S);
+    const size_t lds_bytes = (size_t)S * 64;  // also holds the RT x 4 KB tiles handed over at the end
+    static const bool lds_ok = [] {
+        return hipFuncSetAttribute(reinterpret_cast<const void *>(mmq_b32_kernel<T, RT>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   2048 * 64) == hipSuccess;
+    }();
+    if (!lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", 2048 * 64);
+    // workspace: [activation images: mtiles x nslices x S x 64 bytes][partial sums: nslices x M x N fp32]
+    const size_t img_bytes = (size_t)mtiles * nslices * S * 64;
+    const size_t part_bytes = (size_t)nslices * M * N * sizeof(float);
+    void *ws = nullptr;
+    if (int rc = stream_workspace(s, img_bytes + part_bytes, &ws)) return rc;
+    uint8_t *ximg = reinterpret_cast<uint8_t *>(ws);
+    float *partial = reinterpret_cast<float *>(ximg + img_bytes);
+    const int64_t row_bytes = (K / 32) * B32<T>::kBlockBytes;
+    const int64_t items = (int64_t)mtiles * nslices * (S / 8) * 32;
+    if (int rc = launch(mmq_b32_xprep_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, x, ximg, (int)M, (int)K, S, nslices))
+        return rc;
+    const dim3 grid((unsigned)rowwgs, (unsigned)nslices, (unsigned)mtiles);
+    if (int rc = launch(mmq_b32_kernel<T, RT>, grid, dim3(RT * 128), lds_bytes, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N, row_bytes, S))
+        return rc;
+    const int64_t MN = M * N;
+    return launch(mmq_reduce_kernel, dim3((unsigned)((MN / 4 + 255) / 256)), dim3(256), 0, s, (const float *)partial, nslices, MN, (int)N,
+                  bias, act, y);
+}
+
 }  // namespace
 
 bool mmq_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, const void *bias, const void *y) {
-    return type == kQ4_K && M >= 2 && M <= 256 && K % 256 == 0 && N % 4 == 0 && N <= (int64_t)INT32_MAX / 2 && K <= INT32_MAX &&
-           ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(bias) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
+    const bool shape_ok = M >= 2 && M <= 256 && N % 4 == 0 && N <= (int64_t)INT32_MAX / 2 && K <= INT32_MAX / 2 &&
+                          ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(bias) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
+    if (type == kQ4_K) return shape_ok && K % 256 == 0;
+    if (type == kQ8_0 || type == kQ4_0) return shape_ok && K % 32 == 0;
+    return false;
 }
 
 int launch_mmq(int type, const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act,
                float *y, hipStream_t s) {
+    // (four row tiles per workgroup measured a little faster than two)
+    if (type == kQ8_0) return launch_mmq_b32<kQ8_0, 4>(x, M, K, W, N, bias, act, y, s);
+    if (type == kQ4_0) return launch_mmq_b32<kQ4_0, 4>(x, M, K, W, N, bias, act, y, s);
     if (type != kQ4_K) return fail(GQ_ERR_NOT_IMPLEMENTED, "mmq: ggml type %d is not implemented", type);
     static const bool lds_ok = [] {
         return hipFuncSetAttribute(reinterpret_cast<const void *>(mmq_q4k_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,

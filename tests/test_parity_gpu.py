@@ -158,6 +158,27 @@ def test_small_batches_f32(gpu, oracle, t, M):
     assert rel_err(got, oracle.c_qdense(t, x, W, None, 0)) < TOL_F32, (t, M)
 
 
+@pytest.mark.parametrize("t", [Q4_0, Q8_0])
+@pytest.mark.parametrize("M,K,N", [
+    (10, 32, 4),         # one block, one row tile mostly empty
+    (16, 96, 132),       # K below one slice, weight rows not a multiple of 32
+    (33, 544, 256),      # two column tiles; K = one slice + one block
+    (64, 1056, 300),     # K not a multiple of the slice length
+    (24, 8192, 20000),   # enough work for the longest slices
+    (40, 4096, 4096),
+])
+def test_split_k_small_batches_q8_q4(gpu, oracle, t, M, K, N):
+    """10 .. 64 rows of Q8_0 / Q4_0 (fp32 activations, N a multiple of 4): the split-K MFMA kernel
+    with exact integer weight operands; x -> fp16 is its only rounding."""
+    W = synth.weights(t, 70 + t, N, K)
+    x = synth.activations(71 + t, M, K)
+    bias = synth.normal(72 + t, 0, N).astype(np.float32) * 0.1
+    for act in (0, 1):
+        got = run_dense(gpu, t, x, W, bias, act)
+        want = oracle.c_qdense(t, x, W, bias, act)
+        assert rel_err(got, want) < TOL_F32, (t, M, K, N, act)
+
+
 @pytest.mark.parametrize("t", ALL_TYPES)
 def test_gemv_long_k_is_chunked(gpu, oracle, t):
     """K above the 16384 values one LDS pass holds."""
