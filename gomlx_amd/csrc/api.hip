@@ -293,12 +293,12 @@ int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *d
         return launch_gemv(type, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
     }
     // Small batches: GEMV passes cost about one third of the first pass per extra row; the split-K
-    // MFMA kernels cost 20 .. 37 us (Q8_0 / Q4_0, K = 4096, N = 4096 .. 14336) for up to 32 rows and as
-    // much again per further 32; the two passes 33 .. 62 us for anything up to 128 rows.  Measured
-    // crossovers: GEMV below 10 rows (Q4_K: below 5), split-K up to 64 rows (Q4_K: 96), then two passes.
+    // MFMA kernels cost 19 .. 26 us (Q8_0 / Q4_0, K = 4096, N = 4096 .. 14336) for up to 32 rows and
+    // 5 .. 18 us per further 32; the two passes 33 .. 62 us for anything up to 128 rows.  Measured
+    // crossovers: GEMV below 8 rows (Q4_K: below 5), split-K up to 96 rows, then two passes.
     const bool tp = gemm_two_pass_supported(type, false, M, K, N, dX);
     const bool ks = M <= kGemvMaxRows && gemv_ks_supported(type, K, N, dX);
-    const int64_t mmq_from = type == GQ_Q4_K ? 5 : 10, mmq_to = type == GQ_Q4_K ? 96 : 64;
+    const int64_t mmq_from = type == GQ_Q4_K ? 5 : 8, mmq_to = 96;
     if (ks && M < mmq_from)
         return launch_gemv_ks(type, dX, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
     if (mmq_supported(type, M, K, N, dX, dBias, dY) && (M <= mmq_to || !tp))

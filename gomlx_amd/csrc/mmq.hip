@@ -291,30 +291,35 @@ __global__ __launch_bounds__(256) void mmq_reduce_kernel(const float *__restrict
 
 // ---- small batches of the 32-value-block formats (Q8_0, Q4_0) --------------------------------------
 //
-// Same plan as the Q4_K kernel above, simpler arithmetic: K is split in slices of S = 512, 1024 or
-// 2048 values (the smallest count of slices that still gives the chip a few hundred workgroups); a
+// Same plan as the Q4_K kernel above, simpler arithmetic: K is split in slices of S = 512 or 1024
+// values (the smaller count of slices that still gives the chip a few hundred workgroups); a
 // workgroup keeps the slice of x for 32 batch columns in LDS as fp16 octets in natural order
 // ([octet][column][8 values], copied global -> LDS from an image a pre-pass wrote) and streams
-// 128 rows of W past it: 8 wavefronts = 4 row tiles of 32 x 2 interleaved block sequences.  Lane
-// (col = lane % 32, kg = lane / 32) owns W row `col` of its tile and half the codes of every block:
-//   Q8_0: bytes 16 kg .. 16 kg + 15 -> octets 4 b + 2 kg + j, j = 0, 1;
+// 128 rows of W past it: 8 wavefronts = 4 row tiles of 32 x 2 interleaved sequences of 256-value
+// stretches (8 blocks).
+//
+// Loading: a load instruction whose 64 lanes touch 64 different cache lines (one W row per lane)
+// occupies the texture addresser for ~2.4 cycles per lane, which alone holds a kernel at
+// ~1.5 TB/s.  So a wavefront reads a stretch of its 32 rows as 16-byte chunks in row-major chunk
+// order (consecutive lanes = consecutive chunks of one row: 17 per row for Q8_0, 9 for Q4_0),
+// parks them in a private piece of LDS and only then lets lane (col = lane % 32, kg = lane / 32)
+// pick out the codes of W row `col`:
+//   Q8_0: bytes 16 kg .. 16 kg + 15 of block b -> octets 4 b + 2 kg + j, j = 0, 1;
 //   Q4_0: bytes 8 kg .. 8 kg + 7: low nibbles -> octet 4 b + kg, high nibbles -> octet 4 b + 2 + kg.
+// Blocks start 2 bytes off a dword boundary every other block; the LDS reads are dword windows
+// plus a funnel shift (which block is odd is known at compile time).
 // Codes become exact fp16 integers (magic number 1024 + code, one packed add), two MFMAs contract
 // a block against the activations, and the block's partial tile is scaled by d in fp32:
-// x -> fp16 is the only rounding that is not fp32.  All of a wavefront's blocks of a 512-value
-// stretch are requested before the first is used.
+// x -> fp16 is the only rounding that is not fp32.
 template <int T> struct B32;
 template <> struct B32<kQ8_0> {
-    static constexpr int kBlockBytes = 34;
-    struct Raw { uint32_t d; u128_a2 q; };
-    static __device__ __forceinline__ void load(Raw &r, const uint8_t *blk, int kg) {
-        r.d = load_u16(blk);
-        r.q = *reinterpret_cast<const u128_a2 *>(blk + 2 + 16 * kg);
-    }
+    static constexpr int kBlockBytes = 34, kWin = 5;  // dwords that cover a lane's 16 codes from the dword at or below them
+    static __device__ __forceinline__ int code_byte(int kg) { return 2 + 16 * kg; }
     static __device__ __forceinline__ int octet(int b, int kg, int j) { return 4 * b + 2 * kg + j; }
-    // fragment j: values 8 j .. 8 j + 7 of the lane's sixteen, as fp16 pairs (0,2) (1,3) (4,6) (5,7)
-    static __device__ __forceinline__ h8 frag(const Raw &r, int j, uint32_t magic) {
-        const uint32_t a = r.q.v[2 * j] ^ 0x80808080u, b = r.q.v[2 * j + 1] ^ 0x80808080u;  // code + 128, unsigned
+    // fragment j: values 8 j .. 8 j + 7 of the lane's sixteen, as fp16 pairs (0,2) (1,3) (4,6) (5,7);
+    // c[0..3] are the four code dwords
+    static __device__ __forceinline__ h8 frag(const uint32_t *c, int j, uint32_t magic) {
+        const uint32_t a = c[2 * j] ^ 0x80808080u, b = c[2 * j + 1] ^ 0x80808080u;  // code + 128, unsigned
         const h2 off = as_h2(0xE480E480u);  // (-1152, -1152) = -(1024 + 128)
         uint4 o;
         o.x = __builtin_bit_cast(uint32_t, as_h2(__builtin_amdgcn_perm(magic, a, 0x07020700u)) + off);  // bytes (a0, 0x64, a2, 0x64)
@@ -325,17 +330,12 @@ template <> struct B32<kQ8_0> {
     }
 };
 template <> struct B32<kQ4_0> {
-    static constexpr int kBlockBytes = 18;
-    struct __attribute__((packed, aligned(2))) U2 { uint32_t v[2]; };
-    struct Raw { uint32_t d; U2 q; };
-    static __device__ __forceinline__ void load(Raw &r, const uint8_t *blk, int kg) {
-        r.d = load_u16(blk);
-        r.q = *reinterpret_cast<const U2 *>(blk + 2 + 8 * kg);
-    }
+    static constexpr int kBlockBytes = 18, kWin = 3;
+    static __device__ __forceinline__ int code_byte(int kg) { return 2 + 8 * kg; }
     static __device__ __forceinline__ int octet(int b, int kg, int j) { return 4 * b + 2 * j + kg; }
-    // fragment 0: low nibbles, fragment 1: high nibbles of the lane's eight bytes, minus 8
-    static __device__ __forceinline__ h8 frag(const Raw &r, int j, uint32_t magic) {
-        const uint32_t a = r.q.v[0] >> (4 * j), b = r.q.v[1] >> (4 * j);
+    // fragment 0: low nibbles, fragment 1: high nibbles of the lane's eight bytes (c[0..1]), minus 8
+    static __device__ __forceinline__ h8 frag(const uint32_t *c, int j, uint32_t magic) {
+        const uint32_t a = c[0] >> (4 * j), b = c[1] >> (4 * j);
         const h2 off = as_h2(0xE408E408u);  // (-1032, -1032) = -(1024 + 8)
         uint4 o;
         o.x = __builtin_bit_cast(uint32_t, magic_pair(a, 0x000F000Fu, magic) + off);       // nibbles of bytes (0, 2)
@@ -346,7 +346,15 @@ template <> struct B32<kQ4_0> {
     }
 };
 
-constexpr int kB32Stretch = 8;    // blocks a wavefront requests at once (a 512-value stretch, every other block)
+constexpr int kB32Stretch = 8;    // blocks per stretch (256 values)
+
+template <int T> struct B32Geom {
+    static constexpr int kStretchBytes = kB32Stretch * B32<T>::kBlockBytes;  // 272 / 144 per row
+    static constexpr int kCPR = kStretchBytes / 16;                          // 16-byte chunks per row: 17 / 9
+    static constexpr int kChunks = 32 * kCPR;                                // per wavefront and stretch
+    static constexpr int kLoads = (kChunks + 63) / 64;                       // 9 / 5 load instructions
+    static constexpr int kWaveLds = 32 * kStretchBytes + 16;                 // + slack: a window may end past the last row
+};
 
 // Image of x for the main kernel: [column tile][slice][octet of the slice][32 columns][8 fp16 in the
 // order (0,2,1,3,4,6,5,7)]; columns beyond M and values beyond K are zero.
@@ -370,20 +378,22 @@ __global__ __launch_bounds__(256) void mmq_b32_xprep_kernel(const float *__restr
 }
 
 // partial[slice][m][n] = sum over the slice's k of x[m][k] * w[n][k];  grid (row ranges, slices, column tiles)
-// RT row tiles of 32 W rows per workgroup, two wavefronts each.
+// RT row tiles of 32 W rows per workgroup, two wavefronts each.  K % 256 == 0.
+// LDS: [activation image: S * 64 bytes][per wavefront: one stretch of 32 rows]
 template <int T, int RT>
 __global__ __launch_bounds__(RT * 128) void mmq_b32_kernel(const uint8_t *__restrict__ ximg, const uint8_t *__restrict__ W,
-                                                      float *__restrict__ partial, int M, int K, int N, int64_t row_bytes, int S) {
+                                                           float *__restrict__ partial, int M, int K, int N, int64_t row_bytes, int S) {
     typedef B32<T> F;
+    typedef B32Geom<T> G;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int kg = lane >> 5, col = lane & 31;
     const int rt = wave % RT, par = wave / RT;
     const int slice = blockIdx.y, nslices = gridDim.y, mt = blockIdx.z;
     const int img_bytes = S * 64;
-    const int kblocks = K >> 5, b0 = slice * (S >> 5);       // blocks of a row; first block of the slice
-    const int n = (blockIdx.x * RT + rt) * 32 + col;          // this lane's weight row
-    const uint8_t *wrow = W + (int64_t)min(n, N - 1) * row_bytes;
+    const int kstretches = K >> 8, t0 = slice * (S >> 8);      // stretches of a row; first stretch of the slice
+    const int n0 = (blockIdx.x * RT + rt) * 32;                // first W row of this wavefront's tile
+    uint8_t *park = lds + img_bytes + wave * G::kWaveLds;      // this wavefront's stretch
 
     // the slice's activation image goes straight from global memory into LDS (no registers)
     {
@@ -392,12 +402,25 @@ __global__ __launch_bounds__(RT * 128) void mmq_b32_kernel(const uint8_t *__rest
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(img + i * 1024 + lane * 16),
                                              (__attribute__((address_space(3))) void *)(lds + i * 1024), 16, 0, 0);
     }
-    // Wavefront `par` takes blocks par, par + 2, ...; blocks beyond K re-read the row's last block
-    // (their activations are zero in the image).
-    auto blk_ptr = [&](int i) { return wrow + (int64_t)min(b0 + 2 * i + par, kblocks - 1) * F::kBlockBytes; };
-    typename F::Raw buf[kB32Stretch];
+    // Wavefront `par` takes stretches par, par + 2, ... of the slice; stretches beyond K re-read the
+    // row's last one (their activations are zero in the image).  Chunk c = lane + 64 i of a stretch is
+    // chunk c % kCPR of row c / kCPR.
+    uint32_t coff[G::kLoads];  // byte offset of this lane's chunks from the stretch's start in row n0
 #pragma unroll
-    for (int j = 0; j < kB32Stretch; j++) F::load(buf[j], blk_ptr(j), kg);
+    for (int i = 0; i < G::kLoads; i++) {
+        const int c = min(lane + 64 * i, G::kChunks - 1);
+        coff[i] = (uint32_t)min(c / G::kCPR, max(N - 1 - n0, 0)) * (uint32_t)row_bytes + (uint32_t)(c % G::kCPR) * 16u;
+    }
+    const uint8_t *wtile = W + (int64_t)min(n0, N - 1) * row_bytes;
+    typedef uint32_t Chunk __attribute__((ext_vector_type(4)));
+    typedef Chunk ChunkA4 __attribute__((aligned(4)));  // rows are only 4-byte aligned in general
+    Chunk buf[G::kLoads];
+    auto fetch = [&](int i) __attribute__((always_inline)) {  // i-th stretch of this wavefront
+        const uint8_t *base = wtile + (int64_t)min(t0 + 2 * i + par, kstretches - 1) * G::kStretchBytes;
+#pragma unroll
+        for (int l = 0; l < G::kLoads; l++) buf[l] = *reinterpret_cast<const ChunkA4 *>(base + coff[l]);
+    };
+    fetch(0);
     __syncthreads();
 
     f16v acc;
@@ -405,24 +428,44 @@ __global__ __launch_bounds__(RT * 128) void mmq_b32_kernel(const uint8_t *__rest
     for (int r = 0; r < 16; r++) acc[r] = 0.f;
     uint32_t magic;
     asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));
-    const int nb = S >> 6;  // blocks per wavefront: 8, 16 or 32
-    for (int g = 0; g < nb; g += kB32Stretch) {
-        const bool more = g + kB32Stretch < nb;
+    const int ns = S >> 9;  // stretches per wavefront: 1 or 2
+    const uint8_t *myrow = park + col * G::kStretchBytes;
+    for (int g = 0; g < ns; g++) {
+        // park the stretch (LDS operations of one wavefront execute in order; no other wavefront reads it)
+#pragma unroll
+        for (int l = 0; l < G::kLoads; l++)
+            if (lane + 64 * l < G::kChunks) *reinterpret_cast<Chunk *>(park + (lane + 64 * l) * 16) = buf[l];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        if (g + 1 < ns) fetch(g + 1);
+        const int sb = 8 * (2 * g + par);  // first block of the stretch within the slice
 #pragma unroll
         for (int j = 0; j < kB32Stretch; j++) {
-            const int b = 2 * (g + j) + par;  // block within the slice
+            const int b = sb + j;
             const h8 x0 = *reinterpret_cast<const h8 *>(lds + (F::octet(b, kg, 0) * kMT + col) * 16);
             const h8 x1 = *reinterpret_cast<const h8 *>(lds + (F::octet(b, kg, 1) * kMT + col) * 16);
-            const float d = half_bits_to_float(buf[j].d);
+            // the lane's codes: a dword window from the dword at or below them, funnel-shifted when
+            // the block starts 2 bytes off (every even block: 34 j and 18 j are 2 mod 4 for odd j,
+            // and the codes start 2 bytes into the block)
+            const int at = j * F::kBlockBytes + F::code_byte(kg);
+            const uint32_t *wp = reinterpret_cast<const uint32_t *>(myrow + (at & ~3));
+            uint32_t w[F::kWin], c[F::kWin - 1];
+#pragma unroll
+            for (int q = 0; q < F::kWin; q++) w[q] = wp[q];
+#pragma unroll
+            for (int q = 0; q < F::kWin - 1; q++) c[q] = (j & 1) ? w[q] : __builtin_amdgcn_alignbit(w[q + 1], w[q], 16);
+            const float d = half_bits_to_float(*reinterpret_cast<const uint16_t *>(myrow + j * F::kBlockBytes));
             f16v p;
 #pragma unroll
             for (int r = 0; r < 16; r++) p[r] = 0.f;
-            p = __builtin_amdgcn_mfma_f32_32x32x16_f16(x0, F::frag(buf[j], 0, magic), p, 0, 0, 0);
-            p = __builtin_amdgcn_mfma_f32_32x32x16_f16(x1, F::frag(buf[j], 1, magic), p, 0, 0, 0);
-            if (more) F::load(buf[j], blk_ptr(g + kB32Stretch + j), kg);
+            p = __builtin_amdgcn_mfma_f32_32x32x16_f16(x0, F::frag(c, 0, magic), p, 0, 0, 0);
+            p = __builtin_amdgcn_mfma_f32_32x32x16_f16(x1, F::frag(c, 1, magic), p, 0, 0, 0);
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[r] = fmaf(d, p[r], acc[r]);
         }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // the reads above are done before the next stretch is parked
+        __builtin_amdgcn_wave_barrier();
     }
 
     // the second wavefront of a row tile hands its 32 x 32 partial tile to the first through LDS
@@ -433,6 +476,7 @@ __global__ __launch_bounds__(RT * 128) void mmq_b32_kernel(const uint8_t *__rest
         for (int r = 0; r < 16; r++) xch[r * 64 + lane] = acc[r];
     }
     __syncthreads();
+    const int n = n0 + col;
     if (par == 0 && n < N) {
         // lane holds y[m = 8 (r / 4) + 4 kg + r % 4][n] for its K-slice
 #pragma unroll
@@ -448,16 +492,16 @@ int launch_mmq_b32(const float *x, int64_t M, int64_t K, const uint8_t *W, int64
     const int cus = device_cu_count();
     const int mtiles = (int)((M + kMT - 1) / kMT);
     const int64_t rowwgs = (N + 32 * RT - 1) / (32 * RT);
-    int S = 512;
-    for (int cand : {2048, 1024})
-        if (rowwgs * ((K + cand - 1) / cand) * mtiles >= (int64_t)cus * 3 / 2) { S = cand; break; }
+    // slices of 1024 when that still leaves every CU a workgroup and a half (LDS holds a 1024-value image
+    // next to the parked stretches, not a 2048-value one)
+    const int S = rowwgs * ((K + 1023) / 1024) * mtiles >= (int64_t)cus * 3 / 2 ? 1024 : 512;
     const int nslices = (int)((K + S - 1) / S);
-    const size_t lds_bytes = (size_t)S * 64;  // also holds the RT x 4 KB tiles handed over at the end
+    const size_t lds_bytes = (size_t)S * 64 + (size_t)2 * RT * B32Geom<T>::kWaveLds;  // image (later the handed-over tiles) + parked stretches
     static const bool lds_ok = [] {
         return hipFuncSetAttribute(reinterpret_cast<const void *>(mmq_b32_kernel<T, RT>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   2048 * 64) == hipSuccess;
+                                   1024 * 64 + 2 * RT * B32Geom<T>::kWaveLds) == hipSuccess;
     }();
-    if (!lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", 2048 * 64);
+    if (!lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", 1024 * 64 + 2 * RT * B32Geom<T>::kWaveLds);
     // workspace: [activation images: mtiles x nslices x S x 64 bytes][partial sums: nslices x M x N fp32]
     const size_t img_bytes = (size_t)mtiles * nslices * S * 64;
     const size_t part_bytes = (size_t)nslices * M * N * sizeof(float);
@@ -483,7 +527,7 @@ bool mmq_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, con
     const bool shape_ok = M >= 2 && M <= 256 && N % 4 == 0 && N <= (int64_t)INT32_MAX / 2 && K <= INT32_MAX / 2 &&
                           ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(bias) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
     if (type == kQ4_K) return shape_ok && K % 256 == 0;
-    if (type == kQ8_0 || type == kQ4_0) return shape_ok && K % 32 == 0;
+    if (type == kQ8_0 || type == kQ4_0) return shape_ok && K % 256 == 0;  // whole stretches of 8 blocks
     return false;
 }
 

@@ -160,16 +160,19 @@ def test_small_batches_f32(gpu, oracle, t, M):
 
 @pytest.mark.parametrize("t", [Q4_0, Q8_0])
 @pytest.mark.parametrize("M,K,N", [
-    (10, 32, 4),         # one block, one row tile mostly empty
-    (16, 96, 132),       # K below one slice, weight rows not a multiple of 32
-    (33, 544, 256),      # two column tiles; K = one slice + one block
-    (64, 1056, 300),     # K not a multiple of the slice length
+    (10, 256, 4),        # one stretch, three of four row tiles empty
+    (16, 768, 132),      # K = one slice and a half, weight rows not a multiple of 32
+    (33, 1280, 256),     # two column tiles
+    (64, 2304, 300),     # K not a multiple of the slice length
+    (12, 96, 64),        # K not a multiple of 256: not this kernel's
     (24, 8192, 20000),   # enough work for the longest slices
     (40, 4096, 4096),
+    (96, 512, 512),      # three column tiles
+    (8, 1024, 36),
 ])
 def test_split_k_small_batches_q8_q4(gpu, oracle, t, M, K, N):
-    """10 .. 64 rows of Q8_0 / Q4_0 (fp32 activations, N a multiple of 4): the split-K MFMA kernel
-    with exact integer weight operands; x -> fp16 is its only rounding."""
+    """8 .. 96 rows of Q8_0 / Q4_0 (fp32 activations, N a multiple of 4, K of 256): the split-K MFMA
+    kernel with exact integer weight operands; x -> fp16 is its only rounding."""
     W = synth.weights(t, 70 + t, N, K)
     x = synth.activations(71 + t, M, K)
     bias = synth.normal(72 + t, 0, N).astype(np.float32) * 0.1
