@@ -302,7 +302,7 @@ int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *d
     if (ks && M < mmq_from)
         return launch_gemv_ks(type, dX, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
     if (mmq_supported(type, M, K, N, dX, dBias, dY) && (M <= mmq_to || !tp))
-        return launch_mmq(type, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
+        return launch_mmq(type, dX, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
     if (ks) return launch_gemv_ks(type, dX, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
     if (tp) return two_pass(type, false, dX, M, K, dW, N, dBias, act, dY, (hipStream_t)stream);
     return launch_gemm(type, false, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
@@ -348,10 +348,18 @@ int gq_qdense_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, const voi
     if (int rc = check_dense_args("gq_qdense_bf16", type, dX, M, K, dW, N, dBias, act, dY, 2)) return rc;
     if (M == 0 || N == 0) return GQ_OK;
     if (int rc = use_device()) return rc;
-    // decode batches take the bandwidth-bound GEMV (bf16 widened to fp32 on the fly: exact)
-    if (M <= kGemvMaxRows && gemv_ks_supported(type, K, N, dX))
+    // Same crossovers as for fp32 activations: bf16 widens exactly to fp32 for the GEMV passes and to
+    // the fp16 activation image of the split-K kernels (which have no bf16 rounding of W: tighter than
+    // the bf16 MFMA paths).
+    const bool tp = gemm_two_pass_supported(type, true, M, K, N, dX);
+    const bool ks = M <= kGemvMaxRows && gemv_ks_supported(type, K, N, dX);
+    const int64_t mmq_from = type == GQ_Q4_K ? 5 : 8, mmq_to = 96;
+    if (ks && M < mmq_from)
         return launch_gemv_ks(type, dX, true, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
-    if (gemm_two_pass_supported(type, true, M, K, N, dX)) return two_pass(type, true, dX, M, K, dW, N, dBias, act, dY, (hipStream_t)stream);
+    if (mmq_supported(type, M, K, N, dX, dBias, dY) && (M <= mmq_to || !tp))
+        return launch_mmq(type, dX, true, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
+    if (ks) return launch_gemv_ks(type, dX, true, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
+    if (tp) return two_pass(type, true, dX, M, K, dW, N, dBias, act, dY, (hipStream_t)stream);
     return launch_gemm(type, true, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
 }
 

@@ -73,8 +73,8 @@ bool gemv_ks_supported(int type, int64_t K, int64_t N, const void *x);
 int launch_gemv_ks(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N,
                    const float *bias, int act, float *y, hipStream_t s);
 bool mmq_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, const void *bias, const void *y);
-int launch_mmq(int type, const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act,
-               float *y, hipStream_t s);
+int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias,
+               int act, float *y, hipStream_t s);
 struct XsBatchItem { const float *x; const uint8_t *W; const float *bias; float *y; int64_t K, N; int act; };
 int launch_gemv_xs_batch(int type, int count, const XsBatchItem *items, hipStream_t s);
 int launch_gemv_ks_batch(int type, int count, const XsBatchItem *items, hipStream_t s);

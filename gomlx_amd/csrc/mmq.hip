@@ -51,6 +51,22 @@ __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
 
 __device__ __forceinline__ h2 as_h2(uint32_t u) { return __builtin_bit_cast(h2, u); }
 
+// Eight consecutive activations as fp32: from fp32 memory, or from bf16 memory widened (exact).
+template <bool BF16X>
+__device__ __forceinline__ void load_x8(const void *X, int64_t index, float4 &lo, float4 &hi) {
+    if constexpr (BF16X) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(static_cast<const uint16_t *>(X) + index);
+        lo = make_float4(__builtin_bit_cast(float, v.x << 16), __builtin_bit_cast(float, v.x & 0xFFFF0000u),
+                         __builtin_bit_cast(float, v.y << 16), __builtin_bit_cast(float, v.y & 0xFFFF0000u));
+        hi = make_float4(__builtin_bit_cast(float, v.z << 16), __builtin_bit_cast(float, v.z & 0xFFFF0000u),
+                         __builtin_bit_cast(float, v.w << 16), __builtin_bit_cast(float, v.w & 0xFFFF0000u));
+    } else {
+        const float4 *p = reinterpret_cast<const float4 *>(static_cast<const float *>(X) + index);
+        lo = p[0];
+        hi = p[1];
+    }
+}
+
 // (u & mask) | 0x64006400 as an fp16 pair: 1024 + n (mask 0x000F000F), 1024 + 16 n (0x00F000F0)
 // or 1024 + byte (0x00FF00FF)
 // The 0x64006400 operand is passed in a register: with two literals the compiler has to split the
@@ -74,8 +90,8 @@ __device__ __forceinline__ float dpp_quad_sum(float v) {
 // i.e. different slots with the same m, and the xor spreads their 16-byte stores (and the 32
 // columns a half-wave later reads from one slot) over all LDS banks.
 // The eight sub-block sums of (sbl, m) are stored in the order (0, 2, 1, 3, 4, 6, 5, 7) too.
-template <int ROUNDS>
-__device__ __forceinline__ void stage_x(const float *__restrict__ X, int M, int K, int m0, int k0, uint8_t *__restrict__ lds, int tid,
+template <int ROUNDS, bool BF16X>
+__device__ __forceinline__ void stage_x(const void *__restrict__ X, int M, int K, int m0, int k0, uint8_t *__restrict__ lds, int tid,
                                         int round0) {
     const int oct = tid & 255;  // fixed per thread; its items are columns (tid >> 8) + 2 r
     const int k = k0 + 8 * oct;
@@ -88,14 +104,12 @@ __device__ __forceinline__ void stage_x(const float *__restrict__ X, int M, int 
     uint8_t *xf_base = lds + slot * (kMT * 16);
     uint8_t *xs_base = lds + kXFBytes + sbl * (kMT * 16) + jpos * 2;
     const bool k_ok = k < K;
-    const float *src = X + min(k, K - 8);
+    const int ksrc = min(k, K - 8);
     float4 lo[ROUNDS], hi[ROUNDS];
 #pragma unroll
     for (int r = 0; r < ROUNDS; r++) {
         const int m = (tid >> 8) + 2 * (round0 + r);
-        const float4 *p = reinterpret_cast<const float4 *>(src + (int64_t)min(m0 + m, M - 1) * K);
-        lo[r] = p[0];
-        hi[r] = p[1];
+        load_x8<BF16X>(X, (int64_t)min(m0 + m, M - 1) * K + ksrc, lo[r], hi[r]);
     }
 #pragma unroll
     for (int r = 0; r < ROUNDS; r++) {
@@ -134,9 +148,10 @@ __device__ unsigned long long g_mmq_trace[4096 * 8];
 // activations + sub-block sums) to global memory once; the row-range workgroups of the main
 // kernel then only copy 132 KiB each instead of converting it again.  grid = (slices, column
 // tiles, 8): each workgroup converts four of the tile's 32 columns.
-__global__ __launch_bounds__(512) void mmq_xprep_kernel(const float *__restrict__ X, uint8_t *__restrict__ ximg, int M, int K) {
+template <bool BF16X>
+__global__ __launch_bounds__(512) void mmq_xprep_kernel(const void *__restrict__ X, uint8_t *__restrict__ ximg, int M, int K) {
     const int slice = blockIdx.x, mt = blockIdx.y;
-    stage_x<2>(X, M, K, mt * kMT, slice * kSliceK, ximg + ((size_t)mt * gridDim.x + slice) * kLdsBytes, threadIdx.x,
+    stage_x<2, BF16X>(X, M, K, mt * kMT, slice * kSliceK, ximg + ((size_t)mt * gridDim.x + slice) * kLdsBytes, threadIdx.x,
                2 * blockIdx.z);
 }
 
@@ -358,7 +373,8 @@ template <int T> struct B32Geom {
 
 // Image of x for the main kernel: [column tile][slice][octet of the slice][32 columns][8 fp16 in the
 // order (0,2,1,3,4,6,5,7)]; columns beyond M and values beyond K are zero.
-__global__ __launch_bounds__(256) void mmq_b32_xprep_kernel(const float *__restrict__ X, uint8_t *__restrict__ ximg, int M, int K, int S,
+template <bool BF16X>
+__global__ __launch_bounds__(256) void mmq_b32_xprep_kernel(const void *__restrict__ X, uint8_t *__restrict__ ximg, int M, int K, int S,
                                                             int nslices) {
     const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;  // (column tile, slice, octet, column)
     const int m = (int)(g & 31);
@@ -369,11 +385,7 @@ __global__ __launch_bounds__(256) void mmq_b32_xprep_kernel(const float *__restr
     if (mt * kMT >= M) return;
     const int k = slice * S + oct * 8, row = mt * kMT + m;
     float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
-    if (row < M && k < K) {  // K is a multiple of 32: an octet is inside or outside as a whole
-        const float4 *p = reinterpret_cast<const float4 *>(X + (int64_t)row * K + k);
-        a = p[0];
-        b = p[1];
-    }
+    if (row < M && k < K) load_x8<BF16X>(X, (int64_t)row * K + k, a, b);  // K % 32 == 0: an octet is inside or outside as a whole
     reinterpret_cast<uint4 *>(ximg)[g] = make_uint4(pack_h2(a.x, a.z), pack_h2(a.y, a.w), pack_h2(b.x, b.z), pack_h2(b.y, b.w));
 }
 
@@ -488,7 +500,7 @@ __global__ __launch_bounds__(RT * 128) void mmq_b32_kernel(const uint8_t *__rest
 }
 
 template <int T, int RT>
-int launch_mmq_b32(const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y, hipStream_t s) {
+int launch_mmq_b32(const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y, hipStream_t s) {
     const int cus = device_cu_count();
     const int mtiles = (int)((M + kMT - 1) / kMT);
     const int64_t rowwgs = (N + 32 * RT - 1) / (32 * RT);
@@ -511,7 +523,10 @@ int launch_mmq_b32(const float *x, int64_t M, int64_t K, const uint8_t *W, int64
     float *partial = reinterpret_cast<float *>(ximg + img_bytes);
     const int64_t row_bytes = (K / 32) * B32<T>::kBlockBytes;
     const int64_t items = (int64_t)mtiles * nslices * (S / 8) * 32;
-    if (int rc = launch(mmq_b32_xprep_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, x, ximg, (int)M, (int)K, S, nslices))
+    if (int rc = x_is_bf16 ? launch(mmq_b32_xprep_kernel<true>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, x, ximg, (int)M,
+                                    (int)K, S, nslices)
+                           : launch(mmq_b32_xprep_kernel<false>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, x, ximg, (int)M,
+                                    (int)K, S, nslices))
         return rc;
     const dim3 grid((unsigned)rowwgs, (unsigned)nslices, (unsigned)mtiles);
     if (int rc = launch(mmq_b32_kernel<T, RT>, grid, dim3(RT * 128), lds_bytes, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N, row_bytes, S))
@@ -531,11 +546,11 @@ bool mmq_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, con
     return false;
 }
 
-int launch_mmq(int type, const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act,
-               float *y, hipStream_t s) {
+int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias,
+               int act, float *y, hipStream_t s) {
     // (four row tiles per workgroup measured a little faster than two)
-    if (type == kQ8_0) return launch_mmq_b32<kQ8_0, 4>(x, M, K, W, N, bias, act, y, s);
-    if (type == kQ4_0) return launch_mmq_b32<kQ4_0, 4>(x, M, K, W, N, bias, act, y, s);
+    if (type == kQ8_0) return launch_mmq_b32<kQ8_0, 4>(x, x_is_bf16, M, K, W, N, bias, act, y, s);
+    if (type == kQ4_0) return launch_mmq_b32<kQ4_0, 4>(x, x_is_bf16, M, K, W, N, bias, act, y, s);
     if (type != kQ4_K) return fail(GQ_ERR_NOT_IMPLEMENTED, "mmq: ggml type %d is not implemented", type);
     static const bool lds_ok = [] {
         return hipFuncSetAttribute(reinterpret_cast<const void *>(mmq_q4k_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -552,7 +567,8 @@ int launch_mmq(int type, const float *x, int64_t M, int64_t K, const uint8_t *W,
     uint8_t *ximg = reinterpret_cast<uint8_t *>(ws);
     float *partial = reinterpret_cast<float *>(ximg + img_bytes);
     const int64_t row_bytes = (K / 256) * 144;
-    if (int rc = launch(mmq_xprep_kernel, dim3((unsigned)nslices, (unsigned)mtiles, 8), dim3(512), 0, s, x, ximg, (int)M, (int)K))
+    if (int rc = x_is_bf16 ? launch(mmq_xprep_kernel<true>, dim3((unsigned)nslices, (unsigned)mtiles, 8), dim3(512), 0, s, x, ximg, (int)M, (int)K)
+                           : launch(mmq_xprep_kernel<false>, dim3((unsigned)nslices, (unsigned)mtiles, 8), dim3(512), 0, s, x, ximg, (int)M, (int)K))
         return rc;
     const dim3 grid((unsigned)((N + kRowsPerWG - 1) / kRowsPerWG), (unsigned)nslices);
     for (int64_t m0 = 0; m0 < M; m0 += kMT) {

@@ -180,6 +180,22 @@ def test_split_k_small_batches_q8_q4(gpu, oracle, t, M, K, N):
         got = run_dense(gpu, t, x, W, bias, act)
         want = oracle.c_qdense(t, x, W, bias, act)
         assert rel_err(got, want) < TOL_F32, (t, M, K, N, act)
+    # bf16 activations widen exactly into the kernel's fp16 image: same bound (the shape that is not
+    # this kernel's takes a bf16 MFMA path)
+    xb = bf16_round(x)
+    tol = TOL_F32 if K % 256 == 0 else TOL_BF16
+    assert rel_err(run_dense(gpu, t, xb, W, bias, 0, bf16=True), oracle.c_qdense(t, xb, W, bias, 0)) < tol, (t, M, K, N, "bf16")
+
+
+@pytest.mark.parametrize("M,K,N", [(5, 256, 8), (32, 2048, 260), (70, 4096, 512), (96, 1024, 4096)])
+def test_split_k_small_batches_q4_k(gpu, oracle, M, K, N):
+    """5 .. 96 rows of Q4_K, fp32 and bf16 activations, through the split-K MFMA kernel."""
+    W = synth.weights(Q4_K, 75, N, K)
+    x = synth.activations(76, M, K)
+    bias = synth.normal(77, 0, N).astype(np.float32) * 0.1
+    assert rel_err(run_dense(gpu, Q4_K, x, W, bias, 3), oracle.c_qdense(Q4_K, x, W, bias, 3)) < TOL_F32, (M, K, N, "f32")
+    xb = bf16_round(x)
+    assert rel_err(run_dense(gpu, Q4_K, xb, W, bias, 3, bf16=True), oracle.c_qdense(Q4_K, xb, W, bias, 3)) < TOL_F32, (M, K, N, "bf16")
 
 
 @pytest.mark.parametrize("t", ALL_TYPES)
