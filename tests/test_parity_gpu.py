@@ -475,6 +475,48 @@ def test_recorded_chain_replays_match_eager(gpu, oracle):
     _lib.check(L.gq_graph_destroy(g))
 
 
+def test_recording_needs_the_stream_workspace_to_exist(gpu, oracle):
+    """Paths with a workspace (here the two-pass GEMM) refuse to allocate inside a recording: the
+    call reports an error, the recording stays usable, and after one eager call on the stream the
+    same recording works and replays exactly."""
+    import ctypes
+    from gomlx_amd import _lib
+    torch = gpu
+    L = _lib.lib()
+    M, K, N = 600, 256, 128
+    W = dev(torch, synth.weights(Q4_0, 150, N, K))
+    x = dev(torch, synth.activations(151, M, K))
+    x1 = dev(torch, synth.activations(152, 1, K))
+    y = torch.zeros(M, N, device="cuda")
+    y1 = torch.zeros(1, N, device="cuda")
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()  # a fresh stream: no workspace yet
+    sp = stream.cuda_stream
+    dense = lambda xx, rows, yy: L.gq_qdense_f32(Q4_0, xx.data_ptr(), rows, K, W.data_ptr(), N, None, 0, yy.data_ptr(), sp)
+    _lib.check(L.gq_graph_begin(sp))
+    _lib.check(dense(x1, 1, y1))  # a path without workspace records fine
+    rc = dense(x, M, y)
+    assert rc == _lib.ERR_INVALID
+    assert b"workspace" in L.gq_last_error()
+    g = ctypes.c_void_p()
+    _lib.check(L.gq_graph_end(sp, ctypes.byref(g)))
+    _lib.check(L.gq_graph_destroy(g))
+    _lib.check(dense(x, M, y))  # eager: creates the stream's workspace
+    _lib.check(L.gq_sync(sp))
+    eager = y.clone()
+    assert rel_err(eager.cpu().numpy(), oracle.c_qdense(Q4_0, x.cpu().numpy(), W.cpu().numpy())) < TOL_F32
+    _lib.check(L.gq_graph_begin(sp))
+    _lib.check(dense(x, M, y))
+    _lib.check(L.gq_graph_end(sp, ctypes.byref(g)))
+    for rep in range(3):
+        y.fill_(float("nan"))
+        torch.cuda.synchronize()
+        _lib.check(L.gq_graph_launch(g, sp))
+        _lib.check(L.gq_sync(sp))
+        assert torch.equal(y, eager), rep
+    _lib.check(L.gq_graph_destroy(g))
+
+
 def test_kernel_timing_hook_counts_launches(gpu):
     from gomlx_amd import _lib
     import ctypes
