@@ -1,18 +1,20 @@
-// Large-batch quantised Dense in two passes:
+// Quantised Dense for batches of 17 rows and more, in two passes:
 //   1. the weight matrix is dequantised once into a 16-bit [N, K] image in a workspace (exact
 //      fp32 values, one rounding to the MFMA operand type: the same operand values the fused
 //      kernel of gemm.hip builds tile by tile);
 //   2. a plain 16-bit x 16-bit -> fp32 MFMA GEMM contracts it with the activations.
 //
 // The fused kernel converts a 128-row slab of W again for every 256 rows of activations, and on a
-// SIMD those vector-ALU instructions do not overlap with its MFMAs; from a few hundred rows on it
-// is cheaper to convert once and let the matrix cores run without vector work.  The GEMM moves
+// SIMD those vector-ALU instructions do not overlap with its MFMAs; it is cheaper to convert once
+// and let the matrix cores run without vector work (and small batches get tiles that fill the
+// chip, which the fused kernel's fixed 256 x 128 tile does not).  The GEMM moves
 // both operands from global memory straight into LDS (buffer loads with the LDS modifier: no
 // registers, no vector-ALU instructions) two K steps ahead through a ring of three LDS stages.
 //
 // Tile: 256 x 128 per workgroup, 8 wavefronts x (64 x 64 = 2 x 2 v_mfma_f32_32x32x16), or 128 x 128
-// and 128 x 64 when the problem has too few large tiles to fill the chip; K in steps of 64.  LDS rows are 128 bytes, unpadded (the DMA writes 1 KB = 8 rows per wavefront
-// instruction, lane l -> bytes 16 l ..), and 16-byte chunk c of row r is kept in slot
+// and 128 x 64 when the problem has too few large tiles to fill the chip; K in steps of 64.  LDS
+// rows are 128 bytes, unpadded (the DMA writes 1 KB = 8 rows per wavefront instruction, lane l ->
+// bytes 16 l ..), and 16-byte chunk c of row r is kept in slot
 // c ^ ((r >> 1) & 7): 16 consecutive lanes of a fragment read then cover all 64 banks once.  The
 // swizzle is applied on the global side: lane l of a DMA fetches chunk (l & 7) ^ ((r >> 1) & 7) of
 // row r = 8 * block + (l >> 3), so every 128-byte row is still read as one full line.
