@@ -321,16 +321,19 @@ int gq_qdense_f32_batch(int count, const gq_dense_desc *descs, void *stream) {
     while (i < count) {
         int j = i;
         XsBatchItem items[8];
-        bool all_ks = true;
-        while (j < count && j - i < 8 && descs[j].type == descs[i].type && descs[j].M == 1 && descs[j].N > 0 &&
-               gemv_xs_supported(descs[j].type, descs[j].K, descs[j].N, descs[j].dX)) {
+        // the kernel family of the run is that of its first problem: K-sliced where that applies, else
+        // activation-stationary
+        const bool use_ks = gemv_ks_supported(descs[i].type, descs[i].K, descs[i].N, descs[i].dX);
+        auto fits = [&](const gq_dense_desc &d) {
+            return use_ks ? gemv_ks_supported(d.type, d.K, d.N, d.dX) : gemv_xs_supported(d.type, d.K, d.N, d.dX);
+        };
+        while (j < count && j - i < 8 && descs[j].type == descs[i].type && descs[j].M == 1 && descs[j].N > 0 && fits(descs[j])) {
             const gq_dense_desc &d = descs[j];
             items[j - i] = XsBatchItem{d.dX, (const uint8_t *)d.dW, d.dBias, d.dY, d.K, d.N, d.act};
-            all_ks = all_ks && gemv_ks_supported(d.type, d.K, d.N, d.dX);
             j++;
         }
         if (j - i >= 2) {
-            if (int rc = all_ks ? launch_gemv_ks_batch(descs[i].type, j - i, items, (hipStream_t)stream)
+            if (int rc = use_ks ? launch_gemv_ks_batch(descs[i].type, j - i, items, (hipStream_t)stream)
                                 : launch_gemv_xs_batch(descs[i].type, j - i, items, (hipStream_t)stream))
                 return rc;
             i = j;

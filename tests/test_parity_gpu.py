@@ -407,6 +407,10 @@ def test_batched_submission_equals_separate_calls(gpu, oracle):
     hosts.append((Q4_K, synth.activations(200, 5, 512), synth.weights(Q4_K, 201, 64, 512), None, Activation.NONE))
     hosts.append((Q8_0, synth.activations(202, 1, 2048), synth.weights(Q8_0, 203, 300, 2048), None, Activation.RELU))
     hosts.append((Q8_0, synth.activations(204, 1, 2048), synth.weights(Q8_0, 205, 77, 2048), None, Activation.NONE))
+    # a run of Q6_K problems (K-sliced kernels only), then one whose K has no K-sliced plan
+    hosts.append((Q6_K, synth.activations(206, 1, 1024), synth.weights(Q6_K, 207, 256, 1024), None, Activation.NONE))
+    hosts.append((Q6_K, synth.activations(208, 1, 1024), synth.weights(Q6_K, 209, 520, 1024), None, Activation.GELU))
+    hosts.append((Q6_K, synth.activations(210, 1, 768), synth.weights(Q6_K, 211, 100, 768), None, Activation.NONE))
     for t, x, W, b, act in hosts:
         probs.append((dev(torch, x), dev(torch, W), Quantization(ggml_type=t), None if b is None else dev(torch, b), act))
     outs = nn.quantized_dense_batch(probs)
