@@ -348,6 +348,43 @@ def test_large_batches_few_k_steps(gpu, oracle, K):
     assert rel_err(run_dense(gpu, Q8_0, x, W, None, 0, bf16=True), want) < TOL_BF16, K
 
 
+def _boundary_cases():
+    """Seeded random problems around every batch-size threshold of the dispatcher."""
+    rng = np.random.default_rng(20240607)
+    rows = [1, 2, 4, 5, 7, 8, 9, 16, 17, 31, 32, 33, 64, 95, 96, 97, 128, 129, 256, 257, 300, 511, 512, 513]
+    cases = []
+    for i, M in enumerate(rows):
+        for rep in range(2):
+            t = ALL_TYPES[(i + 2 * rep) % len(ALL_TYPES)]
+            big = t in (Q4_K, Q6_K)
+            if rep == 0:
+                K = int(rng.choice([256, 512, 768, 1024, 2048]))
+            else:
+                K = int(rng.choice([256, 1280]) if big else rng.choice([32, 96, 160, 544, 1056]))
+            N = int(rng.choice([4, 36, 64, 100, 132, 257, 512, 600]))
+            cases.append((t, M, K, N, bool((i + rep) % 2), int(rng.integers(0, 6)), bool(rng.integers(0, 2))))
+    return cases
+
+
+@pytest.mark.parametrize("t,M,K,N,bf16,act,with_bias", _boundary_cases())
+def test_dispatch_boundaries(gpu, oracle, t, M, K, N, bf16, act, with_bias):
+    """The error is measured against the larger of the output and the pre-activation magnitude: a
+    saturating activation (tanh) shrinks the outputs but not the error of the contraction that
+    feeds it (all six activations have slope <= 1.13), and the bound is on that contraction."""
+    W = synth.weights(t, 300 + M, N, K)
+    x = synth.activations(301 + M, M, K)
+    bias = synth.normal(302 + M, 0, N).astype(np.float32) * 0.1 if with_bias else None
+    if bf16:
+        x = bf16_round(x)
+    got = run_dense(gpu, t, x, W, bias, act, bf16=bf16)
+    want = oracle.c_qdense(t, x, W, bias, act)
+    pre = oracle.c_qdense(t, x, W, bias, 0)
+    assert got.shape == (M, N)
+    scale = max(float(np.max(np.abs(want))), float(np.max(np.abs(pre)))) or 1.0
+    err = float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)))) / scale
+    assert err < (TOL_BF16 if bf16 else TOL_F32), (t, M, K, N, bf16, act, err)
+
+
 # ------------------------------------------------------------------------------ benchmark configurations, full size
 
 def test_config0_q8_0_gemv_4096(gpu, oracle):
