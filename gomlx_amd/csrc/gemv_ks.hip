@@ -1,5 +1,5 @@
 // Decode GEMV, K-sliced integer-dot kernels with wavefront-local activation staging
-// (Q4_0, Q8_0, Q4_K, Q6_K; K % 512 == 0).
+// (Q4_0, Q8_0, Q4_K, Q6_K; K % 256 == 0).
 //
 // The activation-stationary kernel of gemv_xs.hip lets every wavefront see all of K, so its
 // workgroup has to convert the whole activation vector together and meet at a barrier before the
@@ -8,7 +8,9 @@
 // 8 activations each, exchange the fixed-point planes through a private piece of LDS (no
 // barrier: LDS operations of one wavefront execute in order) and start on the codes as soon as
 // their own 2 KB of x have arrived.  The wavefronts of a workgroup cover the slices of the same
-// rows and add their partial sums in LDS once, at the very end.
+// rows (slice w, w + waves, ...: one more for the first few when the count does not divide; a last
+// half slice when K is an odd multiple of 256 runs with zero activations for its missing half) and
+// add their partial sums in LDS once, at the very end.
 //
 // Lane l = 8 * rg + c works on row (8 * it + rg) of the workgroup and on 64 values of the slice:
 //   Q4_0: blocks 2c, 2c+1: 36 bytes at a 4-byte-aligned address;
@@ -371,25 +373,35 @@ __device__ unsigned long long g_ks_trace[4096 * 16];
 constexpr int kWaveLdsDwords = 76 * 4;  // per wavefront: 64 uint4 of planes, 16 scales, up to 32 sums
 
 // Workgroup `wg` of a problem: `waves` wavefronts work (threads beyond them only join the final
-// barrier); wavefront w handles slices w, w + waves, ... (spw of them) of the 8 * iters rows
+// barrier); wavefront w handles slices w, w + waves, ... below nslices of the 8 * iters rows
 // starting at wg * 8 * iters.  PF divides iters: rows are consumed in groups of PF, buffer j of a
 // group always holding the row-step with (it % PF == j).
 // WIN <= PF row-steps are kept in flight: WIN go out before the activations are converted, and
 // each consumed step is followed by the load of the step WIN ahead, so that load issue (which
 // blocks while the memory pipeline is full) and arithmetic alternate instead of forming two
-// phases.
+// phases.  (A variant that treats a wavefront's slices x row-steps as one sequence, so that the
+// window also spans slices when there are only one or two row-steps, was measured: its guarded
+// steps cost the unguarded common case 8 % and it was dropped.)
 template <int T, int PF, int WIN>
 __device__ __forceinline__ void ks_body(const void *__restrict__ xv, int x_bf16, const uint8_t *__restrict__ W,
                                         const float *__restrict__ bias, float *__restrict__ y, int N, int64_t row_bytes, int iters,
-                                        int spw, int act, int waves, int wg, uint32_t *lds) {
+                                        int nslices, int half_tail, int act, int waves, int wg, uint32_t *lds) {
     typedef typename KS<T>::Raw Raw;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int rg = lane >> 3, c = lane & 7;
     const int rows_wg = iters * 8;
     const int row0 = wg * rows_wg;
     float *all = reinterpret_cast<float *>(lds + waves * kWaveLdsDwords);  // partial sums [waves][rows_wg]
-    // activations of slice sl for this lane (fp32, or bf16 widened on the fly; x_bf16 is uniform)
+    // activations of slice sl for this lane (fp32, or bf16 widened on the fly; x_bf16 is uniform);
+    // the lanes that face the missing half of a last half slice get zeros
+    const bool upper_half = lane >= 32;  // this lane converts values 256 .. 511 of a slice (in both activation layouts)
     auto x_slice = [&](int sl) -> XPair {
+        if (half_tail && sl == nslices - 1 && upper_half) {
+            XPair z;
+            z.lo = make_float4(0.f, 0.f, 0.f, 0.f);
+            z.hi = z.lo;
+            return z;
+        }
         if (x_bf16) return KS<T>::x_load_bf16(reinterpret_cast<const uint16_t *>(xv) + sl * kSliceValues, lane);
         return KS<T>::x_load(reinterpret_cast<const float *>(xv) + sl * kSliceValues, lane);
     };
@@ -401,15 +413,19 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, int x_bf16,
 
         KS_TRACE(0);
         KS_TRACE_WALL(12);
+        const int spw = (nslices - wave + waves - 1) / waves;  // slices of this wavefront (>= 1)
         XPair xp = x_slice(wave);
         const int last_row = N - 1;
+        // In a last half slice the lanes of the missing half re-read the codes of the present one
+        // (finite scales; their activations are zero).
+        auto lane_c = [&](int j) { return (half_tail && wave + j * waves == nslices - 1) ? (c & 3) : c; };
         auto addr = [&](int j, int it) -> const uint8_t * {
             const int row = min(row0 + it * 8 + rg, last_row);
-            return W + (int64_t)row * row_bytes + (int64_t)(wave + j * waves) * KS<T>::kSliceBytes + KS<T>::lane_offset(c);
+            return W + (int64_t)row * row_bytes + (int64_t)(wave + j * waves) * KS<T>::kSliceBytes + KS<T>::lane_offset(lane_c(j));
         };
         Raw buf[PF];
 #pragma unroll
-        for (int j = 0; j < WIN; j++) ks_load<T>(buf[j], addr(0, j), c);
+        for (int j = 0; j < WIN; j++) ks_load<T>(buf[j], addr(0, j), lane_c(0));
         KS_TRACE(1);
 
         uint4 xq[8];
@@ -451,8 +467,8 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, int x_bf16,
 #pragma unroll
             for (int jj = 0; jj < PF; jj++) {
                 float d = KS<T>::dot(buf[jj], xq, xsc, xsm, c);
-                if (jj + WIN < PF) ks_load<T>(buf[jj + WIN], addr(j, i0 + jj + WIN), c);
-                else if (!last_group) ks_load<T>(buf[jj + WIN - PF], addr(nj, ni0 + jj + WIN - PF), c);
+                if (jj + WIN < PF) ks_load<T>(buf[jj + WIN], addr(j, i0 + jj + WIN), lane_c(j));
+                else if (!last_group) ks_load<T>(buf[jj + WIN - PF], addr(nj, ni0 + jj + WIN - PF), lane_c(nj));
                 d = ks_oct_sum(d);
                 if (c == 0) {
                     float *slot = part + (i0 + jj) * 8 + rg;
@@ -483,10 +499,10 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, int x_bf16,
 template <int T, int PF, int WIN>
 __global__ __launch_bounds__(512) void gemv_ks_kernel(const void *__restrict__ X, int x_bf16, const uint8_t *__restrict__ W,
                                                       const float *__restrict__ bias, float *__restrict__ Y, int K, int N,
-                                                      int64_t row_bytes, int iters, int spw, int act) {
+                                                      int64_t row_bytes, int iters, int nslices, int half_tail, int act) {
     extern __shared__ uint32_t lds[];
     const uint8_t *x = reinterpret_cast<const uint8_t *>(X) + (int64_t)blockIdx.y * K * (x_bf16 ? 2 : 4);
-    ks_body<T, PF, WIN>(x, x_bf16, W, bias, Y + (int64_t)blockIdx.y * N, N, row_bytes, iters, spw, act, (int)(blockDim.x >> 6),
+    ks_body<T, PF, WIN>(x, x_bf16, W, bias, Y + (int64_t)blockIdx.y * N, N, row_bytes, iters, nslices, half_tail, act, (int)(blockDim.x >> 6),
                         (int)blockIdx.x, lds);
 }
 
@@ -501,7 +517,7 @@ struct KsProblem {
     const float *bias;
     float *y;
     int64_t row_bytes;
-    int N, iters, spw, waves, act, wg_begin;
+    int N, iters, nslices, half_tail, waves, act, wg_begin;
 };
 struct KsBatch {
     int count;
@@ -516,10 +532,11 @@ __global__ __launch_bounds__(512) void gemv_ks_batch_kernel(const KsBatch b) {
     for (int j = 1; j < kMaxBatchKs; j++)
         if (j < b.count && (int)blockIdx.x >= b.p[j].wg_begin) i = j;
     const KsProblem &q = b.p[i];
-    ks_body<T, 4, 3>(q.x, 0, q.W, q.bias, q.y, q.N, q.row_bytes, q.iters, q.spw, q.act, q.waves, (int)blockIdx.x - q.wg_begin, lds);
+    ks_body<T, 4, 3>(q.x, 0, q.W, q.bias, q.y, q.N, q.row_bytes, q.iters, q.nslices, q.half_tail, q.act, q.waves,
+                     (int)blockIdx.x - q.wg_begin, lds);
 }
 
-struct KsPlan { int waves, spw, iters, pf, wgs; size_t shmem; };
+struct KsPlan { int waves, nslices, half_tail, iters, pf, wgs; size_t shmem; };
 
 // GOMLX_HIPQ_GEMV_KS="waves_per_cu" overrides the built-in choice (tuning runs only).
 int ks_env_waves() {
@@ -527,22 +544,20 @@ int ks_env_waves() {
     return v;
 }
 
-// wavefronts per workgroup (a divisor of the slice count, at most 8) and slices per wavefront
-bool ks_split(int64_t K, int &waves, int &spw) {
-    if (K % kSliceValues != 0 || K <= 0) return false;
-    const int nslices = (int)(K / kSliceValues);
-    waves = 0;
-    for (int w = 8; w >= 1; w--)
-        if (nslices % w == 0) { waves = w; break; }
-    if (waves < 4 && nslices > 8) return false;  // awkward K (e.g. a large prime number of slices)
-    spw = nslices / waves;
+// Slices of 512 values (a last one of 256 when K is an odd multiple of 256) and wavefronts per
+// workgroup: one per slice up to 8; more slices than that are dealt out round-robin.
+bool ks_split(int64_t K, int &waves, int &nslices, int &half_tail) {
+    if (K <= 0 || K % 256 != 0 || K > (int64_t)INT32_MAX / 4) return false;
+    nslices = (int)((K + kSliceValues - 1) / kSliceValues);
+    half_tail = (K % kSliceValues) != 0 ? 1 : 0;
+    waves = nslices < 8 ? nslices : 8;
     return true;
 }
 
 size_t ks_lds_bytes(int waves, int iters) { return (size_t)waves * kWaveLdsDwords * 4 + (size_t)waves * iters * 8 * sizeof(float); }
 
 bool ks_plan(int64_t K, int64_t N, KsPlan &p) {
-    if (N <= 0 || !ks_split(K, p.waves, p.spw)) return false;
+    if (N <= 0 || !ks_split(K, p.waves, p.nslices, p.half_tail)) return false;
     const int cus = device_cu_count();
     // One 8-wavefront workgroup per CU streams best; problems that would leave a wavefront with
     // only one or two row-steps are launch- and latency-bound and do better with twice the
@@ -570,8 +585,8 @@ int launch_ks_pf(const KsPlan &p, const void *x, int x_bf16, int64_t M, int64_t 
     const int64_t row_bytes = (K / Geom<T>::vpb) * Geom<T>::bpb;
     const dim3 grid((unsigned)p.wgs, (unsigned)M), block((unsigned)p.waves * 64);
     constexpr int WIN = PF < 3 ? PF : 3;
-    return launch(gemv_ks_kernel<T, PF, WIN>, grid, block, p.shmem, s, x, x_bf16, W, bias, y, (int)K, (int)N, row_bytes, p.iters, p.spw,
-                  act);
+    return launch(gemv_ks_kernel<T, PF, WIN>, grid, block, p.shmem, s, x, x_bf16, W, bias, y, (int)K, (int)N, row_bytes, p.iters, p.nslices,
+                  p.half_tail, act);
 }
 
 template <int T>
@@ -607,7 +622,7 @@ int launch_ks_batch(int count, const XsBatchItem *items, hipStream_t s) {
         KsProblem q;
         q.x = it.x; q.W = it.W; q.bias = it.bias; q.y = it.y; q.N = (int)it.N; q.act = it.act;
         q.row_bytes = (int64_t)gq_row_bytes(T, it.K);
-        if (!ks_split(it.K, q.waves, q.spw)) return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv_ks batch: unsupported K");
+        if (!ks_split(it.K, q.waves, q.nslices, q.half_tail)) return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv_ks batch: unsupported K");
         int64_t share = (int64_t)((double)cus * ((double)q.row_bytes * (double)it.N) / total + 0.5);
         if (share < 1) share = 1;
         int64_t iters = (it.N + share * 8 - 1) / (share * 8);
@@ -629,8 +644,8 @@ bool gemv_ks_supported(int type, int64_t K, int64_t N, const void *x) {
     if (reinterpret_cast<uintptr_t>(x) & 15) return false;
     if (type != kQ4_0 && type != kQ8_0 && type != kQ4_K && type != kQ6_K) return false;
     if (N <= 0 || N > (int64_t)INT32_MAX / 2) return false;
-    int waves, spw;
-    return ks_split(K, waves, spw);
+    int waves, nslices, half_tail;
+    return ks_split(K, waves, nslices, half_tail);
 }
 
 int launch_gemv_ks(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias,

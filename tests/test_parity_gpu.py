@@ -116,15 +116,20 @@ def test_gemv_parity(gpu, oracle, t, M, K, N):
 @pytest.mark.parametrize("M,K,N", [
     (1, 1536, 100),     # 3 slices of 512: three wavefronts per workgroup
     (2, 3584, 513),     # 7 slices, rows not a multiple of 8
-    (1, 4608, 40),      # 9 slices: no usable split, activation-stationary fallback
+    (1, 4608, 40),      # 9 slices on 8 wavefronts: the first takes two
+    (2, 256, 33),       # a single half slice
+    (1, 768, 100),      # one slice and a half
+    (3, 5376, 50),      # ten slices and a half: uneven shares and a half tail
+    (1, 9472, 300),     # eighteen and a half
+    (1, 18944, 24),     # 37 slices (a prime): 5 or 4 per wavefront
     (1, 8192, 2100),    # two slices per wavefront
     (3, 2048, 20000),   # five row-steps per wavefront, all in flight
     (1, 512, 300000),   # one wavefront per workgroup, many groups of four row-steps
     (1, 8192, 40000),   # groups of four row-steps wrapping from one slice to the next
 ])
 def test_gemv_k_sliced_plans(gpu, oracle, t, M, K, N):
-    """Shapes that walk through the planner of the K-sliced decode kernel (wavefronts per
-    workgroup, slices per wavefront, prefetch groups) and its fallback."""
+    """Shapes that walk through the planner of the K-sliced decode kernel: wavefronts per
+    workgroup, even and uneven slices per wavefront, a last half slice, prefetch groups."""
     W = synth.weights(t, 40 + t, N, K)
     x = synth.activations(41 + t, M, K)
     bias = synth.normal(42 + t, 0, N).astype(np.float32) * 0.1
@@ -444,10 +449,13 @@ def test_batched_submission_equals_separate_calls(gpu, oracle):
     hosts.append((Q4_K, synth.activations(200, 5, 512), synth.weights(Q4_K, 201, 64, 512), None, Activation.NONE))
     hosts.append((Q8_0, synth.activations(202, 1, 2048), synth.weights(Q8_0, 203, 300, 2048), None, Activation.RELU))
     hosts.append((Q8_0, synth.activations(204, 1, 2048), synth.weights(Q8_0, 205, 77, 2048), None, Activation.NONE))
+    # two problems whose K is an odd multiple of 256 (half tail slice) share a launch too
+    hosts.append((Q4_0, synth.activations(212, 1, 1280), synth.weights(Q4_0, 213, 200, 1280), None, Activation.NONE))
+    hosts.append((Q4_0, synth.activations(214, 1, 4864), synth.weights(Q4_0, 215, 64, 4864), None, Activation.NONE))
     # a run of Q6_K problems (K-sliced kernels only), then one whose K has no K-sliced plan
     hosts.append((Q6_K, synth.activations(206, 1, 1024), synth.weights(Q6_K, 207, 256, 1024), None, Activation.NONE))
     hosts.append((Q6_K, synth.activations(208, 1, 1024), synth.weights(Q6_K, 209, 520, 1024), None, Activation.GELU))
-    hosts.append((Q6_K, synth.activations(210, 1, 768), synth.weights(Q6_K, 211, 100, 768), None, Activation.NONE))
+    hosts.append((Q8_0, synth.activations(210, 1, 96), synth.weights(Q8_0, 211, 100, 96), None, Activation.NONE))
     for t, x, W, b, act in hosts:
         probs.append((dev(torch, x), dev(torch, W), Quantization(ggml_type=t), None if b is None else dev(torch, b), act))
     outs = nn.quantized_dense_batch(probs)
