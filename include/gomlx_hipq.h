@@ -94,11 +94,16 @@ int gq_dequantize(int type, const void *dW, int64_t N, int64_t K, float *dOut, v
 /* ---- compute.Function.FusedQuantizedDense (core/graph/fused_ops.go:231-232), run time:
  * y = act(x . dequant(W)^T + bias), the contract of nn.QuantizedDense
  * (ml/nn/quantized_dense.go:31-57) and ggml.DenseDecomposed (ml/ggml/dense.go:23-62).
- * dBias may be NULL.  fp32 activations: fp32 accumulation. ---- */
+ * dBias may be NULL.  fp32 activations, fp32 accumulation.  Up to about ten rows run as
+ * bandwidth-bound GEMV passes; larger batches contract on the matrix cores with the activations
+ * (and, from 97 rows on, the dequantised weights) rounded to fp16 operands.  Batches of 5 rows and
+ * more may use a per-stream workspace that is created on the first such call on the stream: make
+ * one call outside a recording (gq_graph_begin) before recording the same call. ---- */
 int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *dW, int64_t N,
                   const float *dBias, int act, float *dY, void *stream);
-/* bf16 activations (raw 16-bit patterns): weights are dequantised to bf16 tiles in LDS and
- * contracted on bf16 MFMA with fp32 accumulation; fp32 output. */
+/* bf16 activations (raw 16-bit patterns), fp32 output.  Small batches widen the activations
+ * exactly and take the same GEMV / split-K kernels as fp32 activations; from 97 rows on the
+ * weights are dequantised to bf16 operands and contracted on bf16 MFMA with fp32 accumulation. */
 int gq_qdense_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, const void *dW,
                    int64_t N, const float *dBias, int act, float *dY, void *stream);
 
