@@ -113,6 +113,12 @@ int check_dense_args(const char *fn, int type, const void *x, int64_t M, int64_t
     return GQ_OK;
 }
 
+// Batch sizes served by the split-K small-batch kernels (measured crossovers against the GEMV passes
+// below and the two-pass GEMM above, K = 4096, N = 4096 .. 14336).  The Q6_K kernel pays 16 scale
+// groups per super-block and only wins for a single tile of 32 batch columns.
+int64_t split_k_from(int type) { return type == GQ_Q4_K ? 5 : type == GQ_Q6_K ? 6 : 8; }
+int64_t split_k_to(int type) { return type == GQ_Q6_K ? 32 : 96; }
+
 // large batches: W dequantised once into the stream's workspace, then a plain 16-bit GEMM
 int two_pass(int type, bool x_is_bf16, const void *x, int64_t M, int64_t K, const void *W, int64_t N, const float *bias, int act,
              float *y, hipStream_t s) {
@@ -295,10 +301,10 @@ int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *d
     // Small batches: GEMV passes cost about one third of the first pass per extra row; the split-K
     // MFMA kernels cost 19 .. 26 us (Q8_0 / Q4_0, K = 4096, N = 4096 .. 14336) for up to 32 rows and
     // 5 .. 18 us per further 32; the two passes 33 .. 62 us for anything up to 128 rows.  Measured
-    // crossovers: GEMV below 8 rows (Q4_K: below 5), split-K up to 96 rows, then two passes.
+    // crossovers: split_k_from() / split_k_to().
     const bool tp = gemm_two_pass_supported(type, false, M, K, N, dX);
     const bool ks = M <= kGemvMaxRows && gemv_ks_supported(type, K, N, dX);
-    const int64_t mmq_from = type == GQ_Q4_K ? 5 : 8, mmq_to = 96;
+    const int64_t mmq_from = split_k_from(type), mmq_to = split_k_to(type);
     if (ks && M < mmq_from)
         return launch_gemv_ks(type, dX, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
     if (mmq_supported(type, M, K, N, dX, dBias, dY) && (M <= mmq_to || !tp))
@@ -356,7 +362,7 @@ int gq_qdense_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, const voi
     // the bf16 MFMA paths).
     const bool tp = gemm_two_pass_supported(type, true, M, K, N, dX);
     const bool ks = M <= kGemvMaxRows && gemv_ks_supported(type, K, N, dX);
-    const int64_t mmq_from = type == GQ_Q4_K ? 5 : 8, mmq_to = 96;
+    const int64_t mmq_from = split_k_from(type), mmq_to = split_k_to(type);
     if (ks && M < mmq_from)
         return launch_gemv_ks(type, dX, true, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
     if (mmq_supported(type, M, K, N, dX, dBias, dY) && (M <= mmq_to || !tp))

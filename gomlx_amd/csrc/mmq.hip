@@ -1,5 +1,5 @@
 // Small-batch (decode batch 5..~128) quantised Dense on the gfx950 matrix cores: Q4_K, and further
-// down Q8_0 / Q4_0.
+// down Q8_0 / Q4_0 and Q6_K.
 //
 // At batch 32 the contraction is 228 flop per weight byte: far beyond the vector ALUs, still
 // below the MFMA machine balance, so the kernel should run at the speed the packed weights
@@ -536,6 +536,177 @@ int launch_mmq_b32(const void *x, bool x_is_bf16, int64_t M, int64_t K, const ui
                   bias, act, y);
 }
 
+
+// ---- small batches of Q6_K --------------------------------------------------------------------------
+//
+// Same plan again.  A super-block is 210 bytes (2 bytes off a dword boundary every other one), so a
+// wavefront's unit is a PAIR of super-blocks: 420 bytes = 105 dwords per row, dword-aligned when K
+// is a multiple of 512.  The wavefront reads the pair of its 32 rows as consecutive dwords
+// (coalesced), parks it in its private piece of LDS (row stride 105 dwords: odd, conflict-free) and
+// lane (col = lane % 32, kg = lane / 32) picks row col's codes out of it.  One MFMA (K = 16) is
+// exactly one 16-value scale group: lane kg holds values 8 kg .. 8 kg + 7 of it, assembled from the
+// low nibbles / high bit pairs into bytes, turned into exact fp16 integers code - 32, and the
+// group's partial tile is scaled by d * sc in fp32.
+// Slices are 1024 values (two pairs: one per wavefront of a row tile); RT = 2 row tiles per
+// workgroup, so the 64 KiB activation image and four parked pairs fit LDS.
+constexpr int kQ6PairBytes = 420, kQ6PairDwords = 105;
+constexpr int kQ6Loads = (32 * kQ6PairDwords + 63) / 64;  // 53 dword loads per lane and pair (the last: half a wavefront)
+constexpr int kQ6WaveLds = 32 * kQ6PairBytes + 16;         // + slack for a window that ends past the last row
+constexpr int kQ6Slice = 1024;
+constexpr int kQ6RT = 2;
+
+// two dwords holding the 8 bytes at byte offset `at` of the parked row (at % 4 is 0 or 2, known at compile time)
+__device__ __forceinline__ void q6_bytes8(const uint8_t *row, int at, uint32_t &a, uint32_t &b) {
+    const uint32_t *p = reinterpret_cast<const uint32_t *>(row + (at & ~3));
+    if (at & 2) {
+        const uint32_t w0 = p[0], w1 = p[1], w2 = p[2];
+        a = __builtin_amdgcn_alignbit(w1, w0, 16);
+        b = __builtin_amdgcn_alignbit(w2, w1, 16);
+    } else {
+        a = p[0];
+        b = p[1];
+    }
+}
+
+__global__ __launch_bounds__(kQ6RT * 128) void mmq_q6k_kernel(const uint8_t *__restrict__ ximg, const uint8_t *__restrict__ W,
+                                                              float *__restrict__ partial, int M, int K, int N, int64_t row_bytes) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kg = lane >> 5, col = lane & 31;
+    const int rt = wave % kQ6RT, par = wave / kQ6RT;
+    const int slice = blockIdx.y, nslices = gridDim.y, mt = blockIdx.z;
+    constexpr int img_bytes = kQ6Slice * 64;
+    const int kpairs = K >> 9;                                  // pairs of a row
+    const int n0 = (blockIdx.x * kQ6RT + rt) * 32;              // first W row of this wavefront's tile
+    uint8_t *park = lds + img_bytes + wave * kQ6WaveLds;
+
+    // the slice's activation image goes straight from global memory into LDS (no registers)
+    {
+        const uint8_t *img = ximg + ((size_t)mt * nslices + slice) * img_bytes;
+        for (int i = wave; i < img_bytes / 1024; i += 2 * kQ6RT)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(img + i * 1024 + lane * 16),
+                                             (__attribute__((address_space(3))) void *)(lds + i * 1024), 16, 0, 0);
+    }
+    // This wavefront's pair of the slice (a pair beyond K re-reads the row's last one: its activations
+    // are zero in the image).  Dword lane + 64 i of the pair tile is dword d % 105 of row d / 105.
+    {
+        const uint8_t *base = W + (int64_t)min(n0, N - 1) * row_bytes + (int64_t)min(2 * slice + par, kpairs - 1) * kQ6PairBytes;
+        const int rows_left = max(N - 1 - n0, 0);
+        uint32_t v[kQ6Loads];
+#pragma unroll
+        for (int i = 0; i < kQ6Loads; i++) {
+            const int d = min(lane + 64 * i, 32 * kQ6PairDwords - 1);
+            v[i] = *reinterpret_cast<const uint32_t *>(base + (int64_t)min(d / kQ6PairDwords, rows_left) * row_bytes + (d % kQ6PairDwords) * 4);
+        }
+#pragma unroll
+        for (int i = 0; i < kQ6Loads; i++)
+            if (lane + 64 * i < 32 * kQ6PairDwords) reinterpret_cast<uint32_t *>(park)[lane + 64 * i] = v[i];
+    }
+    __syncthreads();  // image landed; the parked pair is this wavefront's own
+
+    f16v acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+    uint32_t magic;
+    asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));
+    const h2 off = as_h2(0xE420E420u);  // (-1056, -1056) = -(1024 + 32)
+    const uint8_t *myrow = park + col * kQ6PairBytes;
+#pragma unroll
+    for (int sbp = 0; sbp < 2; sbp++) {
+        const int b0 = sbp * 210;                    // byte offset of the super-block in the parked row
+        const int sbg = 2 * par + sbp;               // super-block within the slice
+        const float d = half_bits_to_float(*reinterpret_cast<const uint16_t *>(myrow + b0 + 208));
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            // the half's eight scales (int8), 2 bytes off when sbp = 1
+            uint32_t sc_lo, sc_hi;
+            q6_bytes8(myrow, b0 + 192 + 8 * h, sc_lo, sc_hi);
+#pragma unroll
+            for (int is = 0; is < 2; is++) {
+                uint32_t hq0, hq1;
+                q6_bytes8(myrow, b0 + 128 + 32 * h + 16 * is + 8 * kg, hq0, hq1);
+#pragma unroll
+                for (int e = 0; e < 2; e++) {
+                    uint32_t lq0, lq1;
+                    q6_bytes8(myrow, b0 + 64 * h + 32 * e + 16 * is + 8 * kg, lq0, lq1);
+#pragma unroll
+                    for (int nib = 0; nib < 2; nib++) {
+                        const int qd = 2 * nib + e;  // quadrant of the half: values 32 qd + 16 is + 8 kg ..
+                        const uint32_t c0 = ((lq0 >> (4 * nib)) & 0x0F0F0F0Fu) | (((hq0 >> (2 * qd)) & 0x03030303u) << 4);
+                        const uint32_t c1 = ((lq1 >> (4 * nib)) & 0x0F0F0F0Fu) | (((hq1 >> (2 * qd)) & 0x03030303u) << 4);
+                        uint4 o;  // fp16 pairs (0,2) (1,3) (4,6) (5,7) of code - 32
+                        o.x = __builtin_bit_cast(uint32_t, as_h2(__builtin_amdgcn_perm(magic, c0, 0x07020700u)) + off);
+                        o.y = __builtin_bit_cast(uint32_t, as_h2(__builtin_amdgcn_perm(magic, c0, 0x07030701u)) + off);
+                        o.z = __builtin_bit_cast(uint32_t, as_h2(__builtin_amdgcn_perm(magic, c1, 0x07020700u)) + off);
+                        o.w = __builtin_bit_cast(uint32_t, as_h2(__builtin_amdgcn_perm(magic, c1, 0x07030701u)) + off);
+                        const int oct = sbg * 32 + h * 16 + qd * 4 + is * 2 + kg;
+                        const h8 xo = *reinterpret_cast<const h8 *>(lds + (oct * kMT + col) * 16);
+                        f16v p;
+#pragma unroll
+                        for (int r = 0; r < 16; r++) p[r] = 0.f;
+                        p = __builtin_amdgcn_mfma_f32_32x32x16_f16(xo, __builtin_bit_cast(h8, o), p, 0, 0, 0);
+                        const int si = 2 * qd + is;  // scale index within the half
+                        const int sc = (int)__builtin_amdgcn_sbfe((int)(si < 4 ? sc_lo : sc_hi), 8 * (si & 3), 8);  // (the builtin's result type is unsigned)
+                        const float dsc = d * (float)sc;
+#pragma unroll
+                        for (int r = 0; r < 16; r++) acc[r] = fmaf(dsc, p[r], acc[r]);
+                    }
+                }
+            }
+        }
+    }
+
+    // the second wavefront of a row tile hands its 32 x 32 partial tile to the first through LDS
+    __syncthreads();
+    float *xch = reinterpret_cast<float *>(lds) + rt * (16 * 64);
+    if (par > 0) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) xch[r * 64 + lane] = acc[r];
+    }
+    __syncthreads();
+    const int n = n0 + col;
+    if (par == 0 && n < N) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int m = mt * kMT + 8 * (r >> 2) + 4 * kg + (r & 3);
+            if (m < M) partial[((int64_t)slice * M + m) * N + n] = acc[r] + xch[r * 64 + lane];
+        }
+    }
+}
+
+int launch_mmq_q6k(const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y,
+                   hipStream_t s) {
+    constexpr int kLds = kQ6Slice * 64 + 2 * kQ6RT * kQ6WaveLds;
+    static const bool lds_ok = [] {
+        return hipFuncSetAttribute(reinterpret_cast<const void *>(mmq_q6k_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLds) ==
+               hipSuccess;
+    }();
+    if (!lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", kLds);
+    const int mtiles = (int)((M + kMT - 1) / kMT);
+    const int nslices = (int)((K + kQ6Slice - 1) / kQ6Slice);
+    // workspace: [activation images: mtiles x nslices x 64 KiB][partial sums: nslices x M x N fp32]
+    const size_t img_bytes = (size_t)mtiles * nslices * kQ6Slice * 64;
+    const size_t part_bytes = (size_t)nslices * M * N * sizeof(float);
+    void *ws = nullptr;
+    if (int rc = stream_workspace(s, img_bytes + part_bytes, &ws)) return rc;
+    uint8_t *ximg = reinterpret_cast<uint8_t *>(ws);
+    float *partial = reinterpret_cast<float *>(ximg + img_bytes);
+    const int64_t row_bytes = (K / 256) * 210;
+    const int64_t items = (int64_t)mtiles * nslices * (kQ6Slice / 8) * 32;
+    if (int rc = x_is_bf16 ? launch(mmq_b32_xprep_kernel<true>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, x, ximg, (int)M,
+                                    (int)K, kQ6Slice, nslices)
+                           : launch(mmq_b32_xprep_kernel<false>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, x, ximg, (int)M,
+                                    (int)K, kQ6Slice, nslices))
+        return rc;
+    const dim3 grid((unsigned)((N + 32 * kQ6RT - 1) / (32 * kQ6RT)), (unsigned)nslices, (unsigned)mtiles);
+    if (int rc = launch(mmq_q6k_kernel, grid, dim3(kQ6RT * 128), (size_t)kLds, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N,
+                        row_bytes))
+        return rc;
+    const int64_t MN = M * N;
+    return launch(mmq_reduce_kernel, dim3((unsigned)((MN / 4 + 255) / 256)), dim3(256), 0, s, (const float *)partial, nslices, MN, (int)N,
+                  bias, act, y);
+}
+
 }  // namespace
 
 bool mmq_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, const void *bias, const void *y) {
@@ -543,6 +714,7 @@ bool mmq_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, con
                           ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(bias) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
     if (type == kQ4_K) return shape_ok && K % 256 == 0;
     if (type == kQ8_0 || type == kQ4_0) return shape_ok && K % 256 == 0;  // whole stretches of 8 blocks
+    if (type == kQ6_K) return shape_ok && K % 512 == 0;                   // whole, dword-aligned pairs of super-blocks
     return false;
 }
 
@@ -551,6 +723,7 @@ int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, co
     // (four row tiles per workgroup measured a little faster than two)
     if (type == kQ8_0) return launch_mmq_b32<kQ8_0, 4>(x, x_is_bf16, M, K, W, N, bias, act, y, s);
     if (type == kQ4_0) return launch_mmq_b32<kQ4_0, 4>(x, x_is_bf16, M, K, W, N, bias, act, y, s);
+    if (type == kQ6_K) return launch_mmq_q6k(x, x_is_bf16, M, K, W, N, bias, act, y, s);
     if (type != kQ4_K) return fail(GQ_ERR_NOT_IMPLEMENTED, "mmq: ggml type %d is not implemented", type);
     static const bool lds_ok = [] {
         return hipFuncSetAttribute(reinterpret_cast<const void *>(mmq_q4k_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,

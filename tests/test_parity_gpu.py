@@ -192,15 +192,18 @@ def test_split_k_small_batches_q8_q4(gpu, oracle, t, M, K, N):
     assert rel_err(run_dense(gpu, t, xb, W, bias, 0, bf16=True), oracle.c_qdense(t, xb, W, bias, 0)) < tol, (t, M, K, N, "bf16")
 
 
-@pytest.mark.parametrize("M,K,N", [(5, 256, 8), (32, 2048, 260), (70, 4096, 512), (96, 1024, 4096)])
-def test_split_k_small_batches_q4_k(gpu, oracle, M, K, N):
-    """5 .. 96 rows of Q4_K, fp32 and bf16 activations, through the split-K MFMA kernel."""
-    W = synth.weights(Q4_K, 75, N, K)
+@pytest.mark.parametrize("t", [Q4_K, Q6_K])
+@pytest.mark.parametrize("M,K,N", [(8, 512, 8), (32, 2048, 260), (70, 4096, 512), (96, 1024, 4096), (33, 1536, 100), (12, 7680, 36)])
+def test_split_k_small_batches_k_quants(gpu, oracle, t, M, K, N):
+    """Small batches of Q4_K and Q6_K, fp32 and bf16 activations, through the split-K MFMA kernels
+    (K a multiple of 512; 1536 and 7680 leave the last 1024-value slice of Q6_K half empty)."""
+    W = synth.weights(t, 75, N, K)
     x = synth.activations(76, M, K)
     bias = synth.normal(77, 0, N).astype(np.float32) * 0.1
-    assert rel_err(run_dense(gpu, Q4_K, x, W, bias, 3), oracle.c_qdense(Q4_K, x, W, bias, 3)) < TOL_F32, (M, K, N, "f32")
+    assert rel_err(run_dense(gpu, t, x, W, bias, 3), oracle.c_qdense(t, x, W, bias, 3)) < TOL_F32, (t, M, K, N, "f32")
     xb = bf16_round(x)
-    assert rel_err(run_dense(gpu, Q4_K, xb, W, bias, 3, bf16=True), oracle.c_qdense(Q4_K, xb, W, bias, 3)) < TOL_F32, (M, K, N, "bf16")
+    tol = TOL_F32 if (t == Q4_K or M <= 32) else TOL_BF16  # Q6_K beyond 32 rows takes the bf16 MFMA GEMM
+    assert rel_err(run_dense(gpu, t, xb, W, bias, 3, bf16=True), oracle.c_qdense(t, xb, W, bias, 3)) < tol, (t, M, K, N, "bf16")
 
 
 @pytest.mark.parametrize("t", ALL_TYPES)
