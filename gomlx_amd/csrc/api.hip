@@ -116,7 +116,8 @@ int check_dense_args(const char *fn, int type, const void *x, int64_t M, int64_t
 // Batch sizes served by the split-K small-batch kernels (measured crossovers against the GEMV passes
 // below and the two-pass GEMM above, K = 4096, N = 4096 .. 14336).  The Q6_K kernel pays 16 scale
 // groups per super-block and only wins for a single tile of 32 batch columns.
-int64_t split_k_from(int type) { return type == GQ_Q4_K ? 5 : type == GQ_Q6_K ? 6 : 8; }
+// (IQ4_NL has no integer-dot GEMV: its fp32 passes cost 25 us per row on 14336 x 4096, the split-K kernel 28 us.)
+int64_t split_k_from(int type) { return type == GQ_IQ4_NL ? 2 : type == GQ_Q4_K ? 5 : type == GQ_Q6_K ? 6 : 8; }
 int64_t split_k_to(int type) { return type == GQ_Q6_K ? 32 : 96; }
 
 // large batches: W dequantised once into the stream's workspace, then a plain 16-bit GEMM
@@ -286,30 +287,20 @@ int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *d
     if (int rc = check_dense_args("gq_qdense_f32", type, dX, M, K, dW, N, dBias, act, dY, 4)) return rc;
     if (M == 0 || N == 0) return GQ_OK;
     if (int rc = use_device()) return rc;
-    // Up to four activation rows: one bandwidth-bound pass over W per row, fp32 throughout.
-    // More rows: W is read once per tile of rows and contracted on the matrix cores - except that
-    // up to kGemvMaxRows rows are still cheaper as GEMV passes (later passes find most of W in the
-    // caches: measured +3 us per row on a 33 MB matrix against 85 us for the tiled kernel) when no
-    // small-batch MFMA kernel exists for the format.
-    if (M <= 4) {
-        if (gemv_ks_supported(type, K, N, dX))
-            return launch_gemv_ks(type, dX, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
-        if (gemv_xs_supported(type, K, N, dX))
-            return launch_gemv_xs(type, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
-        return launch_gemv(type, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
-    }
     // Small batches: GEMV passes cost about one third of the first pass per extra row; the split-K
     // MFMA kernels cost 19 .. 26 us (Q8_0 / Q4_0, K = 4096, N = 4096 .. 14336) for up to 32 rows and
     // 5 .. 18 us per further 32; the two passes 33 .. 62 us for anything up to 128 rows.  Measured
     // crossovers: split_k_from() / split_k_to().
     const bool tp = gemm_two_pass_supported(type, false, M, K, N, dX);
     const bool ks = M <= kGemvMaxRows && gemv_ks_supported(type, K, N, dX);
-    const int64_t mmq_from = split_k_from(type), mmq_to = split_k_to(type);
-    if (ks && M < mmq_from)
-        return launch_gemv_ks(type, dX, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
-    if (mmq_supported(type, M, K, N, dX, dBias, dY) && (M <= mmq_to || !tp))
-        return launch_mmq(type, dX, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
-    if (ks) return launch_gemv_ks(type, dX, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
+    const bool sk = M >= split_k_from(type) && mmq_supported(type, M, K, N, dX, dBias, dY) && (M <= split_k_to(type) || !tp);
+    if (ks && !sk) return launch_gemv_ks(type, dX, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
+    if (sk) return launch_mmq(type, dX, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
+    if (M <= 4) {  // shapes or formats without a K-sliced plan: one fp32 pass over W per row
+        if (gemv_xs_supported(type, K, N, dX))
+            return launch_gemv_xs(type, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
+        return launch_gemv(type, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
+    }
     if (tp) return two_pass(type, false, dX, M, K, dW, N, dBias, act, dY, (hipStream_t)stream);
     return launch_gemm(type, false, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
 }
@@ -362,12 +353,9 @@ int gq_qdense_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, const voi
     // the bf16 MFMA paths).
     const bool tp = gemm_two_pass_supported(type, true, M, K, N, dX);
     const bool ks = M <= kGemvMaxRows && gemv_ks_supported(type, K, N, dX);
-    const int64_t mmq_from = split_k_from(type), mmq_to = split_k_to(type);
-    if (ks && M < mmq_from)
-        return launch_gemv_ks(type, dX, true, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
-    if (mmq_supported(type, M, K, N, dX, dBias, dY) && (M <= mmq_to || !tp))
-        return launch_mmq(type, dX, true, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
-    if (ks) return launch_gemv_ks(type, dX, true, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
+    const bool sk = M >= split_k_from(type) && mmq_supported(type, M, K, N, dX, dBias, dY) && (M <= split_k_to(type) || !tp);
+    if (ks && !sk) return launch_gemv_ks(type, dX, true, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
+    if (sk) return launch_mmq(type, dX, true, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
     if (tp) return two_pass(type, true, dX, M, K, dW, N, dBias, act, dY, (hipStream_t)stream);
     return launch_gemm(type, true, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
 }

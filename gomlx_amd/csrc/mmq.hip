@@ -1,5 +1,5 @@
 // Small-batch (decode batch 5..~128) quantised Dense on the gfx950 matrix cores: Q4_K, and further
-// down Q8_0 / Q4_0 and Q6_K.
+// down Q8_0 / Q4_0 / IQ4_NL and Q6_K.
 //
 // At batch 32 the contraction is 228 flop per weight byte: far beyond the vector ALUs, still
 // below the MFMA machine balance, so the kernel should run at the speed the packed weights
@@ -304,7 +304,7 @@ __global__ __launch_bounds__(256) void mmq_reduce_kernel(const float *__restrict
 }
 
 
-// ---- small batches of the 32-value-block formats (Q8_0, Q4_0) --------------------------------------
+// ---- small batches of the 32-value-block formats (Q8_0, Q4_0, IQ4_NL) --------------------------------------
 //
 // Same plan as the Q4_K kernel above, simpler arithmetic: K is split in slices of S = 512 or 1024
 // values (the smaller count of slices that still gives the chip a few hundred workgroups); a
@@ -357,6 +357,31 @@ template <> struct B32<kQ4_0> {
         o.y = __builtin_bit_cast(uint32_t, magic_pair(a >> 8, 0x000F000Fu, magic) + off);  // (1, 3)
         o.z = __builtin_bit_cast(uint32_t, magic_pair(b, 0x000F000Fu, magic) + off);
         o.w = __builtin_bit_cast(uint32_t, magic_pair(b >> 8, 0x000F000Fu, magic) + off);
+        return __builtin_bit_cast(h8, o);
+    }
+};
+
+// IQ4_NL: the layout of Q4_0 with a 16-entry code book instead of nibble - 8.
+template <> struct B32<kIQ4_NL> {
+    static constexpr int kBlockBytes = 18, kWin = 3;
+    static __device__ __forceinline__ int code_byte(int kg) { return 2 + 8 * kg; }
+    static __device__ __forceinline__ int octet(int b, int kg, int j) { return 4 * b + 2 * j + kg; }
+    // four code-book entries (int8, as bytes) for the four nibble indices in the bytes of idx
+    static __device__ __forceinline__ uint32_t book(uint32_t idx) {
+        const uint32_t t0 = 0xBFAD9881u, t1 = 0xF6EADDCFu, t2 = 0x26190D01u, t3 = 0x71594535u;  // -127 .. 113, four per dword
+        const uint32_t low3 = idx & 0x07070707u;
+        const uint32_t lo = __builtin_amdgcn_perm(t1, t0, low3), hi = __builtin_amdgcn_perm(t3, t2, low3);
+        return __builtin_amdgcn_perm(hi, lo, 0x03020100u | ((idx & 0x08080808u) >> 1));  // byte i from hi when bit 3 of index i is set
+    }
+    static __device__ __forceinline__ h8 frag(const uint32_t *c, int j, uint32_t magic) {
+        const uint32_t a = book((c[0] >> (4 * j)) & 0x0F0F0F0Fu) ^ 0x80808080u;  // entry + 128, unsigned
+        const uint32_t b = book((c[1] >> (4 * j)) & 0x0F0F0F0Fu) ^ 0x80808080u;
+        const h2 off = as_h2(0xE480E480u);  // (-1152, -1152) = -(1024 + 128)
+        uint4 o;
+        o.x = __builtin_bit_cast(uint32_t, as_h2(__builtin_amdgcn_perm(magic, a, 0x07020700u)) + off);
+        o.y = __builtin_bit_cast(uint32_t, as_h2(__builtin_amdgcn_perm(magic, a, 0x07030701u)) + off);
+        o.z = __builtin_bit_cast(uint32_t, as_h2(__builtin_amdgcn_perm(magic, b, 0x07020700u)) + off);
+        o.w = __builtin_bit_cast(uint32_t, as_h2(__builtin_amdgcn_perm(magic, b, 0x07030701u)) + off);
         return __builtin_bit_cast(h8, o);
     }
 };
@@ -713,7 +738,7 @@ bool mmq_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, con
     const bool shape_ok = M >= 2 && M <= 256 && N % 4 == 0 && N <= (int64_t)INT32_MAX / 2 && K <= INT32_MAX / 2 &&
                           ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(bias) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
     if (type == kQ4_K) return shape_ok && K % 256 == 0;
-    if (type == kQ8_0 || type == kQ4_0) return shape_ok && K % 256 == 0;  // whole stretches of 8 blocks
+    if (type == kQ8_0 || type == kQ4_0 || type == kIQ4_NL) return shape_ok && K % 256 == 0;  // whole stretches of 8 blocks
     if (type == kQ6_K) return shape_ok && K % 512 == 0;                   // whole, dword-aligned pairs of super-blocks
     return false;
 }
@@ -723,6 +748,7 @@ int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, co
     // (four row tiles per workgroup measured a little faster than two)
     if (type == kQ8_0) return launch_mmq_b32<kQ8_0, 4>(x, x_is_bf16, M, K, W, N, bias, act, y, s);
     if (type == kQ4_0) return launch_mmq_b32<kQ4_0, 4>(x, x_is_bf16, M, K, W, N, bias, act, y, s);
+    if (type == kIQ4_NL) return launch_mmq_b32<kIQ4_NL, 4>(x, x_is_bf16, M, K, W, N, bias, act, y, s);
     if (type == kQ6_K) return launch_mmq_q6k(x, x_is_bf16, M, K, W, N, bias, act, y, s);
     if (type != kQ4_K) return fail(GQ_ERR_NOT_IMPLEMENTED, "mmq: ggml type %d is not implemented", type);
     static const bool lds_ok = [] {

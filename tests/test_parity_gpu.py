@@ -163,7 +163,7 @@ def test_small_batches_f32(gpu, oracle, t, M):
     assert rel_err(got, oracle.c_qdense(t, x, W, None, 0)) < TOL_F32, (t, M)
 
 
-@pytest.mark.parametrize("t", [Q4_0, Q8_0])
+@pytest.mark.parametrize("t", [Q4_0, Q8_0, IQ4_NL])
 @pytest.mark.parametrize("M,K,N", [
     (10, 256, 4),        # one stretch, three of four row tiles empty
     (16, 768, 132),      # K = one slice and a half, weight rows not a multiple of 32
@@ -176,8 +176,8 @@ def test_small_batches_f32(gpu, oracle, t, M):
     (8, 1024, 36),
 ])
 def test_split_k_small_batches_q8_q4(gpu, oracle, t, M, K, N):
-    """8 .. 96 rows of Q8_0 / Q4_0 (fp32 activations, N a multiple of 4, K of 256): the split-K MFMA
-    kernel with exact integer weight operands; x -> fp16 is its only rounding."""
+    """8 .. 96 rows of Q8_0 / Q4_0 / IQ4_NL (N a multiple of 4, K of 256): the split-K MFMA kernel
+    with exact integer weight operands; x -> fp16 is its only rounding."""
     W = synth.weights(t, 70 + t, N, K)
     x = synth.activations(71 + t, M, K)
     bias = synth.normal(72 + t, 0, N).astype(np.float32) * 0.1
