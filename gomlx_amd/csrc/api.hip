@@ -116,8 +116,7 @@ int check_dense_args(const char *fn, int type, const void *x, int64_t M, int64_t
 // Batch sizes served by the split-K small-batch kernels (measured crossovers against the GEMV passes
 // below and the two-pass GEMM above, K = 4096, N = 4096 .. 14336).  The Q6_K kernel pays 16 scale
 // groups per super-block and only wins for a single tile of 32 batch columns.
-// (IQ4_NL has no integer-dot GEMV: its fp32 passes cost 25 us per row on 14336 x 4096, the split-K kernel 28 us.)
-int64_t split_k_from(int type) { return type == GQ_IQ4_NL ? 2 : type == GQ_Q4_K ? 5 : type == GQ_Q6_K ? 6 : 8; }
+int64_t split_k_from(int type) { return type == GQ_Q4_K || type == GQ_IQ4_NL ? 5 : type == GQ_Q6_K ? 6 : 8; }
 int64_t split_k_to(int type) { return type == GQ_Q6_K ? 32 : 96; }
 
 // large batches: W dequantised once into the stream's workspace, then a plain 16-bit GEMM

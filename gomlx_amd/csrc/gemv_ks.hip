@@ -1,5 +1,5 @@
 // Decode GEMV, K-sliced integer-dot kernels with wavefront-local activation staging
-// (Q4_0, Q8_0, Q4_K, Q6_K; K % 256 == 0).
+// (Q4_0, Q8_0, Q4_K, Q6_K, IQ4_NL; K % 256 == 0).
 //
 // The activation-stationary kernel of gemv_xs.hip lets every wavefront see all of K, so its
 // workgroup has to convert the whole activation vector together and meet at a barrier before the
@@ -252,6 +252,55 @@ template <> struct KS<kQ8_0> {
             }
             const int t = (s1 << 8) + s0;
             const float d = half_bits_to_float(h == 0 ? (v[0] & 0xFFFFu) : (v[8] >> 16));
+            out = fmaf((float)t, d * xsc[h], out);
+        }
+        return out;
+    }
+};
+
+// IQ4_NL: the byte layout of Q4_0 (lane c: blocks 2c, 2c+1, 36 bytes), but the nibbles index a
+// 16-entry code book of int8 values, looked up four at a time with byte permutes; the dot products
+// then run on the two signed byte limbs like Q8_0.  Low nibbles of code dword w face values
+// 4w .. 4w+3 of the block (plane dword w), high nibbles values 16+4w .. (plane dword 4+w).
+template <> struct KS<kIQ4_NL> {
+    static constexpr int kSliceBytes = 288;
+    static constexpr int kScales = 2, kSumSpan = 0;
+    static __device__ __forceinline__ int plane_idx(int c, int i) { return 8 * c + i; }
+    static __device__ __forceinline__ int scale_idx(int c, int i) { return 2 * c + i; }
+    static __device__ __forceinline__ int sum_idx(int c, int i) { return 2 * c + i; }
+    struct __attribute__((packed, aligned(4))) Raw { uint32_t v[9]; };
+    static __device__ __forceinline__ int lane_offset(int c) { return c * 36; }
+    static __device__ __forceinline__ void load(Raw &r, const uint8_t *p) { r = *reinterpret_cast<const Raw *>(p); }
+    static __device__ __forceinline__ XPair x_load(const float *__restrict__ xs, int lane) { return limb_x_load(xs, lane); }
+    static __device__ __forceinline__ XPair x_load_bf16(const uint16_t *__restrict__ xs, int lane) { return limb_x_load_bf16(xs, lane); }
+    static __device__ __forceinline__ Staged stage(const XPair &xp) { return limb_stage(xp); }
+    // four code-book entries (int8, as bytes) for the four indices 0..15 in the bytes of idx
+    static __device__ __forceinline__ int book(uint32_t idx) {
+        const uint32_t t0 = 0xBFAD9881u, t1 = 0xF6EADDCFu, t2 = 0x26190D01u, t3 = 0x71594535u;  // -127 .. 113, four per dword
+        const uint32_t low3 = idx & 0x07070707u;
+        const uint32_t lo = __builtin_amdgcn_perm(t1, t0, low3), hi = __builtin_amdgcn_perm(t3, t2, low3);
+        return (int)__builtin_amdgcn_perm(hi, lo, 0x03020100u | ((idx & 0x08080808u) >> 1));  // byte i from hi when bit 3 of index i is set
+    }
+    static __device__ __forceinline__ float dot(const Raw &r, const uint4 *xq, const float *xsc, const float *, int) {
+        const uint32_t *v = r.v;
+        float out = 0.f;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            int s0 = 0, s1 = 0;
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                const uint32_t q = h == 0 ? __builtin_amdgcn_alignbit(v[w + 1], v[w], 16) : v[5 + w];
+                const int lo = book(q & 0x0F0F0F0Fu), hi = book((q >> 4) & 0x0F0F0F0Fu);
+                int p0, p1;
+                limb_planes(xq, h, w, p0, p1);
+                s0 = __builtin_amdgcn_sdot4(lo, p0, s0, false);
+                s1 = __builtin_amdgcn_sdot4(lo, p1, s1, false);
+                limb_planes(xq, h, 4 + w, p0, p1);
+                s0 = __builtin_amdgcn_sdot4(hi, p0, s0, false);
+                s1 = __builtin_amdgcn_sdot4(hi, p1, s1, false);
+            }
+            const int t = (s1 << 8) + s0;
+            const float d = half_bits_to_float(h == 0 ? (v[0] & 0xFFFFu) : (v[4] >> 16));
             out = fmaf((float)t, d * xsc[h], out);
         }
         return out;
@@ -646,7 +695,7 @@ int launch_ks_batch(int count, const XsBatchItem *items, hipStream_t s) {
 
 bool gemv_ks_supported(int type, int64_t K, int64_t N, const void *x) {
     if (reinterpret_cast<uintptr_t>(x) & 15) return false;
-    if (type != kQ4_0 && type != kQ8_0 && type != kQ4_K && type != kQ6_K) return false;
+    if (type != kQ4_0 && type != kQ8_0 && type != kQ4_K && type != kQ6_K && type != kIQ4_NL) return false;
     if (N <= 0 || N > (int64_t)INT32_MAX / 2) return false;
     int waves, nslices, half_tail;
     return ks_split(K, waves, nslices, half_tail);
@@ -660,6 +709,7 @@ int launch_gemv_ks(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K
     case kQ8_0: return launch_ks<kQ8_0>(x, x_bf16, M, K, W, N, bias, act, y, s);
     case kQ4_K: return launch_ks<kQ4_K>(x, x_bf16, M, K, W, N, bias, act, y, s);
     case kQ6_K: return launch_ks<kQ6_K>(x, x_bf16, M, K, W, N, bias, act, y, s);
+    case kIQ4_NL: return launch_ks<kIQ4_NL>(x, x_bf16, M, K, W, N, bias, act, y, s);
     default: return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv_ks: ggml type %d is not implemented", type);
     }
 }
@@ -671,6 +721,7 @@ int launch_gemv_ks_batch(int type, int count, const XsBatchItem *items, hipStrea
     case kQ8_0: return launch_ks_batch<kQ8_0>(count, items, s);
     case kQ4_K: return launch_ks_batch<kQ4_K>(count, items, s);
     case kQ6_K: return launch_ks_batch<kQ6_K>(count, items, s);
+    case kIQ4_NL: return launch_ks_batch<kIQ4_NL>(count, items, s);
     default: return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv batch: ggml type %d is not implemented", type);
     }
 }

@@ -112,7 +112,7 @@ def test_gemv_parity(gpu, oracle, t, M, K, N):
         assert rel_err(got, want) < TOL_F32, (t, M, K, N, act)
 
 
-@pytest.mark.parametrize("t", [Q4_0, Q8_0, Q4_K, Q6_K])
+@pytest.mark.parametrize("t", [Q4_0, Q8_0, Q4_K, Q6_K, IQ4_NL])
 @pytest.mark.parametrize("M,K,N", [
     (1, 1536, 100),     # 3 slices of 512: three wavefronts per workgroup
     (2, 3584, 513),     # 7 slices, rows not a multiple of 8
@@ -139,7 +139,7 @@ def test_gemv_k_sliced_plans(gpu, oracle, t, M, K, N):
     assert rel_err(got, want) < TOL_F32, (t, M, K, N)
 
 
-@pytest.mark.parametrize("t", [Q4_0, Q8_0, Q4_K, Q6_K])
+@pytest.mark.parametrize("t", [Q4_0, Q8_0, Q4_K, Q6_K, IQ4_NL])
 @pytest.mark.parametrize("M,K,N", [(1, 4096, 300), (3, 1024, 257), (16, 2048, 130)])
 def test_bf16_decode_batches_are_exact_widenings(gpu, oracle, t, M, K, N):
     """bf16 activations of a decode batch run through the fp32 GEMV (bf16 -> fp32 is exact), so
