@@ -593,7 +593,9 @@ __device__ __forceinline__ void q6_bytes8(const uint8_t *row, int at, uint32_t &
     }
 }
 
-__global__ __launch_bounds__(kQ6RT * 128) void mmq_q6k_kernel(const uint8_t *__restrict__ ximg, const uint8_t *__restrict__ W,
+// (Launched with kQ6RT * 128 threads.  Declared for up to 512: with a bound of 256 the compiler puts every MFMA
+// result into accumulation registers and copies it back out, 16 extra instructions per MFMA.)
+__global__ __launch_bounds__(512) void mmq_q6k_kernel(const uint8_t *__restrict__ ximg, const uint8_t *__restrict__ W,
                                                               float *__restrict__ partial, int M, int K, int N, int64_t row_bytes) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
