@@ -40,11 +40,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # pattern, not of a particular run, and are re-measured whenever a kernel changes.
 _KIB, _FETCH_SCALE, _WRITE_SCALE = 1024, 65536.0 / 32780.6, 1.0
 COUNTER_KIB = {  # workload -> (FETCH_SIZE, WRITE_SIZE) raw counter KiB per step
-    "c0": (8804.6, 16.0),
-    "c1": (16256.7, 56.0),
-    "c2": (19871.0 + 1822.1 + 911.5, 3584.0 + 512.0 + 924.0),
-    "c3": (74724.6, 32768.0),
-    "c4": (60616.3, 168.0),
+    "c0": (8812.0, 16.0),
+    "c1": (16276.3, 56.0),
+    "c2": (19875.0 + 1833.6 + 911.6, 3584.0 + 512.0 + 924.0),
+    "c3": (74726.7, 32768.0),
+    "c4": (60539.5, 168.0),
 }
 
 
