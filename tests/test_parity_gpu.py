@@ -393,6 +393,37 @@ def test_dispatch_boundaries(gpu, oracle, t, M, K, N, bf16, act, with_bias):
     assert err < (TOL_BF16 if bf16 else TOL_F32), (t, M, K, N, bf16, act, err)
 
 
+def test_randomized_problems(gpu, oracle):
+    """150 seeded random problems over all formats, both activation types, every activation, with
+    and without bias: batch sizes, K and N drawn from lists that include every tile and slice
+    boundary of the kernels.  Error measured on the contraction scale as above."""
+    rng = np.random.default_rng(7)
+    rows = [1, 2, 3, 4, 5, 6, 7, 8, 9, 12, 16, 17, 24, 32, 33, 48, 64, 65, 96, 97, 100, 128, 130, 200, 256, 257, 300, 512, 700, 1024]
+    done = 0
+    while done < 150:
+        t = ALL_TYPES[int(rng.integers(0, len(ALL_TYPES)))]
+        big = t in (Q4_K, Q6_K)
+        M = int(rng.choice(rows))
+        K = (256 if big else 32) * int(rng.choice([1, 2, 3, 4, 5, 6, 7, 8, 9, 12, 16, 17, 20] if big else
+                                                 [1, 2, 3, 5, 8, 9, 16, 17, 24, 32, 33, 48, 64, 96, 128, 136]))
+        N = int(rng.choice([1, 3, 4, 8, 31, 32, 33, 64, 100, 128, 129, 200, 256, 300, 512, 777, 1024]))
+        bf16, act, with_bias = bool(rng.integers(0, 2)), int(rng.integers(0, 6)), bool(rng.integers(0, 2))
+        if M * K * N > 3e8:
+            continue
+        done += 1
+        W = synth.weights(t, 5000 + done, N, K)
+        x = synth.activations(6000 + done, M, K)
+        bias = synth.normal(7000 + done, 0, N).astype(np.float32) * 0.1 if with_bias else None
+        if bf16:
+            x = bf16_round(x)
+        got = run_dense(gpu, t, x, W, bias, act, bf16=bf16)
+        want = oracle.c_qdense(t, x, W, bias, act)
+        pre = oracle.c_qdense(t, x, W, bias, 0)
+        scale = max(float(np.max(np.abs(want))), float(np.max(np.abs(pre)))) or 1.0
+        err = float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)))) / scale
+        assert np.all(np.isfinite(got)) and err < (TOL_BF16 if bf16 else TOL_F32), (t, M, K, N, bf16, act, with_bias, err)
+
+
 # ------------------------------------------------------------------------------ benchmark configurations, full size
 
 def test_config0_q8_0_gemv_4096(gpu, oracle):
