@@ -3,6 +3,9 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1] [--others]
 
+--config takes c0 .. c4 (the BASELINE.json configurations) or ffn (the gated feed-forward front
+of a decoder layer: the callers around the two projections folded into one launch).
+
 A "step" is one quantized Dense call (one pass over one weight matrix) on synthetic data that
 is already resident in HBM.  The headline workload is BASELINE.json configs[1]: Q4_0 decode
 GEMV, batch 1, K=4096 -> N=14336.  Steps rotate over enough distinct weight copies (> 512 MB)
@@ -49,6 +52,8 @@ COUNTER_KIB = {  # workload -> (FETCH_SIZE, WRITE_SIZE) raw counter KiB per step
 
 
 def measured_traffic(name):
+    if name not in COUNTER_KIB:
+        return None
     f, w = COUNTER_KIB[name]
     return int(round((f * _FETCH_SCALE + w * _WRITE_SCALE) * _KIB))
 
@@ -67,6 +72,7 @@ WORKLOAD_TEXT = {
     "c2": "configs[2]: Q4_K dense, decode batch M=32, K=14336 -> N=4096",
     "c3": "configs[3]: Q8_0 prefill GEMM, M=2048 bf16, K=4096, N=4096",
     "c4": "configs[4]: seven Q4_K projections of a Llama-3-8B layer, batch 1",
+    "ffn": "gated feed-forward front of a Llama-3-8B layer, batch 1: RMSNorm, Q4_K gate and up 4096 -> 14336, SiLU(gate) * up, one launch",
 }
 
 
@@ -75,7 +81,7 @@ def parse_args():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=200)
     p.add_argument("--warmup", type=int, default=20)
-    p.add_argument("--config", default="c1", choices=sorted(list(CONFIGS) + ["c4"]))
+    p.add_argument("--config", default="c1", choices=sorted(list(CONFIGS) + ["c4", "ffn"]))
     p.add_argument("--others", action="store_true", help="also measure the other configurations (reported under 'others')")
     p.add_argument("--no-graph", action="store_true", help="submit the timed steps one call at a time")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
@@ -98,11 +104,15 @@ class Problem:
         if name == "c4":
             shapes = [("Q4_K", 1, K, N) for K, N in C4_SHAPES]
             self.dtype, self.bound = "f32", "hbm"
+        elif name == "ffn":  # gate and up matrices of one feed-forward block
+            shapes = [("Q4_K", 1, 4096, 14336)] * 2
+            self.dtype, self.bound = "f32", "hbm"
+            self.gain = torch.from_numpy((synth.normal(1200, 0, 4096) * 0.5 + 1.0).astype(np.float32)).cuda()
         else:
             tn, M, K, N, self.dtype, self.bound = CONFIGS[name]
             shapes = [(tn, M, K, N)]
         self.parts = []
-        seed = 1000 + int(name[1])
+        seed = 1000 + (int(name[1]) if name != "ffn" else 5)
         total_w = 0
         for i, (tn, M, K, N) in enumerate(shapes):
             t = getattr(ggml, tn)
@@ -135,6 +145,13 @@ class Problem:
                 d.type, d.act, d.dX, d.M, d.K = p["t"], 0, p["x"].data_ptr(), p["M"], p["K"]
                 d.dW, d.N, d.dBias, d.dY = p["W"][c].data_ptr(), p["N"], None, p["y"].data_ptr()
             self.check(self.L.gq_qdense_f32_batch(len(self.parts), descs, self.stream))
+            return
+        if self.name == "ffn":
+            from gomlx_amd import _lib
+            g, u = self.parts
+            norm = _lib.RmsNormDesc(self.gain.data_ptr(), 1e-5, 0.0)
+            self.check(self.L.gq_qdense_gated_f32(g["t"], g["x"].data_ptr(), 1, g["K"], ctypes.byref(norm), g["W"][c].data_ptr(), None,
+                                                  u["W"][c].data_ptr(), None, g["N"], 3, g["y"].data_ptr(), self.stream))
             return
         for p in self.parts:
             fn = self.L.gq_qdense_bf16 if self.dtype == "bf16" else self.L.gq_qdense_f32
@@ -218,6 +235,8 @@ def cpu_baseline(name):
     cores = min(os.cpu_count() or 1, 16)
     if name == "c4":
         shapes = [("Q4_K", 1, K, N) for K, N in C4_SHAPES]
+    elif name == "ffn":  # the two projections; the normalisation and the product are negligible beside them
+        shapes = [("Q4_K", 1, 4096, 14336)] * 2
     else:
         tn, M, K, N, _, _ = CONFIGS[name]
         shapes = [(tn, M, K, N)]
@@ -293,7 +312,7 @@ def main():
         return rep
 
     rep = measure(args.config)
-    tn = "Q4_K" if args.config == "c4" else CONFIGS[args.config][0]
+    tn = "Q4_K" if args.config in ("c4", "ffn") else CONFIGS[args.config][0]
     line = {
         "metric": rep["metric"], "value": rep["value"], "unit": rep["unit"], "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": rep["ms_per_step"],
@@ -310,7 +329,7 @@ def main():
         line["cpu_baseline"] = cpu_baseline(args.config)
     if args.others:
         others = {}
-        for name in ["c0", "c1", "c2", "c3", "c4"]:
+        for name in ["c0", "c1", "c2", "c3", "c4", "ffn"]:
             if name == args.config:
                 continue
             steps = args.steps if name != "c3" else max(10, args.steps // 10)

@@ -37,6 +37,9 @@ SIGNATURES = [
     ("gq_qdense_f32", _int, [_int, _vp, _i64, _i64, _vp, _i64, _vp, _int, _vp, _vp]),
     ("gq_qdense_f32_batch", _int, [_int, _vp, _vp]),
     ("gq_qdense_bf16", _int, [_int, _vp, _i64, _i64, _vp, _i64, _vp, _int, _vp, _vp]),
+    ("gq_rmsnorm_f32", _int, [_vp, _i64, _i64, _vp, ctypes.c_float, ctypes.c_float, _vp, _vp]),
+    ("gq_qdense_norm_f32", _int, [_int, _vp, _i64, _i64, _vp, _vp, _i64, _vp, _int, _vp, _vp]),
+    ("gq_qdense_gated_f32", _int, [_int, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _int, _vp, _vp]),
     ("gq_embedding_lookup", _int, [_int, _vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp]),
     ("gq_graph_begin", _int, [_vp]),
     ("gq_graph_end", _int, [_vp, ctypes.POINTER(_vp)]),
@@ -52,6 +55,11 @@ class DenseDesc(ctypes.Structure):
     """gq_dense_desc of include/gomlx_hipq.h."""
     _fields_ = [("type", _int), ("act", _int), ("dX", _vp), ("M", _i64), ("K", _i64), ("dW", _vp), ("N", _i64),
                 ("dBias", _vp), ("dY", _vp)]
+
+
+class RmsNormDesc(ctypes.Structure):
+    """gq_rmsnorm of include/gomlx_hipq.h."""
+    _fields_ = [("dGain", _vp), ("eps", ctypes.c_float), ("gain_offset", ctypes.c_float)]
 
 
 class HipqError(RuntimeError):

@@ -20,7 +20,7 @@ LIB = os.path.join(HERE, "libgomlx_hipq.so")
 HOST = os.path.join(HERE, "host")
 HOST_TEST = os.path.join(HOST, "build", "hipq_backend_test")
 
-SOURCES = ["api.hip", "dequant.hip", "gemv.hip", "gemv_xs.hip", "gemv_ks.hip", "mmq.hip", "gemm.hip", "gemm_dma.hip"]
+SOURCES = ["api.hip", "dequant.hip", "gemv.hip", "gemv_xs.hip", "gemv_ks.hip", "mlp.hip", "mmq.hip", "gemm.hip", "gemm_dma.hip"]
 
 # -packed-fp32-ops (note the minus): keep hipcc from forming v_pk_*_f32 instructions.
 # -ffp-contract=off: dequantisation must round every fp32 operation on its own; fused

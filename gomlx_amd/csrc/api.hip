@@ -49,12 +49,12 @@ int device_cu_count() { return g_cu_count.load(std::memory_order_relaxed); }
 namespace {
 struct Workspace { void *ptr = nullptr; size_t bytes = 0; };
 std::mutex g_ws_mutex;
-std::map<hipStream_t, Workspace> g_ws;
+std::map<std::pair<hipStream_t, int>, Workspace> g_ws;
 }  // namespace
 
-int stream_workspace(hipStream_t s, size_t bytes, void **out) {
+int stream_workspace(hipStream_t s, size_t bytes, void **out, int slot) {
     std::lock_guard<std::mutex> lock(g_ws_mutex);
-    Workspace &w = g_ws[s];
+    Workspace &w = g_ws[std::make_pair(s, slot)];
     if (w.bytes < bytes) {
         hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
         if (s != nullptr && hipStreamIsCapturing(s, &st) == hipSuccess && st != hipStreamCaptureStatusNone)
@@ -357,6 +357,66 @@ int gq_qdense_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, const voi
     if (sk) return launch_mmq(type, dX, true, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
     if (tp) return two_pass(type, true, dX, M, K, dW, N, dBias, act, dY, (hipStream_t)stream);
     return launch_gemm(type, true, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
+}
+
+int gq_rmsnorm_f32(const float *dX, int64_t M, int64_t K, const float *dGain, float eps, float gain_offset, float *dY, void *stream) {
+    if (M < 0 || K <= 0 || K > INT32_MAX) return fail(GQ_ERR_INVALID, "gq_rmsnorm_f32: bad shape [%lld, %lld]", (long long)M, (long long)K);
+    if (!(eps >= 0.f)) return fail(GQ_ERR_INVALID, "gq_rmsnorm_f32: epsilon must be >= 0");
+    if (M == 0) return GQ_OK;
+    if (M > INT32_MAX) return fail(GQ_ERR_NOT_IMPLEMENTED, "gq_rmsnorm_f32: more than 2^31 - 1 rows");
+    if (!dX || !dY) return fail(GQ_ERR_INVALID, "gq_rmsnorm_f32: null device pointer");
+    if (!aligned_to(dX, 4) || !aligned_to(dY, 4) || (dGain && !aligned_to(dGain, 4)))
+        return fail(GQ_ERR_INVALID, "gq_rmsnorm_f32: pointers must be 4-byte aligned");
+    if (int rc = use_device()) return rc;
+    return launch_rmsnorm(dX, M, K, dGain, gain_offset, eps, dY, (hipStream_t)stream);
+}
+
+int gq_qdense_norm_f32(int type, const float *dX, int64_t M, int64_t K, const gq_rmsnorm *norm, const void *dW, int64_t N,
+                       const float *dBias, int act, float *dY, void *stream) {
+    if (!norm) return gq_qdense_f32(type, dX, M, K, dW, N, dBias, act, dY, stream);
+    if (int rc = check_dense_args("gq_qdense_norm_f32", type, dX, M, K, dW, N, dBias, act, dY, 4)) return rc;
+    if (!(norm->eps >= 0.f)) return fail(GQ_ERR_INVALID, "gq_qdense_norm_f32: epsilon must be >= 0");
+    if (norm->dGain && !aligned_to(norm->dGain, 4)) return fail(GQ_ERR_INVALID, "gq_qdense_norm_f32: gain must be 4-byte aligned");
+    if (M == 0 || N == 0) return GQ_OK;
+    if (int rc = use_device()) return rc;
+    const RmsNorm rn{norm->dGain, norm->eps, norm->gain_offset};
+    if (gemv_ks_ext_supported(type, M, K, N, dX, rn.gain))
+        return launch_gemv_ks_ext(type, dX, M, K, &rn, (const uint8_t *)dW, dBias, nullptr, nullptr, N, act, dY, (hipStream_t)stream);
+    // composed: normalised activations into the stream's second workspace, then the dense call
+    void *ws = nullptr;
+    if (int rc = stream_workspace((hipStream_t)stream, (size_t)M * (size_t)K * sizeof(float), &ws, 1)) return rc;
+    float *xn = static_cast<float *>(ws);
+    if (int rc = launch_rmsnorm(dX, M, K, rn.gain, rn.gain_offset, rn.eps, xn, (hipStream_t)stream)) return rc;
+    return gq_qdense_f32(type, xn, M, K, dW, N, dBias, act, dY, stream);
+}
+
+int gq_qdense_gated_f32(int type, const float *dX, int64_t M, int64_t K, const gq_rmsnorm *norm, const void *dWgate,
+                        const float *dBiasGate, const void *dWup, const float *dBiasUp, int64_t N, int act, float *dY, void *stream) {
+    if (int rc = check_dense_args("gq_qdense_gated_f32", type, dX, M, K, dWgate, N, dBiasGate, act, dY, 4)) return rc;
+    if (int rc = check_dense_args("gq_qdense_gated_f32", type, dX, M, K, dWup, N, dBiasUp, act, dY, 4)) return rc;
+    if (norm && !(norm->eps >= 0.f)) return fail(GQ_ERR_INVALID, "gq_qdense_gated_f32: epsilon must be >= 0");
+    if (norm && norm->dGain && !aligned_to(norm->dGain, 4)) return fail(GQ_ERR_INVALID, "gq_qdense_gated_f32: gain must be 4-byte aligned");
+    if (M == 0 || N == 0) return GQ_OK;
+    if (int rc = use_device()) return rc;
+    RmsNorm rn{nullptr, 0.f, 0.f};
+    if (norm) rn = RmsNorm{norm->dGain, norm->eps, norm->gain_offset};
+    if (gemv_ks_ext_supported(type, M, K, N, dX, rn.gain))
+        return launch_gemv_ks_ext(type, dX, M, K, norm ? &rn : nullptr, (const uint8_t *)dWgate, dBiasGate, (const uint8_t *)dWup, dBiasUp, N,
+                                  act, dY, (hipStream_t)stream);
+    // composed: [normalised activations,] act(gate) into the stream's second workspace, up into y, y *= act(gate)
+    const size_t xn_bytes = norm ? ((size_t)M * (size_t)K * sizeof(float) + 255) / 256 * 256 : 0;
+    void *ws = nullptr;
+    if (int rc = stream_workspace((hipStream_t)stream, xn_bytes + (size_t)M * (size_t)N * sizeof(float), &ws, 1)) return rc;
+    const float *x = dX;
+    if (norm) {
+        float *xn = static_cast<float *>(ws);
+        if (int rc = launch_rmsnorm(dX, M, K, rn.gain, rn.gain_offset, rn.eps, xn, (hipStream_t)stream)) return rc;
+        x = xn;
+    }
+    float *gate = reinterpret_cast<float *>(static_cast<uint8_t *>(ws) + xn_bytes);
+    if (int rc = gq_qdense_f32(type, x, M, K, dWgate, N, dBiasGate, act, gate, stream)) return rc;
+    if (int rc = gq_qdense_f32(type, x, M, K, dWup, N, dBiasUp, GQ_ACT_NONE, dY, stream)) return rc;
+    return launch_mul_inplace(dY, gate, M * N, (hipStream_t)stream);
 }
 
 int gq_embedding_lookup(int type, const void *dTable, int64_t vocab, int64_t K, const int32_t *dIndices,

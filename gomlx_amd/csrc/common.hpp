@@ -32,7 +32,8 @@ int use_device();
 int device_cu_count();
 
 // ---- per-stream scratch memory (grows on demand; must exist before a graph recording uses it) ----
-int stream_workspace(hipStream_t s, size_t bytes, void **out);
+// Slot 0 belongs to the dense kernels, slot 1 to the operations composed of several dense calls.
+int stream_workspace(hipStream_t s, size_t bytes, void **out, int slot = 0);
 
 // ---- launch ---------------------------------------------------------------------------
 struct ProfileState {
@@ -75,6 +76,15 @@ int launch_gemv_ks(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K
 bool mmq_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, const void *bias, const void *y);
 int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias,
                int act, float *y, hipStream_t s);
+// RMS normalisation in front of a projection: x / sqrt(mean(x^2) + eps) * (gain + gain_offset); gain may be null.
+struct RmsNorm { const float *gain; float eps, gain_offset; };
+// The K-sliced GEMV with the normalisation folded in and, when W2 is given, the gated product
+// act(x.W + bias) * (x.W2 + bias2); fp32 activations, at most 16 rows.
+bool gemv_ks_ext_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, const void *gain);
+int launch_gemv_ks_ext(int type, const float *x, int64_t M, int64_t K, const RmsNorm *norm, const uint8_t *W, const float *bias,
+                       const uint8_t *W2, const float *bias2, int64_t N, int act, float *y, hipStream_t s);
+int launch_rmsnorm(const float *x, int64_t M, int64_t K, const float *gain, float gain_offset, float eps, float *y, hipStream_t s);
+int launch_mul_inplace(float *y, const float *g, int64_t n, hipStream_t s);
 struct XsBatchItem { const float *x; const uint8_t *W; const float *bias; float *y; int64_t K, N; int act; };
 int launch_gemv_xs_batch(int type, int count, const XsBatchItem *items, hipStream_t s);
 int launch_gemv_ks_batch(int type, int count, const XsBatchItem *items, hipStream_t s);

@@ -1,557 +1,19 @@
-// Decode GEMV, K-sliced integer-dot kernels with wavefront-local activation staging
-// (Q4_0, Q8_0, Q4_K, Q6_K, IQ4_NL; K % 256 == 0).
-//
-// The activation-stationary kernel of gemv_xs.hip lets every wavefront see all of K, so its
-// workgroup has to convert the whole activation vector together and meet at a barrier before the
-// first code byte can be used; on a 5-10 us kernel that prologue is a quarter of the run time.
-// Here a wavefront owns one 512-value slice of K (16 blocks of 32) instead: its 64 lanes convert
-// 8 activations each, exchange the fixed-point planes through a private piece of LDS (no
-// barrier: LDS operations of one wavefront execute in order) and start on the codes as soon as
-// their own 2 KB of x have arrived.  The wavefronts of a workgroup cover the slices of the same
-// rows (slice w, w + waves, ...: one more for the first few when the count does not divide; a last
-// half slice when K is an odd multiple of 256 runs with zero activations for its missing half) and
-// add their partial sums in LDS once, at the very end.
-//
-// Lane l = 8 * rg + c works on row (8 * it + rg) of the workgroup and on 64 values of the slice:
-//   Q4_0: blocks 2c, 2c+1: 36 bytes at a 4-byte-aligned address;
-//   Q8_0: blocks 2c, 2c+1: 68 bytes at a 4-byte-aligned address;
-//   Q4_K: super-block c / 4 of the slice, 64-value group c % 4: the 16-byte header and 32 code bytes;
-//   Q6_K: super-block c / 4, half (c / 2) % 2, and of each of the half's four 32-value quadrants
-//         the 16 values (c % 2) * 16 ..: 16 + 16 bytes of low nibbles, 16 bytes of high bit pairs,
-//         the half's 8 scales and d.
-// A load instruction therefore covers 8 rows x one contiguous slice (288, 544 or 420 bytes).
-//
-// Activation fixed point: 16 bits per 32 values.  Q4_0 uses four balanced base-16 digits (digit
-// planes in the nibble order of a weight dword, one v_dot8_i32_i4 per plane); Q8_0 and Q4_K use
-// two signed base-256 limbs (one v_dot4_i32_i8 per limb).  The rounding is at most 2^-16 of the
-// 32 values' largest magnitude per element; over K = 4096 random terms that is a relative output
-// error of a few 1e-5, well inside the 1e-3 bound of this path.
-#include "blocks.hpp"
-#include "common.hpp"
-
-#include <cstdlib>
+// Decode GEMV, K-sliced integer-dot kernels (Q4_0, Q8_0, Q4_K, Q6_K, IQ4_NL; K % 256 == 0): the
+// kernels and launchers of the plain dense call and of batched submission.  The work of a
+// workgroup is in gemv_ks_body.hpp.
+#include "gemv_ks_body.hpp"
 
 namespace gq {
 
 namespace {
 
-constexpr float kQmax4 = 30500.0f;                   // |q| <= 30583 fits four balanced hex digits
-constexpr float kMagic4 = 12582912.0f + 34952.0f;    // 1.5 * 2^23 + 0x8888
-constexpr float kQmaxL = 32500.0f;                   // |q| <= 32639 fits two balanced base-256 limbs
-constexpr float kMagicL = 12582912.0f + 32896.0f;    // 1.5 * 2^23 + 0x8080
-constexpr int kSliceValues = 512;
-constexpr int kMaxItersKs = 64;                      // rows per workgroup <= 512
-
-__device__ __forceinline__ float ks_quad_max(float v) {
-    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true)));
-    v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true)));
-    return v;
-}
-// sum over the 8 lanes of an aligned group of 8 (every lane ends up with the total)
-__device__ __forceinline__ float ks_oct_sum(float v) {
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // row_half_mirror
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
-    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
-    return v;
-}
-
-// sum over the 4 lanes of a quad (integer)
-__device__ __forceinline__ int ks_quad_sum(int v) {
-    v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, true);
-    v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, true);
-    return v;
-}
-
-struct XPair { float4 lo, hi; };
-
-// bf16 -> fp32 is a shift; two values per dword
-__device__ __forceinline__ float bf16_lo(uint32_t u) { return __builtin_bit_cast(float, u << 16); }
-__device__ __forceinline__ float bf16_hi(uint32_t u) { return __builtin_bit_cast(float, u & 0xFFFF0000u); }
-
-// Scale of 32 activations for a fixed-point range of +-qmax.  All-zero groups quantise to zero; a
-// non-finite group poisons its scale so that the affected outputs come out as NaN.
-__device__ __forceinline__ void ks_scale(const float *e, float qmax, float &inv, float &scale) {
-    float amax = 0.f;
-    bool nan = false;
-#pragma unroll
-    for (int p = 0; p < 8; p++) { amax = fmaxf(amax, fabsf(e[p])); nan |= e[p] != e[p]; }
-    if (nan) amax = __builtin_inff();  // fmaxf would drop a NaN in the cross-lane maximum
-    amax = ks_quad_max(amax);          // the four lanes that hold 32 consecutive values form a quad
-    if (!(amax >= 0x1p-100f)) { inv = 0.f; scale = 0.f; }
-    else if (amax > 3.0e38f) { inv = 0.f; scale = __builtin_nanf(""); }
-    else { inv = qmax / amax; scale = amax / qmax; }
-}
-
-// What a lane publishes for the 8 activations it converts: four plane dwords, the scale of their
-// 32-value group and (limb formats) scale * sum of the group's fixed-point values.
-struct Staged { uint4 planes; float scale, sum; };
-
-// ---- per-format traits -----------------------------------------------------------------------------
-template <int T> struct KS;
-
-template <> struct KS<kQ4_0> {
-    static constexpr int kSliceBytes = 288;
-    // where a lane finds what it needs of the staged slice: plane vector i (0..7), scale i, sum i
-    static constexpr int kScales = 2, kSumSpan = 0;
-    static __device__ __forceinline__ int plane_idx(int c, int i) { return 8 * c + i; }
-    static __device__ __forceinline__ int scale_idx(int c, int i) { return 2 * c + i; }
-    static __device__ __forceinline__ int sum_idx(int c, int i) { return 2 * c + i; }
-    struct __attribute__((packed, aligned(4))) Raw { uint32_t v[9]; };
-    static __device__ __forceinline__ int lane_offset(int c) { return c * 36; }
-    static __device__ __forceinline__ void load(Raw &r, const uint8_t *p) { r = *reinterpret_cast<const Raw *>(p); }
-    // the 8 activations that face weight dword (lane & 3) of block (lane >> 2) of the slice
-    static __device__ __forceinline__ XPair x_load(const float *__restrict__ xs, int lane) {
-        const float4 *x4 = reinterpret_cast<const float4 *>(xs) + (lane >> 2) * 8 + (lane & 3);
-        XPair p;
-        p.lo = x4[0];  // values 4w .. 4w+3 of the block (low nibbles of code bytes 4w .. 4w+3)
-        p.hi = x4[4];  // values 16+4w .. (high nibbles)
-        return p;
-    }
-    static __device__ __forceinline__ XPair x_load_bf16(const uint16_t *__restrict__ xs, int lane) {
-        const uint2 *x2 = reinterpret_cast<const uint2 *>(xs) + (lane >> 2) * 8 + (lane & 3);
-        const uint2 a = x2[0], b = x2[4];
-        XPair p;
-        p.lo = make_float4(bf16_lo(a.x), bf16_hi(a.x), bf16_lo(a.y), bf16_hi(a.y));
-        p.hi = make_float4(bf16_lo(b.x), bf16_hi(b.x), bf16_lo(b.y), bf16_hi(b.y));
-        return p;
-    }
-    // nibble p of plane d = digit d of the activation facing nibble p of the weight dword
-    static __device__ __forceinline__ Staged stage(const XPair &xp) {
-        const float e[8] = {xp.lo.x, xp.hi.x, xp.lo.y, xp.hi.y, xp.lo.z, xp.hi.z, xp.lo.w, xp.hi.w};  // nibble order
-        Staged st;
-        float inv;
-        ks_scale(e, kQmax4, inv, st.scale);
-        st.sum = 0.f;
-        uint32_t z[8];
-#pragma unroll
-        for (int p = 0; p < 8; p++) z[p] = __builtin_bit_cast(uint32_t, fmaf(e[p], inv, kMagic4));  // low 16 bits: q + 0x8888
-        // byte 0 of z = digits 0,1; byte 1 = digits 2,3.  Gather the bytes of the even and of the
-        // odd nibble positions, then interleave nibbles.
-        const uint32_t ga = __builtin_amdgcn_perm(z[2], z[0], 0x05010400u), gb = __builtin_amdgcn_perm(z[6], z[4], 0x05010400u);
-        const uint32_t gc = __builtin_amdgcn_perm(z[3], z[1], 0x05010400u), gd = __builtin_amdgcn_perm(z[7], z[5], 0x05010400u);
-        const uint32_t e0 = __builtin_amdgcn_perm(gb, ga, 0x05040100u) ^ 0x88888888u, e1 = __builtin_amdgcn_perm(gb, ga, 0x07060302u) ^ 0x88888888u;
-        const uint32_t o0 = __builtin_amdgcn_perm(gd, gc, 0x05040100u) ^ 0x88888888u, o1 = __builtin_amdgcn_perm(gd, gc, 0x07060302u) ^ 0x88888888u;
-        constexpr uint32_t m = 0x0F0F0F0Fu;
-        st.planes.x = (e0 & m) | ((o0 & m) << 4);
-        st.planes.y = ((e0 >> 4) & m) | (o0 & ~m);
-        st.planes.z = (e1 & m) | ((o1 & m) << 4);
-        st.planes.w = ((e1 >> 4) & m) | (o1 & ~m);
-        return st;
-    }
-    // xq[4 h + w] = planes facing dword w of block h
-    static __device__ __forceinline__ float dot(const Raw &r, const uint4 *xq, const float *xsc, const float *, int) {
-        const uint32_t *v = r.v;
-#ifdef GQ_KS_NODOT  // tuning builds only: consume the loads without the arithmetic
-        { uint32_t a = xq[0].x; for (int i = 0; i < 9; i++) a ^= v[i]; return __builtin_bit_cast(float, a) * xsc[0]; }
-#endif
-        float out = 0.f;
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-            int s0 = 0, s1 = 0, s2 = 0, s3 = 0;
-#pragma unroll
-            for (int w = 0; w < 4; w++) {
-                const int q = (int)((h == 0 ? __builtin_amdgcn_alignbit(v[w + 1], v[w], 16) : v[5 + w]) ^ 0x88888888u);
-                const uint4 &pl = xq[h * 4 + w];
-                s0 = __builtin_amdgcn_sdot8(q, (int)pl.x, s0, false);
-                s1 = __builtin_amdgcn_sdot8(q, (int)pl.y, s1, false);
-                s2 = __builtin_amdgcn_sdot8(q, (int)pl.z, s2, false);
-                s3 = __builtin_amdgcn_sdot8(q, (int)pl.w, s3, false);
-            }
-            uint32_t t = (uint32_t)s3;
-            t = (t << 4) + (uint32_t)s2;  // v_lshl_add_u32
-            t = (t << 4) + (uint32_t)s1;
-            t = (t << 4) + (uint32_t)s0;
-            const float d = half_bits_to_float(h == 0 ? (v[0] & 0xFFFFu) : (v[4] >> 16));
-            out = fmaf((float)(int)t, d * xsc[h], out);
-        }
-        return out;
-    }
-};
-
-// Q8_0 and Q4_K: lane l converts activations 8l .. 8l+7 of the slice, i.e. the values facing dwords
-// 2j, 2j+1 (j = l & 3) of 32-value group l >> 2.  planes = {limb0, limb1 of dword 2j, limb0, limb1 of
-// dword 2j+1}, byte i of a plane = limb of value 4 * dword + i.
-__device__ __forceinline__ XPair limb_x_load(const float *__restrict__ xs, int lane) {
-    const float4 *x4 = reinterpret_cast<const float4 *>(xs) + 2 * lane;
-    XPair p;
-    p.lo = x4[0];
-    p.hi = x4[1];
-    return p;
-}
-__device__ __forceinline__ XPair limb_x_load_bf16(const uint16_t *__restrict__ xs, int lane) {
-    const uint4 a = reinterpret_cast<const uint4 *>(xs)[lane];
-    XPair p;
-    p.lo = make_float4(bf16_lo(a.x), bf16_hi(a.x), bf16_lo(a.y), bf16_hi(a.y));
-    p.hi = make_float4(bf16_lo(a.z), bf16_hi(a.z), bf16_lo(a.w), bf16_hi(a.w));
-    return p;
-}
-// SUM16: the published sum covers the 16 values of a lane pair and is pre-multiplied by -32 (the
-// offset of a Q6_K code); otherwise it covers the 32 values of the quad.
-template <bool SUM16 = false>
-__device__ __forceinline__ Staged limb_stage(const XPair &xp) {
-    const float e[8] = {xp.lo.x, xp.lo.y, xp.lo.z, xp.lo.w, xp.hi.x, xp.hi.y, xp.hi.z, xp.hi.w};
-    Staged st;
-    float inv;
-    ks_scale(e, kQmaxL, inv, st.scale);
-    uint32_t z[8];
-    int xsum = 0;
-#pragma unroll
-    for (int p = 0; p < 8; p++) {
-        const int zs = (int)(__builtin_bit_cast(uint32_t, fmaf(e[p], inv, kMagicL)) - 0x4B400000u);  // q + 0x8080
-        xsum += zs - 0x8080;
-        z[p] = (uint32_t)zs;
-    }
-    if constexpr (SUM16) {
-        xsum += __builtin_amdgcn_update_dpp(0, xsum, 0xB1, 0xF, 0xF, true);
-        st.sum = -32.f * st.scale * (float)xsum;
-    } else {
-        xsum = ks_quad_sum(xsum);
-        st.sum = st.scale * (float)xsum;
-    }
-    const uint32_t a01 = __builtin_amdgcn_perm(z[1], z[0], 0x05010400u), a23 = __builtin_amdgcn_perm(z[3], z[2], 0x05010400u);
-    const uint32_t b01 = __builtin_amdgcn_perm(z[5], z[4], 0x05010400u), b23 = __builtin_amdgcn_perm(z[7], z[6], 0x05010400u);
-    st.planes.x = __builtin_amdgcn_perm(a23, a01, 0x05040100u) ^ 0x80808080u;
-    st.planes.y = __builtin_amdgcn_perm(a23, a01, 0x07060302u) ^ 0x80808080u;
-    st.planes.z = __builtin_amdgcn_perm(b23, b01, 0x05040100u) ^ 0x80808080u;
-    st.planes.w = __builtin_amdgcn_perm(b23, b01, 0x07060302u) ^ 0x80808080u;
-    return st;
-}
-// planes of dword w (0..7) of group h: limb 0 and limb 1
-__device__ __forceinline__ void limb_planes(const uint4 *xq, int h, int w, int &p0, int &p1) {
-    const uint4 &pl = xq[h * 4 + (w >> 1)];
-    p0 = (int)((w & 1) ? pl.z : pl.x);
-    p1 = (int)((w & 1) ? pl.w : pl.y);
-}
-
-template <> struct KS<kQ8_0> {
-    static constexpr int kSliceBytes = 544;
-    // where a lane finds what it needs of the staged slice: plane vector i (0..7), scale i, sum i
-    static constexpr int kScales = 2, kSumSpan = 0;
-    static __device__ __forceinline__ int plane_idx(int c, int i) { return 8 * c + i; }
-    static __device__ __forceinline__ int scale_idx(int c, int i) { return 2 * c + i; }
-    static __device__ __forceinline__ int sum_idx(int c, int i) { return 2 * c + i; }
-    struct __attribute__((packed, aligned(4))) Raw { uint32_t v[17]; };
-    static __device__ __forceinline__ int lane_offset(int c) { return c * 68; }
-    static __device__ __forceinline__ void load(Raw &r, const uint8_t *p) { r = *reinterpret_cast<const Raw *>(p); }
-    static __device__ __forceinline__ XPair x_load(const float *__restrict__ xs, int lane) { return limb_x_load(xs, lane); }
-    static __device__ __forceinline__ XPair x_load_bf16(const uint16_t *__restrict__ xs, int lane) { return limb_x_load_bf16(xs, lane); }
-    static __device__ __forceinline__ Staged stage(const XPair &xp) { return limb_stage(xp); }
-    static __device__ __forceinline__ float dot(const Raw &r, const uint4 *xq, const float *xsc, const float *, int) {
-        const uint32_t *v = r.v;
-        float out = 0.f;
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-            int s0 = 0, s1 = 0;
-#pragma unroll
-            for (int w = 0; w < 8; w++) {
-                const int q = (int)(h == 0 ? __builtin_amdgcn_alignbit(v[w + 1], v[w], 16) : v[9 + w]);
-                int p0, p1;
-                limb_planes(xq, h, w, p0, p1);
-                s0 = __builtin_amdgcn_sdot4(q, p0, s0, false);
-                s1 = __builtin_amdgcn_sdot4(q, p1, s1, false);
-            }
-            const int t = (s1 << 8) + s0;
-            const float d = half_bits_to_float(h == 0 ? (v[0] & 0xFFFFu) : (v[8] >> 16));
-            out = fmaf((float)t, d * xsc[h], out);
-        }
-        return out;
-    }
-};
-
-// IQ4_NL: the byte layout of Q4_0 (lane c: blocks 2c, 2c+1, 36 bytes), but the nibbles index a
-// 16-entry code book of int8 values, looked up four at a time with byte permutes; the dot products
-// then run on the two signed byte limbs like Q8_0.  Low nibbles of code dword w face values
-// 4w .. 4w+3 of the block (plane dword w), high nibbles values 16+4w .. (plane dword 4+w).
-template <> struct KS<kIQ4_NL> {
-    static constexpr int kSliceBytes = 288;
-    static constexpr int kScales = 2, kSumSpan = 0;
-    static __device__ __forceinline__ int plane_idx(int c, int i) { return 8 * c + i; }
-    static __device__ __forceinline__ int scale_idx(int c, int i) { return 2 * c + i; }
-    static __device__ __forceinline__ int sum_idx(int c, int i) { return 2 * c + i; }
-    struct __attribute__((packed, aligned(4))) Raw { uint32_t v[9]; };
-    static __device__ __forceinline__ int lane_offset(int c) { return c * 36; }
-    static __device__ __forceinline__ void load(Raw &r, const uint8_t *p) { r = *reinterpret_cast<const Raw *>(p); }
-    static __device__ __forceinline__ XPair x_load(const float *__restrict__ xs, int lane) { return limb_x_load(xs, lane); }
-    static __device__ __forceinline__ XPair x_load_bf16(const uint16_t *__restrict__ xs, int lane) { return limb_x_load_bf16(xs, lane); }
-    static __device__ __forceinline__ Staged stage(const XPair &xp) { return limb_stage(xp); }
-    // four code-book entries (int8, as bytes) for the four indices 0..15 in the bytes of idx
-    static __device__ __forceinline__ int book(uint32_t idx) {
-        const uint32_t t0 = 0xBFAD9881u, t1 = 0xF6EADDCFu, t2 = 0x26190D01u, t3 = 0x71594535u;  // -127 .. 113, four per dword
-        const uint32_t low3 = idx & 0x07070707u;
-        const uint32_t lo = __builtin_amdgcn_perm(t1, t0, low3), hi = __builtin_amdgcn_perm(t3, t2, low3);
-        return (int)__builtin_amdgcn_perm(hi, lo, 0x03020100u | ((idx & 0x08080808u) >> 1));  // byte i from hi when bit 3 of index i is set
-    }
-    static __device__ __forceinline__ float dot(const Raw &r, const uint4 *xq, const float *xsc, const float *, int) {
-        const uint32_t *v = r.v;
-        float out = 0.f;
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-            int s0 = 0, s1 = 0;
-#pragma unroll
-            for (int w = 0; w < 4; w++) {
-                const uint32_t q = h == 0 ? __builtin_amdgcn_alignbit(v[w + 1], v[w], 16) : v[5 + w];
-                const int lo = book(q & 0x0F0F0F0Fu), hi = book((q >> 4) & 0x0F0F0F0Fu);
-                int p0, p1;
-                limb_planes(xq, h, w, p0, p1);
-                s0 = __builtin_amdgcn_sdot4(lo, p0, s0, false);
-                s1 = __builtin_amdgcn_sdot4(lo, p1, s1, false);
-                limb_planes(xq, h, 4 + w, p0, p1);
-                s0 = __builtin_amdgcn_sdot4(hi, p0, s0, false);
-                s1 = __builtin_amdgcn_sdot4(hi, p1, s1, false);
-            }
-            const int t = (s1 << 8) + s0;
-            const float d = half_bits_to_float(h == 0 ? (v[0] & 0xFFFFu) : (v[4] >> 16));
-            out = fmaf((float)t, d * xsc[h], out);
-        }
-        return out;
-    }
-};
-
-template <> struct KS<kQ4_K> {
-    static constexpr int kSliceBytes = 288;  // two super-blocks
-    // where a lane finds what it needs of the staged slice: plane vector i (0..7), scale i, sum i
-    static constexpr int kScales = 2, kSumSpan = 32;
-    static __device__ __forceinline__ int plane_idx(int c, int i) { return 8 * c + i; }
-    static __device__ __forceinline__ int scale_idx(int c, int i) { return 2 * c + i; }
-    static __device__ __forceinline__ int sum_idx(int c, int i) { return 2 * c + i; }
-    struct Raw { uint4 hd, q0, q1; };
-    static __device__ __forceinline__ int lane_offset(int c) { return (c >> 2) * 144; }
-    static __device__ __forceinline__ void load(Raw &r, const uint8_t *sb, int c) {
-        r.hd = *reinterpret_cast<const uint4 *>(sb);
-        const uint4 *q = reinterpret_cast<const uint4 *>(sb + 16 + 32 * (c & 3));
-        r.q0 = q[0];
-        r.q1 = q[1];
-    }
-    static __device__ __forceinline__ XPair x_load(const float *__restrict__ xs, int lane) { return limb_x_load(xs, lane); }
-    static __device__ __forceinline__ XPair x_load_bf16(const uint16_t *__restrict__ xs, int lane) { return limb_x_load_bf16(xs, lane); }
-    static __device__ __forceinline__ Staged stage(const XPair &xp) { return limb_stage(xp); }
-    static __device__ __forceinline__ float dot(const Raw &r, const uint4 *xq, const float *xsc, const float *xsm, int c) {
-        const uint32_t q[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
-        const float d = half_bits_to_float(r.hd.x & 0xFFFFu), dmin = half_bits_to_float(r.hd.x >> 16);
-        const int g = c & 3;
-        float out = 0.f;
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-            int s0 = 0, s1 = 0;
-#pragma unroll
-            for (int w = 0; w < 8; w++) {
-                const int cw = (int)((h == 0 ? q[w] : (q[w] >> 4)) & 0x0F0F0F0Fu);  // four codes as bytes 0..15
-                int p0, p1;
-                limb_planes(xq, h, w, p0, p1);
-                s0 = __builtin_amdgcn_sdot4(cw, p0, s0, false);
-                s1 = __builtin_amdgcn_sdot4(cw, p1, s1, false);
-            }
-            const int t = (s1 << 8) + s0;
-            uint32_t sc, mn;
-            q4k_scale_min(r.hd.y, r.hd.z, r.hd.w, 2 * g + h, sc, mn);
-            out = fmaf((float)t, (d * (float)sc) * xsc[h], out);
-            out = fmaf(-(dmin * (float)mn), xsm[h], out);
-        }
-        return out;
-    }
-};
-
-
-// Q6_K: w = d * sc[16-value run] * (code - 32), code = low nibble | two high bits << 4.  The
-// -32 is applied through the activation sums of the run, so the codes stay unsigned bytes.
-template <> struct KS<kQ6_K> {
-    static constexpr int kSliceBytes = 420;  // two super-blocks
-    static constexpr int kScales = 4, kSumSpan = 16;
-    // c = 4 * sb + 2 * half + pp; quadrant qd's run is values 32 * qd + 16 * pp .. of the half
-    static __device__ __forceinline__ int plane_idx(int c, int i) { return 8 * (c & ~1) + 2 * (c & 1) + 4 * (i >> 1) + (i & 1); }
-    static __device__ __forceinline__ int scale_idx(int c, int i) { return 2 * (c & ~1) + i; }
-    static __device__ __forceinline__ int sum_idx(int c, int i) { return 4 * (c & ~1) + 2 * i + (c & 1); }
-    struct __attribute__((packed, aligned(2))) U4 { uint32_t v[4]; };
-    struct __attribute__((packed, aligned(2))) U2 { uint32_t v[2]; };
-    struct Raw { U4 a, b, h; U2 sc; uint32_t d; };
-    static __device__ __forceinline__ int lane_offset(int c) { return (c >> 2) * 210; }
-    static __device__ __forceinline__ void load(Raw &r, const uint8_t *sb, int c) {
-        const int half = (c >> 1) & 1, pp = c & 1;
-        const uint8_t *ql = sb + 64 * half + 16 * pp;
-        r.a = *reinterpret_cast<const U4 *>(ql);
-        r.b = *reinterpret_cast<const U4 *>(ql + 32);
-        r.h = *reinterpret_cast<const U4 *>(sb + 128 + 32 * half + 16 * pp);
-        r.sc = *reinterpret_cast<const U2 *>(sb + 192 + 8 * half);
-        r.d = *reinterpret_cast<const uint16_t *>(sb + 208);
-    }
-    static __device__ __forceinline__ XPair x_load(const float *__restrict__ xs, int lane) { return limb_x_load(xs, lane); }
-    static __device__ __forceinline__ XPair x_load_bf16(const uint16_t *__restrict__ xs, int lane) { return limb_x_load_bf16(xs, lane); }
-    static __device__ __forceinline__ Staged stage(const XPair &xp) { return limb_stage<true>(xp); }
-    // xq[2 qd + e] = planes of values 8 e .. 8 e + 7 of quadrant qd's run; xsc[qd] the scale of the
-    // quadrant's activations, xsm[qd] = -32 * (sum of the run's activations as quantised)
-    static __device__ __forceinline__ float dot(const Raw &r, const uint4 *xq, const float *xsc, const float *xsm, int c) {
-        const int sc_shift = 8 * (c & 1);
-        float out = 0.f;
-#pragma unroll
-        for (int qd = 0; qd < 4; qd++) {
-            int s0 = 0, s1 = 0;
-#pragma unroll
-            for (int w = 0; w < 4; w++) {
-                const uint32_t src = (qd & 1) ? r.b.v[w] : r.a.v[w];
-                const uint32_t lo = ((qd >> 1) ? (src >> 4) : src) & 0x0F0F0F0Fu;
-                const uint32_t hv = r.h.v[w];
-                const uint32_t hs = qd == 0 ? (hv << 4) : qd == 1 ? (hv << 2) : qd == 2 ? hv : (hv >> 2);
-                const int code = (int)((hs & 0x30303030u) | lo);
-                const uint4 &pl = xq[2 * qd + (w >> 1)];
-                s0 = __builtin_amdgcn_sdot4(code, (int)((w & 1) ? pl.z : pl.x), s0, false);
-                s1 = __builtin_amdgcn_sdot4(code, (int)((w & 1) ? pl.w : pl.y), s1, false);
-            }
-            const int t = (s1 << 8) + s0;
-            const int sc = __builtin_amdgcn_sbfe((int)r.sc.v[qd >> 1], 16 * (qd & 1) + sc_shift, 8);
-            out = fmaf((float)sc, fmaf((float)t, xsc[qd], xsm[qd]), out);
-        }
-        return out * half_bits_to_float(r.d & 0xFFFFu);
-    }
-};
-
-template <int T>
-__device__ __forceinline__ void ks_load(typename KS<T>::Raw &r, const uint8_t *p, int c) {
-    if constexpr (T == kQ4_K || T == kQ6_K) KS<T>::load(r, p, c);
-    else KS<T>::load(r, p);
-}
-
-#ifdef GQ_KS_TRACE
-__device__ unsigned long long g_ks_trace[4096 * 16];
-#define KS_TRACE(k) do { if (lane == 0) g_ks_trace[((size_t)wg * waves + wave) % 4096 * 16 + (k)] = __builtin_readcyclecounter(); } while (0)
-#define KS_TRACE_WALL(k) do { if (lane == 0) g_ks_trace[((size_t)wg * waves + wave) % 4096 * 16 + (k)] = __builtin_amdgcn_s_memrealtime(); } while (0)
-#else
-#define KS_TRACE(k) do { } while (0)
-#define KS_TRACE_WALL(k) do { } while (0)
-#endif
-
-constexpr int kWaveLdsDwords = 76 * 4;  // per wavefront: 64 uint4 of planes, 16 scales, up to 32 sums
-
-// Workgroup `wg` of a problem: `waves` wavefronts work (threads beyond them only join the final
-// barrier); wavefront w handles slices w, w + waves, ... below nslices of the 8 * iters rows
-// starting at wg * 8 * iters.  PF divides iters: rows are consumed in groups of PF, buffer j of a
-// group always holding the row-step with (it % PF == j).
-// WIN <= PF row-steps are kept in flight: WIN go out before the activations are converted, and
-// each consumed step is followed by the load of the step WIN ahead, so that load issue (which
-// blocks while the memory pipeline is full) and arithmetic alternate instead of forming two
-// phases.  (A variant that treats a wavefront's slices x row-steps as one sequence, so that the
-// window also spans slices when there are only one or two row-steps, was measured: its guarded
-// steps cost the unguarded common case 8 % and it was dropped.)
-template <int T, int PF, int WIN>
-__device__ __forceinline__ void ks_body(const void *__restrict__ xv, int x_bf16, const uint8_t *__restrict__ W,
-                                        const float *__restrict__ bias, float *__restrict__ y, int N, int64_t row_bytes, int iters,
-                                        int nslices, int half_tail, int act, int waves, int wg, uint32_t *lds) {
-    typedef typename KS<T>::Raw Raw;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int rg = lane >> 3, c = lane & 7;
-    const int rows_wg = iters * 8;
-    const int row0 = wg * rows_wg;
-    float *all = reinterpret_cast<float *>(lds + waves * kWaveLdsDwords);  // partial sums [waves][rows_wg]
-    // activations of slice sl for this lane (fp32, or bf16 widened on the fly; x_bf16 is uniform);
-    // the lanes that face the missing half of a last half slice get zeros
-    const bool upper_half = lane >= 32;  // this lane converts values 256 .. 511 of a slice (in both activation layouts)
-    auto x_slice = [&](int sl) -> XPair {
-        if (half_tail && sl == nslices - 1 && upper_half) {
-            XPair z;
-            z.lo = make_float4(0.f, 0.f, 0.f, 0.f);
-            z.hi = z.lo;
-            return z;
-        }
-        if (x_bf16) return KS<T>::x_load_bf16(reinterpret_cast<const uint16_t *>(xv) + sl * kSliceValues, lane);
-        return KS<T>::x_load(reinterpret_cast<const float *>(xv) + sl * kSliceValues, lane);
-    };
-    if (wave < waves) {
-        uint4 *my_planes = reinterpret_cast<uint4 *>(lds + wave * kWaveLdsDwords);
-        float *my_scales = reinterpret_cast<float *>(my_planes + 64);
-        float *my_sums = my_scales + 16;
-        float *part = all + wave * rows_wg;
-
-        KS_TRACE(0);
-        KS_TRACE_WALL(12);
-        const int spw = (nslices - wave + waves - 1) / waves;  // slices of this wavefront (>= 1)
-        XPair xp = x_slice(wave);
-        const int last_row = N - 1;
-        // In a last half slice the lanes of the missing half re-read the codes of the present one
-        // (finite scales; their activations are zero).
-        auto lane_c = [&](int j) { return (half_tail && wave + j * waves == nslices - 1) ? (c & 3) : c; };
-        auto addr = [&](int j, int it) -> const uint8_t * {
-            const int row = min(row0 + it * 8 + rg, last_row);
-            return W + (int64_t)row * row_bytes + (int64_t)(wave + j * waves) * KS<T>::kSliceBytes + KS<T>::lane_offset(lane_c(j));
-        };
-        Raw buf[PF];
-#pragma unroll
-        for (int j = 0; j < WIN; j++) ks_load<T>(buf[j], addr(0, j), lane_c(0));
-        KS_TRACE(1);
-
-        uint4 xq[8];
-        constexpr int NS = KS<T>::kScales, SPAN = KS<T>::kSumSpan;
-        float xsc[NS], xsm[NS];
-#pragma unroll
-        for (int i = 0; i < NS; i++) xsm[i] = 0.f;
-        auto stage = [&](const XPair &p) {
-            const Staged st = KS<T>::stage(p);
-            my_planes[lane] = st.planes;
-            if ((lane & 3) == 0) my_scales[lane >> 2] = st.scale;
-            if constexpr (SPAN == 32) { if ((lane & 3) == 0) my_sums[lane >> 2] = st.sum; }
-            if constexpr (SPAN == 16) { if ((lane & 1) == 0) my_sums[lane >> 1] = st.sum; }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-            for (int i = 0; i < 8; i++) xq[i] = my_planes[KS<T>::plane_idx(c, i)];
-#pragma unroll
-            for (int i = 0; i < NS; i++) {
-                xsc[i] = my_scales[KS<T>::scale_idx(c, i)];
-                if constexpr (SPAN != 0) xsm[i] = my_sums[KS<T>::sum_idx(c, i)];
-            }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-        };
-        stage(xp);
-        KS_TRACE(2);
-        if (spw > 1) xp = x_slice(wave + waves);
-        KS_TRACE(3);
-
-        const int ngroups = spw * (iters / PF);
-        int j = 0, i0 = 0;  // slice index and first row-step of the current group
-        for (int g = 0; g < ngroups; g++) {
-            const bool last_group = g == ngroups - 1;
-            // where the buffers of this group are refilled from: same slice PF steps on, or the next slice
-            const bool wrap = i0 + PF >= iters;
-            const int nj = wrap ? j + 1 : j, ni0 = wrap ? 0 : i0 + PF;
-#pragma unroll
-            for (int jj = 0; jj < PF; jj++) {
-                float d = KS<T>::dot(buf[jj], xq, xsc, xsm, c);
-                if (jj + WIN < PF) ks_load<T>(buf[jj + WIN], addr(j, i0 + jj + WIN), lane_c(j));
-                else if (!last_group) ks_load<T>(buf[jj + WIN - PF], addr(nj, ni0 + jj + WIN - PF), lane_c(nj));
-                d = ks_oct_sum(d);
-                if (c == 0) {
-                    float *slot = part + (i0 + jj) * 8 + rg;
-                    *slot = j == 0 ? d : *slot + d;
-                }
-            }
-            if (wrap && !last_group) {  // next group starts a new slice: convert its activations
-                stage(xp);
-                if (nj + 1 < spw) xp = x_slice(wave + (nj + 1) * waves);
-            }
-            j = nj;
-            i0 = ni0;
-        }
-        KS_TRACE(14);
-        KS_TRACE_WALL(13);
-    }
-    __syncthreads();
-    for (int r = tid; r < rows_wg; r += blockDim.x) {
-        const int row = row0 + r;
-        if (row < N) {
-            float t = 0.f;
-            for (int w = 0; w < waves; w++) t += all[w * rows_wg + r];
-            y[row] = apply_act(act, t + (bias ? bias[row] : 0.f));
-        }
-    }
-}
-
-template <int T, int PF, int WIN>
-__global__ __launch_bounds__(512) void gemv_ks_kernel(const void *__restrict__ X, int x_bf16, const uint8_t *__restrict__ W,
+template <int T, int PF, int WIN, bool XBF16>
+__global__ __launch_bounds__(512) void gemv_ks_kernel(const void *__restrict__ X, const uint8_t *__restrict__ W,
                                                       const float *__restrict__ bias, float *__restrict__ Y, int K, int N,
                                                       int64_t row_bytes, int iters, int nslices, int half_tail, int act) {
     extern __shared__ uint32_t lds[];
-    const uint8_t *x = reinterpret_cast<const uint8_t *>(X) + (int64_t)blockIdx.y * K * (x_bf16 ? 2 : 4);
-    ks_body<T, PF, WIN>(x, x_bf16, W, bias, Y + (int64_t)blockIdx.y * N, N, row_bytes, iters, nslices, half_tail, act, (int)(blockDim.x >> 6),
+    const uint8_t *x = reinterpret_cast<const uint8_t *>(X) + (int64_t)blockIdx.y * K * (XBF16 ? 2 : 4);
+    ks_body<T, PF, WIN, false, XBF16>(x, W, bias, Y + (int64_t)blockIdx.y * N, N, row_bytes, iters, nslices, half_tail, act, (int)(blockDim.x >> 6),
                         (int)blockIdx.x, lds);
 }
 
@@ -585,52 +47,10 @@ __global__ __launch_bounds__(512) void gemv_ks_batch_kernel(const KsBatch b) {
     for (int j = 1; j < kMaxBatchKs; j++)
         if (j < b.count && (int)blockIdx.x >= b.p[j].wg_begin) i = j;
     const KsProblem &q = b.p[i];
-    ks_body<T, kBatchPF, kBatchPF>(q.x, 0, q.W, q.bias, q.y, q.N, q.row_bytes, q.iters, q.nslices, q.half_tail, q.act, q.waves,
+    ks_body<T, kBatchPF, kBatchPF>(q.x, q.W, q.bias, q.y, q.N, q.row_bytes, q.iters, q.nslices, q.half_tail, q.act, q.waves,
                      (int)blockIdx.x - q.wg_begin, lds);
 }
 
-struct KsPlan { int waves, nslices, half_tail, iters, pf, wgs; size_t shmem; };
-
-// GOMLX_HIPQ_GEMV_KS="waves_per_cu" overrides the built-in choice (tuning runs only).
-int ks_env_waves() {
-    static const int v = [] { const char *e = std::getenv("GOMLX_HIPQ_GEMV_KS"); return e ? std::atoi(e) : 0; }();
-    return v;
-}
-
-// Slices of 512 values (a last one of 256 when K is an odd multiple of 256) and wavefronts per
-// workgroup: one per slice up to 8; more slices than that are dealt out round-robin.
-bool ks_split(int64_t K, int &waves, int &nslices, int &half_tail) {
-    if (K <= 0 || K % 256 != 0 || K > (int64_t)INT32_MAX / 4) return false;
-    nslices = (int)((K + kSliceValues - 1) / kSliceValues);
-    half_tail = (K % kSliceValues) != 0 ? 1 : 0;
-    waves = nslices < 8 ? nslices : 8;
-    return true;
-}
-
-size_t ks_lds_bytes(int waves, int iters) { return (size_t)waves * kWaveLdsDwords * 4 + (size_t)waves * iters * 8 * sizeof(float); }
-
-bool ks_plan(int64_t K, int64_t N, KsPlan &p) {
-    if (N <= 0 || !ks_split(K, p.waves, p.nslices, p.half_tail)) return false;
-    const int cus = device_cu_count();
-    // One 8-wavefront workgroup per CU streams best; problems that would leave a wavefront with
-    // only one or two row-steps are launch- and latency-bound and do better with twice the
-    // wavefronts (more independent prologues in flight).
-    auto iters_for = [&](int waves_per_cu) {
-        int64_t wgs = (int64_t)cus * waves_per_cu / p.waves;
-        if (wgs < 1) wgs = 1;
-        const int64_t it = (N + wgs * 8 - 1) / (wgs * 8);
-        return it < 1 ? (int64_t)1 : it;
-    };
-    int64_t iters = ks_env_waves() > 0 ? iters_for(ks_env_waves()) : iters_for(8);
-    if (ks_env_waves() <= 0 && iters <= 2) iters = iters_for(16);
-    if (iters > 8) iters = (iters + 3) / 4 * 4;  // deep problems run in groups of 4 rows
-    if (iters > kMaxItersKs) iters = kMaxItersKs;
-    p.iters = (int)iters;
-    p.pf = iters <= 8 ? (int)iters : 4;
-    p.wgs = (int)((N + iters * 8 - 1) / (iters * 8));
-    p.shmem = ks_lds_bytes(p.waves, p.iters);
-    return true;
-}
 
 template <int T, int PF>
 int launch_ks_pf(const KsPlan &p, const void *x, int x_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act,
@@ -638,7 +58,10 @@ int launch_ks_pf(const KsPlan &p, const void *x, int x_bf16, int64_t M, int64_t 
     const int64_t row_bytes = (K / Geom<T>::vpb) * Geom<T>::bpb;
     const dim3 grid((unsigned)p.wgs, (unsigned)M), block((unsigned)p.waves * 64);
     constexpr int WIN = PF < 3 ? PF : 3;
-    return launch(gemv_ks_kernel<T, PF, WIN>, grid, block, p.shmem, s, x, x_bf16, W, bias, y, (int)K, (int)N, row_bytes, p.iters, p.nslices,
+    if (x_bf16)
+        return launch(gemv_ks_kernel<T, PF, WIN, true>, grid, block, p.shmem, s, x, W, bias, y, (int)K, (int)N, row_bytes, p.iters, p.nslices,
+                      p.half_tail, act);
+    return launch(gemv_ks_kernel<T, PF, WIN, false>, grid, block, p.shmem, s, x, W, bias, y, (int)K, (int)N, row_bytes, p.iters, p.nslices,
                   p.half_tail, act);
 }
 

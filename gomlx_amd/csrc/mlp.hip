@@ -1,0 +1,127 @@
+// The callers on either side of a quantized dense layer in a decoder block
+// (ml/zoo/transformer/transformer.go:1275-1294): the RMS normalisation in front of the
+// projections (ml/layers/norm/rmsnorm.go:78-113) and the gated feed-forward front
+//     ff = act(x . Wgate^T + bgate) * (x . Wup^T + bup).
+//
+// For up to 16 activation rows both are folded into the K-sliced decode GEMV (gemv_ks_body.hpp,
+// EXT): one launch reads the two weight matrices once and writes only ff.  Larger batches are
+// composed from the dense kernels plus the two small kernels below.
+#include "gemv_ks_body.hpp"
+
+namespace gq {
+
+namespace {
+
+template <int T, int PF, int WIN>
+__global__ __launch_bounds__(512) void gemv_ks_ext_kernel(const float *__restrict__ X, const uint8_t *__restrict__ W,
+                                                          const float *__restrict__ bias, float *__restrict__ Y, int K, int N,
+                                                          int64_t row_bytes, int iters, int nslices, int half_tail, int act,
+                                                          const KsExt ext) {
+    extern __shared__ uint32_t lds[];
+    ks_body<T, PF, WIN, true>(X + (int64_t)blockIdx.y * K, W, bias, Y + (int64_t)blockIdx.y * N, N, row_bytes, iters, nslices, half_tail,
+                              act, (int)(blockDim.x >> 6), (int)blockIdx.x, lds, &ext);
+}
+
+template <int T, int PF>
+int launch_ext_pf(const KsPlan &p, const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y,
+                  const KsExt &ext, hipStream_t s) {
+    const int64_t row_bytes = (K / Geom<T>::vpb) * Geom<T>::bpb;
+    const dim3 grid((unsigned)p.wgs, (unsigned)M), block((unsigned)p.waves * 64);
+    constexpr int WIN = PF < 3 ? PF : 3;
+    return launch(gemv_ks_ext_kernel<T, PF, WIN>, grid, block, p.shmem, s, x, W, bias, y, (int)K, (int)N, row_bytes, p.iters, p.nslices,
+                  p.half_tail, act, ext);
+}
+
+template <int T>
+int launch_ext(const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y, const KsExt &ext,
+               hipStream_t s) {
+    // With two matrices the row-steps alternate between them: plan for 2 N rows and an even count.
+    const bool dual = ext.W2 != nullptr;
+    KsPlan p;
+    if (!ks_plan(K, dual ? 2 * N : N, p)) return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv_ks: unsupported problem");
+    if (dual) {
+        if (p.iters & 1) {
+            p.iters++;
+            p.pf = p.iters;  // odd counts are at most 7
+        }
+        p.wgs = (int)((N + p.iters * 4 - 1) / (p.iters * 4));
+        p.shmem = ks_lds_bytes(p.waves, p.iters);
+    }
+    switch (p.pf) {
+    case 1: return launch_ext_pf<T, 1>(p, x, M, K, W, N, bias, act, y, ext, s);
+    case 2: return launch_ext_pf<T, 2>(p, x, M, K, W, N, bias, act, y, ext, s);
+    case 3: return launch_ext_pf<T, 3>(p, x, M, K, W, N, bias, act, y, ext, s);
+    case 4: return launch_ext_pf<T, 4>(p, x, M, K, W, N, bias, act, y, ext, s);
+    case 5: return launch_ext_pf<T, 5>(p, x, M, K, W, N, bias, act, y, ext, s);
+    case 6: return launch_ext_pf<T, 6>(p, x, M, K, W, N, bias, act, y, ext, s);
+    case 7: return launch_ext_pf<T, 7>(p, x, M, K, W, N, bias, act, y, ext, s);
+    default: return launch_ext_pf<T, 8>(p, x, M, K, W, N, bias, act, y, ext, s);
+    }
+}
+
+// y = x / sqrt(mean(x^2) + eps) * (gain + offset), one workgroup per row (the operations and their
+// order follow ml/layers/norm/rmsnorm.go:86-111: Square, ReduceMean, AddScalar, Sqrt, Div, Mul).
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float *__restrict__ X, const float *__restrict__ gain, float gain_offset, float eps,
+                                                      int K, float *__restrict__ Y) {
+    __shared__ float part[4];
+    const float *x = X + (int64_t)blockIdx.x * K;
+    float *y = Y + (int64_t)blockIdx.x * K;
+    float ss = 0.f;
+    for (int k = threadIdx.x; k < K; k += 256) ss = fmaf(x[k], x[k], ss);
+    for (int m = 1; m < 64; m <<= 1) ss += __shfl_xor(ss, m);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float mean = ((part[0] + part[1]) + (part[2] + part[3])) / (float)K;
+    const float r = sqrtf(mean + eps);
+    for (int k = threadIdx.x; k < K; k += 256) {
+        float v = x[k] / r;
+        if (gain) v *= gain[k] + gain_offset;
+        y[k] = v;
+    }
+}
+
+// y[i] *= g[i]
+__global__ __launch_bounds__(256) void mul_inplace_kernel(float *__restrict__ y, const float *__restrict__ g, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) y[i] *= g[i];
+}
+
+}  // namespace
+
+bool gemv_ks_ext_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, const void *gain) {
+    if (M < 1 || M > 16 || N > (int64_t)INT32_MAX / 8) return false;
+    if (gain && (reinterpret_cast<uintptr_t>(gain) & 15)) return false;
+    return gemv_ks_supported(type, K, N, x);
+}
+
+int launch_gemv_ks_ext(int type, const float *x, int64_t M, int64_t K, const RmsNorm *norm, const uint8_t *W, const float *bias,
+                       const uint8_t *W2, const float *bias2, int64_t N, int act, float *y, hipStream_t s) {
+    KsExt ext = {};
+    ext.W2 = W2;
+    ext.bias2 = bias2;
+    if (norm) {
+        ext.norm = 1;
+        ext.gain = norm->gain;
+        ext.gain_offset = norm->gain_offset;
+        ext.eps = norm->eps;
+        ext.inv_k = 1.0f / (float)K;
+    }
+    switch (type) {
+    case kQ4_0: return launch_ext<kQ4_0>(x, M, K, W, N, bias, act, y, ext, s);
+    case kQ8_0: return launch_ext<kQ8_0>(x, M, K, W, N, bias, act, y, ext, s);
+    case kQ4_K: return launch_ext<kQ4_K>(x, M, K, W, N, bias, act, y, ext, s);
+    case kQ6_K: return launch_ext<kQ6_K>(x, M, K, W, N, bias, act, y, ext, s);
+    case kIQ4_NL: return launch_ext<kIQ4_NL>(x, M, K, W, N, bias, act, y, ext, s);
+    default: return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv_ks: ggml type %d is not implemented", type);
+    }
+}
+
+int launch_rmsnorm(const float *x, int64_t M, int64_t K, const float *gain, float gain_offset, float eps, float *y, hipStream_t s) {
+    return launch(rmsnorm_kernel, dim3((unsigned)M), dim3(256), 0, s, x, gain, gain_offset, eps, (int)K, y);
+}
+
+int launch_mul_inplace(float *y, const float *g, int64_t n, hipStream_t s) {
+    return launch(mul_inplace_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, y, g, n);
+}
+
+}  // namespace gq

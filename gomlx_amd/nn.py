@@ -95,12 +95,84 @@ def dequantize(weights: torch.Tensor, ggml_type: int) -> torch.Tensor:
     return out
 
 
+@dataclass
+class RMSNorm:
+    """Configuration of norm.RMSNorm over the last axis (ml/layers/norm/rmsnorm.go:38-76): ``gain`` is the
+    learned scale [K] (None = WithScale(false)), ``epsilon`` WithEpsilon (default 1e-6), ``scale_offset``
+    WithScaleOffset (Gemma adds 1.0 to the scale)."""
+    gain: torch.Tensor | None = None
+    epsilon: float = 1e-6
+    scale_offset: float = 0.0
+
+    def _desc(self, K: int):
+        if self.gain is not None:
+            _require_cuda("gain", self.gain)
+            if self.gain.dtype != torch.float32 or tuple(self.gain.shape) != (K,):
+                raise ValueError(f"gain must be a float32 [{K}] tensor")
+        return _lib.RmsNormDesc(None if self.gain is None else self.gain.data_ptr(), self.epsilon, self.scale_offset)
+
+
+def rms_norm(x: torch.Tensor, norm: RMSNorm) -> torch.Tensor:
+    """RMSNormBuilder.Done (ml/layers/norm/rmsnorm.go:78-113) over the last axis of a float32 tensor."""
+    _require_cuda("x", x)
+    if x.dtype != torch.float32:
+        raise _lib.NotImplementedByBackend(_lib.ERR_NOT_IMPLEMENTED, f"rms_norm: dtype {x.dtype} is not implemented")
+    K = x.shape[-1]
+    d = norm._desc(K)
+    _lib.init(x.device.index or 0)
+    y = torch.empty_like(x)
+    _lib.check(_lib.lib().gq_rmsnorm_f32(x.data_ptr(), x.numel() // K if K else 0, K, d.dGain, d.eps, d.gain_offset, y.data_ptr(),
+                                         _stream_ptr(x)))
+    return y
+
+
+def gated_feed_forward(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, quant: Quantization, activation: Activation,
+                       bias_gate: torch.Tensor | None = None, bias_up: torch.Tensor | None = None,
+                       norm: RMSNorm | None = None) -> torch.Tensor:
+    """The front of a gated feed-forward block (ml/zoo/transformer/transformer.go:1276-1287):
+    ``activation(dense(xn, w_gate)) * dense(xn, w_up)`` with ``xn = rms_norm(x)`` when ``norm`` is given.
+    x: [batch..., K] float32; both weights [N, bytesPerRow] uint8 of one GGML type."""
+    if quant is None or quant.scheme != QuantizationScheme.GGML:
+        raise _lib.NotImplementedByBackend(_lib.ERR_NOT_IMPLEMENTED, "only the GGML scheme is on this path")
+    for name, t in (("x", x), ("w_gate", w_gate), ("w_up", w_up)):
+        _require_cuda(name, t)
+    _weights_2d(w_gate)
+    _weights_2d(w_up)
+    if w_gate.shape != w_up.shape:
+        raise ValueError(f"gate and up weights differ in shape: {tuple(w_gate.shape)} vs {tuple(w_up.shape)}")
+    if x.dtype != torch.float32:
+        raise _lib.NotImplementedByBackend(_lib.ERR_NOT_IMPLEMENTED, f"gated_feed_forward: dtype {x.dtype} is not implemented")
+    import ctypes
+    L = _lib.lib()
+    N, rb = w_gate.shape
+    K_in = x.shape[-1]
+    M = x.numel() // K_in if K_in else 0
+    K = ctypes.c_int64(0)
+    for b in (bias_gate, bias_up):
+        blen = -1
+        if b is not None:
+            _require_cuda("bias", b)
+            if b.dtype != torch.float32 or b.dim() != 1:
+                raise ValueError("bias must be a float32 [N] tensor")
+            blen = b.shape[0]
+        _lib.check(L.gq_qdense_check(quant.ggml_type, _lib.F32, M, K_in, N, rb, blen, activation.to_backend(), ctypes.byref(K)))
+    d = None if norm is None else norm._desc(K.value)
+    _lib.init(x.device.index or 0)
+    y = torch.empty(x.shape[:-1] + (N,), dtype=torch.float32, device=x.device)
+    _lib.check(L.gq_qdense_gated_f32(quant.ggml_type, x.data_ptr(), M, K.value, None if d is None else ctypes.byref(d),
+                                     w_gate.data_ptr(), None if bias_gate is None else bias_gate.data_ptr(), w_up.data_ptr(),
+                                     None if bias_up is None else bias_up.data_ptr(), N, activation.to_backend(), y.data_ptr(),
+                                     _stream_ptr(x)))
+    return y
+
+
 def quantized_dense(x: torch.Tensor, weights: torch.Tensor, quant: Quantization, bias: torch.Tensor | None = None,
-                    *optional_activation: Activation) -> torch.Tensor:
+                    *optional_activation: Activation, norm: RMSNorm | None = None) -> torch.Tensor:
     """nn.QuantizedDense for the GGML scheme: y = activation(x @ dequant(weights)^T + bias).
 
     x: [batch..., K] float32 or bfloat16; weights: [N, bytesPerRow] uint8; bias: [N] float32.
-    Returns [batch..., N] float32.
+    Returns [batch..., N] float32.  ``norm`` applies an RMS normalisation to x first (float32 x only):
+    Model.normalize followed by a projection, ml/zoo/transformer/transformer.go:1099-1101.
     """
     if len(optional_activation) > 1:
         raise ValueError(f"quantized_dense can only take one optional activation, got {optional_activation}")
@@ -134,6 +206,13 @@ def quantized_dense(x: torch.Tensor, weights: torch.Tensor, quant: Quantization,
     _lib.check(L.gq_qdense_check(quant.ggml_type, xd, M, K_in, N, rb, blen, act.to_backend(), ctypes.byref(K)))
     _lib.init(x.device.index or 0)
     y = torch.empty(x.shape[:-1] + (N,), dtype=torch.float32, device=x.device)
+    if norm is not None:
+        if xd != _lib.F32:
+            raise _lib.NotImplementedByBackend(_lib.ERR_NOT_IMPLEMENTED, "a fused normalisation takes float32 activations")
+        d = norm._desc(K.value)
+        _lib.check(L.gq_qdense_norm_f32(quant.ggml_type, x.data_ptr(), M, K.value, ctypes.byref(d), weights.data_ptr(), N,
+                                        None if bias is None else bias.data_ptr(), act.to_backend(), y.data_ptr(), _stream_ptr(x)))
+        return y
     fn = L.gq_qdense_f32 if xd == _lib.F32 else L.gq_qdense_bf16
     _lib.check(fn(quant.ggml_type, x.data_ptr(), M, K.value, weights.data_ptr(), N,
                   None if bias is None else bias.data_ptr(), act.to_backend(), y.data_ptr(), _stream_ptr(x)))

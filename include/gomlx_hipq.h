@@ -124,6 +124,34 @@ typedef struct {
 } gq_dense_desc;
 int gq_qdense_f32_batch(int count, const gq_dense_desc *descs, void *stream);
 
+/* ---- The callers on either side of the dense layers in a decoder block
+ * (ml/zoo/transformer/transformer.go:1099-1101, 1275-1294).  These have no fused op in the
+ * reference: a backend's Executable would recognise the node pattern. ----
+ *
+ * norm.RMSNorm(...).WithEpsilon(eps).WithScaleOffset(gain_offset).Done() over the last axis
+ * (ml/layers/norm/rmsnorm.go:78-113): y = x / sqrt(mean(x^2) + eps) * (gain + gain_offset).
+ * dGain [K] may be NULL (WithScale(false)). */
+int gq_rmsnorm_f32(const float *dX, int64_t M, int64_t K, const float *dGain, float eps,
+                   float gain_offset, float *dY, void *stream);
+typedef struct {
+    const float *dGain; /* [K] or NULL */
+    float eps;
+    float gain_offset;
+} gq_rmsnorm;
+/* gq_qdense_f32 applied to RMSNorm(x) (Model.normalize followed by a projection,
+ * transformer.go:1099-1101 for q/k/v); norm == NULL is plain gq_qdense_f32.  Up to 16 rows run
+ * in the decode GEMV itself when K is a multiple of 256 and x and gain are 16-byte aligned. */
+int gq_qdense_norm_f32(int type, const float *dX, int64_t M, int64_t K, const gq_rmsnorm *norm,
+                       const void *dW, int64_t N, const float *dBias, int act, float *dY,
+                       void *stream);
+/* The gated feed-forward front (transformer.go:1279-1287, after the pre_feedforward_norm of
+ * :1276 when norm != NULL): y = act(xn . Wgate^T + bgate) * (xn . Wup^T + bup), xn = RMSNorm(x)
+ * or x.  Both matrices are [N, gq_row_bytes(type, K)] of one type.  Same fast-path conditions as
+ * gq_qdense_norm_f32; other shapes are composed of dense calls and use a per-stream workspace. */
+int gq_qdense_gated_f32(int type, const float *dX, int64_t M, int64_t K, const gq_rmsnorm *norm,
+                        const void *dWgate, const float *dBiasGate, const void *dWup,
+                        const float *dBiasUp, int64_t N, int act, float *dY, void *stream);
+
 /* ---- compute.Function.QuantizedEmbeddingLookup (core/graph/fused_ops.go:295-296;
  * nn.QuantizedGather ml/nn/quantized_gather.go:30-43; ml/ggml/gather.go:21-49):
  * dOut[i, :] = dequant(dTable[dIndices[i], :]), bit-exact.  An index outside [0, vocab)

@@ -291,6 +291,64 @@ int gqo_qdense_f32acc(int type, const float *x, int64_t M, int64_t K, const uint
     return 0;
 }
 
+/* ---- callers around the dense layers -------------------------------------- */
+
+/* RMSNormBuilder.Done (ml/layers/norm/rmsnorm.go:78-113) over the last axis, node by node:
+ * Square, ReduceMean (:86-87), AddScalar epsilon (:88-90), Sqrt (:91), Div (:92), and with a gain
+ * AddScalar offset (:101-103), Mul (:111).  Each node's fp32 result is rounded on its own; the
+ * mean is summed in double so that it is the correctly rounded mean whatever order a backend
+ * reduces in. */
+int gqo_rmsnorm(const float *x, int64_t M, int64_t K, const float *gain, float eps, float gain_offset,
+                float *y) {
+    if (M < 0 || K <= 0) return -1;
+    for (int64_t m = 0; m < M; m++) {
+        const float *xr = x + (size_t)m * K;
+        float *yr = y + (size_t)m * K;
+        double acc = 0.0;
+        for (int64_t k = 0; k < K; k++) {
+            const float sq = xr[k] * xr[k];
+            acc += (double)sq;
+        }
+        float mean = (float)(acc / (double)K);
+        if (eps != 0.0f) mean = mean + eps;
+        const float rms = sqrtf(mean);
+        for (int64_t k = 0; k < K; k++) {
+            float v = xr[k] / rms;
+            if (gain) {
+                float g = gain[k];
+                if (gain_offset != 0.0f) g = g + gain_offset;
+                v = v * g;
+            }
+            yr[k] = v;
+        }
+    }
+    return 0;
+}
+
+/* The gated feed-forward front of a decoder layer (ml/zoo/transformer/transformer.go:1276-1287):
+ * x = normalize(x) when use_norm; gate = dense(x), up = dense(x); ff = Mul(activation(gate), up).
+ * The projections are gqo_qdense (fp64 accumulation over the exact fp32 weights). */
+int gqo_gated_ffn(int type, const float *x, int64_t M, int64_t K, int use_norm, const float *gain, float eps,
+                  float gain_offset, const uint8_t *Wgate, const float *bias_gate, const uint8_t *Wup,
+                  const float *bias_up, int64_t N, int act, float *y) {
+    float *xn = NULL, *gate = (float *)malloc((size_t)(M * N > 0 ? M * N : 1) * sizeof(float));
+    if (!gate) return -3;
+    int rc = 0;
+    if (use_norm) {
+        xn = (float *)malloc((size_t)(M * K > 0 ? M * K : 1) * sizeof(float));
+        if (!xn) { free(gate); return -3; }
+        rc = gqo_rmsnorm(x, M, K, gain, eps, gain_offset, xn);
+        x = xn;
+    }
+    if (!rc) rc = gqo_qdense(type, x, M, K, Wgate, N, bias_gate, act, gate);
+    if (!rc) rc = gqo_qdense(type, x, M, K, Wup, N, bias_up, GQO_ACT_NONE, y);
+    if (!rc)
+        for (int64_t i = 0; i < M * N; i++) y[i] = gate[i] * y[i];
+    free(gate);
+    free(xn);
+    return rc;
+}
+
 /* ---- gather ----------------------------------------------------------- */
 
 int gqo_embedding_lookup(int type, const uint8_t *table, int64_t vocab, int64_t K,

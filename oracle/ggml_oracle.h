@@ -12,6 +12,10 @@
  *   IQ4_NL dequant        pinned  - ml/nn/quantized_dense_test.go:406-452 KAT (LUT[8]=1, LUT[9]=13) + public table
  *   dense / bias / act    pinned  - reference KATs, unit-vector probes, linearity, SiLU KAT
  *   gather                pinned  - ml/nn/quantized_gather_test.go:17-169 KATs
+ *   RMS normalisation     pinned  - ml/layers/norm/rmsnorm_test.go:16-45 KAT, closed forms (constant rows,
+ *                                   scale invariance, unit norm), independent numpy form
+ *   gated feed-forward    pinned  - composition of the pinned parts (two dense products, activation, Mul),
+ *                                   checked against that composition written out in numpy
  *   Q4_K dequant          PARITY UNPINNED at the reference: the only implementation lives in the
  *                         third-party module github.com/gomlx/compute v0.1.2 (package gobackend),
  *                         which is not vendored.  Restated from the public GGML block_q4_K
@@ -72,6 +76,17 @@ int gqo_qdense_f32acc(int type, const float *x, int64_t M, int64_t K, const uint
  * dequant(table[indices[i], :]).  Returns -2 if an index is out of range. */
 int gqo_embedding_lookup(int type, const uint8_t *table, int64_t vocab, int64_t K,
                          const int32_t *indices, int64_t count, float *out);
+
+/* norm.RMSNorm over the last axis (ml/layers/norm/rmsnorm.go:78-113):
+ * y = x / sqrt(mean(x^2) + eps) * (gain + gain_offset); gain [K] or NULL (WithScale(false)). */
+int gqo_rmsnorm(const float *x, int64_t M, int64_t K, const float *gain, float eps, float gain_offset,
+                float *y);
+
+/* Gated feed-forward front (ml/zoo/transformer/transformer.go:1276-1287):
+ * y = act(xn . Wgate^T + bias_gate) * (xn . Wup^T + bias_up), xn = RMSNorm(x) if use_norm else x. */
+int gqo_gated_ffn(int type, const float *x, int64_t M, int64_t K, int use_norm, const float *gain, float eps,
+                  float gain_offset, const uint8_t *Wgate, const float *bias_gate, const uint8_t *Wup,
+                  const float *bias_up, int64_t N, int act, float *y);
 
 /* Epilogue of the fused op on one value (activation.Apply formulas,
  * ml/layers/activation/activation.go:161,195,222-243,274-286). */

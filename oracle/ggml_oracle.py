@@ -153,6 +153,27 @@ def np_qdense(t: int, x: np.ndarray, W: np.ndarray, bias: np.ndarray | None = No
     return y.reshape(x.shape[:-1] + (Wd.shape[0],))
 
 
+def np_rmsnorm(x: np.ndarray, gain: np.ndarray | None = None, eps: float = 1e-6, gain_offset: float = 0.0) -> np.ndarray:
+    """norm.RMSNorm over the last axis (ml/layers/norm/rmsnorm.go:78-113), evaluated in float64 and
+    rounded once: an independent form of the C routine, which rounds node by node."""
+    x64 = np.asarray(x, np.float32).astype(np.float64)
+    r = np.sqrt(np.mean(x64 * x64, axis=-1, keepdims=True) + float(np.float32(eps)))
+    y = x64 / r
+    if gain is not None:
+        y = y * (np.asarray(gain, np.float32).astype(np.float64) + float(np.float32(gain_offset)))
+    return y.astype(np.float32)
+
+
+def np_gated_ffn(t: int, x: np.ndarray, Wgate: np.ndarray, Wup: np.ndarray, bias_gate=None, bias_up=None, act: int = ACT_SILU,
+                 norm: tuple | None = None) -> np.ndarray:
+    """ff = activation(dense(xn, Wgate)) * dense(xn, Wup) (ml/zoo/transformer/transformer.go:1276-1287);
+    norm = (gain or None, eps, gain_offset) applies RMSNorm first."""
+    xn = np.asarray(x, np.float32)
+    if norm is not None:
+        xn = np_rmsnorm(xn, norm[0], norm[1], norm[2])
+    return (np_qdense(t, xn, Wgate, bias_gate, act).astype(np.float64) * np_qdense(t, xn, Wup, bias_up, ACT_NONE).astype(np.float64)).astype(np.float32)
+
+
 def np_embedding_lookup(t: int, table: np.ndarray, indices: np.ndarray) -> np.ndarray:
     """ggml.EmbeddingLookupDecomposed (ml/ggml/gather.go:21-49); indices [..., 1]."""
     idx = np.asarray(indices)
@@ -193,6 +214,8 @@ def lib() -> ctypes.CDLL:
         L.gqo_qdense.argtypes = [ci, vp, i64, i64, vp, i64, vp, ci, vp]
         L.gqo_qdense_f32acc.argtypes = [ci, vp, i64, i64, vp, i64, vp, ci, vp, ci]
         L.gqo_embedding_lookup.argtypes = [ci, vp, i64, i64, vp, i64, vp]
+        L.gqo_rmsnorm.argtypes = [vp, i64, i64, vp, ctypes.c_float, ctypes.c_float, vp]
+        L.gqo_gated_ffn.argtypes = [ci, vp, i64, i64, ci, vp, ctypes.c_float, ctypes.c_float, vp, vp, vp, vp, i64, ci, vp]
         L.gqo_activation.restype = ctypes.c_float
         L.gqo_activation.argtypes = [ci, ctypes.c_float]
         _LIB = L
@@ -243,3 +266,31 @@ def c_embedding_lookup(t: int, table: np.ndarray, K: int, indices: np.ndarray) -
     if rc:
         raise ValueError(f"gqo_embedding_lookup failed ({rc})")
     return out.reshape(indices.shape[:-1] + (K,))
+
+
+def c_rmsnorm(x: np.ndarray, gain: np.ndarray | None = None, eps: float = 1e-6, gain_offset: float = 0.0) -> np.ndarray:
+    x2 = np.ascontiguousarray(x, np.float32).reshape(-1, x.shape[-1])
+    g = None if gain is None else np.ascontiguousarray(gain, np.float32)
+    y = np.empty_like(x2)
+    rc = lib().gqo_rmsnorm(_p(x2), x2.shape[0], x2.shape[1], _p(g), eps, gain_offset, _p(y))
+    if rc:
+        raise ValueError(f"gqo_rmsnorm failed ({rc})")
+    return y.reshape(x.shape)
+
+
+def c_gated_ffn(t: int, x: np.ndarray, Wgate: np.ndarray, Wup: np.ndarray, bias_gate=None, bias_up=None, act: int = ACT_SILU,
+                norm: tuple | None = None) -> np.ndarray:
+    """norm = (gain or None, eps, gain_offset), or None for no normalisation."""
+    x2 = np.ascontiguousarray(x, np.float32).reshape(-1, x.shape[-1])
+    Wg, Wu = np.ascontiguousarray(Wgate, np.uint8), np.ascontiguousarray(Wup, np.uint8)
+    bg = None if bias_gate is None else np.ascontiguousarray(bias_gate, np.float32)
+    bu = None if bias_up is None else np.ascontiguousarray(bias_up, np.float32)
+    gain = None if norm is None or norm[0] is None else np.ascontiguousarray(norm[0], np.float32)
+    eps, off = (0.0, 0.0) if norm is None else (norm[1], norm[2])
+    M, K = x2.shape
+    N = Wg.shape[0]
+    y = np.empty((M, N), np.float32)
+    rc = lib().gqo_gated_ffn(t, _p(x2), M, K, 0 if norm is None else 1, _p(gain), eps, off, _p(Wg), _p(bg), _p(Wu), _p(bu), N, act, _p(y))
+    if rc:
+        raise ValueError(f"gqo_gated_ffn failed ({rc})")
+    return y.reshape(x.shape[:-1] + (N,))

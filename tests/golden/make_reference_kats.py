@@ -8,6 +8,8 @@ Sources (gomlx/gomlx):
   ml/nn/quantized_gather_test.go:17-74    Q8_0 gather basic / single
   ml/nn/quantized_gather_test.go:78-121   Q4_0 gather
   ml/nn/quantized_gather_test.go:125-169  IQ4_NL gather
+  ml/layers/norm/rmsnorm_test.go:16-45    RMSNorm over the last two axes of a [2, 3, 2] input (gain = ones),
+                                          stored flattened: rows of 6 values
 
 Nothing from the reference is imported or executed; run `python make_reference_kats.py`
 to regenerate the JSON next to this script.
@@ -67,6 +69,10 @@ kats = {
          "want": [[1.7616, 2.8577]], "tol": 1e-3},
         {"name": "iq4_nl_basic", "type": IQ4_NL, "w": iq_w, "x": [x_basic], "bias": None, "act": NONE,
          "want": [[14.0, 28.0]], "tol": 1e-4},
+    ],
+    "rmsnorm": [
+        {"name": "rmsnorm_two_axes", "x": [[3, 4, 5, 6, 7, 8], [6, 8, 10, 12, 14, 16]], "eps": 1e-6,
+         "want": [[0.52091914, 0.6945589, 0.86819863, 1.0418383, 1.2154781, 1.3891178]] * 2, "tol": 1e-3},
     ],
     "gather": [
         {"name": "q8_0_gather_basic", "type": Q8_0,

@@ -90,6 +90,69 @@ def test_gather_reference_kats(oracle, kats, impl):
         np.testing.assert_allclose(got, np.array(k["want"], np.float32), rtol=0, atol=k["tol"], err_msg=k["name"])
 
 
+@pytest.mark.parametrize("impl", ["np", "c"])
+def test_rmsnorm_reference_kat(oracle, kats, impl):
+    """ml/layers/norm/rmsnorm_test.go:16-45: gain of ones (the variable's initial value), default epsilon."""
+    fn = oracle.np_rmsnorm if impl == "np" else oracle.c_rmsnorm
+    for k in kats["rmsnorm"]:
+        x = np.array(k["x"], np.float32)
+        for gain in (None, np.ones(x.shape[-1], np.float32)):
+            np.testing.assert_allclose(fn(x, gain, k["eps"]), np.array(k["want"], np.float32), rtol=0, atol=k["tol"], err_msg=k["name"])
+        # the published digits are good to float32 precision, not just to the test's 1e-3
+        np.testing.assert_allclose(fn(x, None, k["eps"]), np.array(k["want"], np.float32), rtol=3e-7, atol=0)
+
+
+@pytest.mark.parametrize("impl", ["np", "c"])
+def test_rmsnorm_closed_forms(oracle, impl):
+    fn = oracle.np_rmsnorm if impl == "np" else oracle.c_rmsnorm
+    rng = np.random.default_rng(5)
+    # a constant row c normalises to sign(c) (eps = 0), times the gain plus its offset
+    x = np.full((1, 64), -3.5, np.float32)
+    gain = rng.normal(size=64).astype(np.float32)
+    np.testing.assert_allclose(fn(x, None, 0.0), -np.ones((1, 64), np.float32), rtol=2e-7)
+    np.testing.assert_allclose(fn(x, gain, 0.0, 1.0), -(gain + np.float32(1.0))[None, :], rtol=3e-7)
+    # without gain the output has unit mean square; scaling the input by a power of two changes nothing
+    x = rng.normal(size=(5, 300)).astype(np.float32)
+    y = fn(x, None, 0.0)
+    np.testing.assert_allclose(np.mean(y.astype(np.float64) ** 2, axis=-1), 1.0, rtol=1e-6)
+    assert np.array_equal(fn(x * np.float32(4.0), None, 0.0), y)
+    # a single value with epsilon: x / sqrt(x^2 + eps), here 3 / sqrt(9 + 7) = 0.75
+    np.testing.assert_allclose(fn(np.array([[3.0]], np.float32), None, 7.0), [[0.75]], rtol=1e-7)
+    # a wrong axis or a sum in place of the mean would fail this: rows are independent
+    x2 = np.stack([x[0], 10 * x[0]])
+    np.testing.assert_allclose(fn(x2, None, 0.0)[1], fn(x2, None, 0.0)[0], rtol=3e-7)
+
+
+def test_rmsnorm_c_against_numpy(oracle):
+    rng = np.random.default_rng(6)
+    x = (rng.normal(size=(7, 4096)) * 3).astype(np.float32)
+    gain = rng.normal(size=4096).astype(np.float32)
+    np.testing.assert_allclose(oracle.c_rmsnorm(x, gain, 1e-5, 1.0), oracle.np_rmsnorm(x, gain, 1e-5, 1.0), rtol=4e-7, atol=1e-30)
+
+
+@pytest.mark.parametrize("t", [Q8_0, Q4_K])
+def test_gated_ffn_is_the_composition_of_its_parts(oracle, t):
+    """activation(dense(xn, Wgate)) * dense(xn, Wup) written out with the pinned pieces."""
+    from gomlx_amd import synth
+    M, K, N = 3, 512, 24
+    Wg, Wu = synth.weights(t, 1, N, K), synth.weights(t, 2, N, K)
+    x = synth.activations(3, M, K)
+    gain = synth.normal(4, 0, K).astype(np.float32)
+    bg, bu = synth.normal(5, 0, N).astype(np.float32), synth.normal(6, 0, N).astype(np.float32)
+    for norm in (None, (gain, 1e-6, 1.0), (None, 1e-5, 0.0)):
+        xn = x if norm is None else oracle.c_rmsnorm(x, *norm)
+        want = oracle.c_qdense(t, xn, Wg, bg, oracle.ACT_SILU).astype(np.float64) * oracle.c_qdense(t, xn, Wu, bu, 0).astype(np.float64)
+        got_c = oracle.c_gated_ffn(t, x, Wg, Wu, bg, bu, oracle.ACT_SILU, norm)
+        got_np = oracle.np_gated_ffn(t, x, Wg, Wu, bg, bu, oracle.ACT_SILU, norm)
+        np.testing.assert_allclose(got_c, want.astype(np.float32), rtol=2e-7, atol=1e-30)
+        scale = np.max(np.abs(want))
+        assert np.max(np.abs(got_np - want)) / scale < 1e-5
+    # swapping the two matrices must change the result (the activation sits on the gate)
+    a = oracle.c_gated_ffn(t, x, Wg, Wu, None, None, oracle.ACT_SILU, None)
+    b = oracle.c_gated_ffn(t, x, Wu, Wg, None, None, oracle.ACT_SILU, None)
+    assert np.max(np.abs(a - b)) > 1e-3 * np.max(np.abs(a))
+
+
 # ------------------------------------------------------------------------------ closed forms
 
 D_PATTERNS = [0x0000, 0x0001, 0x0155, 0x03FF, 0x0400, 0x1234, 0x2E66, 0x3555, 0x3C00, 0x4000, 0x4200,

@@ -424,6 +424,125 @@ def test_randomized_problems(gpu, oracle):
         assert np.all(np.isfinite(got)) and err < (TOL_BF16 if bf16 else TOL_F32), (t, M, K, N, bf16, act, with_bias, err)
 
 
+# ------------------------------------------------------------------------------ callers around the dense layers
+
+def test_rmsnorm_reference_kat(gpu, kats):
+    for k in kats["rmsnorm"]:
+        x = np.array(k["x"], np.float32)
+        got = nn.rms_norm(dev(gpu, x), nn.RMSNorm(epsilon=k["eps"])).cpu().numpy()
+        np.testing.assert_allclose(got, np.array(k["want"], np.float32), rtol=0, atol=k["tol"], err_msg=k["name"])
+        ones = dev(gpu, np.ones(x.shape[-1], np.float32))
+        got = nn.rms_norm(dev(gpu, x), nn.RMSNorm(gain=ones, epsilon=k["eps"])).cpu().numpy()
+        np.testing.assert_allclose(got, np.array(k["want"], np.float32), rtol=0, atol=k["tol"], err_msg=k["name"])
+
+
+@pytest.mark.parametrize("M,K", [(1, 1), (3, 33), (2, 4096), (70, 1000)])
+def test_rmsnorm_parity(gpu, oracle, M, K):
+    x = (synth.activations(300, M, K) * 2.5).astype(np.float32)
+    gain = synth.normal(301, 0, K).astype(np.float32)
+    for g, eps, off in ((None, 1e-6, 0.0), (gain, 1e-5, 0.0), (gain, 1e-6, 1.0), (None, 0.0, 0.0)):
+        got = nn.rms_norm(dev(gpu, x), nn.RMSNorm(None if g is None else dev(gpu, g), eps, off)).cpu().numpy()
+        want = oracle.c_rmsnorm(x, g, eps, off)
+        np.testing.assert_allclose(got, want, rtol=2e-6, atol=1e-30)
+
+
+def gated_case(gpu, oracle, t, M, K, N, act, norm_kind, with_bias, seed):
+    Wg, Wu = synth.weights(t, seed, N, K), synth.weights(t, seed + 1, N, K)
+    x = synth.activations(seed + 2, M, K)
+    gain = (synth.normal(seed + 3, 0, K) * 0.5 + 1.0).astype(np.float32)
+    bg = synth.normal(seed + 4, 0, N).astype(np.float32) * 0.1 if with_bias else None
+    bu = synth.normal(seed + 5, 0, N).astype(np.float32) * 0.1 if with_bias else None
+    norm = {0: None, 1: (gain, 1e-6, 0.0), 2: (gain, 1e-5, 1.0), 3: (None, 1e-6, 0.0)}[norm_kind]
+    cfg = None if norm is None else nn.RMSNorm(None if norm[0] is None else dev(gpu, norm[0]), norm[1], norm[2])
+    got = nn.gated_feed_forward(dev(gpu, x), dev(gpu, Wg), dev(gpu, Wu), Quantization(ggml_type=t), BACKEND_ACT[act],
+                                None if bg is None else dev(gpu, bg), None if bu is None else dev(gpu, bu), cfg)
+    gpu.cuda.synchronize()
+    got = got.cpu().numpy()
+    want = oracle.c_gated_ffn(t, x, Wg, Wu, bg, bu, act, norm)
+    # scale of the product of the two contractions: the error of either factor is bounded on its own
+    # contraction's scale, so the product is judged on max|gate| * max|up| (pre-activation for the gate)
+    xn = x if norm is None else oracle.c_rmsnorm(x, *norm)
+    g_pre, g_act = oracle.c_qdense(t, xn, Wg, bg, 0), oracle.c_qdense(t, xn, Wg, bg, act)
+    up = oracle.c_qdense(t, xn, Wu, bu, 0)
+    scale = max(float(np.max(np.abs(g_pre))), float(np.max(np.abs(g_act)))) * float(np.max(np.abs(up))) or 1.0
+    err = float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)))) / scale
+    assert got.shape == (M, N) and np.all(np.isfinite(got))
+    return err
+
+
+@pytest.mark.parametrize("t", ALL_TYPES)
+def test_gated_feed_forward_decode(gpu, oracle, t):
+    """Fused path: up to 16 rows, K a multiple of 256 (one launch over both matrices)."""
+    for i, (M, K, N, act, norm_kind, with_bias) in enumerate([
+            (1, 4096, 1000, 3, 1, False), (1, 512, 8, 3, 0, False), (2, 2304, 333, 1, 2, True), (1, 256, 1, 3, 3, True),
+            (4, 1536, 130, 5, 1, True), (16, 1024, 70, 3, 2, False), (1, 4608, 64, 2, 0, True), (3, 768, 1030, 4, 3, False)]):
+        err = gated_case(gpu, oracle, t, M, K, N, act, norm_kind, with_bias, 400 + 10 * i + t)
+        assert err < 2 * TOL_F32, (t, M, K, N, act, norm_kind, with_bias, err)
+
+
+@pytest.mark.parametrize("t", ALL_TYPES)
+def test_gated_feed_forward_composed(gpu, oracle, t):
+    """Shapes outside the fused path (more rows, ragged K for the 32-value formats) are composed of
+    dense calls; those from 17 rows on contract fp16 operands."""
+    ragged_k = 160 if t in (Q4_0, Q8_0, IQ4_NL) else 768
+    for i, (M, K, N, act, norm_kind, with_bias) in enumerate([
+            (17, 1024, 96, 3, 1, True), (40, 512, 256, 3, 0, False), (2, ragged_k, 50, 3, 2, True),
+            (130, 1024, 128, 1, 1, False)]):
+        err = gated_case(gpu, oracle, t, M, K, N, act, norm_kind, with_bias, 600 + 10 * i + t)
+        assert err < 2 * TOL_F32, (t, M, K, N, act, norm_kind, with_bias, err)
+
+
+@pytest.mark.parametrize("t", ALL_TYPES)
+def test_dense_with_rmsnorm_prologue(gpu, oracle, t):
+    for i, (M, K, N, act) in enumerate([(1, 4096, 512, 0), (3, 768, 100, 3), (16, 256, 33, 0), (20, 512, 64, 0), (1, 2304, 1, 5)]):
+        W = synth.weights(t, 700 + i, N, K)
+        x = (synth.activations(701 + i, M, K) * 3.0).astype(np.float32)
+        gain = (synth.normal(702 + i, 0, K) * 0.5 + 1.0).astype(np.float32)
+        bias = synth.normal(703 + i, 0, N).astype(np.float32) * 0.1
+        got = nn.quantized_dense(dev(gpu, x), dev(gpu, W), Quantization(ggml_type=t), dev(gpu, bias), BACKEND_ACT[act],
+                                 norm=nn.RMSNorm(dev(gpu, gain), 1e-6, 0.0)).cpu().numpy()
+        xn = oracle.c_rmsnorm(x, gain, 1e-6, 0.0)
+        want = oracle.c_qdense(t, xn, W, bias, act)
+        pre = oracle.c_qdense(t, xn, W, bias, 0)
+        scale = max(float(np.max(np.abs(want))), float(np.max(np.abs(pre))))
+        err = float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)))) / scale
+        assert err < TOL_F32, (t, M, K, N, act, err)
+
+
+def test_gated_feed_forward_full_size(gpu, oracle):
+    """Llama-3-8B feed-forward front at full size (Q4_K, 4096 -> 14336 twice, RMSNorm, SiLU), checked on a
+    sample of output columns against the oracle and in full against the unfused calls of this library."""
+    t, K, N = Q4_K, 4096, 14336
+    Wg, Wu = synth.weights(t, 800, N, K), synth.weights(t, 801, N, K)
+    x = synth.activations(802, 1, K)
+    gain = (synth.normal(803, 0, K) * 0.5 + 1.0).astype(np.float32)
+    q = Quantization(ggml_type=t)
+    xd, Wgd, Wud, gd = dev(gpu, x), dev(gpu, Wg), dev(gpu, Wu), dev(gpu, gain)
+    cfg = nn.RMSNorm(gd, 1e-5, 0.0)
+    got = nn.gated_feed_forward(xd, Wgd, Wud, q, Activation.SILU, norm=cfg).cpu().numpy()
+    xn = nn.rms_norm(xd, cfg)
+    unfused = (nn.quantized_dense(xn, Wgd, q, None, Activation.SILU) * nn.quantized_dense(xn, Wud, q)).cpu().numpy()
+    scale = float(np.max(np.abs(unfused)))
+    assert np.max(np.abs(got - unfused)) / scale < 1e-4
+    cols = np.arange(0, N, 97)
+    want = oracle.c_gated_ffn(t, x, Wg[cols], Wu[cols], None, None, 3, (gain, 1e-5, 0.0))
+    assert np.max(np.abs(got[:, cols].astype(np.float64) - want)) / float(np.max(np.abs(want))) < 2 * TOL_F32
+
+
+def test_gated_feed_forward_rejects_bad_arguments(gpu):
+    q = Quantization(ggml_type=Q8_0)
+    x = dev(gpu, np.zeros((1, 64), np.float32))
+    W = dev(gpu, np.zeros((4, 68), np.uint8))
+    with pytest.raises(ValueError):
+        nn.gated_feed_forward(x, W, dev(gpu, np.zeros((5, 68), np.uint8)), q, Activation.SILU)
+    with pytest.raises(ValueError):
+        nn.gated_feed_forward(x, W, W, q, Activation.SILU, norm=nn.RMSNorm(dev(gpu, np.ones(32, np.float32))))
+    with pytest.raises(Exception):
+        nn.gated_feed_forward(dev(gpu, np.zeros((1, 96), np.float32)), W, W, q, Activation.SILU)
+    with pytest.raises(Exception):
+        nn.rms_norm(x, nn.RMSNorm(epsilon=-1.0))
+
+
 # ------------------------------------------------------------------------------ benchmark configurations, full size
 
 def test_config0_q8_0_gemv_4096(gpu, oracle):
