@@ -371,23 +371,61 @@ int gq_rmsnorm_f32(const float *dX, int64_t M, int64_t K, const float *dGain, fl
     return launch_rmsnorm(dX, M, K, dGain, gain_offset, eps, dY, (hipStream_t)stream);
 }
 
-int gq_qdense_norm_f32(int type, const float *dX, int64_t M, int64_t K, const gq_rmsnorm *norm, const void *dW, int64_t N,
-                       const float *dBias, int act, float *dY, void *stream) {
-    if (!norm) return gq_qdense_f32(type, dX, M, K, dW, N, dBias, act, dY, stream);
-    if (int rc = check_dense_args("gq_qdense_norm_f32", type, dX, M, K, dW, N, dBias, act, dY, 4)) return rc;
-    if (!(norm->eps >= 0.f)) return fail(GQ_ERR_INVALID, "gq_qdense_norm_f32: epsilon must be >= 0");
-    if (norm->dGain && !aligned_to(norm->dGain, 4)) return fail(GQ_ERR_INVALID, "gq_qdense_norm_f32: gain must be 4-byte aligned");
+int gq_qdense_block_f32(int type, const float *dX, int64_t M, int64_t K, const gq_rmsnorm *norm, const void *dW, int64_t N,
+                        const float *dBias, int act, const float *dResidual, float *dY, void *stream) {
+    if (!norm && !dResidual) return gq_qdense_f32(type, dX, M, K, dW, N, dBias, act, dY, stream);
+    if (int rc = check_dense_args("gq_qdense_block_f32", type, dX, M, K, dW, N, dBias, act, dY, 4)) return rc;
+    if (norm && !(norm->eps >= 0.f)) return fail(GQ_ERR_INVALID, "gq_qdense_block_f32: epsilon must be >= 0");
+    if (norm && norm->dGain && !aligned_to(norm->dGain, 4)) return fail(GQ_ERR_INVALID, "gq_qdense_block_f32: gain must be 4-byte aligned");
+    if (dResidual && !aligned_to(dResidual, 4)) return fail(GQ_ERR_INVALID, "gq_qdense_block_f32: residual must be 4-byte aligned");
     if (M == 0 || N == 0) return GQ_OK;
     if (int rc = use_device()) return rc;
-    const RmsNorm rn{norm->dGain, norm->eps, norm->gain_offset};
+    RmsNorm rn{nullptr, 0.f, 0.f};
+    if (norm) rn = RmsNorm{norm->dGain, norm->eps, norm->gain_offset};
     if (gemv_ks_ext_supported(type, M, K, N, dX, rn.gain))
-        return launch_gemv_ks_ext(type, dX, M, K, &rn, (const uint8_t *)dW, dBias, nullptr, nullptr, N, act, dY, (hipStream_t)stream);
-    // composed: normalised activations into the stream's second workspace, then the dense call
-    void *ws = nullptr;
-    if (int rc = stream_workspace((hipStream_t)stream, (size_t)M * (size_t)K * sizeof(float), &ws, 1)) return rc;
-    float *xn = static_cast<float *>(ws);
-    if (int rc = launch_rmsnorm(dX, M, K, rn.gain, rn.gain_offset, rn.eps, xn, (hipStream_t)stream)) return rc;
-    return gq_qdense_f32(type, xn, M, K, dW, N, dBias, act, dY, stream);
+        return launch_gemv_ks_ext(type, dX, M, K, norm ? &rn : nullptr, (const uint8_t *)dW, dBias, nullptr, nullptr, dResidual, N, act, dY,
+                                  (hipStream_t)stream);
+    // composed: normalised activations into the stream's second workspace, the dense call, then the residual
+    const float *x = dX;
+    if (norm) {
+        void *ws = nullptr;
+        if (int rc = stream_workspace((hipStream_t)stream, (size_t)M * (size_t)K * sizeof(float), &ws, 1)) return rc;
+        float *xn = static_cast<float *>(ws);
+        if (int rc = launch_rmsnorm(dX, M, K, rn.gain, rn.gain_offset, rn.eps, xn, (hipStream_t)stream)) return rc;
+        x = xn;
+    }
+    if (int rc = gq_qdense_f32(type, x, M, K, dW, N, dBias, act, dY, stream)) return rc;
+    if (dResidual) return launch_add(dY, dResidual, dY, M * N, (hipStream_t)stream);
+    return GQ_OK;
+}
+
+int gq_qdense_norm_f32_batch(int count, const gq_dense_desc *descs, const gq_rmsnorm *norm, void *stream) {
+    if (!norm) return gq_qdense_f32_batch(count, descs, stream);
+    if (count < 0 || (count > 0 && !descs)) return fail(GQ_ERR_INVALID, "gq_qdense_norm_f32_batch: bad descriptor list");
+    for (int i = 0; i < count; i++) {
+        const gq_dense_desc &d = descs[i];
+        if (int rc = check_dense_args("gq_qdense_norm_f32_batch", d.type, d.dX, d.M, d.K, d.dW, d.N, d.dBias, d.act, d.dY, 4)) return rc;
+    }
+    if (!(norm->eps >= 0.f)) return fail(GQ_ERR_INVALID, "gq_qdense_norm_f32_batch: epsilon must be >= 0");
+    if (count == 0) return GQ_OK;
+    if (int rc = use_device()) return rc;
+    // one launch when every problem is a batch-1 projection of one type and one K that the K-sliced GEMV takes
+    bool merged = count >= 2 && count <= 8;
+    XsBatchItem items[8];
+    for (int i = 0; i < count && merged; i++) {
+        const gq_dense_desc &d = descs[i];
+        merged = d.type == descs[0].type && d.K == descs[0].K && d.M == 1 && d.N > 0 && gemv_ks_ext_supported(d.type, 1, d.K, d.N, d.dX, norm->dGain);
+        if (merged) items[i] = XsBatchItem{d.dX, (const uint8_t *)d.dW, d.dBias, d.dY, d.K, d.N, d.act};
+    }
+    if (merged) {
+        const RmsNorm rn{norm->dGain, norm->eps, norm->gain_offset};
+        return launch_gemv_ks_batch_norm(descs[0].type, count, items, &rn, (hipStream_t)stream);
+    }
+    for (int i = 0; i < count; i++) {
+        const gq_dense_desc &d = descs[i];
+        if (int rc = gq_qdense_block_f32(d.type, d.dX, d.M, d.K, norm, d.dW, d.N, d.dBias, d.act, nullptr, d.dY, stream)) return rc;
+    }
+    return GQ_OK;
 }
 
 int gq_qdense_gated_f32(int type, const float *dX, int64_t M, int64_t K, const gq_rmsnorm *norm, const void *dWgate,
@@ -401,8 +439,8 @@ int gq_qdense_gated_f32(int type, const float *dX, int64_t M, int64_t K, const g
     RmsNorm rn{nullptr, 0.f, 0.f};
     if (norm) rn = RmsNorm{norm->dGain, norm->eps, norm->gain_offset};
     if (gemv_ks_ext_supported(type, M, K, N, dX, rn.gain))
-        return launch_gemv_ks_ext(type, dX, M, K, norm ? &rn : nullptr, (const uint8_t *)dWgate, dBiasGate, (const uint8_t *)dWup, dBiasUp, N,
-                                  act, dY, (hipStream_t)stream);
+        return launch_gemv_ks_ext(type, dX, M, K, norm ? &rn : nullptr, (const uint8_t *)dWgate, dBiasGate, (const uint8_t *)dWup, dBiasUp,
+                                  nullptr, N, act, dY, (hipStream_t)stream);
     // composed: [normalised activations,] act(gate) into the stream's second workspace, up into y, y *= act(gate)
     const size_t xn_bytes = norm ? ((size_t)M * (size_t)K * sizeof(float) + 255) / 256 * 256 : 0;
     void *ws = nullptr;

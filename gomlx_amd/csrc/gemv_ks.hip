@@ -17,36 +17,10 @@ __global__ __launch_bounds__(512) void gemv_ks_kernel(const void *__restrict__ X
                         (int)blockIdx.x, lds);
 }
 
-// Several independent batch-1 problems of one format in a single launch: workgroups
-// [wg_begin, next wg_begin) belong to problem i.  This is how the projections of a decoder layer
-// that do not depend on each other (q/k/v, gate/up) share one submission.  Every problem runs in
-// groups of two row-steps, both in flight (its iters is a multiple of 2): measured on the seven
-// projections of a Llama-3-8B layer, groups of 2 take 23.8 us, 3 / 2 in flight 24.1, 4 / 3 24.7 .. 25.4,
-// 8 / 4 25.6 - the finer rounding of rows per workgroup balances the problems better than a deeper
-// window helps.
-constexpr int kMaxBatchKs = 8;
-constexpr int kBatchPF = 2;
-struct KsProblem {
-    const float *x;
-    const uint8_t *W;
-    const float *bias;
-    float *y;
-    int64_t row_bytes;
-    int N, iters, nslices, half_tail, waves, act, wg_begin;
-};
-struct KsBatch {
-    int count;
-    KsProblem p[kMaxBatchKs];
-};
-
 template <int T>
 __global__ __launch_bounds__(512) void gemv_ks_batch_kernel(const KsBatch b) {
     extern __shared__ uint32_t lds[];
-    int i = 0;
-#pragma unroll
-    for (int j = 1; j < kMaxBatchKs; j++)
-        if (j < b.count && (int)blockIdx.x >= b.p[j].wg_begin) i = j;
-    const KsProblem &q = b.p[i];
+    const KsProblem &q = b.p[ks_batch_problem(b, (int)blockIdx.x)];
     ks_body<T, kBatchPF, kBatchPF>(q.x, q.W, q.bias, q.y, q.N, q.row_bytes, q.iters, q.nslices, q.half_tail, q.act, q.waves,
                      (int)blockIdx.x - q.wg_begin, lds);
 }
@@ -82,36 +56,13 @@ int launch_ks(const void *x, int x_bf16, int64_t M, int64_t K, const uint8_t *W,
     }
 }
 
-// One launch for `count` batch-1 problems: the chip's workgroup slots are shared out in proportion
-// to each problem's weight bytes, so every CU streams for about the same time.
 template <int T>
 int launch_ks_batch(int count, const XsBatchItem *items, hipStream_t s) {
     KsBatch b;
-    b.count = count;
-    const int cus = device_cu_count();
-    double total = 0.0;
-    for (int i = 0; i < count; i++) total += (double)gq_row_bytes(T, items[i].K) * (double)items[i].N;
-    size_t shmem = 0;
-    int wg = 0;
-    for (int i = 0; i < count; i++) {
-        const XsBatchItem &it = items[i];
-        KsProblem q;
-        q.x = it.x; q.W = it.W; q.bias = it.bias; q.y = it.y; q.N = (int)it.N; q.act = it.act;
-        q.row_bytes = (int64_t)gq_row_bytes(T, it.K);
-        if (!ks_split(it.K, q.waves, q.nslices, q.half_tail)) return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv_ks batch: unsupported K");
-        int64_t share = (int64_t)((double)cus * ((double)q.row_bytes * (double)it.N) / total + 0.5);
-        if (share < 1) share = 1;
-        int64_t iters = (it.N + share * 8 - 1) / (share * 8);
-        iters = (iters + kBatchPF - 1) / kBatchPF * kBatchPF;
-        if (iters > kMaxItersKs) iters = kMaxItersKs;
-        q.iters = (int)iters;
-        q.wg_begin = wg;
-        wg += (int)((it.N + iters * 8 - 1) / (iters * 8));
-        b.p[i] = q;
-        const size_t need = ks_lds_bytes(q.waves, q.iters);
-        if (need > shmem) shmem = need;
-    }
-    return launch(gemv_ks_batch_kernel<T>, dim3((unsigned)wg), dim3(512), shmem, s, b);
+    size_t shmem;
+    int wgs;
+    if (int rc = plan_ks_batch<T>(count, items, b, shmem, wgs)) return rc;
+    return launch(gemv_ks_batch_kernel<T>, dim3((unsigned)wgs), dim3(512), shmem, s, b);
 }
 
 }  // namespace

@@ -18,8 +18,29 @@ __global__ __launch_bounds__(512) void gemv_ks_ext_kernel(const float *__restric
                                                           int64_t row_bytes, int iters, int nslices, int half_tail, int act,
                                                           const KsExt ext) {
     extern __shared__ uint32_t lds[];
+    KsExt e = ext;
+    if (e.residual) e.residual += (int64_t)blockIdx.y * N;
     ks_body<T, PF, WIN, true>(X + (int64_t)blockIdx.y * K, W, bias, Y + (int64_t)blockIdx.y * N, N, row_bytes, iters, nslices, half_tail,
-                              act, (int)(blockDim.x >> 6), (int)blockIdx.x, lds, &ext);
+                              act, (int)(blockDim.x >> 6), (int)blockIdx.x, lds, &e);
+}
+
+// Batched submission (several batch-1 projections of one format in one launch) with one RMS
+// normalisation shared by all of them: the q/k/v projections behind a layer's input norm.
+template <int T>
+__global__ __launch_bounds__(512) void gemv_ks_batch_ext_kernel(const KsBatch b, const KsExt ext) {
+    extern __shared__ uint32_t lds[];
+    const KsProblem &q = b.p[ks_batch_problem(b, (int)blockIdx.x)];
+    ks_body<T, kBatchPF, kBatchPF, true>(q.x, q.W, q.bias, q.y, q.N, q.row_bytes, q.iters, q.nslices, q.half_tail, q.act, q.waves,
+                                         (int)blockIdx.x - q.wg_begin, lds, &ext);
+}
+
+template <int T>
+int launch_batch_ext(int count, const XsBatchItem *items, const KsExt &ext, hipStream_t s) {
+    KsBatch b;
+    size_t shmem;
+    int wgs;
+    if (int rc = plan_ks_batch<T>(count, items, b, shmem, wgs)) return rc;
+    return launch(gemv_ks_batch_ext_kernel<T>, dim3((unsigned)wgs), dim3(512), shmem, s, b, ext);
 }
 
 template <int T, int PF>
@@ -80,6 +101,12 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float *__restrict__ 
     }
 }
 
+// y[i] = a[i] + r[i]; y may be a or r (one thread per element)
+__global__ __launch_bounds__(256) void add_kernel(const float *a, const float *r, float *y, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) y[i] = a[i] + r[i];
+}
+
 // y[i] *= g[i]
 __global__ __launch_bounds__(256) void mul_inplace_kernel(float *__restrict__ y, const float *__restrict__ g, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -94,11 +121,12 @@ bool gemv_ks_ext_supported(int type, int64_t M, int64_t K, int64_t N, const void
     return gemv_ks_supported(type, K, N, x);
 }
 
-int launch_gemv_ks_ext(int type, const float *x, int64_t M, int64_t K, const RmsNorm *norm, const uint8_t *W, const float *bias,
-                       const uint8_t *W2, const float *bias2, int64_t N, int act, float *y, hipStream_t s) {
+namespace {
+KsExt make_ext(const RmsNorm *norm, int64_t K, const uint8_t *W2, const float *bias2, const float *residual) {
     KsExt ext = {};
     ext.W2 = W2;
     ext.bias2 = bias2;
+    ext.residual = residual;
     if (norm) {
         ext.norm = 1;
         ext.gain = norm->gain;
@@ -106,6 +134,13 @@ int launch_gemv_ks_ext(int type, const float *x, int64_t M, int64_t K, const Rms
         ext.eps = norm->eps;
         ext.inv_k = 1.0f / (float)K;
     }
+    return ext;
+}
+}  // namespace
+
+int launch_gemv_ks_ext(int type, const float *x, int64_t M, int64_t K, const RmsNorm *norm, const uint8_t *W, const float *bias,
+                       const uint8_t *W2, const float *bias2, const float *residual, int64_t N, int act, float *y, hipStream_t s) {
+    const KsExt ext = make_ext(norm, K, W2, bias2, residual);
     switch (type) {
     case kQ4_0: return launch_ext<kQ4_0>(x, M, K, W, N, bias, act, y, ext, s);
     case kQ8_0: return launch_ext<kQ8_0>(x, M, K, W, N, bias, act, y, ext, s);
@@ -114,6 +149,24 @@ int launch_gemv_ks_ext(int type, const float *x, int64_t M, int64_t K, const Rms
     case kIQ4_NL: return launch_ext<kIQ4_NL>(x, M, K, W, N, bias, act, y, ext, s);
     default: return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv_ks: ggml type %d is not implemented", type);
     }
+}
+
+// all problems share K (one normalised input feeds them)
+int launch_gemv_ks_batch_norm(int type, int count, const XsBatchItem *items, const RmsNorm *norm, hipStream_t s) {
+    if (count < 1 || count > kMaxBatchKs) return fail(GQ_ERR_INVALID, "gemv batch: %d problems (1..%d supported per launch)", count, kMaxBatchKs);
+    const KsExt ext = make_ext(norm, items[0].K, nullptr, nullptr, nullptr);
+    switch (type) {
+    case kQ4_0: return launch_batch_ext<kQ4_0>(count, items, ext, s);
+    case kQ8_0: return launch_batch_ext<kQ8_0>(count, items, ext, s);
+    case kQ4_K: return launch_batch_ext<kQ4_K>(count, items, ext, s);
+    case kQ6_K: return launch_batch_ext<kQ6_K>(count, items, ext, s);
+    case kIQ4_NL: return launch_batch_ext<kIQ4_NL>(count, items, ext, s);
+    default: return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv batch: ggml type %d is not implemented", type);
+    }
+}
+
+int launch_add(const float *a, const float *r, float *y, int64_t n, hipStream_t s) {
+    return launch(add_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, a, r, y, n);
 }
 
 int launch_rmsnorm(const float *x, int64_t M, int64_t K, const float *gain, float gain_offset, float eps, float *y, hipStream_t s) {

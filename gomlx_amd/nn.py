@@ -167,12 +167,14 @@ def gated_feed_forward(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor
 
 
 def quantized_dense(x: torch.Tensor, weights: torch.Tensor, quant: Quantization, bias: torch.Tensor | None = None,
-                    *optional_activation: Activation, norm: RMSNorm | None = None) -> torch.Tensor:
+                    *optional_activation: Activation, norm: RMSNorm | None = None,
+                    residual: torch.Tensor | None = None) -> torch.Tensor:
     """nn.QuantizedDense for the GGML scheme: y = activation(x @ dequant(weights)^T + bias).
 
     x: [batch..., K] float32 or bfloat16; weights: [N, bytesPerRow] uint8; bias: [N] float32.
-    Returns [batch..., N] float32.  ``norm`` applies an RMS normalisation to x first (float32 x only):
-    Model.normalize followed by a projection, ml/zoo/transformer/transformer.go:1099-1101.
+    Returns [batch..., N] float32.  ``norm`` applies an RMS normalisation to x first and ``residual``
+    ([batch..., N] float32) is added to the result (float32 x only): Model.normalize followed by a
+    projection and Add(residual, ...) after it, ml/zoo/transformer/transformer.go:1099-1101, 1045, 1055.
     """
     if len(optional_activation) > 1:
         raise ValueError(f"quantized_dense can only take one optional activation, got {optional_activation}")
@@ -206,12 +208,17 @@ def quantized_dense(x: torch.Tensor, weights: torch.Tensor, quant: Quantization,
     _lib.check(L.gq_qdense_check(quant.ggml_type, xd, M, K_in, N, rb, blen, act.to_backend(), ctypes.byref(K)))
     _lib.init(x.device.index or 0)
     y = torch.empty(x.shape[:-1] + (N,), dtype=torch.float32, device=x.device)
-    if norm is not None:
+    if norm is not None or residual is not None:
         if xd != _lib.F32:
-            raise _lib.NotImplementedByBackend(_lib.ERR_NOT_IMPLEMENTED, "a fused normalisation takes float32 activations")
-        d = norm._desc(K.value)
-        _lib.check(L.gq_qdense_norm_f32(quant.ggml_type, x.data_ptr(), M, K.value, ctypes.byref(d), weights.data_ptr(), N,
-                                        None if bias is None else bias.data_ptr(), act.to_backend(), y.data_ptr(), _stream_ptr(x)))
+            raise _lib.NotImplementedByBackend(_lib.ERR_NOT_IMPLEMENTED, "a fused normalisation or residual takes float32 activations")
+        d = None if norm is None else norm._desc(K.value)
+        if residual is not None:
+            _require_cuda("residual", residual)
+            if residual.dtype != torch.float32 or tuple(residual.shape) != tuple(y.shape):
+                raise ValueError(f"residual must be a float32 tensor of shape {tuple(y.shape)}")
+        _lib.check(L.gq_qdense_block_f32(quant.ggml_type, x.data_ptr(), M, K.value, None if d is None else ctypes.byref(d),
+                                         weights.data_ptr(), N, None if bias is None else bias.data_ptr(), act.to_backend(),
+                                         None if residual is None else residual.data_ptr(), y.data_ptr(), _stream_ptr(x)))
         return y
     fn = L.gq_qdense_f32 if xd == _lib.F32 else L.gq_qdense_bf16
     _lib.check(fn(quant.ggml_type, x.data_ptr(), M, K.value, weights.data_ptr(), N,
@@ -246,8 +253,10 @@ def quantized_gather(table: torch.Tensor, indices: torch.Tensor, quant: Quantiza
     return out
 
 
-def quantized_dense_batch(problems) -> list:
-    """Several independent nn.QuantizedDense calls submitted together (gq_qdense_f32_batch).
+def quantized_dense_batch(problems, norm: RMSNorm | None = None) -> list:
+    """Several independent nn.QuantizedDense calls submitted together (gq_qdense_f32_batch); with
+    ``norm`` every problem's activations are RMS-normalised first (the q/k/v projections behind a
+    layer's input norm, gq_qdense_norm_f32_batch).
 
     ``problems`` is a sequence of ``(x, weights, quant, bias, activation)`` tuples with float32
     activations; returns the list of outputs.  Results equal those of separate calls; batch-1
@@ -282,5 +291,9 @@ def quantized_dense_batch(problems) -> list:
         d.dW, d.N, d.dBias, d.dY = weights.data_ptr(), N, (None if bias is None else bias.data_ptr()), y.data_ptr()
     if problems:
         _lib.init(problems[0][0].device.index or 0)
-        _lib.check(L.gq_qdense_f32_batch(len(problems), descs, _stream_ptr(problems[0][0])))
+        if norm is None:
+            _lib.check(L.gq_qdense_f32_batch(len(problems), descs, _stream_ptr(problems[0][0])))
+        else:
+            d = norm._desc(problems[0][0].shape[-1])
+            _lib.check(L.gq_qdense_norm_f32_batch(len(problems), descs, ctypes.byref(d), _stream_ptr(problems[0][0])))
     return outs

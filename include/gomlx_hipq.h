@@ -138,16 +138,25 @@ typedef struct {
     float eps;
     float gain_offset;
 } gq_rmsnorm;
-/* gq_qdense_f32 applied to RMSNorm(x) (Model.normalize followed by a projection,
- * transformer.go:1099-1101 for q/k/v); norm == NULL is plain gq_qdense_f32.  Up to 16 rows run
- * in the decode GEMV itself when K is a multiple of 256 and x and gain are 16-byte aligned. */
-int gq_qdense_norm_f32(int type, const float *dX, int64_t M, int64_t K, const gq_rmsnorm *norm,
-                       const void *dW, int64_t N, const float *dBias, int act, float *dY,
-                       void *stream);
+/* A projection with its neighbours in the layer: y = residual + act(RMSNorm(x) . W^T + bias)
+ * (Model.normalize followed by a projection, transformer.go:1099-1101; Add(residual, ...) after
+ * the output and down projections, :1045, :1055, :1291-1292).  norm and dResidual may each be
+ * NULL (both NULL is plain gq_qdense_f32); dY may be dResidual itself (a residual stream updated
+ * in place).  Up to 16 rows run in the decode GEMV itself when K is a multiple of 256 and x and
+ * gain are 16-byte aligned; other shapes are composed of an RMSNorm kernel, the dense call and
+ * an addition, and use a per-stream workspace. */
+int gq_qdense_block_f32(int type, const float *dX, int64_t M, int64_t K, const gq_rmsnorm *norm,
+                        const void *dW, int64_t N, const float *dBias, int act,
+                        const float *dResidual, float *dY, void *stream);
+/* gq_qdense_f32_batch with one RMS normalisation applied to the activations of every problem:
+ * the q/k/v projections behind a layer's input norm (transformer.go:1099-1130) in one launch
+ * when all are batch-1 problems of one type and one K. */
+int gq_qdense_norm_f32_batch(int count, const gq_dense_desc *descs, const gq_rmsnorm *norm,
+                             void *stream);
 /* The gated feed-forward front (transformer.go:1279-1287, after the pre_feedforward_norm of
  * :1276 when norm != NULL): y = act(xn . Wgate^T + bgate) * (xn . Wup^T + bup), xn = RMSNorm(x)
  * or x.  Both matrices are [N, gq_row_bytes(type, K)] of one type.  Same fast-path conditions as
- * gq_qdense_norm_f32; other shapes are composed of dense calls and use a per-stream workspace. */
+ * gq_qdense_block_f32; other shapes are composed of dense calls and use a per-stream workspace. */
 int gq_qdense_gated_f32(int type, const float *dX, int64_t M, int64_t K, const gq_rmsnorm *norm,
                         const void *dWgate, const float *dBiasGate, const void *dWup,
                         const float *dBiasUp, int64_t N, int act, float *dY, void *stream);

@@ -493,20 +493,59 @@ def test_gated_feed_forward_composed(gpu, oracle, t):
 
 
 @pytest.mark.parametrize("t", ALL_TYPES)
-def test_dense_with_rmsnorm_prologue(gpu, oracle, t):
-    for i, (M, K, N, act) in enumerate([(1, 4096, 512, 0), (3, 768, 100, 3), (16, 256, 33, 0), (20, 512, 64, 0), (1, 2304, 1, 5)]):
+def test_dense_with_rmsnorm_and_residual(gpu, oracle, t):
+    """y = residual + act(RMSNorm(x) . W^T + b): norm alone, residual alone, both; fused shapes (up to 16
+    rows, K % 256 == 0) and composed ones; the residual updated in place."""
+    for i, (M, K, N, act, use_norm, use_res) in enumerate([
+            (1, 4096, 512, 0, True, False), (3, 768, 100, 3, True, True), (16, 256, 33, 0, False, True), (20, 512, 64, 0, True, True),
+            (1, 2304, 1, 5, True, False), (40, 1024, 128, 0, False, True), (2, 4608, 70, 1, True, True)]):
         W = synth.weights(t, 700 + i, N, K)
         x = (synth.activations(701 + i, M, K) * 3.0).astype(np.float32)
         gain = (synth.normal(702 + i, 0, K) * 0.5 + 1.0).astype(np.float32)
         bias = synth.normal(703 + i, 0, N).astype(np.float32) * 0.1
+        res = synth.activations(704 + i, M, N)
+        rd = dev(gpu, res) if use_res else None
         got = nn.quantized_dense(dev(gpu, x), dev(gpu, W), Quantization(ggml_type=t), dev(gpu, bias), BACKEND_ACT[act],
-                                 norm=nn.RMSNorm(dev(gpu, gain), 1e-6, 0.0)).cpu().numpy()
-        xn = oracle.c_rmsnorm(x, gain, 1e-6, 0.0)
-        want = oracle.c_qdense(t, xn, W, bias, act)
+                                 norm=nn.RMSNorm(dev(gpu, gain), 1e-6, 0.0) if use_norm else None, residual=rd).cpu().numpy()
+        xn = oracle.c_rmsnorm(x, gain, 1e-6, 0.0) if use_norm else x
+        dense = oracle.c_qdense(t, xn, W, bias, act)
+        want = dense + res if use_res else dense
         pre = oracle.c_qdense(t, xn, W, bias, 0)
-        scale = max(float(np.max(np.abs(want))), float(np.max(np.abs(pre))))
+        scale = max(float(np.max(np.abs(dense))), float(np.max(np.abs(pre))))
         err = float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)))) / scale
-        assert err < TOL_F32, (t, M, K, N, act, err)
+        assert err < TOL_F32, (t, M, K, N, act, use_norm, use_res, err)
+    # in place: y is the residual buffer itself
+    import ctypes
+    from gomlx_amd import _lib
+    M, K, N = 2, 512, 96
+    W, x, res = synth.weights(t, 720, N, K), synth.activations(721, M, K), synth.activations(722, M, N)
+    xd, Wd, yd = dev(gpu, x), dev(gpu, W), dev(gpu, res)
+    _lib.check(_lib.lib().gq_qdense_block_f32(t, xd.data_ptr(), M, K, None, Wd.data_ptr(), N, None, 0, yd.data_ptr(), yd.data_ptr(),
+                                              gpu.cuda.current_stream().cuda_stream))
+    gpu.cuda.synchronize()
+    assert rel_err(yd.cpu().numpy(), oracle.c_qdense(t, x, W) + res) < TOL_F32
+
+
+@pytest.mark.parametrize("t", ALL_TYPES)
+def test_batched_projections_behind_one_norm(gpu, oracle, t):
+    """q/k/v of a layer: three batch-1 projections of one normalised input in one launch; a list that
+    cannot be merged (a batch of 3 rows among them) gives the same results through separate calls."""
+    K = 2048
+    gain = (synth.normal(740, 0, K) * 0.5 + 1.0).astype(np.float32)
+    cfg = nn.RMSNorm(dev(gpu, gain), 1e-5, 0.0)
+    q = Quantization(ggml_type=t)
+    for rows in ((1, 1, 1), (1, 3, 1)):
+        xs = [synth.activations(741 + j, m, K) for j, m in enumerate(rows)]
+        if rows == (1, 1, 1):
+            xs = [xs[0]] * 3  # one shared input, as in a decoder layer
+        Ws = [synth.weights(t, 750 + j, n, K) for j, n in enumerate((2048, 512, 520))]
+        bs = [None, synth.normal(760, 0, 512).astype(np.float32) * 0.1, None]
+        outs = nn.quantized_dense_batch([(dev(gpu, x), dev(gpu, W), q, None if b is None else dev(gpu, b), None)
+                                         for x, W, b in zip(xs, Ws, bs)], norm=cfg)
+        gpu.cuda.synchronize()
+        for x, W, b, y in zip(xs, Ws, bs, outs):
+            want = oracle.c_qdense(t, oracle.c_rmsnorm(x, gain, 1e-5, 0.0), W, b)
+            assert rel_err(y.cpu().numpy(), want) < TOL_F32
 
 
 def test_gated_feed_forward_full_size(gpu, oracle):
@@ -541,6 +580,33 @@ def test_gated_feed_forward_rejects_bad_arguments(gpu):
         nn.gated_feed_forward(dev(gpu, np.zeros((1, 96), np.float32)), W, W, q, Activation.SILU)
     with pytest.raises(Exception):
         nn.rms_norm(x, nn.RMSNorm(epsilon=-1.0))
+
+
+def test_feed_forward_block_from_a_gguf_file(gpu, oracle, tmp_path):
+    """File -> device -> kernels: the feed-forward weights of a layer stored in a GGUF container
+    (llama.cpp tensor names), uploaded as Uint8 [N, bytesPerRow] and run as norm + gate/up + down."""
+    from gomlx_amd import gguf
+    K, F = 1024, 2816
+    Wg, Wu, Wd = synth.weights(Q4_K, 900, F, K), synth.weights(Q4_K, 901, F, K), synth.weights(Q6_K, 902, K, F)
+    gain = (synth.normal(903, 0, K) * 0.5 + 1.0).astype(np.float32)
+    path = str(tmp_path / "layer.gguf")
+    gguf.write_gguf(path, {"general.architecture": "llama", "llama.attention.layer_norm_rms_epsilon": 1e-5},
+                    [("blk.0.ffn_norm.weight", 0, (K,), gain), ("blk.0.ffn_gate.weight", Q4_K, (K, F), Wg),
+                     ("blk.0.ffn_up.weight", Q4_K, (K, F), Wu), ("blk.0.ffn_down.weight", Q6_K, (F, K), Wd)])
+    with gguf.GGUFFile(path) as g:
+        eps = float(g.metadata["llama.attention.layer_norm_rms_epsilon"])
+        dg, du, dd = (g.to_device(f"blk.0.ffn_{n}.weight") for n in ("gate", "up", "down"))
+        dn = g.to_device("blk.0.ffn_norm.weight")
+        types = {n: g.tensors[f"blk.0.ffn_{n}.weight"].ggml_type for n in ("gate", "up", "down")}
+    assert dg.dtype == gpu.uint8 and tuple(dg.shape) == (F, ggml.row_bytes(Q4_K, K)) and dn.dtype == gpu.float32
+    assert types == {"gate": Q4_K, "up": Q4_K, "down": Q6_K}
+    x = synth.activations(904, 2, K)
+    ff = nn.gated_feed_forward(dev(gpu, x), dg, du, Quantization(ggml_type=types["gate"]), Activation.SILU, norm=nn.RMSNorm(dn, eps))
+    y = nn.quantized_dense(ff, dd, Quantization(ggml_type=types["down"])).cpu().numpy()
+    ff_want = oracle.c_gated_ffn(Q4_K, x, Wg, Wu, None, None, 3, (gain, eps, 0.0))
+    want = oracle.c_qdense(Q6_K, ff_want, Wd)
+    assert rel_err(ff.cpu().numpy(), ff_want) < 2 * TOL_F32
+    assert rel_err(y, want) < 2 * TOL_F32
 
 
 # ------------------------------------------------------------------------------ benchmark configurations, full size
