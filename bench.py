@@ -38,16 +38,17 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM-side traffic per step in bytes, from hardware counters: two `rocprofv3 --pmc` passes per
 # workload (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch, summed over the step's kernels), each
 # scaled by what the same counter reads for the 64 MiB copy of --copy-calibration (FETCH_SIZE
-# reads 32780.6 KiB for 65536 KiB copied: factor 1.99924; WRITE_SIZE reads 65536.0: factor 1.0).
+# reads 32782.2 KiB for 65536 KiB copied: factor 1.99914; WRITE_SIZE reads 65536.0: factor 1.0).
 # The readings are summarised under profiles/; they are properties of the kernels' access
 # pattern, not of a particular run, and are re-measured whenever a kernel changes.
-_KIB, _FETCH_SCALE, _WRITE_SCALE = 1024, 65536.0 / 32780.6, 1.0
+_KIB, _FETCH_SCALE, _WRITE_SCALE = 1024, 65536.0 / 32782.2, 1.0
 COUNTER_KIB = {  # workload -> (FETCH_SIZE, WRITE_SIZE) raw counter KiB per step
     "c0": (8812.0, 16.0),
-    "c1": (16276.3, 56.0),
-    "c2": (19875.0 + 1833.6 + 911.6, 3584.0 + 512.0 + 924.0),
-    "c3": (74726.7, 32768.0),
-    "c4": (60539.5, 168.0),
+    "c1": (16262.9, 56.0),
+    "c2": (19875.1 + 1833.6 + 911.6, 3584.0 + 512.0 + 924.0),
+    "c3": (74726.6, 32768.0),
+    "c4": (60540.6, 168.0),
+    "ffn": (32488.6, 56.0),
 }
 
 

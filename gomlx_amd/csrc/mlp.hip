@@ -59,15 +59,8 @@ int launch_ext(const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N
     // With two matrices the row-steps alternate between them: plan for 2 N rows and an even count.
     const bool dual = ext.W2 != nullptr;
     KsPlan p;
-    if (!ks_plan(K, dual ? 2 * N : N, p)) return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv_ks: unsupported problem");
-    if (dual) {
-        if (p.iters & 1) {
-            p.iters++;
-            p.pf = p.iters;  // odd counts are at most 7
-        }
-        p.wgs = (int)((N + p.iters * 4 - 1) / (p.iters * 4));
-        p.shmem = ks_lds_bytes(p.waves, p.iters);
-    }
+    if (!ks_plan(K, dual ? 2 * N : N, p, dual)) return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv_ks: unsupported problem");
+    if (dual) p.wgs = (int)((N + p.iters * 4 - 1) / (p.iters * 4));
     switch (p.pf) {
     case 1: return launch_ext_pf<T, 1>(p, x, M, K, W, N, bias, act, y, ext, s);
     case 2: return launch_ext_pf<T, 2>(p, x, M, K, W, N, bias, act, y, ext, s);
