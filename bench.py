@@ -288,8 +288,8 @@ def copy_calibration(torch, steps):
 def main():
     args = parse_args()
     if args.gpus != 1:
-        print("bench.py: this build measures one GPU only (the path is a single-GPU kernel; see DESIGN.md "
-              "for how it would shard); run with --gpus 1", file=sys.stderr)
+        print("bench.py: this build measures one GPU only (the path is a single-GPU kernel: rows of W are independent, so it "
+              "would shard by output features); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
     import torch
     if not torch.cuda.is_available():

@@ -113,6 +113,40 @@ def test_argument_errors_are_reported_before_any_device_work():
     assert L.gq_dequantize(ggml.Q8_0, None, 0, 32, None, None) == _lib.OK
 
 
+def test_argument_errors_of_the_calls_around_a_projection():
+    L = _lib.lib()
+    f = ctypes.c_float
+    norm = _lib.RmsNormDesc(None, 1e-6, 0.0)
+    bad_eps = _lib.RmsNormDesc(None, -1.0, 0.0)
+    odd_gain = _lib.RmsNormDesc(18, 1e-6, 0.0)
+    assert L.gq_rmsnorm_f32(16, 2, 0, None, f(1e-6), f(0), 16, None) == _lib.ERR_INVALID            # K = 0
+    assert L.gq_rmsnorm_f32(16, 2, 8, None, f(-1.0), f(0), 16, None) == _lib.ERR_INVALID            # negative epsilon
+    assert L.gq_rmsnorm_f32(None, 2, 8, None, f(1e-6), f(0), 16, None) == _lib.ERR_INVALID
+    assert L.gq_rmsnorm_f32(None, 0, 8, None, f(1e-6), f(0), None, None) == _lib.OK                 # no rows
+    # block dense: the checks of the dense call, then its own
+    assert L.gq_qdense_block_f32(ggml.Q8_0, 16, 1, 33, ctypes.byref(norm), 16, 1, None, 0, None, 16, None) == _lib.ERR_INVALID
+    assert L.gq_qdense_block_f32(99, 16, 1, 32, ctypes.byref(norm), 16, 1, None, 0, None, 16, None) == _lib.ERR_NOT_IMPLEMENTED
+    assert L.gq_qdense_block_f32(ggml.Q8_0, 16, 1, 32, ctypes.byref(bad_eps), 16, 1, None, 0, None, 16, None) == _lib.ERR_INVALID
+    assert b"epsilon" in L.gq_last_error()
+    assert L.gq_qdense_block_f32(ggml.Q8_0, 16, 1, 32, ctypes.byref(odd_gain), 16, 1, None, 0, None, 16, None) == _lib.ERR_INVALID
+    assert L.gq_qdense_block_f32(ggml.Q8_0, 16, 1, 32, None, 16, 1, None, 0, 18, 16, None) == _lib.ERR_INVALID   # residual alignment
+    assert L.gq_qdense_block_f32(ggml.Q8_0, None, 0, 32, ctypes.byref(norm), None, 5, None, 0, None, None, None) == _lib.OK
+    # gated: both matrices are checked
+    assert L.gq_qdense_gated_f32(ggml.Q8_0, 16, 1, 32, None, 16, None, None, None, 1, 3, 16, None) == _lib.ERR_INVALID   # no up matrix
+    assert L.gq_qdense_gated_f32(ggml.Q8_0, 16, 1, 32, None, 16, None, 24, None, 1, 3, 16, None) == _lib.ERR_INVALID     # up not aligned
+    assert L.gq_qdense_gated_f32(ggml.Q8_0, 16, 1, 32, ctypes.byref(bad_eps), 16, None, 32, None, 1, 3, 16, None) == _lib.ERR_INVALID
+    assert L.gq_qdense_gated_f32(13, 16, 1, 256, None, 16, None, 32, None, 1, 3, 16, None) == _lib.ERR_NOT_IMPLEMENTED
+    assert L.gq_qdense_gated_f32(ggml.Q8_0, None, 0, 32, None, None, None, None, None, 5, 3, None, None) == _lib.OK
+    # batched projections behind a norm
+    d = (_lib.DenseDesc * 1)()
+    d[0].type, d[0].act, d[0].dX, d[0].M, d[0].K, d[0].dW, d[0].N, d[0].dBias, d[0].dY = ggml.Q8_0, 0, 16, 1, 33, 16, 1, None, 16
+    assert L.gq_qdense_norm_f32_batch(1, d, ctypes.byref(norm), None) == _lib.ERR_INVALID
+    assert L.gq_qdense_norm_f32_batch(-1, None, ctypes.byref(norm), None) == _lib.ERR_INVALID
+    assert L.gq_qdense_norm_f32_batch(0, None, ctypes.byref(norm), None) == _lib.OK
+    d[0].K = 32
+    assert L.gq_qdense_norm_f32_batch(1, d, ctypes.byref(bad_eps), None) == _lib.ERR_INVALID
+
+
 def test_python_wrapper_maps_statuses_to_exceptions():
     with pytest.raises(_lib.HipqError) as e:
         _lib.check(_lib.lib().gq_qdense_f32(ggml.Q8_0, 16, 1, 33, 16, 1, None, 0, 16, None))
