@@ -3,8 +3,9 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1] [--others]
 
---config takes c0 .. c4 (the BASELINE.json configurations) or ffn (the gated feed-forward front
-of a decoder layer: the callers around the two projections folded into one launch).
+--config takes c0 .. c4 (the BASELINE.json configurations), ffn (the gated feed-forward front of
+a decoder layer: the callers around the two projections folded into one launch) or layer (the
+seven projections of C4 in the order and with the dependencies of a decoder layer).
 
 A "step" is one quantized Dense call (one pass over one weight matrix) on synthetic data that
 is already resident in HBM.  The headline workload is BASELINE.json configs[1]: Q4_0 decode
@@ -38,17 +39,18 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM-side traffic per step in bytes, from hardware counters: two `rocprofv3 --pmc` passes per
 # workload (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch, summed over the step's kernels), each
 # scaled by what the same counter reads for the 64 MiB copy of --copy-calibration (FETCH_SIZE
-# reads 32782.2 KiB for 65536 KiB copied: factor 1.99914; WRITE_SIZE reads 65536.0: factor 1.0).
+# reads 32780.5 KiB for 65536 KiB copied: factor 1.99924; WRITE_SIZE reads 65536.0: factor 1.0).
 # The readings are summarised under profiles/; they are properties of the kernels' access
 # pattern, not of a particular run, and are re-measured whenever a kernel changes.
-_KIB, _FETCH_SCALE, _WRITE_SCALE = 1024, 65536.0 / 32782.2, 1.0
+_KIB, _FETCH_SCALE, _WRITE_SCALE = 1024, 65536.0 / 32780.5, 1.0
 COUNTER_KIB = {  # workload -> (FETCH_SIZE, WRITE_SIZE) raw counter KiB per step
     "c0": (8812.0, 16.0),
-    "c1": (16262.9, 56.0),
-    "c2": (19875.1 + 1833.6 + 911.6, 3584.0 + 512.0 + 924.0),
+    "c1": (16262.8, 56.0),
+    "c2": (19875.0 + 1833.6 + 911.6, 3584.0 + 512.0 + 924.0),
     "c3": (74726.6, 32768.0),
     "c4": (60540.6, 168.0),
-    "ffn": (32488.6, 56.0),
+    "ffn": (32488.5, 56.0),
+    "layer": (7121.9 + 4762.2 + 32488.1 + 16449.1, 24.0 + 16.0 + 56.0 + 16.0),
 }
 
 
@@ -73,6 +75,8 @@ WORKLOAD_TEXT = {
     "c2": "configs[2]: Q4_K dense, decode batch M=32, K=14336 -> N=4096",
     "c3": "configs[3]: Q8_0 prefill GEMM, M=2048 bf16, K=4096, N=4096",
     "c4": "configs[4]: seven Q4_K projections of a Llama-3-8B layer, batch 1",
+    "layer": "the seven Q4_K projections of a Llama-3-8B layer as a decoder runs them, batch 1: four dependent launches "
+             "(RMSNorm + q/k/v, o + residual, RMSNorm + gate/up + SiLU*mul, down + residual)",
     "ffn": "gated feed-forward front of a Llama-3-8B layer, batch 1: RMSNorm, Q4_K gate and up 4096 -> 14336, SiLU(gate) * up, one launch",
 }
 
@@ -82,7 +86,7 @@ def parse_args():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=200)
     p.add_argument("--warmup", type=int, default=20)
-    p.add_argument("--config", default="c1", choices=sorted(list(CONFIGS) + ["c4", "ffn"]))
+    p.add_argument("--config", default="c1", choices=sorted(list(CONFIGS) + ["c4", "ffn", "layer"]))
     p.add_argument("--others", action="store_true", help="also measure the other configurations (reported under 'others')")
     p.add_argument("--no-graph", action="store_true", help="submit the timed steps one call at a time")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
@@ -102,9 +106,10 @@ class Problem:
         self.torch, self.name = torch, name
         self.L = _lib.lib()
         self.check = _lib.check
-        if name == "c4":
+        if name in ("c4", "layer"):
             shapes = [("Q4_K", 1, K, N) for K, N in C4_SHAPES]
             self.dtype, self.bound = "f32", "hbm"
+            self.gain = torch.ones(4096, device="cuda")
         elif name == "ffn":  # gate and up matrices of one feed-forward block
             shapes = [("Q4_K", 1, 4096, 14336)] * 2
             self.dtype, self.bound = "f32", "hbm"
@@ -113,7 +118,7 @@ class Problem:
             tn, M, K, N, self.dtype, self.bound = CONFIGS[name]
             shapes = [(tn, M, K, N)]
         self.parts = []
-        seed = 1000 + (int(name[1]) if name != "ffn" else 5)
+        seed = 1000 + (int(name[1]) if name[0] == "c" else 4 if name == "layer" else 5)
         total_w = 0
         for i, (tn, M, K, N) in enumerate(shapes):
             t = getattr(ggml, tn)
@@ -146,6 +151,24 @@ class Problem:
                 d.type, d.act, d.dX, d.M, d.K = p["t"], 0, p["x"].data_ptr(), p["M"], p["K"]
                 d.dW, d.N, d.dBias, d.dY = p["W"][c].data_ptr(), p["N"], None, p["y"].data_ptr()
             self.check(self.L.gq_qdense_f32_batch(len(self.parts), descs, self.stream))
+            return
+        if self.name == "layer":
+            # q, k, v, o, gate, up, down in C4's order; the attention between v and o is not part of this path: o reads a
+            # fixed vector of the right shape.  Outputs feed the next call where the shapes chain (o -> gate/up -> down).
+            from gomlx_amd import _lib
+            q, k, v, o, g, u, d = self.parts
+            norm = _lib.RmsNormDesc(self.gain.data_ptr(), 1e-5, 0.0)
+            descs = (_lib.DenseDesc * 3)()
+            for ds, p in zip(descs, (q, k, v)):
+                ds.type, ds.act, ds.dX, ds.M, ds.K = p["t"], 0, q["x"].data_ptr(), 1, p["K"]
+                ds.dW, ds.N, ds.dBias, ds.dY = p["W"][c].data_ptr(), p["N"], None, p["y"].data_ptr()
+            self.check(self.L.gq_qdense_norm_f32_batch(3, descs, ctypes.byref(norm), self.stream))
+            self.check(self.L.gq_qdense_block_f32(o["t"], o["x"].data_ptr(), 1, o["K"], None, o["W"][c].data_ptr(), o["N"], None, 0,
+                                                  q["x"].data_ptr(), o["y"].data_ptr(), self.stream))
+            self.check(self.L.gq_qdense_gated_f32(g["t"], o["y"].data_ptr(), 1, g["K"], ctypes.byref(norm), g["W"][c].data_ptr(), None,
+                                                  u["W"][c].data_ptr(), None, g["N"], 3, g["y"].data_ptr(), self.stream))
+            self.check(self.L.gq_qdense_block_f32(d["t"], g["y"].data_ptr(), 1, d["K"], None, d["W"][c].data_ptr(), d["N"], None, 0,
+                                                  o["y"].data_ptr(), d["y"].data_ptr(), self.stream))
             return
         if self.name == "ffn":
             from gomlx_amd import _lib
@@ -234,7 +257,7 @@ def cpu_baseline(name):
     from gomlx_amd import ggml, synth
     from oracle import ggml_oracle as oracle
     cores = min(os.cpu_count() or 1, 16)
-    if name == "c4":
+    if name in ("c4", "layer"):
         shapes = [("Q4_K", 1, K, N) for K, N in C4_SHAPES]
     elif name == "ffn":  # the two projections; the normalisation and the product are negligible beside them
         shapes = [("Q4_K", 1, 4096, 14336)] * 2
@@ -313,7 +336,7 @@ def main():
         return rep
 
     rep = measure(args.config)
-    tn = "Q4_K" if args.config in ("c4", "ffn") else CONFIGS[args.config][0]
+    tn = "Q4_K" if args.config in ("c4", "ffn", "layer") else CONFIGS[args.config][0]
     line = {
         "metric": rep["metric"], "value": rep["value"], "unit": rep["unit"], "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": rep["ms_per_step"],
@@ -330,7 +353,7 @@ def main():
         line["cpu_baseline"] = cpu_baseline(args.config)
     if args.others:
         others = {}
-        for name in ["c0", "c1", "c2", "c3", "c4", "ffn"]:
+        for name in ["c0", "c1", "c2", "c3", "c4", "ffn", "layer"]:
             if name == args.config:
                 continue
             steps = args.steps if name != "c3" else max(10, args.steps // 10)

@@ -682,8 +682,10 @@ bool ks_plan(int64_t K, int64_t N, KsPlan &p, bool even_iters = false) {
     if (N <= 0 || !ks_split(K, p.waves, p.nslices, p.half_tail)) return false;
     const int cus = device_cu_count();
     // One 8-wavefront workgroup per CU streams best; problems that would leave a wavefront with
-    // only one or two row-steps are launch- and latency-bound and do better with twice the
-    // wavefronts (more independent prologues in flight).
+    // only one or two row-steps of a single slice are launch- and latency-bound and get twice the
+    // wavefronts (more independent prologues in flight).  Not when a wavefront walks several
+    // slices: there two row-steps per slice keep two loads in flight where one row-step keeps
+    // one (K = 14336 -> N = 4096: Q4_K 9.9 -> 8.8 us, Q4_0 9.5 -> 8.6, Q6_K 13.2 -> 12.2).
     auto iters_for = [&](int waves_per_cu) {
         int64_t wgs = (int64_t)cus * waves_per_cu / p.waves;
         if (wgs < 1) wgs = 1;
@@ -691,7 +693,7 @@ bool ks_plan(int64_t K, int64_t N, KsPlan &p, bool even_iters = false) {
         return it < 1 ? (int64_t)1 : it;
     };
     int64_t iters = ks_env_waves() > 0 ? iters_for(ks_env_waves()) : iters_for(8);
-    if (ks_env_waves() <= 0 && iters <= 2) iters = iters_for(16);
+    if (ks_env_waves() <= 0 && iters <= 2 && p.nslices <= p.waves) iters = iters_for(16);
     if (iters > kMaxItersKs) iters = kMaxItersKs;
     ks_group(iters, even_iters, p.iters, p.pf);
     p.wgs = (int)((N + (int64_t)p.iters * 8 - 1) / ((int64_t)p.iters * 8));
