@@ -436,9 +436,9 @@ constexpr int kWaveLdsDwords = 76 * 4;  // per wavefront: 64 uint4 of planes, 16
 // each consumed step is followed by the load of the step WIN ahead, so that load issue (which
 // blocks while the memory pipeline is full) and arithmetic alternate instead of forming two
 // phases.  Deeper windows lose: on Q4_0 4096 -> 14336 (7 row-steps per wavefront) windows of 3, 4, 5
-// and all 7 take 8.0, 8.4, 8.9 and 9.7 us.  (A variant that treats a wavefront's slices x row-steps as one sequence, so that the
-// window also spans slices when there are only one or two row-steps, was measured: its guarded
-// steps cost the unguarded common case 8 % and it was dropped.)
+// and all 7 take 8.0, 8.4, 8.9 and 9.7 us.  (A variant that treats a wavefront's slices x
+// row-steps as one sequence, so that the window also spans slices when there are only one or two
+// row-steps, was measured: its guarded steps cost the unguarded common case 8 % and it was dropped.)
 //
 // EXT adds what the callers around a dense layer ask for (fp32 activations only), described by a KsExt:
 //   * an RMS normalisation of the activations in front: the gain is multiplied in while a slice
