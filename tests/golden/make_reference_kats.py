@@ -8,6 +8,9 @@ Sources (gomlx/gomlx):
   ml/nn/quantized_gather_test.go:17-74    Q8_0 gather basic / single
   ml/nn/quantized_gather_test.go:78-121   Q4_0 gather
   ml/nn/quantized_gather_test.go:125-169  IQ4_NL gather
+  ml/layers/activation/activation_test.go:17-112  Relu, Swish, Gelu (exact), GeluApproximate, HardSwish on
+                                          x = [0, -1, 2, -3, 4, -5, 6]; tolerances as in the tests
+                                          (xslices.Epsilon is defined outside the repository: 1e-4 is used here)
   ml/layers/norm/rmsnorm_test.go:16-45    RMSNorm over the last two axes of a [2, 3, 2] input (gain = ones),
                                           stored flattened: rows of 6 values
 
@@ -36,6 +39,7 @@ def q4_row(scale_hi, byte_with_9):
     return row
 
 
+ACT_X = [0, -1, 2, -3, 4, -5, 6]
 x_basic = [1.0, 1.0] + [0.0] * 30
 x_half = [0.5] + [0.0] * 31
 q8_w = [q8_row(0x40, [0]), q8_row(0x42, [1])]
@@ -69,6 +73,17 @@ kats = {
          "want": [[1.7616, 2.8577]], "tol": 1e-3},
         {"name": "iq4_nl_basic", "type": IQ4_NL, "w": iq_w, "x": [x_basic], "bias": None, "act": NONE,
          "want": [[14.0, 28.0]], "tol": 1e-4},
+    ],
+    # act = compute.ActivationType the type maps to (activation.go:58-75): GeluApproximate also maps to Gelu (exact)
+    "activation": [
+        {"name": "relu", "act": 2, "x": ACT_X, "want": [0, 0, 2, 0, 4, 0, 6], "tol": 1e-4},
+        {"name": "swish", "act": 3, "x": ACT_X,
+         "want": [0, -0.26894143, 1.7615942, -0.14227763, 3.928055, -0.03346425, 5.9851646], "tol": 1e-4},
+        {"name": "gelu_exact", "act": 1, "x": ACT_X,
+         "want": [0, -0.15865526, 1.9544997, -4.0496886e-03, 3.9998736, -1.3411045e-06, 6], "tol": 1e-5},
+        {"name": "gelu_approximate_through_the_backend_enum", "act": 1, "x": ACT_X,
+         "want": [0, -0.15880796, 1.9545977, -3.6375225e-03, 3.9999294, 0, 6], "tol": 0.01},
+        {"name": "hard_swish", "act": 4, "x": ACT_X, "want": [0, -0.33333334, 1.6666666, 0, 4, 0, 6], "tol": 1e-4},
     ],
     "rmsnorm": [
         {"name": "rmsnorm_two_axes", "x": [[3, 4, 5, 6, 7, 8], [6, 8, 10, 12, 14, 16]], "eps": 1e-6,

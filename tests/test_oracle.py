@@ -90,6 +90,17 @@ def test_gather_reference_kats(oracle, kats, impl):
         np.testing.assert_allclose(got, np.array(k["want"], np.float32), rtol=0, atol=k["tol"], err_msg=k["name"])
 
 
+def test_activation_reference_kats(oracle, kats):
+    """ml/layers/activation/activation_test.go:17-112, through both implementations."""
+    for k in kats["activation"]:
+        x, want = np.array(k["x"], np.float32), np.array(k["want"], np.float32)
+        np.testing.assert_allclose(oracle.np_activation(k["act"], x), want, rtol=0, atol=k["tol"], err_msg=k["name"])
+        got_c = np.array([oracle.lib().gqo_activation(k["act"], float(v)) for v in x], np.float32)
+        np.testing.assert_allclose(got_c, want, rtol=0, atol=k["tol"], err_msg=k["name"])
+        if k["tol"] <= 1e-4:  # the published digits are float32-accurate
+            np.testing.assert_allclose(got_c, want, rtol=2e-6, atol=2e-7, err_msg=k["name"])
+
+
 @pytest.mark.parametrize("impl", ["np", "c"])
 def test_rmsnorm_reference_kat(oracle, kats, impl):
     """ml/layers/norm/rmsnorm_test.go:16-45: gain of ones (the variable's initial value), default epsilon."""

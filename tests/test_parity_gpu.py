@@ -63,6 +63,24 @@ def test_reference_gather_kats(gpu, kats):
                                    err_msg=k["name"])
 
 
+def test_reference_activation_kats(gpu, kats):
+    """The reference's activation vectors (ml/layers/activation/activation_test.go:17-112) through the
+    fused epilogue: a Q8_0 identity matrix (scale 1.0, code 1 on the diagonal) hands x to the activation
+    unchanged, at one row (decode GEMV) and at 40 rows (MFMA path)."""
+    K = 32
+    W = np.zeros((7, 34), np.uint8)
+    W[:, 1] = 0x3C  # fp16 1.0, little-endian
+    for i in range(7):
+        W[i, 2 + i] = 1
+    for k in kats["activation"]:
+        x = np.zeros((1, K), np.float32)
+        x[0, :7] = k["x"]
+        for rows in (1, 40):
+            got = run_dense(gpu, Q8_0, np.repeat(x, rows, axis=0), W, None, k["act"])
+            np.testing.assert_allclose(got, np.repeat(np.array([k["want"]], np.float32), rows, axis=0), rtol=0, atol=k["tol"],
+                                       err_msg=k["name"])
+
+
 # ------------------------------------------------------------------------------ dequantisation (bit-exact)
 
 @pytest.mark.parametrize("t", ALL_TYPES)
