@@ -10,7 +10,8 @@
  *   gqo_fp16_to_fp32      pinned  - exhaustive comparison with IEEE binary16 (numpy) + reference KATs
  *   Q8_0 / Q4_0 dequant   pinned  - ml/nn/quantized_dense_test.go:272-401 KATs, closed form, brute force
  *   IQ4_NL dequant        pinned  - ml/nn/quantized_dense_test.go:406-452 KAT (LUT[8]=1, LUT[9]=13) + public table
- *   dense / bias / act    pinned  - reference KATs, unit-vector probes, linearity, SiLU KAT
+ *   dense / bias / act    pinned  - reference KATs, unit-vector probes, linearity, SiLU KAT, the activation vectors
+ *                                   of ml/layers/activation/activation_test.go:17-112
  *   gather                pinned  - ml/nn/quantized_gather_test.go:17-169 KATs
  *   RMS normalisation     pinned  - ml/layers/norm/rmsnorm_test.go:16-45 KAT, closed forms (constant rows,
  *                                   scale invariance, unit norm), independent numpy form
