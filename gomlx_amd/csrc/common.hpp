@@ -79,7 +79,7 @@ int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, co
 // RMS normalisation in front of a projection: x / sqrt(mean(x^2) + eps) * (gain + gain_offset); gain may be null.
 struct RmsNorm { const float *gain; float eps, gain_offset; };
 // The K-sliced GEMV with the normalisation folded in and, when W2 is given, the gated product
-// act(x.W + bias) * (x.W2 + bias2); fp32 activations, at most 16 rows.
+// act(x.W + bias) * (x.W2 + bias2); fp32 activations, at most 16 rows (the entry points use it below 8 rows, where a pass per row still wins).
 bool gemv_ks_ext_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, const void *gain);
 int launch_gemv_ks_ext(int type, const float *x, int64_t M, int64_t K, const RmsNorm *norm, const uint8_t *W, const float *bias,
                        const uint8_t *W2, const float *bias2, const float *residual, int64_t N, int act, float *y, hipStream_t s);

@@ -3,9 +3,9 @@
 // projections (ml/layers/norm/rmsnorm.go:78-113) and the gated feed-forward front
 //     ff = act(x . Wgate^T + bgate) * (x . Wup^T + bup).
 //
-// For up to 16 activation rows both are folded into the K-sliced decode GEMV (gemv_ks_body.hpp,
+// For a few activation rows both are folded into the K-sliced decode GEMV (gemv_ks_body.hpp,
 // EXT): one launch reads the two weight matrices once and writes only ff.  Larger batches are
-// composed from the dense kernels plus the two small kernels below.
+// composed from the dense kernels plus the small kernels below.
 #include "gemv_ks_body.hpp"
 
 namespace gq {

@@ -142,8 +142,9 @@ typedef struct {
  * (Model.normalize followed by a projection, transformer.go:1099-1101; Add(residual, ...) after
  * the output and down projections, :1045, :1055, :1291-1292).  norm and dResidual may each be
  * NULL (both NULL is plain gq_qdense_f32); dY may be dResidual itself (a residual stream updated
- * in place).  Up to 16 rows run in the decode GEMV itself when K is a multiple of 256 and x and
- * gain are 16-byte aligned; other shapes are composed of an RMSNorm kernel, the dense call and
+ * in place).  Small batches (up to 7 rows; up to 16 where the split-K kernels do not apply) run in
+ * the decode GEMV itself when K is a multiple of 256 and x and gain are 16-byte aligned; other
+ * shapes are composed of an RMSNorm kernel, the dense call and
  * an addition, and use a per-stream workspace. */
 int gq_qdense_block_f32(int type, const float *dX, int64_t M, int64_t K, const gq_rmsnorm *norm,
                         const void *dW, int64_t N, const float *dBias, int act,
