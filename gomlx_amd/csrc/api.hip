@@ -5,6 +5,7 @@
 
 #include <atomic>
 #include <cstring>
+#include <cstdlib>
 #include <map>
 #include <mutex>
 
@@ -113,10 +114,29 @@ int check_dense_args(const char *fn, int type, const void *x, int64_t M, int64_t
     return GQ_OK;
 }
 
-// Batch sizes served by the split-K small-batch kernels (measured crossovers against the GEMV passes
-// below and the two-pass GEMM above, K = 4096, N = 4096 .. 14336).  The Q6_K kernel pays 16 scale
-// groups per super-block and only wins for a single tile of 32 batch columns.
-int64_t split_k_from(int type) { return type == GQ_Q4_K || type == GQ_IQ4_NL ? 5 : type == GQ_Q6_K ? 6 : 8; }
+// Batch sizes served by the split-K small-batch kernels: measured crossovers against the GEMV passes
+// below and the two-pass GEMM above.  A GEMV pass per row costs time in proportion to the weight
+// bytes, the split-K kernels a fixed part plus less per byte, so large matrices change over earlier.
+// Measured (us, rows 2 3 4 5 6 7 8 10; GEMV passes | split-K):
+//   Q8_0 4096x4096 (18 MB)   8.8 10.5 12.3 14.8 16.4 18.2 20.2 24.0 | 16.6     4096x14336 (62 MB) 20.4 27.4 35.4 43.7 51.6 .. | 29.5
+//   Q4_0 4096x4096 (9 MB)    7.0  7.6  9.4 11.6 12.8 14.1 15.8 19.0 | 15.5     4096x14336 (33 MB) 13.3 16.7 20.5 22.9 26.2 29.7 | 24.8
+//   Q4_K 4096x4096           7.9  9.1 11.3 13.9 15.5 17.6 20.5 22.9 | 18.8     4096x14336         14.9 18.6 23.1 27.5 31.9 .. | 20.8
+//   Q6_K 4096x4096 (14 MB)   9.3 11.9 14.3 16.7 18.7 21.6 22.9 27.5 | 18.6     4096x14336 (48 MB) 20.8 26.7 34.1 41.5 49.1 .. | 42.0
+//   IQ4_NL 4096x4096         8.2  9.6 12.0 14.5 16.1 18.6 20.1 23.6 | 16.0     4096x14336         18.9 21.8 28.6 34.5 40.1 .. | 27.3
+// The Q6_K kernel pays 16 scale groups per super-block and only wins for a single tile of 32 batch columns.
+constexpr int64_t kLargeWeightBytes = (int64_t)24 << 20;
+int64_t split_k_from(int type, int64_t weight_bytes) {
+    const bool large = weight_bytes >= kLargeWeightBytes;
+    switch (type) {
+    case GQ_Q8_0: return large ? 4 : 7;
+    case GQ_Q4_0: return large ? 6 : 9;
+    case GQ_Q4_K: return large ? 4 : 8;
+    case GQ_Q6_K: return large ? 6 : 7;
+    case GQ_IQ4_NL: return large ? 4 : 7;
+    default: return 8;
+    }
+}
+int64_t weight_bytes_of(int type, int64_t K, int64_t N) { return (int64_t)gq_row_bytes(type, K) * N; }
 int64_t split_k_to(int type) { return type == GQ_Q6_K ? 32 : 96; }
 
 // large batches: W dequantised once into the stream's workspace, then a plain 16-bit GEMM
@@ -292,7 +312,8 @@ int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *d
     // crossovers: split_k_from() / split_k_to().
     const bool tp = gemm_two_pass_supported(type, false, M, K, N, dX);
     const bool ks = M <= kGemvMaxRows && gemv_ks_supported(type, K, N, dX);
-    const bool sk = M >= split_k_from(type) && mmq_supported(type, M, K, N, dX, dBias, dY) && (M <= split_k_to(type) || !tp);
+    const bool sk = M >= split_k_from(type, weight_bytes_of(type, K, N)) && mmq_supported(type, M, K, N, dX, dBias, dY) &&
+                    (M <= split_k_to(type) || !tp);
     if (ks && !sk) return launch_gemv_ks(type, dX, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
     if (sk) return launch_mmq(type, dX, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
     if (M <= 4) {  // shapes or formats without a K-sliced plan: one fp32 pass over W per row
@@ -352,7 +373,8 @@ int gq_qdense_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, const voi
     // the bf16 MFMA paths).
     const bool tp = gemm_two_pass_supported(type, true, M, K, N, dX);
     const bool ks = M <= kGemvMaxRows && gemv_ks_supported(type, K, N, dX);
-    const bool sk = M >= split_k_from(type) && mmq_supported(type, M, K, N, dX, dBias, dY) && (M <= split_k_to(type) || !tp);
+    const bool sk = M >= split_k_from(type, weight_bytes_of(type, K, N)) && mmq_supported(type, M, K, N, dX, dBias, dY) &&
+                    (M <= split_k_to(type) || !tp);
     if (ks && !sk) return launch_gemv_ks(type, dX, true, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
     if (sk) return launch_mmq(type, dX, true, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
     if (tp) return two_pass(type, true, dX, M, K, dW, N, dBias, act, dY, (hipStream_t)stream);
@@ -374,11 +396,14 @@ int gq_rmsnorm_f32(const float *dX, int64_t M, int64_t K, const float *dGain, fl
 namespace {
 // The calls around a projection run inside the decode GEMV while that kernel is the right one for
 // the batch: its time grows by a full pass per row (Q4_K gate/up 4096 -> 14336: 25, 39, 56, 70, 137 us
-// for 2, 4, 6, 8, 16 rows), and from 8 rows on the composed form on the split-K kernels wins (57 us
+// for 2, 4, 6, 8, 16 rows), and beyond a few rows the composed form on the split-K kernels wins (57 us
 // for 6 .. 24 rows).
 bool fold_into_gemv(int type, int64_t M, int64_t K, int64_t N, const float *x, const float *gain, const float *bias, const float *y) {
     if (!gemv_ks_ext_supported(type, M, K, N, x, gain)) return false;
-    return !(M >= 8 && mmq_supported(type, M, K, N, x, bias, y));
+    // the composed form pays its extra small kernels (about 6 us): one or two rows later than a plain dense call
+    const int64_t wb = weight_bytes_of(type, K, N);
+    const int64_t from = split_k_from(type, wb) + (wb >= kLargeWeightBytes ? 1 : 2);
+    return !(M >= from && mmq_supported(type, M, K, N, x, bias, y));
 }
 }  // namespace
 

@@ -94,10 +94,10 @@ int gq_dequantize(int type, const void *dW, int64_t N, int64_t K, float *dOut, v
 /* ---- compute.Function.FusedQuantizedDense (core/graph/fused_ops.go:231-232), run time:
  * y = act(x . dequant(W)^T + bias), the contract of nn.QuantizedDense
  * (ml/nn/quantized_dense.go:31-57) and ggml.DenseDecomposed (ml/ggml/dense.go:23-62).
- * dBias may be NULL.  fp32 activations, fp32 accumulation.  Up to about ten rows run as
- * bandwidth-bound GEMV passes; larger batches contract on the matrix cores with the activations
- * (and, from 97 rows on, the dequantised weights) rounded to fp16 operands.  Batches of 5 rows and
- * more may use a per-stream workspace that is created on the first such call on the stream: make
+ * dBias may be NULL.  fp32 activations, fp32 accumulation.  The first few rows (3 to 8, depending
+ * on format and matrix size) run as bandwidth-bound GEMV passes; larger batches contract on the
+ * matrix cores with the activations (and, from 97 rows on, the dequantised weights) rounded to
+ * fp16 operands.  Batches of 4 rows and more may use a per-stream workspace that is created on the first such call on the stream: make
  * one call outside a recording (gq_graph_begin) before recording the same call. ---- */
 int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *dW, int64_t N,
                   const float *dBias, int act, float *dY, void *stream);
@@ -142,7 +142,7 @@ typedef struct {
  * (Model.normalize followed by a projection, transformer.go:1099-1101; Add(residual, ...) after
  * the output and down projections, :1045, :1055, :1291-1292).  norm and dResidual may each be
  * NULL (both NULL is plain gq_qdense_f32); dY may be dResidual itself (a residual stream updated
- * in place).  Small batches (up to 7 rows; up to 16 where the split-K kernels do not apply) run in
+ * in place).  Small batches (a few rows; up to 16 where the split-K kernels do not apply) run in
  * the decode GEMV itself when K is a multiple of 256 and x and gain are 16-byte aligned; other
  * shapes are composed of an RMSNorm kernel, the dense call and
  * an addition, and use a per-stream workspace. */

@@ -411,6 +411,22 @@ def test_dispatch_boundaries(gpu, oracle, t, M, K, N, bf16, act, with_bias):
     assert err < (TOL_BF16 if bf16 else TOL_F32), (t, M, K, N, bf16, act, err)
 
 
+@pytest.mark.parametrize("t,N,first", [(Q8_0, 6400, 4), (Q4_0, 11264, 6), (Q4_K, 11264, 4), (Q6_K, 8192, 6), (IQ4_NL, 11264, 4)])
+def test_split_k_crossover_on_large_matrices(gpu, oracle, t, N, first):
+    """Matrices of 24 MB and more hand over from GEMV passes to the split-K kernels at fewer rows than
+    small ones: the batch sizes either side of that point, fp32 and bf16 activations."""
+    K = 4096
+    assert N * ggml.row_bytes(t, K) >= 24 << 20
+    W = synth.weights(t, 330 + t, N, K)
+    bias = synth.normal(331 + t, 0, N).astype(np.float32) * 0.1
+    for M in (first - 1, first, first + 1):
+        x = synth.activations(332 + M, M, K)
+        want = oracle.c_qdense(t, x, W, bias, 3)
+        assert rel_err(run_dense(gpu, t, x, W, bias, 3), want) < TOL_F32, (t, M)
+    xb = bf16_round(synth.activations(340, first, K))
+    assert rel_err(run_dense(gpu, t, xb, W, bias, 3, bf16=True), oracle.c_qdense(t, xb, W, bias, 3)) < TOL_BF16, t
+
+
 def test_randomized_problems(gpu, oracle):
     """150 seeded random problems over all formats, both activation types, every activation, with
     and without bias: batch sizes, K and N drawn from lists that include every tile and slice
