@@ -405,6 +405,18 @@ bool fold_into_gemv(int type, int64_t M, int64_t K, int64_t N, const float *x, c
     const int64_t from = split_k_from(type, wb) + (wb >= kLargeWeightBytes ? 1 : 2);
     return !(M >= from && mmq_supported(type, M, K, N, x, bias, y));
 }
+// Batches that a plain dense call would hand to the two-pass GEMM take its block form: the
+// normalisation rides on the activation pass, the residual and the gated product on the epilogue.
+bool block_takes_two_pass(int type, int64_t M, int64_t K, int64_t N, const float *x, const float *gain, const float *bias, const float *y,
+                          bool gated) {
+    if (M <= kGemvMaxRows || !gemm_two_pass_block_supported(type, M, K, N, x, gated)) return false;
+    // A gated pair as one GEMM pays off from a few hundred rows (4096 -> 2 x 14336 in Q4_K: 237 against 255 us at 512 rows,
+    // 660 against 743 us at 2048; at 128 rows, where dequantising the two matrices dominates, 147 against 132 us).
+    if (gated && M < 256) return false;
+    if (gain && !aligned_to(gain, 16)) return false;
+    const bool sk = M >= split_k_from(type, weight_bytes_of(type, K, N)) && mmq_supported(type, M, K, N, x, bias, y) && M <= split_k_to(type);
+    return !sk;
+}
 }  // namespace
 
 int gq_qdense_block_f32(int type, const float *dX, int64_t M, int64_t K, const gq_rmsnorm *norm, const void *dW, int64_t N,
@@ -421,6 +433,12 @@ int gq_qdense_block_f32(int type, const float *dX, int64_t M, int64_t K, const g
     if (fold_into_gemv(type, M, K, N, dX, rn.gain, dBias, dY))
         return launch_gemv_ks_ext(type, dX, M, K, norm ? &rn : nullptr, (const uint8_t *)dW, dBias, nullptr, nullptr, dResidual, N, act, dY,
                                   (hipStream_t)stream);
+    if (block_takes_two_pass(type, M, K, N, dX, rn.gain, dBias, dY, false)) {
+        void *ws = nullptr;
+        if (int rc = stream_workspace((hipStream_t)stream, gemm_two_pass_block_workspace(M, K, N, false), &ws)) return rc;
+        return launch_gemm_two_pass_block(type, dX, M, K, norm ? &rn : nullptr, (const uint8_t *)dW, dBias, nullptr, nullptr, dResidual, N, act,
+                                          dY, ws, (hipStream_t)stream);
+    }
     // composed: normalised activations into the stream's second workspace, the dense call, then the residual
     const float *x = dX;
     if (norm) {
@@ -477,6 +495,12 @@ int gq_qdense_gated_f32(int type, const float *dX, int64_t M, int64_t K, const g
     if (fold_into_gemv(type, M, K, N, dX, rn.gain, dBiasGate, dY))
         return launch_gemv_ks_ext(type, dX, M, K, norm ? &rn : nullptr, (const uint8_t *)dWgate, dBiasGate, (const uint8_t *)dWup, dBiasUp,
                                   nullptr, N, act, dY, (hipStream_t)stream);
+    if (block_takes_two_pass(type, M, K, N, dX, rn.gain, dBiasGate, dY, true)) {
+        void *ws = nullptr;
+        if (int rc = stream_workspace((hipStream_t)stream, gemm_two_pass_block_workspace(M, K, N, true), &ws)) return rc;
+        return launch_gemm_two_pass_block(type, dX, M, K, norm ? &rn : nullptr, (const uint8_t *)dWgate, dBiasGate, (const uint8_t *)dWup, dBiasUp,
+                                          nullptr, N, act, dY, ws, (hipStream_t)stream);
+    }
     // composed: [normalised activations,] act(gate) into the stream's second workspace, up into y, y *= act(gate)
     const size_t xn_bytes = norm ? ((size_t)M * (size_t)K * sizeof(float) + 255) / 256 * 256 : 0;
     void *ws = nullptr;

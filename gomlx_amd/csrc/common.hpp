@@ -97,6 +97,14 @@ bool gemm_two_pass_supported(int type, bool x_is_bf16, int64_t M, int64_t K, int
 size_t gemm_two_pass_workspace(bool x_is_bf16, int64_t M, int64_t K, int64_t N);
 int launch_gemm_two_pass(int type, bool x_is_bf16, const void *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias,
                          int act, float *y, void *workspace, hipStream_t s);
+// The two passes with the neighbours of a projection folded in (fp32 activations; same conditions as
+// gemm_two_pass_supported): RMS normalisation in the activation pass, residual in the GEMM epilogue;
+// with W2 one GEMM over the interleaved image of both matrices forms the gated product in registers.
+size_t gemm_two_pass_block_workspace(int64_t M, int64_t K, int64_t N, bool gated);
+bool gemm_two_pass_block_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, bool gated);
+int launch_gemm_two_pass_block(int type, const float *x, int64_t M, int64_t K, const RmsNorm *norm, const uint8_t *W, const float *bias,
+                               const uint8_t *W2, const float *bias2, const float *residual, int64_t N, int act, float *y, void *workspace,
+                               hipStream_t s);
 int launch_gemm(int type, bool x_is_bf16, const void *x, int64_t M, int64_t K, const uint8_t *W, int64_t N,
                 const float *bias, int act, float *y, hipStream_t s);
 

@@ -60,16 +60,20 @@ template <> struct Op16<false> {
 };
 
 // ---- pass 1: GGML blocks -> 16-bit [N, K] -------------------------------------------------------
-// One thread per run of 16 weights (32 output bytes).
+// One thread per run of 16 weights (32 output bytes).  half = 0: image row = weight row.  half = 1 / 2:
+// the matrix is the first / second of a gated pair, whose images interleave in chunks of 32 rows
+// (image rows 64 c .. 64 c + 31 = rows 32 c .. of the first matrix, the next 32 = the same rows of
+// the second), so that a wavefront's 64-column tile holds both projections of 32 outputs.
 template <int T, bool BF16>
 __global__ __launch_bounds__(256) void dequant16bit_kernel(const uint8_t *__restrict__ W, uint16_t *__restrict__ out, int64_t runs_per_row,
-                                                          int64_t total_runs, int64_t row_bytes) {
+                                                          int64_t total_runs, int64_t row_bytes, int half) {
     const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (g >= total_runs) return;
     const int64_t row = g / runs_per_row, run = g % runs_per_row;
     float w[16];
     dequant16<T>(W + row * row_bytes, run, w);
-    uint4 *dst = reinterpret_cast<uint4 *>(out + g * 16);
+    const int64_t out_row = half == 0 ? row : (row >> 5) * 64 + (half - 1) * 32 + (row & 31);
+    uint4 *dst = reinterpret_cast<uint4 *>(out + (out_row * runs_per_row + run) * 16);
     dst[0] = make_uint4(Op16<BF16>::pack(w[0], w[1]), Op16<BF16>::pack(w[2], w[3]), Op16<BF16>::pack(w[4], w[5]), Op16<BF16>::pack(w[6], w[7]));
     dst[1] = make_uint4(Op16<BF16>::pack(w[8], w[9]), Op16<BF16>::pack(w[10], w[11]), Op16<BF16>::pack(w[12], w[13]),
                         Op16<BF16>::pack(w[14], w[15]));
@@ -82,6 +86,35 @@ __global__ __launch_bounds__(256) void x_to_f16_kernel(const float *__restrict__
     const float4 a = reinterpret_cast<const float4 *>(x)[2 * g], b = reinterpret_cast<const float4 *>(x)[2 * g + 1];
     reinterpret_cast<uint4 *>(out)[g] =
         make_uint4(Op16<false>::pack(a.x, a.y), Op16<false>::pack(a.z, a.w), Op16<false>::pack(b.x, b.y), Op16<false>::pack(b.z, b.w));
+}
+
+// The same pass with an RMS normalisation in front: fp16(x / sqrt(mean(x^2) + eps) * (gain + offset)),
+// one workgroup per activation row (the row is read twice, the second time from cache).  K % 8 == 0.
+__global__ __launch_bounds__(256) void x_rmsnorm_to_f16_kernel(const float *__restrict__ X, const float *__restrict__ gain, float gain_offset,
+                                                               float eps, int K, uint16_t *__restrict__ out) {
+    __shared__ float part[4];
+    const float4 *x = reinterpret_cast<const float4 *>(X + (int64_t)blockIdx.x * K);
+    const int k8 = K / 8;
+    float ss = 0.f;
+    for (int g = threadIdx.x; g < k8; g += 256) {
+        const float4 a = x[2 * g], b = x[2 * g + 1];
+        ss += (a.x * a.x + a.y * a.y) + (a.z * a.z + a.w * a.w) + (b.x * b.x + b.y * b.y) + (b.z * b.z + b.w * b.w);
+    }
+    for (int m = 1; m < 64; m <<= 1) ss += __shfl_xor(ss, m);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float r = sqrtf(((part[0] + part[1]) + (part[2] + part[3])) / (float)K + eps);
+    uint4 *o = reinterpret_cast<uint4 *>(out + (int64_t)blockIdx.x * K);
+    for (int g = threadIdx.x; g < k8; g += 256) {
+        float4 a = x[2 * g], b = x[2 * g + 1];
+        a.x /= r; a.y /= r; a.z /= r; a.w /= r; b.x /= r; b.y /= r; b.z /= r; b.w /= r;
+        if (gain) {
+            const float4 ga = reinterpret_cast<const float4 *>(gain)[2 * g], gb = reinterpret_cast<const float4 *>(gain)[2 * g + 1];
+            a.x *= ga.x + gain_offset; a.y *= ga.y + gain_offset; a.z *= ga.z + gain_offset; a.w *= ga.w + gain_offset;
+            b.x *= gb.x + gain_offset; b.y *= gb.y + gain_offset; b.z *= gb.z + gain_offset; b.w *= gb.w + gain_offset;
+        }
+        o[g] = make_uint4(Op16<false>::pack(a.x, a.y), Op16<false>::pack(a.z, a.w), Op16<false>::pack(b.x, b.y), Op16<false>::pack(b.z, b.w));
+    }
 }
 
 // ---- pass 2: 16-bit GEMM with global -> LDS DMA --------------------------------------------------
@@ -121,9 +154,13 @@ template <int TM, int TN> struct DmaTile {
     static constexpr int kLdsBytes = NS * kStageBytes;
 };
 
-template <bool BF16, int TM, int TN>
+// GATED (TN == 2): Wh is the interleaved image of a gated pair (N counts its rows); column block j = 0
+// of a wavefront's tile is the first projection, j = 1 the second, of the same 32 outputs, and the
+// result is act(first + bias) * (second + bias2) in a [M, n_out] matrix.
+template <bool BF16, int TM, int TN, bool GATED = false>
 __global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const uint16_t *Wh, const float *__restrict__ bias,
-                                                       float *__restrict__ Y, int M, int K, int N, int act) {
+                                                       float *Y, int M, int K, int N, int act, const float *__restrict__ bias2, int n_out,
+                                                       const float *residual) {
     typedef Op16<BF16> Op;
     typedef DmaTile<TM, TN> G;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -239,6 +276,27 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the re-read DMAs of the last steps
 
     // ---- epilogue: acc[i][j][r] is Y[m, n] with n = lane % 32, m = 8*(r/4) + 4*(lane/32) + r%4
+    if constexpr (GATED) {
+        static_assert(TN == 2, "a gated tile pairs two 32-column blocks");
+        const int n = ((bn + wn) >> 1) + (lane & 31);
+        if (n < n_out) {
+            const float bg = bias ? bias[n] : 0.f, bu = bias2 ? bias2[n] : 0.f;
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int m = bm + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                    if (m < M) {
+                        const int64_t at = (int64_t)m * n_out + n;
+                        float v = apply_act(act, acc[i][0][r] + bg) * (acc[i][1][r] + bu);
+                        if (residual) v += residual[at];
+                        Y[at] = v;
+                    }
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < TN; j++) {
         const int n = bn + wn + j * 32 + (lane & 31);
@@ -249,42 +307,50 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const 
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int m = bm + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (m < M) Y[(int64_t)m * N + n] = apply_act(act, acc[i][j][r] + bv);
+                if (m < M) {
+                    // act(x.W + bias) plus a residual (which may be Y itself: one thread reads and writes an element)
+                    const int64_t at = (int64_t)m * N + n;
+                    float v = apply_act(act, acc[i][j][r] + bv);
+                    if (residual) v += residual[at];
+                    Y[at] = v;
+                }
             }
         }
     }
 }
 
 template <int T, bool BF16>
-int launch_dequant16bit(const uint8_t *W, int64_t N, int64_t K, uint16_t *out, hipStream_t s) {
+int launch_dequant16bit(const uint8_t *W, int64_t N, int64_t K, uint16_t *out, hipStream_t s, int half) {
     const int64_t runs_per_row = K / 16, total = N * runs_per_row;
     const int64_t row_bytes = (K / Geom<T>::vpb) * Geom<T>::bpb;
-    return launch(dequant16bit_kernel<T, BF16>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, W, out, runs_per_row, total, row_bytes);
+    return launch(dequant16bit_kernel<T, BF16>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, W, out, runs_per_row, total, row_bytes, half);
 }
 
 template <bool BF16>
-int launch_dequant16bit_type(int type, const uint8_t *W, int64_t N, int64_t K, uint16_t *out, hipStream_t s) {
+int launch_dequant16bit_type(int type, const uint8_t *W, int64_t N, int64_t K, uint16_t *out, hipStream_t s, int half = 0) {
     switch (type) {
-    case kQ4_0: return launch_dequant16bit<kQ4_0, BF16>(W, N, K, out, s);
-    case kQ8_0: return launch_dequant16bit<kQ8_0, BF16>(W, N, K, out, s);
-    case kIQ4_NL: return launch_dequant16bit<kIQ4_NL, BF16>(W, N, K, out, s);
-    case kQ4_K: return launch_dequant16bit<kQ4_K, BF16>(W, N, K, out, s);
-    case kQ6_K: return launch_dequant16bit<kQ6_K, BF16>(W, N, K, out, s);
+    case kQ4_0: return launch_dequant16bit<kQ4_0, BF16>(W, N, K, out, s, half);
+    case kQ8_0: return launch_dequant16bit<kQ8_0, BF16>(W, N, K, out, s, half);
+    case kIQ4_NL: return launch_dequant16bit<kIQ4_NL, BF16>(W, N, K, out, s, half);
+    case kQ4_K: return launch_dequant16bit<kQ4_K, BF16>(W, N, K, out, s, half);
+    case kQ6_K: return launch_dequant16bit<kQ6_K, BF16>(W, N, K, out, s, half);
     default: return fail(GQ_ERR_NOT_IMPLEMENTED, "qdense: ggml type %d is not implemented", type);
     }
 }
 
-template <bool BF16, int TM, int TN>
+// N counts the rows of the weight image (for a gated pair: both halves, 64 per 32 outputs)
+template <bool BF16, int TM, int TN, bool GATED = false>
 int launch_gemm16_tile(const uint16_t *x, int64_t M, int64_t K, const uint16_t *Wh, int64_t N, const float *bias, int act, float *y,
-                       hipStream_t s) {
+                       const float *bias2, int64_t n_out, const float *residual, hipStream_t s) {
     typedef DmaTile<TM, TN> G;
     static const bool lds_ok = [] {
-        return hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_dma_kernel<BF16, TM, TN>),
+        return hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_dma_kernel<BF16, TM, TN, GATED>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, G::kLdsBytes) == hipSuccess;
     }();
     if (!lds_ok) return fail(GQ_ERR_HIP, "gemm: cannot reserve %d bytes of LDS", G::kLdsBytes);
     const dim3 grid((unsigned)((N + G::DN - 1) / G::DN), (unsigned)((M + G::DM - 1) / G::DM));
-    return launch(gemm_dma_kernel<BF16, TM, TN>, grid, dim3(512), (size_t)G::kLdsBytes, s, x, Wh, bias, y, (int)M, (int)K, (int)N, act);
+    return launch(gemm_dma_kernel<BF16, TM, TN, GATED>, grid, dim3(512), (size_t)G::kLdsBytes, s, x, Wh, bias, y, (int)M, (int)K, (int)N, act,
+                  bias2, (int)n_out, residual);
 }
 
 // GOMLX_HIPQ_GEMM_TILE=0|1|2 forces the 256x128 / 128x128 / 128x64 tile (tuning runs only).
@@ -295,16 +361,28 @@ int tile_env() {
 
 // The largest tile that still gives the chip about one workgroup per CU.
 template <bool BF16>
-int launch_gemm16(const uint16_t *x, int64_t M, int64_t K, const uint16_t *Wh, int64_t N, const float *bias, int act, float *y, hipStream_t s) {
+int launch_gemm16(const uint16_t *x, int64_t M, int64_t K, const uint16_t *Wh, int64_t N, const float *bias, int act, float *y, hipStream_t s,
+                  const float *residual = nullptr) {
     const int64_t want = (int64_t)device_cu_count() * 3 / 4;
     auto tiles = [&](int64_t dm, int64_t dn) { return ((M + dm - 1) / dm) * ((N + dn - 1) / dn); };
-    int choice = tiles(256, 128) >= want ? 0 : tiles(128, 128) >= want ? 1 : 2;
+    int choice = (tiles(256, 128) >= want && M > 128) ? 0 : tiles(128, 128) >= want ? 1 : 2;  // (no half-empty 256-row tiles)
     if (tile_env() >= 0 && tile_env() <= 2) choice = tile_env();
     switch (choice) {
-    case 0: return launch_gemm16_tile<BF16, 2, 2>(x, M, K, Wh, N, bias, act, y, s);
-    case 1: return launch_gemm16_tile<BF16, 1, 2>(x, M, K, Wh, N, bias, act, y, s);
-    default: return launch_gemm16_tile<BF16, 1, 1>(x, M, K, Wh, N, bias, act, y, s);
+    case 0: return launch_gemm16_tile<BF16, 2, 2>(x, M, K, Wh, N, bias, act, y, nullptr, N, residual, s);
+    case 1: return launch_gemm16_tile<BF16, 1, 2>(x, M, K, Wh, N, bias, act, y, nullptr, N, residual, s);
+    default: return launch_gemm16_tile<BF16, 1, 1>(x, M, K, Wh, N, bias, act, y, nullptr, N, residual, s);
     }
+}
+
+// Gated pair (fp16 operands): the interleaved image has 64 rows per 32 outputs.
+int64_t gated_image_rows(int64_t N) { return (N + 31) / 32 * 64; }
+int launch_gemm16_gated(const uint16_t *x, int64_t M, int64_t K, const uint16_t *Wh, int64_t N, const float *bias, const float *bias2, int act,
+                        float *y, const float *residual, hipStream_t s) {
+    const int64_t rows = gated_image_rows(N);
+    const int64_t want = (int64_t)device_cu_count() * 3 / 4;
+    const bool big = M > 128 && ((M + 255) / 256) * ((rows + 127) / 128) >= want;
+    if (big && tile_env() != 1) return launch_gemm16_tile<false, 2, 2, true>(x, M, K, Wh, rows, bias, act, y, bias2, N, residual, s);
+    return launch_gemm16_tile<false, 1, 2, true>(x, M, K, Wh, rows, bias, act, y, bias2, N, residual, s);
 }
 
 // Measured against the fused kernel (K = 4096, N = 4096 .. 14336): the two passes win from the
@@ -354,6 +432,42 @@ int launch_gemm_two_pass(int type, bool x_is_bf16, const void *x, int64_t M, int
     if (int rc = launch(x_to_f16_kernel, dim3((unsigned)((total8 + 255) / 256)), dim3(256), 0, s, static_cast<const float *>(x), xh, total8))
         return rc;
     return launch_gemm16<false>(xh, M, K, wh, N, bias, act, y, s);
+}
+
+// The two passes for a projection with its neighbours (fp32 activations): the RMS normalisation
+// is folded into the activation pass, the residual into the GEMM's epilogue; a gated pair
+// act(xn.W + bias) * (xn.W2 + bias2) is ONE GEMM over the interleaved image of both matrices, the
+// product formed in registers, so neither projection is ever written out.
+size_t gemm_two_pass_block_workspace(int64_t M, int64_t K, int64_t N, bool gated) {
+    const int64_t rows = gated ? gated_image_rows(N) : N;
+    return (((size_t)rows * K * 2 + 255) & ~(size_t)255) + (size_t)M * K * 2;
+}
+
+bool gemm_two_pass_block_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, bool gated) {
+    if (!gemm_two_pass_supported(type, false, M, K, N, x)) return false;
+    return !gated || (uint64_t)gated_image_rows(N) * (uint64_t)K * 2 <= kMaxImageBytes;
+}
+
+int launch_gemm_two_pass_block(int type, const float *x, int64_t M, int64_t K, const RmsNorm *norm, const uint8_t *W, const float *bias,
+                               const uint8_t *W2, const float *bias2, const float *residual, int64_t N, int act, float *y, void *workspace,
+                               hipStream_t s) {
+    const int64_t rows = W2 ? gated_image_rows(N) : N;
+    uint16_t *wh = static_cast<uint16_t *>(workspace);
+    uint16_t *xh = wh + (((size_t)rows * K * 2 + 255) & ~(size_t)255) / 2;
+    if (norm) {
+        if (int rc = launch(x_rmsnorm_to_f16_kernel, dim3((unsigned)M), dim3(256), 0, s, x, norm->gain, norm->gain_offset, norm->eps, (int)K, xh))
+            return rc;
+    } else {
+        const int64_t total8 = M * K / 8;
+        if (int rc = launch(x_to_f16_kernel, dim3((unsigned)((total8 + 255) / 256)), dim3(256), 0, s, x, xh, total8)) return rc;
+    }
+    if (!W2) {
+        if (int rc = launch_dequant16bit_type<false>(type, W, N, K, wh, s)) return rc;
+        return launch_gemm16<false>(xh, M, K, wh, N, bias, act, y, s, residual);
+    }
+    if (int rc = launch_dequant16bit_type<false>(type, W, N, K, wh, s, 1)) return rc;
+    if (int rc = launch_dequant16bit_type<false>(type, W2, N, K, wh, s, 2)) return rc;
+    return launch_gemm16_gated(xh, M, K, wh, N, bias, bias2, act, y, residual, s);
 }
 
 }  // namespace gq

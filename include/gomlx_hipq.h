@@ -143,9 +143,10 @@ typedef struct {
  * the output and down projections, :1045, :1055, :1291-1292).  norm and dResidual may each be
  * NULL (both NULL is plain gq_qdense_f32); dY may be dResidual itself (a residual stream updated
  * in place).  Small batches (a few rows; up to 16 where the split-K kernels do not apply) run in
- * the decode GEMV itself when K is a multiple of 256 and x and gain are 16-byte aligned; other
- * shapes are composed of an RMSNorm kernel, the dense call and
- * an addition, and use a per-stream workspace. */
+ * the decode GEMV itself when K is a multiple of 256 and x and gain are 16-byte aligned; large batches (those a plain call hands to the two-pass GEMM) fold the
+ * normalisation into the activation pass and the residual into the GEMM epilogue; what is left
+ * is composed of an RMSNorm kernel, the dense call and an addition.  All but the first use a
+ * per-stream workspace. */
 int gq_qdense_block_f32(int type, const float *dX, int64_t M, int64_t K, const gq_rmsnorm *norm,
                         const void *dW, int64_t N, const float *dBias, int act,
                         const float *dResidual, float *dY, void *stream);
@@ -156,8 +157,11 @@ int gq_qdense_norm_f32_batch(int count, const gq_dense_desc *descs, const gq_rms
                              void *stream);
 /* The gated feed-forward front (transformer.go:1279-1287, after the pre_feedforward_norm of
  * :1276 when norm != NULL): y = act(xn . Wgate^T + bgate) * (xn . Wup^T + bup), xn = RMSNorm(x)
- * or x.  Both matrices are [N, gq_row_bytes(type, K)] of one type.  Same fast-path conditions as
- * gq_qdense_block_f32; other shapes are composed of dense calls and use a per-stream workspace. */
+ * or x.  Both matrices are [N, gq_row_bytes(type, K)] of one type.  A few rows run as one launch
+ * of the decode GEMV (conditions as for gq_qdense_block_f32); from 256 rows the two matrices are
+ * dequantised into one interleaved 16-bit image and a single GEMM forms the product in
+ * registers; sizes in between are composed of dense calls.  All but the first use a per-stream
+ * workspace. */
 int gq_qdense_gated_f32(int type, const float *dX, int64_t M, int64_t K, const gq_rmsnorm *norm,
                         const void *dWgate, const float *dBiasGate, const void *dWup,
                         const float *dBiasUp, int64_t N, int act, float *dY, void *stream);

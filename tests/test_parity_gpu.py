@@ -582,6 +582,34 @@ def test_batched_projections_behind_one_norm(gpu, oracle, t):
             assert rel_err(y.cpu().numpy(), want) < TOL_F32
 
 
+@pytest.mark.parametrize("t", ALL_TYPES)
+def test_large_batches_with_neighbours_folded_into_the_two_passes(gpu, oracle, t):
+    """From the batch sizes a plain dense call hands to the two-pass GEMM, the normalisation rides on
+    the activation pass and the residual / gated product on the GEMM epilogue (fp16 operands)."""
+    for i, (M, K, N, act, norm_kind, with_bias) in enumerate([(130, 1024, 132, 3, 1, True), (300, 512, 257, 1, 2, False),
+                                                              (40, 768, 130, 3, 3, True), (257, 256, 64, 5, 0, True),
+                                                              (256, 1024, 1000, 3, 1, True), (700, 256, 33, 2, 3, False)]):
+        err = gated_case(gpu, oracle, t, M, K, N, act, norm_kind, with_bias, 820 + 10 * i + t)
+        assert err < 2 * TOL_F32, ("gated", t, M, K, N, act, norm_kind, err)
+    for i, (M, K, N, act, use_norm, use_res) in enumerate([(130, 1024, 132, 0, True, True), (300, 512, 257, 3, True, False),
+                                                           (40, 768, 130, 0, False, True), (600, 256, 64, 2, True, True)]):
+        W = synth.weights(t, 860 + i, N, K)
+        x = (synth.activations(861 + i, M, K) * 3.0).astype(np.float32)
+        gain = (synth.normal(862 + i, 0, K) * 0.5 + 1.0).astype(np.float32)
+        bias = synth.normal(863 + i, 0, N).astype(np.float32) * 0.1
+        res = synth.activations(864 + i, M, N)
+        yd = dev(gpu, res)  # the residual buffer is also the output when there is a residual
+        got = nn.quantized_dense(dev(gpu, x), dev(gpu, W), Quantization(ggml_type=t), dev(gpu, bias), BACKEND_ACT[act],
+                                 norm=nn.RMSNorm(dev(gpu, gain), 1e-6, 0.0) if use_norm else None,
+                                 residual=yd if use_res else None).cpu().numpy()
+        xn = oracle.c_rmsnorm(x, gain, 1e-6, 0.0) if use_norm else x
+        dense = oracle.c_qdense(t, xn, W, bias, act)
+        want = dense + res if use_res else dense
+        scale = max(float(np.max(np.abs(dense))), float(np.max(np.abs(oracle.c_qdense(t, xn, W, bias, 0)))))
+        err = float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)))) / scale
+        assert err < TOL_F32, ("block", t, M, K, N, act, use_norm, use_res, err)
+
+
 def test_gated_feed_forward_full_size(gpu, oracle):
     """Llama-3-8B feed-forward front at full size (Q4_K, 4096 -> 14336 twice, RMSNorm, SiLU), checked on a
     sample of output columns against the oracle and in full against the unfused calls of this library."""
