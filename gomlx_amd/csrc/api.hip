@@ -395,16 +395,25 @@ int gq_rmsnorm_f32(const float *dX, int64_t M, int64_t K, const float *dGain, fl
 
 namespace {
 // The calls around a projection run inside the decode GEMV while that kernel is the right one for
-// the batch: its time grows by a full pass per row (Q4_K gate/up 4096 -> 14336: 25, 39, 56, 70, 137 us
-// for 2, 4, 6, 8, 16 rows), and beyond a few rows the composed form on the split-K kernels wins (57 us
-// for 6 .. 24 rows).
-bool fold_into_gemv(int type, int64_t M, int64_t K, int64_t N, const float *x, const float *gain, const float *bias, const float *y) {
+// the batch: its time grows by a full pass per row, the split-K form costs the same for any batch up
+// to 32 rows.  Measured on gate/up 4096 -> 14336 with RMSNorm and SiLU (us; GEMV at 2, 4, 6 rows | split-K):
+// Q4_K 24 39 56 | 44, Q8_0 40 69 102 | 61, Q4_0 24 38 54 | 51, Q6_K 39 65 94 | 90: the change-over sits at the
+// point where a plain dense call changes kernels, one row later for Q4_K; a single projection with
+// norm or residual pays one small extra kernel in the split-K form and changes one or two rows later.
+bool fold_into_gemv(int type, int64_t M, int64_t K, int64_t N, const float *x, const float *gain, const float *bias, const float *y, bool gated) {
     if (!gemv_ks_ext_supported(type, M, K, N, x, gain)) return false;
-    // the composed form pays its extra small kernels (about 6 us): one or two rows later than a plain dense call
     const int64_t wb = weight_bytes_of(type, K, N);
-    const int64_t from = split_k_from(type, wb) + (wb >= kLargeWeightBytes ? 1 : 2);
-    return !(M >= from && mmq_supported(type, M, K, N, x, bias, y));
+    const bool large = wb >= kLargeWeightBytes;
+    const int64_t margin = gated ? (large && type == GQ_Q4_K ? 1 : 0) : (large ? 1 : 2);
+    return !(M >= split_k_from(type, wb) + margin && mmq_supported(type, M, K, N, x, bias, y));
 }
+
+// Whether a plain dense call on these operands runs on the split-K kernels (the dispatch of gq_qdense_f32).
+bool dense_takes_split_k(int type, int64_t M, int64_t K, int64_t N, const float *x, const float *bias, const float *y) {
+    const bool tp = gemm_two_pass_supported(type, false, M, K, N, x);
+    return M >= split_k_from(type, weight_bytes_of(type, K, N)) && mmq_supported(type, M, K, N, x, bias, y) && (M <= split_k_to(type) || !tp);
+}
+
 // Batches that a plain dense call would hand to the two-pass GEMM take its block form: the
 // normalisation rides on the activation pass, the residual and the gated product on the epilogue.
 bool block_takes_two_pass(int type, int64_t M, int64_t K, int64_t N, const float *x, const float *gain, const float *bias, const float *y,
@@ -430,7 +439,7 @@ int gq_qdense_block_f32(int type, const float *dX, int64_t M, int64_t K, const g
     if (int rc = use_device()) return rc;
     RmsNorm rn{nullptr, 0.f, 0.f};
     if (norm) rn = RmsNorm{norm->dGain, norm->eps, norm->gain_offset};
-    if (fold_into_gemv(type, M, K, N, dX, rn.gain, dBias, dY))
+    if (fold_into_gemv(type, M, K, N, dX, rn.gain, dBias, dY, false))
         return launch_gemv_ks_ext(type, dX, M, K, norm ? &rn : nullptr, (const uint8_t *)dW, dBias, nullptr, nullptr, dResidual, N, act, dY,
                                   (hipStream_t)stream);
     if (block_takes_two_pass(type, M, K, N, dX, rn.gain, dBias, dY, false)) {
@@ -447,6 +456,10 @@ int gq_qdense_block_f32(int type, const float *dX, int64_t M, int64_t K, const g
         float *xn = static_cast<float *>(ws);
         if (int rc = launch_rmsnorm(dX, M, K, rn.gain, rn.gain_offset, rn.eps, xn, (hipStream_t)stream)) return rc;
         x = xn;
+    }
+    if (dResidual && dense_takes_split_k(type, M, K, N, x, dBias, dY) && aligned_to(dResidual, 16)) {  // the residual rides on the reduction
+        const MmqExtra ex{nullptr, nullptr, dResidual};
+        return launch_mmq(type, x, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream, &ex);
     }
     if (int rc = gq_qdense_f32(type, x, M, K, dW, N, dBias, act, dY, stream)) return rc;
     if (dResidual) return launch_add(dY, dResidual, dY, M * N, (hipStream_t)stream);
@@ -492,7 +505,7 @@ int gq_qdense_gated_f32(int type, const float *dX, int64_t M, int64_t K, const g
     if (int rc = use_device()) return rc;
     RmsNorm rn{nullptr, 0.f, 0.f};
     if (norm) rn = RmsNorm{norm->dGain, norm->eps, norm->gain_offset};
-    if (fold_into_gemv(type, M, K, N, dX, rn.gain, dBiasGate, dY))
+    if (fold_into_gemv(type, M, K, N, dX, rn.gain, dBiasGate, dY, true))
         return launch_gemv_ks_ext(type, dX, M, K, norm ? &rn : nullptr, (const uint8_t *)dWgate, dBiasGate, (const uint8_t *)dWup, dBiasUp,
                                   nullptr, N, act, dY, (hipStream_t)stream);
     if (block_takes_two_pass(type, M, K, N, dX, rn.gain, dBiasGate, dY, true)) {
@@ -510,6 +523,11 @@ int gq_qdense_gated_f32(int type, const float *dX, int64_t M, int64_t K, const g
         float *xn = static_cast<float *>(ws);
         if (int rc = launch_rmsnorm(dX, M, K, rn.gain, rn.gain_offset, rn.eps, xn, (hipStream_t)stream)) return rc;
         x = xn;
+    }
+    if (dense_takes_split_k(type, M, K, N, x, dBiasGate, dY) && (!dBiasUp || aligned_to(dBiasUp, 16))) {
+        // both matrices against one activation image; the reduction forms act(gate) * up
+        const MmqExtra ex{(const uint8_t *)dWup, dBiasUp, nullptr};
+        return launch_mmq(type, x, false, M, K, (const uint8_t *)dWgate, N, dBiasGate, act, dY, (hipStream_t)stream, &ex);
     }
     float *gate = reinterpret_cast<float *>(static_cast<uint8_t *>(ws) + xn_bytes);
     if (int rc = gq_qdense_f32(type, x, M, K, dWgate, N, dBiasGate, act, gate, stream)) return rc;

@@ -286,21 +286,44 @@ __global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__
     }
 }
 
-// y[m][n] = act(sum_s partial[s][m][n] + bias[n]); N % 4 == 0 is guaranteed by the caller
-__global__ __launch_bounds__(256) void mmq_reduce_kernel(const float *__restrict__ partial, int nslices, int64_t MN, int N,
-                                                         const float *__restrict__ bias, int act, float *__restrict__ Y) {
+// y[m][n] = act(sum_s partial[s][m][n] + bias[n]); N % 4 == 0 is guaranteed by the caller.  With a second
+// set of partial sums (the other matrix of a gated pair) the result is multiplied by
+// sum_s partial2[s][m][n] + bias2[n]; a residual (which may be Y itself) is added last.
+__global__ __launch_bounds__(256) void mmq_reduce_kernel(const float *__restrict__ partial, const float *__restrict__ partial2, int nslices,
+                                                         int64_t MN, int N, const float *__restrict__ bias, const float *__restrict__ bias2,
+                                                         int act, const float *residual, float *Y) {
     const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= MN) return;
-    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int k = 0; k < nslices; k++) {
-        const float4 p = *reinterpret_cast<const float4 *>(partial + (int64_t)k * MN + i);
-        s.x += p.x; s.y += p.y; s.z += p.z; s.w += p.w;
+    auto total = [&](const float *p, const float *b) {
+        float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int k = 0; k < nslices; k++) {
+            const float4 v = *reinterpret_cast<const float4 *>(p + (int64_t)k * MN + i);
+            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        }
+        if (b) {
+            const float4 v = *reinterpret_cast<const float4 *>(b + (int)(i % N));
+            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        }
+        return s;
+    };
+    const float4 s = total(partial, bias);
+    float4 v = make_float4(apply_act(act, s.x), apply_act(act, s.y), apply_act(act, s.z), apply_act(act, s.w));
+    if (partial2) {
+        const float4 u = total(partial2, bias2);
+        v.x *= u.x; v.y *= u.y; v.z *= u.z; v.w *= u.w;
     }
-    if (bias) {
-        const float4 b = *reinterpret_cast<const float4 *>(bias + (int)(i % N));
-        s.x += b.x; s.y += b.y; s.z += b.z; s.w += b.w;
+    if (residual) {
+        const float4 r = *reinterpret_cast<const float4 *>(residual + i);
+        v.x += r.x; v.y += r.y; v.z += r.z; v.w += r.w;
     }
-    *reinterpret_cast<float4 *>(Y + i) = make_float4(apply_act(act, s.x), apply_act(act, s.y), apply_act(act, s.z), apply_act(act, s.w));
+    *reinterpret_cast<float4 *>(Y + i) = v;
+}
+
+int launch_mmq_reduce(const float *partial, const float *partial2, int nslices, int64_t M, int64_t N, const float *bias, int act, float *y,
+                      const MmqExtra *ex, hipStream_t s) {
+    const int64_t MN = M * N;
+    return launch(mmq_reduce_kernel, dim3((unsigned)((MN / 4 + 255) / 256)), dim3(256), 0, s, partial, partial2, nslices, MN, (int)N, bias,
+                  ex ? ex->bias2 : nullptr, act, ex ? ex->residual : nullptr, y);
 }
 
 
@@ -525,7 +548,9 @@ __global__ __launch_bounds__(RT * 128) void mmq_b32_kernel(const uint8_t *__rest
 }
 
 template <int T, int RT>
-int launch_mmq_b32(const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y, hipStream_t s) {
+int launch_mmq_b32(const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y, hipStream_t s,
+                   const MmqExtra *ex) {
+    const uint8_t *W2 = ex ? ex->W2 : nullptr;
     const int cus = device_cu_count();
     const int mtiles = (int)((M + kMT - 1) / kMT);
     const int64_t rowwgs = (N + 32 * RT - 1) / (32 * RT);
@@ -539,11 +564,11 @@ int launch_mmq_b32(const void *x, bool x_is_bf16, int64_t M, int64_t K, const ui
                                    1024 * 64 + 2 * RT * B32Geom<T>::kWaveLds) == hipSuccess;
     }();
     if (!lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", 1024 * 64 + 2 * RT * B32Geom<T>::kWaveLds);
-    // workspace: [activation images: mtiles x nslices x S x 64 bytes][partial sums: nslices x M x N fp32]
+    // workspace: [activation images: mtiles x nslices x S x 64 bytes][partial sums: nslices x M x N fp32, twice for a gated pair]
     const size_t img_bytes = (size_t)mtiles * nslices * S * 64;
     const size_t part_bytes = (size_t)nslices * M * N * sizeof(float);
     void *ws = nullptr;
-    if (int rc = stream_workspace(s, img_bytes + part_bytes, &ws)) return rc;
+    if (int rc = stream_workspace(s, img_bytes + part_bytes * (W2 ? 2 : 1), &ws)) return rc;
     uint8_t *ximg = reinterpret_cast<uint8_t *>(ws);
     float *partial = reinterpret_cast<float *>(ximg + img_bytes);
     const int64_t row_bytes = (K / 32) * B32<T>::kBlockBytes;
@@ -556,9 +581,12 @@ int launch_mmq_b32(const void *x, bool x_is_bf16, int64_t M, int64_t K, const ui
     const dim3 grid((unsigned)rowwgs, (unsigned)nslices, (unsigned)mtiles);
     if (int rc = launch(mmq_b32_kernel<T, RT>, grid, dim3(RT * 128), lds_bytes, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N, row_bytes, S))
         return rc;
-    const int64_t MN = M * N;
-    return launch(mmq_reduce_kernel, dim3((unsigned)((MN / 4 + 255) / 256)), dim3(256), 0, s, (const float *)partial, nslices, MN, (int)N,
-                  bias, act, y);
+    float *partial2 = W2 ? partial + (size_t)nslices * M * N : nullptr;
+    if (W2)
+        if (int rc = launch(mmq_b32_kernel<T, RT>, grid, dim3(RT * 128), lds_bytes, s, (const uint8_t *)ximg, W2, partial2, (int)M, (int)K, (int)N,
+                            row_bytes, S))
+            return rc;
+    return launch_mmq_reduce(partial, partial2, nslices, M, N, bias, act, y, ex, s);
 }
 
 
@@ -701,7 +729,7 @@ __global__ __launch_bounds__(512) void mmq_q6k_kernel(const uint8_t *__restrict_
     }
 }
 
-int launch_mmq_q6k(const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y,
+int launch_mmq_q6k(const MmqExtra *ex, const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y,
                    hipStream_t s) {
     constexpr int kLds = kQ6Slice * 64 + 2 * kQ6RT * kQ6WaveLds;
     static const bool lds_ok = [] {
@@ -711,11 +739,12 @@ int launch_mmq_q6k(const void *x, bool x_is_bf16, int64_t M, int64_t K, const ui
     if (!lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", kLds);
     const int mtiles = (int)((M + kMT - 1) / kMT);
     const int nslices = (int)((K + kQ6Slice - 1) / kQ6Slice);
-    // workspace: [activation images: mtiles x nslices x 64 KiB][partial sums: nslices x M x N fp32]
+    // workspace: [activation images: mtiles x nslices x 64 KiB][partial sums: nslices x M x N fp32, twice for a gated pair]
+    const uint8_t *W2 = ex ? ex->W2 : nullptr;
     const size_t img_bytes = (size_t)mtiles * nslices * kQ6Slice * 64;
     const size_t part_bytes = (size_t)nslices * M * N * sizeof(float);
     void *ws = nullptr;
-    if (int rc = stream_workspace(s, img_bytes + part_bytes, &ws)) return rc;
+    if (int rc = stream_workspace(s, img_bytes + part_bytes * (W2 ? 2 : 1), &ws)) return rc;
     uint8_t *ximg = reinterpret_cast<uint8_t *>(ws);
     float *partial = reinterpret_cast<float *>(ximg + img_bytes);
     const int64_t row_bytes = (K / 256) * 210;
@@ -729,9 +758,12 @@ int launch_mmq_q6k(const void *x, bool x_is_bf16, int64_t M, int64_t K, const ui
     if (int rc = launch(mmq_q6k_kernel, grid, dim3(kQ6RT * 128), (size_t)kLds, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N,
                         row_bytes))
         return rc;
-    const int64_t MN = M * N;
-    return launch(mmq_reduce_kernel, dim3((unsigned)((MN / 4 + 255) / 256)), dim3(256), 0, s, (const float *)partial, nslices, MN, (int)N,
-                  bias, act, y);
+    float *partial2 = W2 ? partial + (size_t)nslices * M * N : nullptr;
+    if (W2)
+        if (int rc = launch(mmq_q6k_kernel, grid, dim3(kQ6RT * 128), (size_t)kLds, s, (const uint8_t *)ximg, W2, partial2, (int)M, (int)K, (int)N,
+                            row_bytes))
+            return rc;
+    return launch_mmq_reduce(partial, partial2, nslices, M, N, bias, act, y, ex, s);
 }
 
 }  // namespace
@@ -746,12 +778,13 @@ bool mmq_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, con
 }
 
 int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias,
-               int act, float *y, hipStream_t s) {
+               int act, float *y, hipStream_t s, const MmqExtra *ex) {
+    const uint8_t *W2 = ex ? ex->W2 : nullptr;
     // (four row tiles per workgroup measured a little faster than two)
-    if (type == kQ8_0) return launch_mmq_b32<kQ8_0, 4>(x, x_is_bf16, M, K, W, N, bias, act, y, s);
-    if (type == kQ4_0) return launch_mmq_b32<kQ4_0, 4>(x, x_is_bf16, M, K, W, N, bias, act, y, s);
-    if (type == kIQ4_NL) return launch_mmq_b32<kIQ4_NL, 4>(x, x_is_bf16, M, K, W, N, bias, act, y, s);
-    if (type == kQ6_K) return launch_mmq_q6k(x, x_is_bf16, M, K, W, N, bias, act, y, s);
+    if (type == kQ8_0) return launch_mmq_b32<kQ8_0, 4>(x, x_is_bf16, M, K, W, N, bias, act, y, s, ex);
+    if (type == kQ4_0) return launch_mmq_b32<kQ4_0, 4>(x, x_is_bf16, M, K, W, N, bias, act, y, s, ex);
+    if (type == kIQ4_NL) return launch_mmq_b32<kIQ4_NL, 4>(x, x_is_bf16, M, K, W, N, bias, act, y, s, ex);
+    if (type == kQ6_K) return launch_mmq_q6k(ex, x, x_is_bf16, M, K, W, N, bias, act, y, s);
     if (type != kQ4_K) return fail(GQ_ERR_NOT_IMPLEMENTED, "mmq: ggml type %d is not implemented", type);
     static const bool lds_ok = [] {
         return hipFuncSetAttribute(reinterpret_cast<const void *>(mmq_q4k_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -760,11 +793,11 @@ int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, co
     if (!lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", kLdsBytes);
     const int nslices = (int)((K + kSliceK - 1) / kSliceK);
     const int mtiles = (int)((M + kMT - 1) / kMT);
-    // workspace: [activation images: mtiles x nslices x kLdsBytes][partial sums: nslices x M x N fp32]
+    // workspace: [activation images: mtiles x nslices x kLdsBytes][partial sums: nslices x M x N fp32, twice for a gated pair]
     const size_t img_bytes = (size_t)mtiles * nslices * kLdsBytes;
     const size_t part_bytes = (size_t)nslices * M * N * sizeof(float);
     void *ws = nullptr;
-    if (int rc = stream_workspace(s, img_bytes + part_bytes, &ws)) return rc;
+    if (int rc = stream_workspace(s, img_bytes + part_bytes * (W2 ? 2 : 1), &ws)) return rc;
     uint8_t *ximg = reinterpret_cast<uint8_t *>(ws);
     float *partial = reinterpret_cast<float *>(ximg + img_bytes);
     const int64_t row_bytes = (K / 256) * 144;
@@ -772,14 +805,14 @@ int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, co
                            : launch(mmq_xprep_kernel<false>, dim3((unsigned)nslices, (unsigned)mtiles, 8), dim3(512), 0, s, x, ximg, (int)M, (int)K))
         return rc;
     const dim3 grid((unsigned)((N + kRowsPerWG - 1) / kRowsPerWG), (unsigned)nslices);
-    for (int64_t m0 = 0; m0 < M; m0 += kMT) {
-        if (int rc = launch(mmq_q4k_kernel, grid, dim3(256 * kParts), (size_t)kLdsBytes, s, (const uint8_t *)ximg, W, partial, (int)M,
-                            (int)K, (int)N, row_bytes, (int)m0))
-            return rc;
-    }
-    const int64_t MN = M * N;
-    return launch(mmq_reduce_kernel, dim3((unsigned)((MN / 4 + 255) / 256)), dim3(256), 0, s, (const float *)partial, nslices, MN,
-                  (int)N, bias, act, y);
+    float *partial2 = W2 ? partial + (size_t)nslices * M * N : nullptr;
+    for (int which = 0; which < (W2 ? 2 : 1); which++)
+        for (int64_t m0 = 0; m0 < M; m0 += kMT) {
+            if (int rc = launch(mmq_q4k_kernel, grid, dim3(256 * kParts), (size_t)kLdsBytes, s, (const uint8_t *)ximg, which ? W2 : W,
+                                which ? partial2 : partial, (int)M, (int)K, (int)N, row_bytes, (int)m0))
+                return rc;
+        }
+    return launch_mmq_reduce(partial, partial2, nslices, M, N, bias, act, y, ex, s);
 }
 
 }  // namespace gq
