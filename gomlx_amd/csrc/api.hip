@@ -115,24 +115,25 @@ int check_dense_args(const char *fn, int type, const void *x, int64_t M, int64_t
 }
 
 // Batch sizes served by the split-K small-batch kernels: measured crossovers against the GEMV passes
-// below and the two-pass GEMM above.  A GEMV pass per row costs time in proportion to the weight
-// bytes, the split-K kernels a fixed part plus less per byte, so large matrices change over earlier.
+// below and the two-pass GEMM above.  GEMV passes cost time in proportion to the weight bytes (small
+// matrices: a pass per row, sharing W through the caches; large ones: a pass per four rows, two for
+// Q6_K), the split-K kernels a fixed part plus less per byte.
 // Measured (us, rows 2 3 4 5 6 7 8 10; GEMV passes | split-K):
-//   Q8_0 4096x4096 (18 MB)   8.8 10.5 12.3 14.8 16.4 18.2 20.2 24.0 | 16.6     4096x14336 (62 MB) 20.4 27.4 35.4 43.7 51.6 .. | 29.5
-//   Q4_0 4096x4096 (9 MB)    7.0  7.6  9.4 11.6 12.8 14.1 15.8 19.0 | 15.5     4096x14336 (33 MB) 13.3 16.7 20.5 22.9 26.2 29.7 | 24.8
-//   Q4_K 4096x4096           7.9  9.1 11.3 13.9 15.5 17.6 20.5 22.9 | 18.8     4096x14336         14.9 18.6 23.1 27.5 31.9 .. | 20.8
-//   Q6_K 4096x4096 (14 MB)   9.3 11.9 14.3 16.7 18.7 21.6 22.9 27.5 | 18.6     4096x14336 (48 MB) 20.8 26.7 34.1 41.5 49.1 .. | 42.0
-//   IQ4_NL 4096x4096         8.2  9.6 12.0 14.5 16.1 18.6 20.1 23.6 | 16.0     4096x14336         18.9 21.8 28.6 34.5 40.1 .. | 27.3
+//   Q8_0 4096x4096 (18 MB)   9.5 10.5 12.8 15.1 17.4 19.4 21.5 25.9 | 16.6   4096x14336 (62 MB) 15.2 15.9 16.1 25.8 26.9 28.5 26.0 36.7 | 29.5
+//                                                                            14336x4096         16.0 20.2 20.5 30.5 32.7 38.4 36.6 49.8 | 30.8
+//   Q4_0 4096x4096 (9 MB)    7.1  8.1 10.9 12.0 13.2 15.1 16.6 19.7 | 15.5   4096x14336 (33 MB) 11.1 15.1 14.8 20.9 22.2 28.2 25.7 33.3 | 24.8
+//   Q4_K 4096x4096           7.8  9.7 11.9 14.0 16.9 18.7 20.6 24.4 | 18.8   4096x14336         12.6 15.9 15.5 22.6 25.8 28.7 27.2 36.3 | 20.8
+//   Q6_K 4096x4096 (14 MB)   9.2 11.5 14.3 17.6 19.5 21.5 23.7 28.9 | 18.6   4096x14336 (48 MB) 15.8 24.8 24.0 33.3 33.9 43.0 43.3 52.9 | 42.0
+//   IQ4_NL 4096x4096         8.1 10.1 12.3 14.3 16.7 18.7 20.5 23.9 | 16.0   4096x14336         14.1 16.7 17.1 26.3 26.7 31.7 29.5 40.0 | 27.3
 // The Q6_K kernel pays 16 scale groups per super-block and only wins for a single tile of 32 batch columns.
-constexpr int64_t kLargeWeightBytes = (int64_t)24 << 20;
 int64_t split_k_from(int type, int64_t weight_bytes) {
     const bool large = weight_bytes >= kLargeWeightBytes;
     switch (type) {
-    case GQ_Q8_0: return large ? 4 : 7;
+    case GQ_Q8_0: return large ? 6 : 7;
     case GQ_Q4_0: return large ? 6 : 9;
-    case GQ_Q4_K: return large ? 4 : 8;
-    case GQ_Q6_K: return large ? 6 : 7;
-    case GQ_IQ4_NL: return large ? 4 : 7;
+    case GQ_Q4_K: return large ? 5 : 8;
+    case GQ_Q6_K: return 7;
+    case GQ_IQ4_NL: return large ? 6 : 7;
     default: return 8;
     }
 }
@@ -395,16 +396,17 @@ int gq_rmsnorm_f32(const float *dX, int64_t M, int64_t K, const float *dGain, fl
 
 namespace {
 // The calls around a projection run inside the decode GEMV while that kernel is the right one for
-// the batch: its time grows by a full pass per row, the split-K form costs the same for any batch up
-// to 32 rows.  Measured on gate/up 4096 -> 14336 with RMSNorm and SiLU (us; GEMV at 2, 4, 6 rows | split-K):
-// Q4_K 24 39 56 | 44, Q8_0 40 69 102 | 61, Q4_0 24 38 54 | 51, Q6_K 39 65 94 | 90: the change-over sits at the
-// point where a plain dense call changes kernels, one row later for Q4_K; a single projection with
-// norm or residual pays one small extra kernel in the split-K form and changes one or two rows later.
+// the batch: over a large matrix its time grows by a pass per two rows, the split-K form costs the
+// same for any batch up to 32 rows.  Measured on gate/up 4096 -> 14336 with RMSNorm and SiLU (us; GEMV
+// at 2, 4 rows | split-K): Q4_K 22 35 | 45, Q8_0 27 43 | 61, Q4_0 19 32 | 51, Q6_K 27 45 (63 at 6) | 90: the
+// change-over sits at or just past the point where a plain dense call changes kernels; a single
+// projection with norm or residual pays one small extra kernel in the split-K form and changes one
+// or two rows later.
 bool fold_into_gemv(int type, int64_t M, int64_t K, int64_t N, const float *x, const float *gain, const float *bias, const float *y, bool gated) {
     if (!gemv_ks_ext_supported(type, M, K, N, x, gain)) return false;
     const int64_t wb = weight_bytes_of(type, K, N);
     const bool large = wb >= kLargeWeightBytes;
-    const int64_t margin = gated ? (large && type == GQ_Q4_K ? 1 : 0) : (large ? 1 : 2);
+    const int64_t margin = gated ? (!large ? 0 : type == GQ_Q6_K ? 2 : (type == GQ_Q4_K || type == GQ_Q4_0) ? 1 : 0) : (large ? 1 : 2);
     return !(M >= split_k_from(type, wb) + margin && mmq_supported(type, M, K, N, x, bias, y));
 }
 

@@ -61,6 +61,9 @@ int launch(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t shmem, hipStr
     return GQ_OK;
 }
 
+// Weight matrices from this size on count as large where kernels choose by size (batched GEMV passes, split-K crossovers).
+constexpr int64_t kLargeWeightBytes = (int64_t)24 << 20;
+
 // ---- kernel families (one translation unit each) -----------------------------------------
 int launch_dequantize(int type, const uint8_t *W, int64_t N, int64_t K, float *out, hipStream_t s);
 int launch_embedding_lookup(int type, const uint8_t *table, int64_t vocab, int64_t K, const int32_t *idx,

@@ -411,6 +411,10 @@ template <> struct KS<kQ6_K> {
     }
 };
 
+// Activation rows a pass can serve at once: the planes of four rows fit the register file next to
+// the loads in flight, except for Q6_K (four scale and sum registers per row, the widest decoder).
+template <int T> constexpr int ks_max_rows() { return T == kQ6_K ? 2 : 4; }
+
 template <int T>
 __device__ __forceinline__ void ks_load(typename KS<T>::Raw &r, const uint8_t *p, int c) {
     if constexpr (T == kQ4_K || T == kQ6_K) KS<T>::load(r, p, c);
@@ -460,10 +464,17 @@ struct KsExt {
     int norm;            // apply the RMS normalisation
 };
 
-template <int T, int PF, int WIN, bool EXT = false, bool XBF16 = false>
+//
+// R > 1: the pass serves R activation rows at once (xrows <= R of them exist; row r of x lies
+// x_stride bytes after row r - 1, of y and of the residual N values): the fixed-point planes of all R
+// rows stay in registers and every weight load is contracted against each of them, so a batch of
+// two to four rows costs one pass over W, not one per row (the arithmetic stays well below the
+// memory time up to four rows).
+template <int T, int PF, int WIN, bool EXT = false, bool XBF16 = false, int R = 1>
 __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8_t *__restrict__ W,
                                         const float *__restrict__ bias, float *__restrict__ y, int N, int64_t row_bytes, int iters,
-                                        int nslices, int half_tail, int act, int waves, int wg, uint32_t *lds, const KsExt *extp = nullptr) {
+                                        int nslices, int half_tail, int act, int waves, int wg, uint32_t *lds, const KsExt *extp = nullptr,
+                                        int xrows = 1, int64_t x_stride = 0) {
     typedef typename KS<T>::Raw Raw;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int rg = lane >> 3, c = lane & 7;
@@ -472,15 +483,17 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8
     if constexpr (EXT) ext = *extp;
     const bool dual = EXT && ext.W2 != nullptr;
     const int row0 = wg * (dual ? rows_wg >> 1 : rows_wg);
-    float *all = reinterpret_cast<float *>(lds + waves * kWaveLdsDwords);  // partial sums [waves][rows_wg]
-    float *ssq_w = all + waves * rows_wg;                                  // EXT: sum of squares per wavefront
-    float ssq = 0.f;
+    float *all = reinterpret_cast<float *>(lds + waves * kWaveLdsDwords);  // partial sums [waves][R][rows_wg]
+    float *ssq_w = all + waves * R * rows_wg;                              // EXT: sum of squares [waves][R]
+    float ssq[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) ssq[r] = 0.f;
     // What a lane fetches of slice sl, kept raw until the slice is converted: nothing between the
     // load and the conversion may depend on the loaded values or sit behind a branch, or the
     // wavefront would wait for its activations before it issues the first weight load.  fp32: two
     // float4; bf16: one uint4 (widened at conversion).  The lanes that face the missing half of a
     // last half slice re-read the present half and are zeroed at conversion.
-    struct XRaw { uint4 a, b, ga, gb; bool zero; };
+    struct XRaw { uint4 a[R], b[R], ga, gb; bool zero; };
     const bool upper_half = lane >= 32;  // this lane converts values 256 .. 511 of a slice (in both activation layouts)
     const float *gsrc = nullptr;         // EXT: the gain, or any readable stand-in of K floats when there is none
     if constexpr (EXT) gsrc = ext.gain ? ext.gain : reinterpret_cast<const float *>(xv);
@@ -488,13 +501,15 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8
         XRaw r;
         r.zero = half_tail && sl == nslices - 1 && upper_half;
         const int xl = r.zero ? lane - 32 : lane;
-        r.b = r.ga = r.gb = make_uint4(0, 0, 0, 0);
-        if constexpr (XBF16) {
-            r.a = KS<T>::x_fetch_bf16(reinterpret_cast<const uint16_t *>(xv) + sl * kSliceValues, xl);
-        } else {
-            KS<T>::x_fetch(reinterpret_cast<const float *>(xv) + sl * kSliceValues, xl, r.a, r.b);
-            if constexpr (EXT) KS<T>::x_fetch(gsrc + sl * kSliceValues, xl, r.ga, r.gb);
+        r.ga = r.gb = make_uint4(0, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < R; i++) {  // rows past the last one re-read it (their results are not stored)
+            const uint8_t *xrow = reinterpret_cast<const uint8_t *>(xv) + (int64_t)min(i, xrows - 1) * x_stride;
+            r.b[i] = make_uint4(0, 0, 0, 0);
+            if constexpr (XBF16) r.a[i] = KS<T>::x_fetch_bf16(reinterpret_cast<const uint16_t *>(xrow) + sl * kSliceValues, xl);
+            else KS<T>::x_fetch(reinterpret_cast<const float *>(xrow) + sl * kSliceValues, xl, r.a[i], r.b[i]);
         }
+        if constexpr (EXT) KS<T>::x_fetch(gsrc + sl * kSliceValues, xl, r.ga, r.gb);
         return r;
     };
     auto as_f4 = [](const uint4 &u) {
@@ -502,13 +517,13 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8
                            __builtin_bit_cast(float, u.w));
     };
     // the activations a fetched slice stands for (EXT: sum of squares taken, gain applied)
-    auto x_values = [&](const XRaw &r) -> XPair {
+    auto x_values = [&](const XRaw &r, int i) -> XPair {
         XPair p;
-        if constexpr (XBF16) p = KS<T>::x_widen_bf16(r.a);
-        else { p.lo = as_f4(r.a); p.hi = as_f4(r.b); }
+        if constexpr (XBF16) p = KS<T>::x_widen_bf16(r.a[i]);
+        else { p.lo = as_f4(r.a[i]); p.hi = as_f4(r.b[i]); }
         if (r.zero) { p.lo = make_float4(0.f, 0.f, 0.f, 0.f); p.hi = p.lo; }
         if constexpr (EXT) {
-            ssq += (p.lo.x * p.lo.x + p.lo.y * p.lo.y) + (p.lo.z * p.lo.z + p.lo.w * p.lo.w) + (p.hi.x * p.hi.x + p.hi.y * p.hi.y) +
+            ssq[i] += (p.lo.x * p.lo.x + p.lo.y * p.lo.y) + (p.lo.z * p.lo.z + p.lo.w * p.lo.w) + (p.hi.x * p.hi.x + p.hi.y * p.hi.y) +
                    (p.hi.z * p.hi.z + p.hi.w * p.hi.w);
             if (ext.gain) {
                 const float4 gl = as_f4(r.ga), gh = as_f4(r.gb);
@@ -523,7 +538,7 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8
         uint4 *my_planes = reinterpret_cast<uint4 *>(lds + wave * kWaveLdsDwords);
         float *my_scales = reinterpret_cast<float *>(my_planes + 64);
         float *my_sums = my_scales + 16;
-        float *part = all + wave * rows_wg;
+        float *part = all + wave * R * rows_wg;
 
         KS_TRACE(0);
         KS_TRACE_WALL(12);
@@ -543,30 +558,35 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8
         for (int j = 0; j < WIN; j++) ks_load<T>(buf[j], addr(0, j), lane_c(0));
         KS_TRACE(1);
 
-        uint4 xq[8];
+        uint4 xq[R][8];
         constexpr int NS = KS<T>::kScales, SPAN = KS<T>::kSumSpan;
-        float xsc[NS], xsm[NS];
+        float xsc[R][NS], xsm[R][NS];
 #pragma unroll
-        for (int i = 0; i < NS; i++) xsm[i] = 0.f;
+        for (int q = 0; q < R; q++)
+#pragma unroll
+            for (int i = 0; i < NS; i++) xsm[q][i] = 0.f;
         auto stage = [&](const XRaw &r) {
-            const XPair p = x_values(r);
-            const Staged st = KS<T>::stage(p);
-            my_planes[lane] = st.planes;
-            if ((lane & 3) == 0) my_scales[lane >> 2] = st.scale;
-            if constexpr (SPAN == 32) { if ((lane & 3) == 0) my_sums[lane >> 2] = st.sum; }
-            if constexpr (SPAN == 16) { if ((lane & 1) == 0) my_sums[lane >> 1] = st.sum; }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-            for (int i = 0; i < 8; i++) xq[i] = my_planes[KS<T>::plane_idx(c, i)];
+            for (int q = 0; q < R; q++) {  // the activation rows take turns in the wavefront's piece of LDS
+                const XPair p = x_values(r, q);
+                const Staged st = KS<T>::stage(p);
+                my_planes[lane] = st.planes;
+                if ((lane & 3) == 0) my_scales[lane >> 2] = st.scale;
+                if constexpr (SPAN == 32) { if ((lane & 3) == 0) my_sums[lane >> 2] = st.sum; }
+                if constexpr (SPAN == 16) { if ((lane & 1) == 0) my_sums[lane >> 1] = st.sum; }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-            for (int i = 0; i < NS; i++) {
-                xsc[i] = my_scales[KS<T>::scale_idx(c, i)];
-                if constexpr (SPAN != 0) xsm[i] = my_sums[KS<T>::sum_idx(c, i)];
+                for (int i = 0; i < 8; i++) xq[q][i] = my_planes[KS<T>::plane_idx(c, i)];
+#pragma unroll
+                for (int i = 0; i < NS; i++) {
+                    xsc[q][i] = my_scales[KS<T>::scale_idx(c, i)];
+                    if constexpr (SPAN != 0) xsm[q][i] = my_sums[KS<T>::sum_idx(c, i)];
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
             }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
         };
         stage(xr);
         KS_TRACE(2);
@@ -582,13 +602,18 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8
             const int nj = wrap ? j + 1 : j, ni0 = wrap ? 0 : i0 + PF;
 #pragma unroll
             for (int jj = 0; jj < PF; jj++) {
-                float d = KS<T>::dot(buf[jj], xq, xsc, xsm, c);
+                float d[R];
+#pragma unroll
+                for (int q = 0; q < R; q++) d[q] = KS<T>::dot(buf[jj], xq[q], xsc[q], xsm[q], c);
                 if (jj + WIN < PF) ks_load<T>(buf[jj + WIN], addr(j, i0 + jj + WIN), lane_c(j));
                 else if (!last_group) ks_load<T>(buf[jj + WIN - PF], addr(nj, ni0 + jj + WIN - PF), lane_c(nj));
-                d = ks_oct_sum(d);
-                if (c == 0) {
-                    float *slot = part + (i0 + jj) * 8 + rg;
-                    *slot = j == 0 ? d : *slot + d;
+#pragma unroll
+                for (int q = 0; q < R; q++) {
+                    const float t = ks_oct_sum(d[q]);
+                    if (c == 0) {
+                        float *slot = part + q * rows_wg + (i0 + jj) * 8 + rg;
+                        *slot = j == 0 ? t : *slot + t;
+                    }
                 }
             }
             if (wrap && !last_group) {  // next group starts a new slice: convert its activations
@@ -602,45 +627,46 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8
         KS_TRACE_WALL(13);
         if constexpr (EXT) {
             if (ext.norm) {
-                ssq = ks_oct_sum(ssq);
-                ssq += __shfl_xor(ssq, 8);
-                ssq += __shfl_xor(ssq, 16);
-                ssq += __shfl_xor(ssq, 32);
-                if (lane == 0) ssq_w[wave] = ssq;
+#pragma unroll
+                for (int q = 0; q < R; q++) {
+                    float t = ks_oct_sum(ssq[q]);
+                    t += __shfl_xor(t, 8);
+                    t += __shfl_xor(t, 16);
+                    t += __shfl_xor(t, 32);
+                    if (lane == 0) ssq_w[wave * R + q] = t;
+                }
             }
         }
     }
     __syncthreads();
-    if constexpr (EXT) {
-        float inv = 1.f;
-        if (ext.norm) {
-            float t = 0.f;
-            for (int w = 0; w < waves; w++) t += ssq_w[w];
-            inv = 1.f / sqrtf(t * ext.inv_k + ext.eps);
-        }
-        const int rows_out = dual ? rows_wg >> 1 : rows_wg;
-        for (int r = tid; r < rows_out; r += blockDim.x) {
-            const int row = row0 + r;
-            if (row >= N) continue;
+    // output row r of activation row q: the wavefronts' partial sums meet here
+    const int rows_out = dual ? rows_wg >> 1 : rows_wg;
+    for (int e = tid; e < rows_out * R; e += blockDim.x) {
+        const int q = e / rows_out, r = e - q * rows_out;
+        const int row = row0 + r;
+        if (row >= N || q >= xrows) continue;
+        const int64_t at = (int64_t)q * N + row;
+        if constexpr (EXT) {
+            float inv = 1.f;
+            if (ext.norm) {
+                float t = 0.f;
+                for (int w = 0; w < waves; w++) t += ssq_w[w * R + q];
+                inv = 1.f / sqrtf(t * ext.inv_k + ext.eps);
+            }
             const int slot = dual ? ((r >> 3) * 16 + (r & 7)) : r;  // row-step 2 * (r / 8) of the alternation
             float t = 0.f, u = 0.f;
             for (int w = 0; w < waves; w++) {
-                t += all[w * rows_wg + slot];
-                if (dual) u += all[w * rows_wg + slot + 8];
+                t += all[(w * R + q) * rows_wg + slot];
+                if (dual) u += all[(w * R + q) * rows_wg + slot + 8];
             }
             t = apply_act(act, fmaf(t, inv, bias ? bias[row] : 0.f));
             if (dual) t *= fmaf(u, inv, ext.bias2 ? ext.bias2[row] : 0.f);
-            if (ext.residual) t += ext.residual[row];
-            y[row] = t;
-        }
-        return;
-    }
-    for (int r = tid; r < rows_wg; r += blockDim.x) {
-        const int row = row0 + r;
-        if (row < N) {
+            if (ext.residual) t += ext.residual[at];
+            y[at] = t;
+        } else {
             float t = 0.f;
-            for (int w = 0; w < waves; w++) t += all[w * rows_wg + r];
-            y[row] = apply_act(act, t + (bias ? bias[row] : 0.f));
+            for (int w = 0; w < waves; w++) t += all[(w * R + q) * rows_wg + r];
+            y[at] = apply_act(act, t + (bias ? bias[row] : 0.f));
         }
     }
 }
@@ -663,8 +689,8 @@ bool ks_split(int64_t K, int &waves, int &nslices, int &half_tail) {
     return true;
 }
 
-size_t ks_lds_bytes(int waves, int iters) {
-    return (size_t)waves * kWaveLdsDwords * 4 + (size_t)waves * iters * 8 * sizeof(float) + 8 * sizeof(float);  // + sums of squares (EXT)
+size_t ks_lds_bytes(int waves, int iters, int xrows = 1) {  // xrows: activation rows per pass
+    return (size_t)waves * kWaveLdsDwords * 4 + (size_t)waves * xrows * iters * 8 * sizeof(float) + 8 * xrows * sizeof(float);  // + sums of squares (EXT)
 }
 
 // Row-steps per workgroup and per group: up to 8 row-steps form one group (an even count when two
@@ -700,6 +726,17 @@ bool ks_plan(int64_t K, int64_t N, KsPlan &p, bool even_iters = false) {
     p.wgs = (int)((N + (int64_t)p.iters * 8 - 1) / ((int64_t)p.iters * 8));
     p.shmem = ks_lds_bytes(p.waves, p.iters);
     return true;
+}
+
+// A plan whose row-steps come in groups of 1, 2 or (if max_pf allows) 4: the multi-row kernels
+// exist for those only, and four rows' planes leave registers for two row-steps in flight.
+void ks_regroup(KsPlan &p, int64_t N, bool dual, int max_pf) {
+    if (p.pf > max_pf || p.pf == 3) {
+        p.iters = (p.iters + max_pf - 1) / max_pf * max_pf;
+        p.pf = max_pf;
+    }
+    const int64_t rows_wg = (int64_t)p.iters * (dual ? 4 : 8);
+    p.wgs = (int)((N + rows_wg - 1) / rows_wg);
 }
 
 // Several independent batch-1 problems of one format in a single launch: workgroups

@@ -12,16 +12,17 @@ namespace gq {
 
 namespace {
 
-template <int T, int PF, int WIN>
+template <int T, int PF, int WIN, int R>
 __global__ __launch_bounds__(512) void gemv_ks_ext_kernel(const float *__restrict__ X, const uint8_t *__restrict__ W,
-                                                          const float *__restrict__ bias, float *__restrict__ Y, int K, int N,
+                                                          const float *__restrict__ bias, float *__restrict__ Y, int M, int K, int N,
                                                           int64_t row_bytes, int iters, int nslices, int half_tail, int act,
                                                           const KsExt ext) {
     extern __shared__ uint32_t lds[];
+    const int r0 = (int)blockIdx.y * R;
     KsExt e = ext;
-    if (e.residual) e.residual += (int64_t)blockIdx.y * N;
-    ks_body<T, PF, WIN, true>(X + (int64_t)blockIdx.y * K, W, bias, Y + (int64_t)blockIdx.y * N, N, row_bytes, iters, nslices, half_tail,
-                              act, (int)(blockDim.x >> 6), (int)blockIdx.x, lds, &e);
+    if (e.residual) e.residual += (int64_t)r0 * N;
+    ks_body<T, PF, WIN, true, false, R>(X + (int64_t)r0 * K, W, bias, Y + (int64_t)r0 * N, N, row_bytes, iters, nslices, half_tail, act,
+                                        (int)(blockDim.x >> 6), (int)blockIdx.x, lds, &e, min(R, M - r0), (int64_t)K * 4);
 }
 
 // Batched submission (several batch-1 projections of one format in one launch) with one RMS
@@ -43,14 +44,25 @@ int launch_batch_ext(int count, const XsBatchItem *items, const KsExt &ext, hipS
     return launch(gemv_ks_batch_ext_kernel<T>, dim3((unsigned)wgs), dim3(512), shmem, s, b, ext);
 }
 
-template <int T, int PF>
+template <int T, int PF, int R = 1>
 int launch_ext_pf(const KsPlan &p, const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y,
                   const KsExt &ext, hipStream_t s) {
     const int64_t row_bytes = (K / Geom<T>::vpb) * Geom<T>::bpb;
-    const dim3 grid((unsigned)p.wgs, (unsigned)M), block((unsigned)p.waves * 64);
+    const dim3 grid((unsigned)p.wgs, (unsigned)((M + R - 1) / R)), block((unsigned)p.waves * 64);
     constexpr int WIN = PF < 3 ? PF : 3;
-    return launch(gemv_ks_ext_kernel<T, PF, WIN>, grid, block, p.shmem, s, x, W, bias, y, (int)K, (int)N, row_bytes, p.iters, p.nslices,
-                  p.half_tail, act, ext);
+    return launch(gemv_ks_ext_kernel<T, PF, WIN, R>, grid, block, ks_lds_bytes(p.waves, p.iters, R), s, x, W, bias, y, (int)M, (int)K, (int)N,
+                  row_bytes, p.iters, p.nslices, p.half_tail, act, ext);
+}
+
+template <int T, int R>
+int launch_ext_rows(KsPlan p, bool dual, const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y,
+                    const KsExt &ext, hipStream_t s) {
+    ks_regroup(p, N, dual, 4);  // (two alternating matrices: 2 or 4, both even)
+    switch (p.pf) {
+    case 1: return launch_ext_pf<T, 1, R>(p, x, M, K, W, N, bias, act, y, ext, s);
+    case 2: return launch_ext_pf<T, 2, R>(p, x, M, K, W, N, bias, act, y, ext, s);
+    default: return launch_ext_pf<T, 4, R>(p, x, M, K, W, N, bias, act, y, ext, s);
+    }
 }
 
 template <int T>
@@ -61,6 +73,9 @@ int launch_ext(const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N
     KsPlan p;
     if (!ks_plan(K, dual ? 2 * N : N, p, dual)) return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv_ks: unsupported problem");
     if (dual) p.wgs = (int)((N + p.iters * 4 - 1) / (p.iters * 4));
+    // batches over a large matrix run as passes of two rows (the extras leave no registers for the planes of four)
+    if (M >= 2 && (int64_t)gq_row_bytes(T, K) * N * (dual ? 2 : 1) >= kLargeWeightBytes)
+        return launch_ext_rows<T, 2>(p, dual, x, M, K, W, N, bias, act, y, ext, s);
     switch (p.pf) {
     case 1: return launch_ext_pf<T, 1>(p, x, M, K, W, N, bias, act, y, ext, s);
     case 2: return launch_ext_pf<T, 2>(p, x, M, K, W, N, bias, act, y, ext, s);

@@ -411,20 +411,42 @@ def test_dispatch_boundaries(gpu, oracle, t, M, K, N, bf16, act, with_bias):
     assert err < (TOL_BF16 if bf16 else TOL_F32), (t, M, K, N, bf16, act, err)
 
 
-@pytest.mark.parametrize("t,N,first", [(Q8_0, 6400, 4), (Q4_0, 11264, 6), (Q4_K, 11264, 4), (Q6_K, 8192, 6), (IQ4_NL, 11264, 4)])
-def test_split_k_crossover_on_large_matrices(gpu, oracle, t, N, first):
-    """Matrices of 24 MB and more hand over from GEMV passes to the split-K kernels at fewer rows than
-    small ones: the batch sizes either side of that point, fp32 and bf16 activations."""
+@pytest.mark.parametrize("t,N", [(Q8_0, 6400), (Q4_0, 11264), (Q4_K, 11264), (Q6_K, 8192), (IQ4_NL, 11264)])
+def test_small_batches_on_large_matrices(gpu, oracle, t, N):
+    """Matrices of 24 MB and more: batches of 2 .. 8 rows run as GEMV passes of up to four rows against one
+    reading of W (remainders of 1, 2, 3 rows included) and hand over to the split-K kernels after 5 - 7 rows."""
     K = 4096
     assert N * ggml.row_bytes(t, K) >= 24 << 20
     W = synth.weights(t, 330 + t, N, K)
     bias = synth.normal(331 + t, 0, N).astype(np.float32) * 0.1
-    for M in (first - 1, first, first + 1):
+    for M in (2, 3, 4, 5, 6, 7, 8):
         x = synth.activations(332 + M, M, K)
         want = oracle.c_qdense(t, x, W, bias, 3)
         assert rel_err(run_dense(gpu, t, x, W, bias, 3), want) < TOL_F32, (t, M)
-    xb = bf16_round(synth.activations(340, first, K))
-    assert rel_err(run_dense(gpu, t, xb, W, bias, 3, bf16=True), oracle.c_qdense(t, xb, W, bias, 3)) < TOL_BF16, t
+    for M in (3, 5):
+        xb = bf16_round(synth.activations(340 + M, M, K))
+        assert rel_err(run_dense(gpu, t, xb, W, bias, 3, bf16=True), oracle.c_qdense(t, xb, W, bias, 3)) < TOL_BF16, (t, M)
+
+
+@pytest.mark.parametrize("t,N", [(Q8_0, 3328), (Q4_K, 5632), (Q6_K, 4096)])
+def test_small_batches_with_neighbours_on_large_matrices(gpu, oracle, t, N):
+    """The same batches through the calls around a projection: passes of two rows inside the decode GEMV."""
+    K = 4096
+    assert 2 * N * ggml.row_bytes(t, K) >= 24 << 20
+    for i, M in enumerate((2, 3, 4, 5)):
+        err = gated_case(gpu, oracle, t, M, K, N, 3, 1 + i % 3, bool(i % 2), 350 + 10 * i + t)
+        assert err < 2 * TOL_F32, ("gated", t, M, err)
+    N2 = 2 * N
+    W = synth.weights(t, 360 + t, N2, K)
+    gain = (synth.normal(361, 0, K) * 0.5 + 1.0).astype(np.float32)
+    for M in (2, 3, 5):
+        x = (synth.activations(362 + M, M, K) * 2.0).astype(np.float32)
+        res = synth.activations(363 + M, M, N2)
+        got = nn.quantized_dense(dev(gpu, x), dev(gpu, W), Quantization(ggml_type=t), None, BACKEND_ACT[0],
+                                 norm=nn.RMSNorm(dev(gpu, gain), 1e-6, 0.0), residual=dev(gpu, res)).cpu().numpy()
+        dense = oracle.c_qdense(t, oracle.c_rmsnorm(x, gain, 1e-6, 0.0), W)
+        err = float(np.max(np.abs(got.astype(np.float64) - (dense + res)))) / float(np.max(np.abs(dense)))
+        assert err < TOL_F32, ("block", t, M, err)
 
 
 def test_randomized_problems(gpu, oracle):
