@@ -504,7 +504,8 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8
         r.ga = r.gb = make_uint4(0, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < R; i++) {  // rows past the last one re-read it (their results are not stored)
-            const uint8_t *xrow = reinterpret_cast<const uint8_t *>(xv) + (int64_t)min(i, xrows - 1) * x_stride;
+            const uint8_t *xrow = reinterpret_cast<const uint8_t *>(xv);
+            if constexpr (R > 1) xrow += (int64_t)min(i, xrows - 1) * x_stride;
             r.b[i] = make_uint4(0, 0, 0, 0);
             if constexpr (XBF16) r.a[i] = KS<T>::x_fetch_bf16(reinterpret_cast<const uint16_t *>(xrow) + sl * kSliceValues, xl);
             else KS<T>::x_fetch(reinterpret_cast<const float *>(xrow) + sl * kSliceValues, xl, r.a[i], r.b[i]);
@@ -642,9 +643,11 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8
     // output row r of activation row q: the wavefronts' partial sums meet here
     const int rows_out = dual ? rows_wg >> 1 : rows_wg;
     for (int e = tid; e < rows_out * R; e += blockDim.x) {
-        const int q = e / rows_out, r = e - q * rows_out;
+        int q = 0, r = e;
+        if constexpr (R > 1) { q = e / rows_out; r = e - q * rows_out; }
         const int row = row0 + r;
-        if (row >= N || q >= xrows) continue;
+        if (row >= N) continue;
+        if constexpr (R > 1) { if (q >= xrows) continue; }
         const int64_t at = (int64_t)q * N + row;
         if constexpr (EXT) {
             float inv = 1.f;
