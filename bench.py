@@ -44,13 +44,13 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # pattern, not of a particular run, and are re-measured whenever a kernel changes.
 _KIB, _FETCH_SCALE, _WRITE_SCALE = 1024, 65536.0 / 32780.5, 1.0
 COUNTER_KIB = {  # workload -> (FETCH_SIZE, WRITE_SIZE) raw counter KiB per step
-    "c0": (8812.0, 16.0),
-    "c1": (16262.8, 56.0),
-    "c2": (19875.0 + 1833.6 + 911.6, 3584.0 + 512.0 + 924.0),
-    "c3": (74726.6, 32768.0),
-    "c4": (60540.6, 168.0),
-    "ffn": (32488.5, 56.0),
-    "layer": (7121.9 + 4762.2 + 32488.1 + 16449.1, 24.0 + 16.0 + 56.0 + 16.0),
+    "c0": (8811.9, 16.0),
+    "c1": (16262.6, 56.0),
+    "c2": (19875.1 + 1842.5 + 911.6, 3584.0 + 512.0 + 924.0),
+    "c3": (74726.7, 32768.0),
+    "c4": (60543.5, 168.0),
+    "ffn": (32484.0, 56.0),
+    "layer": (7126.2 + 4756.1 + 32483.6 + 16449.7, 24.0 + 16.0 + 56.0 + 16.0),
 }
 
 
