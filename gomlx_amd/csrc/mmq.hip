@@ -148,10 +148,13 @@ __device__ unsigned long long g_mmq_trace[4096 * 8];
 // activations + sub-block sums) to global memory once; the row-range workgroups of the main
 // kernel then only copy 132 KiB each instead of converting it again.  grid = (slices, column
 // tiles, 8): each workgroup converts four of the tile's 32 columns.
+// slice_sb <= 8 super-blocks per slice: a thread whose octet lies beyond them has nothing to do (the
+// image keeps its 8-super-block layout; the main kernel copies and uses the first slice_sb only).
 template <bool BF16X>
-__global__ __launch_bounds__(512) void mmq_xprep_kernel(const void *__restrict__ X, uint8_t *__restrict__ ximg, int M, int K) {
+__global__ __launch_bounds__(512) void mmq_xprep_kernel(const void *__restrict__ X, uint8_t *__restrict__ ximg, int M, int K, int slice_sb) {
     const int slice = blockIdx.x, mt = blockIdx.y;
-    stage_x<2, BF16X>(X, M, K, mt * kMT, slice * kSliceK, ximg + ((size_t)mt * gridDim.x + slice) * kLdsBytes, threadIdx.x,
+    if (((int)threadIdx.x & 255) >> 5 >= slice_sb) return;
+    stage_x<2, BF16X>(X, M, K, mt * kMT, slice * slice_sb * 256, ximg + ((size_t)mt * gridDim.x + slice) * kLdsBytes, threadIdx.x,
                2 * blockIdx.z);
 }
 
@@ -163,14 +166,14 @@ __global__ __launch_bounds__(512) void mmq_xprep_kernel(const void *__restrict__
 // read per lane feeds 16384 multiply-adds, and a lane's 16 results all belong to its own row.
 __global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__restrict__ ximg, const uint8_t *__restrict__ W,
                                                       float *__restrict__ partial, int M, int K, int N,
-                                                      int64_t row_bytes, int m0) {
+                                                      int64_t row_bytes, int m0, int slice_sb) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int kg = lane >> 5, col = lane & 31;
     const int rt = wave & 3, par = wave >> 2;  // par = 0 .. kParts-1
     const int slice = blockIdx.y;
-    const int k0 = slice * kSliceK;
-    const int nsb = min(kSliceSB, (K - k0) >> 8);
+    const int k0 = slice * slice_sb * 256;
+    const int nsb = min(slice_sb, (K - k0) >> 8);
     const int n = blockIdx.x * kRowsPerWG + rt * 32 + col;  // this lane's weight row
     const uint8_t *wrow = W + (int64_t)min(n, N - 1) * row_bytes + (int64_t)(k0 >> 8) * 144;
 
@@ -179,9 +182,13 @@ __global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__
     // the slice's activation image goes straight from global memory into LDS (no registers)
     {
         const uint8_t *img = ximg + ((size_t)(m0 / kMT) * gridDim.y + slice) * kLdsBytes;
-        for (int i = wave; i < kLdsBytes / 1024; i += 4 * kParts)
+        // fragments of the slice's first slice_sb super-blocks (16 KiB each), then the 4 KiB of sub-block sums
+        const int frag_kib = slice_sb * 16;
+        for (int i0 = wave; i0 < frag_kib + kXSBytes / 1024; i0 += 4 * kParts) {
+            const int i = i0 < frag_kib ? i0 : kXFBytes / 1024 + (i0 - frag_kib);
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(img + i * 1024 + lane * 16),
                                              (__attribute__((address_space(3))) void *)(lds + i * 1024), 16, 0, 0);
+        }
     }
     RawSB cur;
     load_sb(cur, wrow + (int64_t)min(par, nsb - 1) * 144, kg);
@@ -791,8 +798,14 @@ int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, co
                                    kLdsBytes) == hipSuccess;
     }();
     if (!lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", kLdsBytes);
-    const int nslices = (int)((K + kSliceK - 1) / kSliceK);
+    // K-slices of 8 super-blocks, or of 4 / 2 when the problem would otherwise leave more than a quarter of the
+    // CUs without a workgroup (4096 x 4096: 2 slices x 32 row ranges = 64 workgroups with 8, 256 with 2: 18.8 -> 16.6 us;
+    // splitting 224 workgroups into 448 costs more than it brings: 20.8 -> 24.9 us on 4096 -> 14336)
     const int mtiles = (int)((M + kMT - 1) / kMT);
+    const int64_t rowwgs = (N + kRowsPerWG - 1) / kRowsPerWG, sbs = K / 256;
+    int slice_sb = kSliceSB;
+    while (slice_sb > 2 && rowwgs * ((sbs + slice_sb - 1) / slice_sb) < (int64_t)device_cu_count() * 3 / 4) slice_sb >>= 1;
+    const int nslices = (int)((sbs + slice_sb - 1) / slice_sb);
     // workspace: [activation images: mtiles x nslices x kLdsBytes][partial sums: nslices x M x N fp32, twice for a gated pair]
     const size_t img_bytes = (size_t)mtiles * nslices * kLdsBytes;
     const size_t part_bytes = (size_t)nslices * M * N * sizeof(float);
@@ -801,15 +814,17 @@ int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, co
     uint8_t *ximg = reinterpret_cast<uint8_t *>(ws);
     float *partial = reinterpret_cast<float *>(ximg + img_bytes);
     const int64_t row_bytes = (K / 256) * 144;
-    if (int rc = x_is_bf16 ? launch(mmq_xprep_kernel<true>, dim3((unsigned)nslices, (unsigned)mtiles, 8), dim3(512), 0, s, x, ximg, (int)M, (int)K)
-                           : launch(mmq_xprep_kernel<false>, dim3((unsigned)nslices, (unsigned)mtiles, 8), dim3(512), 0, s, x, ximg, (int)M, (int)K))
+    if (int rc = x_is_bf16 ? launch(mmq_xprep_kernel<true>, dim3((unsigned)nslices, (unsigned)mtiles, 8), dim3(512), 0, s, x, ximg, (int)M, (int)K,
+                                    slice_sb)
+                           : launch(mmq_xprep_kernel<false>, dim3((unsigned)nslices, (unsigned)mtiles, 8), dim3(512), 0, s, x, ximg, (int)M, (int)K,
+                                    slice_sb))
         return rc;
     const dim3 grid((unsigned)((N + kRowsPerWG - 1) / kRowsPerWG), (unsigned)nslices);
     float *partial2 = W2 ? partial + (size_t)nslices * M * N : nullptr;
     for (int which = 0; which < (W2 ? 2 : 1); which++)
         for (int64_t m0 = 0; m0 < M; m0 += kMT) {
             if (int rc = launch(mmq_q4k_kernel, grid, dim3(256 * kParts), (size_t)kLdsBytes, s, (const uint8_t *)ximg, which ? W2 : W,
-                                which ? partial2 : partial, (int)M, (int)K, (int)N, row_bytes, (int)m0))
+                                which ? partial2 : partial, (int)M, (int)K, (int)N, row_bytes, (int)m0, slice_sb))
                 return rc;
         }
     return launch_mmq_reduce(partial, partial2, nslices, M, N, bias, act, y, ex, s);
