@@ -908,3 +908,63 @@ def test_operator_rejects_bad_arguments(gpu):
     y0 = nn.quantized_dense(x + 1.0, W, q)
     y1 = nn.quantized_dense(x + 1.0, W, q, None, Activation.SIGMOID)
     assert gpu.equal(y0, y1)
+
+
+@pytest.mark.parametrize("rows", [1, 3, 24, 300])
+def test_decoder_layer_calls_replay_as_a_graph(gpu, rows):
+    """The calls of a decoder layer (q/k/v behind a norm, o + residual, norm + gate/up product, down +
+    residual in place) recorded once and replayed four times, with eager work between the replays:
+    every replay must reproduce the eager results exactly.  Batch sizes of all three kernel
+    families; one eager pass first creates the workspaces the larger ones need."""
+    import ctypes
+    from gomlx_amd import _lib
+    torch = gpu
+    L = _lib.lib()
+    t, H, KV, F = Q4_K, 512, 256, 1024
+    mk = lambda seed, n, k: dev(torch, synth.weights(t, seed, n, k))
+    Wq, Wk, Wv, Wo, Wg, Wu, Wd = mk(1, H, H), mk(2, KV, H), mk(3, KV, H), mk(4, H, H), mk(5, F, H), mk(6, F, H), mk(7, H, F)
+    x0 = dev(torch, synth.activations(8, rows, H))
+    attn = dev(torch, synth.activations(9, rows, H))
+    # (a small gain keeps the gated product of these synthetic weights inside the fp16 range that the
+    # activations of the MFMA paths are rounded to)
+    g1 = dev(torch, ((synth.normal(10, 0, H) * 0.5 + 1.0) * 0.02).astype(np.float32))
+    q, k, v = (torch.zeros(rows, n, device="cuda") for n in (H, KV, KV))
+    h, ff, x = torch.zeros(rows, H, device="cuda"), torch.zeros(rows, F, device="cuda"), torch.zeros(rows, H, device="cuda")
+    norm = _lib.RmsNormDesc(g1.data_ptr(), 1e-5, 0.0)
+    stream = torch.cuda.Stream()
+    sp = stream.cuda_stream
+
+    def layer():
+        d = (_lib.DenseDesc * 3)()
+        for dd, (W, y, n) in zip(d, ((Wq, q, H), (Wk, k, KV), (Wv, v, KV))):
+            dd.type, dd.act, dd.dX, dd.M, dd.K, dd.dW, dd.N, dd.dBias, dd.dY = t, 0, x.data_ptr(), rows, H, W.data_ptr(), n, None, y.data_ptr()
+        _lib.check(L.gq_qdense_norm_f32_batch(3, d, ctypes.byref(norm), sp))
+        _lib.check(L.gq_qdense_block_f32(t, attn.data_ptr(), rows, H, None, Wo.data_ptr(), H, None, 0, x.data_ptr(), h.data_ptr(), sp))
+        _lib.check(L.gq_qdense_gated_f32(t, h.data_ptr(), rows, H, ctypes.byref(norm), Wg.data_ptr(), None, Wu.data_ptr(), None, F, 3,
+                                         ff.data_ptr(), sp))
+        _lib.check(L.gq_qdense_block_f32(t, ff.data_ptr(), rows, F, None, Wd.data_ptr(), H, None, 0, h.data_ptr(), h.data_ptr(), sp))
+
+    def reset():
+        x.copy_(x0)
+        for b in (q, k, v, h, ff):
+            b.fill_(float("nan"))
+        torch.cuda.synchronize()
+
+    reset()
+    layer()
+    _lib.check(L.gq_sync(sp))
+    eager = [b.clone() for b in (q, k, v, h, ff)]
+    assert all(bool(torch.isfinite(b).all()) for b in eager)
+    _lib.check(L.gq_graph_begin(sp))
+    layer()
+    g = ctypes.c_void_p()
+    _lib.check(L.gq_graph_end(sp, ctypes.byref(g)))
+    for rep in range(4):
+        reset()
+        _lib.check(L.gq_graph_launch(g, sp))
+        _lib.check(L.gq_sync(sp))
+        for got, want in zip((q, k, v, h, ff), eager):
+            assert torch.equal(got, want), rep
+        (x0 * 2.0).sum().item()  # unrelated eager work and a synchronisation between replays
+    _lib.check(L.gq_graph_destroy(g))
+
