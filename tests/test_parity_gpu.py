@@ -449,6 +449,20 @@ def test_small_batches_with_neighbours_on_large_matrices(gpu, oracle, t, N):
         assert err < TOL_F32, ("block", t, M, err)
 
 
+@pytest.mark.parametrize("t", [Q4_0, Q8_0, IQ4_NL])
+def test_small_batches_over_a_single_block_are_exact_passes(gpu, oracle, t):
+    """K of one or a few blocks leaves no averaging for 16-bit operands to lean on: batches of 5 .. 16 rows
+    on such shapes run as fp32 passes and stay well inside the bound (a seeded sweep once found 1.25e-3
+    on a 7 x 32 x 8 problem through the fp16-operand GEMM)."""
+    for M, K, N in ((7, 32, 8), (16, 96, 5), (5, 160, 33), (12, 544, 16)):
+        W = synth.weights(t, 380 + M, N, K)
+        x = synth.activations(381 + M, M, K)
+        bias = synth.normal(382 + M, 0, N).astype(np.float32) * 0.1
+        for seed in range(3):
+            x = synth.activations(383 + 7 * seed + M, M, K)
+            assert rel_err(run_dense(gpu, t, x, W, bias, 0), oracle.c_qdense(t, x, W, bias, 0)) < 1e-4, (t, M, K, N)
+
+
 def test_randomized_problems(gpu, oracle):
     """150 seeded random problems over all formats, both activation types, every activation, with
     and without bias: batch sizes, K and N drawn from lists that include every tile and slice
