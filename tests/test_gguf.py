@@ -134,3 +134,39 @@ def test_malformed_files(tmp_path):
         load(head + b"\0" * 4096)
     with pytest.raises(gguf.GGUFError):
         gguf.write_gguf(str(tmp_path / "w.gguf"), {}, [("w", ggml.Q8_0, (64, 3), np.zeros(10, np.uint8))])
+
+
+def test_round_trip_property(tmp_path):
+    """Random files: any mix of tensor types, ranks and alignments written by write_gguf reads back byte for byte."""
+    from hypothesis import given, settings, strategies as st, HealthCheck
+
+    types = [ggml.Q4_0, ggml.Q8_0, ggml.Q4_K, ggml.Q6_K, ggml.IQ4_NL, 0, 1, 24, 26, 30]
+    tensor = st.tuples(st.sampled_from(types), st.integers(1, 3), st.lists(st.integers(1, 5), min_size=0, max_size=2), st.integers(0, 2 ** 31))
+    counter = [0]
+
+    @settings(max_examples=40, deadline=None, suppress_health_check=[HealthCheck.function_scoped_fixture])
+    @given(st.lists(tensor, min_size=0, max_size=6), st.sampled_from([32, 64, 4096]),
+           st.dictionaries(st.text(min_size=1, max_size=12), st.one_of(st.integers(-2 ** 62, 2 ** 62), st.text(max_size=20), st.booleans()), max_size=5))
+    def run(tensors, alignment, meta):
+        meta = {k: v for k, v in meta.items() if k != "general.alignment"}
+        specs, want = [], {}
+        for i, (t, blocks, outer, seed) in enumerate(tensors):
+            _, vpb, bpb = gguf.GGML_TYPES[t]
+            ne = (blocks * vpb, *outer)
+            n = gguf.tensor_nbytes(t, ne)
+            data = np.random.default_rng(seed).integers(0, 256, size=n, dtype=np.uint8)
+            specs.append((f"t{i}", t, ne, data))
+            want[f"t{i}"] = (ne, data)
+        counter[0] += 1
+        path = str(tmp_path / f"p{counter[0]}.gguf")
+        gguf.write_gguf(path, meta, specs, alignment=alignment)
+        with gguf.GGUFFile(path) as g:
+            assert g.alignment == alignment and list(g.tensors) == list(want)
+            for name, (ne, data) in want.items():
+                assert g.tensors[name].ne == tuple(ne)
+                assert np.array_equal(g.raw(name), data)
+                assert (g.data_start + g.tensors[name].offset) % alignment == 0
+            for k, v in meta.items():
+                assert g.metadata[k] == v
+
+    run()
