@@ -79,6 +79,31 @@ __device__ __forceinline__ float dpp_quad_sum(float v) {
     return v;
 }
 
+// The activations of one batch column within one K-slice are scaled by a power of two before they
+// are rounded to fp16, so that their largest magnitude lands in [512, 1024): whatever the range
+// of the inputs, nothing overflows (a sub-block sum of 32 values stays below 32768) and nothing
+// falls into fp16's subnormals that matters next to the largest value.  The slice's partial sums
+// are multiplied by the inverse (exact) in the reduction.  Zero, subnormal-tiny and non-finite
+// maxima leave the slice unscaled.
+__device__ __forceinline__ void pow2_scale(float amax, float &s, float &inv) {
+    const int e = (int)((__builtin_bit_cast(uint32_t, amax) >> 23) & 0xFFu);
+    if (e >= 10 && e <= 254) {
+        s = __builtin_bit_cast(float, (uint32_t)(263 - e) << 23);    // 2^(136 - e): amax * s in [2^9, 2^10)
+        inv = __builtin_bit_cast(float, (uint32_t)(e - 9) << 23);    // 2^(e - 136)
+    } else {
+        s = 1.f;
+        inv = 1.f;
+    }
+}
+__device__ __forceinline__ float amax8(const float4 &a, const float4 &b) {
+    return fmaxf(fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))),
+                 fmaxf(fmaxf(fabsf(b.x), fabsf(b.y)), fmaxf(fabsf(b.z), fabsf(b.w))));
+}
+__device__ __forceinline__ float wave_max(float v) {
+    for (int m = 1; m < 64; m <<= 1) v = fmaxf(v, __shfl_xor(v, m));
+    return v;
+}
+
 // ---- stage the K-slice of x into LDS in MFMA fragment order ---------------------------------
 //
 // One item = 8 consecutive activations of one batch column ("octet").  Inside a super-block the
@@ -90,9 +115,11 @@ __device__ __forceinline__ float dpp_quad_sum(float v) {
 // i.e. different slots with the same m, and the xor spreads their 16-byte stores (and the 32
 // columns a half-wave later reads from one slot) over all LDS banks.
 // The eight sub-block sums of (sbl, m) are stored in the order (0, 2, 1, 3, 4, 6, 5, 7) too.
+// `active`: the thread's octet belongs to the slice (slices may hold fewer than 8 super-blocks).
+// red: [2][ROUNDS][4] floats of shared memory; inv_scale[m] receives the slice's inverse scale of column m0 + m.
 template <int ROUNDS, bool BF16X>
 __device__ __forceinline__ void stage_x(const void *__restrict__ X, int M, int K, int m0, int k0, uint8_t *__restrict__ lds, int tid,
-                                        int round0) {
+                                        int round0, bool active, float *red, float *__restrict__ inv_scale) {
     const int oct = tid & 255;  // fixed per thread; its items are columns (tid >> 8) + 2 r
     const int k = k0 + 8 * oct;
     const int sbl = oct >> 5, v8 = oct & 31;
@@ -103,20 +130,35 @@ __device__ __forceinline__ void stage_x(const void *__restrict__ X, int M, int K
     const int jpos = (j & 4) | ((j & 1) << 1) | ((j >> 1) & 1);
     uint8_t *xf_base = lds + slot * (kMT * 16);
     uint8_t *xs_base = lds + kXFBytes + sbl * (kMT * 16) + jpos * 2;
-    const bool k_ok = k < K;
-    const int ksrc = min(k, K - 8);
+    const bool k_ok = active && k < K;
+    const int ksrc = max(min(k, K - 8), 0);
     float4 lo[ROUNDS], hi[ROUNDS];
 #pragma unroll
     for (int r = 0; r < ROUNDS; r++) {
         const int m = (tid >> 8) + 2 * (round0 + r);
         load_x8<BF16X>(X, (int64_t)min(m0 + m, M - 1) * K + ksrc, lo[r], hi[r]);
     }
+    // largest magnitude of each column's slice: its 256 octets sit in the four wavefronts of one half of the workgroup
+    const int half = tid >> 8, wih = (tid >> 6) & 3;
+#pragma unroll
+    for (int r = 0; r < ROUNDS; r++) {
+        const bool ok = k_ok && (m0 + half + 2 * (round0 + r) < M);
+        const float am = wave_max(ok ? amax8(lo[r], hi[r]) : 0.f);
+        if ((tid & 63) == 0) red[(half * ROUNDS + r) * 4 + wih] = am;
+    }
+    __syncthreads();
 #pragma unroll
     for (int r = 0; r < ROUNDS; r++) {
         const int m = (tid >> 8) + 2 * (round0 + r);
         const bool ok = k_ok && (m0 + m < M);
+        const float *rr = red + (half * ROUNDS + r) * 4;
+        float sc, inv;
+        pow2_scale(fmaxf(fmaxf(rr[0], rr[1]), fmaxf(rr[2], rr[3])), sc, inv);
+        if (oct == 0 && m0 + m < M) inv_scale[m0 + m] = inv;
+        if (!active) continue;
         const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
-        const float4 a = ok ? lo[r] : z, b = ok ? hi[r] : z;
+        float4 a = ok ? lo[r] : z, b = ok ? hi[r] : z;
+        a.x *= sc; a.y *= sc; a.z *= sc; a.w *= sc; b.x *= sc; b.y *= sc; b.z *= sc; b.w *= sc;
         uint4 o;  // bytes (0,2,1,3,4,6,5,7)
         o.x = pack_h2(a.x, a.z);
         o.y = pack_h2(a.y, a.w);
@@ -150,12 +192,15 @@ __device__ unsigned long long g_mmq_trace[4096 * 8];
 // tiles, 8): each workgroup converts four of the tile's 32 columns.
 // slice_sb <= 8 super-blocks per slice: a thread whose octet lies beyond them has nothing to do (the
 // image keeps its 8-super-block layout; the main kernel copies and uses the first slice_sb only).
+// xscale[slice][M]: the inverse of the power of two that (slice, column) was scaled by.
 template <bool BF16X>
-__global__ __launch_bounds__(512) void mmq_xprep_kernel(const void *__restrict__ X, uint8_t *__restrict__ ximg, int M, int K, int slice_sb) {
+__global__ __launch_bounds__(512) void mmq_xprep_kernel(const void *__restrict__ X, uint8_t *__restrict__ ximg, float *__restrict__ xscale, int M,
+                                                        int K, int slice_sb) {
+    __shared__ float red[2 * 2 * 4];
     const int slice = blockIdx.x, mt = blockIdx.y;
-    if (((int)threadIdx.x & 255) >> 5 >= slice_sb) return;
+    const bool active = (((int)threadIdx.x & 255) >> 5) < slice_sb;
     stage_x<2, BF16X>(X, M, K, mt * kMT, slice * slice_sb * 256, ximg + ((size_t)mt * gridDim.x + slice) * kLdsBytes, threadIdx.x,
-               2 * blockIdx.z);
+                      2 * blockIdx.z, active, red, xscale + (size_t)slice * M);
 }
 
 // partial[slice][m][n] = sum over the slice's k of x[m][k] * w[n][k]
@@ -296,16 +341,19 @@ __global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__
 // y[m][n] = act(sum_s partial[s][m][n] + bias[n]); N % 4 == 0 is guaranteed by the caller.  With a second
 // set of partial sums (the other matrix of a gated pair) the result is multiplied by
 // sum_s partial2[s][m][n] + bias2[n]; a residual (which may be Y itself) is added last.
+// xscale[slice][M]: factor of each slice's partial sums of row m (the activations of a slice were scaled by its inverse).
 __global__ __launch_bounds__(256) void mmq_reduce_kernel(const float *__restrict__ partial, const float *__restrict__ partial2, int nslices,
                                                          int64_t MN, int N, const float *__restrict__ bias, const float *__restrict__ bias2,
-                                                         int act, const float *residual, float *Y) {
+                                                         int act, const float *residual, float *Y, const float *__restrict__ xscale) {
     const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= MN) return;
+    const int M = (int)(MN / N), m = (int)(i / N);
     auto total = [&](const float *p, const float *b) {
         float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
         for (int k = 0; k < nslices; k++) {
             const float4 v = *reinterpret_cast<const float4 *>(p + (int64_t)k * MN + i);
-            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+            const float f = xscale[(int64_t)k * M + m];
+            s.x = fmaf(v.x, f, s.x); s.y = fmaf(v.y, f, s.y); s.z = fmaf(v.z, f, s.z); s.w = fmaf(v.w, f, s.w);
         }
         if (b) {
             const float4 v = *reinterpret_cast<const float4 *>(b + (int)(i % N));
@@ -326,12 +374,13 @@ __global__ __launch_bounds__(256) void mmq_reduce_kernel(const float *__restrict
     *reinterpret_cast<float4 *>(Y + i) = v;
 }
 
-int launch_mmq_reduce(const float *partial, const float *partial2, int nslices, int64_t M, int64_t N, const float *bias, int act, float *y,
-                      const MmqExtra *ex, hipStream_t s) {
+int launch_mmq_reduce(const float *partial, const float *partial2, const float *xscale, int nslices, int64_t M, int64_t N, const float *bias,
+                      int act, float *y, const MmqExtra *ex, hipStream_t s) {
     const int64_t MN = M * N;
     return launch(mmq_reduce_kernel, dim3((unsigned)((MN / 4 + 255) / 256)), dim3(256), 0, s, partial, partial2, nslices, MN, (int)N, bias,
-                  ex ? ex->bias2 : nullptr, act, ex ? ex->residual : nullptr, y);
+                  ex ? ex->bias2 : nullptr, act, ex ? ex->residual : nullptr, y, xscale);
 }
+size_t mmq_scale_bytes(int nslices, int64_t M) { return ((size_t)nslices * M * sizeof(float) + 255) & ~(size_t)255; }
 
 
 // ---- small batches of the 32-value-block formats (Q8_0, Q4_0, IQ4_NL) --------------------------------------
@@ -427,21 +476,48 @@ template <int T> struct B32Geom {
 };
 
 // Image of x for the main kernel: [column tile][slice][octet of the slice][32 columns][8 fp16 in the
-// order (0,2,1,3,4,6,5,7)]; columns beyond M and values beyond K are zero.
+// order (0,2,1,3,4,6,5,7)]; columns beyond M and values beyond K are zero.  One workgroup converts 8
+// columns of one slice (S / 256 octets per thread, consecutive threads on consecutive octets of a
+// column) and scales each column's slice by a power of two (pow2_scale); xscale[slice][M] receives the
+// inverse factors.  grid = column tiles x slices x 4.
 template <bool BF16X>
-__global__ __launch_bounds__(256) void mmq_b32_xprep_kernel(const void *__restrict__ X, uint8_t *__restrict__ ximg, int M, int K, int S,
-                                                            int nslices) {
-    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;  // (column tile, slice, octet, column)
-    const int m = (int)(g & 31);
-    const int64_t o = g >> 5;  // octet index over (column tile, slice, octet of slice)
-    const int opers = S / 8;
-    const int64_t ts = o / opers;
-    const int oct = (int)(o % opers), slice = (int)(ts % nslices), mt = (int)(ts / nslices);
-    if (mt * kMT >= M) return;
-    const int k = slice * S + oct * 8, row = mt * kMT + m;
-    float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
-    if (row < M && k < K) load_x8<BF16X>(X, (int64_t)row * K + k, a, b);  // K % 32 == 0: an octet is inside or outside as a whole
-    reinterpret_cast<uint4 *>(ximg)[g] = make_uint4(pack_h2(a.x, a.z), pack_h2(a.y, a.w), pack_h2(b.x, b.z), pack_h2(b.y, b.w));
+__global__ __launch_bounds__(256) void mmq_b32_xprep_kernel(const void *__restrict__ X, uint8_t *__restrict__ ximg, float *__restrict__ xscale,
+                                                            int M, int K, int S, int nslices) {
+    __shared__ uint32_t red[8];
+    const int tid = threadIdx.x;
+    const int rg = (int)blockIdx.x & 3, ts = (int)blockIdx.x >> 2;
+    const int slice = ts % nslices, mt = ts / nslices;
+    const int opers = S / 8, its = S / 256;  // octets per column and slice; items per thread
+    if (tid < 8) red[tid] = 0u;
+    __syncthreads();
+    float4 a[4], b[4];
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        a[it] = make_float4(0.f, 0.f, 0.f, 0.f);
+        b[it] = a[it];
+        if (it < its) {
+            const int j = it * 256 + tid, c = j / opers, oct = j - c * opers;
+            const int k = slice * S + oct * 8, row = mt * kMT + rg * 8 + c;
+            if (row < M && k < K) load_x8<BF16X>(X, (int64_t)row * K + k, a[it], b[it]);  // K % 32 == 0: an octet is inside or outside as a whole
+            const float am = wave_max(amax8(a[it], b[it]));  // a wavefront's 64 octets belong to one column
+            if ((tid & 63) == 0) atomicMax(&red[c], __builtin_bit_cast(uint32_t, am));  // (non-negative floats order like their bits)
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        if (it < its) {
+            const int j = it * 256 + tid, c = j / opers, oct = j - c * opers;
+            const int m = rg * 8 + c, row = mt * kMT + m;
+            float sc, inv;
+            pow2_scale(__builtin_bit_cast(float, red[c]), sc, inv);
+            if (oct == 0 && row < M) xscale[(size_t)slice * M + row] = inv;
+            const float4 p = a[it], q = b[it];
+            const size_t g = (((size_t)mt * nslices + slice) * opers + oct) * 32 + m;
+            reinterpret_cast<uint4 *>(ximg)[g] = make_uint4(pack_h2(p.x * sc, p.z * sc), pack_h2(p.y * sc, p.w * sc), pack_h2(q.x * sc, q.z * sc),
+                                                            pack_h2(q.y * sc, q.w * sc));
+        }
+    }
 }
 
 // partial[slice][m][n] = sum over the slice's k of x[m][k] * w[n][k];  grid (row ranges, slices, column tiles)
@@ -571,19 +647,19 @@ int launch_mmq_b32(const void *x, bool x_is_bf16, int64_t M, int64_t K, const ui
                                    1024 * 64 + 2 * RT * B32Geom<T>::kWaveLds) == hipSuccess;
     }();
     if (!lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", 1024 * 64 + 2 * RT * B32Geom<T>::kWaveLds);
-    // workspace: [activation images: mtiles x nslices x S x 64 bytes][partial sums: nslices x M x N fp32, twice for a gated pair]
+    // workspace: [activation images: mtiles x nslices x S x 64 bytes][slice scales: nslices x M][partial sums: nslices x M x N fp32,
+    // twice for a gated pair]
     const size_t img_bytes = (size_t)mtiles * nslices * S * 64;
     const size_t part_bytes = (size_t)nslices * M * N * sizeof(float);
     void *ws = nullptr;
-    if (int rc = stream_workspace(s, img_bytes + part_bytes * (W2 ? 2 : 1), &ws)) return rc;
+    if (int rc = stream_workspace(s, img_bytes + mmq_scale_bytes(nslices, M) + part_bytes * (W2 ? 2 : 1), &ws)) return rc;
     uint8_t *ximg = reinterpret_cast<uint8_t *>(ws);
-    float *partial = reinterpret_cast<float *>(ximg + img_bytes);
+    float *xscale = reinterpret_cast<float *>(ximg + img_bytes);
+    float *partial = reinterpret_cast<float *>(ximg + img_bytes + mmq_scale_bytes(nslices, M));
     const int64_t row_bytes = (K / 32) * B32<T>::kBlockBytes;
-    const int64_t items = (int64_t)mtiles * nslices * (S / 8) * 32;
-    if (int rc = x_is_bf16 ? launch(mmq_b32_xprep_kernel<true>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, x, ximg, (int)M,
-                                    (int)K, S, nslices)
-                           : launch(mmq_b32_xprep_kernel<false>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, x, ximg, (int)M,
-                                    (int)K, S, nslices))
+    const dim3 xgrid((unsigned)(mtiles * nslices * 4));
+    if (int rc = x_is_bf16 ? launch(mmq_b32_xprep_kernel<true>, xgrid, dim3(256), 0, s, x, ximg, xscale, (int)M, (int)K, S, nslices)
+                           : launch(mmq_b32_xprep_kernel<false>, xgrid, dim3(256), 0, s, x, ximg, xscale, (int)M, (int)K, S, nslices))
         return rc;
     const dim3 grid((unsigned)rowwgs, (unsigned)nslices, (unsigned)mtiles);
     if (int rc = launch(mmq_b32_kernel<T, RT>, grid, dim3(RT * 128), lds_bytes, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N, row_bytes, S))
@@ -593,7 +669,7 @@ int launch_mmq_b32(const void *x, bool x_is_bf16, int64_t M, int64_t K, const ui
         if (int rc = launch(mmq_b32_kernel<T, RT>, grid, dim3(RT * 128), lds_bytes, s, (const uint8_t *)ximg, W2, partial2, (int)M, (int)K, (int)N,
                             row_bytes, S))
             return rc;
-    return launch_mmq_reduce(partial, partial2, nslices, M, N, bias, act, y, ex, s);
+    return launch_mmq_reduce(partial, partial2, xscale, nslices, M, N, bias, act, y, ex, s);
 }
 
 
@@ -751,15 +827,14 @@ int launch_mmq_q6k(const MmqExtra *ex, const void *x, bool x_is_bf16, int64_t M,
     const size_t img_bytes = (size_t)mtiles * nslices * kQ6Slice * 64;
     const size_t part_bytes = (size_t)nslices * M * N * sizeof(float);
     void *ws = nullptr;
-    if (int rc = stream_workspace(s, img_bytes + part_bytes * (W2 ? 2 : 1), &ws)) return rc;
+    if (int rc = stream_workspace(s, img_bytes + mmq_scale_bytes(nslices, M) + part_bytes * (W2 ? 2 : 1), &ws)) return rc;
     uint8_t *ximg = reinterpret_cast<uint8_t *>(ws);
-    float *partial = reinterpret_cast<float *>(ximg + img_bytes);
+    float *xscale = reinterpret_cast<float *>(ximg + img_bytes);
+    float *partial = reinterpret_cast<float *>(ximg + img_bytes + mmq_scale_bytes(nslices, M));
     const int64_t row_bytes = (K / 256) * 210;
-    const int64_t items = (int64_t)mtiles * nslices * (kQ6Slice / 8) * 32;
-    if (int rc = x_is_bf16 ? launch(mmq_b32_xprep_kernel<true>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, x, ximg, (int)M,
-                                    (int)K, kQ6Slice, nslices)
-                           : launch(mmq_b32_xprep_kernel<false>, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, s, x, ximg, (int)M,
-                                    (int)K, kQ6Slice, nslices))
+    const dim3 xgrid((unsigned)(mtiles * nslices * 4));
+    if (int rc = x_is_bf16 ? launch(mmq_b32_xprep_kernel<true>, xgrid, dim3(256), 0, s, x, ximg, xscale, (int)M, (int)K, kQ6Slice, nslices)
+                           : launch(mmq_b32_xprep_kernel<false>, xgrid, dim3(256), 0, s, x, ximg, xscale, (int)M, (int)K, kQ6Slice, nslices))
         return rc;
     const dim3 grid((unsigned)((N + 32 * kQ6RT - 1) / (32 * kQ6RT)), (unsigned)nslices, (unsigned)mtiles);
     if (int rc = launch(mmq_q6k_kernel, grid, dim3(kQ6RT * 128), (size_t)kLds, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N,
@@ -770,7 +845,7 @@ int launch_mmq_q6k(const MmqExtra *ex, const void *x, bool x_is_bf16, int64_t M,
         if (int rc = launch(mmq_q6k_kernel, grid, dim3(kQ6RT * 128), (size_t)kLds, s, (const uint8_t *)ximg, W2, partial2, (int)M, (int)K, (int)N,
                             row_bytes))
             return rc;
-    return launch_mmq_reduce(partial, partial2, nslices, M, N, bias, act, y, ex, s);
+    return launch_mmq_reduce(partial, partial2, xscale, nslices, M, N, bias, act, y, ex, s);
 }
 
 }  // namespace
@@ -806,18 +881,20 @@ int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, co
     int slice_sb = kSliceSB;
     while (slice_sb > 2 && rowwgs * ((sbs + slice_sb - 1) / slice_sb) < (int64_t)device_cu_count() * 3 / 4) slice_sb >>= 1;
     const int nslices = (int)((sbs + slice_sb - 1) / slice_sb);
-    // workspace: [activation images: mtiles x nslices x kLdsBytes][partial sums: nslices x M x N fp32, twice for a gated pair]
+    // workspace: [activation images: mtiles x nslices x kLdsBytes][slice scales: nslices x M][partial sums: nslices x M x N fp32,
+    // twice for a gated pair]
     const size_t img_bytes = (size_t)mtiles * nslices * kLdsBytes;
     const size_t part_bytes = (size_t)nslices * M * N * sizeof(float);
     void *ws = nullptr;
-    if (int rc = stream_workspace(s, img_bytes + part_bytes * (W2 ? 2 : 1), &ws)) return rc;
+    if (int rc = stream_workspace(s, img_bytes + mmq_scale_bytes(nslices, M) + part_bytes * (W2 ? 2 : 1), &ws)) return rc;
     uint8_t *ximg = reinterpret_cast<uint8_t *>(ws);
-    float *partial = reinterpret_cast<float *>(ximg + img_bytes);
+    float *xscale = reinterpret_cast<float *>(ximg + img_bytes);
+    float *partial = reinterpret_cast<float *>(ximg + img_bytes + mmq_scale_bytes(nslices, M));
     const int64_t row_bytes = (K / 256) * 144;
-    if (int rc = x_is_bf16 ? launch(mmq_xprep_kernel<true>, dim3((unsigned)nslices, (unsigned)mtiles, 8), dim3(512), 0, s, x, ximg, (int)M, (int)K,
-                                    slice_sb)
-                           : launch(mmq_xprep_kernel<false>, dim3((unsigned)nslices, (unsigned)mtiles, 8), dim3(512), 0, s, x, ximg, (int)M, (int)K,
-                                    slice_sb))
+    if (int rc = x_is_bf16 ? launch(mmq_xprep_kernel<true>, dim3((unsigned)nslices, (unsigned)mtiles, 8), dim3(512), 0, s, x, ximg, xscale, (int)M,
+                                    (int)K, slice_sb)
+                           : launch(mmq_xprep_kernel<false>, dim3((unsigned)nslices, (unsigned)mtiles, 8), dim3(512), 0, s, x, ximg, xscale, (int)M,
+                                    (int)K, slice_sb))
         return rc;
     const dim3 grid((unsigned)((N + kRowsPerWG - 1) / kRowsPerWG), (unsigned)nslices);
     float *partial2 = W2 ? partial + (size_t)nslices * M * N : nullptr;
@@ -827,7 +904,7 @@ int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, co
                                 which ? partial2 : partial, (int)M, (int)K, (int)N, row_bytes, (int)m0, slice_sb))
                 return rc;
         }
-    return launch_mmq_reduce(partial, partial2, nslices, M, N, bias, act, y, ex, s);
+    return launch_mmq_reduce(partial, partial2, xscale, nslices, M, N, bias, act, y, ex, s);
 }
 
 }  // namespace gq
