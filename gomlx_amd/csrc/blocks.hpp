@@ -178,6 +178,40 @@ __device__ __forceinline__ void dequant16<kQ6_K>(const uint8_t *__restrict__ row
 
 // Epilogue of the fused op: activation.Apply formulas
 // (ml/layers/activation/activation.go:161,195,222-243,274-286); Gelu is the exact erf form.
+// Activations that are rounded to fp16 operands are first scaled by a power of two per batch row
+// (split-K kernels: per row and K-slice), so that their largest magnitude lands in [512, 1024):
+// whatever the range of the inputs, nothing overflows (a sum of 32 values stays below 32768) and
+// nothing that matters next to the largest value falls into fp16's subnormals.  The results are
+// multiplied by the inverse (exact).  Zero, tiny-subnormal and non-finite maxima mean no scaling.
+__device__ __forceinline__ void pow2_scale(float amax, float &s, float &inv) {
+    const int e = (int)((__builtin_bit_cast(uint32_t, amax) >> 23) & 0xFFu);
+    if (e >= 10 && e <= 254) {
+        s = __builtin_bit_cast(float, (uint32_t)(263 - e) << 23);    // 2^(136 - e): amax * s in [2^9, 2^10)
+        inv = __builtin_bit_cast(float, (uint32_t)(e - 9) << 23);    // 2^(e - 136)
+    } else {
+        s = 1.f;
+        inv = 1.f;
+    }
+}
+__device__ __forceinline__ float amax8(const float4 &a, const float4 &b) {
+    return fmaxf(fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))),
+                 fmaxf(fmaxf(fabsf(b.x), fabsf(b.y)), fmaxf(fabsf(b.z), fabsf(b.w))));
+}
+// maximum over a full wavefront (all 64 lanes active): within rows of 16 lanes by data-parallel
+// permutes, then over the four rows through scalar reads
+__device__ __forceinline__ float wave_max(float v) {
+#define GQ_DPP_MAX(ctrl) v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xF, 0xF, true)))
+    GQ_DPP_MAX(0xB1);   // quad_perm [1,0,3,2]
+    GQ_DPP_MAX(0x4E);   // quad_perm [2,3,0,1]
+    GQ_DPP_MAX(0x141);  // row_half_mirror
+    GQ_DPP_MAX(0x140);  // row_mirror
+#undef GQ_DPP_MAX
+    const int b = __builtin_bit_cast(int, v);
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0)), r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)), r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+    return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+}
+
 __device__ __forceinline__ float apply_act(int act, float v) {
     switch (act) {
     case kActRelu: return fmaxf(v, 0.0f);

@@ -79,19 +79,33 @@ __global__ __launch_bounds__(256) void dequant16bit_kernel(const uint8_t *__rest
                         Op16<BF16>::pack(w[14], w[15]));
 }
 
-// fp32 activations -> fp16 [M, K] (the generic batched path rounds activations to fp16 operands)
-__global__ __launch_bounds__(256) void x_to_f16_kernel(const float *__restrict__ x, uint16_t *__restrict__ out, int64_t total8) {
-    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (g >= total8) return;
-    const float4 a = reinterpret_cast<const float4 *>(x)[2 * g], b = reinterpret_cast<const float4 *>(x)[2 * g + 1];
-    reinterpret_cast<uint4 *>(out)[g] =
-        make_uint4(Op16<false>::pack(a.x, a.y), Op16<false>::pack(a.z, a.w), Op16<false>::pack(b.x, b.y), Op16<false>::pack(b.z, b.w));
+// fp32 activations -> fp16 [M, K], one workgroup per row: the row is scaled by a power of two
+// (pow2_scale) so that neither large nor tiny inputs leave fp16's range; rowscale[m] receives the
+// inverse, which the GEMM's epilogue applies.  (The row is read twice, the second time from cache.)
+__global__ __launch_bounds__(256) void x_to_f16_kernel(const float *__restrict__ X, int K, uint16_t *__restrict__ out, float *__restrict__ rowscale) {
+    __shared__ float part[4];
+    const float4 *x = reinterpret_cast<const float4 *>(X + (int64_t)blockIdx.x * K);
+    const int k8 = K / 8;
+    float am = 0.f;
+    for (int g = threadIdx.x; g < k8; g += 256) am = fmaxf(am, amax8(x[2 * g], x[2 * g + 1]));
+    am = wave_max(am);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = am;
+    __syncthreads();
+    float sc, inv;
+    pow2_scale(fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3])), sc, inv);
+    if (threadIdx.x == 0) rowscale[blockIdx.x] = inv;
+    uint4 *o = reinterpret_cast<uint4 *>(out + (int64_t)blockIdx.x * K);
+    for (int g = threadIdx.x; g < k8; g += 256) {
+        const float4 a = x[2 * g], b = x[2 * g + 1];
+        o[g] = make_uint4(Op16<false>::pack(a.x * sc, a.y * sc), Op16<false>::pack(a.z * sc, a.w * sc), Op16<false>::pack(b.x * sc, b.y * sc),
+                          Op16<false>::pack(b.z * sc, b.w * sc));
+    }
 }
 
 // The same pass with an RMS normalisation in front: fp16(x / sqrt(mean(x^2) + eps) * (gain + offset)),
 // one workgroup per activation row (the row is read twice, the second time from cache).  K % 8 == 0.
 __global__ __launch_bounds__(256) void x_rmsnorm_to_f16_kernel(const float *__restrict__ X, const float *__restrict__ gain, float gain_offset,
-                                                               float eps, int K, uint16_t *__restrict__ out) {
+                                                               float eps, int K, uint16_t *__restrict__ out, float *__restrict__ rowscale) {
     __shared__ float part[4];
     const float4 *x = reinterpret_cast<const float4 *>(X + (int64_t)blockIdx.x * K);
     const int k8 = K / 8;
@@ -104,6 +118,7 @@ __global__ __launch_bounds__(256) void x_rmsnorm_to_f16_kernel(const float *__re
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
     __syncthreads();
     const float r = sqrtf(((part[0] + part[1]) + (part[2] + part[3])) / (float)K + eps);
+    if (threadIdx.x == 0) rowscale[blockIdx.x] = 1.f;  // normalised rows are O(gain): no scaling
     uint4 *o = reinterpret_cast<uint4 *>(out + (int64_t)blockIdx.x * K);
     for (int g = threadIdx.x; g < k8; g += 256) {
         float4 a = x[2 * g], b = x[2 * g + 1];
@@ -160,7 +175,7 @@ template <int TM, int TN> struct DmaTile {
 template <bool BF16, int TM, int TN, bool GATED = false>
 __global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const uint16_t *Wh, const float *__restrict__ bias,
                                                        float *Y, int M, int K, int N, int act, const float *__restrict__ bias2, int n_out,
-                                                       const float *residual) {
+                                                       const float *residual, const float *__restrict__ rowscale) {
     typedef Op16<BF16> Op;
     typedef DmaTile<TM, TN> G;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -288,7 +303,8 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const 
                     const int m = bm + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                     if (m < M) {
                         const int64_t at = (int64_t)m * n_out + n;
-                        float v = apply_act(act, acc[i][0][r] + bg) * (acc[i][1][r] + bu);
+                        const float rs = rowscale ? rowscale[m] : 1.f;
+                        float v = apply_act(act, fmaf(acc[i][0][r], rs, bg)) * fmaf(acc[i][1][r], rs, bu);
                         if (residual) v += residual[at];
                         Y[at] = v;
                     }
@@ -310,7 +326,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const 
                 if (m < M) {
                     // act(x.W + bias) plus a residual (which may be Y itself: one thread reads and writes an element)
                     const int64_t at = (int64_t)m * N + n;
-                    float v = apply_act(act, acc[i][j][r] + bv);
+                    float v = apply_act(act, rowscale ? fmaf(acc[i][j][r], rowscale[m], bv) : acc[i][j][r] + bv);
                     if (residual) v += residual[at];
                     Y[at] = v;
                 }
@@ -341,7 +357,7 @@ int launch_dequant16bit_type(int type, const uint8_t *W, int64_t N, int64_t K, u
 // N counts the rows of the weight image (for a gated pair: both halves, 64 per 32 outputs)
 template <bool BF16, int TM, int TN, bool GATED = false>
 int launch_gemm16_tile(const uint16_t *x, int64_t M, int64_t K, const uint16_t *Wh, int64_t N, const float *bias, int act, float *y,
-                       const float *bias2, int64_t n_out, const float *residual, hipStream_t s) {
+                       const float *bias2, int64_t n_out, const float *residual, const float *rowscale, hipStream_t s) {
     typedef DmaTile<TM, TN> G;
     static const bool lds_ok = [] {
         return hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_dma_kernel<BF16, TM, TN, GATED>),
@@ -350,7 +366,7 @@ int launch_gemm16_tile(const uint16_t *x, int64_t M, int64_t K, const uint16_t *
     if (!lds_ok) return fail(GQ_ERR_HIP, "gemm: cannot reserve %d bytes of LDS", G::kLdsBytes);
     const dim3 grid((unsigned)((N + G::DN - 1) / G::DN), (unsigned)((M + G::DM - 1) / G::DM));
     return launch(gemm_dma_kernel<BF16, TM, TN, GATED>, grid, dim3(512), (size_t)G::kLdsBytes, s, x, Wh, bias, y, (int)M, (int)K, (int)N, act,
-                  bias2, (int)n_out, residual);
+                  bias2, (int)n_out, residual, rowscale);
 }
 
 // GOMLX_HIPQ_GEMM_TILE=0|1|2 forces the 256x128 / 128x128 / 128x64 tile (tuning runs only).
@@ -362,27 +378,27 @@ int tile_env() {
 // The largest tile that still gives the chip about one workgroup per CU.
 template <bool BF16>
 int launch_gemm16(const uint16_t *x, int64_t M, int64_t K, const uint16_t *Wh, int64_t N, const float *bias, int act, float *y, hipStream_t s,
-                  const float *residual = nullptr) {
+                  const float *residual = nullptr, const float *rowscale = nullptr) {
     const int64_t want = (int64_t)device_cu_count() * 3 / 4;
     auto tiles = [&](int64_t dm, int64_t dn) { return ((M + dm - 1) / dm) * ((N + dn - 1) / dn); };
     int choice = (tiles(256, 128) >= want && M > 128) ? 0 : tiles(128, 128) >= want ? 1 : 2;  // (no half-empty 256-row tiles)
     if (tile_env() >= 0 && tile_env() <= 2) choice = tile_env();
     switch (choice) {
-    case 0: return launch_gemm16_tile<BF16, 2, 2>(x, M, K, Wh, N, bias, act, y, nullptr, N, residual, s);
-    case 1: return launch_gemm16_tile<BF16, 1, 2>(x, M, K, Wh, N, bias, act, y, nullptr, N, residual, s);
-    default: return launch_gemm16_tile<BF16, 1, 1>(x, M, K, Wh, N, bias, act, y, nullptr, N, residual, s);
+    case 0: return launch_gemm16_tile<BF16, 2, 2>(x, M, K, Wh, N, bias, act, y, nullptr, N, residual, rowscale, s);
+    case 1: return launch_gemm16_tile<BF16, 1, 2>(x, M, K, Wh, N, bias, act, y, nullptr, N, residual, rowscale, s);
+    default: return launch_gemm16_tile<BF16, 1, 1>(x, M, K, Wh, N, bias, act, y, nullptr, N, residual, rowscale, s);
     }
 }
 
 // Gated pair (fp16 operands): the interleaved image has 64 rows per 32 outputs.
 int64_t gated_image_rows(int64_t N) { return (N + 31) / 32 * 64; }
 int launch_gemm16_gated(const uint16_t *x, int64_t M, int64_t K, const uint16_t *Wh, int64_t N, const float *bias, const float *bias2, int act,
-                        float *y, const float *residual, hipStream_t s) {
+                        float *y, const float *residual, const float *rowscale, hipStream_t s) {
     const int64_t rows = gated_image_rows(N);
     const int64_t want = (int64_t)device_cu_count() * 3 / 4;
     const bool big = M > 128 && ((M + 255) / 256) * ((rows + 127) / 128) >= want;
-    if (big && tile_env() != 1) return launch_gemm16_tile<false, 2, 2, true>(x, M, K, Wh, rows, bias, act, y, bias2, N, residual, s);
-    return launch_gemm16_tile<false, 1, 2, true>(x, M, K, Wh, rows, bias, act, y, bias2, N, residual, s);
+    if (big && tile_env() != 1) return launch_gemm16_tile<false, 2, 2, true>(x, M, K, Wh, rows, bias, act, y, bias2, N, residual, rowscale, s);
+    return launch_gemm16_tile<false, 1, 2, true>(x, M, K, Wh, rows, bias, act, y, bias2, N, residual, rowscale, s);
 }
 
 // Measured against the fused kernel (K = 4096, N = 4096 .. 14336): the two passes win from the
@@ -414,9 +430,10 @@ bool gemm_two_pass_supported(int type, bool x_is_bf16, int64_t M, int64_t K, int
     return (reinterpret_cast<uintptr_t>(x) & 15) == 0;
 }
 
+// [16-bit weight image][fp32 activations only: fp16 activation image, M row scales]
 size_t gemm_two_pass_workspace(bool x_is_bf16, int64_t M, int64_t K, int64_t N) {
     const size_t w = ((size_t)N * K * 2 + 255) & ~(size_t)255;
-    return w + (x_is_bf16 ? 0 : (size_t)M * K * 2);
+    return w + (x_is_bf16 ? 0 : (((size_t)M * K * 2 + 255) & ~(size_t)255) + (size_t)M * sizeof(float));
 }
 
 int launch_gemm_two_pass(int type, bool x_is_bf16, const void *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias,
@@ -427,11 +444,10 @@ int launch_gemm_two_pass(int type, bool x_is_bf16, const void *x, int64_t M, int
         return launch_gemm16<true>(static_cast<const uint16_t *>(x), M, K, wh, N, bias, act, y, s);
     }
     uint16_t *xh = wh + (((size_t)N * K * 2 + 255) & ~(size_t)255) / 2;
+    float *rowscale = reinterpret_cast<float *>(xh + (((size_t)M * K * 2 + 255) & ~(size_t)255) / 2);
     if (int rc = launch_dequant16bit_type<false>(type, W, N, K, wh, s)) return rc;
-    const int64_t total8 = M * K / 8;
-    if (int rc = launch(x_to_f16_kernel, dim3((unsigned)((total8 + 255) / 256)), dim3(256), 0, s, static_cast<const float *>(x), xh, total8))
-        return rc;
-    return launch_gemm16<false>(xh, M, K, wh, N, bias, act, y, s);
+    if (int rc = launch(x_to_f16_kernel, dim3((unsigned)M), dim3(256), 0, s, static_cast<const float *>(x), (int)K, xh, rowscale)) return rc;
+    return launch_gemm16<false>(xh, M, K, wh, N, bias, act, y, s, nullptr, rowscale);
 }
 
 // The two passes for a projection with its neighbours (fp32 activations): the RMS normalisation
@@ -440,7 +456,7 @@ int launch_gemm_two_pass(int type, bool x_is_bf16, const void *x, int64_t M, int
 // product formed in registers, so neither projection is ever written out.
 size_t gemm_two_pass_block_workspace(int64_t M, int64_t K, int64_t N, bool gated) {
     const int64_t rows = gated ? gated_image_rows(N) : N;
-    return (((size_t)rows * K * 2 + 255) & ~(size_t)255) + (size_t)M * K * 2;
+    return (((size_t)rows * K * 2 + 255) & ~(size_t)255) + (((size_t)M * K * 2 + 255) & ~(size_t)255) + (size_t)M * sizeof(float);
 }
 
 bool gemm_two_pass_block_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, bool gated) {
@@ -454,20 +470,21 @@ int launch_gemm_two_pass_block(int type, const float *x, int64_t M, int64_t K, c
     const int64_t rows = W2 ? gated_image_rows(N) : N;
     uint16_t *wh = static_cast<uint16_t *>(workspace);
     uint16_t *xh = wh + (((size_t)rows * K * 2 + 255) & ~(size_t)255) / 2;
+    float *rowscale = reinterpret_cast<float *>(xh + (((size_t)M * K * 2 + 255) & ~(size_t)255) / 2);
     if (norm) {
-        if (int rc = launch(x_rmsnorm_to_f16_kernel, dim3((unsigned)M), dim3(256), 0, s, x, norm->gain, norm->gain_offset, norm->eps, (int)K, xh))
+        if (int rc = launch(x_rmsnorm_to_f16_kernel, dim3((unsigned)M), dim3(256), 0, s, x, norm->gain, norm->gain_offset, norm->eps, (int)K, xh,
+                            rowscale))
             return rc;
     } else {
-        const int64_t total8 = M * K / 8;
-        if (int rc = launch(x_to_f16_kernel, dim3((unsigned)((total8 + 255) / 256)), dim3(256), 0, s, x, xh, total8)) return rc;
+        if (int rc = launch(x_to_f16_kernel, dim3((unsigned)M), dim3(256), 0, s, x, (int)K, xh, rowscale)) return rc;
     }
     if (!W2) {
         if (int rc = launch_dequant16bit_type<false>(type, W, N, K, wh, s)) return rc;
-        return launch_gemm16<false>(xh, M, K, wh, N, bias, act, y, s, residual);
+        return launch_gemm16<false>(xh, M, K, wh, N, bias, act, y, s, residual, rowscale);
     }
     if (int rc = launch_dequant16bit_type<false>(type, W, N, K, wh, s, 1)) return rc;
     if (int rc = launch_dequant16bit_type<false>(type, W2, N, K, wh, s, 2)) return rc;
-    return launch_gemm16_gated(xh, M, K, wh, N, bias, bias2, act, y, residual, s);
+    return launch_gemm16_gated(xh, M, K, wh, N, bias, bias2, act, y, residual, rowscale, s);
 }
 
 }  // namespace gq

@@ -79,31 +79,6 @@ __device__ __forceinline__ float dpp_quad_sum(float v) {
     return v;
 }
 
-// The activations of one batch column within one K-slice are scaled by a power of two before they
-// are rounded to fp16, so that their largest magnitude lands in [512, 1024): whatever the range
-// of the inputs, nothing overflows (a sub-block sum of 32 values stays below 32768) and nothing
-// falls into fp16's subnormals that matters next to the largest value.  The slice's partial sums
-// are multiplied by the inverse (exact) in the reduction.  Zero, subnormal-tiny and non-finite
-// maxima leave the slice unscaled.
-__device__ __forceinline__ void pow2_scale(float amax, float &s, float &inv) {
-    const int e = (int)((__builtin_bit_cast(uint32_t, amax) >> 23) & 0xFFu);
-    if (e >= 10 && e <= 254) {
-        s = __builtin_bit_cast(float, (uint32_t)(263 - e) << 23);    // 2^(136 - e): amax * s in [2^9, 2^10)
-        inv = __builtin_bit_cast(float, (uint32_t)(e - 9) << 23);    // 2^(e - 136)
-    } else {
-        s = 1.f;
-        inv = 1.f;
-    }
-}
-__device__ __forceinline__ float amax8(const float4 &a, const float4 &b) {
-    return fmaxf(fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))),
-                 fmaxf(fmaxf(fabsf(b.x), fabsf(b.y)), fmaxf(fabsf(b.z), fabsf(b.w))));
-}
-__device__ __forceinline__ float wave_max(float v) {
-    for (int m = 1; m < 64; m <<= 1) v = fmaxf(v, __shfl_xor(v, m));
-    return v;
-}
-
 // ---- stage the K-slice of x into LDS in MFMA fragment order ---------------------------------
 //
 // One item = 8 consecutive activations of one batch column ("octet").  Inside a super-block the
@@ -347,7 +322,9 @@ __global__ __launch_bounds__(256) void mmq_reduce_kernel(const float *__restrict
                                                          int act, const float *residual, float *Y, const float *__restrict__ xscale) {
     const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= MN) return;
-    const int M = (int)(MN / N), m = (int)(i / N);
+    const bool small = MN <= (int64_t)INT32_MAX;  // (32-bit divisions are a fraction of the cost of 64-bit ones)
+    const int M = small ? (int)((uint32_t)MN / (uint32_t)N) : (int)(MN / N);
+    const int m = small ? (int)((uint32_t)i / (uint32_t)N) : (int)(i / N);
     auto total = [&](const float *p, const float *b) {
         float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
         for (int k = 0; k < nslices; k++) {

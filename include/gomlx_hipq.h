@@ -97,8 +97,8 @@ int gq_dequantize(int type, const void *dW, int64_t N, int64_t K, float *dOut, v
  * dBias may be NULL.  fp32 activations, fp32 accumulation.  The first few rows (4 to 8, depending
  * on format and matrix size) run as bandwidth-bound GEMV passes; larger batches contract on the
  * matrix cores with the activations (and, from 97 rows on, the dequantised weights) rounded to
- * fp16 operands (activations beyond +-65504 overflow there, and rows whose values are all below
- * about 1e-4 lose precision to fp16 subnormals).  Batches of 5 rows and more may use a
+ * fp16 operands (each batch row scaled by a power of two first, so the magnitude of x does not
+ * matter).  Batches of 5 rows and more may use a
  * per-stream workspace that is created on the first such call on the stream: make
  * one call outside a recording (gq_graph_begin) before recording the same call. ---- */
 int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *dW, int64_t N,

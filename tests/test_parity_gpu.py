@@ -463,6 +463,28 @@ def test_small_batches_over_a_single_block_are_exact_passes(gpu, oracle, t):
             assert rel_err(run_dense(gpu, t, x, W, bias, 0), oracle.c_qdense(t, x, W, bias, 0)) < 1e-4, (t, M, K, N)
 
 
+@pytest.mark.parametrize("t", [Q8_0, Q4_K, Q6_K])
+def test_activation_magnitude_does_not_matter(gpu, oracle, t):
+    """The reference computes in fp32 and is indifferent to the scale of x.  So is every kernel family
+    here: the GEMV quantises every 32 activations on their own, the MFMA paths scale every batch row
+    (split-K: every K-slice of it) by a power of two before rounding to fp16.  Rows of very different
+    magnitude in one batch included."""
+    K, N = 1024, 256
+    W = synth.weights(t, 390 + t, N, K)
+    for M in (1, 3, 8, 32, 300):
+        base = synth.activations(391 + M, M, K)
+        for sc in (1e-7, 1e-4, 1.0, 3e4, 1e9):
+            x = (base * np.float32(sc)).astype(np.float32)
+            got = run_dense(gpu, t, x, W)
+            assert rel_err(got, oracle.c_qdense(t, x, W)) < TOL_F32, (t, M, sc)
+        if M > 1:
+            rows = (base * np.logspace(-6, 8, M, dtype=np.float32)[:, None]).astype(np.float32)
+            got = run_dense(gpu, t, rows, W)
+            want = oracle.c_qdense(t, rows, W)
+            per_row = np.max(np.abs(got.astype(np.float64) - want), axis=1) / np.max(np.abs(want), axis=1)
+            assert np.all(per_row < TOL_F32), (t, M, float(per_row.max()))
+
+
 def test_randomized_problems(gpu, oracle):
     """150 seeded random problems over all formats, both activation types, every activation, with
     and without bias: batch sizes, K and N drawn from lists that include every tile and slice
