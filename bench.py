@@ -46,7 +46,7 @@ _KIB, _FETCH_SCALE, _WRITE_SCALE = 1024, 65536.0 / 32780.5, 1.0
 COUNTER_KIB = {  # workload -> (FETCH_SIZE, WRITE_SIZE) raw counter KiB per step
     "c0": (8811.9, 16.0),
     "c1": (16262.6, 56.0),
-    "c2": (19875.1 + 1842.5 + 911.6, 3584.0 + 512.0 + 924.0),
+    "c2": (19875.5 + 1859.6 + 916.6, 3584.0 + 512.0 + 925.8),
     "c3": (74726.7, 32768.0),
     "c4": (60543.5, 168.0),
     "ffn": (32484.0, 56.0),
