@@ -59,19 +59,30 @@ template <> struct Op16<false> {
     static __device__ __forceinline__ f32x16 mfma(vec8 a, vec8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
 };
 
+// K rounded up to the GEMM's step: both 16-bit images are written with this row length (zeros behind
+// K), so any K that is a whole number of blocks goes through.
+__host__ __device__ inline int64_t padded_k(int64_t K) { return (K + 63) / 64 * 64; }
+
 // ---- pass 1: GGML blocks -> 16-bit [N, K] -------------------------------------------------------
 // One thread per run of 16 weights (32 output bytes).  half = 0: image row = weight row.  half = 1 / 2:
 // the matrix is the first / second of a gated pair, whose images interleave in chunks of 32 rows
 // (image rows 64 c .. 64 c + 31 = rows 32 c .. of the first matrix, the next 32 = the same rows of
 // the second), so that a wavefront's 64-column tile holds both projections of 32 outputs.
+// The image's rows hold runs_per_row runs, of which the first `runs` come from W and the rest (padding
+// of K to the GEMM's step of 64) are zero.
 template <int T, bool BF16>
 __global__ __launch_bounds__(256) void dequant16bit_kernel(const uint8_t *__restrict__ W, uint16_t *__restrict__ out, int64_t runs_per_row,
-                                                          int64_t total_runs, int64_t row_bytes, int half) {
+                                                          int64_t total_runs, int64_t row_bytes, int half, int64_t runs) {
     const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (g >= total_runs) return;
     const int64_t row = g / runs_per_row, run = g % runs_per_row;
     float w[16];
-    dequant16<T>(W + row * row_bytes, run, w);
+    if (run < runs) {
+        dequant16<T>(W + row * row_bytes, run, w);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; i++) w[i] = 0.f;
+    }
     const int64_t out_row = half == 0 ? row : (row >> 5) * 64 + (half - 1) * 32 + (row & 31);
     uint4 *dst = reinterpret_cast<uint4 *>(out + (out_row * runs_per_row + run) * 16);
     dst[0] = make_uint4(Op16<BF16>::pack(w[0], w[1]), Op16<BF16>::pack(w[2], w[3]), Op16<BF16>::pack(w[4], w[5]), Op16<BF16>::pack(w[6], w[7]));
@@ -85,7 +96,7 @@ __global__ __launch_bounds__(256) void dequant16bit_kernel(const uint8_t *__rest
 __global__ __launch_bounds__(256) void x_to_f16_kernel(const float *__restrict__ X, int K, uint16_t *__restrict__ out, float *__restrict__ rowscale) {
     __shared__ float part[4];
     const float4 *x = reinterpret_cast<const float4 *>(X + (int64_t)blockIdx.x * K);
-    const int k8 = K / 8;
+    const int k8 = K / 8, kp8 = (int)(padded_k(K) / 8);
     float am = 0.f;
     for (int g = threadIdx.x; g < k8; g += 256) am = fmaxf(am, amax8(x[2 * g], x[2 * g + 1]));
     am = wave_max(am);
@@ -94,8 +105,9 @@ __global__ __launch_bounds__(256) void x_to_f16_kernel(const float *__restrict__
     float sc, inv;
     pow2_scale(fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3])), sc, inv);
     if (threadIdx.x == 0) rowscale[blockIdx.x] = inv;
-    uint4 *o = reinterpret_cast<uint4 *>(out + (int64_t)blockIdx.x * K);
-    for (int g = threadIdx.x; g < k8; g += 256) {
+    uint4 *o = reinterpret_cast<uint4 *>(out + (int64_t)blockIdx.x * (kp8 * 8));
+    for (int g = threadIdx.x; g < kp8; g += 256) {
+        if (g >= k8) { o[g] = make_uint4(0u, 0u, 0u, 0u); continue; }
         const float4 a = x[2 * g], b = x[2 * g + 1];
         o[g] = make_uint4(Op16<false>::pack(a.x * sc, a.y * sc), Op16<false>::pack(a.z * sc, a.w * sc), Op16<false>::pack(b.x * sc, b.y * sc),
                           Op16<false>::pack(b.z * sc, b.w * sc));
@@ -108,7 +120,7 @@ __global__ __launch_bounds__(256) void x_rmsnorm_to_f16_kernel(const float *__re
                                                                float eps, int K, uint16_t *__restrict__ out, float *__restrict__ rowscale) {
     __shared__ float part[4];
     const float4 *x = reinterpret_cast<const float4 *>(X + (int64_t)blockIdx.x * K);
-    const int k8 = K / 8;
+    const int k8 = K / 8, kp8 = (int)(padded_k(K) / 8);
     float ss = 0.f;
     for (int g = threadIdx.x; g < k8; g += 256) {
         const float4 a = x[2 * g], b = x[2 * g + 1];
@@ -119,8 +131,9 @@ __global__ __launch_bounds__(256) void x_rmsnorm_to_f16_kernel(const float *__re
     __syncthreads();
     const float r = sqrtf(((part[0] + part[1]) + (part[2] + part[3])) / (float)K + eps);
     if (threadIdx.x == 0) rowscale[blockIdx.x] = 1.f;  // normalised rows are O(gain): no scaling
-    uint4 *o = reinterpret_cast<uint4 *>(out + (int64_t)blockIdx.x * K);
-    for (int g = threadIdx.x; g < k8; g += 256) {
+    uint4 *o = reinterpret_cast<uint4 *>(out + (int64_t)blockIdx.x * (kp8 * 8));
+    for (int g = threadIdx.x; g < kp8; g += 256) {
+        if (g >= k8) { o[g] = make_uint4(0u, 0u, 0u, 0u); continue; }
         float4 a = x[2 * g], b = x[2 * g + 1];
         a.x /= r; a.y /= r; a.z /= r; a.w /= r; b.x /= r; b.y /= r; b.z /= r; b.w /= r;
         if (gain) {
@@ -337,9 +350,9 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const 
 
 template <int T, bool BF16>
 int launch_dequant16bit(const uint8_t *W, int64_t N, int64_t K, uint16_t *out, hipStream_t s, int half) {
-    const int64_t runs_per_row = K / 16, total = N * runs_per_row;
+    const int64_t runs = K / 16, runs_per_row = padded_k(K) / 16, total = N * runs_per_row;
     const int64_t row_bytes = (K / Geom<T>::vpb) * Geom<T>::bpb;
-    return launch(dequant16bit_kernel<T, BF16>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, W, out, runs_per_row, total, row_bytes, half);
+    return launch(dequant16bit_kernel<T, BF16>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, W, out, runs_per_row, total, row_bytes, half, runs);
 }
 
 template <bool BF16>
@@ -418,20 +431,22 @@ int64_t two_pass_env_rows() {
 
 }  // namespace
 
-// K a multiple of 64 (whole LDS rows; also whole blocks of every format), per-thread byte offsets of
-// a 256-row tile within 32 bits, 16-byte aligned activations.
+// Per-thread byte offsets of a 256-row tile within 32 bits, 16-byte aligned activations.  The GEMM
+// steps through K in 64s (whole LDS rows): bf16 activations are read in place and need K % 64 == 0,
+// fp32 activations are rewritten anyway and get rows padded to that.
 bool gemm_two_pass_supported(int type, bool x_is_bf16, int64_t M, int64_t K, int64_t N, const void *x) {
     if (type != kQ4_0 && type != kQ8_0 && type != kIQ4_NL && type != kQ4_K && type != kQ6_K) return false;
     if (type == kQ8_0 && x_is_bf16 && M >= kFusedQ8Bf16From && M < kFusedQ8Bf16Below && two_pass_env_rows() <= 0) return false;
     const int64_t min_rows = two_pass_env_rows() > 0 ? two_pass_env_rows() : kMinRowsTwoPass;
-    if (M < min_rows || K % 64 != 0) return false;
+    if (M < min_rows || K % (x_is_bf16 ? 64 : 32) != 0) return false;
     if (K > (1 << 22) || N > INT32_MAX || M > INT32_MAX || (M + 127) / 128 > 65535) return false;
-    if ((uint64_t)N * (uint64_t)K * 2 > kMaxImageBytes) return false;
+    if ((uint64_t)N * (uint64_t)padded_k(K) * 2 > kMaxImageBytes) return false;
     return (reinterpret_cast<uintptr_t>(x) & 15) == 0;
 }
 
 // [16-bit weight image][fp32 activations only: fp16 activation image, M row scales]
 size_t gemm_two_pass_workspace(bool x_is_bf16, int64_t M, int64_t K, int64_t N) {
+    K = padded_k(K);
     const size_t w = ((size_t)N * K * 2 + 255) & ~(size_t)255;
     return w + (x_is_bf16 ? 0 : (((size_t)M * K * 2 + 255) & ~(size_t)255) + (size_t)M * sizeof(float));
 }
@@ -443,11 +458,12 @@ int launch_gemm_two_pass(int type, bool x_is_bf16, const void *x, int64_t M, int
         if (int rc = launch_dequant16bit_type<true>(type, W, N, K, wh, s)) return rc;
         return launch_gemm16<true>(static_cast<const uint16_t *>(x), M, K, wh, N, bias, act, y, s);
     }
-    uint16_t *xh = wh + (((size_t)N * K * 2 + 255) & ~(size_t)255) / 2;
-    float *rowscale = reinterpret_cast<float *>(xh + (((size_t)M * K * 2 + 255) & ~(size_t)255) / 2);
+    const int64_t Kp = padded_k(K);
+    uint16_t *xh = wh + (((size_t)N * Kp * 2 + 255) & ~(size_t)255) / 2;
+    float *rowscale = reinterpret_cast<float *>(xh + (((size_t)M * Kp * 2 + 255) & ~(size_t)255) / 2);
     if (int rc = launch_dequant16bit_type<false>(type, W, N, K, wh, s)) return rc;
     if (int rc = launch(x_to_f16_kernel, dim3((unsigned)M), dim3(256), 0, s, static_cast<const float *>(x), (int)K, xh, rowscale)) return rc;
-    return launch_gemm16<false>(xh, M, K, wh, N, bias, act, y, s, nullptr, rowscale);
+    return launch_gemm16<false>(xh, M, Kp, wh, N, bias, act, y, s, nullptr, rowscale);
 }
 
 // The two passes for a projection with its neighbours (fp32 activations): the RMS normalisation
@@ -456,12 +472,13 @@ int launch_gemm_two_pass(int type, bool x_is_bf16, const void *x, int64_t M, int
 // product formed in registers, so neither projection is ever written out.
 size_t gemm_two_pass_block_workspace(int64_t M, int64_t K, int64_t N, bool gated) {
     const int64_t rows = gated ? gated_image_rows(N) : N;
+    K = padded_k(K);
     return (((size_t)rows * K * 2 + 255) & ~(size_t)255) + (((size_t)M * K * 2 + 255) & ~(size_t)255) + (size_t)M * sizeof(float);
 }
 
 bool gemm_two_pass_block_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, bool gated) {
     if (!gemm_two_pass_supported(type, false, M, K, N, x)) return false;
-    return !gated || (uint64_t)gated_image_rows(N) * (uint64_t)K * 2 <= kMaxImageBytes;
+    return !gated || (uint64_t)gated_image_rows(N) * (uint64_t)padded_k(K) * 2 <= kMaxImageBytes;
 }
 
 int launch_gemm_two_pass_block(int type, const float *x, int64_t M, int64_t K, const RmsNorm *norm, const uint8_t *W, const float *bias,
@@ -469,8 +486,9 @@ int launch_gemm_two_pass_block(int type, const float *x, int64_t M, int64_t K, c
                                hipStream_t s) {
     const int64_t rows = W2 ? gated_image_rows(N) : N;
     uint16_t *wh = static_cast<uint16_t *>(workspace);
-    uint16_t *xh = wh + (((size_t)rows * K * 2 + 255) & ~(size_t)255) / 2;
-    float *rowscale = reinterpret_cast<float *>(xh + (((size_t)M * K * 2 + 255) & ~(size_t)255) / 2);
+    const int64_t Kp = padded_k(K);
+    uint16_t *xh = wh + (((size_t)rows * Kp * 2 + 255) & ~(size_t)255) / 2;
+    float *rowscale = reinterpret_cast<float *>(xh + (((size_t)M * Kp * 2 + 255) & ~(size_t)255) / 2);
     if (norm) {
         if (int rc = launch(x_rmsnorm_to_f16_kernel, dim3((unsigned)M), dim3(256), 0, s, x, norm->gain, norm->gain_offset, norm->eps, (int)K, xh,
                             rowscale))
@@ -480,11 +498,11 @@ int launch_gemm_two_pass_block(int type, const float *x, int64_t M, int64_t K, c
     }
     if (!W2) {
         if (int rc = launch_dequant16bit_type<false>(type, W, N, K, wh, s)) return rc;
-        return launch_gemm16<false>(xh, M, K, wh, N, bias, act, y, s, residual, rowscale);
+        return launch_gemm16<false>(xh, M, Kp, wh, N, bias, act, y, s, residual, rowscale);
     }
     if (int rc = launch_dequant16bit_type<false>(type, W, N, K, wh, s, 1)) return rc;
     if (int rc = launch_dequant16bit_type<false>(type, W2, N, K, wh, s, 2)) return rc;
-    return launch_gemm16_gated(xh, M, K, wh, N, bias, bias2, act, y, residual, rowscale, s);
+    return launch_gemm16_gated(xh, M, Kp, wh, N, bias, bias2, act, y, residual, rowscale, s);
 }
 
 }  // namespace gq

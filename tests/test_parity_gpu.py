@@ -366,7 +366,7 @@ def test_batches_of_17_to_128_rows(gpu, oracle, t, M, K, N):
 @pytest.mark.parametrize("K", [64, 128, 192, 96])
 def test_large_batches_few_k_steps(gpu, oracle, K):
     """One, two and three K steps (shorter than the stage ring) and a K that is not a multiple of
-    64, which stays on the fused kernel."""
+    64, which for bf16 activations (read in place) stays on the fused kernel."""
     M, N = 600, 200
     W = synth.weights(Q8_0, 98, N, K)
     x = bf16_round(synth.activations(99, M, K))
@@ -483,6 +483,27 @@ def test_activation_magnitude_does_not_matter(gpu, oracle, t):
             want = oracle.c_qdense(t, rows, W)
             per_row = np.max(np.abs(got.astype(np.float64) - want), axis=1) / np.max(np.abs(want), axis=1)
             assert np.all(per_row < TOL_F32), (t, M, float(per_row.max()))
+
+
+@pytest.mark.parametrize("t", [Q8_0, Q4_0, IQ4_NL])
+def test_large_batches_over_an_odd_number_of_blocks(gpu, oracle, t):
+    """K an odd multiple of 32 with more than 16 fp32 rows: both 16-bit images get rows padded with
+    zeros to the GEMM's step of 64, so these shapes take the two scaled passes like every other and
+    are as indifferent to the magnitude of x; with the neighbours of a decoder block as well."""
+    for i, (M, K, N) in enumerate([(17, 32, 8), (40, 96, 130), (300, 160, 257), (130, 1056, 132)]):
+        W = synth.weights(t, 440 + i, N, K)
+        base = synth.activations(441 + i, M, K)
+        bias = synth.normal(442 + i, 0, N).astype(np.float32) * 0.1
+        for sc in (1e-7, 1.0, 1e9):
+            x = (base * np.float32(sc)).astype(np.float32)
+            assert rel_err(run_dense(gpu, t, x, W), oracle.c_qdense(t, x, W)) < TOL_F32, (t, M, K, N, sc)
+        got = run_dense(gpu, t, base, W, bias, 3)
+        want, pre = oracle.c_qdense(t, base, W, bias, 3), oracle.c_qdense(t, base, W, bias, 0)
+        err = float(np.max(np.abs(got.astype(np.float64) - want))) / max(float(np.max(np.abs(want))), float(np.max(np.abs(pre))))
+        assert err < TOL_F32, (t, M, K, N, err)
+        for norm_kind in (0, 1):
+            err = gated_case(gpu, oracle, t, M, K, N, 3, norm_kind, True, 450 + 10 * i + t)
+            assert err < 2 * TOL_F32, ("gated", t, M, K, N, norm_kind, err)
 
 
 def test_randomized_problems(gpu, oracle):
