@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1] [--others]
 
---config takes c0 .. c4 (the BASELINE.json configurations), ffn (the gated feed-forward front of
+--config takes c0 .. c4 (the BASELINE.json configurations), prefill (C3's shape with fp32 activations), ffn (the gated feed-forward front of
 a decoder layer: the callers around the two projections folded into one launch) or layer (the
 seven projections of C4 in the order and with the dependencies of a decoder layer).
 
@@ -49,6 +49,7 @@ COUNTER_KIB = {  # workload -> (FETCH_SIZE, WRITE_SIZE) raw counter KiB per step
     "c2": (19875.5 + 1859.6 + 916.6, 3584.0 + 512.0 + 925.8),
     "c3": (74726.7, 32768.0),
     "c4": (60543.5, 168.0),
+    "prefill": (4631.4 + 24107.9 + 82461.1, 32768.1 + 16449.2 + 32768.0),
     "ffn": (32484.0, 56.0),
     "layer": (7126.2 + 4756.1 + 32483.6 + 16449.7, 24.0 + 16.0 + 56.0 + 16.0),
 }
@@ -67,6 +68,7 @@ CONFIGS = {
     "c1": ("Q4_0", 1, 4096, 14336, "f32", "hbm"),
     "c2": ("Q4_K", 32, 14336, 4096, "f32", "hbm"),
     "c3": ("Q8_0", 2048, 4096, 4096, "bf16", "mfma"),
+    "prefill": ("Q4_K", 2048, 4096, 4096, "f32", "mfma"),
 }
 C4_SHAPES = [(4096, 4096), (4096, 1024), (4096, 1024), (4096, 4096), (4096, 14336), (4096, 14336), (14336, 4096)]
 WORKLOAD_TEXT = {
@@ -75,6 +77,8 @@ WORKLOAD_TEXT = {
     "c2": "configs[2]: Q4_K dense, decode batch M=32, K=14336 -> N=4096",
     "c3": "configs[3]: Q8_0 prefill GEMM, M=2048 bf16, K=4096, N=4096",
     "c4": "configs[4]: seven Q4_K projections of a Llama-3-8B layer, batch 1",
+    "prefill": "C3's shape with fp32 activations and Q4_K weights (M=2048, K=4096, N=4096): weights to an fp16 image, activations "
+               "to scaled fp16 rows, fp16 MFMA GEMM (three launches)",
     "layer": "the seven Q4_K projections of a Llama-3-8B layer as a decoder runs them, batch 1: four dependent launches "
              "(RMSNorm + q/k/v, o + residual, RMSNorm + gate/up + SiLU*mul, down + residual)",
     "ffn": "gated feed-forward front of a Llama-3-8B layer, batch 1: RMSNorm, Q4_K gate and up 4096 -> 14336, SiLU(gate) * up, one launch",
@@ -118,7 +122,7 @@ class Problem:
             tn, M, K, N, self.dtype, self.bound = CONFIGS[name]
             shapes = [(tn, M, K, N)]
         self.parts = []
-        seed = 1000 + (int(name[1]) if name[0] == "c" else 4 if name == "layer" else 5)
+        seed = 1000 + (int(name[1]) if name[0] == "c" else {"layer": 4, "ffn": 5, "prefill": 6}[name])
         total_w = 0
         for i, (tn, M, K, N) in enumerate(shapes):
             t = getattr(ggml, tn)
@@ -265,8 +269,8 @@ def cpu_baseline(name):
         tn, M, K, N, _, _ = CONFIGS[name]
         shapes = [(tn, M, K, N)]
     sample = "full workload"
-    if name == "c3":  # 34 GMAC per pass is minutes of CPU time: a 64-row slice of the 2048 activations
-        shapes = [("Q8_0", 64, 4096, 4096)]
+    if name in ("c3", "prefill"):  # 34 GMAC per pass is minutes of CPU time: a 64-row slice of the 2048 activations
+        shapes = [(CONFIGS[name][0], 64, 4096, 4096)]
         sample = "64 of the 2048 activation rows (1/32 of the FLOPs), all of W"
     probs = []
     for i, (tn, M, K, N) in enumerate(shapes):
@@ -288,7 +292,7 @@ def cpu_baseline(name):
         if (runs >= 5 and el >= 3.0) or el >= 25.0:
             break
     per = el / runs
-    if name == "c3":
+    if name in ("c3", "prefill"):
         return {"value": flops / per / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
                 "sample": f"{sample}; {runs} runs, {per * 1e3:.2f} ms each"}
     return {"value": wbytes / per / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
@@ -341,7 +345,7 @@ def main():
         "metric": rep["metric"], "value": rep["value"], "unit": rep["unit"], "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": rep["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16" if args.config == "c3" else "f32", "data": "synthetic",
+        "dtype": {"c3": "bf16", "prefill": "f16"}.get(args.config, "f32"), "data": "synthetic",
         "config": {"workload": WORKLOAD_TEXT[args.config], "ggml_type": tn,
                    "weights": "cache-resident single buffer" if args.hot else
                    f"cold: rotation over {rep['weight_copies']} distinct weight copies",
@@ -353,10 +357,10 @@ def main():
         line["cpu_baseline"] = cpu_baseline(args.config)
     if args.others:
         others = {}
-        for name in ["c0", "c1", "c2", "c3", "c4", "ffn", "layer"]:
+        for name in ["c0", "c1", "c2", "c3", "c4", "prefill", "ffn", "layer"]:
             if name == args.config:
                 continue
-            steps = args.steps if name != "c3" else max(10, args.steps // 10)
+            steps = args.steps if name not in ("c3", "prefill") else max(10, args.steps // 10)
             saved = args.steps
             args.steps = steps
             r = measure(name)
