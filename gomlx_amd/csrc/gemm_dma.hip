@@ -71,23 +71,36 @@ __host__ __device__ inline int64_t padded_k(int64_t K) { return (K + 63) / 64 * 
 // The image's rows hold runs_per_row runs, of which the first `runs` come from W and the rest (padding
 // of K to the GEMM's step of 64) are zero.
 template <int T, bool BF16>
-__global__ __launch_bounds__(256) void dequant16bit_kernel(const uint8_t *__restrict__ W, uint16_t *__restrict__ out, int64_t runs_per_row,
-                                                          int64_t total_runs, int64_t row_bytes, int half, int64_t runs) {
-    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (g >= total_runs) return;
-    const int64_t row = g / runs_per_row, run = g % runs_per_row;
-    float w[16];
-    if (run < runs) {
-        dequant16<T>(W + row * row_bytes, run, w);
-    } else {
+__global__ __launch_bounds__(256) void dequant16bit_kernel(const uint8_t *__restrict__ W, uint16_t *__restrict__ out, uint32_t runs_per_row,
+                                                          uint32_t total_runs, int64_t row_bytes, int half, uint32_t runs) {
+    // The 16-byte halves of the runs meet in LDS so that consecutive lanes store consecutive 16 bytes
+    // (whole cache lines per store instruction; a lane storing its own 32 bytes in two instructions
+    // half-fills twice as many).  An image holds at most 2^27 runs: 32-bit index arithmetic.
+    __shared__ uint4 halves[512];
+    const uint32_t tid = threadIdx.x, g0 = blockIdx.x * 256u, g = g0 + tid;
+    if (g < total_runs) {
+        const uint32_t row = g / runs_per_row, run = g % runs_per_row;
+        float w[16];
+        if (run < runs) {
+            dequant16<T>(W + (int64_t)row * row_bytes, run, w);
+        } else {
 #pragma unroll
-        for (int i = 0; i < 16; i++) w[i] = 0.f;
+            for (int i = 0; i < 16; i++) w[i] = 0.f;
+        }
+        halves[2 * tid] = make_uint4(Op16<BF16>::pack(w[0], w[1]), Op16<BF16>::pack(w[2], w[3]), Op16<BF16>::pack(w[4], w[5]),
+                                     Op16<BF16>::pack(w[6], w[7]));
+        halves[2 * tid + 1] = make_uint4(Op16<BF16>::pack(w[8], w[9]), Op16<BF16>::pack(w[10], w[11]), Op16<BF16>::pack(w[12], w[13]),
+                                         Op16<BF16>::pack(w[14], w[15]));
     }
-    const int64_t out_row = half == 0 ? row : (row >> 5) * 64 + (half - 1) * 32 + (row & 31);
-    uint4 *dst = reinterpret_cast<uint4 *>(out + (out_row * runs_per_row + run) * 16);
-    dst[0] = make_uint4(Op16<BF16>::pack(w[0], w[1]), Op16<BF16>::pack(w[2], w[3]), Op16<BF16>::pack(w[4], w[5]), Op16<BF16>::pack(w[6], w[7]));
-    dst[1] = make_uint4(Op16<BF16>::pack(w[8], w[9]), Op16<BF16>::pack(w[10], w[11]), Op16<BF16>::pack(w[12], w[13]),
-                        Op16<BF16>::pack(w[14], w[15]));
+    __syncthreads();
+#pragma unroll
+    for (int p = 0; p < 2; p++) {
+        const uint32_t c = tid + 256u * p, gg = g0 + (c >> 1);
+        if (gg >= total_runs) continue;
+        const uint32_t row = gg / runs_per_row, run = gg % runs_per_row;
+        const int64_t out_row = half == 0 ? (int64_t)row : (int64_t)(row >> 5) * 64 + (half - 1) * 32 + (row & 31);
+        *reinterpret_cast<uint4 *>(out + (out_row * runs_per_row + run) * 16 + (c & 1u) * 8u) = halves[c];
+    }
 }
 
 // fp32 activations -> fp16 [M, K], one workgroup per row: the row is scaled by a power of two
@@ -352,7 +365,9 @@ template <int T, bool BF16>
 int launch_dequant16bit(const uint8_t *W, int64_t N, int64_t K, uint16_t *out, hipStream_t s, int half) {
     const int64_t runs = K / 16, runs_per_row = padded_k(K) / 16, total = N * runs_per_row;
     const int64_t row_bytes = (K / Geom<T>::vpb) * Geom<T>::bpb;
-    return launch(dequant16bit_kernel<T, BF16>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, W, out, runs_per_row, total, row_bytes, half, runs);
+    if (total > ((int64_t)1 << 27)) return fail(GQ_ERR_INVALID, "gemm: a 16-bit image of %lld x %lld values is too large", (long long)N, (long long)K);
+    return launch(dequant16bit_kernel<T, BF16>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, W, out, (uint32_t)runs_per_row, (uint32_t)total,
+                  row_bytes, half, (uint32_t)runs);
 }
 
 template <bool BF16>
