@@ -325,12 +325,25 @@ __global__ __launch_bounds__(256) void mmq_reduce_kernel(const float *__restrict
     const bool small = MN <= (int64_t)INT32_MAX;  // (32-bit divisions are a fraction of the cost of 64-bit ones)
     const int M = small ? (int)((uint32_t)MN / (uint32_t)N) : (int)(MN / N);
     const int m = small ? (int)((uint32_t)i / (uint32_t)N) : (int)(i / N);
+    // Slices are added in order, eight at a time: their loads (each a trip to another XCD's freshly written
+    // lines) are all issued before the first sum needs one; a slice past the end re-reads the last and is not added.
     auto total = [&](const float *p, const float *b) {
         float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
-        for (int k = 0; k < nslices; k++) {
-            const float4 v = *reinterpret_cast<const float4 *>(p + (int64_t)k * MN + i);
-            const float f = xscale[(int64_t)k * M + m];
-            s.x = fmaf(v.x, f, s.x); s.y = fmaf(v.y, f, s.y); s.z = fmaf(v.z, f, s.z); s.w = fmaf(v.w, f, s.w);
+        for (int k0 = 0; k0 < nslices; k0 += 8) {
+            float4 v[8];
+            float f[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int k = min(k0 + j, nslices - 1);
+                v[j] = *reinterpret_cast<const float4 *>(p + (int64_t)k * MN + i);
+                f[j] = xscale[(int64_t)k * M + m];
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const bool in = k0 + j < nslices;
+                s.x = in ? fmaf(v[j].x, f[j], s.x) : s.x; s.y = in ? fmaf(v[j].y, f[j], s.y) : s.y;
+                s.z = in ? fmaf(v[j].z, f[j], s.z) : s.z; s.w = in ? fmaf(v[j].w, f[j], s.w) : s.w;
+            }
         }
         if (b) {
             const float4 v = *reinterpret_cast<const float4 *>(b + (int)(i % N));
