@@ -118,22 +118,30 @@ int check_dense_args(const char *fn, int type, const void *x, int64_t M, int64_t
 // below and the two-pass GEMM above.  GEMV passes cost time in proportion to the weight bytes (small
 // matrices: a pass per row, sharing W through the caches; large ones: a pass per four rows, two for
 // Q6_K), the split-K kernels a fixed part plus less per byte.
-// Measured (us, rows 2 3 4 5 6 7 8 10; GEMV passes | split-K):
-//   Q8_0 4096x4096 (18 MB)   9.5 10.5 12.8 15.1 17.4 19.4 21.5 25.9 | 16.6   4096x14336 (62 MB) 15.2 15.9 16.1 25.8 26.9 28.5 26.0 36.7 | 29.5
-//                                                                            14336x4096         16.0 20.2 20.5 30.5 32.7 38.4 36.6 49.8 | 30.8
-//   Q4_0 4096x4096 (9 MB)    7.1  8.1 10.9 12.0 13.2 15.1 16.6 19.7 | 15.5   4096x14336 (33 MB) 11.1 15.1 14.8 20.9 22.2 28.2 25.7 33.3 | 24.8
-//   Q4_K 4096x4096           7.8  9.7 11.9 14.0 16.9 18.7 20.6 24.4 | 18.8   4096x14336         12.6 15.9 15.5 22.6 25.8 28.7 27.2 36.3 | 20.8
-//   Q6_K 4096x4096 (14 MB)   9.2 11.5 14.3 17.6 19.5 21.5 23.7 28.9 | 18.6   4096x14336 (48 MB) 15.8 24.8 24.0 33.3 33.9 43.0 43.3 52.9 | 42.0
-//   IQ4_NL 4096x4096         8.1 10.1 12.3 14.3 16.7 18.7 20.5 23.9 | 16.0   4096x14336         14.1 16.7 17.1 26.3 26.7 31.7 29.5 40.0 | 27.3
+// Measured (us per call in a replayed graph of dependent calls; rows 4 5 6 7 8 9 10; GEMV passes | split-K, flat over these rows):
+//   Q8_0   4096x4096 (18 MB)  12.5 14.3 16.2 17.9 19.9 21.9 23.9 | 14.4   4096x14336 (62 MB) 17.3 27.2 28.0 30.2 27.7 37.9 38.9 | 29.3
+//          4096x1024 (4 MB)    4.8  5.6  6.1  6.4  6.6  8.1  8.2 | 12.9   14336x4096         23.0 32.5 34.0 38.7 36.7 47.3 49.6 | 30.1
+//   Q4_0   4096x4096 (9 MB)    9.6 10.7 12.0 13.5 15.1 16.5 18.0 | 13.0   4096x14336 (33 MB) 14.9 20.7 22.0 27.3 25.8 32.6 34.0 | 23.7
+//          4096x1024 (2 MB)    4.2  4.8  4.8  5.5  5.6  6.2  6.3 | 12.1   14336x4096         19.4 25.2 28.1 34.8 33.0 40.1 43.2 | 24.7
+//   Q4_K   4096x4096          11.1 12.6 14.6 16.6 18.6 20.5 22.5 | 13.1   4096x14336         15.8 22.3 24.1 29.1 27.5 34.9 36.8 | 19.3
+//          4096x1024           4.4  5.4  6.2  6.4  6.5  7.4  8.0 | 12.3   14336x4096         20.4 26.9 29.8 36.7 35.0 42.7 46.0 | 19.6
+//   Q6_K   4096x4096 (14 MB)  13.5 15.3 17.6 19.9 22.3 24.6 27.0 | 17.0   4096x14336 (48 MB) 25.6 34.6 34.6 44.2 44.3 54.0 54.2 | 43.0
+//          4096x1024 (3 MB)    5.1  6.1  6.2  7.2  7.3  8.4  8.5 | 16.4   14336x4096         28.6 37.1 37.3 46.9 48.0 57.6 58.8 | 43.0
+//   IQ4_NL 4096x4096          11.8 12.9 15.0 16.9 18.9 20.9 22.8 | 13.7   4096x14336         17.0 24.0 26.7 31.1 29.4 37.7 40.4 | 26.3
+//          4096x1024           4.8  5.7  5.7  6.6  6.7  7.6  7.7 | 12.8   14336x4096         20.9 28.6 31.1 37.7 35.9 45.0 47.8 | 27.2
+// The split-K route is three dependent launches with a floor of about 12 us: matrices of a few megabytes (the k / v
+// projections of a grouped-query layer) stay on GEMV passes for every batch the GEMV takes.
 // The Q6_K kernel pays 16 scale groups per super-block and only wins for a single tile of 32 batch columns.
+constexpr int64_t kTinyWeightBytes = (int64_t)6 << 20;
 int64_t split_k_from(int type, int64_t weight_bytes) {
+    if (weight_bytes < kTinyWeightBytes) return kGemvMaxRows + 1;
     const bool large = weight_bytes >= kLargeWeightBytes;
     switch (type) {
-    case GQ_Q8_0: return large ? 6 : 7;
-    case GQ_Q4_0: return large ? 6 : 9;
-    case GQ_Q4_K: return large ? 5 : 8;
-    case GQ_Q6_K: return 7;
-    case GQ_IQ4_NL: return large ? 6 : 7;
+    case GQ_Q8_0: return 6;
+    case GQ_Q4_0: return large ? 6 : 7;
+    case GQ_Q4_K: return large ? 5 : 6;
+    case GQ_Q6_K: return large ? 7 : 6;
+    case GQ_IQ4_NL: return 6;
     default: return 8;
     }
 }
