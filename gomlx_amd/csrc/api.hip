@@ -461,6 +461,11 @@ int gq_qdense_block_f32(int type, const float *dX, int64_t M, int64_t K, const g
         return launch_gemm_two_pass_block(type, dX, M, K, norm ? &rn : nullptr, (const uint8_t *)dW, dBias, nullptr, nullptr, dResidual, N, act,
                                           dY, ws, (hipStream_t)stream);
     }
+    // split-K range: the normalisation rides on the activation pre-pass and the reduction, the residual on the reduction
+    if (dense_takes_split_k(type, M, K, N, dX, dBias, dY) && (!dResidual || aligned_to(dResidual, 16)) && (!rn.gain || aligned_to(rn.gain, 16))) {
+        const MmqExtra ex{nullptr, nullptr, dResidual, norm ? &rn : nullptr};
+        return launch_mmq(type, dX, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream, &ex);
+    }
     // composed: normalised activations into the stream's second workspace, the dense call, then the residual
     const float *x = dX;
     if (norm) {
@@ -471,7 +476,7 @@ int gq_qdense_block_f32(int type, const float *dX, int64_t M, int64_t K, const g
         x = xn;
     }
     if (dResidual && dense_takes_split_k(type, M, K, N, x, dBias, dY) && aligned_to(dResidual, 16)) {  // the residual rides on the reduction
-        const MmqExtra ex{nullptr, nullptr, dResidual};
+        const MmqExtra ex{nullptr, nullptr, dResidual, nullptr};
         return launch_mmq(type, x, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream, &ex);
     }
     if (int rc = gq_qdense_f32(type, x, M, K, dW, N, dBias, act, dY, stream)) return rc;
@@ -527,6 +532,11 @@ int gq_qdense_gated_f32(int type, const float *dX, int64_t M, int64_t K, const g
         return launch_gemm_two_pass_block(type, dX, M, K, norm ? &rn : nullptr, (const uint8_t *)dWgate, dBiasGate, (const uint8_t *)dWup, dBiasUp,
                                           nullptr, N, act, dY, ws, (hipStream_t)stream);
     }
+    if (dense_takes_split_k(type, M, K, N, dX, dBiasGate, dY) && (!dBiasUp || aligned_to(dBiasUp, 16)) && (!rn.gain || aligned_to(rn.gain, 16))) {
+        // both matrices against one activation image (which carries the gain); the reduction normalises and forms act(gate) * up
+        const MmqExtra ex{(const uint8_t *)dWup, dBiasUp, nullptr, norm ? &rn : nullptr};
+        return launch_mmq(type, dX, false, M, K, (const uint8_t *)dWgate, N, dBiasGate, act, dY, (hipStream_t)stream, &ex);
+    }
     // composed: [normalised activations,] act(gate) into the stream's second workspace, up into y, y *= act(gate)
     const size_t xn_bytes = norm ? ((size_t)M * (size_t)K * sizeof(float) + 255) / 256 * 256 : 0;
     void *ws = nullptr;
@@ -539,7 +549,7 @@ int gq_qdense_gated_f32(int type, const float *dX, int64_t M, int64_t K, const g
     }
     if (dense_takes_split_k(type, M, K, N, x, dBiasGate, dY) && (!dBiasUp || aligned_to(dBiasUp, 16))) {
         // both matrices against one activation image; the reduction forms act(gate) * up
-        const MmqExtra ex{(const uint8_t *)dWup, dBiasUp, nullptr};
+        const MmqExtra ex{(const uint8_t *)dWup, dBiasUp, nullptr, nullptr};
         return launch_mmq(type, x, false, M, K, (const uint8_t *)dWgate, N, dBiasGate, act, dY, (hipStream_t)stream, &ex);
     }
     float *gate = reinterpret_cast<float *>(static_cast<uint8_t *>(ws) + xn_bytes);

@@ -77,13 +77,15 @@ bool gemv_ks_supported(int type, int64_t K, int64_t N, const void *x);
 int launch_gemv_ks(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N,
                    const float *bias, int act, float *y, hipStream_t s);
 bool mmq_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, const void *bias, const void *y);
-// Optional extras of a split-K call: a second matrix (the result becomes act(x.W + bias) * (x.W2 + bias2), both
-// contracted against one activation image and combined in the reduction) and a residual added last.
-struct MmqExtra { const uint8_t *W2; const float *bias2; const float *residual; };
-int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias,
-               int act, float *y, hipStream_t s, const MmqExtra *ex = nullptr);
 // RMS normalisation in front of a projection: x / sqrt(mean(x^2) + eps) * (gain + gain_offset); gain may be null.
 struct RmsNorm { const float *gain; float eps, gain_offset; };
+// Optional extras of a split-K call: a second matrix (the result becomes act(x.W + bias) * (x.W2 + bias2), both
+// contracted against one activation image and combined in the reduction), a residual added last, and an RMS
+// normalisation of the (fp32) activations (gain 16-byte aligned or null): the gain is applied where the activation
+// image is written, the division by the root mean square in the reduction.
+struct MmqExtra { const uint8_t *W2; const float *bias2; const float *residual; const RmsNorm *norm; };
+int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias,
+               int act, float *y, hipStream_t s, const MmqExtra *ex = nullptr);
 // The K-sliced GEMV with the normalisation folded in and, when W2 is given, the gated product
 // act(x.W + bias) * (x.W2 + bias2); fp32 activations, at most 16 rows (the entry points use it below 8 rows, where a pass per row still wins).
 bool gemv_ks_ext_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, const void *gain);

@@ -79,6 +79,22 @@ __device__ __forceinline__ float dpp_quad_sum(float v) {
     return v;
 }
 
+// RMS normalisation folded into the split-K route: the pre-pass multiplies x by (gain + offset) before it scales and
+// rounds, and leaves each (slice, column)'s sum of squares of the raw x in xss[slice][M]; the reduction divides the
+// finished sums of column m by sqrt(sum_s xss[s][m] / K + eps) (the contraction is linear in x).
+__device__ __forceinline__ float sumsq8(const float4 &a, const float4 &b) {
+    return ((a.x * a.x + a.y * a.y) + (a.z * a.z + a.w * a.w)) + ((b.x * b.x + b.y * b.y) + (b.z * b.z + b.w * b.w));
+}
+__device__ __forceinline__ void apply_gain8(const float *__restrict__ gain, float off, int k, float4 &a, float4 &b) {  // gain 16-byte aligned, k % 8 == 0
+    const float4 g0 = *reinterpret_cast<const float4 *>(gain + k), g1 = *reinterpret_cast<const float4 *>(gain + k + 4);
+    a.x *= g0.x + off; a.y *= g0.y + off; a.z *= g0.z + off; a.w *= g0.w + off;
+    b.x *= g1.x + off; b.y *= g1.y + off; b.z *= g1.z + off; b.w *= g1.w + off;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+    for (int m = 1; m < 64; m <<= 1) v += __shfl_xor(v, m);
+    return v;
+}
+
 // ---- stage the K-slice of x into LDS in MFMA fragment order ---------------------------------
 //
 // One item = 8 consecutive activations of one batch column ("octet").  Inside a super-block the
@@ -91,10 +107,13 @@ __device__ __forceinline__ float dpp_quad_sum(float v) {
 // columns a half-wave later reads from one slot) over all LDS banks.
 // The eight sub-block sums of (sbl, m) are stored in the order (0, 2, 1, 3, 4, 6, 5, 7) too.
 // `active`: the thread's octet belongs to the slice (slices may hold fewer than 8 super-blocks).
-// red: [2][ROUNDS][4] floats of shared memory; inv_scale[m] receives the slice's inverse scale of column m0 + m.
+// red: [2][2][ROUNDS][4] floats of shared memory; inv_scale[m] receives the slice's inverse scale of column m0 + m.
+// With xss (normalisation folded in): x is multiplied by gain + gain_offset (gain may be null) and xss[m0 + m] receives
+// the slice's sum of squares of the raw x.
 template <int ROUNDS, bool BF16X>
 __device__ __forceinline__ void stage_x(const void *__restrict__ X, int M, int K, int m0, int k0, uint8_t *__restrict__ lds, int tid,
-                                        int round0, bool active, float *red, float *__restrict__ inv_scale) {
+                                        int round0, bool active, float *red, float *__restrict__ inv_scale, const float *__restrict__ gain,
+                                        float gain_offset, float *__restrict__ xss) {
     const int oct = tid & 255;  // fixed per thread; its items are columns (tid >> 8) + 2 r
     const int k = k0 + 8 * oct;
     const int sbl = oct >> 5, v8 = oct & 31;
@@ -115,9 +134,15 @@ __device__ __forceinline__ void stage_x(const void *__restrict__ X, int M, int K
     }
     // largest magnitude of each column's slice: its 256 octets sit in the four wavefronts of one half of the workgroup
     const int half = tid >> 8, wih = (tid >> 6) & 3;
+    float *red_ss = red + 2 * ROUNDS * 4;
 #pragma unroll
     for (int r = 0; r < ROUNDS; r++) {
         const bool ok = k_ok && (m0 + half + 2 * (round0 + r) < M);
+        if (xss) {
+            const float ss = wave_sum(ok ? sumsq8(lo[r], hi[r]) : 0.f);
+            if ((tid & 63) == 0) red_ss[(half * ROUNDS + r) * 4 + wih] = ss;
+            if (gain) apply_gain8(gain, gain_offset, ksrc, lo[r], hi[r]);
+        }
         const float am = wave_max(ok ? amax8(lo[r], hi[r]) : 0.f);
         if ((tid & 63) == 0) red[(half * ROUNDS + r) * 4 + wih] = am;
     }
@@ -129,7 +154,13 @@ __device__ __forceinline__ void stage_x(const void *__restrict__ X, int M, int K
         const float *rr = red + (half * ROUNDS + r) * 4;
         float sc, inv;
         pow2_scale(fmaxf(fmaxf(rr[0], rr[1]), fmaxf(rr[2], rr[3])), sc, inv);
-        if (oct == 0 && m0 + m < M) inv_scale[m0 + m] = inv;
+        if (oct == 0 && m0 + m < M) {
+            inv_scale[m0 + m] = inv;
+            if (xss) {
+                const float *rs = red_ss + (half * ROUNDS + r) * 4;
+                xss[m0 + m] = (rs[0] + rs[1]) + (rs[2] + rs[3]);
+            }
+        }
         if (!active) continue;
         const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
         float4 a = ok ? lo[r] : z, b = ok ? hi[r] : z;
@@ -170,12 +201,13 @@ __device__ unsigned long long g_mmq_trace[4096 * 8];
 // xscale[slice][M]: the inverse of the power of two that (slice, column) was scaled by.
 template <bool BF16X>
 __global__ __launch_bounds__(512) void mmq_xprep_kernel(const void *__restrict__ X, uint8_t *__restrict__ ximg, float *__restrict__ xscale, int M,
-                                                        int K, int slice_sb) {
-    __shared__ float red[2 * 2 * 4];
+                                                        int K, int slice_sb, const float *__restrict__ gain, float gain_offset,
+                                                        float *__restrict__ xss) {
+    __shared__ float red[2 * 2 * 2 * 4];
     const int slice = blockIdx.x, mt = blockIdx.y;
     const bool active = (((int)threadIdx.x & 255) >> 5) < slice_sb;
     stage_x<2, BF16X>(X, M, K, mt * kMT, slice * slice_sb * 256, ximg + ((size_t)mt * gridDim.x + slice) * kLdsBytes, threadIdx.x,
-                      2 * blockIdx.z, active, red, xscale + (size_t)slice * M);
+                      2 * blockIdx.z, active, red, xscale + (size_t)slice * M, gain, gain_offset, xss ? xss + (size_t)slice * M : nullptr);
 }
 
 // partial[slice][m][n] = sum over the slice's k of x[m][k] * w[n][k]
@@ -319,7 +351,8 @@ __global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__
 // xscale[slice][M]: factor of each slice's partial sums of row m (the activations of a slice were scaled by its inverse).
 __global__ __launch_bounds__(256) void mmq_reduce_kernel(const float *__restrict__ partial, const float *__restrict__ partial2, int nslices,
                                                          int64_t MN, int N, const float *__restrict__ bias, const float *__restrict__ bias2,
-                                                         int act, const float *residual, float *Y, const float *__restrict__ xscale) {
+                                                         int act, const float *residual, float *Y, const float *__restrict__ xscale,
+                                                         const float *__restrict__ xss, float eps, float inv_k) {
     const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= MN) return;
     const bool small = MN <= (int64_t)INT32_MAX;  // (32-bit divisions are a fraction of the cost of 64-bit ones)
@@ -327,23 +360,31 @@ __global__ __launch_bounds__(256) void mmq_reduce_kernel(const float *__restrict
     const int m = small ? (int)((uint32_t)i / (uint32_t)N) : (int)(i / N);
     // Slices are added in order, eight at a time: their loads (each a trip to another XCD's freshly written
     // lines) are all issued before the first sum needs one; a slice past the end re-reads the last and is not added.
+    // xss: the activations carry an RMS normalisation whose 1 / sqrt(mean(x^2) + eps) is applied here, to the finished sums.
     auto total = [&](const float *p, const float *b) {
         float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+        float ss = 0.f;
         for (int k0 = 0; k0 < nslices; k0 += 8) {
             float4 v[8];
-            float f[8];
+            float f[8], q[8];
 #pragma unroll
             for (int j = 0; j < 8; j++) {
                 const int k = min(k0 + j, nslices - 1);
                 v[j] = *reinterpret_cast<const float4 *>(p + (int64_t)k * MN + i);
                 f[j] = xscale[(int64_t)k * M + m];
+                q[j] = xss ? xss[(int64_t)k * M + m] : 0.f;
             }
 #pragma unroll
             for (int j = 0; j < 8; j++) {
                 const bool in = k0 + j < nslices;
                 s.x = in ? fmaf(v[j].x, f[j], s.x) : s.x; s.y = in ? fmaf(v[j].y, f[j], s.y) : s.y;
                 s.z = in ? fmaf(v[j].z, f[j], s.z) : s.z; s.w = in ? fmaf(v[j].w, f[j], s.w) : s.w;
+                ss = in ? ss + q[j] : ss;
             }
+        }
+        if (xss) {
+            const float r = sqrtf(ss * inv_k + eps);
+            s.x /= r; s.y /= r; s.z /= r; s.w /= r;
         }
         if (b) {
             const float4 v = *reinterpret_cast<const float4 *>(b + (int)(i % N));
@@ -364,13 +405,18 @@ __global__ __launch_bounds__(256) void mmq_reduce_kernel(const float *__restrict
     *reinterpret_cast<float4 *>(Y + i) = v;
 }
 
-int launch_mmq_reduce(const float *partial, const float *partial2, const float *xscale, int nslices, int64_t M, int64_t N, const float *bias,
-                      int act, float *y, const MmqExtra *ex, hipStream_t s) {
+// [xscale: nslices x M][xss: nslices x M] (the second only used with a normalisation)
+size_t mmq_scale_bytes(int nslices, int64_t M) { return ((size_t)2 * nslices * M * sizeof(float) + 255) & ~(size_t)255; }
+float *mmq_xss(const float *xscale, int nslices, int64_t M) { return const_cast<float *>(xscale) + (size_t)nslices * M; }
+
+int launch_mmq_reduce(const float *partial, const float *partial2, const float *xscale, int nslices, int64_t M, int64_t K, int64_t N,
+                      const float *bias, int act, float *y, const MmqExtra *ex, hipStream_t s) {
     const int64_t MN = M * N;
+    const RmsNorm *norm = ex ? ex->norm : nullptr;
     return launch(mmq_reduce_kernel, dim3((unsigned)((MN / 4 + 255) / 256)), dim3(256), 0, s, partial, partial2, nslices, MN, (int)N, bias,
-                  ex ? ex->bias2 : nullptr, act, ex ? ex->residual : nullptr, y, xscale);
+                  ex ? ex->bias2 : nullptr, act, ex ? ex->residual : nullptr, y, xscale, norm ? mmq_xss(xscale, nslices, M) : nullptr,
+                  norm ? norm->eps : 0.f, 1.0f / (float)K);
 }
-size_t mmq_scale_bytes(int nslices, int64_t M) { return ((size_t)nslices * M * sizeof(float) + 255) & ~(size_t)255; }
 
 
 // ---- small batches of the 32-value-block formats (Q8_0, Q4_0, IQ4_NL) --------------------------------------
@@ -472,13 +518,19 @@ template <int T> struct B32Geom {
 // inverse factors.  grid = column tiles x slices x 4.
 template <bool BF16X>
 __global__ __launch_bounds__(256) void mmq_b32_xprep_kernel(const void *__restrict__ X, uint8_t *__restrict__ ximg, float *__restrict__ xscale,
-                                                            int M, int K, int S, int nslices) {
+                                                            int M, int K, int S, int nslices, const float *__restrict__ gain, float gain_offset,
+                                                            float *__restrict__ xss) {
     __shared__ uint32_t red[8];
+    __shared__ float red_ss[8][2];  // a column's slice is one or two wavefronts' worth of octets
     const int tid = threadIdx.x;
     const int rg = (int)blockIdx.x & 3, ts = (int)blockIdx.x >> 2;
     const int slice = ts % nslices, mt = ts / nslices;
     const int opers = S / 8, its = S / 256;  // octets per column and slice; items per thread
-    if (tid < 8) red[tid] = 0u;
+    if (tid < 8) {
+        red[tid] = 0u;
+        red_ss[tid][0] = 0.f;
+        red_ss[tid][1] = 0.f;
+    }
     __syncthreads();
     float4 a[4], b[4];
 #pragma unroll
@@ -488,7 +540,13 @@ __global__ __launch_bounds__(256) void mmq_b32_xprep_kernel(const void *__restri
         if (it < its) {
             const int j = it * 256 + tid, c = j / opers, oct = j - c * opers;
             const int k = slice * S + oct * 8, row = mt * kMT + rg * 8 + c;
-            if (row < M && k < K) load_x8<BF16X>(X, (int64_t)row * K + k, a[it], b[it]);  // K % 32 == 0: an octet is inside or outside as a whole
+            const bool ok = row < M && k < K;  // K % 32 == 0: an octet is inside or outside as a whole
+            if (ok) load_x8<BF16X>(X, (int64_t)row * K + k, a[it], b[it]);
+            if (xss) {
+                const float ss = wave_sum(sumsq8(a[it], b[it]));
+                if ((tid & 63) == 0) red_ss[c][(oct >> 6) & 1] = ss;
+                if (gain && ok) apply_gain8(gain, gain_offset, k, a[it], b[it]);
+            }
             const float am = wave_max(amax8(a[it], b[it]));  // a wavefront's 64 octets belong to one column
             if ((tid & 63) == 0) atomicMax(&red[c], __builtin_bit_cast(uint32_t, am));  // (non-negative floats order like their bits)
         }
@@ -501,7 +559,10 @@ __global__ __launch_bounds__(256) void mmq_b32_xprep_kernel(const void *__restri
             const int m = rg * 8 + c, row = mt * kMT + m;
             float sc, inv;
             pow2_scale(__builtin_bit_cast(float, red[c]), sc, inv);
-            if (oct == 0 && row < M) xscale[(size_t)slice * M + row] = inv;
+            if (oct == 0 && row < M) {
+                xscale[(size_t)slice * M + row] = inv;
+                if (xss) xss[(size_t)slice * M + row] = red_ss[c][0] + red_ss[c][1];
+            }
             const float4 p = a[it], q = b[it];
             const size_t g = (((size_t)mt * nslices + slice) * opers + oct) * 32 + m;
             reinterpret_cast<uint4 *>(ximg)[g] = make_uint4(pack_h2(p.x * sc, p.z * sc), pack_h2(p.y * sc, p.w * sc), pack_h2(q.x * sc, q.z * sc),
@@ -624,6 +685,7 @@ template <int T, int RT>
 int launch_mmq_b32(const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y, hipStream_t s,
                    const MmqExtra *ex) {
     const uint8_t *W2 = ex ? ex->W2 : nullptr;
+    const RmsNorm *norm = ex ? ex->norm : nullptr;
     const int cus = device_cu_count();
     const int mtiles = (int)((M + kMT - 1) / kMT);
     const int64_t rowwgs = (N + 32 * RT - 1) / (32 * RT);
@@ -648,8 +710,9 @@ int launch_mmq_b32(const void *x, bool x_is_bf16, int64_t M, int64_t K, const ui
     float *partial = reinterpret_cast<float *>(ximg + img_bytes + mmq_scale_bytes(nslices, M));
     const int64_t row_bytes = (K / 32) * B32<T>::kBlockBytes;
     const dim3 xgrid((unsigned)(mtiles * nslices * 4));
-    if (int rc = x_is_bf16 ? launch(mmq_b32_xprep_kernel<true>, xgrid, dim3(256), 0, s, x, ximg, xscale, (int)M, (int)K, S, nslices)
-                           : launch(mmq_b32_xprep_kernel<false>, xgrid, dim3(256), 0, s, x, ximg, xscale, (int)M, (int)K, S, nslices))
+    if (int rc = x_is_bf16 ? launch(mmq_b32_xprep_kernel<true>, xgrid, dim3(256), 0, s, x, ximg, xscale, (int)M, (int)K, S, nslices, nullptr, 0.f, nullptr)
+                           : launch(mmq_b32_xprep_kernel<false>, xgrid, dim3(256), 0, s, x, ximg, xscale, (int)M, (int)K, S, nslices, norm ? norm->gain : nullptr,
+                                    norm ? norm->gain_offset : 0.f, norm ? mmq_xss(xscale, nslices, M) : nullptr))
         return rc;
     const dim3 grid((unsigned)rowwgs, (unsigned)nslices, (unsigned)mtiles);
     if (int rc = launch(mmq_b32_kernel<T, RT>, grid, dim3(RT * 128), lds_bytes, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N, row_bytes, S))
@@ -659,7 +722,7 @@ int launch_mmq_b32(const void *x, bool x_is_bf16, int64_t M, int64_t K, const ui
         if (int rc = launch(mmq_b32_kernel<T, RT>, grid, dim3(RT * 128), lds_bytes, s, (const uint8_t *)ximg, W2, partial2, (int)M, (int)K, (int)N,
                             row_bytes, S))
             return rc;
-    return launch_mmq_reduce(partial, partial2, xscale, nslices, M, N, bias, act, y, ex, s);
+    return launch_mmq_reduce(partial, partial2, xscale, nslices, M, K, N, bias, act, y, ex, s);
 }
 
 
@@ -814,6 +877,7 @@ int launch_mmq_q6k(const MmqExtra *ex, const void *x, bool x_is_bf16, int64_t M,
     const int nslices = (int)((K + kQ6Slice - 1) / kQ6Slice);
     // workspace: [activation images: mtiles x nslices x 64 KiB][partial sums: nslices x M x N fp32, twice for a gated pair]
     const uint8_t *W2 = ex ? ex->W2 : nullptr;
+    const RmsNorm *norm = ex ? ex->norm : nullptr;
     const size_t img_bytes = (size_t)mtiles * nslices * kQ6Slice * 64;
     const size_t part_bytes = (size_t)nslices * M * N * sizeof(float);
     void *ws = nullptr;
@@ -823,8 +887,9 @@ int launch_mmq_q6k(const MmqExtra *ex, const void *x, bool x_is_bf16, int64_t M,
     float *partial = reinterpret_cast<float *>(ximg + img_bytes + mmq_scale_bytes(nslices, M));
     const int64_t row_bytes = (K / 256) * 210;
     const dim3 xgrid((unsigned)(mtiles * nslices * 4));
-    if (int rc = x_is_bf16 ? launch(mmq_b32_xprep_kernel<true>, xgrid, dim3(256), 0, s, x, ximg, xscale, (int)M, (int)K, kQ6Slice, nslices)
-                           : launch(mmq_b32_xprep_kernel<false>, xgrid, dim3(256), 0, s, x, ximg, xscale, (int)M, (int)K, kQ6Slice, nslices))
+    if (int rc = x_is_bf16 ? launch(mmq_b32_xprep_kernel<true>, xgrid, dim3(256), 0, s, x, ximg, xscale, (int)M, (int)K, kQ6Slice, nslices, nullptr, 0.f, nullptr)
+                           : launch(mmq_b32_xprep_kernel<false>, xgrid, dim3(256), 0, s, x, ximg, xscale, (int)M, (int)K, kQ6Slice, nslices, norm ? norm->gain : nullptr,
+                                    norm ? norm->gain_offset : 0.f, norm ? mmq_xss(xscale, nslices, M) : nullptr))
         return rc;
     const dim3 grid((unsigned)((N + 32 * kQ6RT - 1) / (32 * kQ6RT)), (unsigned)nslices, (unsigned)mtiles);
     if (int rc = launch(mmq_q6k_kernel, grid, dim3(kQ6RT * 128), (size_t)kLds, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N,
@@ -835,7 +900,7 @@ int launch_mmq_q6k(const MmqExtra *ex, const void *x, bool x_is_bf16, int64_t M,
         if (int rc = launch(mmq_q6k_kernel, grid, dim3(kQ6RT * 128), (size_t)kLds, s, (const uint8_t *)ximg, W2, partial2, (int)M, (int)K, (int)N,
                             row_bytes))
             return rc;
-    return launch_mmq_reduce(partial, partial2, xscale, nslices, M, N, bias, act, y, ex, s);
+    return launch_mmq_reduce(partial, partial2, xscale, nslices, M, K, N, bias, act, y, ex, s);
 }
 
 }  // namespace
@@ -881,10 +946,12 @@ int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, co
     float *xscale = reinterpret_cast<float *>(ximg + img_bytes);
     float *partial = reinterpret_cast<float *>(ximg + img_bytes + mmq_scale_bytes(nslices, M));
     const int64_t row_bytes = (K / 256) * 144;
+    const RmsNorm *norm = ex ? ex->norm : nullptr;
     if (int rc = x_is_bf16 ? launch(mmq_xprep_kernel<true>, dim3((unsigned)nslices, (unsigned)mtiles, 8), dim3(512), 0, s, x, ximg, xscale, (int)M,
-                                    (int)K, slice_sb)
+                                    (int)K, slice_sb, nullptr, 0.f, nullptr)
                            : launch(mmq_xprep_kernel<false>, dim3((unsigned)nslices, (unsigned)mtiles, 8), dim3(512), 0, s, x, ximg, xscale, (int)M,
-                                    (int)K, slice_sb))
+                                    (int)K, slice_sb, norm ? norm->gain : nullptr, norm ? norm->gain_offset : 0.f,
+                                    norm ? mmq_xss(xscale, nslices, M) : nullptr))
         return rc;
     const dim3 grid((unsigned)((N + kRowsPerWG - 1) / kRowsPerWG), (unsigned)nslices);
     float *partial2 = W2 ? partial + (size_t)nslices * M * N : nullptr;
@@ -894,7 +961,7 @@ int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, co
                                 which ? partial2 : partial, (int)M, (int)K, (int)N, row_bytes, (int)m0, slice_sb))
                 return rc;
         }
-    return launch_mmq_reduce(partial, partial2, xscale, nslices, M, N, bias, act, y, ex, s);
+    return launch_mmq_reduce(partial, partial2, xscale, nslices, M, K, N, bias, act, y, ex, s);
 }
 
 }  // namespace gq

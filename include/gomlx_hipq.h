@@ -146,9 +146,10 @@ typedef struct {
  * NULL (both NULL is plain gq_qdense_f32); dY may be dResidual itself (a residual stream updated
  * in place).  Small batches (a few rows; up to 16 where the split-K kernels do not apply) run in
  * the decode GEMV itself when K is a multiple of 256 and x and gain are 16-byte aligned; large batches (those a plain call hands to the two-pass GEMM) fold the
- * normalisation into the activation pass and the residual into the GEMM epilogue; what is left
- * is composed of an RMSNorm kernel, the dense call and an addition.  All but the first use a
- * per-stream workspace. */
+ * normalisation into the activation pass and the residual into the GEMM epilogue; the batches in
+ * between (split-K kernels) apply the gain where their activation image is written and the
+ * division and the residual in their reduction; what is left is composed of an RMSNorm kernel,
+ * the dense call and an addition.  All but the first use a per-stream workspace. */
 int gq_qdense_block_f32(int type, const float *dX, int64_t M, int64_t K, const gq_rmsnorm *norm,
                         const void *dW, int64_t N, const float *dBias, int act,
                         const float *dResidual, float *dY, void *stream);

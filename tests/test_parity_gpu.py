@@ -640,6 +640,41 @@ def test_dense_with_rmsnorm_and_residual(gpu, oracle, t):
 
 
 @pytest.mark.parametrize("t", ALL_TYPES)
+def test_split_k_batches_carry_the_normalisation(gpu, oracle, t):
+    """In the split-K range the gain is applied where the activation image is written and the division by the root
+    mean square in the reduction over K-slices (one to sixteen slices here): with and without gain, with a gain
+    offset, a large epsilon, a residual, the gated product, and a gain whose address is not 16-byte aligned (which
+    takes the separate normalisation kernel)."""
+    q = Quantization(ggml_type=t)
+    cases = [(17, 512, 132, 1, 1e-6, 0.0, True, False), (33, 1024, 512, 0, 1e-2, 0.0, False, False), (96, 2560, 64, 1, 1e-5, 1.0, True, False),
+             (20, 4096, 260, 1, 1e-6, 0.0, False, True), (64, 8192, 36, 2, 1e-6, 0.0, True, False), (24, 1536, 128, 1, 1e-5, 1.0, False, True)]
+    for i, (M, K, N, gain_kind, eps, off, use_res, gated) in enumerate(cases):
+        x = (synth.activations(771 + i, M, K) * 4.0).astype(np.float32)
+        gain = (synth.normal(772 + i, 0, K + 1) * 0.5 + 1.0 - off).astype(np.float32)
+        gd = dev(gpu, gain)
+        g_host, g_dev = (None, None) if gain_kind == 0 else (gain[:K], gd[:K]) if gain_kind == 1 else (gain[1:], gd[1:])
+        cfg = nn.RMSNorm(g_dev, eps, off)
+        xn = oracle.c_rmsnorm(x, g_host, eps, off)
+        W = synth.weights(t, 773 + i, N, K)
+        bias = synth.normal(774 + i, 0, N).astype(np.float32) * 0.1
+        if gated:
+            W2 = synth.weights(t, 775 + i, N, K)
+            got = nn.gated_feed_forward(dev(gpu, x), dev(gpu, W), dev(gpu, W2), q, Activation.SILU, dev(gpu, bias), None, norm=cfg).cpu().numpy()
+            gate, up = oracle.c_qdense(t, xn, W, bias, 0), oracle.c_qdense(t, xn, W2, None, 0)
+            want = oracle.c_qdense(t, xn, W, bias, 3).astype(np.float64) * up
+            err = float(np.max(np.abs(got - want))) / (float(np.max(np.abs(gate))) * float(np.max(np.abs(up))))
+            assert err < 2 * TOL_F32, ("gated", t, M, K, N, err)
+            continue
+        res = synth.activations(776 + i, M, N)
+        got = nn.quantized_dense(dev(gpu, x), dev(gpu, W), q, dev(gpu, bias), Activation.NONE, norm=cfg,
+                                 residual=dev(gpu, res) if use_res else None).cpu().numpy()
+        dense = oracle.c_qdense(t, xn, W, bias, 0)
+        want = dense + res if use_res else dense
+        err = float(np.max(np.abs(got.astype(np.float64) - want))) / float(np.max(np.abs(dense)))
+        assert err < TOL_F32, (t, M, K, N, gain_kind, eps, off, use_res, err)
+
+
+@pytest.mark.parametrize("t", ALL_TYPES)
 def test_batched_projections_behind_one_norm(gpu, oracle, t):
     """q/k/v of a layer: three batch-1 projections of one normalised input in one launch; a list that
     cannot be merged (a batch of 3 rows among them) gives the same results through separate calls."""
