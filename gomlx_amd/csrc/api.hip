@@ -146,7 +146,26 @@ int64_t split_k_from(int type, int64_t weight_bytes) {
     }
 }
 int64_t weight_bytes_of(int type, int64_t K, int64_t N) { return (int64_t)gq_row_bytes(type, K) * N; }
-int64_t split_k_to(int type) { return type == GQ_Q6_K ? 32 : 96; }
+// Last batch size of the split-K kernels before the two-pass GEMM takes over.  The split-K route streams W once per 32
+// batch rows; the two passes pay the 16-bit image (in proportion to N K) and a GEMM that, below a few hundred rows, has
+// only N / 64 workgroups walking all of K: cheap for a small matrix, costly for a long-K one (the down projection).
+// Measured (us per call in a replayed graph; rows 32 64 96 128 160 192 256; split-K | two passes, flat up to 128 rows):
+//   Q8_0   4096x4096  17 22 27 29 35 37 44 | 38-40    4096x14336  33 52  71  85 102 119 148 | 62-65, 80 from 160    14336x4096  33 52  72  85 104 124 153 |  95-109
+//   Q4_0   4096x4096  15 19 25 27 33 34 41 | 38-41    4096x14336  27 42  56  66  81  94 120 | 60-64, 80 from 160    14336x4096  28 43  57  69  83  97 122 |  92-103
+//   Q4_K   4096x4096  15 23 31 39 46 50 64 | 38-41    4096x14336  21 34  47  58  71  85 108 | 65-70, 85 from 160    14336x4096  22 35  49  61  74  87 113 |  98-108
+//   Q6_K   4096x4096  18 26 34 42 49 57 71 | 37-41    4096x14336  46 72 103 128 160 184 241 | 64-69, 86 from 160    14336x4096  46 71 101 126 156 183 240 |  96-109
+//   IQ4_NL 4096x4096  16 21 27 29 36 38 45 | 40-42    4096x14336  30 47  64  75  92 108 137 | 68-75, 89 from 160    14336x4096  30 47  64  78  94 110 141 | 100-111
+int64_t split_k_to(int type, int64_t K, int64_t N) {
+    const bool large = weight_bytes_of(type, K, N) >= kLargeWeightBytes, long_k = K > N;
+    switch (type) {
+    case GQ_Q8_0: return !large ? 192 : long_k ? 160 : 64;
+    case GQ_Q4_0: return !large ? 192 : long_k ? 192 : 96;
+    case GQ_Q4_K: return !large ? 128 : long_k ? 192 : 160;
+    case GQ_Q6_K: return !large ? 96 : long_k ? 64 : 32;
+    case GQ_IQ4_NL: return !large ? 192 : long_k ? 160 : 96;
+    default: return 96;
+    }
+}
 
 // large batches: W dequantised once into the stream's workspace, then a plain 16-bit GEMM
 int two_pass(int type, bool x_is_bf16, const void *x, int64_t M, int64_t K, const void *W, int64_t N, const float *bias, int act,
@@ -322,7 +341,7 @@ int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *d
     const bool tp = gemm_two_pass_supported(type, false, M, K, N, dX);
     const bool ks = M <= kGemvMaxRows && gemv_ks_supported(type, K, N, dX);
     const bool sk = M >= split_k_from(type, weight_bytes_of(type, K, N)) && mmq_supported(type, M, K, N, dX, dBias, dY) &&
-                    (M <= split_k_to(type) || !tp);
+                    (M <= split_k_to(type, K, N) || !tp);
     if (ks && !sk) return launch_gemv_ks(type, dX, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
     if (sk) return launch_mmq(type, dX, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
     // Shapes without a K-sliced plan (K not a multiple of 256: rare in models): a pass over W per row for up to 16
@@ -386,7 +405,7 @@ int gq_qdense_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, const voi
     const bool tp = gemm_two_pass_supported(type, true, M, K, N, dX);
     const bool ks = M <= kGemvMaxRows && gemv_ks_supported(type, K, N, dX);
     const bool sk = M >= split_k_from(type, weight_bytes_of(type, K, N)) && mmq_supported(type, M, K, N, dX, dBias, dY) &&
-                    (M <= split_k_to(type) || !tp);
+                    (M <= split_k_to(type, K, N) || !tp);
     if (ks && !sk) return launch_gemv_ks(type, dX, true, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
     if (sk) return launch_mmq(type, dX, true, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
     if (tp) return two_pass(type, true, dX, M, K, dW, N, dBias, act, dY, (hipStream_t)stream);
@@ -424,7 +443,7 @@ bool fold_into_gemv(int type, int64_t M, int64_t K, int64_t N, const float *x, c
 // Whether a plain dense call on these operands runs on the split-K kernels (the dispatch of gq_qdense_f32).
 bool dense_takes_split_k(int type, int64_t M, int64_t K, int64_t N, const float *x, const float *bias, const float *y) {
     const bool tp = gemm_two_pass_supported(type, false, M, K, N, x);
-    return M >= split_k_from(type, weight_bytes_of(type, K, N)) && mmq_supported(type, M, K, N, x, bias, y) && (M <= split_k_to(type) || !tp);
+    return M >= split_k_from(type, weight_bytes_of(type, K, N)) && mmq_supported(type, M, K, N, x, bias, y) && (M <= split_k_to(type, K, N) || !tp);
 }
 
 // Batches that a plain dense call would hand to the two-pass GEMM take its block form: the
@@ -436,7 +455,7 @@ bool block_takes_two_pass(int type, int64_t M, int64_t K, int64_t N, const float
     // 660 against 743 us at 2048; at 128 rows, where dequantising the two matrices dominates, 147 against 132 us).
     if (gated && M < 256) return false;
     if (gain && !aligned_to(gain, 16)) return false;
-    const bool sk = M >= split_k_from(type, weight_bytes_of(type, K, N)) && mmq_supported(type, M, K, N, x, bias, y) && M <= split_k_to(type);
+    const bool sk = M >= split_k_from(type, weight_bytes_of(type, K, N)) && mmq_supported(type, M, K, N, x, bias, y) && M <= split_k_to(type, K, N);
     return !sk;
 }
 }  // namespace

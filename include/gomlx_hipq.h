@@ -94,18 +94,18 @@ int gq_dequantize(int type, const void *dW, int64_t N, int64_t K, float *dOut, v
 /* ---- compute.Function.FusedQuantizedDense (core/graph/fused_ops.go:231-232), run time:
  * y = act(x . dequant(W)^T + bias), the contract of nn.QuantizedDense
  * (ml/nn/quantized_dense.go:31-57) and ggml.DenseDecomposed (ml/ggml/dense.go:23-62).
- * dBias may be NULL.  fp32 activations, fp32 accumulation.  The first few rows (4 to 8, depending
- * on format and matrix size) run as bandwidth-bound GEMV passes; larger batches contract on the
- * matrix cores with the activations (and, from 97 rows on, the dequantised weights) rounded to
- * fp16 operands (each batch row scaled by a power of two first, so the magnitude of x does not
+ * dBias may be NULL.  fp32 activations, fp32 accumulation.  The first few rows (4 to 6, depending
+ * on format and matrix size; 16 for matrices of a few megabytes) run as bandwidth-bound GEMV
+ * passes; larger batches contract on the matrix cores with the activations (and, from 65 to 193
+ * rows on, depending on format and shape, the dequantised weights) rounded to fp16 operands (each batch row scaled by a power of two first, so the magnitude of x does not
  * matter).  Batches of 5 rows and more may use a
  * per-stream workspace that is created on the first such call on the stream: make
  * one call outside a recording (gq_graph_begin) before recording the same call. ---- */
 int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *dW, int64_t N,
                   const float *dBias, int act, float *dY, void *stream);
 /* bf16 activations (raw 16-bit patterns), fp32 output.  Small batches widen the activations
- * exactly and take the same GEMV / split-K kernels as fp32 activations; from 97 rows on the
- * weights are dequantised to bf16 operands and contracted on bf16 MFMA with fp32 accumulation. */
+ * exactly and take the same GEMV / split-K kernels as fp32 activations; beyond those batch
+ * sizes the weights are dequantised to bf16 operands and contracted on bf16 MFMA with fp32 accumulation. */
 int gq_qdense_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, const void *dW,
                    int64_t N, const float *dBias, int act, float *dY, void *stream);
 

@@ -194,7 +194,7 @@ def test_small_batches_f32(gpu, oracle, t, M):
     (8, 1024, 36),
 ])
 def test_split_k_small_batches_q8_q4(gpu, oracle, t, M, K, N):
-    """8 .. 96 rows of Q8_0 / Q4_0 / IQ4_NL (N a multiple of 4, K of 256): the split-K MFMA kernel
+    """8 .. 96 rows (the range extends to 192 by shape) of Q8_0 / Q4_0 / IQ4_NL (N a multiple of 4, K of 256): the split-K MFMA kernel
     with exact integer weight operands; x -> fp16 is its only rounding."""
     W = synth.weights(t, 70 + t, N, K)
     x = synth.activations(71 + t, M, K)
@@ -208,6 +208,20 @@ def test_split_k_small_batches_q8_q4(gpu, oracle, t, M, K, N):
     xb = bf16_round(x)
     tol = TOL_F32 if K % 256 == 0 else TOL_BF16
     assert rel_err(run_dense(gpu, t, xb, W, bias, 0, bf16=True), oracle.c_qdense(t, xb, W, bias, 0)) < tol, (t, M, K, N, "bf16")
+
+
+@pytest.mark.parametrize("t,M,K,N", [(Q8_0, 192, 1024, 256), (Q4_0, 160, 2048, 132), (Q4_0, 97, 4096, 64), (Q4_K, 128, 1024, 260),
+                                     (Q4_K, 100, 2048, 36), (Q6_K, 96, 1024, 64), (Q6_K, 70, 2560, 128), (IQ4_NL, 192, 512, 128)])
+def test_split_k_up_to_six_tiles_of_batch_rows(gpu, oracle, t, M, K, N):
+    """Where the two-pass GEMM is the dearer route (small and long-K matrices) the split-K kernels serve up to 192 rows:
+    several tiles of 32 batch rows, the last one partly filled."""
+    W = synth.weights(t, 170 + t, N, K)
+    x = (synth.activations(171 + t, M, K) * np.logspace(-3, 3, M, dtype=np.float32)[:, None]).astype(np.float32)
+    bias = synth.normal(172 + t, 0, N).astype(np.float32) * 0.1
+    got = run_dense(gpu, t, x, W, bias, 0)
+    want = oracle.c_qdense(t, x, W, bias, 0)
+    per_row = np.max(np.abs(got.astype(np.float64) - want), axis=1) / np.max(np.abs(want), axis=1)
+    assert np.all(per_row < TOL_F32), (t, M, K, N, float(per_row.max()))
 
 
 @pytest.mark.parametrize("t", [Q4_K, Q6_K])
