@@ -46,7 +46,7 @@ _KIB, _FETCH_SCALE, _WRITE_SCALE = 1024, 65536.0 / 32780.5, 1.0
 COUNTER_KIB = {  # workload -> (FETCH_SIZE, WRITE_SIZE) raw counter KiB per step
     "c0": (8811.9, 16.0),
     "c1": (16262.6, 56.0),
-    "c2": (19875.6 + 1864.5 + 920.1, 3584.0 + 512.0 + 925.8),
+    "c2": (19871.1 + 1867.0 + 928.1, 3584.0 + 512.0 + 925.8),
     "c3": (74726.7, 32768.0),
     "c4": (60543.5, 168.0),
     "prefill": (4628.9 + 24121.3 + 82460.4, 32768.0 + 16448.9 + 32768.0),
