@@ -49,7 +49,7 @@ COUNTER_KIB = {  # workload -> (FETCH_SIZE, WRITE_SIZE) raw counter KiB per step
     "c2": (19871.1 + 1867.0 + 928.1, 3584.0 + 512.0 + 925.8),
     "c3": (74726.7, 32768.0),
     "c4": (60543.5, 168.0),
-    "prefill": (4628.9 + 24121.3 + 82460.4, 32768.0 + 16448.9 + 32768.0),
+    "prefill": (4628.9 + 24154.3 + 82460.9, 32768.0 + 16449.3 + 32768.0),
     "ffn": (32484.0, 56.0),
     "layer": (7126.2 + 4756.1 + 32483.6 + 16449.7, 24.0 + 16.0 + 56.0 + 16.0),
 }
