@@ -158,6 +158,84 @@ __global__ __launch_bounds__(256) void x_rmsnorm_to_f16_kernel(const float *__re
     }
 }
 
+// Both activation passes for rows of at most 2048 IT values: the row stays in registers between the reduction and
+// the conversion, so it is read once.  NORM: the RMS normalisation variant.
+template <int IT, bool NORM>
+__global__ __launch_bounds__(256) void x_row_to_f16_kernel(const float *__restrict__ X, const float *__restrict__ gain, float gain_offset, float eps,
+                                                           int K, uint16_t *__restrict__ out, float *__restrict__ rowscale) {
+    __shared__ float part[4];
+    const float4 *x = reinterpret_cast<const float4 *>(X + (int64_t)blockIdx.x * K);
+    const int k8 = K / 8, kp8 = (int)(padded_k(K) / 8);
+    float4 a[IT], b[IT];
+#pragma unroll
+    for (int i = 0; i < IT; i++) {  // (groups past the row re-read its last one: no branch around the loads)
+        const int g = min((int)threadIdx.x + 256 * i, k8 - 1);
+        a[i] = x[2 * g];
+        b[i] = x[2 * g + 1];
+    }
+    float red = 0.f;
+#pragma unroll
+    for (int i = 0; i < IT; i++) {
+        if ((int)threadIdx.x + 256 * i >= k8) continue;
+        if constexpr (NORM)
+            red += (a[i].x * a[i].x + a[i].y * a[i].y) + (a[i].z * a[i].z + a[i].w * a[i].w) + (b[i].x * b[i].x + b[i].y * b[i].y) +
+                   (b[i].z * b[i].z + b[i].w * b[i].w);
+        else
+            red = fmaxf(red, amax8(a[i], b[i]));
+    }
+    if constexpr (NORM) {
+        for (int m = 1; m < 64; m <<= 1) red += __shfl_xor(red, m);
+    } else {
+        red = wave_max(red);
+    }
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = red;
+    __syncthreads();
+    float sc = 1.f, r = 1.f;
+    if constexpr (NORM) {
+        r = sqrtf(((part[0] + part[1]) + (part[2] + part[3])) / (float)K + eps);
+        if (threadIdx.x == 0) rowscale[blockIdx.x] = 1.f;  // normalised rows are O(gain): no scaling
+    } else {
+        float inv;
+        pow2_scale(fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3])), sc, inv);
+        if (threadIdx.x == 0) rowscale[blockIdx.x] = inv;
+    }
+    uint4 *o = reinterpret_cast<uint4 *>(out + (int64_t)blockIdx.x * (kp8 * 8));
+#pragma unroll
+    for (int i = 0; i < IT; i++) {
+        const int g = (int)threadIdx.x + 256 * i;
+        if (g >= kp8) continue;
+        if (g >= k8) { o[g] = make_uint4(0u, 0u, 0u, 0u); continue; }
+        float4 p = a[i], q = b[i];
+        if constexpr (NORM) {
+            p.x /= r; p.y /= r; p.z /= r; p.w /= r; q.x /= r; q.y /= r; q.z /= r; q.w /= r;
+            if (gain) {
+                const float4 ga = reinterpret_cast<const float4 *>(gain)[2 * g], gb = reinterpret_cast<const float4 *>(gain)[2 * g + 1];
+                p.x *= ga.x + gain_offset; p.y *= ga.y + gain_offset; p.z *= ga.z + gain_offset; p.w *= ga.w + gain_offset;
+                q.x *= gb.x + gain_offset; q.y *= gb.y + gain_offset; q.z *= gb.z + gain_offset; q.w *= gb.w + gain_offset;
+            }
+        } else {
+            p.x *= sc; p.y *= sc; p.z *= sc; p.w *= sc; q.x *= sc; q.y *= sc; q.z *= sc; q.w *= sc;
+        }
+        o[g] = make_uint4(Op16<false>::pack(p.x, p.y), Op16<false>::pack(p.z, p.w), Op16<false>::pack(q.x, q.y), Op16<false>::pack(q.z, q.w));
+    }
+}
+
+// x -> fp16 rows (+ row scales), with the normalisation when norm is given
+int launch_x_to_f16(const float *x, int64_t M, int64_t K, const RmsNorm *norm, uint16_t *xh, float *rowscale, hipStream_t s) {
+    const dim3 grid((unsigned)M), block(256);
+    const float *gain = norm ? norm->gain : nullptr;
+    const float off = norm ? norm->gain_offset : 0.f, eps = norm ? norm->eps : 0.f;
+    const int64_t kp = padded_k(K);
+    if (kp <= 4096)
+        return norm ? launch(x_row_to_f16_kernel<2, true>, grid, block, 0, s, x, gain, off, eps, (int)K, xh, rowscale)
+                    : launch(x_row_to_f16_kernel<2, false>, grid, block, 0, s, x, gain, off, eps, (int)K, xh, rowscale);
+    if (kp <= 8192)
+        return norm ? launch(x_row_to_f16_kernel<4, true>, grid, block, 0, s, x, gain, off, eps, (int)K, xh, rowscale)
+                    : launch(x_row_to_f16_kernel<4, false>, grid, block, 0, s, x, gain, off, eps, (int)K, xh, rowscale);
+    return norm ? launch(x_rmsnorm_to_f16_kernel, grid, block, 0, s, x, gain, off, eps, (int)K, xh, rowscale)
+                : launch(x_to_f16_kernel, grid, block, 0, s, x, (int)K, xh, rowscale);
+}
+
 // ---- pass 2: 16-bit GEMM with global -> LDS DMA --------------------------------------------------
 // One 16-byte-per-lane buffer load whose data goes to LDS at lds_addr + 16 * lane.  The compiler
 // does not see that the instruction writes LDS or that it is counted by vmcnt: the kernel orders
@@ -477,7 +555,7 @@ int launch_gemm_two_pass(int type, bool x_is_bf16, const void *x, int64_t M, int
     uint16_t *xh = wh + (((size_t)N * Kp * 2 + 255) & ~(size_t)255) / 2;
     float *rowscale = reinterpret_cast<float *>(xh + (((size_t)M * Kp * 2 + 255) & ~(size_t)255) / 2);
     if (int rc = launch_dequant16bit_type<false>(type, W, N, K, wh, s)) return rc;
-    if (int rc = launch(x_to_f16_kernel, dim3((unsigned)M), dim3(256), 0, s, static_cast<const float *>(x), (int)K, xh, rowscale)) return rc;
+    if (int rc = launch_x_to_f16(static_cast<const float *>(x), M, K, nullptr, xh, rowscale, s)) return rc;
     return launch_gemm16<false>(xh, M, Kp, wh, N, bias, act, y, s, nullptr, rowscale);
 }
 
@@ -504,13 +582,7 @@ int launch_gemm_two_pass_block(int type, const float *x, int64_t M, int64_t K, c
     const int64_t Kp = padded_k(K);
     uint16_t *xh = wh + (((size_t)rows * Kp * 2 + 255) & ~(size_t)255) / 2;
     float *rowscale = reinterpret_cast<float *>(xh + (((size_t)M * Kp * 2 + 255) & ~(size_t)255) / 2);
-    if (norm) {
-        if (int rc = launch(x_rmsnorm_to_f16_kernel, dim3((unsigned)M), dim3(256), 0, s, x, norm->gain, norm->gain_offset, norm->eps, (int)K, xh,
-                            rowscale))
-            return rc;
-    } else {
-        if (int rc = launch(x_to_f16_kernel, dim3((unsigned)M), dim3(256), 0, s, x, (int)K, xh, rowscale)) return rc;
-    }
+    if (int rc = launch_x_to_f16(x, M, K, norm, xh, rowscale, s)) return rc;
     if (!W2) {
         if (int rc = launch_dequant16bit_type<false>(type, W, N, K, wh, s)) return rc;
         return launch_gemm16<false>(xh, M, Kp, wh, N, bias, act, y, s, residual, rowscale);
