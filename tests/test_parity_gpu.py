@@ -238,6 +238,23 @@ def test_split_k_small_batches_k_quants(gpu, oracle, t, M, K, N):
     assert rel_err(run_dense(gpu, t, xb, W, bias, 3, bf16=True), oracle.c_qdense(t, xb, W, bias, 3)) < tol, (t, M, K, N, "bf16")
 
 
+@pytest.mark.parametrize("t", [Q6_K, Q4_K])
+def test_output_head_of_a_128k_vocabulary(gpu, oracle, t):
+    """The largest projection of a decoder: hidden state -> logits over 128 256 tokens (K = 4096; several hundred
+    megabytes of weights, row offsets beyond 2^28 bytes).  One row and a small batch, checked on a sample of 3000
+    output columns that includes the first and the last."""
+    K, N = 4096, 128256
+    W = synth.weights(t, 480 + t, N, K)
+    rng = np.random.default_rng(481)
+    cols = np.unique(np.concatenate([[0, 1, N - 2, N - 1], rng.integers(0, N, 3000)]))
+    for M in (1, 8, 40):
+        x = synth.activations(482 + M, M, K)
+        got = run_dense(gpu, t, x, W)
+        assert got.shape == (M, N) and np.all(np.isfinite(got))
+        want = oracle.c_qdense(t, x, np.ascontiguousarray(W[cols]))
+        assert rel_err(got[:, cols], want) < TOL_F32, (t, M)
+
+
 @pytest.mark.parametrize("t", ALL_TYPES)
 def test_gemv_long_k_is_chunked(gpu, oracle, t):
     """K above the 16384 values one LDS pass holds."""
