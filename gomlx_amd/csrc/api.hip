@@ -125,13 +125,13 @@ int check_dense_args(const char *fn, int type, const void *x, int64_t M, int64_t
 //          4096x1024 (2 MB)    4.2  4.8  4.8  5.5  5.6  6.2  6.3 | 12.1   14336x4096         19.4 25.2 28.1 34.8 33.0 40.1 43.2 | 24.7
 //   Q4_K   4096x4096          11.1 12.6 14.6 16.6 18.6 20.5 22.5 | 13.1   4096x14336         15.8 22.3 24.1 29.1 27.5 34.9 36.8 | 19.3
 //          4096x1024           4.4  5.4  6.2  6.4  6.5  7.4  8.0 | 12.3   14336x4096         20.4 26.9 29.8 36.7 35.0 42.7 46.0 | 19.6
-//   Q6_K   4096x4096 (14 MB)  13.5 15.3 17.6 19.9 22.3 24.6 27.0 | 17.0   4096x14336 (48 MB) 25.6 34.6 34.6 44.2 44.3 54.0 54.2 | 43.0
-//          4096x1024 (3 MB)    5.1  6.1  6.2  7.2  7.3  8.4  8.5 | 16.4   14336x4096         28.6 37.1 37.3 46.9 48.0 57.6 58.8 | 43.0
+//   Q6_K   4096x4096 (14 MB)  13.5 15.3 17.6 19.9 22.3 24.6 27.0 | 17.8   4096x14336 (48 MB) 25.6 34.6 34.6 44.2 44.3 54.0 54.2 | 33.0
+//          4096x1024 (3 MB)    5.1  6.1  6.2  7.2  7.3  8.4  8.5 | 16.4   14336x4096         28.6 37.1 37.3 46.9 48.0 57.6 58.8 | 34.0
 //   IQ4_NL 4096x4096          11.8 12.9 15.0 16.9 18.9 20.9 22.8 | 13.7   4096x14336         17.0 24.0 26.7 31.1 29.4 37.7 40.4 | 26.3
 //          4096x1024           4.8  5.7  5.7  6.6  6.7  7.6  7.7 | 12.8   14336x4096         20.9 28.6 31.1 37.7 35.9 45.0 47.8 | 27.2
 // The split-K route is three dependent launches with a floor of about 12 us: matrices of a few megabytes (the k / v
 // projections of a grouped-query layer) stay on GEMV passes for every batch the GEMV takes.
-// The Q6_K kernel pays 16 scale groups per super-block and only wins for a single tile of 32 batch columns.
+// (The Q6_K kernel pays 16 scale groups per super-block: twice the time of the others per byte.)
 constexpr int64_t kTinyWeightBytes = (int64_t)6 << 20;
 int64_t split_k_from(int type, int64_t weight_bytes) {
     if (weight_bytes < kTinyWeightBytes) return kGemvMaxRows + 1;
@@ -140,7 +140,7 @@ int64_t split_k_from(int type, int64_t weight_bytes) {
     case GQ_Q8_0: return 6;
     case GQ_Q4_0: return large ? 6 : 7;
     case GQ_Q4_K: return large ? 5 : 6;
-    case GQ_Q6_K: return large ? 7 : 6;
+    case GQ_Q6_K: return large ? 5 : 6;
     case GQ_IQ4_NL: return 6;
     default: return 8;
     }
@@ -153,7 +153,7 @@ int64_t weight_bytes_of(int type, int64_t K, int64_t N) { return (int64_t)gq_row
 //   Q8_0   4096x4096  17 22 27 29 35 37 44 | 38-40    4096x14336  33 52  71  85 102 119 148 | 62-65, 80 from 160    14336x4096  33 52  72  85 104 124 153 |  95-109
 //   Q4_0   4096x4096  15 19 25 27 33 34 41 | 38-41    4096x14336  27 42  56  66  81  94 120 | 60-64, 80 from 160    14336x4096  28 43  57  69  83  97 122 |  92-103
 //   Q4_K   4096x4096  15 23 31 39 46 50 64 | 38-41    4096x14336  21 34  47  58  71  85 108 | 65-70, 85 from 160    14336x4096  22 35  49  61  74  87 113 |  98-108
-//   Q6_K   4096x4096  18 26 34 42 49 57 71 | 37-41    4096x14336  46 72 103 128 160 184 241 | 64-69, 86 from 160    14336x4096  46 71 101 126 156 183 240 |  96-109
+//   Q6_K   4096x4096  19 22 30 33 41 41  - | 37-41    4096x14336  36 56  78  92 111 133   - | 64-67, 84 from 160    14336x4096  37 57  79  94 114 136   - |  96-109
 //   IQ4_NL 4096x4096  16 21 27 29 36 38 45 | 40-42    4096x14336  30 47  64  75  92 108 137 | 68-75, 89 from 160    14336x4096  30 47  64  78  94 110 141 | 100-111
 int64_t split_k_to(int type, int64_t K, int64_t N) {
     const bool large = weight_bytes_of(type, K, N) >= kLargeWeightBytes, long_k = K > N;
@@ -161,7 +161,7 @@ int64_t split_k_to(int type, int64_t K, int64_t N) {
     case GQ_Q8_0: return !large ? 192 : long_k ? 160 : 64;
     case GQ_Q4_0: return !large ? 192 : long_k ? 192 : 96;
     case GQ_Q4_K: return !large ? 128 : long_k ? 192 : 160;
-    case GQ_Q6_K: return !large ? 96 : long_k ? 64 : 32;
+    case GQ_Q6_K: return !large ? 128 : long_k ? 128 : 64;
     case GQ_IQ4_NL: return !large ? 192 : long_k ? 160 : 96;
     default: return 96;
     }

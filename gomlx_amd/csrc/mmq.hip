@@ -736,13 +736,17 @@ int launch_mmq_b32(const void *x, bool x_is_bf16, int64_t M, int64_t K, const ui
 // exactly one 16-value scale group: lane kg holds values 8 kg .. 8 kg + 7 of it, assembled from the
 // low nibbles / high bit pairs into bytes, turned into exact fp16 integers code - 32, and the
 // group's partial tile is scaled by d * sc in fp32.
-// Slices are 1024 values (two pairs: one per wavefront of a row tile); RT = 2 row tiles per
-// workgroup, so the 64 KiB activation image and four parked pairs fit LDS.
-constexpr int kQ6PairBytes = 420, kQ6PairDwords = 105;
-constexpr int kQ6Loads = (32 * kQ6PairDwords + 63) / 64;  // 53 dword loads per lane and pair (the last: half a wavefront)
-constexpr int kQ6WaveLds = 32 * kQ6PairBytes + 16;         // + slack for a window that ends past the last row
+// Slices are 1024 values (two pairs: one per wavefront of a row tile); RT = 4 row tiles per workgroup (2 for problems
+// that would not give every CU a workgroup otherwise).
+// A wavefront parks its pair one super-block at a time (dwords 0 .. 52 of the pair, then dwords 52 .. 104: the
+// second super-block starts 2 bytes into dword 52), so that the 64 KiB activation image and the parked halves of
+// EIGHT wavefronts fit LDS: with two wavefronts per SIMD one's arithmetic hides the other's LDS and memory waits
+// (four wavefronts parking whole pairs left every SIMD a single wavefront: 43 us on 4096 -> 14336 at 8 rows).
+constexpr int kQ6PairBytes = 420;
+constexpr int kQ6HalfDwords = 53, kQ6HalfBytes = 4 * kQ6HalfDwords;  // 212 bytes per row (odd dword stride: conflict-free)
+constexpr int kQ6Loads = (32 * kQ6HalfDwords + 63) / 64;  // 27 dword loads per lane and half (the last: half a wavefront)
+constexpr int kQ6WaveLds = 32 * kQ6HalfBytes + 16;         // + slack for a window that ends past the last row
 constexpr int kQ6Slice = 1024;
-constexpr int kQ6RT = 2;
 
 // two dwords holding the 8 bytes at byte offset `at` of the parked row (at % 4 is 0 or 2, known at compile time)
 __device__ __forceinline__ void q6_bytes8(const uint8_t *row, int at, uint32_t &a, uint32_t &b) {
@@ -757,43 +761,46 @@ __device__ __forceinline__ void q6_bytes8(const uint8_t *row, int at, uint32_t &
     }
 }
 
-// (Launched with kQ6RT * 128 threads.  Declared for up to 512: with a bound of 256 the compiler puts every MFMA
+// (Launched with RT * 128 threads, RT = 2 or 4 row tiles.  Declared for up to 512: with a bound of 256 the compiler puts every MFMA
 // result into accumulation registers and copies it back out, 16 extra instructions per MFMA.)
+template <int RT>
 __global__ __launch_bounds__(512) void mmq_q6k_kernel(const uint8_t *__restrict__ ximg, const uint8_t *__restrict__ W,
                                                               float *__restrict__ partial, int M, int K, int N, int64_t row_bytes) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int kg = lane >> 5, col = lane & 31;
-    const int rt = wave % kQ6RT, par = wave / kQ6RT;
+    const int rt = wave % RT, par = wave / RT;
     const int slice = blockIdx.y, nslices = gridDim.y, mt = blockIdx.z;
     constexpr int img_bytes = kQ6Slice * 64;
     const int kpairs = K >> 9;                                  // pairs of a row
-    const int n0 = (blockIdx.x * kQ6RT + rt) * 32;              // first W row of this wavefront's tile
+    const int n0 = (blockIdx.x * RT + rt) * 32;              // first W row of this wavefront's tile
     uint8_t *park = lds + img_bytes + wave * kQ6WaveLds;
 
     // the slice's activation image goes straight from global memory into LDS (no registers)
     {
         const uint8_t *img = ximg + ((size_t)mt * nslices + slice) * img_bytes;
-        for (int i = wave; i < img_bytes / 1024; i += 2 * kQ6RT)
+        for (int i = wave; i < img_bytes / 1024; i += 2 * RT)
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(img + i * 1024 + lane * 16),
                                              (__attribute__((address_space(3))) void *)(lds + i * 1024), 16, 0, 0);
     }
     // This wavefront's pair of the slice (a pair beyond K re-reads the row's last one: its activations
-    // are zero in the image).  Dword lane + 64 i of the pair tile is dword d % 105 of row d / 105.
-    {
-        const uint8_t *base = W + (int64_t)min(n0, N - 1) * row_bytes + (int64_t)min(2 * slice + par, kpairs - 1) * kQ6PairBytes;
-        const int rows_left = max(N - 1 - n0, 0);
+    // are zero in the image), one half at a time.  Dword lane + 64 i of a half tile is dword d % 53 of row d / 53.
+    const uint8_t *pair = W + (int64_t)min(n0, N - 1) * row_bytes + (int64_t)min(2 * slice + par, kpairs - 1) * kQ6PairBytes;
+    const int rows_left = max(N - 1 - n0, 0);
+    auto park_half = [&](int sbp) __attribute__((always_inline)) {
         uint32_t v[kQ6Loads];
 #pragma unroll
         for (int i = 0; i < kQ6Loads; i++) {
-            const int d = min(lane + 64 * i, 32 * kQ6PairDwords - 1);
-            v[i] = *reinterpret_cast<const uint32_t *>(base + (int64_t)min(d / kQ6PairDwords, rows_left) * row_bytes + (d % kQ6PairDwords) * 4);
+            const int d = min(lane + 64 * i, 32 * kQ6HalfDwords - 1);
+            v[i] = *reinterpret_cast<const uint32_t *>(pair + (int64_t)min(d / kQ6HalfDwords, rows_left) * row_bytes +
+                                                       (sbp * (kQ6HalfDwords - 1) + d % kQ6HalfDwords) * 4);
         }
 #pragma unroll
         for (int i = 0; i < kQ6Loads; i++)
-            if (lane + 64 * i < 32 * kQ6PairDwords) reinterpret_cast<uint32_t *>(park)[lane + 64 * i] = v[i];
-    }
-    __syncthreads();  // image landed; the parked pair is this wavefront's own
+            if (lane + 64 * i < 32 * kQ6HalfDwords) reinterpret_cast<uint32_t *>(park)[lane + 64 * i] = v[i];
+    };
+    park_half(0);
+    __syncthreads();  // image landed; the parked half is this wavefront's own
 
     f16v acc;
 #pragma unroll
@@ -801,10 +808,19 @@ __global__ __launch_bounds__(512) void mmq_q6k_kernel(const uint8_t *__restrict_
     uint32_t magic;
     asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));
     const h2 off = as_h2(0xE420E420u);  // (-1056, -1056) = -(1024 + 32)
-    const uint8_t *myrow = park + col * kQ6PairBytes;
+    const uint8_t *myrow = park + col * kQ6HalfBytes;
 #pragma unroll
     for (int sbp = 0; sbp < 2; sbp++) {
-        const int b0 = sbp * 210;                    // byte offset of the super-block in the parked row
+        if (sbp == 1) {
+            // (LDS operations of one wavefront execute in order; no other wavefront touches its parked half)
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            park_half(1);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        }
+        const int b0 = sbp * 2;                      // byte offset of the super-block in the parked row
         const int sbg = 2 * par + sbp;               // super-block within the slice
         const float d = half_bits_to_float(*reinterpret_cast<const uint16_t *>(myrow + b0 + 208));
 #pragma unroll
@@ -865,11 +881,12 @@ __global__ __launch_bounds__(512) void mmq_q6k_kernel(const uint8_t *__restrict_
     }
 }
 
-int launch_mmq_q6k(const MmqExtra *ex, const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y,
+template <int RT>
+int launch_mmq_q6k_rt(const MmqExtra *ex, const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y,
                    hipStream_t s) {
-    constexpr int kLds = kQ6Slice * 64 + 2 * kQ6RT * kQ6WaveLds;
+    constexpr int kLds = kQ6Slice * 64 + 2 * RT * kQ6WaveLds;
     static const bool lds_ok = [] {
-        return hipFuncSetAttribute(reinterpret_cast<const void *>(mmq_q6k_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLds) ==
+        return hipFuncSetAttribute(reinterpret_cast<const void *>(mmq_q6k_kernel<RT>), hipFuncAttributeMaxDynamicSharedMemorySize, kLds) ==
                hipSuccess;
     }();
     if (!lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", kLds);
@@ -891,16 +908,24 @@ int launch_mmq_q6k(const MmqExtra *ex, const void *x, bool x_is_bf16, int64_t M,
                            : launch(mmq_b32_xprep_kernel<false>, xgrid, dim3(256), 0, s, x, ximg, xscale, (int)M, (int)K, kQ6Slice, nslices, norm ? norm->gain : nullptr,
                                     norm ? norm->gain_offset : 0.f, norm ? mmq_xss(xscale, nslices, M) : nullptr))
         return rc;
-    const dim3 grid((unsigned)((N + 32 * kQ6RT - 1) / (32 * kQ6RT)), (unsigned)nslices, (unsigned)mtiles);
-    if (int rc = launch(mmq_q6k_kernel, grid, dim3(kQ6RT * 128), (size_t)kLds, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N,
+    const dim3 grid((unsigned)((N + 32 * RT - 1) / (32 * RT)), (unsigned)nslices, (unsigned)mtiles);
+    if (int rc = launch(mmq_q6k_kernel<RT>, grid, dim3(RT * 128), (size_t)kLds, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N,
                         row_bytes))
         return rc;
     float *partial2 = W2 ? partial + (size_t)nslices * M * N : nullptr;
     if (W2)
-        if (int rc = launch(mmq_q6k_kernel, grid, dim3(kQ6RT * 128), (size_t)kLds, s, (const uint8_t *)ximg, W2, partial2, (int)M, (int)K, (int)N,
+        if (int rc = launch(mmq_q6k_kernel<RT>, grid, dim3(RT * 128), (size_t)kLds, s, (const uint8_t *)ximg, W2, partial2, (int)M, (int)K, (int)N,
                             row_bytes))
             return rc;
     return launch_mmq_reduce(partial, partial2, xscale, nslices, M, K, N, bias, act, y, ex, s);
+}
+
+// Four row tiles per workgroup (eight wavefronts) when that still gives every CU a workgroup, else two.
+int launch_mmq_q6k(const MmqExtra *ex, const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y,
+                   hipStream_t s) {
+    const int64_t wgs4 = ((N + 127) / 128) * ((K + kQ6Slice - 1) / kQ6Slice) * ((M + kMT - 1) / kMT);
+    return wgs4 >= device_cu_count() ? launch_mmq_q6k_rt<4>(ex, x, x_is_bf16, M, K, W, N, bias, act, y, s)
+                                     : launch_mmq_q6k_rt<2>(ex, x, x_is_bf16, M, K, W, N, bias, act, y, s);
 }
 
 }  // namespace
