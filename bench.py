@@ -91,6 +91,7 @@ def parse_args():
     p.add_argument("--steps", type=int, default=200)
     p.add_argument("--warmup", type=int, default=20)
     p.add_argument("--config", default="c1", choices=sorted(list(CONFIGS) + ["c4", "ffn", "layer"]))
+    p.add_argument("--rows", type=int, default=1, help="activation rows of the ffn and layer workloads (a decode batch); default 1")
     p.add_argument("--others", action="store_true", help="also measure the other configurations (reported under 'others')")
     p.add_argument("--no-graph", action="store_true", help="submit the timed steps one call at a time")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
@@ -104,18 +105,19 @@ def parse_args():
 class Problem:
     """One (x, W-rotation, y) set resident on the GPU plus the launch closure."""
 
-    def __init__(self, torch, name, hot=False):
+    def __init__(self, torch, name, hot=False, rows=1):
         from gomlx_amd import _lib, ggml, synth
         import numpy as np
         self.torch, self.name = torch, name
         self.L = _lib.lib()
         self.check = _lib.check
+        self.rows = rows if name in ("ffn", "layer") else 1
         if name in ("c4", "layer"):
-            shapes = [("Q4_K", 1, K, N) for K, N in C4_SHAPES]
+            shapes = [("Q4_K", self.rows, K, N) for K, N in C4_SHAPES]
             self.dtype, self.bound = "f32", "hbm"
             self.gain = torch.ones(4096, device="cuda")
         elif name == "ffn":  # gate and up matrices of one feed-forward block
-            shapes = [("Q4_K", 1, 4096, 14336)] * 2
+            shapes = [("Q4_K", self.rows, 4096, 14336)] * 2
             self.dtype, self.bound = "f32", "hbm"
             self.gain = torch.from_numpy((synth.normal(1200, 0, 4096) * 0.5 + 1.0).astype(np.float32)).cuda()
         else:
@@ -164,21 +166,21 @@ class Problem:
             norm = _lib.RmsNormDesc(self.gain.data_ptr(), 1e-5, 0.0)
             descs = (_lib.DenseDesc * 3)()
             for ds, p in zip(descs, (q, k, v)):
-                ds.type, ds.act, ds.dX, ds.M, ds.K = p["t"], 0, q["x"].data_ptr(), 1, p["K"]
+                ds.type, ds.act, ds.dX, ds.M, ds.K = p["t"], 0, q["x"].data_ptr(), self.rows, p["K"]
                 ds.dW, ds.N, ds.dBias, ds.dY = p["W"][c].data_ptr(), p["N"], None, p["y"].data_ptr()
             self.check(self.L.gq_qdense_norm_f32_batch(3, descs, ctypes.byref(norm), self.stream))
-            self.check(self.L.gq_qdense_block_f32(o["t"], o["x"].data_ptr(), 1, o["K"], None, o["W"][c].data_ptr(), o["N"], None, 0,
+            self.check(self.L.gq_qdense_block_f32(o["t"], o["x"].data_ptr(), self.rows, o["K"], None, o["W"][c].data_ptr(), o["N"], None, 0,
                                                   q["x"].data_ptr(), o["y"].data_ptr(), self.stream))
-            self.check(self.L.gq_qdense_gated_f32(g["t"], o["y"].data_ptr(), 1, g["K"], ctypes.byref(norm), g["W"][c].data_ptr(), None,
+            self.check(self.L.gq_qdense_gated_f32(g["t"], o["y"].data_ptr(), self.rows, g["K"], ctypes.byref(norm), g["W"][c].data_ptr(), None,
                                                   u["W"][c].data_ptr(), None, g["N"], 3, g["y"].data_ptr(), self.stream))
-            self.check(self.L.gq_qdense_block_f32(d["t"], g["y"].data_ptr(), 1, d["K"], None, d["W"][c].data_ptr(), d["N"], None, 0,
+            self.check(self.L.gq_qdense_block_f32(d["t"], g["y"].data_ptr(), self.rows, d["K"], None, d["W"][c].data_ptr(), d["N"], None, 0,
                                                   o["y"].data_ptr(), d["y"].data_ptr(), self.stream))
             return
         if self.name == "ffn":
             from gomlx_amd import _lib
             g, u = self.parts
             norm = _lib.RmsNormDesc(self.gain.data_ptr(), 1e-5, 0.0)
-            self.check(self.L.gq_qdense_gated_f32(g["t"], g["x"].data_ptr(), 1, g["K"], ctypes.byref(norm), g["W"][c].data_ptr(), None,
+            self.check(self.L.gq_qdense_gated_f32(g["t"], g["x"].data_ptr(), self.rows, g["K"], ctypes.byref(norm), g["W"][c].data_ptr(), None,
                                                   u["W"][c].data_ptr(), None, g["N"], 3, g["y"].data_ptr(), self.stream))
             return
         for p in self.parts:
@@ -238,7 +240,7 @@ class Problem:
             out["value"] = self.weight_bytes * steps / wall / 1e9
             ach = self.weight_bytes / (kernel_us * 1e-6) / 1e9
             out["roofline"] = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                               "frac": ach / HBM_PEAK_GBS, "traffic": measured_traffic(self.name),
+                               "frac": ach / HBM_PEAK_GBS, "traffic": measured_traffic(self.name) if self.rows == 1 else None,
                                "algorithmic_bytes_per_launch": self.weight_bytes, "kernel_us": kernel_us}
         else:
             out["metric"], out["unit"] = "prefill GEMM TFLOP/s", "TFLOP/s"
@@ -330,7 +332,7 @@ def main():
     _lib.init(0)
 
     def measure(name):
-        prob = Problem(torch, name, hot=args.hot)
+        prob = Problem(torch, name, hot=args.hot, rows=args.rows)
         wall, kus, launches = prob.run(args.steps, args.warmup, not args.no_graph)
         rep = prob.report(wall, kus, args.steps)
         rep["weight_copies"] = prob.copies
@@ -346,7 +348,8 @@ def main():
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": rep["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": {"c3": "bf16", "prefill": "f16"}.get(args.config, "f32"), "data": "synthetic",
-        "config": {"workload": WORKLOAD_TEXT[args.config], "ggml_type": tn,
+        "config": {"workload": WORKLOAD_TEXT[args.config] + (f" [run with {args.rows} activation rows]" if args.rows != 1 and args.config in ("ffn", "layer") else ""),
+                   "ggml_type": tn,
                    "weights": "cache-resident single buffer" if args.hot else
                    f"cold: rotation over {rep['weight_copies']} distinct weight copies",
                    "submission": "eager" if args.no_graph else "one recorded HIP graph of all timed steps",
