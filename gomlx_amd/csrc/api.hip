@@ -94,6 +94,10 @@ bool type_info(int type, TypeInfo &ti) {
 }
 
 constexpr int64_t kGemvMaxRows = 16;  // above this many activation rows the tiled MFMA kernels win
+// Batched submissions merge problems of up to this many activation rows each into one K-sliced GEMV launch (q/k/v
+// of a decoder layer behind one normalisation, 2 / 4 / 8 rows: the layer's four calls take 50.6 / 83.1 / 86.8 us
+// merged against 59.1 / 97.6 / 97.7 us as three calls).
+int64_t batch_rows_max() { return 8; }
 
 bool aligned_to(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
@@ -375,13 +379,15 @@ int gq_qdense_f32_batch(int count, const gq_dense_desc *descs, void *stream) {
         auto fits = [&](const gq_dense_desc &d) {
             return use_ks ? gemv_ks_supported(d.type, d.K, d.N, d.dX) : gemv_xs_supported(d.type, d.K, d.N, d.dX);
         };
-        while (j < count && j - i < 8 && descs[j].type == descs[i].type && descs[j].M == 1 && descs[j].N > 0 && fits(descs[j])) {
+        const int64_t rows = descs[i].M;
+        const bool rows_ok = rows == 1 || (use_ks && rows >= 1 && rows <= batch_rows_max());
+        while (j < count && j - i < 8 && rows_ok && descs[j].type == descs[i].type && descs[j].M == rows && descs[j].N > 0 && fits(descs[j])) {
             const gq_dense_desc &d = descs[j];
             items[j - i] = XsBatchItem{d.dX, (const uint8_t *)d.dW, d.dBias, d.dY, d.K, d.N, d.act};
             j++;
         }
         if (j - i >= 2) {
-            if (int rc = use_ks ? launch_gemv_ks_batch(descs[i].type, j - i, items, (hipStream_t)stream)
+            if (int rc = use_ks ? launch_gemv_ks_batch(descs[i].type, j - i, items, (hipStream_t)stream, (int)rows)
                                 : launch_gemv_xs_batch(descs[i].type, j - i, items, (hipStream_t)stream))
                 return rc;
             i = j;
@@ -425,19 +431,40 @@ int gq_rmsnorm_f32(const float *dX, int64_t M, int64_t K, const float *dGain, fl
 }
 
 namespace {
-// The calls around a projection run inside the decode GEMV while that kernel is the right one for
-// the batch: over a large matrix its time grows by a pass per two rows, the split-K form costs the
-// same for any batch up to 32 rows.  Measured on gate/up 4096 -> 14336 with RMSNorm and SiLU (us; GEMV
-// at 2, 4 rows | split-K): Q4_K 22 35 | 45, Q8_0 27 43 | 61, Q4_0 19 32 | 51, Q6_K 27 45 (63 at 6) | 90: the
-// change-over sits at or just past the point where a plain dense call changes kernels; a single
-// projection with norm or residual pays one small extra kernel in the split-K form and changes one
-// or two rows later.
+// First batch size at which a projection with its neighbours leaves the GEMV for the split-K kernels.  The GEMV with
+// the extras walks a large matrix once per two rows (not four), the split-K form costs the same for any batch up to 32
+// rows and carries the normalisation and the residual at no extra launch.  Measured (us per call in a replayed graph,
+// RMSNorm in front; rows 2 3 4 5 6 7 8 on the GEMV | split-K):
+//   block (one projection + residual)                                    gated pair (SiLU)
+//   Q8_0   4096x4096 10 14 16 19 22 25 28 | 15   4096x14336 16 26 26 36 36 47 47 | 30      12 19 19 26 26 33 33 | 25   28 46 45 62 62 80 80 | 54
+//   Q4_0   4096x4096  9 12 14 17 20 22 25 | 13   4096x14336 12 20 20 28 28 36 36 | 25      10 12 14 16 18 20 22 | 22   19 33 32 46 46 59 59 | 43
+//   Q4_K   4096x4096  9 12 15 18 20 23 26 | 13   4096x14336 13 22 22 31 31 40 40 | 19      10 12 15 17 20 22 24 | 22   21 36 35 50 50 65 65 | 34
+//   Q6_K   4096x4096 11 14 17 20 23 26 30 | 19   4096x14336 16 28 28 39 39 51 51 | 33      12 20 20 28 28 35 35 | 32   29 47 47 64 64 83 83 | 60
+//   IQ4_NL 4096x4096 10 13 16 19 22 25 28 | 14   4096x14336 14 25 25 35 35 46 46 | 28      12 15 18 21 24 27 31 | 23   24 42 41 59 59 77 77 | 48
+// (14336x4096 behaves like 4096x14336.)  Matrices of a few megabytes stay on the GEMV for every batch it takes.
+int64_t block_split_k_from(int type, int64_t weight_bytes, bool gated) {
+    if (weight_bytes < kTinyWeightBytes) return kGemvMaxRows + 1;
+    if (weight_bytes >= kLargeWeightBytes) return type == GQ_Q4_K ? 3 : 5;
+    switch (type) {
+    case GQ_Q8_0: return gated ? 5 : 4;
+    case GQ_Q4_0: return gated ? 9 : 5;
+    case GQ_Q4_K: return gated ? 8 : 4;
+    case GQ_Q6_K: return gated ? 7 : 5;
+    case GQ_IQ4_NL: return gated ? 6 : 4;
+    default: return 8;
+    }
+}
+
 bool fold_into_gemv(int type, int64_t M, int64_t K, int64_t N, const float *x, const float *gain, const float *bias, const float *y, bool gated) {
     if (!gemv_ks_ext_supported(type, M, K, N, x, gain)) return false;
-    const int64_t wb = weight_bytes_of(type, K, N);
-    const bool large = wb >= kLargeWeightBytes;
-    const int64_t margin = gated ? (!large ? 0 : type == GQ_Q6_K ? 2 : (type == GQ_Q4_K || type == GQ_Q4_0) ? 1 : 0) : (large ? 1 : 2);
-    return !(M >= split_k_from(type, wb) + margin && mmq_supported(type, M, K, N, x, bias, y));
+    return !(M >= block_split_k_from(type, weight_bytes_of(type, K, N), gated) && mmq_supported(type, M, K, N, x, bias, y));
+}
+
+// Whether a projection with its neighbours runs on the split-K kernels (after fold_into_gemv() has declined).
+bool block_takes_split_k(int type, int64_t M, int64_t K, int64_t N, const float *x, const float *bias, const float *y, bool gated) {
+    const bool tp = gemm_two_pass_supported(type, false, M, K, N, x);
+    return M >= block_split_k_from(type, weight_bytes_of(type, K, N), gated) && mmq_supported(type, M, K, N, x, bias, y) &&
+           (M <= split_k_to(type, K, N) || !tp);
 }
 
 // Whether a plain dense call on these operands runs on the split-K kernels (the dispatch of gq_qdense_f32).
@@ -481,7 +508,7 @@ int gq_qdense_block_f32(int type, const float *dX, int64_t M, int64_t K, const g
                                           dY, ws, (hipStream_t)stream);
     }
     // split-K range: the normalisation rides on the activation pre-pass and the reduction, the residual on the reduction
-    if (dense_takes_split_k(type, M, K, N, dX, dBias, dY) && (!dResidual || aligned_to(dResidual, 16)) && (!rn.gain || aligned_to(rn.gain, 16))) {
+    if (block_takes_split_k(type, M, K, N, dX, dBias, dY, false) && (!dResidual || aligned_to(dResidual, 16)) && (!rn.gain || aligned_to(rn.gain, 16))) {
         const MmqExtra ex{nullptr, nullptr, dResidual, norm ? &rn : nullptr};
         return launch_mmq(type, dX, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream, &ex);
     }
@@ -513,17 +540,18 @@ int gq_qdense_norm_f32_batch(int count, const gq_dense_desc *descs, const gq_rms
     if (!(norm->eps >= 0.f)) return fail(GQ_ERR_INVALID, "gq_qdense_norm_f32_batch: epsilon must be >= 0");
     if (count == 0) return GQ_OK;
     if (int rc = use_device()) return rc;
-    // one launch when every problem is a batch-1 projection of one type and one K that the K-sliced GEMV takes
-    bool merged = count >= 2 && count <= 8;
+    // one launch when every problem is a projection of one type, one K and one (small) batch size that the K-sliced GEMV takes
+    const int64_t rows = descs[0].M;
+    bool merged = count >= 2 && count <= 8 && rows >= 1 && rows <= batch_rows_max();
     XsBatchItem items[8];
     for (int i = 0; i < count && merged; i++) {
         const gq_dense_desc &d = descs[i];
-        merged = d.type == descs[0].type && d.K == descs[0].K && d.M == 1 && d.N > 0 && gemv_ks_ext_supported(d.type, 1, d.K, d.N, d.dX, norm->dGain);
+        merged = d.type == descs[0].type && d.K == descs[0].K && d.M == rows && d.N > 0 && gemv_ks_ext_supported(d.type, rows, d.K, d.N, d.dX, norm->dGain);
         if (merged) items[i] = XsBatchItem{d.dX, (const uint8_t *)d.dW, d.dBias, d.dY, d.K, d.N, d.act};
     }
     if (merged) {
         const RmsNorm rn{norm->dGain, norm->eps, norm->gain_offset};
-        return launch_gemv_ks_batch_norm(descs[0].type, count, items, &rn, (hipStream_t)stream);
+        return launch_gemv_ks_batch_norm(descs[0].type, count, items, &rn, (hipStream_t)stream, (int)rows);
     }
     for (int i = 0; i < count; i++) {
         const gq_dense_desc &d = descs[i];
@@ -551,7 +579,7 @@ int gq_qdense_gated_f32(int type, const float *dX, int64_t M, int64_t K, const g
         return launch_gemm_two_pass_block(type, dX, M, K, norm ? &rn : nullptr, (const uint8_t *)dWgate, dBiasGate, (const uint8_t *)dWup, dBiasUp,
                                           nullptr, N, act, dY, ws, (hipStream_t)stream);
     }
-    if (dense_takes_split_k(type, M, K, N, dX, dBiasGate, dY) && (!dBiasUp || aligned_to(dBiasUp, 16)) && (!rn.gain || aligned_to(rn.gain, 16))) {
+    if (block_takes_split_k(type, M, K, N, dX, dBiasGate, dY, true) && (!dBiasUp || aligned_to(dBiasUp, 16)) && (!rn.gain || aligned_to(rn.gain, 16))) {
         // both matrices against one activation image (which carries the gain); the reduction normalises and forms act(gate) * up
         const MmqExtra ex{(const uint8_t *)dWup, dBiasUp, nullptr, norm ? &rn : nullptr};
         return launch_mmq(type, dX, false, M, K, (const uint8_t *)dWgate, N, dBiasGate, act, dY, (hipStream_t)stream, &ex);

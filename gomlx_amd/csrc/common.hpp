@@ -96,9 +96,10 @@ int launch_rmsnorm(const float *x, int64_t M, int64_t K, const float *gain, floa
 int launch_mul_inplace(float *y, const float *g, int64_t n, hipStream_t s);
 struct XsBatchItem { const float *x; const uint8_t *W; const float *bias; float *y; int64_t K, N; int act; };
 int launch_gemv_xs_batch(int type, int count, const XsBatchItem *items, hipStream_t s);
-int launch_gemv_ks_batch(int type, int count, const XsBatchItem *items, hipStream_t s);
+// (K-sliced: `rows` activation rows per problem, the same count for all: x and y are [rows, K] and [rows, N])
+int launch_gemv_ks_batch(int type, int count, const XsBatchItem *items, hipStream_t s, int rows = 1);
 // the same with one RMS normalisation applied to every problem's activations (all of one K)
-int launch_gemv_ks_batch_norm(int type, int count, const XsBatchItem *items, const RmsNorm *norm, hipStream_t s);
+int launch_gemv_ks_batch_norm(int type, int count, const XsBatchItem *items, const RmsNorm *norm, hipStream_t s, int rows = 1);
 // Large batches: dequantise W once into a 16-bit image (in `workspace`, gemm_two_pass_workspace()
 // bytes), then a plain 16-bit MFMA GEMM.
 bool gemm_two_pass_supported(int type, bool x_is_bf16, int64_t M, int64_t K, int64_t N, const void *x);

@@ -24,7 +24,8 @@ template <int T>
 __global__ __launch_bounds__(512) void gemv_ks_batch_kernel(const KsBatch b) {
     extern __shared__ uint32_t lds[];
     const KsProblem &q = b.p[ks_batch_problem(b, (int)blockIdx.x)];
-    ks_body<T, kBatchPF, kBatchPF>(q.x, q.W, q.bias, q.y, q.N, q.row_bytes, q.iters, q.nslices, q.half_tail, q.act, q.waves,
+    const int64_t row = blockIdx.y;  // activation row of every problem
+    ks_body<T, kBatchPF, kBatchPF>(q.x + row * q.K, q.W, q.bias, q.y + row * q.N, q.N, q.row_bytes, q.iters, q.nslices, q.half_tail, q.act, q.waves,
                      (int)blockIdx.x - q.wg_begin, lds);
 }
 
@@ -98,12 +99,12 @@ int launch_ks(const void *x, int x_bf16, int64_t M, int64_t K, const uint8_t *W,
 }
 
 template <int T>
-int launch_ks_batch(int count, const XsBatchItem *items, hipStream_t s) {
+int launch_ks_batch(int count, const XsBatchItem *items, int rows, hipStream_t s) {
     KsBatch b;
     size_t shmem;
     int wgs;
     if (int rc = plan_ks_batch<T>(count, items, b, shmem, wgs)) return rc;
-    return launch(gemv_ks_batch_kernel<T>, dim3((unsigned)wgs), dim3(512), shmem, s, b);
+    return launch(gemv_ks_batch_kernel<T>, dim3((unsigned)wgs, (unsigned)rows), dim3(512), shmem, s, b);
 }
 
 }  // namespace
@@ -129,14 +130,14 @@ int launch_gemv_ks(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K
     }
 }
 
-int launch_gemv_ks_batch(int type, int count, const XsBatchItem *items, hipStream_t s) {
+int launch_gemv_ks_batch(int type, int count, const XsBatchItem *items, hipStream_t s, int rows) {
     if (count < 1 || count > kMaxBatchKs) return fail(GQ_ERR_INVALID, "gemv batch: %d problems (1..%d supported per launch)", count, kMaxBatchKs);
     switch (type) {
-    case kQ4_0: return launch_ks_batch<kQ4_0>(count, items, s);
-    case kQ8_0: return launch_ks_batch<kQ8_0>(count, items, s);
-    case kQ4_K: return launch_ks_batch<kQ4_K>(count, items, s);
-    case kQ6_K: return launch_ks_batch<kQ6_K>(count, items, s);
-    case kIQ4_NL: return launch_ks_batch<kIQ4_NL>(count, items, s);
+    case kQ4_0: return launch_ks_batch<kQ4_0>(count, items, rows, s);
+    case kQ8_0: return launch_ks_batch<kQ8_0>(count, items, rows, s);
+    case kQ4_K: return launch_ks_batch<kQ4_K>(count, items, rows, s);
+    case kQ6_K: return launch_ks_batch<kQ6_K>(count, items, rows, s);
+    case kIQ4_NL: return launch_ks_batch<kIQ4_NL>(count, items, rows, s);
     default: return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv batch: ggml type %d is not implemented", type);
     }
 }

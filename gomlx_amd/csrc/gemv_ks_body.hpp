@@ -757,14 +757,14 @@ struct KsProblem {
     const float *bias;
     float *y;
     int64_t row_bytes;
-    int N, iters, nslices, half_tail, waves, act, wg_begin;
+    int N, K, iters, nslices, half_tail, waves, act, wg_begin;
 };
 struct KsBatch {
     int count;
     KsProblem p[kMaxBatchKs];
 };
 
-// Plans one launch for `count` batch-1 problems: the chip's workgroup slots are shared out in
+// Plans one launch for `count` problems (blockIdx.y of the launch walks their activation rows, all of one count): the chip's workgroup slots are shared out in
 // proportion to each problem's weight bytes, so every CU streams for about the same time.
 template <int T>
 int plan_ks_batch(int count, const XsBatchItem *items, KsBatch &b, size_t &shmem, int &wgs) {
@@ -777,7 +777,7 @@ int plan_ks_batch(int count, const XsBatchItem *items, KsBatch &b, size_t &shmem
     for (int i = 0; i < count; i++) {
         const XsBatchItem &it = items[i];
         KsProblem q;
-        q.x = it.x; q.W = it.W; q.bias = it.bias; q.y = it.y; q.N = (int)it.N; q.act = it.act;
+        q.x = it.x; q.W = it.W; q.bias = it.bias; q.y = it.y; q.N = (int)it.N; q.K = (int)it.K; q.act = it.act;
         q.row_bytes = (int64_t)gq_row_bytes(T, it.K);
         if (!ks_split(it.K, q.waves, q.nslices, q.half_tail)) return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv_ks batch: unsupported K");
         int64_t share = (int64_t)((double)cus * ((double)q.row_bytes * (double)it.N) / total + 0.5);

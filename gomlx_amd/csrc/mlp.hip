@@ -31,17 +31,18 @@ template <int T>
 __global__ __launch_bounds__(512) void gemv_ks_batch_ext_kernel(const KsBatch b, const KsExt ext) {
     extern __shared__ uint32_t lds[];
     const KsProblem &q = b.p[ks_batch_problem(b, (int)blockIdx.x)];
-    ks_body<T, kBatchPF, kBatchPF, true>(q.x, q.W, q.bias, q.y, q.N, q.row_bytes, q.iters, q.nslices, q.half_tail, q.act, q.waves,
+    const int64_t row = blockIdx.y;  // activation row of every problem
+    ks_body<T, kBatchPF, kBatchPF, true>(q.x + row * q.K, q.W, q.bias, q.y + row * q.N, q.N, q.row_bytes, q.iters, q.nslices, q.half_tail, q.act, q.waves,
                                          (int)blockIdx.x - q.wg_begin, lds, &ext);
 }
 
 template <int T>
-int launch_batch_ext(int count, const XsBatchItem *items, const KsExt &ext, hipStream_t s) {
+int launch_batch_ext(int count, const XsBatchItem *items, const KsExt &ext, int rows, hipStream_t s) {
     KsBatch b;
     size_t shmem;
     int wgs;
     if (int rc = plan_ks_batch<T>(count, items, b, shmem, wgs)) return rc;
-    return launch(gemv_ks_batch_ext_kernel<T>, dim3((unsigned)wgs), dim3(512), shmem, s, b, ext);
+    return launch(gemv_ks_batch_ext_kernel<T>, dim3((unsigned)wgs, (unsigned)rows), dim3(512), shmem, s, b, ext);
 }
 
 template <int T, int PF, int R = 1>
@@ -160,15 +161,15 @@ int launch_gemv_ks_ext(int type, const float *x, int64_t M, int64_t K, const Rms
 }
 
 // all problems share K (one normalised input feeds them)
-int launch_gemv_ks_batch_norm(int type, int count, const XsBatchItem *items, const RmsNorm *norm, hipStream_t s) {
+int launch_gemv_ks_batch_norm(int type, int count, const XsBatchItem *items, const RmsNorm *norm, hipStream_t s, int rows) {
     if (count < 1 || count > kMaxBatchKs) return fail(GQ_ERR_INVALID, "gemv batch: %d problems (1..%d supported per launch)", count, kMaxBatchKs);
     const KsExt ext = make_ext(norm, items[0].K, nullptr, nullptr, nullptr);
     switch (type) {
-    case kQ4_0: return launch_batch_ext<kQ4_0>(count, items, ext, s);
-    case kQ8_0: return launch_batch_ext<kQ8_0>(count, items, ext, s);
-    case kQ4_K: return launch_batch_ext<kQ4_K>(count, items, ext, s);
-    case kQ6_K: return launch_batch_ext<kQ6_K>(count, items, ext, s);
-    case kIQ4_NL: return launch_batch_ext<kIQ4_NL>(count, items, ext, s);
+    case kQ4_0: return launch_batch_ext<kQ4_0>(count, items, ext, rows, s);
+    case kQ8_0: return launch_batch_ext<kQ8_0>(count, items, ext, rows, s);
+    case kQ4_K: return launch_batch_ext<kQ4_K>(count, items, ext, rows, s);
+    case kQ6_K: return launch_batch_ext<kQ6_K>(count, items, ext, rows, s);
+    case kIQ4_NL: return launch_batch_ext<kIQ4_NL>(count, items, ext, rows, s);
     default: return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv batch: ggml type %d is not implemented", type);
     }
 }

@@ -259,8 +259,8 @@ def quantized_dense_batch(problems, norm: RMSNorm | None = None) -> list:
     layer's input norm, gq_qdense_norm_f32_batch).
 
     ``problems`` is a sequence of ``(x, weights, quant, bias, activation)`` tuples with float32
-    activations; returns the list of outputs.  Results equal those of separate calls; batch-1
-    problems of one GGML type share a single kernel launch.
+    activations; returns the list of outputs.  Results equal those of separate calls; problems
+    of one GGML type and one batch size of up to 8 rows share a single kernel launch.
     """
     import ctypes
     L = _lib.lib()
