@@ -713,9 +713,9 @@ def test_batched_projections_behind_one_norm(gpu, oracle, t):
     gain = (synth.normal(740, 0, K) * 0.5 + 1.0).astype(np.float32)
     cfg = nn.RMSNorm(dev(gpu, gain), 1e-5, 0.0)
     q = Quantization(ggml_type=t)
-    for rows in ((1, 1, 1), (1, 3, 1)):
+    for rows in ((1, 1, 1), (1, 3, 1), (4, 4, 4), (8, 8, 8), (9, 9, 9)):  # (up to 8 rows each share the launch too)
         xs = [synth.activations(741 + j, m, K) for j, m in enumerate(rows)]
-        if rows == (1, 1, 1):
+        if len(set(rows)) == 1:
             xs = [xs[0]] * 3  # one shared input, as in a decoder layer
         Ws = [synth.weights(t, 750 + j, n, K) for j, n in enumerate((2048, 512, 520))]
         bs = [None, synth.normal(760, 0, 512).astype(np.float32) * 0.1, None]
@@ -725,6 +725,11 @@ def test_batched_projections_behind_one_norm(gpu, oracle, t):
         for x, W, b, y in zip(xs, Ws, bs, outs):
             want = oracle.c_qdense(t, oracle.c_rmsnorm(x, gain, 1e-5, 0.0), W, b)
             assert rel_err(y.cpu().numpy(), want) < TOL_F32
+        plain = nn.quantized_dense_batch([(dev(gpu, x), dev(gpu, W), q, None if b is None else dev(gpu, b), None)
+                                          for x, W, b in zip(xs, Ws, bs)])
+        gpu.cuda.synchronize()
+        for x, W, b, y in zip(xs, Ws, bs, plain):
+            assert rel_err(y.cpu().numpy(), oracle.c_qdense(t, x, W, b)) < TOL_F32
 
 
 @pytest.mark.parametrize("t", ALL_TYPES)
