@@ -46,10 +46,10 @@ _KIB, _FETCH_SCALE, _WRITE_SCALE = 1024, 65536.0 / 32780.5, 1.0
 COUNTER_KIB = {  # workload -> (FETCH_SIZE, WRITE_SIZE) raw counter KiB per step
     "c0": (8811.9, 16.0),
     "c1": (16262.6, 56.0),
-    "c2": (19875.5 + 1866.1 + 928.1, 3584.0 + 512.0 + 925.8),
+    "c2": (19876.6 + 1869.1 + 921.1, 3584.0 + 512.0 + 925.8),
     "c3": (74726.7, 32768.0),
     "c4": (60543.5, 168.0),
-    "prefill": (4628.9 + 16401.1 + 82462.5, 32768.0 + 16448.0 + 32768.0),
+    "prefill": (4628.9 + 16401.2 + 82465.3, 32768.0 + 16448.0 + 32768.0),
     "ffn": (32484.0, 56.0),
     "layer": (7126.2 + 4756.1 + 32483.6 + 16449.7, 24.0 + 16.0 + 56.0 + 16.0),
 }

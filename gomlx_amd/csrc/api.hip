@@ -436,21 +436,21 @@ namespace {
 // rows and carries the normalisation and the residual at no extra launch.  Measured (us per call in a replayed graph,
 // RMSNorm in front; rows 2 3 4 5 6 7 8 on the GEMV | split-K):
 //   block (one projection + residual)                                    gated pair (SiLU)
-//   Q8_0   4096x4096 10 14 16 19 22 25 28 | 15   4096x14336 16 26 26 36 36 47 47 | 30      12 19 19 26 26 33 33 | 25   28 46 45 62 62 80 80 | 54
-//   Q4_0   4096x4096  9 12 14 17 20 22 25 | 13   4096x14336 12 20 20 28 28 36 36 | 25      10 12 14 16 18 20 22 | 22   19 33 32 46 46 59 59 | 43
-//   Q4_K   4096x4096  9 12 15 18 20 23 26 | 13   4096x14336 13 22 22 31 31 40 40 | 19      10 12 15 17 20 22 24 | 22   21 36 35 50 50 65 65 | 34
-//   Q6_K   4096x4096 11 14 17 20 23 26 30 | 19   4096x14336 16 28 28 39 39 51 51 | 33      12 20 20 28 28 35 35 | 32   29 47 47 64 64 83 83 | 60
-//   IQ4_NL 4096x4096 10 13 16 19 22 25 28 | 14   4096x14336 14 25 25 35 35 46 46 | 28      12 15 18 21 24 27 31 | 23   24 42 41 59 59 77 77 | 48
+//   Q8_0   4096x4096 10 14 16 19 22 25 28 | 15   4096x14336 16 26 26 36 36 47 47 | 30      12 19 19 26 26 33 33 | 23   28 46 45 62 62 80 80 | 52
+//   Q4_0   4096x4096  9 12 14 17 20 22 25 | 13   4096x14336 12 20 20 28 28 36 36 | 25      10 12 14 16 18 20 22 | 20   19 33 32 46 46 59 59 | 41
+//   Q4_K   4096x4096  9 12 15 18 20 23 26 | 13   4096x14336 13 22 22 31 31 40 40 | 19      10 12 15 17 20 22 24 | 21   21 36 35 50 50 65 65 | 33
+//   Q6_K   4096x4096 11 14 17 20 23 26 30 | 19   4096x14336 16 28 28 39 39 51 51 | 33      12 20 20 28 28 35 35 | 31   29 47 47 64 64 83 83 | 59
+//   IQ4_NL 4096x4096 10 13 16 19 22 25 28 | 14   4096x14336 14 25 25 35 35 46 46 | 28      12 15 18 21 24 27 31 | 19   24 42 41 59 59 77 77 | 46
 // (14336x4096 behaves like 4096x14336.)  Matrices of a few megabytes stay on the GEMV for every batch it takes.
 int64_t block_split_k_from(int type, int64_t weight_bytes, bool gated) {
     if (weight_bytes < kTinyWeightBytes) return kGemvMaxRows + 1;
     if (weight_bytes >= kLargeWeightBytes) return type == GQ_Q4_K ? 3 : 5;
     switch (type) {
     case GQ_Q8_0: return gated ? 5 : 4;
-    case GQ_Q4_0: return gated ? 9 : 5;
-    case GQ_Q4_K: return gated ? 8 : 4;
+    case GQ_Q4_0: return gated ? 8 : 5;
+    case GQ_Q4_K: return gated ? 7 : 4;
     case GQ_Q6_K: return gated ? 7 : 5;
-    case GQ_IQ4_NL: return gated ? 6 : 4;
+    case GQ_IQ4_NL: return gated ? 5 : 4;
     default: return 8;
     }
 }

@@ -216,10 +216,14 @@ __global__ __launch_bounds__(512) void mmq_xprep_kernel(const void *__restrict__
 // super-blocks (w >> 2), (w >> 2) + kParts, ... of the slice; the partial tiles meet in LDS at the end.  v_mfma_f32_32x32x16_f16 with
 // A = activations (32 batch columns x 16 k) and B = weights (16 k x 32 rows): one 16-byte LDS
 // read per lane feeds 16384 multiply-adds, and a lane's 16 results all belong to its own row.
-__global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__restrict__ ximg, const uint8_t *__restrict__ W,
-                                                      float *__restrict__ partial, int M, int K, int N,
-                                                      int64_t row_bytes, int m0, int slice_sb) {
+__global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__restrict__ ximg, const uint8_t *__restrict__ W0,
+                                                      float *__restrict__ partial0, int M, int K, int N,
+                                                      int64_t row_bytes, int m0, int slice_sb, const uint8_t *__restrict__ W2,
+                                                      float *__restrict__ partial2) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    // blockIdx.z = 1: the second matrix of a gated pair (same activation image, its own partial sums)
+    const uint8_t *__restrict__ W = blockIdx.z ? W2 : W0;
+    float *__restrict__ partial = blockIdx.z ? partial2 : partial0;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int kg = lane >> 5, col = lane & 31;
     const int rt = wave & 3, par = wave >> 2;  // par = 0 .. kParts-1
@@ -575,15 +579,20 @@ __global__ __launch_bounds__(256) void mmq_b32_xprep_kernel(const void *__restri
 // RT row tiles of 32 W rows per workgroup, two wavefronts each.  K % 256 == 0.
 // LDS: [activation image: S * 64 bytes][per wavefront: one stretch of 32 rows]
 template <int T, int RT>
-__global__ __launch_bounds__(RT * 128) void mmq_b32_kernel(const uint8_t *__restrict__ ximg, const uint8_t *__restrict__ W,
-                                                           float *__restrict__ partial, int M, int K, int N, int64_t row_bytes, int S) {
+__global__ __launch_bounds__(RT * 128) void mmq_b32_kernel(const uint8_t *__restrict__ ximg, const uint8_t *__restrict__ W0,
+                                                           float *__restrict__ partial0, int M, int K, int N, int64_t row_bytes, int S, int mtiles,
+                                                           const uint8_t *__restrict__ W2, float *__restrict__ partial2) {
+    // blockIdx.z >= mtiles: the second matrix of a gated pair (same activation image, its own partial sums)
+    const bool second = (int)blockIdx.z >= mtiles;
+    const uint8_t *__restrict__ W = second ? W2 : W0;
+    float *__restrict__ partial = second ? partial2 : partial0;
     typedef B32<T> F;
     typedef B32Geom<T> G;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int kg = lane >> 5, col = lane & 31;
     const int rt = wave % RT, par = wave / RT;
-    const int slice = blockIdx.y, nslices = gridDim.y, mt = blockIdx.z;
+    const int slice = blockIdx.y, nslices = gridDim.y, mt = second ? (int)blockIdx.z - mtiles : (int)blockIdx.z;
     const int img_bytes = S * 64;
     const int kstretches = K >> 8, t0 = slice * (S >> 8);      // stretches of a row; first stretch of the slice
     const int n0 = (blockIdx.x * RT + rt) * 32;                // first W row of this wavefront's tile
@@ -714,14 +723,11 @@ int launch_mmq_b32(const void *x, bool x_is_bf16, int64_t M, int64_t K, const ui
                            : launch(mmq_b32_xprep_kernel<false>, xgrid, dim3(256), 0, s, x, ximg, xscale, (int)M, (int)K, S, nslices, norm ? norm->gain : nullptr,
                                     norm ? norm->gain_offset : 0.f, norm ? mmq_xss(xscale, nslices, M) : nullptr))
         return rc;
-    const dim3 grid((unsigned)rowwgs, (unsigned)nslices, (unsigned)mtiles);
-    if (int rc = launch(mmq_b32_kernel<T, RT>, grid, dim3(RT * 128), lds_bytes, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N, row_bytes, S))
-        return rc;
+    const dim3 grid((unsigned)rowwgs, (unsigned)nslices, (unsigned)mtiles * (W2 ? 2u : 1u));  // (both matrices of a gated pair in one launch)
     float *partial2 = W2 ? partial + (size_t)nslices * M * N : nullptr;
-    if (W2)
-        if (int rc = launch(mmq_b32_kernel<T, RT>, grid, dim3(RT * 128), lds_bytes, s, (const uint8_t *)ximg, W2, partial2, (int)M, (int)K, (int)N,
-                            row_bytes, S))
-            return rc;
+    if (int rc = launch(mmq_b32_kernel<T, RT>, grid, dim3(RT * 128), lds_bytes, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N, row_bytes, S,
+                        mtiles, W2, partial2))
+        return rc;
     return launch_mmq_reduce(partial, partial2, xscale, nslices, M, K, N, bias, act, y, ex, s);
 }
 
@@ -765,12 +771,16 @@ __device__ __forceinline__ void q6_bytes8(const uint8_t *row, int at, uint32_t &
 // result into accumulation registers and copies it back out, 16 extra instructions per MFMA.)
 template <int RT>
 __global__ __launch_bounds__(512) void mmq_q6k_kernel(const uint8_t *__restrict__ ximg, const uint8_t *__restrict__ W,
-                                                              float *__restrict__ partial, int M, int K, int N, int64_t row_bytes) {
+                                                              float *__restrict__ partial0, int M, int K, int N, int64_t row_bytes, int mtiles,
+                                                              const uint8_t *__restrict__ W2, float *__restrict__ partial2) {
+    const bool second = (int)blockIdx.z >= mtiles;  // the second matrix of a gated pair
+    const uint8_t *__restrict__ Wm = second ? W2 : W;
+    float *__restrict__ partial = second ? partial2 : partial0;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int kg = lane >> 5, col = lane & 31;
     const int rt = wave % RT, par = wave / RT;
-    const int slice = blockIdx.y, nslices = gridDim.y, mt = blockIdx.z;
+    const int slice = blockIdx.y, nslices = gridDim.y, mt = second ? (int)blockIdx.z - mtiles : (int)blockIdx.z;
     constexpr int img_bytes = kQ6Slice * 64;
     const int kpairs = K >> 9;                                  // pairs of a row
     const int n0 = (blockIdx.x * RT + rt) * 32;              // first W row of this wavefront's tile
@@ -785,7 +795,7 @@ __global__ __launch_bounds__(512) void mmq_q6k_kernel(const uint8_t *__restrict_
     }
     // This wavefront's pair of the slice (a pair beyond K re-reads the row's last one: its activations
     // are zero in the image), one half at a time.  Dword lane + 64 i of a half tile is dword d % 53 of row d / 53.
-    const uint8_t *pair = W + (int64_t)min(n0, N - 1) * row_bytes + (int64_t)min(2 * slice + par, kpairs - 1) * kQ6PairBytes;
+    const uint8_t *pair = Wm + (int64_t)min(n0, N - 1) * row_bytes + (int64_t)min(2 * slice + par, kpairs - 1) * kQ6PairBytes;
     const int rows_left = max(N - 1 - n0, 0);
     auto park_half = [&](int sbp) __attribute__((always_inline)) {
         uint32_t v[kQ6Loads];
@@ -908,15 +918,11 @@ int launch_mmq_q6k_rt(const MmqExtra *ex, const void *x, bool x_is_bf16, int64_t
                            : launch(mmq_b32_xprep_kernel<false>, xgrid, dim3(256), 0, s, x, ximg, xscale, (int)M, (int)K, kQ6Slice, nslices, norm ? norm->gain : nullptr,
                                     norm ? norm->gain_offset : 0.f, norm ? mmq_xss(xscale, nslices, M) : nullptr))
         return rc;
-    const dim3 grid((unsigned)((N + 32 * RT - 1) / (32 * RT)), (unsigned)nslices, (unsigned)mtiles);
-    if (int rc = launch(mmq_q6k_kernel<RT>, grid, dim3(RT * 128), (size_t)kLds, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N,
-                        row_bytes))
-        return rc;
+    const dim3 grid((unsigned)((N + 32 * RT - 1) / (32 * RT)), (unsigned)nslices, (unsigned)mtiles * (W2 ? 2u : 1u));  // (a gated pair: one launch)
     float *partial2 = W2 ? partial + (size_t)nslices * M * N : nullptr;
-    if (W2)
-        if (int rc = launch(mmq_q6k_kernel<RT>, grid, dim3(RT * 128), (size_t)kLds, s, (const uint8_t *)ximg, W2, partial2, (int)M, (int)K, (int)N,
-                            row_bytes))
-            return rc;
+    if (int rc = launch(mmq_q6k_kernel<RT>, grid, dim3(RT * 128), (size_t)kLds, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N,
+                        row_bytes, mtiles, W2, partial2))
+        return rc;
     return launch_mmq_reduce(partial, partial2, xscale, nslices, M, K, N, bias, act, y, ex, s);
 }
 
@@ -978,14 +984,13 @@ int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, co
                                     (int)K, slice_sb, norm ? norm->gain : nullptr, norm ? norm->gain_offset : 0.f,
                                     norm ? mmq_xss(xscale, nslices, M) : nullptr))
         return rc;
-    const dim3 grid((unsigned)((N + kRowsPerWG - 1) / kRowsPerWG), (unsigned)nslices);
+    const dim3 grid((unsigned)((N + kRowsPerWG - 1) / kRowsPerWG), (unsigned)nslices, W2 ? 2u : 1u);  // (both matrices of a gated pair in one launch)
     float *partial2 = W2 ? partial + (size_t)nslices * M * N : nullptr;
-    for (int which = 0; which < (W2 ? 2 : 1); which++)
-        for (int64_t m0 = 0; m0 < M; m0 += kMT) {
-            if (int rc = launch(mmq_q4k_kernel, grid, dim3(256 * kParts), (size_t)kLdsBytes, s, (const uint8_t *)ximg, which ? W2 : W,
-                                which ? partial2 : partial, (int)M, (int)K, (int)N, row_bytes, (int)m0, slice_sb))
-                return rc;
-        }
+    for (int64_t m0 = 0; m0 < M; m0 += kMT) {
+        if (int rc = launch(mmq_q4k_kernel, grid, dim3(256 * kParts), (size_t)kLdsBytes, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N,
+                            row_bytes, (int)m0, slice_sb, W2, partial2))
+            return rc;
+    }
     return launch_mmq_reduce(partial, partial2, xscale, nslices, M, K, N, bias, act, y, ex, s);
 }
 
