@@ -97,6 +97,7 @@ constexpr int64_t kGemvMaxRows = 16;  // above this many activation rows the til
 // Batched submissions merge problems of up to this many activation rows each into one K-sliced GEMV launch (q/k/v
 // of a decoder layer behind one normalisation, 2 / 4 / 8 rows: the layer's four calls take 50.6 / 83.1 / 86.8 us
 // merged against 59.1 / 97.6 / 97.7 us as three calls).
+// Only matrices under 24 MB are merged at several rows: over larger ones a single call serves several rows per pass.
 int64_t batch_rows_max() { return 8; }
 
 bool aligned_to(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
@@ -381,7 +382,10 @@ int gq_qdense_f32_batch(int count, const gq_dense_desc *descs, void *stream) {
         };
         const int64_t rows = descs[i].M;
         const bool rows_ok = rows == 1 || (use_ks && rows >= 1 && rows <= batch_rows_max());
-        while (j < count && j - i < 8 && rows_ok && descs[j].type == descs[i].type && descs[j].M == rows && descs[j].N > 0 && fits(descs[j])) {
+        // (several rows per problem: only over matrices below the size from which one pass serves several rows)
+        auto size_ok = [&](const gq_dense_desc &d) { return rows == 1 || weight_bytes_of(d.type, d.K, d.N) < kLargeWeightBytes; };
+        while (j < count && j - i < 8 && rows_ok && descs[j].type == descs[i].type && descs[j].M == rows && descs[j].N > 0 && fits(descs[j]) &&
+               size_ok(descs[j])) {
             const gq_dense_desc &d = descs[j];
             items[j - i] = XsBatchItem{d.dX, (const uint8_t *)d.dW, d.dBias, d.dY, d.K, d.N, d.act};
             j++;
@@ -546,7 +550,8 @@ int gq_qdense_norm_f32_batch(int count, const gq_dense_desc *descs, const gq_rms
     XsBatchItem items[8];
     for (int i = 0; i < count && merged; i++) {
         const gq_dense_desc &d = descs[i];
-        merged = d.type == descs[0].type && d.K == descs[0].K && d.M == rows && d.N > 0 && gemv_ks_ext_supported(d.type, rows, d.K, d.N, d.dX, norm->dGain);
+        merged = d.type == descs[0].type && d.K == descs[0].K && d.M == rows && d.N > 0 && gemv_ks_ext_supported(d.type, rows, d.K, d.N, d.dX, norm->dGain) &&
+                 (rows == 1 || weight_bytes_of(d.type, d.K, d.N) < kLargeWeightBytes);
         if (merged) items[i] = XsBatchItem{d.dX, (const uint8_t *)d.dW, d.dBias, d.dY, d.K, d.N, d.act};
     }
     if (merged) {
