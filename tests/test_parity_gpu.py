@@ -461,16 +461,17 @@ def test_small_batches_on_large_matrices(gpu, oracle, t, N):
 
 @pytest.mark.parametrize("t,N", [(Q8_0, 3328), (Q4_K, 5632), (Q6_K, 4096)])
 def test_small_batches_with_neighbours_on_large_matrices(gpu, oracle, t, N):
-    """The same batches through the calls around a projection: passes of two rows inside the decode GEMV."""
+    """The same batches through the calls around a projection: passes of two rows inside the decode GEMV up to the
+    measured change-over of each format and matrix class (3 to 8 rows), the split-K kernels with the extras beyond."""
     K = 4096
     assert 2 * N * ggml.row_bytes(t, K) >= 24 << 20
-    for i, M in enumerate((2, 3, 4, 5)):
+    for i, M in enumerate((2, 3, 4, 5, 7, 8)):
         err = gated_case(gpu, oracle, t, M, K, N, 3, 1 + i % 3, bool(i % 2), 350 + 10 * i + t)
         assert err < 2 * TOL_F32, ("gated", t, M, err)
     N2 = 2 * N
     W = synth.weights(t, 360 + t, N2, K)
     gain = (synth.normal(361, 0, K) * 0.5 + 1.0).astype(np.float32)
-    for M in (2, 3, 5):
+    for M in (2, 3, 4, 5, 6):
         x = (synth.activations(362 + M, M, K) * 2.0).astype(np.float32)
         res = synth.activations(363 + M, M, N2)
         got = nn.quantized_dense(dev(gpu, x), dev(gpu, W), Quantization(ggml_type=t), None, BACKEND_ACT[0],
