@@ -163,8 +163,10 @@ int gq_qdense_norm_f32_batch(int count, const gq_dense_desc *descs, const gq_rms
  * or x.  Both matrices are [N, gq_row_bytes(type, K)] of one type.  A few rows run as one launch
  * of the decode GEMV (conditions as for gq_qdense_block_f32); from 256 rows the two matrices are
  * dequantised into one interleaved 16-bit image and a single GEMM forms the product in
- * registers; sizes in between are composed of dense calls.  All but the first use a per-stream
- * workspace. */
+ * registers; in between, the split-K kernels contract both matrices against one activation
+ * image in one launch (the normalisation in their pre-pass and reduction, the product in the
+ * reduction) up to their batch limit, and dense calls are composed beyond it.  All but the
+ * first use a per-stream workspace. */
 int gq_qdense_gated_f32(int type, const float *dX, int64_t M, int64_t K, const gq_rmsnorm *norm,
                         const void *dWgate, const float *dBiasGate, const void *dWup,
                         const float *dBiasUp, int64_t N, int act, float *dY, void *stream);
