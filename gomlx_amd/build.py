@@ -19,6 +19,7 @@ LIB = os.path.join(HERE, "libgomlx_hipq.so")
 
 HOST = os.path.join(HERE, "host")
 HOST_TEST = os.path.join(HOST, "build", "hipq_backend_test")
+WORKSPACE_TEST = os.path.join(HOST, "build", "workspace_test")
 
 SOURCES = ["api.hip", "dequant.hip", "gemv.hip", "gemv_xs.hip", "gemv_ks.hip", "mlp.hip", "mmq.hip", "gemm.hip", "gemm_dma.hip"]
 
@@ -109,6 +110,15 @@ def build_host_test(verbose: bool = True) -> str:
         sys.stderr.write(r.stderr)
     if verbose:
         print(f"built {HOST_TEST}")
+    # the scratch-memory bookkeeping against fake device hooks (host only, no HIP)
+    cmd = ["g++", "-O1", "-std=c++17", "-Wall", "-Wextra", "-pthread", os.path.join(HOST, "workspace_test.cpp"), "-o", WORKSPACE_TEST]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"workspace test build failed:\n{r.stdout}\n{r.stderr}")
+    if r.stderr.strip():
+        sys.stderr.write(r.stderr)
+    if verbose:
+        print(f"built {WORKSPACE_TEST}")
     return HOST_TEST
 
 

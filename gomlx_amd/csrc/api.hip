@@ -2,12 +2,14 @@
 // families, HIP-graph recording and per-kernel timing.  See include/gomlx_hipq.h for the
 // contract of every entry point and the reference interface it replaces.
 #include "common.hpp"
+#include "workspace.hpp"
 
 #include <atomic>
 #include <cstring>
 #include <cstdlib>
 #include <map>
 #include <mutex>
+#include <new>
 
 namespace gq {
 
@@ -43,34 +45,55 @@ int use_device() {
 
 int device_cu_count() { return g_cu_count.load(std::memory_order_relaxed); }
 
-// ---- per-stream workspace ---------------------------------------------------------------------
-// Scratch for the paths that need more than their inputs and outputs (split-K partial sums, the
-// 16-bit weight image of the two-pass GEMM).  Work on one stream is ordered, so one buffer per
-// stream suffices; it grows geometrically and lives until the process ends.
+// ---- scratch memory ------------------------------------------------------------------------------
+// Per-stream buffers come from the pool of workspace.hpp (sequence lock per stream, buffers pinned by
+// recorded graphs, released with their stream).
 namespace {
-struct Workspace { void *ptr = nullptr; size_t bytes = 0; };
-std::mutex g_ws_mutex;
-std::map<std::pair<hipStream_t, int>, Workspace> g_ws;
+
+int ws_alloc(void **p, size_t bytes) {
+    GQ_HIP(hipMalloc(p, bytes));
+    return GQ_OK;
+}
+void ws_release(void *p) { (void)hipFree(p); }
+void ws_sync(const void *s) { (void)hipStreamSynchronize((hipStream_t)const_cast<void *>(s)); }
+bool ws_capturing(const void *s) {
+    if (!s) return false;
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    return hipStreamIsCapturing((hipStream_t)const_cast<void *>(s), &st) == hipSuccess && st != hipStreamCaptureStatusNone;
+}
+WorkspacePool &pool() {
+    static WorkspacePool *p = new WorkspacePool(WsHooks{ws_alloc, ws_release, ws_sync, ws_capturing});  // never destroyed: outlives every caller
+    return *p;
+}
+
+// One per ABI call that may reach a path with scratch memory; nested calls share the outermost one.
+struct RecordedGraph {  // what gq_graph_end hands out
+    hipGraphExec_t exec;
+    hipStream_t stream;               // the stream it was recorded on, the only one it replays on
+    std::vector<WsBlockRef> blocks;   // workspaces its launches point at
+};
+
+struct CallScope;
+thread_local CallScope *t_scope = nullptr;
+struct CallScope {
+    SeqLock lock;
+    bool outer;
+    CallScope() : outer(t_scope == nullptr) { if (outer) t_scope = this; }
+    ~CallScope() { if (outer) t_scope = nullptr; }
+};
+
 }  // namespace
 
 int stream_workspace(hipStream_t s, size_t bytes, void **out, int slot) {
-    std::lock_guard<std::mutex> lock(g_ws_mutex);
-    Workspace &w = g_ws[std::make_pair(s, slot)];
-    if (w.bytes < bytes) {
-        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
-        if (s != nullptr && hipStreamIsCapturing(s, &st) == hipSuccess && st != hipStreamCaptureStatusNone)
-            return fail(GQ_ERR_INVALID, "qdense: the %zu-byte workspace of this stream must exist before a graph is recorded; run the "
-                        "same call once outside the recording first", bytes);
-        // An outgrown buffer is retired, not freed: a recorded graph may still point at it.
-        size_t want = bytes < (size_t)(4u << 20) ? (size_t)(4u << 20) : bytes;
-        if (want < 2 * w.bytes) want = 2 * w.bytes;
-        void *p = nullptr;
-        GQ_HIP(hipMalloc(&p, want));
-        w.ptr = p;
-        w.bytes = want;
-    }
-    *out = w.ptr;
-    return GQ_OK;
+    CallScope *sc = t_scope;
+    if (!sc) return fail(GQ_ERR_INVALID, "internal: scratch memory requested outside an entry point");
+    if (slot < 0 || slot >= kWsSlots) return fail(GQ_ERR_INVALID, "internal: workspace slot %d", slot);
+    if (!sc->lock.held()) sc->lock.lock(pool().stream(s));
+    const int rc = pool().acquire(*sc->lock.held(), s, slot, bytes, out);
+    if (rc == kWsWouldAllocateInRecording)
+        return fail(GQ_ERR_INVALID, "qdense: the %zu-byte workspace of this stream must exist before a graph is recorded; run the "
+                    "same call once outside the recording first", bytes);
+    return rc;
 }
 
 ProfileState &profile_state() {
@@ -310,6 +333,7 @@ int gq_stream_create(void **stream) {
 int gq_stream_destroy(void *stream) {
     if (!stream) return GQ_OK;
     if (int rc = use_device()) return rc;
+    pool().destroy_stream(stream);  // waits for the stream, then frees its workspaces (those a recorded graph points at go with the graph)
     GQ_HIP(hipStreamDestroy((hipStream_t)stream));
     return GQ_OK;
 }
@@ -339,6 +363,7 @@ int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *d
     if (int rc = check_dense_args("gq_qdense_f32", type, dX, M, K, dW, N, dBias, act, dY, 4)) return rc;
     if (M == 0 || N == 0) return GQ_OK;
     if (int rc = use_device()) return rc;
+    CallScope scope;
     // Small batches: GEMV passes cost about one third of the first pass per extra row; the split-K
     // MFMA kernels cost 19 .. 26 us (Q8_0 / Q4_0, K = 4096, N = 4096 .. 14336) for up to 32 rows and
     // 5 .. 18 us per further 32; the two passes 33 .. 62 us for anything up to 128 rows.  Measured
@@ -369,6 +394,7 @@ int gq_qdense_f32_batch(int count, const gq_dense_desc *descs, void *stream) {
     }
     if (count == 0) return GQ_OK;
     if (int rc = use_device()) return rc;
+    CallScope scope;
     // merge runs of batch-1 problems of one type that the streaming GEMV handles; the rest go one by one
     int i = 0;
     while (i < count) {
@@ -409,6 +435,7 @@ int gq_qdense_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, const voi
     if (int rc = check_dense_args("gq_qdense_bf16", type, dX, M, K, dW, N, dBias, act, dY, 2)) return rc;
     if (M == 0 || N == 0) return GQ_OK;
     if (int rc = use_device()) return rc;
+    CallScope scope;
     // Same crossovers as for fp32 activations: bf16 widens exactly to fp32 for the GEMV passes and to
     // the fp16 activation image of the split-K kernels (which have no bf16 rounding of W: tighter than
     // the bf16 MFMA paths).
@@ -500,6 +527,7 @@ int gq_qdense_block_f32(int type, const float *dX, int64_t M, int64_t K, const g
     if (dResidual && !aligned_to(dResidual, 4)) return fail(GQ_ERR_INVALID, "gq_qdense_block_f32: residual must be 4-byte aligned");
     if (M == 0 || N == 0) return GQ_OK;
     if (int rc = use_device()) return rc;
+    CallScope scope;
     RmsNorm rn{nullptr, 0.f, 0.f};
     if (norm) rn = RmsNorm{norm->dGain, norm->eps, norm->gain_offset};
     if (fold_into_gemv(type, M, K, N, dX, rn.gain, dBias, dY, false))
@@ -516,21 +544,32 @@ int gq_qdense_block_f32(int type, const float *dX, int64_t M, int64_t K, const g
         const MmqExtra ex{nullptr, nullptr, dResidual, norm ? &rn : nullptr};
         return launch_mmq(type, dX, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream, &ex);
     }
-    // composed: normalised activations into the stream's second workspace, the dense call, then the residual
+    // composed: normalised activations into the stream's second workspace, the dense call, then the residual.  When y
+    // overlaps the residual (a residual stream updated in place) the dense result goes to the workspace first: written
+    // straight to y it would destroy the residual before the addition reads it.
     const float *x = dX;
-    if (norm) {
+    const size_t y_bytes = (size_t)M * (size_t)N * sizeof(float);
+    const bool in_place = dResidual && reinterpret_cast<uintptr_t>(dY) < reinterpret_cast<uintptr_t>(dResidual) + y_bytes &&
+                          reinterpret_cast<uintptr_t>(dResidual) < reinterpret_cast<uintptr_t>(dY) + y_bytes;
+    const size_t xn_bytes = norm ? ((size_t)M * (size_t)K * sizeof(float) + 255) / 256 * 256 : 0;
+    float *tmp = nullptr;
+    if (norm || in_place) {
         void *ws = nullptr;
-        if (int rc = stream_workspace((hipStream_t)stream, (size_t)M * (size_t)K * sizeof(float), &ws, 1)) return rc;
-        float *xn = static_cast<float *>(ws);
-        if (int rc = launch_rmsnorm(dX, M, K, rn.gain, rn.gain_offset, rn.eps, xn, (hipStream_t)stream)) return rc;
-        x = xn;
+        if (int rc = stream_workspace((hipStream_t)stream, xn_bytes + (in_place ? y_bytes : 0), &ws, 1)) return rc;
+        tmp = reinterpret_cast<float *>(static_cast<uint8_t *>(ws) + xn_bytes);
+        if (norm) {
+            float *xn = static_cast<float *>(ws);
+            if (int rc = launch_rmsnorm(dX, M, K, rn.gain, rn.gain_offset, rn.eps, xn, (hipStream_t)stream)) return rc;
+            x = xn;
+        }
     }
     if (dResidual && dense_takes_split_k(type, M, K, N, x, dBias, dY) && aligned_to(dResidual, 16)) {  // the residual rides on the reduction
         const MmqExtra ex{nullptr, nullptr, dResidual, nullptr};
         return launch_mmq(type, x, false, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream, &ex);
     }
-    if (int rc = gq_qdense_f32(type, x, M, K, dW, N, dBias, act, dY, stream)) return rc;
-    if (dResidual) return launch_add(dY, dResidual, dY, M * N, (hipStream_t)stream);
+    float *dense_out = in_place ? tmp : dY;
+    if (int rc = gq_qdense_f32(type, x, M, K, dW, N, dBias, act, dense_out, stream)) return rc;
+    if (dResidual) return launch_add(dense_out, dResidual, dY, M * N, (hipStream_t)stream);
     return GQ_OK;
 }
 
@@ -544,6 +583,7 @@ int gq_qdense_norm_f32_batch(int count, const gq_dense_desc *descs, const gq_rms
     if (!(norm->eps >= 0.f)) return fail(GQ_ERR_INVALID, "gq_qdense_norm_f32_batch: epsilon must be >= 0");
     if (count == 0) return GQ_OK;
     if (int rc = use_device()) return rc;
+    CallScope scope;
     // one launch when every problem is a projection of one type, one K and one (small) batch size that the K-sliced GEMV takes
     const int64_t rows = descs[0].M;
     bool merged = count >= 2 && count <= 8 && rows >= 1 && rows <= batch_rows_max();
@@ -573,6 +613,7 @@ int gq_qdense_gated_f32(int type, const float *dX, int64_t M, int64_t K, const g
     if (norm && norm->dGain && !aligned_to(norm->dGain, 4)) return fail(GQ_ERR_INVALID, "gq_qdense_gated_f32: gain must be 4-byte aligned");
     if (M == 0 || N == 0) return GQ_OK;
     if (int rc = use_device()) return rc;
+    CallScope scope;
     RmsNorm rn{nullptr, 0.f, 0.f};
     if (norm) rn = RmsNorm{norm->dGain, norm->eps, norm->gain_offset};
     if (fold_into_gemv(type, M, K, N, dX, rn.gain, dBiasGate, dY, true))
@@ -631,6 +672,7 @@ int gq_graph_begin(void *stream) {
     if (!stream) return fail(GQ_ERR_INVALID, "gq_graph_begin: recording needs an explicit stream");
     if (profile_state().active) return fail(GQ_ERR_INVALID, "gq_graph_begin: kernel timing is active on this thread");
     if (int rc = use_device()) return rc;
+    pool().begin_recording(stream);
     GQ_HIP(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal));
     return GQ_OK;
 }
@@ -640,26 +682,45 @@ int gq_graph_end(void *stream, void **graph_exec) {
     *graph_exec = nullptr;
     if (int rc = use_device()) return rc;
     hipGraph_t graph = nullptr;
-    GQ_HIP(hipStreamEndCapture((hipStream_t)stream, &graph));
+    const hipError_t ce = hipStreamEndCapture((hipStream_t)stream, &graph);
+    std::vector<WsBlockRef> blocks = pool().end_recording(stream);  // the workspaces the recorded launches point at
+    if (ce != hipSuccess) { pool().unpin(blocks); return hip_fail(ce, "hipStreamEndCapture"); }
     hipGraphExec_t exec = nullptr;
     const hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
     (void)hipGraphDestroy(graph);
-    if (e != hipSuccess) return hip_fail(e, "hipGraphInstantiate");
-    *graph_exec = exec;
+    if (e != hipSuccess) { pool().unpin(blocks); return hip_fail(e, "hipGraphInstantiate"); }
+    RecordedGraph *g = new (std::nothrow) RecordedGraph;
+    if (!g) { (void)hipGraphExecDestroy(exec); pool().unpin(blocks); return fail(GQ_ERR_OOM, "gq_graph_end: out of host memory"); }
+    g->exec = exec;
+    g->stream = (hipStream_t)stream;
+    g->blocks.swap(blocks);
+    *graph_exec = g;
     return GQ_OK;
 }
 
 int gq_graph_launch(void *graph_exec, void *stream) {
     if (!graph_exec) return fail(GQ_ERR_INVALID, "gq_graph_launch: null graph");
+    RecordedGraph *g = static_cast<RecordedGraph *>(graph_exec);
+    // The recorded launches point at the recording stream's workspace, which eager calls on that stream share in
+    // stream order: a replay on another stream would run unordered against them.
+    if ((hipStream_t)stream != g->stream)
+        return fail(GQ_ERR_INVALID, "gq_graph_launch: a graph replays on the stream it was recorded on");
     if (int rc = use_device()) return rc;
-    GQ_HIP(hipGraphLaunch((hipGraphExec_t)graph_exec, (hipStream_t)stream));
+    // (replays and eager sequences that share the workspace must not interleave their submissions)
+    WsStreamRef st = pool().stream(stream);
+    std::lock_guard<std::recursive_mutex> seq(st->seq);
+    GQ_HIP(hipGraphLaunch(g->exec, g->stream));
     return GQ_OK;
 }
 
 int gq_graph_destroy(void *graph_exec) {
     if (!graph_exec) return GQ_OK;
     if (int rc = use_device()) return rc;
-    GQ_HIP(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
+    RecordedGraph *g = static_cast<RecordedGraph *>(graph_exec);
+    const hipError_t e = hipGraphExecDestroy(g->exec);
+    pool().unpin(g->blocks);
+    delete g;
+    if (e != hipSuccess) return hip_fail(e, "hipGraphExecDestroy");
     return GQ_OK;
 }
 

@@ -14,6 +14,9 @@
  *   - All pointers named d* are device pointers owned by the caller; the library keeps no
  *     reference to them after the call returns (launches are asynchronous on `stream`, so
  *     the memory must stay valid until the stream has been synchronised).
+ *   - Entry points are re-entrant.  Host threads that issue calls on the SAME stream are
+ *     serialised for the length of one call's launches (multi-kernel paths share the stream's
+ *     workspace); calls on different streams proceed independently.
  *   - stream == NULL selects the null stream of the active device.  Otherwise it is a
  *     hipStream_t.  The active device is the one given to gq_init(); every entry point
  *     makes it current on the calling thread itself (cgo may move a goroutine to another
@@ -84,7 +87,7 @@ int gq_free(void *dptr);
 int gq_h2d(void *d, const void *h, size_t bytes, void *stream);  /* returns after the copy is done */
 int gq_d2h(void *h, const void *d, size_t bytes, void *stream);  /* returns after the copy is done */
 int gq_stream_create(void **stream);     /* default priority */
-int gq_stream_destroy(void *stream);
+int gq_stream_destroy(void *stream);    /* waits for the stream and frees its workspaces */
 int gq_sync(void *stream);
 
 /* ---- ggml.Dequantize (ml/ggml/dequant.go:39-54): dW [N, row_bytes] -> dOut [N, K] fp32,
@@ -181,7 +184,10 @@ int gq_embedding_lookup(int type, const void *dTable, int64_t vocab, int64_t K,
 
 /* ---- Executable.Execute of a compiled graph (core/graph/graph.go:669): a sequence of
  * launches recorded once and replayed with one submission (HIP graph).  Between begin
- * and end, entry points called with this stream are recorded, not run. ---- */
+ * and end, entry points called with this stream are recorded, not run.  A graph replays on
+ * the stream it was recorded on (its launches share that stream's workspace with eager calls,
+ * in stream order); gq_graph_launch rejects any other.  The workspaces a graph points at
+ * stay allocated until gq_graph_destroy, also after gq_stream_destroy. ---- */
 int gq_graph_begin(void *stream);
 int gq_graph_end(void *stream, void **graph_exec);
 int gq_graph_launch(void *graph_exec, void *stream);

@@ -18,8 +18,8 @@ def _binary():
     return build.HOST_TEST
 
 
-def _run(*args):
-    r = subprocess.run([_binary(), *args], capture_output=True, text=True, timeout=100)
+def _run(*args, binary=None):
+    r = subprocess.run([binary or _binary(), *args], capture_output=True, text=True, timeout=100)
     print(r.stdout)
     print(r.stderr)
     return r
@@ -28,6 +28,17 @@ def _run(*args):
 def test_host_layer_build_time_rules():
     """Graph-build validation, ErrNotImplemented vs hard errors, GOMLX_FUSION: no GPU needed."""
     r = _run("--build-only")
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "0 failed" in r.stdout and "FAIL" not in r.stdout
+
+
+def test_workspace_bookkeeping():
+    """Scratch-memory pool against fake device hooks: growth, graph pinning, stream destruction, and two host threads
+    on one stream never interleaving their launch sequences."""
+    _binary()
+    if not os.path.exists(build.WORKSPACE_TEST):
+        build.build_host_test(verbose=False)
+    r = _run(binary=build.WORKSPACE_TEST)
     assert r.returncode == 0, r.stdout + r.stderr
     assert "0 failed" in r.stdout and "FAIL" not in r.stdout
 

@@ -671,6 +671,81 @@ def test_dense_with_rmsnorm_and_residual(gpu, oracle, t):
     assert rel_err(yd.cpu().numpy(), oracle.c_qdense(t, x, W) + res) < TOL_F32
 
 
+def test_residual_in_place_on_the_composed_path(gpu, oracle):
+    """y == residual on shapes that none of the fused routes take (K not a multiple of 256; N not a multiple of 4
+    beyond 16 rows): the dense result must not overwrite the residual before it is added."""
+    from gomlx_amd import _lib
+    L = _lib.lib()
+    stream = gpu.cuda.current_stream().cuda_stream
+    for i, (t, M, K, N, use_norm) in enumerate([(Q8_0, 2, 160, 64, False), (Q8_0, 20, 160, 33, False), (Q4_0, 20, 512, 33, True),
+                                               (Q4_K, 24, 768, 30, False), (Q8_0, 3, 96, 10, True)]):
+        W, x, res = synth.weights(t, 730 + i, N, K), synth.activations(740 + i, M, K), synth.activations(750 + i, M, N)
+        gain = (synth.normal(760 + i, 0, K) * 0.5 + 1.0).astype(np.float32)
+        xd, Wd, yd, gd = dev(gpu, x), dev(gpu, W), dev(gpu, res), dev(gpu, gain)
+        norm = _lib.RmsNormDesc(gd.data_ptr(), 1e-6, 0.0)
+        import ctypes
+        _lib.check(L.gq_qdense_block_f32(t, xd.data_ptr(), M, K, ctypes.byref(norm) if use_norm else None, Wd.data_ptr(), N, None, 0,
+                                         yd.data_ptr(), yd.data_ptr(), stream))
+        gpu.cuda.synchronize()
+        xn = oracle.c_rmsnorm(x, gain, 1e-6, 0.0) if use_norm else x
+        dense = oracle.c_qdense(t, xn, W)
+        err = float(np.max(np.abs(yd.cpu().numpy().astype(np.float64) - (dense + res)))) / float(np.max(np.abs(dense)))
+        assert err < TOL_F32, (ggml.name(t), M, K, N, use_norm, err)
+
+
+def test_two_host_threads_share_the_null_stream(gpu, oracle):
+    """Split-K calls (three kernels that share the stream's workspace) issued concurrently from two host threads on the
+    null stream: every result matches the oracle, i.e. the launch sequences were not interleaved."""
+    import threading
+    from gomlx_amd import _lib
+    L = _lib.lib()
+    t, M, K, N = Q4_K, 32, 2048, 512
+    jobs = []
+    for i in range(2):
+        W, x = synth.weights(t, 7800 + i, N, K), synth.activations(7810 + i, M, K) * (1.0 + 3.0 * i)
+        jobs.append(dict(W=W, x=x.astype(np.float32), Wd=dev(gpu, W), xd=dev(gpu, x.astype(np.float32)),
+                         ys=[gpu.zeros((M, N), device="cuda") for _ in range(40)], rc=[]))
+    gpu.cuda.synchronize()
+    start = threading.Barrier(2)
+
+    def work(j):
+        start.wait()
+        for y in j["ys"]:
+            j["rc"].append(L.gq_qdense_f32(t, j["xd"].data_ptr(), M, K, j["Wd"].data_ptr(), N, None, 0, y.data_ptr(), None))
+
+    threads = [threading.Thread(target=work, args=(j,)) for j in jobs]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    gpu.cuda.synchronize()
+    for j in jobs:
+        assert all(rc == 0 for rc in j["rc"])
+        want = oracle.c_qdense(t, j["x"], j["W"])
+        for y in j["ys"]:
+            assert rel_err(y.cpu().numpy(), want) < TOL_F32
+
+
+def test_graph_replays_only_on_its_recording_stream(gpu):
+    import ctypes
+    from gomlx_amd import _lib
+    L = _lib.lib()
+    t, M, K, N = Q8_0, 8, 1024, 256
+    W, x = dev(gpu, synth.weights(t, 7900, N, K)), dev(gpu, synth.activations(7901, M, K))
+    y = gpu.zeros((M, N), device="cuda")
+    s1, s2 = gpu.cuda.Stream(), gpu.cuda.Stream()
+    _lib.check(L.gq_qdense_f32(t, x.data_ptr(), M, K, W.data_ptr(), N, None, 0, y.data_ptr(), s1.cuda_stream))
+    gpu.cuda.synchronize()
+    _lib.check(L.gq_graph_begin(s1.cuda_stream))
+    _lib.check(L.gq_qdense_f32(t, x.data_ptr(), M, K, W.data_ptr(), N, None, 0, y.data_ptr(), s1.cuda_stream))
+    g = ctypes.c_void_p()
+    _lib.check(L.gq_graph_end(s1.cuda_stream, ctypes.byref(g)))
+    assert L.gq_graph_launch(g, s2.cuda_stream) == _lib.ERR_INVALID
+    _lib.check(L.gq_graph_launch(g, s1.cuda_stream))
+    gpu.cuda.synchronize()
+    _lib.check(L.gq_graph_destroy(g))
+
+
 @pytest.mark.parametrize("t", ALL_TYPES)
 def test_split_k_batches_carry_the_normalisation(gpu, oracle, t):
     """In the split-K range the gain is applied where the activation image is written and the division by the root
