@@ -35,6 +35,7 @@ SIGNATURES = [
     ("gq_sync", _int, [_vp]),
     ("gq_dequantize", _int, [_int, _vp, _i64, _i64, _vp, _vp]),
     ("gq_qdense_f32", _int, [_int, _vp, _i64, _i64, _vp, _i64, _vp, _int, _vp, _vp]),
+    ("gq_qdense_f32_static", _int, [_int, _vp, _i64, _i64, _vp, _i64, _vp, _int, _vp, _vp]),
     ("gq_qdense_f32_batch", _int, [_int, _vp, _vp]),
     ("gq_qdense_bf16", _int, [_int, _vp, _i64, _i64, _vp, _i64, _vp, _int, _vp, _vp]),
     ("gq_rmsnorm_f32", _int, [_vp, _i64, _i64, _vp, ctypes.c_float, ctypes.c_float, _vp, _vp]),

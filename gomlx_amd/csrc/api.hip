@@ -47,8 +47,16 @@ int device_cu_count() { return g_cu_count.load(std::memory_order_relaxed); }
 
 // ---- scratch memory ------------------------------------------------------------------------------
 // Per-stream buffers come from the pool of workspace.hpp (sequence lock per stream, buffers pinned by
-// recorded graphs, released with their stream).
+// recorded graphs, released with their stream).  A call through gq_qdense_f32_static is served from
+// the fixed device array below instead and never allocates.
 namespace {
+
+constexpr size_t kStaticScratchBytes = (size_t)16 << 20;
+constexpr int kMaxDevices = 64;
+// Scratch of the entry point that allocates nothing.  Host code never uses this name as an address:
+// g_scratch_ptr[device] holds the array's device address, taken once in gq_init().
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+void *g_scratch_ptr[kMaxDevices] = {};
 
 int ws_alloc(void **p, size_t bytes) {
     GQ_HIP(hipMalloc(p, bytes));
@@ -77,6 +85,7 @@ struct CallScope;
 thread_local CallScope *t_scope = nullptr;
 struct CallScope {
     SeqLock lock;
+    unsigned char *static_ptr = nullptr;  // set: requests are served from the static array
     bool outer;
     CallScope() : outer(t_scope == nullptr) { if (outer) t_scope = this; }
     ~CallScope() { if (outer) t_scope = nullptr; }
@@ -87,6 +96,13 @@ struct CallScope {
 int stream_workspace(hipStream_t s, size_t bytes, void **out, int slot) {
     CallScope *sc = t_scope;
     if (!sc) return fail(GQ_ERR_INVALID, "internal: scratch memory requested outside an entry point");
+    if (sc->static_ptr) {
+        if (slot != 0 || bytes > kStaticScratchBytes)
+            return fail(GQ_ERR_INVALID, "gq_qdense_f32_static: this call needs %zu bytes of scratch memory, the static buffer holds %zu; use gq_qdense_f32",
+                        bytes, kStaticScratchBytes);
+        *out = sc->static_ptr;
+        return GQ_OK;
+    }
     if (slot < 0 || slot >= kWsSlots) return fail(GQ_ERR_INVALID, "internal: workspace slot %d", slot);
     if (!sc->lock.held()) sc->lock.lock(pool().stream(s));
     const int rc = pool().acquire(*sc->lock.held(), s, slot, bytes, out);
@@ -273,6 +289,12 @@ int gq_init(int device) {
     if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(GQ_ERR_NO_DEVICE, "gq_init: device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName);
     GQ_HIP(hipSetDevice(device));
+    if (device >= kMaxDevices) return fail(GQ_ERR_NO_DEVICE, "gq_init: device %d is beyond the %d this library keeps state for", device, kMaxDevices);
+    if (!g_scratch_ptr[device]) {  // this device's copy of the static scratch array (each device has its own, at its own address)
+        void *p = nullptr;
+        GQ_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        g_scratch_ptr[device] = p;
+    }
     g_cu_count.store(prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256);
     g_device.store(device, std::memory_order_release);
     return GQ_OK;
@@ -384,6 +406,20 @@ int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *d
     }
     if (tp) return two_pass(type, false, dX, M, K, dW, N, dBias, act, dY, (hipStream_t)stream);
     return launch_gemm(type, false, dX, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream);
+}
+
+int gq_qdense_f32_static(int type, const float *dX, int64_t M, int64_t K, const void *dW, int64_t N, const float *dBias,
+                         int act, float *dY, void *stream) {
+    if (int rc = check_dense_args("gq_qdense_f32_static", type, dX, M, K, dW, N, dBias, act, dY, 4)) return rc;
+    if (M == 0 || N == 0) return GQ_OK;
+    if (int rc = use_device()) return rc;
+    if (profile_state().active) return fail(GQ_ERR_INVALID, "gq_qdense_f32_static: kernel timing creates events; not available on this entry point");
+    if (t_scope) return fail(GQ_ERR_INVALID, "gq_qdense_f32_static: not callable from inside another entry point");
+    unsigned char *sp = static_cast<unsigned char *>(g_scratch_ptr[g_device.load(std::memory_order_acquire)]);
+    if (!sp) return fail(GQ_ERR_NO_DEVICE, "gq_qdense_f32_static: gq_init() has not taken the scratch array's address on this device");
+    CallScope scope;
+    scope.static_ptr = sp;  // every scratch request below is served from the static array, or fails
+    return gq_qdense_f32(type, dX, M, K, dW, N, dBias, act, dY, stream);
 }
 
 int gq_qdense_f32_batch(int count, const gq_dense_desc *descs, void *stream) {

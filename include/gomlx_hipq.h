@@ -106,6 +106,19 @@ int gq_dequantize(int type, const void *dW, int64_t N, int64_t K, float *dOut, v
  * one call outside a recording (gq_graph_begin) before recording the same call. ---- */
 int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *dW, int64_t N,
                   const float *dBias, int act, float *dY, void *stream);
+/* gq_qdense_f32 for callers that cannot allocate device memory (code under HIP-graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same
+ * arguments, same kernels and bit-identical results; the scratch memory that batches of 5 rows and
+ * more use (activation image, split-K partial sums) is a fixed 16 MiB device array inside the library
+ * instead of a per-stream workspace, and the call makes no hipMalloc / hipFree at all.  A problem
+ * that needs more scratch than that (the two-pass GEMM's 16-bit weight image of a large matrix, or
+ * about M * N * K / 2048 > 3.5 Mi for the split-K kernels) fails with GQ_ERR_INVALID and a message
+ * naming the size; nothing is launched then.  Every call on a GPU shares that GPU's array: calls
+ * that overlap in time on one GPU (different streams, or host threads that interleave) race; calls
+ * on one stream from one thread are ordered and safe.  Not available while gq_profile_begin() is
+ * active on the thread (event creation allocates). */
+int gq_qdense_f32_static(int type, const float *dX, int64_t M, int64_t K, const void *dW, int64_t N,
+                         const float *dBias, int act, float *dY, void *stream);
 /* bf16 activations (raw 16-bit patterns), fp32 output.  Small batches widen the activations
  * exactly and take the same GEMV / split-K kernels as fp32 activations; beyond those batch
  * sizes the weights are dequantised to bf16 operands and contracted on bf16 MFMA with fp32 accumulation. */
