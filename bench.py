@@ -1,32 +1,43 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized Dense hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1] [--others]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c4] [--no-others] [--all]
 
---config takes c0 .. c4 (the BASELINE.json configurations), prefill (C3's shape with fp32 activations), ffn (the gated feed-forward front of
-a decoder layer: the callers around the two projections folded into one launch) or layer (the
-seven projections of C4 in the order and with the dependencies of a decoder layer).
+Workloads: c0 .. c4 are the BASELINE.json configurations; prefill is C3's shape with fp32
+activations and Q4_K weights; ffn is the gated feed-forward front of a decoder layer in one
+launch; layer is C4's seven projections in the order and with the dependencies of a decoder layer.
 
-A "step" is one quantized Dense call (one pass over one weight matrix) on synthetic data that
-is already resident in HBM.  The headline workload is BASELINE.json configs[1]: Q4_0 decode
-GEMV, batch 1, K=4096 -> N=14336.  Steps rotate over enough distinct weight copies (> 512 MB)
-that every pass streams its weights from HBM rather than from the 256 MB Infinity Cache.
+The headline (--config, default c4) is the largest decode GEMV configuration in a format the
+metric names: the seven Q4_K projections of a Llama-3-8B layer at batch 1, 122.7 MB of weights in
+one batched submission.  The other BASELINE configurations (c0 .. c3) are measured in the same run
+and reported under "others" (--no-others skips them, --all adds prefill / ffn / layer).
 
-Prints ONE JSON line.  `value` is weight-GB/s over the wall clock of the K timed steps
-(submitted as one recorded HIP graph unless --no-graph).  `roofline` is the dominant kernel's
-own rate: algorithmic weight bytes per launch / mean kernel duration from start/stop HIP
-events attached to each launch on its stream (a second pass over the same K steps).
-The kernel time is taken two ways with HIP events and the smaller is used (both are upper
-bounds): events bracketing every launch, and two events around the timed region divided by K.
-`cpu_baseline` times the CPU oracle's fused fp32 restatement on the host cores (rank 0, N=1).
+A "step" is one pass of the workload over synthetic data that is already resident in HBM.  Steps
+rotate over enough distinct weight copies (> 512 MB) that every pass streams its weights from HBM
+rather than from the 256 MB Infinity Cache.
+
+Prints ONE JSON line.  `value` is weight-GB/s (or TFLOP/s) over the wall clock of exactly K timed
+steps, submitted as one recorded HIP graph unless --no-graph.  `roofline` is the dominant kernels'
+own rate: algorithmic weight bytes (or FLOP) per step / kernel time per step, the latter measured
+live with HIP events on the launch stream, two ways, the smaller taken (both bound it from above):
+start/stop events attached to every launch, and two events around a replay of the K steps.
+Per workload the line also carries: the same measurement with a single weight buffer, labelled
+cache-resident (NOT the metric); the time a plain read-only kernel takes for the same bytes (the
+rate this chip hands a one-shot kernel of that size, gomlx_amd/csrc/yardstick.hip); the HBM-side
+traffic from hardware counters (read from profiles/traffic.json, where the profiling runs put it);
+shader / memory clocks and socket power sampled while the workload loops.
+`cpu_baseline` times the CPU oracle's fused fp32 restatement (kind "port": the reference is Go and
+no Go toolchain exists here) on the host cores, on the same seeded inputs as the GPU leg.
 """
 from __future__ import annotations
 
 import argparse
 import ctypes
+import glob
 import json
 import os
 import sys
+import threading
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
@@ -35,32 +46,6 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0
-
-# HBM-side traffic per step in bytes, from hardware counters: two `rocprofv3 --pmc` passes per
-# workload (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch, summed over the step's kernels), each
-# scaled by what the same counter reads for the 64 MiB copy of --copy-calibration (FETCH_SIZE
-# reads 32780.5 KiB for 65536 KiB copied: factor 1.99924; WRITE_SIZE reads 65536.0: factor 1.0).
-# The readings are summarised under profiles/; they are properties of the kernels' access
-# pattern, not of a particular run, and are re-measured whenever a kernel changes.
-_KIB, _FETCH_SCALE, _WRITE_SCALE = 1024, 65536.0 / 32780.5, 1.0
-COUNTER_KIB = {  # workload -> (FETCH_SIZE, WRITE_SIZE) raw counter KiB per step
-    "c0": (8811.9, 16.0),
-    "c1": (16262.6, 56.0),
-    "c2": (19876.6 + 1869.1 + 921.1, 3584.0 + 512.0 + 925.8),
-    "c3": (74726.7, 32768.0),
-    "c4": (60543.5, 168.0),
-    "prefill": (4628.9 + 16401.2 + 82465.3, 32768.0 + 16448.0 + 32768.0),
-    "ffn": (32484.0, 56.0),
-    "layer": (7126.2 + 4756.1 + 32483.6 + 16449.7, 24.0 + 16.0 + 56.0 + 16.0),
-}
-
-
-def measured_traffic(name):
-    if name not in COUNTER_KIB:
-        return None
-    f, w = COUNTER_KIB[name]
-    return int(round((f * _FETCH_SCALE + w * _WRITE_SCALE) * _KIB))
-
 
 # name -> (ggml type name, M, K, N, activation dtype, bound)
 CONFIGS = {
@@ -76,13 +61,26 @@ WORKLOAD_TEXT = {
     "c1": "configs[1]: Q4_0 dense GEMV, batch 1, K=4096 -> N=14336",
     "c2": "configs[2]: Q4_K dense, decode batch M=32, K=14336 -> N=4096",
     "c3": "configs[3]: Q8_0 prefill GEMM, M=2048 bf16, K=4096, N=4096",
-    "c4": "configs[4]: seven Q4_K projections of a Llama-3-8B layer, batch 1",
+    "c4": "configs[4]: seven Q4_K projections of a Llama-3-8B layer, batch 1 (q, k, v, o, gate, up, down: 122.7 MB of weights, one batched submission)",
     "prefill": "C3's shape with fp32 activations and Q4_K weights (M=2048, K=4096, N=4096): weights to an fp16 image, activations "
                "to scaled fp16 rows, fp16 MFMA GEMM (three launches)",
     "layer": "the seven Q4_K projections of a Llama-3-8B layer as a decoder runs them, batch 1: four dependent launches "
              "(RMSNorm + q/k/v, o + residual, RMSNorm + gate/up + SiLU*mul, down + residual)",
     "ffn": "gated feed-forward front of a Llama-3-8B layer, batch 1: RMSNorm, Q4_K gate and up 4096 -> 14336, SiLU(gate) * up, one launch",
 }
+# What the path computes in (inputs and outputs are fp32 unless stated): this is `dtype` of the JSON line.
+ARITHMETIC = {
+    "c0": "f32 in/out; x -> 16-bit block fixed point (two int8 limbs per 32 values), v_dot4_i32_i8 against the int8 codes, i32 sums scaled and added in f32",
+    "c1": "f32 in/out; x -> 16-bit block fixed point (four int4 digits per 32 values), v_dot8_i32_i4 against the 4-bit codes, i32 sums scaled and added in f32",
+    "c2": "f32 in/out; x -> f16 (each row and K-slice scaled by a power of two), 4-bit codes x 6-bit scales as exact f16 integers, f16 MFMA with f32 accumulation, d / dmin and the K-slice sums in f32",
+    "c3": "bf16 activations, weights dequantised (exact f32 value, one rounding) to bf16 operands in LDS, bf16 MFMA with f32 accumulation, f32 out",
+    "c4": "f32 in/out; x -> 16-bit block fixed point (two int8 limbs per 32 values), v_dot4_i32_i8 against the 4-bit codes, i32 sums scaled (d * 6-bit scale, dmin * 6-bit minimum) and added in f32",
+    "prefill": "f32 in/out; x and dequantised W rounded to f16 operands (x rows scaled by a power of two), f16 MFMA with f32 accumulation",
+}
+ARITHMETIC["ffn"] = ARITHMETIC["layer"] = ARITHMETIC["c4"]
+DTYPE = {"c0": "int8 x int16 -> i32 dot, f32 accumulate", "c1": "int4 x int16 -> i32 dot, f32 accumulate",
+         "c2": "f16 MFMA, f32 accumulate", "c3": "bf16 MFMA, f32 accumulate", "c4": "int4 x int16 -> i32 dot, f32 accumulate",
+         "prefill": "f16 MFMA, f32 accumulate", "ffn": "int4 x int16 -> i32 dot, f32 accumulate", "layer": "int4 x int16 -> i32 dot, f32 accumulate"}
 
 
 def parse_args():
@@ -90,16 +88,156 @@ def parse_args():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=200)
     p.add_argument("--warmup", type=int, default=20)
-    p.add_argument("--config", default="c1", choices=sorted(list(CONFIGS) + ["c4", "ffn", "layer"]))
+    p.add_argument("--config", default="c4", choices=sorted(list(CONFIGS) + ["c4", "ffn", "layer"]))
     p.add_argument("--rows", type=int, default=1, help="activation rows of the ffn and layer workloads (a decode batch); default 1")
-    p.add_argument("--others", action="store_true", help="also measure the other configurations (reported under 'others')")
+    p.add_argument("--no-others", action="store_true", help="measure the headline workload only")
+    p.add_argument("--others", action="store_true", help="(default) also measure c0 .. c3; kept for older command lines")
+    p.add_argument("--all", action="store_true", help="also measure prefill, ffn and layer")
     p.add_argument("--no-graph", action="store_true", help="submit the timed steps one call at a time")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    p.add_argument("--hot", action="store_true", help="single weight buffer (Infinity-Cache resident) instead of the cold rotation")
+    p.add_argument("--no-extras", action="store_true", help="skip the cache-resident pass, the plain-read yardstick and the clock sampling")
+    p.add_argument("--hot", action="store_true", help="single weight buffer (Infinity-Cache resident) for the main measurement as well")
     p.add_argument("--copy-calibration", action="store_true",
                    help="instead of the benchmark, run a plain 64 MiB device-to-device copy kernel --steps times: the known-size "
                         "workload that hardware counter readings (FETCH_SIZE / WRITE_SIZE) are scaled by")
+    p.add_argument("--yardstick", action="store_true",
+                   help="instead of the benchmark, time the plain read-only kernel on 17.8 / 33.0 / 122.7 MB of cold weights")
     return p.parse_args()
+
+
+# ---- HBM-side traffic per step, from hardware counters ------------------------------------------------------------
+def measured_traffic(name):
+    """Bytes per step from profiles/traffic.json: FETCH_SIZE and WRITE_SIZE (KiB per dispatch, summed over the step's
+    kernels, one rocprofv3 --pmc run each), scaled by what the same counters read for the 64 MiB copy of
+    --copy-calibration.  None when the file or the entry is missing (e.g. a kernel changed and was not re-profiled)."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            t = json.load(f)
+        e, cal = t["workloads"][name], t["copy_calibration"]
+        fs = cal["copied_kib"] / cal["fetch_size_kib"]
+        ws = cal["copied_kib"] / cal["write_size_kib"]
+        return int(round((e["fetch_size_kib"] * fs + e["write_size_kib"] * ws) * 1024))
+    except (OSError, KeyError, ValueError, ZeroDivisionError):
+        return None
+
+
+# ---- clocks and power while a workload loops --------------------------------------------------------------------------
+def _read(path):
+    try:
+        with open(path) as f:
+            return f.read()
+    except OSError:
+        return None
+
+
+def _active_mhz(text):
+    if not text:
+        return None
+    for line in text.splitlines():
+        if line.rstrip().endswith("*"):
+            try:
+                return float(line.split(":")[1].lower().replace("mhz", "").replace("*", "").strip())
+            except (IndexError, ValueError):
+                return None
+    return None
+
+
+def sample_clock_state(busy_fn, seconds=0.25):
+    """Runs busy_fn() in a loop for `seconds` and samples the first GPU's sysfs clock / power files from a second thread."""
+    cards = sorted(glob.glob("/sys/class/drm/card[0-9]*/device/pp_dpm_sclk"))
+    if not cards:
+        return None
+    dev = os.path.dirname(cards[0])
+    power = sorted(glob.glob(os.path.join(dev, "hwmon", "hwmon*", "power1_average")) + glob.glob(os.path.join(dev, "hwmon", "hwmon*", "power1_input")))
+    sclk, mclk, watts, stop = [], [], [], threading.Event()
+
+    def sampler():
+        while not stop.is_set():
+            a, b = _active_mhz(_read(os.path.join(dev, "pp_dpm_sclk"))), _active_mhz(_read(os.path.join(dev, "pp_dpm_mclk")))
+            if a:
+                sclk.append(a)
+            if b:
+                mclk.append(b)
+            if power:
+                w = _read(power[0])
+                try:
+                    watts.append(float(w) / 1e6)
+                except (TypeError, ValueError):
+                    pass
+            time.sleep(0.01)
+
+    th = threading.Thread(target=sampler, daemon=True)
+    th.start()
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        busy_fn()
+    stop.set()
+    th.join()
+    if not sclk and not mclk:
+        return None
+    med = lambda v: sorted(v)[len(v) // 2] if v else None
+    return {"sclk_mhz": med(sclk), "sclk_mhz_min": min(sclk) if sclk else None, "mclk_mhz": med(mclk), "power_w": med(watts),
+            "samples": len(sclk), "source": "sysfs pp_dpm_sclk / pp_dpm_mclk / hwmon power, sampled every 10 ms while the workload loops"}
+
+
+# ---- the plain read-only kernel ---------------------------------------------------------------------------------------
+class Yardstick:
+    """gomlx_amd/libgq_yardstick.so: a kernel that loads every byte of a buffer once and does nothing else."""
+
+    def __init__(self):
+        path = os.path.join(ROOT, "gomlx_amd", "libgq_yardstick.so")
+        self.lib = ctypes.CDLL(path)
+        vp, i64 = ctypes.c_void_p, ctypes.c_int64
+        self.lib.gqy_read.argtypes = [vp, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, i64, i64, ctypes.c_int, vp, vp]
+        self.lib.gqy_read.restype = ctypes.c_int
+
+    # (workgroups, threads, loads in flight per thread): the shapes that read fastest on this chip at 18 .. 123 MB
+    SHAPES = ((2048, 256, 2), (1024, 256, 4), (512, 256, 8), (256, 512, 8))
+
+    def time_buffers(self, torch, bufs, stream, tstream, steps):
+        """Best mean time (us) per launch over SHAPES: one recorded graph of `steps` launches rotating over `bufs`."""
+        nbytes = bufs[0].numel() * bufs[0].element_size()
+        out = torch.zeros(2048 * 256 + 16, dtype=torch.int32, device="cuda")
+        best = None
+        for wgs, threads, depth in self.SHAPES:
+            def launch(i):
+                rc = self.lib.gqy_read(bufs[i % len(bufs)].data_ptr(), nbytes, 0, wgs, threads, depth, 0, 0, 0, out.data_ptr(), stream)
+                if rc:
+                    raise RuntimeError(f"gqy_read failed ({rc})")
+            for i in range(4):
+                launch(i)
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=tstream):
+                for i in range(steps):
+                    launch(i)
+            with torch.cuda.stream(tstream):  # (a torch graph replays on the current stream)
+                g.replay()
+                torch.cuda.synchronize()
+                for _ in range(3):
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record(tstream)
+                    g.replay()
+                    e1.record(tstream)
+                    torch.cuda.synchronize()
+                    us = e0.elapsed_time(e1) * 1e3 / steps
+                    if best is None or us < best[0]:
+                        best = (us, wgs, threads, depth)
+            del g
+        return best
+
+
+_YARD = None
+
+
+def yardstick():
+    global _YARD
+    if _YARD is None:
+        try:
+            _YARD = Yardstick()
+        except OSError:
+            _YARD = False
+    return _YARD or None
 
 
 class Problem:
@@ -124,7 +262,7 @@ class Problem:
             tn, M, K, N, self.dtype, self.bound = CONFIGS[name]
             shapes = [(tn, M, K, N)]
         self.parts = []
-        seed = 1000 + (int(name[1]) if name[0] == "c" else {"layer": 4, "ffn": 5, "prefill": 6}[name])
+        seed = workload_seed(name)
         total_w = 0
         for i, (tn, M, K, N) in enumerate(shapes):
             t = getattr(ggml, tn)
@@ -142,6 +280,7 @@ class Problem:
         for p in self.parts:
             for c in range(1, self.copies):
                 p["W"].append(torch.roll(p["W"][0], shifts=c, dims=0).contiguous())
+        self.use_copies = self.copies
         # one explicit stream for everything: warm-up, the recorded graph and the timed launches
         # (per-stream workspaces of the library must exist before a recording starts)
         self.tstream = torch.cuda.Stream()
@@ -149,7 +288,7 @@ class Problem:
         torch.cuda.synchronize()
 
     def launch(self, step):
-        c = step % self.copies
+        c = step % self.use_copies
         if self.name == "c4":  # the seven independent projections go out as one batched submission
             from gomlx_amd import _lib
             descs = (_lib.DenseDesc * len(self.parts))()
@@ -188,7 +327,18 @@ class Problem:
             self.check(fn(p["t"], p["x"].data_ptr(), p["M"], p["K"], p["W"][c].data_ptr(), p["N"], None, 0,
                           p["y"].data_ptr(), self.stream))
 
-    def run(self, steps, warmup, use_graph):
+    def record(self, steps, first_step):
+        L = self.L
+        self.check(L.gq_graph_begin(self.stream))
+        for s in range(steps):
+            self.launch(first_step + s)
+        g = ctypes.c_void_p()
+        self.check(L.gq_graph_end(self.stream, ctypes.byref(g)))
+        return g
+
+    def run(self, steps, warmup, use_graph, extra_replays=2):
+        """W untimed warm-up steps, then exactly K timed steps (the wall clock `value` is computed from); further
+        replays of the same K steps only refine the kernel-time estimate."""
         torch, L = self.torch, self.L
         for s in range(warmup):
             self.launch(s)
@@ -198,29 +348,30 @@ class Problem:
             if warmup == 0:
                 self.launch(0)  # creates the stream's workspace, if the path needs one
                 torch.cuda.synchronize()
-            self.check(L.gq_graph_begin(self.stream))
-            for s in range(steps):
-                self.launch(warmup + s)
-            g = ctypes.c_void_p()
-            self.check(L.gq_graph_end(self.stream, ctypes.byref(g)))
-            graph = g
+            graph = self.record(steps, warmup)
             if warmup > 0:  # untimed first replay: uploads the graph
                 self.check(L.gq_graph_launch(graph, self.stream))
             torch.cuda.synchronize()
-        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        t0 = time.perf_counter()
-        ev0.record(self.tstream)  # events on the stream the kernels are launched on
-        if graph is not None:
-            self.check(L.gq_graph_launch(graph, self.stream))
-        else:
-            for s in range(steps):
-                self.launch(warmup + s)
-        ev1.record(self.tstream)
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        self.region_us_per_step = ev0.elapsed_time(ev1) * 1e3 / steps
-        if graph is not None:
-            self.check(L.gq_graph_destroy(graph))
+
+        def timed():
+            ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t0 = time.perf_counter()
+            ev0.record(self.tstream)  # events on the stream the kernels are launched on
+            if graph is not None:
+                self.check(L.gq_graph_launch(graph, self.stream))
+            else:
+                for s in range(steps):
+                    self.launch(warmup + s)
+            ev1.record(self.tstream)
+            torch.cuda.synchronize()
+            return time.perf_counter() - t0, ev0.elapsed_time(ev1) * 1e3 / steps
+
+        wall, region = timed()  # THE timed region: exactly K steps
+        regions = [region]
+        for _ in range(extra_replays if graph is not None else 0):
+            regions.append(timed()[1])
+        self.region_us_per_step = min(regions)
+        self.graph = graph
         # second pass over the same steps: per-launch start/stop events on the launch stream
         self.check(L.gq_profile_begin())
         for s in range(steps):
@@ -233,36 +384,113 @@ class Problem:
         kernel_us_per_step = min(self.bracketed_us_per_step, self.region_us_per_step)
         return wall, kernel_us_per_step, n.value // steps
 
+    def rate(self, kernel_us):
+        if self.bound == "hbm":
+            return self.weight_bytes / (kernel_us * 1e-6) / 1e9, HBM_PEAK_GBS
+        return self.flops / (kernel_us * 1e-6) / 1e12, MFMA_BF16_PEAK_TFLOPS
+
+    def cache_resident(self, steps):
+        """The same steps on a single weight buffer (everything but the largest workloads is then served from the
+        Infinity Cache): not the metric, reported beside it."""
+        torch, L = self.torch, self.L
+        saved, self.use_copies = self.use_copies, 1
+        try:
+            for s in range(3):
+                self.launch(s)
+            torch.cuda.synchronize()
+            g = self.record(steps, 0)
+            self.check(L.gq_graph_launch(g, self.stream))
+            torch.cuda.synchronize()
+            best = None
+            for _ in range(3):
+                ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                ev0.record(self.tstream)
+                self.check(L.gq_graph_launch(g, self.stream))
+                ev1.record(self.tstream)
+                torch.cuda.synchronize()
+                us = ev0.elapsed_time(ev1) * 1e3 / steps
+                best = us if best is None else min(best, us)
+            self.check(L.gq_graph_destroy(g))
+        finally:
+            self.use_copies = saved
+        ach, peak = self.rate(best)
+        return {"kernel_us": best, "achieved": ach, "frac": ach / peak, "note": "single weight buffer: cache-resident, not the metric"}
+
+    def plain_read(self, steps):
+        """Time of the read-only kernel over the same cold bytes (concatenated weight copies of one step)."""
+        ys = yardstick()
+        if ys is None or self.bound != "hbm":
+            return None
+        torch = self.torch
+        bufs = []
+        for c in range(self.copies):
+            parts = [p["W"][c].reshape(-1) for p in self.parts]
+            bufs.append(parts[0] if len(parts) == 1 else torch.cat(parts))
+        us, wgs, threads, depth = ys.time_buffers(torch, bufs, self.stream, self.tstream, max(10, min(steps, 50)))
+        return {"us": us, "gbps": self.weight_bytes / us / 1e3, "frac_of_peak": self.weight_bytes / us / 1e3 / HBM_PEAK_GBS,
+                "grid": f"{wgs} workgroups x {threads} threads, {depth} 16-byte loads in flight per thread",
+                "note": "read-only kernel over the same cold bytes, no arithmetic: what a one-shot kernel of this size can reach"}
+
+    def clock_state(self):
+        if getattr(self, "graph", None) is None:
+            return None
+
+        def busy():
+            self.check(self.L.gq_graph_launch(self.graph, self.stream))
+            self.torch.cuda.synchronize()
+        return sample_clock_state(busy)
+
     def report(self, wall, kernel_us, steps):
         out = {}
+        ach, peak = self.rate(kernel_us)
         if self.bound == "hbm":
             out["metric"], out["unit"] = "dense GEMV weight-GB/s", "GB/s"
             out["value"] = self.weight_bytes * steps / wall / 1e9
-            ach = self.weight_bytes / (kernel_us * 1e-6) / 1e9
-            out["roofline"] = {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                               "frac": ach / HBM_PEAK_GBS, "traffic": measured_traffic(self.name) if self.rows == 1 else None,
+            out["roofline"] = {"bound": "hbm", "achieved": ach, "peak": peak, "unit": "GB/s",
+                               "frac": ach / peak, "traffic": measured_traffic(self.name) if self.rows == 1 else None,
                                "algorithmic_bytes_per_launch": self.weight_bytes, "kernel_us": kernel_us}
         else:
             out["metric"], out["unit"] = "prefill GEMM TFLOP/s", "TFLOP/s"
             out["value"] = self.flops * steps / wall / 1e12
-            ach = self.flops / (kernel_us * 1e-6) / 1e12
-            out["roofline"] = {"bound": "mfma", "achieved": ach, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                               "frac": ach / MFMA_BF16_PEAK_TFLOPS, "traffic": measured_traffic(self.name),
+            out["roofline"] = {"bound": "mfma", "achieved": ach, "peak": peak, "unit": "TFLOP/s",
+                               "frac": ach / peak, "traffic": measured_traffic(self.name),
                                "algorithmic_flops_per_launch": self.flops, "kernel_us": kernel_us}
         out["roofline"]["kernel_us_bracketed"] = self.bracketed_us_per_step
         out["roofline"]["kernel_us_region"] = self.region_us_per_step
         out["ms_per_step"] = wall / steps * 1e3
         return out
 
+    def close(self):
+        if getattr(self, "graph", None) is not None:
+            self.check(self.L.gq_graph_destroy(self.graph))
+            self.graph = None
+
+
+def workload_seed(name):
+    return 1000 + (int(name[1]) if name[0] == "c" else {"layer": 4, "ffn": 5, "prefill": 6}[name])
+
+
+def host_threads():
+    """Threads for the CPU baseline: the CPUs this process may run on, within the share the box grants a one-GPU job
+    (it exports OMP_NUM_THREADS for that)."""
+    try:
+        n = len(os.sched_getaffinity(0))
+    except (AttributeError, OSError):
+        n = os.cpu_count() or 1
+    try:
+        cap = int(os.environ.get("OMP_NUM_THREADS", "0"))
+    except ValueError:
+        cap = 0
+    return max(1, min(n, cap) if cap > 0 else n)
+
 
 def cpu_baseline(name):
-    """The CPU oracle's fused fp32 restatement on the host cores (checker code used as a
-    reported baseline only): >= 2 warm-ups, then >= 5 runs and >= 3 s, like the reference's own
-    timing protocol (internal/perf/dotgeneral_perf_test.go:366-381), capped at ~25 s."""
-    import numpy as np
+    """The CPU oracle's fused fp32 restatement on the host cores (checker code used as a reported baseline only), on the
+    inputs the GPU leg uses (same seeds): >= 2 warm-ups, then >= 5 runs and >= 3 s, like the reference's own timing
+    protocol (internal/perf/dotgeneral_perf_test.go:366-381), capped at ~25 s."""
     from gomlx_amd import ggml, synth
     from oracle import ggml_oracle as oracle
-    cores = min(os.cpu_count() or 1, 16)
+    cores = host_threads()
     if name in ("c4", "layer"):
         shapes = [("Q4_K", 1, K, N) for K, N in C4_SHAPES]
     elif name == "ffn":  # the two projections; the normalisation and the product are negligible beside them
@@ -271,13 +499,21 @@ def cpu_baseline(name):
         tn, M, K, N, _, _ = CONFIGS[name]
         shapes = [(tn, M, K, N)]
     sample = "full workload"
-    if name in ("c3", "prefill"):  # 34 GMAC per pass is minutes of CPU time: a 64-row slice of the 2048 activations
-        shapes = [(CONFIGS[name][0], 64, 4096, 4096)]
-        sample = "64 of the 2048 activation rows (1/32 of the FLOPs), all of W"
+    rows = None
+    if name in ("c3", "prefill"):  # 34 GMAC per pass is minutes of CPU time: the first 64 of the 2048 activation rows
+        rows = 64
+        sample = "the first 64 of the 2048 activation rows (1/32 of the FLOPs), all of W"
+    seed = workload_seed(name)
     probs = []
     for i, (tn, M, K, N) in enumerate(shapes):
         t = getattr(ggml, tn)
-        probs.append((t, synth.activations(5 + i, M, K), synth.weights(t, 6 + i, N, K)))
+        x = synth.activations(seed + 100 + i, M, K)
+        if rows:
+            x = x[:rows]
+        if name == "c3":
+            import torch
+            x = torch.from_numpy(x).to(torch.bfloat16).to(torch.float32).numpy()
+        probs.append((t, x, synth.weights(t, seed + i, N, K)))
     wbytes = sum(p[2].size for p in probs)
     flops = sum(2 * p[1].shape[0] * p[1].shape[1] * p[2].shape[0] for p in probs)
 
@@ -294,11 +530,11 @@ def cpu_baseline(name):
         if (runs >= 5 and el >= 3.0) or el >= 25.0:
             break
     per = el / runs
+    common = {"cores": cores, "host_cpus": os.cpu_count(), "kind": "port",
+              "sample": f"{sample}, same seeded inputs as the GPU leg; {runs} runs, {per * 1e3:.2f} ms each; OpenMP over output rows"}
     if name in ("c3", "prefill"):
-        return {"value": flops / per / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
-                "sample": f"{sample}; {runs} runs, {per * 1e3:.2f} ms each"}
-    return {"value": wbytes / per / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
-            "sample": f"{sample}; {runs} runs, {per * 1e3:.2f} ms each"}
+        return {"value": flops / per / 1e12, "unit": "TFLOP/s", **common}
+    return {"value": wbytes / per / 1e9, "unit": "GB/s", **common}
 
 
 def copy_calibration(torch, steps):
@@ -312,6 +548,25 @@ def copy_calibration(torch, steps):
         torch.add(srcs[s % len(srcs)], 0.0, out=dst)
     torch.cuda.synchronize()
     print(json.dumps({"copy_calibration": True, "launches": steps, "read_bytes_per_launch": n * 4, "write_bytes_per_launch": n * 4}))
+
+
+def yardstick_only(torch, steps):
+    """The plain read-only kernel on cold buffers of the three decode workloads' sizes."""
+    ys = yardstick()
+    if ys is None:
+        print("bench.py: gomlx_amd/libgq_yardstick.so is missing (python -m gomlx_amd.build)", file=sys.stderr)
+        sys.exit(4)
+    tstream = torch.cuda.Stream()
+    out = {"yardstick": "read-only kernel, every byte loaded once, no arithmetic; cold: rotation over > 512 MB of distinct buffers", "sizes": {}}
+    for name, nbytes in (("c0", 17825792), ("c1", 33030144), ("c2", 33030144), ("c4", 122683392)):
+        copies = max(2, -(-(512 << 20) // nbytes) + 1)
+        bufs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device="cuda") for _ in range(copies)]
+        us, wgs, threads, depth = ys.time_buffers(torch, bufs, tstream.cuda_stream, tstream, steps)
+        out["sizes"][name] = {"bytes": nbytes, "us": us, "gbps": nbytes / us / 1e3, "frac_of_peak": nbytes / us / 1e3 / HBM_PEAK_GBS,
+                              "grid": f"{wgs} x {threads}, depth {depth}", "copies": copies}
+        del bufs
+        torch.cuda.empty_cache()
+    print(json.dumps(out))
 
 
 def main():
@@ -328,48 +583,61 @@ def main():
     if args.copy_calibration:
         copy_calibration(torch, args.steps)
         return
+    if args.yardstick:
+        yardstick_only(torch, min(args.steps, 50))
+        return
     from gomlx_amd import _lib
     _lib.init(0)
 
-    def measure(name):
+    def measure(name, steps):
         prob = Problem(torch, name, hot=args.hot, rows=args.rows)
-        wall, kus, launches = prob.run(args.steps, args.warmup, not args.no_graph)
-        rep = prob.report(wall, kus, args.steps)
+        wall, kus, launches = prob.run(steps, args.warmup, not args.no_graph)
+        rep = prob.report(wall, kus, steps)
         rep["weight_copies"] = prob.copies
         rep["launches_per_step"] = launches
+        if not args.no_extras:
+            if not args.hot:
+                rep["roofline"]["cache_resident"] = prob.cache_resident(steps)
+            pr = prob.plain_read(steps)
+            if pr is not None:
+                pr["kernel_over_plain_read"] = rep["roofline"]["kernel_us"] / pr["us"]
+                rep["roofline"]["plain_read"] = pr
+            rep["clock_state"] = prob.clock_state()
+        prob.close()
         del prob
         torch.cuda.empty_cache()
         return rep
 
-    rep = measure(args.config)
+    rep = measure(args.config, args.steps)
     tn = "Q4_K" if args.config in ("c4", "ffn", "layer") else CONFIGS[args.config][0]
     line = {
         "metric": rep["metric"], "value": rep["value"], "unit": rep["unit"], "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": rep["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": {"c3": "bf16", "prefill": "f16"}.get(args.config, "f32"), "data": "synthetic",
+        "dtype": DTYPE[args.config], "data": "synthetic",
         "config": {"workload": WORKLOAD_TEXT[args.config] + (f" [run with {args.rows} activation rows]" if args.rows != 1 and args.config in ("ffn", "layer") else ""),
                    "ggml_type": tn,
+                   "arithmetic": ARITHMETIC[args.config],
                    "weights": "cache-resident single buffer" if args.hot else
                    f"cold: rotation over {rep['weight_copies']} distinct weight copies",
                    "submission": "eager" if args.no_graph else "one recorded HIP graph of all timed steps",
                    "launches_per_step": rep["launches_per_step"]},
         "roofline": rep["roofline"],
+        "clock_state": rep.get("clock_state"),
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(args.config)
-    if args.others:
+    if not args.no_others:
+        names = ["c0", "c1", "c2", "c3", "c4"] + (["prefill", "ffn", "layer"] if args.all else [])
         others = {}
-        for name in ["c0", "c1", "c2", "c3", "c4", "prefill", "ffn", "layer"]:
+        for name in names:
             if name == args.config:
                 continue
             steps = args.steps if name not in ("c3", "prefill") else max(10, args.steps // 10)
-            saved = args.steps
-            args.steps = steps
-            r = measure(name)
-            args.steps = saved
-            others[name] = {"workload": WORKLOAD_TEXT[name], "metric": r["metric"], "value": r["value"], "unit": r["unit"],
-                            "ms_per_step": r["ms_per_step"], "roofline": r["roofline"], "steps": steps}
+            r = measure(name, steps)
+            others[name] = {"workload": WORKLOAD_TEXT[name], "dtype": DTYPE[name], "arithmetic": ARITHMETIC[name], "metric": r["metric"],
+                            "value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"], "roofline": r["roofline"],
+                            "clock_state": r.get("clock_state"), "steps": steps, "launches_per_step": r["launches_per_step"]}
         line["others"] = others
     print(json.dumps(line))
 

@@ -16,6 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "csrc", "build")
 LIB = os.path.join(HERE, "libgomlx_hipq.so")
+YARDSTICK_LIB = os.path.join(HERE, "libgq_yardstick.so")  # read-only kernels for the benchmark; not part of the product library
 
 HOST = os.path.join(HERE, "host")
 HOST_TEST = os.path.join(HOST, "build", "hipq_backend_test")
@@ -94,6 +95,12 @@ def build(verbose: bool = True) -> str:
         raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
     if verbose:
         print(f"built {LIB}")
+    cmd = [hipcc(), *[f for f in HIPCC_FLAGS if not f.startswith("-Rpass")], "-shared", os.path.join(CSRC, "yardstick.hip"), "-o", YARDSTICK_LIB]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"yardstick build failed:\n{r.stdout}\n{r.stderr}")
+    if verbose:
+        print(f"built {YARDSTICK_LIB}")
     build_host_test(verbose)
     return LIB
 
