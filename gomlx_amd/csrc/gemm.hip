@@ -167,9 +167,6 @@ template <> struct XRaw<false> {
     }
 };
 
-#ifdef GQ_GEMM_TRACE
-__device__ unsigned long long g_gemm_trace[4 * 8 * 8];
-#endif
 
 // X must be 16-byte aligned; K % 32 == 0.
 template <int T, bool BF16>
@@ -218,14 +215,7 @@ __global__ __launch_bounds__(512) void gemm_kernel(const void *Xv, const uint8_t
     const uint8_t *xtile = reinterpret_cast<const uint8_t *>(Xv) + (int64_t)bm * K * XRaw<BF16>::ESIZE;
     const uint8_t *wtile = W + (int64_t)bn * row_bytes;
     auto fetch = [&](int kt, XRaw<BF16> &x, WRaw<T> &w) __attribute__((always_inline)) {  // unconditional: steps past the end re-read the last one
-#ifdef GQ_GEMM_NOFETCH  // tuning builds only
-        if (kt > 2) return;
-#endif
-#ifdef GQ_GEMM_HOTFETCH  // tuning builds only: every step re-reads step 0
-        const int kc = min(kt, 0);
-#else
         const int kc = min(kt, nk - 1);  // uniform
-#endif
         const bool tail = ktail && kc == nk - 1;
         const uint8_t *xb = xtile + (int64_t)kc * (BK * XRaw<BF16>::ESIZE);
         uint32_t o[XRaw<BF16>::NCH];
@@ -235,11 +225,6 @@ __global__ __launch_bounds__(512) void gemm_kernel(const void *Xv, const uint8_t
         w.load(wtile + (int64_t)kc * (BK / 32 * 34), tail ? woff_t : woff, (uint32_t)wrun,
                min((int64_t)kc * (BK / 16) + wrun, n16 - 1));
     };
-#ifdef GQ_GEMM_TRACE  // tuning builds only: cycle stamps of one pair of steps per wavefront
-#define GEMM_TRACE(slot) do { if (kt == 16 && lane == 0 && blockIdx.x < 4 && blockIdx.y == 0) g_gemm_trace[(blockIdx.x * 8 + wave) * 8 + (slot)] = __builtin_readcyclecounter(); } while (0)
-#else
-#define GEMM_TRACE(slot) do { } while (0)
-#endif
     // One K step.  The MFMAs run in four groups of four, each group followed in program order by a
     // quarter of the staging of step kt + 1 into `nxt` (MFMAs are issued asynchronously, so the
     // vector ALU work that follows them runs in their shadow).  Fragments are read one group ahead,
@@ -252,23 +237,17 @@ __global__ __launch_bounds__(512) void gemm_kernel(const void *Xv, const uint8_t
     constexpr bool SKEW = BF16;
     typename Op::vec8 fa[2][2], fb[2][2];  // [set][tile]; with SKEW set 1 carries group 3 across the barrier
     auto mfma_group = [&](int set) __attribute__((always_inline)) {
-#ifndef GQ_GEMM_NOMFMA  // tuning builds only
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int j = 0; j < 2; j++) acc[i][j] = Op::mfma(fa[set][i], fb[set][j], acc[i][j]);
-#endif
     };
     auto step = [&](int kt, const uint16_t *cur, uint16_t *nxt, XRaw<BF16> &x, WRaw<T> &wq, auto masked, auto first) __attribute__((always_inline)) {
         constexpr bool MASKED = decltype(masked)::value, FIRST = decltype(first)::value;
         const uint16_t *xs = cur, *ws = cur + BM * LDS_STRIDE;
         const int k1 = (kt + 1) * BK;
         // the register set staged here is refilled, piece by piece, with step kt + 3
-#ifdef GQ_GEMM_HOTFETCH  // tuning builds only: every step re-reads step 0
-        const int kc = 0;
-#else
         const int kc = min(kt + 3, nk - 1);  // uniform; steps past the end re-read the last one
-#endif
         const bool ftail = ktail && kc == nk - 1;
         const uint8_t *xb = xtile + (int64_t)kc * (BK * XRaw<BF16>::ESIZE);
         uint32_t fo[XRaw<BF16>::NCH];
@@ -296,25 +275,18 @@ __global__ __launch_bounds__(512) void gemm_kernel(const void *Xv, const uint8_t
                 if (kk < 3) frags(kk + 1);
                 mfma_group(kk & 1);
             }
-#ifndef GQ_GEMM_NOSTAGE  // tuning builds only
             x.template store_part<MASKED>(kk, nxt, k1, K, tid);
             wq.part(kk, w);
-#endif
-#ifndef GQ_GEMM_NOFETCH
             x.load_part(kk, xb, fo);
-#endif
             if (kk == 1 || kk == 3) {
                 const int o = (kk >> 1) * 8;
                 wd[kk >> 1] = make_uint4(Op::pack(w[o], w[o + 1]) & wmask, Op::pack(w[o + 2], w[o + 3]) & wmask,
                                          Op::pack(w[o + 4], w[o + 5]) & wmask, Op::pack(w[o + 6], w[o + 7]) & wmask);
             }
             __builtin_amdgcn_sched_barrier(0);
-            if (cur == lds) GEMM_TRACE(1 + kk);
         }
-#ifndef GQ_GEMM_NOFETCH
         wq.load(wtile + (int64_t)kc * (BK / 32 * 34), ftail ? woff_t : woff, (uint32_t)wrun,
                 min((int64_t)kc * (BK / 16) + wrun, n16 - 1));
-#endif
     };
     auto stage_first = [&](uint16_t *buf, const XRaw<BF16> &x, const WRaw<T> &wq) __attribute__((always_inline)) {
         float w[16];
@@ -347,15 +319,11 @@ __global__ __launch_bounds__(512) void gemm_kernel(const void *Xv, const uint8_t
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
     auto pair = [&](int kt, auto masked, auto first) __attribute__((always_inline)) {
-        GEMM_TRACE(0);
         step(kt, lds, lds + LDS_BUF, xr[1], wr[1], masked, first);
         __builtin_amdgcn_sched_barrier(0);
-        GEMM_TRACE(5);
         __syncthreads();
-        GEMM_TRACE(6);
         step(kt + 1, lds + LDS_BUF, lds, xr[0], wr[0], masked, std::false_type());
         __builtin_amdgcn_sched_barrier(0);
-        GEMM_TRACE(7);
         __syncthreads();
     };
     // The first pair runs outside the loop so that the loop is entered with exactly the loads in

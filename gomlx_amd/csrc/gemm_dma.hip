@@ -309,14 +309,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const 
     const uint32_t xdst = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)(G::XI * wave) * 1024u);
     const uint32_t wdst = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)(G::DM * ROWB) + (uint32_t)(G::WI * wave) * 1024u);
     auto issue = [&](int kt, int stage) __attribute__((always_inline)) {  // steps past the end re-read the last one (the data is never used)
-#ifdef GQ_DMA_NOISSUE  // tuning builds only: nothing is loaded after the prologue
-        if (kt > 1) return;
-#endif
-#ifdef GQ_DMA_HOT  // tuning builds only: every step re-reads step 0
-        const uint32_t soff = 0;
-#else
         const uint32_t soff = (uint32_t)min(kt, nk - 1) * (uint32_t)(DK * 2);
-#endif
         const uint32_t sb = (uint32_t)stage * (uint32_t)G::kStageBytes;
 #pragma unroll
         for (int j = 0; j < G::XI; j++) dma16(xdst + sb + (uint32_t)j * 1024u, xrsrc, xvoff[j], soff);

@@ -144,9 +144,6 @@ template <> struct KS<kQ4_0> {
     // xq[4 h + w] = planes facing dword w of block h
     static __device__ __forceinline__ float dot(const Raw &r, const uint4 *xq, const float *xsc, const float *, int) {
         const uint32_t *v = r.v;
-#ifdef GQ_KS_NODOT  // tuning builds only: consume the loads without the arithmetic
-        { uint32_t a = xq[0].x; for (int i = 0; i < 9; i++) a ^= v[i]; return __builtin_bit_cast(float, a) * xsc[0]; }
-#endif
         float out = 0.f;
 #pragma unroll
         for (int h = 0; h < 2; h++) {
@@ -421,14 +418,6 @@ __device__ __forceinline__ void ks_load(typename KS<T>::Raw &r, const uint8_t *p
     else KS<T>::load(r, p);
 }
 
-#ifdef GQ_KS_TRACE
-__device__ unsigned long long g_ks_trace[4096 * 16];
-#define KS_TRACE(k) do { if (lane == 0) g_ks_trace[((size_t)wg * waves + wave) % 4096 * 16 + (k)] = __builtin_readcyclecounter(); } while (0)
-#define KS_TRACE_WALL(k) do { if (lane == 0) g_ks_trace[((size_t)wg * waves + wave) % 4096 * 16 + (k)] = __builtin_amdgcn_s_memrealtime(); } while (0)
-#else
-#define KS_TRACE(k) do { } while (0)
-#define KS_TRACE_WALL(k) do { } while (0)
-#endif
 
 constexpr int kWaveLdsDwords = 76 * 4;  // per wavefront: 64 uint4 of planes, 16 scales, up to 32 sums
 
@@ -541,8 +530,6 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8
         float *my_sums = my_scales + 16;
         float *part = all + wave * R * rows_wg;
 
-        KS_TRACE(0);
-        KS_TRACE_WALL(12);
         const int spw = (nslices - wave + waves - 1) / waves;  // slices of this wavefront (>= 1)
         XRaw xr = x_fetch(wave);
         const int last_row = N - 1;
@@ -557,7 +544,6 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8
         Raw buf[PF];
 #pragma unroll
         for (int j = 0; j < WIN; j++) ks_load<T>(buf[j], addr(0, j), lane_c(0));
-        KS_TRACE(1);
 
         uint4 xq[R][8];
         constexpr int NS = KS<T>::kScales, SPAN = KS<T>::kSumSpan;
@@ -590,9 +576,7 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8
             }
         };
         stage(xr);
-        KS_TRACE(2);
         if (spw > 1) xr = x_fetch(wave + waves);
-        KS_TRACE(3);
 
         const int ngroups = spw * (iters / PF);
         int j = 0, i0 = 0;  // slice index and first row-step of the current group
@@ -624,8 +608,6 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8
             j = nj;
             i0 = ni0;
         }
-        KS_TRACE(14);
-        KS_TRACE_WALL(13);
         if constexpr (EXT) {
             if (ext.norm) {
 #pragma unroll

@@ -334,14 +334,6 @@ template <> struct JointSum<2> {
 // Order of issue matters: vector-memory loads return in order, so the (small, cache-resident)
 // activation loads go out first and the PF rows of codes right behind them; the wait for the
 // activations then leaves the code loads in flight while the digit planes are being built.
-#ifdef GQ_XS_TRACE
-__device__ unsigned long long g_xs_trace[4096 * 16];
-#define XS_TRACE(k) do { if (lane == 0) g_xs_trace[((size_t)wg * (blockDim.x >> 6) + wave) % 4096 * 16 + (k)] = __builtin_readcyclecounter(); } while (0)
-#define XS_TRACE_WALL(k) do { if (lane == 0) g_xs_trace[((size_t)wg * (blockDim.x >> 6) + wave) % 4096 * 16 + (k)] = __builtin_amdgcn_s_memrealtime(); } while (0)
-#else
-#define XS_TRACE(k) do { } while (0)
-#define XS_TRACE_WALL(k) do { } while (0)
-#endif
 
 template <int T, int PF>
 __device__ __forceinline__ void gemv_xs_body(const float *__restrict__ x, const uint8_t *__restrict__ W,
@@ -372,8 +364,6 @@ __device__ __forceinline__ void gemv_xs_body(const float *__restrict__ x, const 
     // host only selects this kernel when that covers K).  The loads sit in blocks of their own
     // so that they are issued here, ahead of the code loads, and not next to their use.
     const int nrounds = (nitems + nthreads - 1) / nthreads;
-    XS_TRACE(0);
-    XS_TRACE_WALL(12);
     constexpr int kMaxRounds = XS<T>::kMaxRounds;
     Item its[kMaxRounds];
 #pragma unroll
@@ -388,7 +378,6 @@ __device__ __forceinline__ void gemv_xs_body(const float *__restrict__ x, const 
     XS<T>::load(buf[0], W + (int64_t)min(first, my_last) * row_bytes, uc);
 
     // 2. activations -> digit planes (LDS) -> registers of the owning lanes
-    XS_TRACE(1);
 #pragma unroll
     for (int m = 0; m < kMaxRounds; m++) {
         if (m < nrounds) {
@@ -398,9 +387,7 @@ __device__ __forceinline__ void gemv_xs_body(const float *__restrict__ x, const 
     }
 #pragma unroll
     for (int j = 1; j < PF; j++) XS<T>::load(buf[j], W + (int64_t)min(first + j, my_last) * row_bytes, uc);
-    XS_TRACE(2);
     __syncthreads();
-    XS_TRACE(3);
     uint32_t xq[NX];
     {
         const uint4 *l4 = reinterpret_cast<const uint4 *>(lds);
@@ -411,7 +398,6 @@ __device__ __forceinline__ void gemv_xs_body(const float *__restrict__ x, const 
         }
     }
 
-    XS_TRACE(4);
     // 3. stream over the rows, PF at a time.  All groups but the last also fetch the next
     // group's rows (rows past the wavefront's range are clamped to its own last row).
     float mine = 0.f;  // lane i: result of this wavefront's i-th row (its slice of K)
@@ -451,8 +437,6 @@ __device__ __forceinline__ void gemv_xs_body(const float *__restrict__ x, const 
         finish_group(part, i0);
     }
 
-    XS_TRACE(14);
-    XS_TRACE_WALL(13);
     // 4. combine the S slices of every row and write
     if (S == 1) {
         const int row = first + lane;

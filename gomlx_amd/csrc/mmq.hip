@@ -185,12 +185,6 @@ __device__ __forceinline__ void load_sb(RawSB &r, const uint8_t *sb, int kg) {
     for (int st = 0; st < 4; st++) r.c[st] = *reinterpret_cast<const uint4 *>(sb + 16 + 32 * st + 16 * kg);
 }
 
-#ifdef GQ_MMQ_TRACE
-__device__ unsigned long long g_mmq_trace[4096 * 8];
-#define MMQ_TRACE(k) do { if (lane == 0) g_mmq_trace[(((size_t)blockIdx.y * gridDim.x + blockIdx.x) * (4 * kParts) + wave) % 4096 * 8 + (k)] = (k) >= 6 ? __builtin_amdgcn_s_memrealtime() : __builtin_readcyclecounter(); } while (0)
-#else
-#define MMQ_TRACE(k) do { } while (0)
-#endif
 
 // Activation pre-pass: writes each (K-slice, column tile)'s LDS image (fragment-ordered fp16
 // activations + sub-block sums) to global memory once; the row-range workgroups of the main
@@ -233,8 +227,6 @@ __global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__
     const int n = blockIdx.x * kRowsPerWG + rt * 32 + col;  // this lane's weight row
     const uint8_t *wrow = W + (int64_t)min(n, N - 1) * row_bytes + (int64_t)(k0 >> 8) * 144;
 
-    MMQ_TRACE(0);
-    MMQ_TRACE(6);
     // the slice's activation image goes straight from global memory into LDS (no registers)
     {
         const uint8_t *img = ximg + ((size_t)(m0 / kMT) * gridDim.y + slice) * kLdsBytes;
@@ -248,9 +240,7 @@ __global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__
     }
     RawSB cur;
     load_sb(cur, wrow + (int64_t)min(par, nsb - 1) * 144, kg);
-    MMQ_TRACE(1);
     __syncthreads();
-    MMQ_TRACE(2);
 
     f16v acc, acc2;
 #pragma unroll
@@ -325,7 +315,6 @@ __global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__
     }
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] -= acc2[r];
-    MMQ_TRACE(3);
 
     // wavefronts 1..kParts-1 of a row tile hand their 32 x 32 partial tiles to wavefront 0 through LDS
     __syncthreads();
@@ -335,7 +324,6 @@ __global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__
         for (int r = 0; r < 16; r++) xch[((par - 1) * 16 + r) * 64 + lane] = acc[r];
     }
     __syncthreads();
-    MMQ_TRACE(7);
     if (par == 0 && n < N) {
         // lane holds y[m = 8 (r / 4) + 4 kg + r % 4][n] for its K-slice
 #pragma unroll

@@ -20,7 +20,11 @@
  *   Q4_K dequant          PARITY UNPINNED at the reference: the only implementation lives in the
  *                         third-party module github.com/gomlx/compute v0.1.2 (package gobackend),
  *                         which is not vendored.  Restated from the public GGML block_q4_K
- *                         specification; self-consistency checks only.
+ *                         specification.  What stays open is the BYTE LAYOUT only: given the fields,
+ *                         the value is fixed by the mathematics - d*sc, (d*sc)*q, d*(sc*q) and dmin*m
+ *                         are exact in binary32, so w = fl(d*sc*q - dmin*m) is one correctly rounded
+ *                         subtraction under every order of operations, with or without a fused
+ *                         multiply-add (checked against exact rationals rounded once).
  *   Q6_K dequant          PARITY UNPINNED at the reference, for the same reason (the reference names
  *                         the type, docs/CHANGELOG.md:251-252, but holds neither its arithmetic nor a
  *                         test vector).  Restated from the public GGML block_q6_K specification;

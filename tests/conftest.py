@@ -35,3 +35,22 @@ def gpu():
     from gomlx_amd import _lib
     _lib.init(0)
     return torch
+
+
+def pytest_terminal_summary(terminalreporter):
+    """Margins of the GPU parity tests: per test, the worst max-norm error and the worst per-element error scaled by
+    rms(want) over all comparisons it made."""
+    mod = sys.modules.get("tests.test_parity_gpu") or sys.modules.get("test_parity_gpu")
+    margins = getattr(mod, "MARGINS", None)
+    if not margins:
+        return
+    terminalreporter.write_line("parity margins: test, max|d|/max|want|, max|d|/rms(want)")
+    for name, (a, b) in sorted(margins.items(), key=lambda kv: -kv[1][1])[:25]:
+        terminalreporter.write_line(f"  {name:64s} {a:9.2e} {b:9.2e}")
+    try:
+        out = os.path.join(ROOT, "gpurun_out")
+        os.makedirs(out, exist_ok=True)
+        with open(os.path.join(out, "parity_margins.json"), "w") as f:
+            json.dump({k: {"max_norm": v[0], "rms_scaled": v[1]} for k, v in margins.items()}, f, indent=1)
+    except OSError:
+        pass

@@ -31,6 +31,28 @@ def round_fraction_to_f32(fr: Fraction) -> np.float32:
     return np.float32(float(fr))
 
 
+def exact_round_f32(fr: Fraction) -> np.float32:
+    """Round-to-nearest-even of an exact rational to binary32, in integer arithmetic (no double in between)."""
+    if fr == 0:
+        return np.float32(0.0)
+    sign, a = (-1, -fr) if fr < 0 else (1, fr)
+    n, d = a.numerator, a.denominator
+    e = n.bit_length() - d.bit_length()          # 2^e <= a < 2^(e+2), roughly
+    if Fraction(2) ** e > a:
+        e -= 1
+    e = max(e, -126)                             # below 2^-126 the spacing stays 2^-149
+    q = a / Fraction(2) ** (e - 23)              # in units of the last place
+    m, rem = divmod(q.numerator, q.denominator)
+    twice = 2 * rem
+    if twice > q.denominator or (twice == q.denominator and (m & 1)):
+        m += 1
+    return np.float32(sign * float(m) * float(2.0 ** (e - 23)))   # m < 2^25 and a power of two: exact in double
+
+
+def is_exact_f32(fr: Fraction) -> bool:
+    return Fraction(float(exact_round_f32(fr))) == fr
+
+
 def half_value(bits: int) -> Fraction:
     """Exact value of a finite binary16 pattern."""
     s = -1 if bits & 0x8000 else 1
@@ -266,6 +288,44 @@ def test_q4_k_full_block_against_exact_arithmetic(oracle, impl):
             prod = round_fraction_to_f32(Fraction(float(ds)) * codes[i])   # ds * q rounded
             want = round_fraction_to_f32(Fraction(float(prod)) - Fraction(float(dm)))
             assert got[0, i] == want, (trial, i)
+
+
+@pytest.mark.parametrize("impl", ["np", "c"])
+def test_q4_k_value_is_one_correctly_rounded_subtraction(oracle, impl):
+    """w = d*sc*q - dmin*m needs ONE rounding whatever the order of operations: d*sc (11 + 6 bits), (d*sc)*q and d*(sc*q)
+    (<= 21 bits) and dmin*m (<= 17 bits) are all exact in binary32, so every association of the products, with or
+    without a fused multiply-add for the subtraction, yields fl(d*sc*q - dmin*m).  The oracle is compared with that
+    closed form, rounded once from exact rationals; what this leaves open about the external Go code is the byte layout
+    alone, not its arithmetic."""
+    rng = np.random.default_rng(2024)
+    dpats = [0x0001, 0x0155, 0x03FF, 0x0400, 0x1A00, 0x2E66, 0x3555, 0x3C00, 0x3FFF, 0x7BFF, 0x4D2B, 0x12AB]
+    for trial in range(40):
+        dbits, dminbits = dpats[trial % len(dpats)], dpats[(5 * trial + 3) % len(dpats)]
+        if trial >= 24:
+            dbits, dminbits = int(rng.integers(1, 0x7C00)), int(rng.integers(1, 0x7C00))
+        sc = [int(v) for v in rng.integers(0, 64, 8)]
+        mn = [int(v) for v in rng.integers(0, 64, 8)]
+        sc[0], mn[0], sc[1], mn[1] = 63, 63, 63, 0
+        codes = [int(v) for v in rng.integers(0, 16, 256)]
+        codes[0], codes[1], codes[32] = 15, 0, 15
+        W = make_q4k_block(dbits, dminbits, sc, mn, codes)[None, :]
+        got = oracle.np_dequantize(Q4_K, W) if impl == "np" else oracle.c_dequantize(Q4_K, W, 256)
+        d, dmin = half_value(dbits), half_value(dminbits)
+        for i in range(256):
+            j, q = i // 32, codes[i]
+            # every intermediate product is a binary32 number: no association of the multiplications rounds
+            assert is_exact_f32(d * sc[j]) and is_exact_f32(d * sc[j] * q) and is_exact_f32(d * (sc[j] * q)) and is_exact_f32(dmin * mn[j])
+            want = exact_round_f32(d * sc[j] * q - dmin * mn[j])
+            assert got[0, i] == want, (trial, i, dbits, dminbits)
+
+
+def test_exact_rounding_helper():
+    for v in (Fraction(1, 3), Fraction(-7, 5), Fraction(1, 1 << 140), Fraction(3, 1 << 149), Fraction((1 << 24) + 1, 1), Fraction((1 << 25) + 2, 3),
+              Fraction(16777215, 1 << 150), Fraction(1, 1 << 150)):
+        assert exact_round_f32(v) == np.float32(float(v)), v   # (doubles are exact or far from a tie for these)
+    assert exact_round_f32(Fraction((1 << 24) + 1, 1)) == np.float32(16777216.0)       # tie to even
+    assert exact_round_f32(Fraction((1 << 24) + 3, 1)) == np.float32(16777220.0)
+    assert exact_round_f32(Fraction(1, 1 << 150)) == np.float32(0.0)                   # half the smallest subnormal: tie to even
 
 
 @pytest.mark.parametrize("impl", ["np", "c"])

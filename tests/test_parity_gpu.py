@@ -26,9 +26,25 @@ def dev(torch, a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
 
+# test name -> [worst max|d| / max|want|, worst max|d| / rms(want)] over every comparison the test made; printed at the end
+# of the session (tests/conftest.py) so that the margin to the bounds is visible per kernel family.
+MARGINS = {}
+
+
+def rms_err(got, want):
+    """The per-element form of the bound: the largest |got - want| over rms(want) (|d| <= tol * rms(want) for every element)."""
+    rms = float(np.sqrt(np.mean(np.square(want.astype(np.float64))))) or 1.0
+    return float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)))) / rms
+
+
 def rel_err(got, want):
+    import os
     scale = float(np.max(np.abs(want))) or 1.0
-    return float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)))) / scale
+    err = float(np.max(np.abs(got.astype(np.float64) - want.astype(np.float64)))) / scale
+    key = os.environ.get("PYTEST_CURRENT_TEST", "?").split("::")[-1].split(" ")[0].split("[")[0]
+    rec = MARGINS.setdefault(key, [0.0, 0.0])
+    rec[0], rec[1] = max(rec[0], err), max(rec[1], rms_err(got, want))
+    return err
 
 
 def run_dense(torch, t, x, W, bias=None, act=0, bf16=False):
@@ -669,6 +685,31 @@ def test_dense_with_rmsnorm_and_residual(gpu, oracle, t):
                                               gpu.cuda.current_stream().cuda_stream))
     gpu.cuda.synchronize()
     assert rel_err(yd.cpu().numpy(), oracle.c_qdense(t, x, W) + res) < TOL_F32
+
+
+# Bounds of the per-element form |got - want| <= tol * rms(want), by route.  For Gaussian outputs max|want| is 3.5 to
+# 4.5 times rms(want), so this form is that much stricter than the max-norm metric above.  The integer-dot GEMV keeps
+# fp32-path accuracy with a wide margin; the routes that contract fp32 activations on the matrix cores round x (split-K)
+# or x and W (two passes) to fp16 operands, which puts them at about the 1e-3 mark in this form: they are the MFMA class of
+# the accuracy statement (2e-2), and are held here to a bound an order of magnitude tighter than that.
+RMS_TOL = {"gemv": 1e-3, "split-k": 3e-3, "two-pass f32": 4e-3, "bf16": 2e-2}
+
+
+def test_error_scaled_by_rms_per_route(gpu, oracle):
+    K, N = 4096, 512
+    worst = {}
+    for t in ALL_TYPES:
+        W = synth.weights(t, 8100 + t, N, K)
+        for route, M, bf16 in (("gemv", 1, False), ("gemv", 4, False), ("split-k", 8, False), ("split-k", 32, False), ("two-pass f32", 256, False),
+                               ("bf16", 32, True), ("bf16", 256, True)):
+            x = synth.activations(8200 + M, M, K)
+            want = oracle.c_qdense(t, bf16_round(x) if bf16 else x, W)
+            got = run_dense(gpu, t, x, W, None, 0, bf16=bf16)
+            e = rms_err(got, want)
+            rel_err(got, want)
+            worst[route] = max(worst.get(route, 0.0), e)
+            assert e < RMS_TOL[route], (ggml.name(t), route, M, e)
+    print("max|d| / rms(want) by route:", {k: f"{v:.2e}" for k, v in worst.items()})
 
 
 def test_residual_in_place_on_the_composed_path(gpu, oracle):
