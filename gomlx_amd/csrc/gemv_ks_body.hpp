@@ -752,25 +752,42 @@ template <int T>
 int plan_ks_batch(int count, const XsBatchItem *items, KsBatch &b, size_t &shmem, int &wgs) {
     b.count = count;
     const int cus = device_cu_count();
-    double total = 0.0;
-    for (int i = 0; i < count; i++) total += (double)gq_row_bytes(T, items[i].K) * (double)items[i].N;
-    shmem = 0;
-    int wg = 0;
+    // A workgroup's time goes with the row-steps of its busiest wavefront: iters x the slices that wavefront walks
+    // (more than 8 slices are dealt out round-robin: K = 14336 gives the first four wavefronts 4 slices, the others 3).
+    // The smallest common budget of such steps for which all problems together still fit one workgroup per CU decides
+    // every problem's rows per workgroup; sharing the CUs out by bytes alone let the problems with uneven slices run a
+    // quarter longer than the rest.
+    int spw[kMaxBatchKs];  // slices of the busiest wavefront
     for (int i = 0; i < count; i++) {
+        KsProblem &q = b.p[i];
         const XsBatchItem &it = items[i];
-        KsProblem q;
         q.x = it.x; q.W = it.W; q.bias = it.bias; q.y = it.y; q.N = (int)it.N; q.K = (int)it.K; q.act = it.act;
         q.row_bytes = (int64_t)gq_row_bytes(T, it.K);
         if (!ks_split(it.K, q.waves, q.nslices, q.half_tail)) return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv_ks batch: unsupported K");
-        int64_t share = (int64_t)((double)cus * ((double)q.row_bytes * (double)it.N) / total + 0.5);
-        if (share < 1) share = 1;
-        int64_t iters = (it.N + share * 8 - 1) / (share * 8);
-        iters = (iters + kBatchPF - 1) / kBatchPF * kBatchPF;
+        spw[i] = (q.nslices + q.waves - 1) / q.waves;
+    }
+    auto iters_for = [&](int i, int budget) {
+        int64_t iters = budget / spw[i] / kBatchPF * kBatchPF;
+        if (iters < kBatchPF) iters = kBatchPF;
         if (iters > kMaxItersKs) iters = kMaxItersKs;
+        return iters;
+    };
+    auto wgs_for = [&](int budget) {
+        int64_t n = 0;
+        for (int i = 0; i < count; i++) n += (items[i].N + iters_for(i, budget) * 8 - 1) / (iters_for(i, budget) * 8);
+        return n;
+    };
+    int budget = kBatchPF;
+    const int budget_max = kMaxItersKs * 64;
+    while (budget < budget_max && wgs_for(budget) > cus) budget += kBatchPF;
+    shmem = 0;
+    int wg = 0;
+    for (int i = 0; i < count; i++) {
+        KsProblem &q = b.p[i];
+        const int64_t iters = iters_for(i, budget);
         q.iters = (int)iters;
         q.wg_begin = wg;
-        wg += (int)((it.N + iters * 8 - 1) / (iters * 8));
-        b.p[i] = q;
+        wg += (int)((items[i].N + iters * 8 - 1) / (iters * 8));
         const size_t need = ks_lds_bytes(q.waves, q.iters);
         if (need > shmem) shmem = need;
     }

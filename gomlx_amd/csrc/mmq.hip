@@ -41,6 +41,15 @@ constexpr int kMT = 32;                     // batch columns per pass
 constexpr int kXFBytes = kSliceK * kMT * 2;          // 131072: fp16 activations, fragment order
 constexpr int kXSBytes = kSliceSB * kMT * 16;        // 4096: eight sub-block sums per (super-block, column)
 constexpr int kLdsBytes = kXFBytes + kXSBytes;
+// Weights are read as consecutive 16-byte chunks of a row (nine per 144-byte super-block, seven rows per load
+// instruction) and parked in a wavefront-private piece of LDS, from which lane (row, k-group) picks its header and code
+// bytes.  Read one row per lane pair instead (each load instruction touching 32 rows), the same 33 MB of a
+// 14336 -> 4096 matrix take 10.9 us against 8.4 us with nothing else going on: the address pattern alone.
+constexpr int kParkBytes = 32 * 144;                 // one super-block of a 32-row tile
+constexpr int kParkLoads = 5;                        // 288 chunks / 64 lanes
+constexpr int kParkedSliceSB = 7;                    // longest slice whose image fits LDS next to eight parked tiles
+constexpr int kMainLdsBytes = kParkedSliceSB * 16384 + kXSBytes + 4 * kParts * kParkBytes;
+static_assert(kMainLdsBytes <= 160 * 1024, "image + parked tiles exceed LDS");
 
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
     h2 v;
@@ -179,11 +188,6 @@ __device__ __forceinline__ void stage_x(const void *__restrict__ X, int M, int K
 
 struct RawSB { uint4 hd, c[4]; };  // header + this lane's four chunks (steps 0..3)
 
-__device__ __forceinline__ void load_sb(RawSB &r, const uint8_t *sb, int kg) {
-    r.hd = *reinterpret_cast<const uint4 *>(sb);
-#pragma unroll
-    for (int st = 0; st < 4; st++) r.c[st] = *reinterpret_cast<const uint4 *>(sb + 16 + 32 * st + 16 * kg);
-}
 
 
 // Activation pre-pass: writes each (K-slice, column tile)'s LDS image (fragment-ordered fp16
@@ -225,7 +229,6 @@ __global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__
     const int k0 = slice * slice_sb * 256;
     const int nsb = min(slice_sb, (K - k0) >> 8);
     const int n = blockIdx.x * kRowsPerWG + rt * 32 + col;  // this lane's weight row
-    const uint8_t *wrow = W + (int64_t)min(n, N - 1) * row_bytes + (int64_t)(k0 >> 8) * 144;
 
     // the slice's activation image goes straight from global memory into LDS (no registers)
     {
@@ -234,12 +237,31 @@ __global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__
         const int frag_kib = slice_sb * 16;
         for (int i0 = wave; i0 < frag_kib + kXSBytes / 1024; i0 += 4 * kParts) {
             const int i = i0 < frag_kib ? i0 : kXFBytes / 1024 + (i0 - frag_kib);
+            // (in LDS the sums follow the fragments directly; the image in memory keeps room for 8 super-blocks)
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(img + i * 1024 + lane * 16),
-                                             (__attribute__((address_space(3))) void *)(lds + i * 1024), 16, 0, 0);
+                                             (__attribute__((address_space(3))) void *)(lds + i0 * 1024), 16, 0, 0);
         }
     }
-    RawSB cur;
-    load_sb(cur, wrow + (int64_t)min(par, nsb - 1) * 144, kg);
+    const int xs_off = slice_sb * 16384;
+    // Chunk c = lane + 64 l of a (32 rows x 144 bytes) tile is piece c % 9 of row c / 9.
+    typedef uint32_t Chunk __attribute__((ext_vector_type(4)));
+    const uint8_t *csrc[kParkLoads];
+    {
+        const int row0 = blockIdx.x * kRowsPerWG + rt * 32;
+#pragma unroll
+        for (int l = 0; l < kParkLoads; l++) {
+            const int c = min(lane + 64 * l, 32 * 9 - 1);
+            csrc[l] = W + (int64_t)min(row0 + c / 9, N - 1) * row_bytes + (int64_t)(k0 >> 8) * 144 + (c % 9) * 16;
+        }
+    }
+    auto fetch = [&](Chunk *dst, int sb) __attribute__((always_inline)) {
+#pragma unroll
+        for (int l = 0; l < kParkLoads; l++) dst[l] = *reinterpret_cast<const Chunk *>(csrc[l] + (int64_t)min(sb, nsb - 1) * 144);
+    };
+    Chunk craw[kParkLoads];
+    fetch(craw, par);
+    uint8_t *park = lds + xs_off + kXSBytes + wave * kParkBytes;
+    const uint8_t *myrow = park + col * 144;
     __syncthreads();
 
     f16v acc, acc2;
@@ -249,8 +271,21 @@ __global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__
     asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));
 
     for (int sbl = par; sbl < nsb; sbl += kParts) {
-        RawSB nxt;
-        load_sb(nxt, wrow + (int64_t)min(sbl + kParts, nsb - 1) * 144, kg);
+        // park the tile's super-block and pick out this lane's part (LDS operations of one wavefront execute in order;
+        // no other wavefront touches this piece of LDS), then request the next one
+#pragma unroll
+        for (int l = 0; l < kParkLoads; l++)
+            if (lane + 64 * l < 32 * 9) *reinterpret_cast<Chunk *>(park + (lane + 64 * l) * 16) = craw[l];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        fetch(craw, sbl + kParts);
+        RawSB cur;
+        cur.hd = *reinterpret_cast<const uint4 *>(myrow);
+#pragma unroll
+        for (int st = 0; st < 4; st++) cur.c[st] = *reinterpret_cast<const uint4 *>(myrow + 16 + 32 * st + 16 * kg);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // these reads are done before the next super-block is parked
+        __builtin_amdgcn_wave_barrier();
         const float d = half_bits_to_float(cur.hd.x & 0xFFFFu), dmin = half_bits_to_float(cur.hd.x >> 16);
         // all eight 6-bit scales / minima as bytes: sc0..3, sc4..7, m0..3, m4..7
         const uint32_t a = cur.hd.y, b = cur.hd.z, c = cur.hd.w;
@@ -306,12 +341,11 @@ __global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__
             mv.y = __builtin_bit_cast(uint32_t, (magic_pair(mn_lo >> 8, 0x00FF00FFu, magic) + off) * dm2);
             mv.z = __builtin_bit_cast(uint32_t, (magic_pair(mn_hi, 0x00FF00FFu, magic) + off) * dm2);
             mv.w = __builtin_bit_cast(uint32_t, (magic_pair(mn_hi >> 8, 0x00FF00FFu, magic) + off) * dm2);
-            sv = *reinterpret_cast<const uint4 *>(lds + kXFBytes + (sbl * kMT + col) * 16);
+            sv = *reinterpret_cast<const uint4 *>(lds + xs_off + (sbl * kMT + col) * 16);
         }
         acc2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, sv), __builtin_bit_cast(h8, mv), acc2, 0, 0, 0);
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[r] = fmaf(d, p1[r], acc[r]);
-        cur = nxt;
     }
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] -= acc2[r];
@@ -944,16 +978,27 @@ int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, co
     if (type != kQ4_K) return fail(GQ_ERR_NOT_IMPLEMENTED, "mmq: ggml type %d is not implemented", type);
     static const bool lds_ok = [] {
         return hipFuncSetAttribute(reinterpret_cast<const void *>(mmq_q4k_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   kLdsBytes) == hipSuccess;
+                                   kMainLdsBytes) == hipSuccess;
     }();
-    if (!lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", kLdsBytes);
+    if (!lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", kMainLdsBytes);
     // K-slices of 8 super-blocks, or of 4 / 2 when the problem would otherwise leave more than a quarter of the
     // CUs without a workgroup (4096 x 4096: 2 slices x 32 row ranges = 64 workgroups with 8, 256 with 2: 18.8 -> 16.6 us;
     // splitting 224 workgroups into 448 costs more than it brings: 20.8 -> 24.9 us on 4096 -> 14336)
     const int mtiles = (int)((M + kMT - 1) / kMT);
     const int64_t rowwgs = (N + kRowsPerWG - 1) / kRowsPerWG, sbs = K / 256;
-    int slice_sb = kSliceSB;
-    while (slice_sb > 2 && rowwgs * ((sbs + slice_sb - 1) / slice_sb) < (int64_t)device_cu_count() * 3 / 4) slice_sb >>= 1;
+    // Super-blocks per K-slice (at most 7: the image shares LDS with the parked tiles): the count that needs the fewest
+    // rounds of workgroups over the chip times the length of a round (+3: what a workgroup costs beyond its
+    // super-blocks); ties go to the longer slice (fewer partial sums).
+    int slice_sb = kParkedSliceSB;
+    {
+        const int64_t cus = device_cu_count(), z = W2 ? 2 : 1;
+        int64_t best_cost = INT64_MAX;
+        for (int ssb = kParkedSliceSB; ssb >= 2; ssb--) {
+            const int64_t wgs = rowwgs * ((sbs + ssb - 1) / ssb) * z;
+            const int64_t cost = ((wgs + cus - 1) / cus) * (ssb + 3);
+            if (cost < best_cost) { best_cost = cost; slice_sb = ssb; }
+        }
+    }
     const int nslices = (int)((sbs + slice_sb - 1) / slice_sb);
     // workspace: [activation images: mtiles x nslices x kLdsBytes][slice scales: nslices x M][partial sums: nslices x M x N fp32,
     // twice for a gated pair]
@@ -975,7 +1020,7 @@ int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, co
     const dim3 grid((unsigned)((N + kRowsPerWG - 1) / kRowsPerWG), (unsigned)nslices, W2 ? 2u : 1u);  // (both matrices of a gated pair in one launch)
     float *partial2 = W2 ? partial + (size_t)nslices * M * N : nullptr;
     for (int64_t m0 = 0; m0 < M; m0 += kMT) {
-        if (int rc = launch(mmq_q4k_kernel, grid, dim3(256 * kParts), (size_t)kLdsBytes, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N,
+        if (int rc = launch(mmq_q4k_kernel, grid, dim3(256 * kParts), (size_t)kMainLdsBytes, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N,
                             row_bytes, (int)m0, slice_sb, W2, partial2))
             return rc;
     }
