@@ -42,6 +42,9 @@ SIGNATURES = [
     ("gq_qdense_block_f32", _int, [_int, _vp, _i64, _i64, _vp, _vp, _i64, _vp, _int, _vp, _vp, _vp]),
     ("gq_qdense_norm_f32_batch", _int, [_int, _vp, _vp, _vp]),
     ("gq_qdense_gated_f32", _int, [_int, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _int, _vp, _vp]),
+    ("gq_qdense_block_bf16", _int, [_int, _vp, _i64, _i64, _vp, _vp, _i64, _vp, _int, _vp, _vp, _vp]),
+    ("gq_qdense_norm_bf16_batch", _int, [_int, _vp, _vp, _vp]),
+    ("gq_qdense_gated_bf16", _int, [_int, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _int, _vp, _vp]),
     ("gq_embedding_lookup", _int, [_int, _vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp]),
     ("gq_graph_begin", _int, [_vp]),
     ("gq_graph_end", _int, [_vp, ctypes.POINTER(_vp)]),

@@ -687,6 +687,82 @@ int gq_qdense_gated_f32(int type, const float *dX, int64_t M, int64_t K, const g
     return launch_mul_inplace(dY, gate, M * N, (hipStream_t)stream);
 }
 
+// ---- the same callers with bf16 activations: widened exactly to fp32 in the stream's third workspace, then the fp32 routes ----
+namespace {
+// fp32 copy of a bf16 [M, K] matrix at `offset` bytes into the widening workspace, whose size the caller has fixed
+int widen_into(void *ws, size_t offset, const uint16_t *x, int64_t M, int64_t K, hipStream_t s, const float **out) {
+    float *dst = reinterpret_cast<float *>(static_cast<uint8_t *>(ws) + offset);
+    if (int rc = launch_widen_bf16(x, dst, M * K, s)) return rc;
+    *out = dst;
+    return GQ_OK;
+}
+size_t widened_bytes(int64_t M, int64_t K) { return ((size_t)M * (size_t)K * sizeof(float) + 255) & ~(size_t)255; }
+}  // namespace
+
+int gq_qdense_block_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, const gq_rmsnorm *norm, const void *dW, int64_t N,
+                         const float *dBias, int act, const float *dResidual, float *dY, void *stream) {
+    if (!norm && !dResidual) return gq_qdense_bf16(type, dX, M, K, dW, N, dBias, act, dY, stream);
+    if (int rc = check_dense_args("gq_qdense_block_bf16", type, dX, M, K, dW, N, dBias, act, dY, 16)) return rc;
+    if (M == 0 || N == 0) return GQ_OK;
+    if (int rc = use_device()) return rc;
+    CallScope scope;
+    void *ws = nullptr;
+    if (int rc = stream_workspace((hipStream_t)stream, widened_bytes(M, K), &ws, kWsWidenSlot)) return rc;
+    const float *x32 = nullptr;
+    if (int rc = widen_into(ws, 0, dX, M, K, (hipStream_t)stream, &x32)) return rc;
+    return gq_qdense_block_f32(type, x32, M, K, norm, dW, N, dBias, act, dResidual, dY, stream);
+}
+
+int gq_qdense_gated_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, const gq_rmsnorm *norm, const void *dWgate,
+                         const float *dBiasGate, const void *dWup, const float *dBiasUp, int64_t N, int act, float *dY, void *stream) {
+    if (int rc = check_dense_args("gq_qdense_gated_bf16", type, dX, M, K, dWgate, N, dBiasGate, act, dY, 16)) return rc;
+    if (M == 0 || N == 0) return GQ_OK;
+    if (int rc = use_device()) return rc;
+    CallScope scope;
+    void *ws = nullptr;
+    if (int rc = stream_workspace((hipStream_t)stream, widened_bytes(M, K), &ws, kWsWidenSlot)) return rc;
+    const float *x32 = nullptr;
+    if (int rc = widen_into(ws, 0, dX, M, K, (hipStream_t)stream, &x32)) return rc;
+    return gq_qdense_gated_f32(type, x32, M, K, norm, dWgate, dBiasGate, dWup, dBiasUp, N, act, dY, stream);
+}
+
+int gq_qdense_norm_bf16_batch(int count, const gq_dense_desc *descs, const gq_rmsnorm *norm, void *stream) {
+    if (count < 0 || (count > 0 && !descs)) return fail(GQ_ERR_INVALID, "gq_qdense_norm_bf16_batch: bad descriptor list");
+    if (count > 64) return fail(GQ_ERR_NOT_IMPLEMENTED, "gq_qdense_norm_bf16_batch: more than 64 problems in one submission");
+    for (int i = 0; i < count; i++) {
+        const gq_dense_desc &d = descs[i];
+        if (int rc = check_dense_args("gq_qdense_norm_bf16_batch", d.type, d.dX, d.M, d.K, d.dW, d.N, d.dBias, d.act, d.dY, 16)) return rc;
+    }
+    if (count == 0) return GQ_OK;
+    if (int rc = use_device()) return rc;
+    CallScope scope;
+    // every distinct activation matrix (q / k / v share theirs) is widened once
+    gq_dense_desc wide[64];
+    size_t offset[64], total = 0;
+    int first[64];
+    for (int i = 0; i < count; i++) {
+        first[i] = i;
+        for (int j = 0; j < i; j++)
+            if (descs[j].dX == descs[i].dX && descs[j].M == descs[i].M && descs[j].K == descs[i].K) { first[i] = first[j]; break; }
+        if (first[i] == i) { offset[i] = total; total += widened_bytes(descs[i].M, descs[i].K); }
+    }
+    void *ws = nullptr;
+    if (total)
+        if (int rc = stream_workspace((hipStream_t)stream, total, &ws, kWsWidenSlot)) return rc;
+    for (int i = 0; i < count; i++) {
+        wide[i] = descs[i];
+        if (descs[i].M == 0 || descs[i].N == 0) continue;
+        if (first[i] == i) {
+            const float *x32 = nullptr;
+            if (int rc = widen_into(ws, offset[i], reinterpret_cast<const uint16_t *>(descs[i].dX), descs[i].M, descs[i].K, (hipStream_t)stream, &x32)) return rc;
+            wide[i].dX = x32;
+        } else {
+            wide[i].dX = wide[first[i]].dX;
+        }
+    }
+    return gq_qdense_norm_f32_batch(count, wide, norm, stream);
+}
+
 int gq_embedding_lookup(int type, const void *dTable, int64_t vocab, int64_t K, const int32_t *dIndices,
                         int64_t count, float *dOut, int32_t *dErrFlag, void *stream) {
     TypeInfo ti;

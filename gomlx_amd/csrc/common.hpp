@@ -94,6 +94,7 @@ int launch_gemv_ks_ext(int type, const float *x, int64_t M, int64_t K, const Rms
 int launch_add(const float *a, const float *r, float *y, int64_t n, hipStream_t s);
 int launch_rmsnorm(const float *x, int64_t M, int64_t K, const float *gain, float gain_offset, float eps, float *y, hipStream_t s);
 int launch_mul_inplace(float *y, const float *g, int64_t n, hipStream_t s);
+int launch_widen_bf16(const uint16_t *x, float *y, int64_t n, hipStream_t s);  // bf16 -> fp32 (exact); both 16-byte aligned
 struct XsBatchItem { const float *x; const uint8_t *W; const float *bias; float *y; int64_t K, N; int act; };
 int launch_gemv_xs_batch(int type, int count, const XsBatchItem *items, hipStream_t s);
 // (K-sliced: `rows` activation rows per problem, the same count for all: x and y are [rows, K] and [rows, N])

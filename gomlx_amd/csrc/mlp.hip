@@ -116,6 +116,20 @@ __global__ __launch_bounds__(256) void add_kernel(const float *a, const float *r
     if (i < n) y[i] = a[i] + r[i];
 }
 
+// y[i] = x[i] widened from bf16 (exact: a shift); eight values per thread, n % 8 == 0 handled by the caller's padding rule
+__global__ __launch_bounds__(256) void widen_bf16_kernel(const uint16_t *__restrict__ x, float *__restrict__ y, int64_t n) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (i + 8 <= n) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(x + i);
+        float4 lo = make_float4(bf16_lo(v.x), bf16_hi(v.x), bf16_lo(v.y), bf16_hi(v.y));
+        float4 hi = make_float4(bf16_lo(v.z), bf16_hi(v.z), bf16_lo(v.w), bf16_hi(v.w));
+        *reinterpret_cast<float4 *>(y + i) = lo;
+        *reinterpret_cast<float4 *>(y + i + 4) = hi;
+    } else {
+        for (int64_t j = i; j < n; j++) y[j] = __builtin_bit_cast(float, (uint32_t)x[j] << 16);
+    }
+}
+
 // y[i] *= g[i]
 __global__ __launch_bounds__(256) void mul_inplace_kernel(float *__restrict__ y, const float *__restrict__ g, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -180,6 +194,11 @@ int launch_add(const float *a, const float *r, float *y, int64_t n, hipStream_t 
 
 int launch_rmsnorm(const float *x, int64_t M, int64_t K, const float *gain, float gain_offset, float eps, float *y, hipStream_t s) {
     return launch(rmsnorm_kernel, dim3((unsigned)M), dim3(256), 0, s, x, gain, gain_offset, eps, (int)K, y);
+}
+
+int launch_widen_bf16(const uint16_t *x, float *y, int64_t n, hipStream_t s) {
+    if ((reinterpret_cast<uintptr_t>(x) & 15) || (reinterpret_cast<uintptr_t>(y) & 15)) return fail(GQ_ERR_INVALID, "bf16 activations must be 16-byte aligned");
+    return launch(widen_bf16_kernel, dim3((unsigned)((n + 2047) / 2048)), dim3(256), 0, s, x, y, n);
 }
 
 int launch_mul_inplace(float *y, const float *g, int64_t n, hipStream_t s) {

@@ -32,7 +32,9 @@ struct WsHooks {
     bool (*capturing)(const void *stream);    // a graph is being recorded on the stream
 };
 
-constexpr int kWsSlots = 2;                   // 0: the dense kernels, 1: operations composed of several dense calls
+// 0: the dense kernels, 1: operations composed of several dense calls, 2: bf16 activations widened to fp32 for the
+// entry points that take the callers around a projection in bf16
+constexpr int kWsSlots = 3, kWsWidenSlot = 2;
 constexpr size_t kWsMinBytes = (size_t)4 << 20;
 
 struct WsBlock {

@@ -131,7 +131,7 @@ def gated_feed_forward(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor
                        norm: RMSNorm | None = None) -> torch.Tensor:
     """The front of a gated feed-forward block (ml/zoo/transformer/transformer.go:1276-1287):
     ``activation(dense(xn, w_gate)) * dense(xn, w_up)`` with ``xn = rms_norm(x)`` when ``norm`` is given.
-    x: [batch..., K] float32; both weights [N, bytesPerRow] uint8 of one GGML type."""
+    x: [batch..., K] float32 or bfloat16 (gain, biases and the result stay float32); both weights [N, bytesPerRow] uint8 of one GGML type."""
     if quant is None or quant.scheme != QuantizationScheme.GGML:
         raise _lib.NotImplementedByBackend(_lib.ERR_NOT_IMPLEMENTED, "only the GGML scheme is on this path")
     for name, t in (("x", x), ("w_gate", w_gate), ("w_up", w_up)):
@@ -140,8 +140,9 @@ def gated_feed_forward(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor
     _weights_2d(w_up)
     if w_gate.shape != w_up.shape:
         raise ValueError(f"gate and up weights differ in shape: {tuple(w_gate.shape)} vs {tuple(w_up.shape)}")
-    if x.dtype != torch.float32:
+    if x.dtype not in (torch.float32, torch.bfloat16):
         raise _lib.NotImplementedByBackend(_lib.ERR_NOT_IMPLEMENTED, f"gated_feed_forward: dtype {x.dtype} is not implemented")
+    xd = _lib.F32 if x.dtype == torch.float32 else _lib.BF16
     import ctypes
     L = _lib.lib()
     N, rb = w_gate.shape
@@ -155,11 +156,12 @@ def gated_feed_forward(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor
             if b.dtype != torch.float32 or b.dim() != 1:
                 raise ValueError("bias must be a float32 [N] tensor")
             blen = b.shape[0]
-        _lib.check(L.gq_qdense_check(quant.ggml_type, _lib.F32, M, K_in, N, rb, blen, activation.to_backend(), ctypes.byref(K)))
+        _lib.check(L.gq_qdense_check(quant.ggml_type, xd, M, K_in, N, rb, blen, activation.to_backend(), ctypes.byref(K)))
     d = None if norm is None else norm._desc(K.value)
     _lib.init(x.device.index or 0)
     y = torch.empty(x.shape[:-1] + (N,), dtype=torch.float32, device=x.device)
-    _lib.check(L.gq_qdense_gated_f32(quant.ggml_type, x.data_ptr(), M, K.value, None if d is None else ctypes.byref(d),
+    fn = L.gq_qdense_gated_f32 if xd == _lib.F32 else L.gq_qdense_gated_bf16
+    _lib.check(fn(quant.ggml_type, x.data_ptr(), M, K.value, None if d is None else ctypes.byref(d),
                                      w_gate.data_ptr(), None if bias_gate is None else bias_gate.data_ptr(), w_up.data_ptr(),
                                      None if bias_up is None else bias_up.data_ptr(), N, activation.to_backend(), y.data_ptr(),
                                      _stream_ptr(x)))
@@ -173,7 +175,7 @@ def quantized_dense(x: torch.Tensor, weights: torch.Tensor, quant: Quantization,
 
     x: [batch..., K] float32 or bfloat16; weights: [N, bytesPerRow] uint8; bias: [N] float32.
     Returns [batch..., N] float32.  ``norm`` applies an RMS normalisation to x first and ``residual``
-    ([batch..., N] float32) is added to the result (float32 x only): Model.normalize followed by a
+    ([batch..., N] float32) is added to the result (gain and residual are float32 also for bfloat16 x): Model.normalize followed by a
     projection and Add(residual, ...) after it, ml/zoo/transformer/transformer.go:1099-1101, 1045, 1055.
     """
     if len(optional_activation) > 1:
@@ -209,14 +211,13 @@ def quantized_dense(x: torch.Tensor, weights: torch.Tensor, quant: Quantization,
     _lib.init(x.device.index or 0)
     y = torch.empty(x.shape[:-1] + (N,), dtype=torch.float32, device=x.device)
     if norm is not None or residual is not None:
-        if xd != _lib.F32:
-            raise _lib.NotImplementedByBackend(_lib.ERR_NOT_IMPLEMENTED, "a fused normalisation or residual takes float32 activations")
         d = None if norm is None else norm._desc(K.value)
         if residual is not None:
             _require_cuda("residual", residual)
             if residual.dtype != torch.float32 or tuple(residual.shape) != tuple(y.shape):
                 raise ValueError(f"residual must be a float32 tensor of shape {tuple(y.shape)}")
-        _lib.check(L.gq_qdense_block_f32(quant.ggml_type, x.data_ptr(), M, K.value, None if d is None else ctypes.byref(d),
+        block = L.gq_qdense_block_f32 if xd == _lib.F32 else L.gq_qdense_block_bf16
+        _lib.check(block(quant.ggml_type, x.data_ptr(), M, K.value, None if d is None else ctypes.byref(d),
                                          weights.data_ptr(), N, None if bias is None else bias.data_ptr(), act.to_backend(),
                                          None if residual is None else residual.data_ptr(), y.data_ptr(), _stream_ptr(x)))
         return y
@@ -259,7 +260,7 @@ def quantized_dense_batch(problems, norm: RMSNorm | None = None) -> list:
     layer's input norm, gq_qdense_norm_f32_batch).
 
     ``problems`` is a sequence of ``(x, weights, quant, bias, activation)`` tuples with float32
-    activations; returns the list of outputs.  Results equal those of separate calls; problems
+    activations (with ``norm``: all float32 or all bfloat16); returns the list of outputs.  Results equal those of separate calls; problems
     of one GGML type and one batch size of up to 8 rows share a single kernel launch.
     """
     import ctypes
@@ -273,8 +274,10 @@ def quantized_dense_batch(problems, norm: RMSNorm | None = None) -> list:
         _require_cuda("x", x)
         _require_cuda("weights", weights)
         _weights_2d(weights)
-        if x.dtype != torch.float32:
-            raise _lib.NotImplementedByBackend(_lib.ERR_NOT_IMPLEMENTED, "batched submission takes float32 activations")
+        bf16 = norm is not None and x.dtype == torch.bfloat16 and all(p[0].dtype == torch.bfloat16 for p in problems)
+        if x.dtype != torch.float32 and not bf16:
+            raise _lib.NotImplementedByBackend(_lib.ERR_NOT_IMPLEMENTED, "batched submission takes float32 activations "
+                                               "(behind a shared normalisation: all float32 or all bfloat16)")
         N, rb = weights.shape
         K_in = x.shape[-1]
         M = x.numel() // K_in if K_in else 0
@@ -283,7 +286,7 @@ def quantized_dense_batch(problems, norm: RMSNorm | None = None) -> list:
             _require_cuda("bias", bias)
             blen = bias.shape[0]
         K = ctypes.c_int64(0)
-        _lib.check(L.gq_qdense_check(quant.ggml_type, _lib.F32, M, K_in, N, rb, blen, act.to_backend(), ctypes.byref(K)))
+        _lib.check(L.gq_qdense_check(quant.ggml_type, _lib.BF16 if bf16 else _lib.F32, M, K_in, N, rb, blen, act.to_backend(), ctypes.byref(K)))
         y = torch.empty(x.shape[:-1] + (N,), dtype=torch.float32, device=x.device)
         outs.append(y)
         d = descs[i]
@@ -295,5 +298,6 @@ def quantized_dense_batch(problems, norm: RMSNorm | None = None) -> list:
             _lib.check(L.gq_qdense_f32_batch(len(problems), descs, _stream_ptr(problems[0][0])))
         else:
             d = norm._desc(problems[0][0].shape[-1])
-            _lib.check(L.gq_qdense_norm_f32_batch(len(problems), descs, ctypes.byref(d), _stream_ptr(problems[0][0])))
+            fn = L.gq_qdense_norm_bf16_batch if problems[0][0].dtype == torch.bfloat16 else L.gq_qdense_norm_f32_batch
+            _lib.check(fn(len(problems), descs, ctypes.byref(d), _stream_ptr(problems[0][0])))
     return outs

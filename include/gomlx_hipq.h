@@ -187,6 +187,20 @@ int gq_qdense_gated_f32(int type, const float *dX, int64_t M, int64_t K, const g
                         const void *dWgate, const float *dBiasGate, const void *dWup,
                         const float *dBiasUp, int64_t N, int act, float *dY, void *stream);
 
+/* The three calls above for bf16 activations (raw 16-bit patterns, 16-byte aligned; in the batched form every
+ * descriptor's dX points at bf16 data): what the same layer code (transformer.go:1099-1101, 1276-1294) builds when the
+ * model runs in bfloat16.  Gain, bias and residual stay fp32 and the result is fp32, as for gq_qdense_bf16.  The
+ * activations are widened to fp32 (exact) in a per-stream workspace - activation matrices shared by several problems of
+ * a batch once - and then take the fp32 routes, so results equal those of the fp32 entry points on the widened inputs. */
+int gq_qdense_block_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, const gq_rmsnorm *norm,
+                         const void *dW, int64_t N, const float *dBias, int act,
+                         const float *dResidual, float *dY, void *stream);
+int gq_qdense_norm_bf16_batch(int count, const gq_dense_desc *descs, const gq_rmsnorm *norm,
+                              void *stream);
+int gq_qdense_gated_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, const gq_rmsnorm *norm,
+                         const void *dWgate, const float *dBiasGate, const void *dWup,
+                         const float *dBiasUp, int64_t N, int act, float *dY, void *stream);
+
 /* ---- compute.Function.QuantizedEmbeddingLookup (core/graph/fused_ops.go:295-296;
  * nn.QuantizedGather ml/nn/quantized_gather.go:30-43; ml/ggml/gather.go:21-49):
  * dOut[i, :] = dequant(dTable[dIndices[i], :]), bit-exact.  An index outside [0, vocab)

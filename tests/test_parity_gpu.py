@@ -712,6 +712,44 @@ def test_error_scaled_by_rms_per_route(gpu, oracle):
     print("max|d| / rms(want) by route:", {k: f"{v:.2e}" for k, v in worst.items()})
 
 
+@pytest.mark.parametrize("t", ALL_TYPES)
+def test_callers_around_a_projection_with_bf16_activations(gpu, oracle, t):
+    """RMSNorm + projection + residual, q/k/v behind one norm, and the gated feed-forward front for bf16 activations:
+    bit-identical to the fp32 entry points on the widened inputs (the widening is exact), and within the fp32-path
+    bound of the oracle on the bf16-rounded inputs; decode rows, split-K batches and a two-pass batch."""
+    q = Quantization(ggml_type=t)
+    for i, (M, K, N, act) in enumerate([(1, 4096, 384, 0), (3, 1024, 200, 3), (24, 2048, 260, 0), (200, 1024, 128, 1)]):
+        x32 = bf16_round((synth.activations(8300 + i, M, K) * 2.5).astype(np.float32))
+        xb = dev(gpu, x32).to(gpu.bfloat16)
+        gain = (synth.normal(8310 + i, 0, K) * 0.5 + 1.0).astype(np.float32)
+        bias = synth.normal(8320 + i, 0, N).astype(np.float32) * 0.1
+        res = synth.activations(8330 + i, M, N)
+        W, W2 = synth.weights(t, 8340 + i, N, K), synth.weights(t, 8350 + i, N, K)
+        norm = nn.RMSNorm(dev(gpu, gain), 1e-6, 0.0)
+        xn = oracle.c_rmsnorm(x32, gain, 1e-6, 0.0)
+        # projection with norm and residual
+        got = nn.quantized_dense(xb, dev(gpu, W), q, dev(gpu, bias), BACKEND_ACT[act], norm=norm, residual=dev(gpu, res)).cpu().numpy()
+        same = nn.quantized_dense(dev(gpu, x32), dev(gpu, W), q, dev(gpu, bias), BACKEND_ACT[act], norm=norm, residual=dev(gpu, res)).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), same.view(np.uint32)), (ggml.name(t), M, K, N)
+        dense, pre = oracle.c_qdense(t, xn, W, bias, act), oracle.c_qdense(t, xn, W, bias, 0)
+        scale = max(float(np.max(np.abs(dense))), float(np.max(np.abs(pre))))
+        tol = TOL_F32 if M <= 192 else 2 * TOL_F32
+        assert float(np.max(np.abs(got.astype(np.float64) - (dense + res)))) / scale < tol, (ggml.name(t), M, K, N)
+        # gated feed-forward front
+        got = nn.gated_feed_forward(xb, dev(gpu, W), dev(gpu, W2), q, Activation.SILU, dev(gpu, bias), None, norm=norm).cpu().numpy()
+        same = nn.gated_feed_forward(dev(gpu, x32), dev(gpu, W), dev(gpu, W2), q, Activation.SILU, dev(gpu, bias), None, norm=norm).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), same.view(np.uint32)), ("gated", ggml.name(t), M, K, N)
+        gate, up = oracle.c_qdense(t, xn, W, bias, 0), oracle.c_qdense(t, xn, W2, None, 0)
+        want = oracle.c_qdense(t, xn, W, bias, 3).astype(np.float64) * up
+        assert float(np.max(np.abs(got - want))) / (float(np.max(np.abs(gate))) * float(np.max(np.abs(up)))) < 2 * tol, ("gated", ggml.name(t), M, K, N)
+        # q / k / v behind one norm: one shared activation matrix, widened once
+        if M <= 8:
+            probs = [(xb, dev(gpu, W), q, None, None), (xb, dev(gpu, W2), q, dev(gpu, bias), None), (xb, dev(gpu, W[: N // 2]), q, None, None)]
+            outs = nn.quantized_dense_batch(probs, norm=norm)
+            for out, (Wm, b) in zip(outs, ((W, None), (W2, bias), (W[: N // 2], None))):
+                assert rel_err(out.cpu().numpy(), oracle.c_qdense(t, xn, Wm, b, 0)) < TOL_F32
+
+
 def test_residual_in_place_on_the_composed_path(gpu, oracle):
     """y == residual on shapes that none of the fused routes take (K not a multiple of 256; N not a multiple of 4
     beyond 16 rows): the dense result must not overwrite the residual before it is added."""
