@@ -102,6 +102,9 @@ def parse_args():
                         "workload that hardware counter readings (FETCH_SIZE / WRITE_SIZE) are scaled by")
     p.add_argument("--yardstick", action="store_true",
                    help="instead of the benchmark, time the plain read-only kernel on 17.8 / 33.0 / 122.7 MB of cold weights")
+    p.add_argument("--matmul-yardstick", action="store_true",
+                   help="instead of the benchmark, time the vendor library's plain bf16 GEMM (torch.matmul) on C3's shape, 2048 x 4096 x 4096: "
+                        "what a 16-bit GEMM with no dequantisation reaches on this chip")
     return p.parse_args()
 
 
@@ -569,6 +572,32 @@ def yardstick_only(torch, steps):
     print(json.dumps(out))
 
 
+def matmul_yardstick(torch, steps):
+    """torch.matmul in bf16 on C3's shape (x [2048, 4096] . W^T, W [4096, 4096] already a 16-bit matrix), fp32 result via a bf16
+    output widened afterwards is NOT included: the vendor kernel writes bf16, half the output bytes of this library's fp32."""
+    M, K, N = 2048, 4096, 4096
+    x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+    ws = [torch.randn(N, K, device="cuda").to(torch.bfloat16) for _ in range(17)]  # > 512 MB: cold, like the benchmark's rotation
+    st = torch.cuda.Stream()
+    with torch.cuda.stream(st):
+        for i in range(5):
+            torch.matmul(x, ws[i % len(ws)].t())
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(st)
+            for i in range(steps):
+                torch.matmul(x, ws[i % len(ws)].t())
+            e1.record(st)
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / steps
+            best = us if best is None else min(best, us)
+    flops = 2.0 * M * K * N
+    print(json.dumps({"matmul_yardstick": "torch.matmul bf16 [2048,4096] x [4096,4096]^T, bf16 output, cold weights", "us": best,
+                      "tflops": flops / best / 1e6, "frac_of_peak": flops / best / 1e6 / MFMA_BF16_PEAK_TFLOPS, "steps": steps}))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -585,6 +614,9 @@ def main():
         return
     if args.yardstick:
         yardstick_only(torch, min(args.steps, 50))
+        return
+    if args.matmul_yardstick:
+        matmul_yardstick(torch, min(args.steps, 50))
         return
     from gomlx_amd import _lib
     _lib.init(0)
