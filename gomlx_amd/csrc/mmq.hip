@@ -254,9 +254,17 @@ __global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__
             csrc[l] = W + (int64_t)min(row0 + c / 9, N - 1) * row_bytes + (int64_t)(k0 >> 8) * 144 + (c % 9) * 16;
         }
     }
+    // The loads are written as instructions so that they are issued where they stand (left to the compiler, the first
+    // fetch sinks below the barrier that waits for the image, and every workgroup then sits out a full HBM round trip
+    // after it); their results may be used after chunks_arrived() only.
     auto fetch = [&](Chunk *dst, int sb) __attribute__((always_inline)) {
 #pragma unroll
-        for (int l = 0; l < kParkLoads; l++) dst[l] = *reinterpret_cast<const Chunk *>(csrc[l] + (int64_t)min(sb, nsb - 1) * 144);
+        for (int l = 0; l < kParkLoads; l++)
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst[l]) : "v"(csrc[l] + (int64_t)min(sb, nsb - 1) * 144) : "memory");
+    };
+    auto chunks_arrived = [&](Chunk *c) __attribute__((always_inline)) {
+        static_assert(kParkLoads == 5, "one operand per chunk below");
+        asm volatile("s_waitcnt vmcnt(0)" : "+v"(c[0]), "+v"(c[1]), "+v"(c[2]), "+v"(c[3]), "+v"(c[4])::"memory");
     };
     Chunk craw[kParkLoads];
     fetch(craw, par);
@@ -273,6 +281,7 @@ __global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__
     for (int sbl = par; sbl < nsb; sbl += kParts) {
         // park the tile's super-block and pick out this lane's part (LDS operations of one wavefront execute in order;
         // no other wavefront touches this piece of LDS), then request the next one
+        chunks_arrived(craw);
 #pragma unroll
         for (int l = 0; l < kParkLoads; l++)
             if (lane + 64 * l < 32 * 9) *reinterpret_cast<Chunk *>(park + (lane + 64 * l) * 16) = craw[l];
@@ -347,6 +356,9 @@ __global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[r] = fmaf(d, p1[r], acc[r]);
     }
+    // The request past the end of the slice (clamped to its last super-block) still writes its registers: nothing
+    // else may live there before it has landed.
+    chunks_arrived(craw);
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] -= acc2[r];
 
