@@ -105,6 +105,9 @@ def parse_args():
     p.add_argument("--matmul-yardstick", action="store_true",
                    help="instead of the benchmark, time the vendor library's plain bf16 GEMM (torch.matmul) on C3's shape, 2048 x 4096 x 4096: "
                         "what a 16-bit GEMM with no dequantisation reaches on this chip")
+    p.add_argument("--mfma-yardstick", action="store_true",
+                   help="instead of the benchmark, time matrix instructions alone (the prefill GEMM's count and occupancy, no data movement) "
+                        "with random and with zero operands and on a quarter of the CUs, with the shader clock the kernel measured itself")
     return p.parse_args()
 
 
@@ -193,6 +196,8 @@ class Yardstick:
         vp, i64 = ctypes.c_void_p, ctypes.c_int64
         self.lib.gqy_read.argtypes = [vp, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, i64, i64, ctypes.c_int, vp, vp]
         self.lib.gqy_read.restype = ctypes.c_int
+        self.lib.gqy_mfma.argtypes = [vp, ctypes.c_int, ctypes.c_int, vp, vp, vp]
+        self.lib.gqy_mfma.restype = ctypes.c_int
 
     # (workgroups, threads, loads in flight per thread): the shapes that read fastest on this chip at 18 .. 123 MB
     SHAPES = ((2048, 256, 2), (1024, 256, 4), (512, 256, 8), (256, 512, 8))
@@ -594,8 +599,56 @@ def matmul_yardstick(torch, steps):
             us = e0.elapsed_time(e1) * 1e3 / steps
             best = us if best is None else min(best, us)
     flops = 2.0 * M * K * N
-    print(json.dumps({"matmul_yardstick": "torch.matmul bf16 [2048,4096] x [4096,4096]^T, bf16 output, cold weights", "us": best,
-                      "tflops": flops / best / 1e6, "frac_of_peak": flops / best / 1e6 / MFMA_BF16_PEAK_TFLOPS, "steps": steps}))
+    return {"matmul_yardstick": "torch.matmul bf16 [2048,4096] x [4096,4096]^T, bf16 output, cold weights", "us": best,
+            "tflops": flops / best / 1e6, "frac_of_peak": flops / best / 1e6 / MFMA_BF16_PEAK_TFLOPS, "steps": steps}
+
+
+def mfma_yardstick(torch, steps, only_first=False):
+    """Matrix instructions only (gomlx_amd/csrc/yardstick.hip, gqy_mfma): the prefill GEMM's instruction count per wavefront
+    (64 K-steps x 16 v_mfma_f32_32x32x16_bf16) and its occupancy (8 wavefronts per CU), no data movement at all.  Reported per
+    case: time per launch (HIP events over `steps` back-to-back launches), the rate that corresponds to, and the shader clock
+    the workgroups measured themselves (clock counter over the constant 100 MHz counter)."""
+    ys = yardstick()
+    if ys is None:
+        return None
+    groups, cus = 64 * 4, torch.cuda.get_device_properties(0).multi_processor_count
+    st = torch.cuda.Stream()
+    out = {"mfma_yardstick": "v_mfma_f32_32x32x16_bf16 only: 1024 per wavefront, 8 wavefronts per workgroup, no loads, LDS or barriers in the loop",
+           "published_peak_tflops": MFMA_BF16_PEAK_TFLOPS, "cases": {}}
+    sink = torch.zeros(cus * 512, device="cuda")
+    cases = (("random operands, one workgroup per CU", "randn", cus), ("zero operands, one workgroup per CU", "zeros", cus),
+             ("random operands, a quarter of the CUs", "randn", cus // 4))
+    for label, fill, wgs in cases[:1] if only_first else cases:
+        frags = (torch.randn(8 * 4 * 64 * 8, device="cuda") if fill == "randn" else torch.zeros(8 * 4 * 64 * 8, device="cuda")).to(torch.bfloat16)
+        clocks = torch.zeros(4 * wgs, dtype=torch.int64, device="cuda")
+
+        def launch():
+            rc = ys.lib.gqy_mfma(frags.data_ptr(), groups, wgs, clocks.data_ptr(), sink.data_ptr(), st.cuda_stream)
+            if rc:
+                raise RuntimeError(f"gqy_mfma failed ({rc})")
+        with torch.cuda.stream(st):
+            for _ in range(5):
+                launch()
+            torch.cuda.synchronize()
+            best = None
+            for _ in range(3):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(st)
+                for _ in range(steps):
+                    launch()
+                e1.record(st)
+                torch.cuda.synchronize()
+                us = e0.elapsed_time(e1) * 1e3 / steps
+                best = us if best is None else min(best, us)
+        c = clocks.cpu().view(wgs, 4).double()
+        loop_us = (c[:, 3] - c[:, 1]) / 100.0
+        mhz = (c[:, 2] - c[:, 0]) / loop_us
+        flops = wgs * 8 * 4 * groups * 2.0 * 32 * 32 * 16
+        out["cases"][label] = {"workgroups": wgs, "us_per_launch": best, "tflops": flops / best / 1e6,
+                               "frac_of_published_peak": flops / best / 1e6 / (MFMA_BF16_PEAK_TFLOPS * wgs / cus),
+                               "shader_mhz_mean": float(mhz.mean()), "shader_mhz_min": float(mhz.min()),
+                               "wavefront0_loop_us_mean": float(loop_us.mean())}
+    return out
 
 
 def main():
@@ -616,7 +669,14 @@ def main():
         yardstick_only(torch, min(args.steps, 50))
         return
     if args.matmul_yardstick:
-        matmul_yardstick(torch, min(args.steps, 50))
+        print(json.dumps(matmul_yardstick(torch, min(args.steps, 50))))
+        return
+    if args.mfma_yardstick:
+        out = mfma_yardstick(torch, min(args.steps, 200))
+        if out is None:
+            print("bench.py: gomlx_amd/libgq_yardstick.so is missing (python -m gomlx_amd.build)", file=sys.stderr)
+            sys.exit(4)
+        print(json.dumps(out))
         return
     from gomlx_amd import _lib
     _lib.init(0)
@@ -635,9 +695,25 @@ def main():
                 pr["kernel_over_plain_read"] = rep["roofline"]["kernel_us"] / pr["us"]
                 rep["roofline"]["plain_read"] = pr
             rep["clock_state"] = prob.clock_state()
+        bound = prob.bound
         prob.close()
         del prob
         torch.cuda.empty_cache()
+        if not args.no_extras and bound == "mfma":
+            # measured in the same process right after the workload: the vendor library's plain bf16 GEMM on the same shape
+            # (no dequantisation, bf16 result) and the matrix instructions of such a GEMM alone
+            ku = rep["roofline"]["kernel_us"]
+            vg = matmul_yardstick(torch, 30)
+            rep["roofline"]["vendor_gemm"] = {"us": vg["us"], "tflops": vg["tflops"], "kernel_over_vendor_gemm": ku / vg["us"],
+                                              "note": "torch.matmul bf16 2048 x 4096 x 4096, weights already 16-bit, bf16 result, same run"}
+            torch.cuda.empty_cache()
+            mo = mfma_yardstick(torch, 100, only_first=True)
+            if mo is not None:
+                c = next(iter(mo["cases"].values()))
+                rep["roofline"]["mfma_only"] = {"us": c["us_per_launch"], "tflops": c["tflops"], "shader_mhz": c["shader_mhz_mean"],
+                                                "kernel_over_mfma_only": ku / c["us_per_launch"],
+                                                "note": "the same number of v_mfma_f32_32x32x16_bf16 per wavefront at the same occupancy and "
+                                                        "nothing else (random operands): what the chip sustains under its power limit"}
         return rep
 
     rep = measure(args.config, args.steps)

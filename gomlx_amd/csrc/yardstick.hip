@@ -11,6 +11,13 @@
 //     (1) one row per lane pair (header + four 16-byte pieces per lane: each load instruction touches
 //     32 different rows), (2) as consecutive 16-byte chunks of a row (nine per row, seven rows per
 //     load instruction).  The difference between 1 and 2 is the price of the address pattern alone.
+//   gqy_mfma: matrix instructions and nothing else.  Every wavefront of `wgs` workgroups (8 wavefronts each, two per
+//     SIMD, the prefill GEMM's occupancy) loads four operand fragments once and then issues `groups` groups of four
+//     independent v_mfma_f32_32x32x16_bf16 on its four accumulators: no memory traffic, no LDS, no barrier, no
+//     vector-ALU work inside the loop.  Each workgroup also reads the shader clock counter and the constant
+//     100 MHz counter before and after its loop, which gives the clock the chip actually ran at.  This is the rate at
+//     which this chip issues that many matrix instructions under its power limit: the ceiling for a GEMM of the
+//     same instruction count, whatever its data movement costs.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -66,9 +73,62 @@ __global__ __launch_bounds__(512) void read_q4k_tiles_kernel(const uint8_t *__re
     if (acc == 0x9E3779B9u) out[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 512 + tid] = acc;
 }
 
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+// clocks[4 wg .. 4 wg + 3] = shader clock at start, 100 MHz clock at start, shader clock at end, 100 MHz clock at end
+__global__ __launch_bounds__(512) void mfma_only_kernel(const uint4 *__restrict__ frags, int groups, unsigned long long *__restrict__ clocks,
+                                                        float *__restrict__ sink) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    bf16x8 a[2], b[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        a[i] = __builtin_bit_cast(bf16x8, frags[(wave * 4 + i) * 64 + lane]);
+        b[i] = __builtin_bit_cast(bf16x8, frags[(wave * 4 + 2 + i) * 64 + lane]);
+    }
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+    if (threadIdx.x == 0) {
+        clocks[4 * blockIdx.x] = clock64();
+        clocks[4 * blockIdx.x + 1] = wall_clock64();
+    }
+    for (int g = 0; g < groups; g++) {
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) t += acc[i][j][r];
+    // (wavefront 0's last accumulator is read above: the end stamp is taken after its matrix instructions have completed)
+    if (threadIdx.x == 0) {
+        clocks[4 * blockIdx.x + 2] = clock64() + (t == 12345.678f ? 1 : 0);
+        clocks[4 * blockIdx.x + 3] = wall_clock64();
+    }
+    if (t == 12345.678f) sink[blockIdx.x * 512 + threadIdx.x] = t;  // (practically never: keeps the instructions alive)
+}
+
 }  // namespace
 
 extern "C" {
+
+// frags: 8 wavefronts x 4 fragments x 64 lanes x 16 bytes (32 KiB) of bf16 operands; clocks: 4 x wgs uint64; sink: wgs x 512 floats.
+// Each wavefront issues 4 * groups matrix instructions (2 * 32 * 32 * 16 flop each).  Returns 0 or a hipError_t.
+int gqy_mfma(const void *frags, int groups, int wgs, void *clocks, void *sink, void *stream) {
+    hipLaunchKernelGGL(mfma_only_kernel, dim3(wgs), dim3(512), 0, (hipStream_t)stream, static_cast<const uint4 *>(frags), groups,
+                       static_cast<unsigned long long *>(clocks), static_cast<float *>(sink));
+    return (int)hipGetLastError();
+}
 
 // pattern 0: linear (N, row_bytes, slice_sb ignored).  pattern 1 / 2: Q4_K tiles, row per lane / coalesced.
 // `out` must hold wgs * threads (pattern 0) or (N / 128) * slices * 512 (patterns 1, 2) uint32.  Returns 0 or a hipError_t.
