@@ -35,8 +35,7 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 
 constexpr int kSliceSB = 8;                 // super-blocks per K-slice
 constexpr int kSliceK = kSliceSB * 256;     // 2048 values
-constexpr int kRowsPerWG = 128;             // 4 row tiles of 32; kParts wavefronts (interleaved super-blocks) per tile
-constexpr int kParts = 2;                   // wavefronts sharing a row tile
+constexpr int kParts = 2;                   // wavefronts sharing a row tile of 32 (interleaved super-blocks)
 constexpr int kMT = 32;                     // batch columns per pass
 constexpr int kXFBytes = kSliceK * kMT * 2;          // 131072: fp16 activations, fragment order
 constexpr int kXSBytes = kSliceSB * kMT * 16;        // 4096: eight sub-block sums per (super-block, column)
@@ -47,9 +46,18 @@ constexpr int kLdsBytes = kXFBytes + kXSBytes;
 // 14336 -> 4096 matrix take 10.9 us against 8.4 us with nothing else going on: the address pattern alone.
 constexpr int kParkBytes = 32 * 144;                 // one super-block of a 32-row tile
 constexpr int kParkLoads = 5;                        // 288 chunks / 64 lanes
-constexpr int kParkedSliceSB = 7;                    // longest slice whose image fits LDS next to eight parked tiles
-constexpr int kMainLdsBytes = kParkedSliceSB * 16384 + kXSBytes + 4 * kParts * kParkBytes;
-static_assert(kMainLdsBytes <= 160 * 1024, "image + parked tiles exceed LDS");
+// A workgroup of the Q4_K kernel covers RT row tiles with RT * kParts wavefronts; its LDS holds the slice's image and one
+// parked tile per wavefront, which bounds the slice: 7 super-blocks with 4 row tiles (8 wavefronts).  (8 row tiles on 16
+// wavefronts with slices of 4 super-blocks, four wavefronts per SIMD and half the image traffic, measured 22.8 us against
+// 20.0 us on a 14336 -> 4096 matrix at 32 rows: not built.)
+template <int RT> struct Q4KTile {
+    static_assert(RT == 4, "LDS budget below is for four row tiles");
+    static constexpr int kWaves = RT * kParts, kRows = 32 * RT;
+    static constexpr int kMaxSliceSB = 7;
+    static constexpr int kLds = kMaxSliceSB * 16384 + kXSBytes + kWaves * kParkBytes;
+    static_assert(kLds <= 160 * 1024, "image + parked tiles exceed LDS");
+};
+constexpr int kQ4KRowTiles = 4;
 
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
     h2 v;
@@ -210,11 +218,12 @@ __global__ __launch_bounds__(512) void mmq_xprep_kernel(const void *__restrict__
 
 // partial[slice][m][n] = sum over the slice's k of x[m][k] * w[n][k]
 //
-// 4 * kParts wavefronts: wavefront w contracts row tile (w & 3) (32 rows of W) over the
-// super-blocks (w >> 2), (w >> 2) + kParts, ... of the slice; the partial tiles meet in LDS at the end.  v_mfma_f32_32x32x16_f16 with
+// RT * kParts wavefronts: wavefront w contracts row tile w % RT (32 rows of W) over the
+// super-blocks w / RT, w / RT + kParts, ... of the slice; the partial tiles meet in LDS at the end.  v_mfma_f32_32x32x16_f16 with
 // A = activations (32 batch columns x 16 k) and B = weights (16 k x 32 rows): one 16-byte LDS
 // read per lane feeds 16384 multiply-adds, and a lane's 16 results all belong to its own row.
-__global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__restrict__ ximg, const uint8_t *__restrict__ W0,
+template <int RT>
+__global__ __launch_bounds__(64 * RT * kParts) void mmq_q4k_kernel(const uint8_t *__restrict__ ximg, const uint8_t *__restrict__ W0,
                                                       float *__restrict__ partial0, int M, int K, int N,
                                                       int64_t row_bytes, int m0, int slice_sb, const uint8_t *__restrict__ W2,
                                                       float *__restrict__ partial2) {
@@ -224,18 +233,18 @@ __global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__
     float *__restrict__ partial = blockIdx.z ? partial2 : partial0;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int kg = lane >> 5, col = lane & 31;
-    const int rt = wave & 3, par = wave >> 2;  // par = 0 .. kParts-1
+    const int rt = wave % RT, par = wave / RT;  // par = 0 .. kParts-1
     const int slice = blockIdx.y;
     const int k0 = slice * slice_sb * 256;
     const int nsb = min(slice_sb, (K - k0) >> 8);
-    const int n = blockIdx.x * kRowsPerWG + rt * 32 + col;  // this lane's weight row
+    const int n = blockIdx.x * (32 * RT) + rt * 32 + col;  // this lane's weight row
 
     // the slice's activation image goes straight from global memory into LDS (no registers)
     {
         const uint8_t *img = ximg + ((size_t)(m0 / kMT) * gridDim.y + slice) * kLdsBytes;
         // fragments of the slice's first slice_sb super-blocks (16 KiB each), then the 4 KiB of sub-block sums
         const int frag_kib = slice_sb * 16;
-        for (int i0 = wave; i0 < frag_kib + kXSBytes / 1024; i0 += 4 * kParts) {
+        for (int i0 = wave; i0 < frag_kib + kXSBytes / 1024; i0 += RT * kParts) {
             const int i = i0 < frag_kib ? i0 : kXFBytes / 1024 + (i0 - frag_kib);
             // (in LDS the sums follow the fragments directly; the image in memory keeps room for 8 super-blocks)
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(img + i * 1024 + lane * 16),
@@ -243,58 +252,53 @@ __global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__
         }
     }
     const int xs_off = slice_sb * 16384;
-    // Chunk c = lane + 64 l of a (32 rows x 144 bytes) tile is piece c % 9 of row c / 9.
-    typedef uint32_t Chunk __attribute__((ext_vector_type(4)));
-    const uint8_t *csrc[kParkLoads];
-    {
-        const int row0 = blockIdx.x * kRowsPerWG + rt * 32;
+    // Chunk c = lane + 64 l of a (32 rows x 144 bytes) tile is piece c % 9 of row c / 9.  The chunks go from global
+    // memory straight into the wavefront's piece of LDS (no registers held while they are in flight): each load
+    // instruction writes 64 lanes x 16 bytes to consecutive LDS addresses, which is the tile's own layout.
+    // (byte offsets from the first row of the tile: 32 rows of a matrix the index range admits stay far below 2^32)
+    const int row0 = blockIdx.x * (32 * RT) + rt * 32;
+    const uint8_t *wtile = W + (int64_t)min(row0, N - 1) * row_bytes + (int64_t)(k0 >> 8) * 144;
+    uint32_t csrc[kParkLoads];
 #pragma unroll
-        for (int l = 0; l < kParkLoads; l++) {
-            const int c = min(lane + 64 * l, 32 * 9 - 1);
-            csrc[l] = W + (int64_t)min(row0 + c / 9, N - 1) * row_bytes + (int64_t)(k0 >> 8) * 144 + (c % 9) * 16;
-        }
+    for (int l = 0; l < kParkLoads; l++) {
+        const int c = min(lane + 64 * l, 32 * 9 - 1);
+        csrc[l] = (uint32_t)(min(row0 + c / 9, N - 1) - min(row0, N - 1)) * (uint32_t)row_bytes + (uint32_t)((c % 9) * 16);
     }
-    // The loads are written as instructions so that they are issued where they stand (left to the compiler, the first
-    // fetch sinks below the barrier that waits for the image, and every workgroup then sits out a full HBM round trip
-    // after it); their results may be used after chunks_arrived() only.
-    auto fetch = [&](Chunk *dst, int sb) __attribute__((always_inline)) {
+    uint8_t *park = lds + xs_off + kXSBytes + wave * kParkBytes;
+    auto fetch = [&](int sb) __attribute__((always_inline)) {
+        const uint8_t *base = wtile + sb * 144;
 #pragma unroll
         for (int l = 0; l < kParkLoads; l++)
-            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst[l]) : "v"(csrc[l] + (int64_t)min(sb, nsb - 1) * 144) : "memory");
+            if (64 * l + 64 <= 32 * 9 || lane < 32 * 9 - 64 * l)  // (the last instruction carries 32 chunks)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(base + csrc[l]),
+                                                 (__attribute__((address_space(3))) void *)(park + l * 1024), 16, 0, 0);
     };
-    auto chunks_arrived = [&](Chunk *c) __attribute__((always_inline)) {
-        static_assert(kParkLoads == 5, "one operand per chunk below");
-        asm volatile("s_waitcnt vmcnt(0)" : "+v"(c[0]), "+v"(c[1]), "+v"(c[2]), "+v"(c[3]), "+v"(c[4])::"memory");
-    };
-    Chunk craw[kParkLoads];
-    fetch(craw, par);
-    uint8_t *park = lds + xs_off + kXSBytes + wave * kParkBytes;
+    if (par < nsb) fetch(par);
     const uint8_t *myrow = park + col * 144;
     __syncthreads();
 
-    f16v acc, acc2;
+    f16v acc;
 #pragma unroll
-    for (int r = 0; r < 16; r++) { acc[r] = 0.f; acc2[r] = 0.f; }
+    for (int r = 0; r < 16; r++) acc[r] = 0.f;
     uint32_t magic;
     asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));
 
     for (int sbl = par; sbl < nsb; sbl += kParts) {
-        // park the tile's super-block and pick out this lane's part (LDS operations of one wavefront execute in order;
-        // no other wavefront touches this piece of LDS), then request the next one
-        chunks_arrived(craw);
-#pragma unroll
-        for (int l = 0; l < kParkLoads; l++)
-            if (lane + 64 * l < 32 * 9) *reinterpret_cast<Chunk *>(park + (lane + 64 * l) * 16) = craw[l];
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        // the tile's super-block has landed in this wavefront's piece of LDS: pick out this lane's part, and once those
+        // reads are done request the next super-block into the same place
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        fetch(craw, sbl + kParts);
+        typedef uint32_t Chunk __attribute__((ext_vector_type(4)));
+        Chunk rhd = *reinterpret_cast<const Chunk *>(myrow), rc[4];
+#pragma unroll
+        for (int st = 0; st < 4; st++) rc[st] = *reinterpret_cast<const Chunk *>(myrow + 16 + 32 * st + 16 * kg);
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(rhd), "+v"(rc[0]), "+v"(rc[1]), "+v"(rc[2]), "+v"(rc[3])::"memory");
         RawSB cur;
-        cur.hd = *reinterpret_cast<const uint4 *>(myrow);
+        cur.hd = make_uint4(rhd.x, rhd.y, rhd.z, rhd.w);
 #pragma unroll
-        for (int st = 0; st < 4; st++) cur.c[st] = *reinterpret_cast<const uint4 *>(myrow + 16 + 32 * st + 16 * kg);
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // these reads are done before the next super-block is parked
+        for (int st = 0; st < 4; st++) cur.c[st] = make_uint4(rc[st].x, rc[st].y, rc[st].z, rc[st].w);
         __builtin_amdgcn_wave_barrier();
+        if (sbl + kParts < nsb) fetch(sbl + kParts);
         const float d = half_bits_to_float(cur.hd.x & 0xFFFFu), dmin = half_bits_to_float(cur.hd.x >> 16);
         // all eight 6-bit scales / minima as bytes: sc0..3, sc4..7, m0..3, m4..7
         const uint32_t a = cur.hd.y, b = cur.hd.z, c = cur.hd.w;
@@ -342,7 +346,7 @@ __global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__
         uint4 mv = make_uint4(0u, 0u, 0u, 0u), sv = make_uint4(0u, 0u, 0u, 0u);
         if (kg == 0) {
             const h2 off = as_h2(0xE400E400u);  // (-1024, -1024)
-            const _Float16 dmh = (_Float16)dmin;
+            const _Float16 dmh = (_Float16)-dmin;  // (the minima are subtracted)
             h2 dm2;
             dm2.x = dmh;
             dm2.y = dmh;
@@ -352,15 +356,10 @@ __global__ __launch_bounds__(256 * kParts) void mmq_q4k_kernel(const uint8_t *__
             mv.w = __builtin_bit_cast(uint32_t, (magic_pair(mn_hi >> 8, 0x00FF00FFu, magic) + off) * dm2);
             sv = *reinterpret_cast<const uint4 *>(lds + xs_off + (sbl * kMT + col) * 16);
         }
-        acc2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, sv), __builtin_bit_cast(h8, mv), acc2, 0, 0, 0);
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[r] = fmaf(d, p1[r], acc[r]);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, sv), __builtin_bit_cast(h8, mv), acc, 0, 0, 0);
     }
-    // The request past the end of the slice (clamped to its last super-block) still writes its registers: nothing
-    // else may live there before it has landed.
-    chunks_arrived(craw);
-#pragma unroll
-    for (int r = 0; r < 16; r++) acc[r] -= acc2[r];
 
     // wavefronts 1..kParts-1 of a row tile hand their 32 x 32 partial tiles to wavefront 0 through LDS
     __syncthreads();
@@ -988,24 +987,22 @@ int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, co
     if (type == kIQ4_NL) return launch_mmq_b32<kIQ4_NL, 4>(x, x_is_bf16, M, K, W, N, bias, act, y, s, ex);
     if (type == kQ6_K) return launch_mmq_q6k(ex, x, x_is_bf16, M, K, W, N, bias, act, y, s);
     if (type != kQ4_K) return fail(GQ_ERR_NOT_IMPLEMENTED, "mmq: ggml type %d is not implemented", type);
+    typedef Q4KTile<kQ4KRowTiles> Tile;
     static const bool lds_ok = [] {
-        return hipFuncSetAttribute(reinterpret_cast<const void *>(mmq_q4k_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   kMainLdsBytes) == hipSuccess;
+        return hipFuncSetAttribute(reinterpret_cast<const void *>(mmq_q4k_kernel<kQ4KRowTiles>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   Tile::kLds) == hipSuccess;
     }();
-    if (!lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", kMainLdsBytes);
-    // K-slices of 8 super-blocks, or of 4 / 2 when the problem would otherwise leave more than a quarter of the
-    // CUs without a workgroup (4096 x 4096: 2 slices x 32 row ranges = 64 workgroups with 8, 256 with 2: 18.8 -> 16.6 us;
-    // splitting 224 workgroups into 448 costs more than it brings: 20.8 -> 24.9 us on 4096 -> 14336)
+    if (!lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", Tile::kLds);
     const int mtiles = (int)((M + kMT - 1) / kMT);
-    const int64_t rowwgs = (N + kRowsPerWG - 1) / kRowsPerWG, sbs = K / 256;
+    const int64_t rowwgs = (N + Tile::kRows - 1) / Tile::kRows, sbs = K / 256;
     // Super-blocks per K-slice (at most 7: the image shares LDS with the parked tiles): the count that needs the fewest
     // rounds of workgroups over the chip times the length of a round (+3: what a workgroup costs beyond its
     // super-blocks); ties go to the longer slice (fewer partial sums).
-    int slice_sb = kParkedSliceSB;
+    int slice_sb = Tile::kMaxSliceSB;
     {
         const int64_t cus = device_cu_count(), z = W2 ? 2 : 1;
         int64_t best_cost = INT64_MAX;
-        for (int ssb = kParkedSliceSB; ssb >= 2; ssb--) {
+        for (int ssb = Tile::kMaxSliceSB; ssb >= 2; ssb--) {
             const int64_t wgs = rowwgs * ((sbs + ssb - 1) / ssb) * z;
             const int64_t cost = ((wgs + cus - 1) / cus) * (ssb + 3);
             if (cost < best_cost) { best_cost = cost; slice_sb = ssb; }
@@ -1029,11 +1026,11 @@ int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, co
                                     (int)K, slice_sb, norm ? norm->gain : nullptr, norm ? norm->gain_offset : 0.f,
                                     norm ? mmq_xss(xscale, nslices, M) : nullptr))
         return rc;
-    const dim3 grid((unsigned)((N + kRowsPerWG - 1) / kRowsPerWG), (unsigned)nslices, W2 ? 2u : 1u);  // (both matrices of a gated pair in one launch)
+    const dim3 grid((unsigned)rowwgs, (unsigned)nslices, W2 ? 2u : 1u);  // (both matrices of a gated pair in one launch)
     float *partial2 = W2 ? partial + (size_t)nslices * M * N : nullptr;
     for (int64_t m0 = 0; m0 < M; m0 += kMT) {
-        if (int rc = launch(mmq_q4k_kernel, grid, dim3(256 * kParts), (size_t)kMainLdsBytes, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N,
-                            row_bytes, (int)m0, slice_sb, W2, partial2))
+        if (int rc = launch(mmq_q4k_kernel<kQ4KRowTiles>, grid, dim3(64 * Tile::kWaves), (size_t)Tile::kLds, s, (const uint8_t *)ximg, W, partial,
+                            (int)M, (int)K, (int)N, row_bytes, (int)m0, slice_sb, W2, partial2))
             return rc;
     }
     return launch_mmq_reduce(partial, partial2, xscale, nslices, M, K, N, bias, act, y, ex, s);
