@@ -342,23 +342,28 @@ __global__ __launch_bounds__(64 * RT * kParts) void mmq_q4k_kernel(const uint8_t
                 p1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xfr[4 * st + q], wfrag, p1, 0, 0, 0);
             }
         }
-        // minima: k-group 0 carries dmin * (m0, m2, m1, m3, m4, m6, m5, m7) against the sums in the same order
-        uint4 mv = make_uint4(0u, 0u, 0u, 0u), sv = make_uint4(0u, 0u, 0u, 0u);
-        if (kg == 0) {
-            const h2 off = as_h2(0xE400E400u);  // (-1024, -1024)
-            const _Float16 dmh = (_Float16)-dmin;  // (the minima are subtracted)
-            h2 dm2;
-            dm2.x = dmh;
-            dm2.y = dmh;
-            mv.x = __builtin_bit_cast(uint32_t, (magic_pair(mn_lo, 0x00FF00FFu, magic) + off) * dm2);
-            mv.y = __builtin_bit_cast(uint32_t, (magic_pair(mn_lo >> 8, 0x00FF00FFu, magic) + off) * dm2);
-            mv.z = __builtin_bit_cast(uint32_t, (magic_pair(mn_hi, 0x00FF00FFu, magic) + off) * dm2);
-            mv.w = __builtin_bit_cast(uint32_t, (magic_pair(mn_hi >> 8, 0x00FF00FFu, magic) + off) * dm2);
-            sv = *reinterpret_cast<const uint4 *>(lds + xs_off + (sbl * kMT + col) * 16);
+        // minima: k-group 0 carries the exact integers (m0, m2, m1, m3, m4, m6, m5, m7) against the sub-block sums of x in
+        // the same order; dmin multiplies the finished fp32 sums below, as d multiplies p1 (in an fp16 operand dmin * m
+        // would be rounded to 11 bits, and overflow from dmin = 1040 on)
+        f16v p2, zero16;
+#pragma unroll
+        for (int r = 0; r < 16; r++) zero16[r] = 0.f;
+        {
+            uint4 mv = make_uint4(0u, 0u, 0u, 0u), sv = make_uint4(0u, 0u, 0u, 0u);
+            if (kg == 0) {
+                const h2 off = as_h2(0xE400E400u);  // (-1024, -1024)
+                mv.x = __builtin_bit_cast(uint32_t, magic_pair(mn_lo, 0x00FF00FFu, magic) + off);
+                mv.y = __builtin_bit_cast(uint32_t, magic_pair(mn_lo >> 8, 0x00FF00FFu, magic) + off);
+                mv.z = __builtin_bit_cast(uint32_t, magic_pair(mn_hi, 0x00FF00FFu, magic) + off);
+                mv.w = __builtin_bit_cast(uint32_t, magic_pair(mn_hi >> 8, 0x00FF00FFu, magic) + off);
+                sv = *reinterpret_cast<const uint4 *>(lds + xs_off + (sbl * kMT + col) * 16);
+            }
+            p2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, sv), __builtin_bit_cast(h8, mv), zero16, 0, 0, 0);
         }
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[r] = fmaf(d, p1[r], acc[r]);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, sv), __builtin_bit_cast(h8, mv), acc, 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = fmaf(-dmin, p2[r], acc[r]);
     }
 
     // wavefronts 1..kParts-1 of a row tile hand their 32 x 32 partial tiles to wavefront 0 through LDS

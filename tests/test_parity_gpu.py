@@ -254,6 +254,30 @@ def test_split_k_small_batches_k_quants(gpu, oracle, t, M, K, N):
     assert rel_err(run_dense(gpu, t, xb, W, bias, 3, bf16=True), oracle.c_qdense(t, xb, W, bias, 3)) < tol, (t, M, K, N, "bf16")
 
 
+def test_q4_k_large_minima_through_the_split_k_kernel(gpu, oracle):
+    """Q4_K super-blocks whose minimum term is as large as the format allows to matter: dmin = 2048 with every 6-bit minimum at
+    63 (dmin * m = 129 024 lies beyond the largest fp16, 65 504, and has 17 significant bits).  The small-batch kernel must
+    carry dmin in fp32, as the decode GEMV and the dequantisation do: 8 and 32 rows against the oracle, and against the
+    one-row result of the same activations."""
+    N, K = 256, 2048
+    W = synth.weights(Q4_K, 91, N, K).copy().reshape(N, K // 256, 144)
+    W[:, :, 2:4] = np.frombuffer(np.float16(2048.0).tobytes(), dtype=np.uint8)   # dmin
+    W[:, :, 0:2] = np.frombuffer(np.float16(0.5).tobytes(), dtype=np.uint8)      # d
+    sc = W[:, :, 4:16].copy()                   # the 12 bytes of packed 6-bit scales and minima
+    sc[:, :, 4:8] = 0xFF                        # m0..m3 = 63 (low six bits) and the two high bits of m4..m7
+    sc[:, :, 8:12] |= 0xF0                      # the low four bits of m4..m7
+    W[:, :, 4:16] = sc
+    W = W.reshape(N, -1)
+    for M in (8, 32):
+        x = synth.activations(92, M, K)
+        want = oracle.c_qdense(Q4_K, x, W, None, 0)
+        got = run_dense(gpu, Q4_K, x, W)
+        assert np.all(np.isfinite(got)), M
+        assert rel_err(got, want) < TOL_F32, (M, rel_err(got, want))
+        one = np.concatenate([run_dense(gpu, Q4_K, x[m:m + 1], W) for m in range(2)])
+        assert rel_err(got[:2], one) < TOL_F32, M
+
+
 @pytest.mark.parametrize("t", [Q6_K, Q4_K])
 def test_output_head_of_a_128k_vocabulary(gpu, oracle, t):
     """The largest projection of a decoder: hidden state -> logits over 128 256 tokens (K = 4096; several hundred
