@@ -205,15 +205,15 @@ struct RawSB { uint4 hd, c[4]; };  // header + this lane's four chunks (steps 0.
 // slice_sb <= 8 super-blocks per slice: a thread whose octet lies beyond them has nothing to do (the
 // image keeps its 8-super-block layout; the main kernel copies and uses the first slice_sb only).
 // xscale[slice][M]: the inverse of the power of two that (slice, column) was scaled by.
-template <bool BF16X>
+template <bool BF16X, int ROUNDS>
 __global__ __launch_bounds__(512) void mmq_xprep_kernel(const void *__restrict__ X, uint8_t *__restrict__ ximg, float *__restrict__ xscale, int M,
                                                         int K, int slice_sb, const float *__restrict__ gain, float gain_offset,
                                                         float *__restrict__ xss) {
-    __shared__ float red[2 * 2 * 2 * 4];
+    __shared__ float red[2 * 2 * ROUNDS * 4];
     const int slice = blockIdx.x, mt = blockIdx.y;
     const bool active = (((int)threadIdx.x & 255) >> 5) < slice_sb;
-    stage_x<2, BF16X>(X, M, K, mt * kMT, slice * slice_sb * 256, ximg + ((size_t)mt * gridDim.x + slice) * kLdsBytes, threadIdx.x,
-                      2 * blockIdx.z, active, red, xscale + (size_t)slice * M, gain, gain_offset, xss ? xss + (size_t)slice * M : nullptr);
+    stage_x<ROUNDS, BF16X>(X, M, K, mt * kMT, slice * slice_sb * 256, ximg + ((size_t)mt * gridDim.x + slice) * kLdsBytes, threadIdx.x,
+                      ROUNDS * blockIdx.z, active, red, xscale + (size_t)slice * M, gain, gain_offset, xss ? xss + (size_t)slice * M : nullptr);
 }
 
 // partial[slice][m][n] = sum over the slice's k of x[m][k] * w[n][k]
@@ -395,7 +395,7 @@ __global__ __launch_bounds__(256) void mmq_reduce_kernel(const float *__restrict
                                                          int64_t MN, int N, const float *__restrict__ bias, const float *__restrict__ bias2,
                                                          int act, const float *residual, float *Y, const float *__restrict__ xscale,
                                                          const float *__restrict__ xss, float eps, float inv_k) {
-    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
     if (i >= MN) return;
     const bool small = MN <= (int64_t)INT32_MAX;  // (32-bit divisions are a fraction of the cost of 64-bit ones)
     const int M = small ? (int)((uint32_t)MN / (uint32_t)N) : (int)(MN / N);
@@ -455,7 +455,9 @@ int launch_mmq_reduce(const float *partial, const float *partial2, const float *
                       const float *bias, int act, float *y, const MmqExtra *ex, hipStream_t s) {
     const int64_t MN = M * N;
     const RmsNorm *norm = ex ? ex->norm : nullptr;
-    return launch(mmq_reduce_kernel, dim3((unsigned)((MN / 4 + 255) / 256)), dim3(256), 0, s, partial, partial2, nslices, MN, (int)N, bias,
+    // (workgroups of 64 threads while 256 would leave CUs without one: the kernel is one round trip to memory long)
+    const int threads = MN / 4 / 256 >= 2 * device_cu_count() ? 256 : 64;
+    return launch(mmq_reduce_kernel, dim3((unsigned)((MN / 4 + threads - 1) / threads)), dim3(threads), 0, s, partial, partial2, nslices, MN, (int)N, bias,
                   ex ? ex->bias2 : nullptr, act, ex ? ex->residual : nullptr, y, xscale, norm ? mmq_xss(xscale, nslices, M) : nullptr,
                   norm ? norm->eps : 0.f, 1.0f / (float)K);
 }
@@ -1025,11 +1027,15 @@ int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, co
     float *partial = reinterpret_cast<float *>(ximg + img_bytes + mmq_scale_bytes(nslices, M));
     const int64_t row_bytes = (K / 256) * 144;
     const RmsNorm *norm = ex ? ex->norm : nullptr;
-    if (int rc = x_is_bf16 ? launch(mmq_xprep_kernel<true>, dim3((unsigned)nslices, (unsigned)mtiles, 8), dim3(512), 0, s, x, ximg, xscale, (int)M,
-                                    (int)K, slice_sb, nullptr, 0.f, nullptr)
-                           : launch(mmq_xprep_kernel<false>, dim3((unsigned)nslices, (unsigned)mtiles, 8), dim3(512), 0, s, x, ximg, xscale, (int)M,
-                                    (int)K, slice_sb, norm ? norm->gain : nullptr, norm ? norm->gain_offset : 0.f,
-                                    norm ? mmq_xss(xscale, nslices, M) : nullptr))
+    // (each workgroup of the pre-pass converts 2 or 4 of a tile's 32 columns: the finer split while it still leaves CUs idle)
+    const bool fine = (int64_t)nslices * mtiles * 8 * 2 <= device_cu_count();
+    const dim3 pgrid((unsigned)nslices, (unsigned)mtiles, fine ? 16u : 8u);
+    const float *gain = norm ? norm->gain : nullptr;
+    const float goff = norm ? norm->gain_offset : 0.f;
+    float *xss = norm && !x_is_bf16 ? mmq_xss(xscale, nslices, M) : nullptr;
+    auto prep = [&](auto kernel) { return launch(kernel, pgrid, dim3(512), 0, s, x, ximg, xscale, (int)M, (int)K, slice_sb, x_is_bf16 ? nullptr : gain, x_is_bf16 ? 0.f : goff, xss); };
+    if (int rc = x_is_bf16 ? (fine ? prep(mmq_xprep_kernel<true, 1>) : prep(mmq_xprep_kernel<true, 2>))
+                           : (fine ? prep(mmq_xprep_kernel<false, 1>) : prep(mmq_xprep_kernel<false, 2>)))
         return rc;
     const dim3 grid((unsigned)rowwgs, (unsigned)nslices, W2 ? 2u : 1u);  // (both matrices of a gated pair in one launch)
     float *partial2 = W2 ? partial + (size_t)nslices * M * N : nullptr;
