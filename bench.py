@@ -741,7 +741,9 @@ def main():
         for name in names:
             if name == args.config:
                 continue
-            steps = args.steps if name not in ("c3", "prefill") else max(10, args.steps // 10)
+            # (the side measurements choose their own step counts: --steps is the headline's; short runs of the small
+            # workloads read up to 10 % slow)
+            steps = max(args.steps, 200) if name not in ("c3", "prefill") else max(30, args.steps // 10)
             r = measure(name, steps)
             others[name] = {"workload": WORKLOAD_TEXT[name], "dtype": DTYPE[name], "arithmetic": ARITHMETIC[name], "metric": r["metric"],
                             "value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"], "roofline": r["roofline"],
