@@ -5,10 +5,11 @@
 // below the MFMA machine balance, so the kernel should run at the speed the packed weights
 // stream from HBM.  Two things decide whether it does:
 //
-//  * Activation traffic.  Every 16-row tile of W needs all of x.  Fetching x per tile through
-//    the CU's vector-memory path would move ~7x more bytes than the weights themselves, so the
-//    work is split along K instead: a workgroup owns a K-slice of 2048 values (8 super-blocks),
-//    keeps the slice of x for 32 batch columns resident in LDS (fp16, 128 KiB) and streams
+//  * Activation traffic.  Every row tile of W needs all of x.  Fetching x per tile through
+//    the CU's vector-memory path would move several times more bytes than the weights themselves, so the
+//    work is split along K instead: a workgroup owns a K-slice of up to 7 super-blocks (1792 values),
+//    keeps the slice of x for 32 batch columns resident in LDS (fp16 in MFMA fragment order, written
+//    once by a pre-pass and copied global -> LDS without passing registers) and streams
 //    128 rows of W past it.  Slices are summed by a second, tiny kernel that also applies
 //    bias and activation (deterministic order, no atomics).
 //
@@ -16,12 +17,12 @@
 //    becomes four MFMA operand fragments directly in registers: (dword & 0x000F000F) | 0x6400
 //    is the fp16 pair (1024 + n_a, 1024 + n_b); one packed fma with the 6-bit sub-block scale
 //    gives the exact integers sc*n (<= 945, exact in fp16); these accumulate over a whole
-//    super-block on v_mfma_f32_16x16x32_f16, and only then are scaled by the fp16 d in fp32.
-//    The sub-block minima ride on one extra MFMA per super-block against per-sub-block sums
-//    of x.  The only rounding that is not fp32 is x -> fp16 (2^-12 relative).
+//    super-block on v_mfma_f32_32x32x16_f16, and only then are scaled by the fp16 d in fp32.
+//    The sub-block minima (exact 6-bit integers) ride on one extra MFMA per super-block against
+//    per-sub-block sums of x, scaled by dmin in fp32.  The only rounding that is not fp32 is x -> fp16 (2^-12 relative).
 //
 // MFMA roles: A = activations (rows = batch columns), B = weights (columns = W rows), so a
-// lane's four results belong to ONE weight row, the one whose header it has already loaded.
+// lane's sixteen results belong to ONE weight row, the one whose header it has already loaded.
 #include "blocks.hpp"
 #include "common.hpp"
 
@@ -33,7 +34,7 @@ typedef _Float16 h2 __attribute__((ext_vector_type(2)));
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 typedef float f16v __attribute__((ext_vector_type(16)));
 
-constexpr int kSliceSB = 8;                 // super-blocks per K-slice
+constexpr int kSliceSB = 8;                 // super-blocks a slice's activation image has room for (a slice uses up to 7)
 constexpr int kSliceK = kSliceSB * 256;     // 2048 values
 constexpr int kParts = 2;                   // wavefronts sharing a row tile of 32 (interleaved super-blocks)
 constexpr int kMT = 32;                     // batch columns per pass
