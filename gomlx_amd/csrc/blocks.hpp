@@ -43,6 +43,11 @@ __device__ __forceinline__ float ubyte0(uint32_t v) { float f; asm("v_cvt_f32_ub
 __device__ __forceinline__ float ubyte1(uint32_t v) { float f; asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(v)); return f; }
 __device__ __forceinline__ float ubyte2(uint32_t v) { float f; asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(v)); return f; }
 __device__ __forceinline__ float ubyte3(uint32_t v) { float f; asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(v)); return f; }
+// byte n of v as a signed 8-bit integer, converted to float in one instruction (sub-dword operand select with sign extension)
+__device__ __forceinline__ float sbyte0(uint32_t v) { float f; asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_0" : "=v"(f) : "v"(v)); return f; }
+__device__ __forceinline__ float sbyte1(uint32_t v) { float f; asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1" : "=v"(f) : "v"(v)); return f; }
+__device__ __forceinline__ float sbyte2(uint32_t v) { float f; asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_2" : "=v"(f) : "v"(v)); return f; }
+__device__ __forceinline__ float sbyte3(uint32_t v) { float f; asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_3" : "=v"(f) : "v"(v)); return f; }
 
 // Public GGML IQ4_NL code book (compute.IQ4NLLookupTable, ml/ggml/dequant.go:130).
 __device__ __forceinline__ float iq4nl_value(uint32_t nib) {

@@ -75,16 +75,15 @@ template <> struct WRaw<kQ8_0> {
         d = load_u16(blk);
         q = *reinterpret_cast<const u128_a2 *>(blk + 2 + 16 * (run & 1));
     }
-    // Values 4 part .. 4 part + 3 of the run.  int8 q = (q ^ 0x80) - 128 with the xor-ed byte read
-    // as unsigned; fma(u, d, -128 d) = d * q exactly (the product has at most 18 significant
-    // bits), i.e. the reference's f32(d) * f32(q).
+    // Values 4 part .. 4 part + 3 of the run: f32(d) * f32(q), the reference's product (exact: at most 18 significant
+    // bits), each int8 converted by one instruction.
     __device__ __forceinline__ void part(int i, float *w) const {
-        const float df = half_bits_to_float(d), off = -128.0f * df;
-        const uint32_t a = q.v[i] ^ 0x80808080u;
-        w[4 * i + 0] = fmaf(ubyte0(a), df, off);
-        w[4 * i + 1] = fmaf(ubyte1(a), df, off);
-        w[4 * i + 2] = fmaf(ubyte2(a), df, off);
-        w[4 * i + 3] = fmaf(ubyte3(a), df, off);
+        const float df = half_bits_to_float(d);
+        const uint32_t a = q.v[i];
+        w[4 * i + 0] = sbyte0(a) * df;
+        w[4 * i + 1] = sbyte1(a) * df;
+        w[4 * i + 2] = sbyte2(a) * df;
+        w[4 * i + 3] = sbyte3(a) * df;
     }
 };
 
@@ -169,7 +168,9 @@ template <> struct XRaw<false> {
 
 
 // X must be 16-byte aligned; K % 32 == 0.
-template <int T, bool BF16>
+// KTAIL: K is not a multiple of the 64-wide step (the last step covers 32 columns); without it the step's address
+// selects and masks drop out of the loop.
+template <int T, bool BF16, bool KTAIL>
 // (Xv and W are deliberately not __restrict__: loads through restrict-qualified read-only pointers
 // may be moved across the workgroup barriers, away from the place that gives them two steps of
 // latency cover.)
@@ -202,7 +203,7 @@ __global__ __launch_bounds__(512) void gemm_kernel(const void *Xv, const uint8_t
     wr[1].set_row(W + (int64_t)(bn + wrow_c) * row_bytes);
     const int nk = (K + BK - 1) / BK;
     const int64_t n16 = K >> 4;
-    const bool ktail = (K % BK) != 0;  // the last step covers 32 columns only
+    constexpr bool ktail = KTAIL;  // the last step covers 32 columns only
     // constant per-thread byte offsets, for full steps and for a half last step
     uint32_t xoff[XRaw<BF16>::NCH], xoff_t[XRaw<BF16>::NCH];
 #pragma unroll
@@ -354,18 +355,23 @@ __global__ __launch_bounds__(512) void gemm_kernel(const void *Xv, const uint8_t
     }
 }
 
-template <int T, bool BF16>
-int launch_one(const void *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y,
+template <int T, bool BF16, bool KTAIL>
+int launch_one_k(const void *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y,
                hipStream_t s) {
     static const bool lds_ok = [] {
-        return hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kernel<T, BF16>),
+        return hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_kernel<T, BF16, KTAIL>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) == hipSuccess;
     }();
     if (!lds_ok) return fail(GQ_ERR_HIP, "gemm: cannot reserve %d bytes of LDS", LDS_BYTES);
     const int64_t row_bytes = (K / Geom<T>::vpb) * Geom<T>::bpb;
     const dim3 grid((unsigned)((N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM));
-    return launch(gemm_kernel<T, BF16>, grid, dim3(512), (size_t)LDS_BYTES, s, x, W, bias, y, (int)M, (int)K, (int)N, row_bytes,
+    return launch(gemm_kernel<T, BF16, KTAIL>, grid, dim3(512), (size_t)LDS_BYTES, s, x, W, bias, y, (int)M, (int)K, (int)N, row_bytes,
                   act);
+}
+
+template <int T, bool BF16>
+int launch_one(const void *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y, hipStream_t s) {
+    return K % BK ? launch_one_k<T, BF16, true>(x, M, K, W, N, bias, act, y, s) : launch_one_k<T, BF16, false>(x, M, K, W, N, bias, act, y, s);
 }
 
 template <int T>
