@@ -634,6 +634,28 @@ int gq_qdense_norm_f32_batch(int count, const gq_dense_desc *descs, const gq_rms
         const RmsNorm rn{norm->dGain, norm->eps, norm->gain_offset};
         return launch_gemv_ks_batch_norm(descs[0].type, count, items, &rn, (hipStream_t)stream, (int)rows);
     }
+    // Beyond the GEMV's rows: projections of the same activations (q / k / v) share one split-K pass - one activation
+    // image, one main launch over all their rows, one reduction - where the matrices taken together are in that
+    // kernel's range (three calls would convert the activations three times and pay nine launches).
+    if (count >= 2 && count <= 4 && (!norm->dGain || aligned_to(norm->dGain, 16))) {
+        MmqSetItem set[4];
+        bool same = true;
+        int64_t ntot = 0;
+        for (int i = 0; i < count && same; i++) {
+            const gq_dense_desc &d = descs[i];
+            same = d.type == descs[0].type && d.dX == descs[0].dX && d.M == rows && d.K == descs[0].K && d.N > 0;
+            set[i] = MmqSetItem{(const uint8_t *)d.dW, d.N, d.dBias, d.act, d.dY};
+            ntot += d.N;
+        }
+        const int type = descs[0].type;
+        const int64_t K = descs[0].K;
+        if (same && mmq_set_supported(type, count, set, rows, K, descs[0].dX) &&
+            rows >= block_split_k_from(type, weight_bytes_of(type, K, ntot), false) &&
+            (rows <= split_k_to(type, K, ntot) || !gemm_two_pass_supported(type, false, rows, K, ntot, descs[0].dX))) {
+            const RmsNorm rn{norm->dGain, norm->eps, norm->gain_offset};
+            return launch_mmq_set(type, descs[0].dX, false, rows, K, count, set, &rn, (hipStream_t)stream);
+        }
+    }
     for (int i = 0; i < count; i++) {
         const gq_dense_desc &d = descs[i];
         if (int rc = gq_qdense_block_f32(d.type, d.dX, d.M, d.K, norm, d.dW, d.N, d.dBias, d.act, nullptr, d.dY, stream)) return rc;

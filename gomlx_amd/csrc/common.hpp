@@ -86,6 +86,12 @@ struct RmsNorm { const float *gain; float eps, gain_offset; };
 struct MmqExtra { const uint8_t *W2; const float *bias2; const float *residual; const RmsNorm *norm; };
 int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias,
                int act, float *y, hipStream_t s, const MmqExtra *ex = nullptr);
+// Several matrices of one K contracted against the same activations (fp32 or bf16 [M, K]) in one split-K pass: one
+// activation pre-pass, one main launch over all their rows, one reduction (Q4_K; 2 to 4 matrices, each as mmq_supported asks).
+struct MmqSetItem { const uint8_t *W; int64_t N; const float *bias; int act; float *y; };
+bool mmq_set_supported(int type, int count, const MmqSetItem *items, int64_t M, int64_t K, const void *x);
+int launch_mmq_set(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, int count, const MmqSetItem *items, const RmsNorm *norm,
+                   hipStream_t s);
 // The K-sliced GEMV with the normalisation folded in and, when W2 is given, the gated product
 // act(x.W + bias) * (x.W2 + bias2); fp32 activations, at most 16 rows (the entry points use it below 8 rows, where a pass per row still wins).
 bool gemv_ks_ext_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, const void *gain);

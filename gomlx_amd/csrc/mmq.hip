@@ -217,28 +217,43 @@ __global__ __launch_bounds__(512) void mmq_xprep_kernel(const void *__restrict__
                       ROUNDS * blockIdx.z, active, red, xscale + (size_t)slice * M, gain, gain_offset, xss ? xss + (size_t)slice * M : nullptr);
 }
 
-// partial[slice][m][n] = sum over the slice's k of x[m][k] * w[n][k]
+// Up to four matrices that are contracted against one activation image in one launch (the q / k / v projections behind
+// one normalisation): matrix p owns workgroups wg0[p] .. of grid.x and columns n0[p] .. n0[p] + N[p] - 1 of the
+// partial sums, whose rows are ntot = sum of N[p] long.
+constexpr int kMaxSet = 4;
+struct Q4KSet {
+    const uint8_t *W[kMaxSet];
+    int N[kMaxSet], wg0[kMaxSet], n0[kMaxSet];
+    int count, ntot;
+};
+
+// partial[slice][m][n0[p] + n] = sum over the slice's k of x[m][k] * w_p[n][k]
 //
 // RT * kParts wavefronts: wavefront w contracts row tile w % RT (32 rows of W) over the
 // super-blocks w / RT, w / RT + kParts, ... of the slice; the partial tiles meet in LDS at the end.  v_mfma_f32_32x32x16_f16 with
 // A = activations (32 batch columns x 16 k) and B = weights (16 k x 32 rows): one 16-byte LDS
 // read per lane feeds 16384 multiply-adds, and a lane's 16 results all belong to its own row.
 template <int RT>
-__global__ __launch_bounds__(64 * RT * kParts) void mmq_q4k_kernel(const uint8_t *__restrict__ ximg, const uint8_t *__restrict__ W0,
-                                                      float *__restrict__ partial0, int M, int K, int N,
+__global__ __launch_bounds__(64 * RT * kParts) void mmq_q4k_kernel(const uint8_t *__restrict__ ximg, Q4KSet set,
+                                                      float *__restrict__ partial0, int M, int K,
                                                       int64_t row_bytes, int m0, int slice_sb, const uint8_t *__restrict__ W2,
                                                       float *__restrict__ partial2) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     // blockIdx.z = 1: the second matrix of a gated pair (same activation image, its own partial sums)
-    const uint8_t *__restrict__ W = blockIdx.z ? W2 : W0;
+    int prob = 0;
+#pragma unroll
+    for (int j = 1; j < kMaxSet; j++)
+        if (j < set.count && (int)blockIdx.x >= set.wg0[j]) prob = j;
+    const uint8_t *__restrict__ W = blockIdx.z ? W2 : set.W[prob];
     float *__restrict__ partial = blockIdx.z ? partial2 : partial0;
+    const int N = set.N[prob], xblk = (int)blockIdx.x - set.wg0[prob];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int kg = lane >> 5, col = lane & 31;
     const int rt = wave % RT, par = wave / RT;  // par = 0 .. kParts-1
     const int slice = blockIdx.y;
     const int k0 = slice * slice_sb * 256;
     const int nsb = min(slice_sb, (K - k0) >> 8);
-    const int n = blockIdx.x * (32 * RT) + rt * 32 + col;  // this lane's weight row
+    const int n = xblk * (32 * RT) + rt * 32 + col;  // this lane's weight row
 
     // the slice's activation image goes straight from global memory into LDS (no registers)
     {
@@ -257,7 +272,7 @@ __global__ __launch_bounds__(64 * RT * kParts) void mmq_q4k_kernel(const uint8_t
     // memory straight into the wavefront's piece of LDS (no registers held while they are in flight): each load
     // instruction writes 64 lanes x 16 bytes to consecutive LDS addresses, which is the tile's own layout.
     // (byte offsets from the first row of the tile: 32 rows of a matrix the index range admits stay far below 2^32)
-    const int row0 = blockIdx.x * (32 * RT) + rt * 32;
+    const int row0 = xblk * (32 * RT) + rt * 32;
     const uint8_t *wtile = W + (int64_t)min(row0, N - 1) * row_bytes + (int64_t)(k0 >> 8) * 144;
     uint32_t csrc[kParkLoads];
 #pragma unroll
@@ -383,7 +398,7 @@ __global__ __launch_bounds__(64 * RT * kParts) void mmq_q4k_kernel(const uint8_t
             float v = acc[r];
 #pragma unroll
             for (int p = 0; p < kParts - 1; p++) v += xch[(p * 16 + r) * 64 + lane];
-            if (m < M) partial[((int64_t)slice * M + m) * N + n] = v;
+            if (m < M) partial[((int64_t)slice * M + m) * set.ntot + set.n0[prob] + n] = v;
         }
     }
 }
@@ -463,6 +478,59 @@ int launch_mmq_reduce(const float *partial, const float *partial2, const float *
                   norm ? norm->eps : 0.f, 1.0f / (float)K);
 }
 
+
+// The reduction for a set of matrices contracted in one launch: partial[slice][m][ntot] holds their columns side by
+// side; matrix p's columns n0[p] .. go to its own y[p] ([M, N[p]]) with its own bias and activation.  Every N[p] % 4 == 0.
+struct MmqSetOut {
+    const float *bias[kMaxSet];
+    float *y[kMaxSet];
+    int N[kMaxSet], n0[kMaxSet], act[kMaxSet];
+    int count, ntot;
+};
+__global__ __launch_bounds__(256) void mmq_reduce_set_kernel(const float *__restrict__ partial, int nslices, int M, MmqSetOut out,
+                                                             const float *__restrict__ xscale, const float *__restrict__ xss, float eps,
+                                                             float inv_k) {
+    const int64_t total = (int64_t)M * out.ntot;
+    const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (i >= total) return;
+    const int m = (int)(i / out.ntot), nt = (int)(i - (int64_t)m * out.ntot);
+    int p = 0;
+#pragma unroll
+    for (int j = 1; j < kMaxSet; j++)
+        if (j < out.count && nt >= out.n0[j]) p = j;
+    const int n = nt - out.n0[p];
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    float ss = 0.f;
+    for (int k0 = 0; k0 < nslices; k0 += 8) {  // (all of a round's loads are issued before the first sum needs one)
+        float4 v[8];
+        float f[8], q[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int k = min(k0 + j, nslices - 1);
+            v[j] = *reinterpret_cast<const float4 *>(partial + (int64_t)k * total + i);
+            f[j] = xscale[(int64_t)k * M + m];
+            q[j] = xss ? xss[(int64_t)k * M + m] : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const bool in = k0 + j < nslices;
+            s.x = in ? fmaf(v[j].x, f[j], s.x) : s.x; s.y = in ? fmaf(v[j].y, f[j], s.y) : s.y;
+            s.z = in ? fmaf(v[j].z, f[j], s.z) : s.z; s.w = in ? fmaf(v[j].w, f[j], s.w) : s.w;
+            ss = in ? ss + q[j] : ss;
+        }
+    }
+    if (xss) {
+        const float r = sqrtf(ss * inv_k + eps);
+        s.x /= r; s.y /= r; s.z /= r; s.w /= r;
+    }
+    if (out.bias[p]) {
+        const float4 b = *reinterpret_cast<const float4 *>(out.bias[p] + n);
+        s.x += b.x; s.y += b.y; s.z += b.z; s.w += b.w;
+    }
+    const int act = out.act[p];
+    *reinterpret_cast<float4 *>(out.y[p] + (int64_t)m * out.N[p] + n) =
+        make_float4(apply_act(act, s.x), apply_act(act, s.y), apply_act(act, s.z), apply_act(act, s.w));
+}
 
 // ---- small batches of the 32-value-block formats (Q8_0, Q4_0, IQ4_NL) --------------------------------------
 //
@@ -986,15 +1054,11 @@ bool mmq_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, con
     return false;
 }
 
-int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias,
-               int act, float *y, hipStream_t s, const MmqExtra *ex) {
-    const uint8_t *W2 = ex ? ex->W2 : nullptr;
-    // (four row tiles per workgroup measured a little faster than two)
-    if (type == kQ8_0) return launch_mmq_b32<kQ8_0, 4>(x, x_is_bf16, M, K, W, N, bias, act, y, s, ex);
-    if (type == kQ4_0) return launch_mmq_b32<kQ4_0, 4>(x, x_is_bf16, M, K, W, N, bias, act, y, s, ex);
-    if (type == kIQ4_NL) return launch_mmq_b32<kIQ4_NL, 4>(x, x_is_bf16, M, K, W, N, bias, act, y, s, ex);
-    if (type == kQ6_K) return launch_mmq_q6k(ex, x, x_is_bf16, M, K, W, N, bias, act, y, s);
-    if (type != kQ4_K) return fail(GQ_ERR_NOT_IMPLEMENTED, "mmq: ggml type %d is not implemented", type);
+namespace {
+// `count` Q4_K matrices against one activation image: the pre-pass once, every matrix's row ranges in one launch of the
+// main kernel, one reduction.  A single matrix may carry the extras (gated pair, residual); a set carries a normalisation only.
+int run_q4k_set(const void *x, bool x_is_bf16, int64_t M, int64_t K, int count, const MmqSetItem *items, const MmqExtra *ex, hipStream_t s) {
+    const uint8_t *W2 = (ex && count == 1) ? ex->W2 : nullptr;
     typedef Q4KTile<kQ4KRowTiles> Tile;
     static const bool lds_ok = [] {
         return hipFuncSetAttribute(reinterpret_cast<const void *>(mmq_q4k_kernel<kQ4KRowTiles>), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -1002,7 +1066,18 @@ int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, co
     }();
     if (!lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", Tile::kLds);
     const int mtiles = (int)((M + kMT - 1) / kMT);
-    const int64_t rowwgs = (N + Tile::kRows - 1) / Tile::kRows, sbs = K / 256;
+    const int64_t sbs = K / 256;
+    Q4KSet set = {};
+    MmqSetOut out = {};
+    int64_t rowwgs = 0, N = 0;  // workgroups along the rows of all matrices; their columns side by side
+    for (int i = 0; i < count; i++) {
+        set.W[i] = items[i].W; set.N[i] = (int)items[i].N; set.wg0[i] = (int)rowwgs; set.n0[i] = (int)N;
+        out.bias[i] = items[i].bias; out.y[i] = items[i].y; out.N[i] = (int)items[i].N; out.n0[i] = (int)N; out.act[i] = items[i].act;
+        rowwgs += (items[i].N + Tile::kRows - 1) / Tile::kRows;
+        N += items[i].N;
+    }
+    set.count = out.count = count;
+    set.ntot = out.ntot = (int)N;
     // Super-blocks per K-slice (at most 7: the image shares LDS with the parked tiles): the count that needs the fewest
     // rounds of workgroups over the chip times the length of a round (+3: what a workgroup costs beyond its
     // super-blocks); ties go to the longer slice (fewer partial sums).
@@ -1041,11 +1116,46 @@ int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, co
     const dim3 grid((unsigned)rowwgs, (unsigned)nslices, W2 ? 2u : 1u);  // (both matrices of a gated pair in one launch)
     float *partial2 = W2 ? partial + (size_t)nslices * M * N : nullptr;
     for (int64_t m0 = 0; m0 < M; m0 += kMT) {
-        if (int rc = launch(mmq_q4k_kernel<kQ4KRowTiles>, grid, dim3(64 * Tile::kWaves), (size_t)Tile::kLds, s, (const uint8_t *)ximg, W, partial,
-                            (int)M, (int)K, (int)N, row_bytes, (int)m0, slice_sb, W2, partial2))
+        if (int rc = launch(mmq_q4k_kernel<kQ4KRowTiles>, grid, dim3(64 * Tile::kWaves), (size_t)Tile::kLds, s, (const uint8_t *)ximg, set, partial,
+                            (int)M, (int)K, row_bytes, (int)m0, slice_sb, W2, partial2))
             return rc;
     }
-    return launch_mmq_reduce(partial, partial2, xscale, nslices, M, K, N, bias, act, y, ex, s);
+    if (count == 1) return launch_mmq_reduce(partial, partial2, xscale, nslices, M, K, N, items[0].bias, items[0].act, items[0].y, ex, s);
+    const int64_t quads = M * N / 4;
+    const int threads = quads / 256 >= 2 * device_cu_count() ? 256 : 64;
+    return launch(mmq_reduce_set_kernel, dim3((unsigned)((quads + threads - 1) / threads)), dim3(threads), 0, s, (const float *)partial, nslices, (int)M,
+                  out, (const float *)xscale, (const float *)(norm && !x_is_bf16 ? mmq_xss(xscale, nslices, M) : nullptr), norm ? norm->eps : 0.f,
+                  1.0f / (float)K);
+}
+}  // namespace
+
+int launch_mmq(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias,
+               int act, float *y, hipStream_t s, const MmqExtra *ex) {
+    // (four row tiles per workgroup measured a little faster than two)
+    if (type == kQ8_0) return launch_mmq_b32<kQ8_0, 4>(x, x_is_bf16, M, K, W, N, bias, act, y, s, ex);
+    if (type == kQ4_0) return launch_mmq_b32<kQ4_0, 4>(x, x_is_bf16, M, K, W, N, bias, act, y, s, ex);
+    if (type == kIQ4_NL) return launch_mmq_b32<kIQ4_NL, 4>(x, x_is_bf16, M, K, W, N, bias, act, y, s, ex);
+    if (type == kQ6_K) return launch_mmq_q6k(ex, x, x_is_bf16, M, K, W, N, bias, act, y, s);
+    if (type != kQ4_K) return fail(GQ_ERR_NOT_IMPLEMENTED, "mmq: ggml type %d is not implemented", type);
+    const MmqSetItem one{W, N, bias, act, y};
+    return run_q4k_set(x, x_is_bf16, M, K, 1, &one, ex, s);
+}
+
+bool mmq_set_supported(int type, int count, const MmqSetItem *items, int64_t M, int64_t K, const void *x) {
+    if (type != kQ4_K || count < 2 || count > kMaxSet) return false;
+    int64_t total = 0;
+    for (int i = 0; i < count; i++) {
+        if (!mmq_supported(type, M, K, items[i].N, x, items[i].bias, items[i].y)) return false;
+        total += items[i].N;
+    }
+    return total <= (int64_t)INT32_MAX / 2;
+}
+
+int launch_mmq_set(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, int count, const MmqSetItem *items, const RmsNorm *norm,
+                   hipStream_t s) {
+    if (type != kQ4_K || count < 1 || count > kMaxSet) return fail(GQ_ERR_NOT_IMPLEMENTED, "mmq: a set of %d matrices of type %d is not implemented", count, type);
+    const MmqExtra ex{nullptr, nullptr, nullptr, norm};
+    return run_q4k_set(x, x_is_bf16, M, K, count, items, norm ? &ex : nullptr, s);
 }
 
 }  // namespace gq

@@ -911,6 +911,43 @@ def test_batched_projections_behind_one_norm(gpu, oracle, t):
             assert rel_err(y.cpu().numpy(), oracle.c_qdense(t, x, W, b)) < TOL_F32
 
 
+@pytest.mark.parametrize("rows,K", [(12, 2048), (32, 4096), (70, 2048), (33, 1536)])
+def test_projections_of_one_input_share_a_split_k_pass(gpu, oracle, rows, K):
+    """q / k / v beyond the GEMV's rows: three Q4_K projections of ONE device buffer of activations behind one normalisation
+    (one activation image, one main launch over all rows, one reduction), each with its own width, bias and activation; the
+    same list without the normalisation, and with distinct inputs, goes through separate calls."""
+    t = Q4_K
+    gain = (synth.normal(770, 0, K) * 0.5 + 1.0).astype(np.float32)
+    cfg = nn.RMSNorm(dev(gpu, gain), 1e-5, 0.0)
+    q = Quantization(ggml_type=t)
+    x = synth.activations(771, rows, K)
+    xd = dev(gpu, x)
+    Ws = [synth.weights(t, 772 + j, n, K) for j, n in enumerate((2048, 512, 260))]
+    bs = [None, synth.normal(775, 0, 512).astype(np.float32) * 0.1, synth.normal(776, 0, 260).astype(np.float32) * 0.1]
+    acts = [0, 3, 0]
+    outs = nn.quantized_dense_batch([(xd, dev(gpu, W), q, None if b is None else dev(gpu, b), BACKEND_ACT[a])
+                                     for W, b, a in zip(Ws, bs, acts)], norm=cfg)
+    gpu.cuda.synchronize()
+    xn = oracle.c_rmsnorm(x, gain, 1e-5, 0.0)
+    for W, b, a, y in zip(Ws, bs, acts, outs):
+        assert rel_err(y.cpu().numpy(), oracle.c_qdense(t, xn, W, b, a)) < TOL_F32, (rows, K, W.shape)
+    # two projections only, and a fourth
+    more = Ws + [synth.weights(t, 779, 128, K)]
+    for count in (2, 4):
+        outs = nn.quantized_dense_batch([(xd, dev(gpu, W), q, None, None) for W in more[:count]], norm=cfg)
+        gpu.cuda.synchronize()
+        for W, y in zip(more, outs):
+            assert rel_err(y.cpu().numpy(), oracle.c_qdense(t, xn, W, None)) < TOL_F32, (rows, K, count, W.shape)
+    # bf16 activations behind the normalisation: widened exactly, then the same pass
+    xb = bf16_round(x)
+    xbd = dev(gpu, xb).to(gpu.bfloat16)
+    outs = nn.quantized_dense_batch([(xbd, dev(gpu, W), q, None, None) for W in Ws], norm=cfg)
+    gpu.cuda.synchronize()
+    xbn = oracle.c_rmsnorm(xb, gain, 1e-5, 0.0)
+    for W, y in zip(Ws, outs):
+        assert rel_err(y.cpu().numpy(), oracle.c_qdense(t, xbn, W, None)) < TOL_F32, (rows, K, "bf16")
+
+
 @pytest.mark.parametrize("t", ALL_TYPES)
 def test_large_batches_with_neighbours_folded_into_the_two_passes(gpu, oracle, t):
     """From the batch sizes a plain dense call hands to the two-pass GEMM, the normalisation rides on
