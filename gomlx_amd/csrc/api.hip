@@ -620,9 +620,31 @@ int gq_qdense_norm_f32_batch(int count, const gq_dense_desc *descs, const gq_rms
     if (count == 0) return GQ_OK;
     if (int rc = use_device()) return rc;
     CallScope scope;
-    // one launch when every problem is a projection of one type, one K and one (small) batch size that the K-sliced GEMV takes
     const int64_t rows = descs[0].M;
-    bool merged = count >= 2 && count <= 8 && rows >= 1 && rows <= batch_rows_max();
+    // Projections of the same activations (q / k / v) can share one split-K pass - one activation image, one main launch
+    // over all their rows, one reduction - where the matrices taken together are in that kernel's range (three calls
+    // would convert the activations three times and pay nine launches).
+    MmqSetItem set[4];
+    bool shared_pass = count >= 2 && count <= 4 && (!norm->dGain || aligned_to(norm->dGain, 16));
+    {
+        int64_t ntot = 0;
+        for (int i = 0; i < count && shared_pass; i++) {
+            const gq_dense_desc &d = descs[i];
+            shared_pass = d.type == descs[0].type && d.dX == descs[0].dX && d.M == rows && d.K == descs[0].K && d.N > 0;
+            set[i] = MmqSetItem{(const uint8_t *)d.dW, d.N, d.dBias, d.act, d.dY};
+            ntot += d.N;
+        }
+        const int type = descs[0].type;
+        const int64_t K = descs[0].K;
+        shared_pass = shared_pass && mmq_set_supported(type, count, set, rows, K, descs[0].dX) &&
+                      rows >= block_split_k_from(type, weight_bytes_of(type, K, ntot), false) &&
+                      (rows <= split_k_to(type, K, ntot) || !gemm_two_pass_supported(type, false, rows, K, ntot, descs[0].dX));
+    }
+    // one launch when every problem is a projection of one type, one K and one (small) batch size that the K-sliced GEMV takes;
+    // from 6 rows the shared split-K pass is ahead (a decoder layer's q / k / v, 4096 -> 4096 + 2 x 1024, with the rest of the
+    // layer: 79.2 against 80.0 us at 5 rows, 81.6 against 79.9 at 6, 84.7 against 80.3 at 8)
+    constexpr int64_t kSharedPassFromRows = 6;
+    bool merged = count >= 2 && count <= 8 && rows >= 1 && rows <= batch_rows_max() && !(shared_pass && rows >= kSharedPassFromRows);
     XsBatchItem items[8];
     for (int i = 0; i < count && merged; i++) {
         const gq_dense_desc &d = descs[i];
@@ -634,27 +656,9 @@ int gq_qdense_norm_f32_batch(int count, const gq_dense_desc *descs, const gq_rms
         const RmsNorm rn{norm->dGain, norm->eps, norm->gain_offset};
         return launch_gemv_ks_batch_norm(descs[0].type, count, items, &rn, (hipStream_t)stream, (int)rows);
     }
-    // Beyond the GEMV's rows: projections of the same activations (q / k / v) share one split-K pass - one activation
-    // image, one main launch over all their rows, one reduction - where the matrices taken together are in that
-    // kernel's range (three calls would convert the activations three times and pay nine launches).
-    if (count >= 2 && count <= 4 && (!norm->dGain || aligned_to(norm->dGain, 16))) {
-        MmqSetItem set[4];
-        bool same = true;
-        int64_t ntot = 0;
-        for (int i = 0; i < count && same; i++) {
-            const gq_dense_desc &d = descs[i];
-            same = d.type == descs[0].type && d.dX == descs[0].dX && d.M == rows && d.K == descs[0].K && d.N > 0;
-            set[i] = MmqSetItem{(const uint8_t *)d.dW, d.N, d.dBias, d.act, d.dY};
-            ntot += d.N;
-        }
-        const int type = descs[0].type;
-        const int64_t K = descs[0].K;
-        if (same && mmq_set_supported(type, count, set, rows, K, descs[0].dX) &&
-            rows >= block_split_k_from(type, weight_bytes_of(type, K, ntot), false) &&
-            (rows <= split_k_to(type, K, ntot) || !gemm_two_pass_supported(type, false, rows, K, ntot, descs[0].dX))) {
-            const RmsNorm rn{norm->dGain, norm->eps, norm->gain_offset};
-            return launch_mmq_set(type, descs[0].dX, false, rows, K, count, set, &rn, (hipStream_t)stream);
-        }
+    if (shared_pass) {
+        const RmsNorm rn{norm->dGain, norm->eps, norm->gain_offset};
+        return launch_mmq_set(descs[0].type, descs[0].dX, false, rows, descs[0].K, count, set, &rn, (hipStream_t)stream);
     }
     for (int i = 0; i < count; i++) {
         const gq_dense_desc &d = descs[i];

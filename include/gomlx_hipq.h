@@ -171,7 +171,10 @@ int gq_qdense_block_f32(int type, const float *dX, int64_t M, int64_t K, const g
                         const float *dResidual, float *dY, void *stream);
 /* gq_qdense_f32_batch with one RMS normalisation applied to the activations of every problem:
  * the q/k/v projections behind a layer's input norm (transformer.go:1099-1130) in one launch
- * when all are problems of one type, one K and one batch size of at most 8 rows. */
+ * when all are problems of one type, one K and one batch size of at most 8 rows.  Two to four
+ * Q4_K projections of the SAME activation buffer (equal dX, M, K) with more rows than that share
+ * one split-K pass (activations converted once, one main launch, one reduction; uses the
+ * per-stream workspace); anything else runs as separate gq_qdense_block_f32 calls. */
 int gq_qdense_norm_f32_batch(int count, const gq_dense_desc *descs, const gq_rmsnorm *norm,
                              void *stream);
 /* The gated feed-forward front (transformer.go:1279-1287, after the pre_feedforward_norm of

@@ -911,7 +911,7 @@ def test_batched_projections_behind_one_norm(gpu, oracle, t):
             assert rel_err(y.cpu().numpy(), oracle.c_qdense(t, x, W, b)) < TOL_F32
 
 
-@pytest.mark.parametrize("rows,K", [(12, 2048), (32, 4096), (70, 2048), (33, 1536)])
+@pytest.mark.parametrize("rows,K", [(6, 2048), (8, 4096), (12, 2048), (32, 4096), (70, 2048), (33, 1536)])
 def test_projections_of_one_input_share_a_split_k_pass(gpu, oracle, rows, K):
     """q / k / v beyond the GEMV's rows: three Q4_K projections of ONE device buffer of activations behind one normalisation
     (one activation image, one main launch over all rows, one reduction), each with its own width, bias and activation; the
