@@ -422,6 +422,13 @@ int gq_qdense_f32_static(int type, const float *dX, int64_t M, int64_t K, const 
     return gq_qdense_f32(type, dX, M, K, dW, N, dBias, act, dY, stream);
 }
 
+namespace {
+bool takes_shared_pass(int count, const gq_dense_desc *descs, const float *gain, MmqSetItem *set);  // (defined with the dispatch thresholds below)
+// From 6 rows the shared split-K pass is ahead of the merged GEMV launch: a decoder layer's q / k / v, 4096 -> 4096 + 2 x 1024,
+// with the rest of the layer: 79.2 against 80.0 us at 5 rows, 81.6 against 79.9 at 6, 84.7 against 80.3 at 8.
+constexpr int64_t kSharedPassFromRows = 6;
+}  // namespace
+
 int gq_qdense_f32_batch(int count, const gq_dense_desc *descs, void *stream) {
     if (count < 0 || (count > 0 && !descs)) return fail(GQ_ERR_INVALID, "gq_qdense_f32_batch: bad descriptor list");
     for (int i = 0; i < count; i++) {
@@ -431,6 +438,11 @@ int gq_qdense_f32_batch(int count, const gq_dense_desc *descs, void *stream) {
     if (count == 0) return GQ_OK;
     if (int rc = use_device()) return rc;
     CallScope scope;
+    {   // projections of one input beyond the GEMV's best rows: one split-K pass for all of them
+        MmqSetItem set[4];
+        if (descs[0].M >= kSharedPassFromRows && takes_shared_pass(count, descs, nullptr, set))
+            return launch_mmq_set(descs[0].type, descs[0].dX, false, descs[0].M, descs[0].K, count, set, nullptr, (hipStream_t)stream);
+    }
     // merge runs of batch-1 problems of one type that the streaming GEMV handles; the rest go one by one
     int i = 0;
     while (i < count) {
@@ -552,6 +564,23 @@ bool block_takes_two_pass(int type, int64_t M, int64_t K, int64_t N, const float
     const bool sk = M >= split_k_from(type, weight_bytes_of(type, K, N)) && mmq_supported(type, M, K, N, x, bias, y) && M <= split_k_to(type, K, N);
     return !sk;
 }
+// Whether a list of projections is one input contracted with two to four matrices that the shared split-K pass takes
+// (launch_mmq_set): equal type, activations, rows and K, the matrices taken together in the split-K kernels' range.
+bool takes_shared_pass(int count, const gq_dense_desc *descs, const float *gain, MmqSetItem *set) {
+    if (count < 2 || count > 4 || (gain && !aligned_to(gain, 16))) return false;
+    const int type = descs[0].type;
+    const int64_t rows = descs[0].M, K = descs[0].K;
+    int64_t ntot = 0;
+    for (int i = 0; i < count; i++) {
+        const gq_dense_desc &d = descs[i];
+        if (d.type != type || d.dX != descs[0].dX || d.M != rows || d.K != K || d.N <= 0) return false;
+        set[i] = MmqSetItem{(const uint8_t *)d.dW, d.N, d.dBias, d.act, d.dY};
+        ntot += d.N;
+    }
+    return mmq_set_supported(type, count, set, rows, K, descs[0].dX) &&
+           rows >= block_split_k_from(type, weight_bytes_of(type, K, ntot), false) &&
+           (rows <= split_k_to(type, K, ntot) || !gemm_two_pass_supported(type, false, rows, K, ntot, descs[0].dX));
+}
 }  // namespace
 
 int gq_qdense_block_f32(int type, const float *dX, int64_t M, int64_t K, const gq_rmsnorm *norm, const void *dW, int64_t N,
@@ -625,25 +654,8 @@ int gq_qdense_norm_f32_batch(int count, const gq_dense_desc *descs, const gq_rms
     // over all their rows, one reduction - where the matrices taken together are in that kernel's range (three calls
     // would convert the activations three times and pay nine launches).
     MmqSetItem set[4];
-    bool shared_pass = count >= 2 && count <= 4 && (!norm->dGain || aligned_to(norm->dGain, 16));
-    {
-        int64_t ntot = 0;
-        for (int i = 0; i < count && shared_pass; i++) {
-            const gq_dense_desc &d = descs[i];
-            shared_pass = d.type == descs[0].type && d.dX == descs[0].dX && d.M == rows && d.K == descs[0].K && d.N > 0;
-            set[i] = MmqSetItem{(const uint8_t *)d.dW, d.N, d.dBias, d.act, d.dY};
-            ntot += d.N;
-        }
-        const int type = descs[0].type;
-        const int64_t K = descs[0].K;
-        shared_pass = shared_pass && mmq_set_supported(type, count, set, rows, K, descs[0].dX) &&
-                      rows >= block_split_k_from(type, weight_bytes_of(type, K, ntot), false) &&
-                      (rows <= split_k_to(type, K, ntot) || !gemm_two_pass_supported(type, false, rows, K, ntot, descs[0].dX));
-    }
-    // one launch when every problem is a projection of one type, one K and one (small) batch size that the K-sliced GEMV takes;
-    // from 6 rows the shared split-K pass is ahead (a decoder layer's q / k / v, 4096 -> 4096 + 2 x 1024, with the rest of the
-    // layer: 79.2 against 80.0 us at 5 rows, 81.6 against 79.9 at 6, 84.7 against 80.3 at 8)
-    constexpr int64_t kSharedPassFromRows = 6;
+    const bool shared_pass = takes_shared_pass(count, descs, norm->dGain, set);
+    // one launch when every problem is a projection of one type, one K and one (small) batch size that the K-sliced GEMV takes
     bool merged = count >= 2 && count <= 8 && rows >= 1 && rows <= batch_rows_max() && !(shared_pass && rows >= kSharedPassFromRows);
     XsBatchItem items[8];
     for (int i = 0; i < count && merged; i++) {

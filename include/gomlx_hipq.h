@@ -129,7 +129,8 @@ int gq_qdense_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, const voi
  * (e.g. the q/k/v or gate/up projections of a decoder layer) submitted together: the work an
  * Executable.Execute (core/graph/graph.go:669) is free to overlap.  Equivalent to calling
  * gq_qdense_f32 once per descriptor, in any order; outputs must not alias any input.  Batch-1
- * problems of one GGML type are merged into a single launch. ---- */
+ * problems of one GGML type are merged into a single launch; two to four Q4_K projections of the
+ * same activation buffer with 6 rows or more share one split-K pass (activations converted once). ---- */
 typedef struct {
     int type;            /* gq_type */
     int act;             /* gq_act */

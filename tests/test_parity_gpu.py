@@ -938,6 +938,12 @@ def test_projections_of_one_input_share_a_split_k_pass(gpu, oracle, rows, K):
         gpu.cuda.synchronize()
         for W, y in zip(more, outs):
             assert rel_err(y.cpu().numpy(), oracle.c_qdense(t, xn, W, None)) < TOL_F32, (rows, K, count, W.shape)
+    # the same list without a normalisation (gq_qdense_f32_batch)
+    outs = nn.quantized_dense_batch([(xd, dev(gpu, W), q, None if b is None else dev(gpu, b), BACKEND_ACT[a])
+                                     for W, b, a in zip(Ws, bs, acts)])
+    gpu.cuda.synchronize()
+    for W, b, a, y in zip(Ws, bs, acts, outs):
+        assert rel_err(y.cpu().numpy(), oracle.c_qdense(t, x, W, b, a)) < TOL_F32, (rows, K, W.shape, "no norm")
     # bf16 activations behind the normalisation: widened exactly, then the same pass
     xb = bf16_round(x)
     xbd = dev(gpu, xb).to(gpu.bfloat16)
