@@ -954,6 +954,34 @@ def test_projections_of_one_input_share_a_split_k_pass(gpu, oracle, rows, K):
         assert rel_err(y.cpu().numpy(), oracle.c_qdense(t, xbn, W, None)) < TOL_F32, (rows, K, "bf16")
 
 
+def test_shared_split_k_pass_randomized(gpu, oracle):
+    """Seeded random lists of two to four Q4_K projections of one input, 6 to 99 rows, any widths that are multiples of 4
+    (most not multiples of the 128-row workgroup), with and without normalisation, gain, bias; activations without tanh
+    (saturated outputs measure nothing of the contraction)."""
+    rng = np.random.default_rng(4242)
+    q = Quantization(ggml_type=Q4_K)
+    for case in range(16):
+        rows, K, count = int(rng.integers(6, 100)), 256 * int(rng.integers(1, 17)), int(rng.integers(2, 5))
+        Ns = [4 * int(rng.integers(1, 400)) for _ in range(count)]
+        use_norm, use_gain = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        x = (synth.activations(7000 + case, rows, K) * float(10.0 ** rng.uniform(-3, 3))).astype(np.float32)
+        gain = (synth.normal(7100 + case, 0, K) * 0.5 + 1.0).astype(np.float32)
+        cfg = nn.RMSNorm(dev(gpu, gain) if use_gain else None, 1e-5, 0.0) if use_norm else None
+        xin = oracle.c_rmsnorm(x, gain if use_gain else None, 1e-5, 0.0) if use_norm else x
+        xd = dev(gpu, x)
+        probs, wants = [], []
+        for j, N in enumerate(Ns):
+            W = synth.weights(Q4_K, 7200 + 10 * case + j, N, K)
+            b = synth.normal(7300 + 10 * case + j, 0, N).astype(np.float32) * 0.1 if rng.integers(0, 2) else None
+            a = int(rng.integers(0, 5))
+            probs.append((xd, dev(gpu, W), q, None if b is None else dev(gpu, b), BACKEND_ACT[a]))
+            wants.append(oracle.c_qdense(Q4_K, xin, W, b, a))
+        outs = nn.quantized_dense_batch(probs, norm=cfg)
+        gpu.cuda.synchronize()
+        for y, want in zip(outs, wants):
+            assert rel_err(y.cpu().numpy(), want) < TOL_F32, (case, rows, K, Ns, use_norm, use_gain)
+
+
 @pytest.mark.parametrize("t", ALL_TYPES)
 def test_large_batches_with_neighbours_folded_into_the_two_passes(gpu, oracle, t):
     """From the batch sizes a plain dense call hands to the two-pass GEMM, the normalisation rides on
