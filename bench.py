@@ -200,7 +200,8 @@ class Yardstick:
         self.lib.gqy_mfma.restype = ctypes.c_int
 
     # (workgroups, threads, loads in flight per thread): the shapes that read fastest on this chip at 18 .. 123 MB
-    SHAPES = ((2048, 256, 2), (1024, 256, 4), (512, 256, 8), (256, 512, 8))
+    # (depth 100 + d: the same d loads in flight, issued as non-temporal loads)
+    SHAPES = ((2048, 256, 2), (1024, 256, 4), (512, 256, 8), (256, 512, 8), (1024, 256, 104), (512, 256, 108))
 
     def time_buffers(self, torch, bufs, stream, tstream, steps):
         """Best mean time (us) per launch over SHAPES: one recorded graph of `steps` launches rotating over `bufs`."""
@@ -436,7 +437,7 @@ class Problem:
             bufs.append(parts[0] if len(parts) == 1 else torch.cat(parts))
         us, wgs, threads, depth = ys.time_buffers(torch, bufs, self.stream, self.tstream, max(10, min(steps, 50)))
         return {"us": us, "gbps": self.weight_bytes / us / 1e3, "frac_of_peak": self.weight_bytes / us / 1e3 / HBM_PEAK_GBS,
-                "grid": f"{wgs} workgroups x {threads} threads, {depth} 16-byte loads in flight per thread",
+                "grid": f"{wgs} workgroups x {threads} threads, {depth % 100} {'non-temporal ' if depth >= 100 else ''}16-byte loads in flight per thread",
                 "note": "read-only kernel over the same cold bytes, no arithmetic: what a one-shot kernel of this size can reach"}
 
     def clock_state(self):

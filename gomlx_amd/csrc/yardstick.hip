@@ -23,7 +23,8 @@
 
 namespace {
 
-template <int DEPTH>
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+template <int DEPTH, bool NT = false>
 __global__ __launch_bounds__(1024) void read_linear_kernel(const uint4 *__restrict__ p, size_t chunks, uint32_t *__restrict__ out) {
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -31,7 +32,12 @@ __global__ __launch_bounds__(1024) void read_linear_kernel(const uint4 *__restri
     for (; i + (DEPTH - 1) * stride < chunks; i += DEPTH * stride) {
         uint4 v[DEPTH];
 #pragma unroll
-        for (int j = 0; j < DEPTH; j++) v[j] = p[i + j * stride];
+        for (int j = 0; j < DEPTH; j++) {
+            if constexpr (NT) {  // non-temporal: the line is not kept in the caches behind the load
+                const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p + i + j * stride));
+                v[j] = make_uint4(t.x, t.y, t.z, t.w);
+            } else v[j] = p[i + j * stride];
+        }
 #pragma unroll
         for (int j = 0; j < DEPTH; j++) acc ^= v[j].x ^ v[j].y ^ v[j].z ^ v[j].w;
     }
@@ -139,6 +145,14 @@ int gqy_read(const void *p, size_t bytes, int pattern, int wgs, int threads, int
         const size_t chunks = bytes / 16;
         const uint4 *q = static_cast<const uint4 *>(p);
         uint32_t *o = static_cast<uint32_t *>(out);
+        if (pattern == 0 && depth >= 100) {  // depth 102 / 104 / 108: non-temporal loads, 2 / 4 / 8 in flight
+            switch (depth - 100) {
+            case 2: hipLaunchKernelGGL((read_linear_kernel<2, true>), dim3(wgs), dim3(threads), 0, s, q, chunks, o); break;
+            case 4: hipLaunchKernelGGL((read_linear_kernel<4, true>), dim3(wgs), dim3(threads), 0, s, q, chunks, o); break;
+            default: hipLaunchKernelGGL((read_linear_kernel<8, true>), dim3(wgs), dim3(threads), 0, s, q, chunks, o); break;
+            }
+            return (int)hipGetLastError();
+        }
         switch (depth) {
         case 1: hipLaunchKernelGGL(read_linear_kernel<1>, dim3(wgs), dim3(threads), 0, s, q, chunks, o); break;
         case 2: hipLaunchKernelGGL(read_linear_kernel<2>, dim3(wgs), dim3(threads), 0, s, q, chunks, o); break;
