@@ -596,7 +596,7 @@ int gq_qdense_block_f32(int type, const float *dX, int64_t M, int64_t K, const g
     RmsNorm rn{nullptr, 0.f, 0.f};
     if (norm) rn = RmsNorm{norm->dGain, norm->eps, norm->gain_offset};
     if (fold_into_gemv(type, M, K, N, dX, rn.gain, dBias, dY, false))
-        return launch_gemv_ks_ext(type, dX, M, K, norm ? &rn : nullptr, (const uint8_t *)dW, dBias, nullptr, nullptr, dResidual, N, act, dY,
+        return launch_gemv_ks_ext(type, dX, false, M, K, norm ? &rn : nullptr, (const uint8_t *)dW, dBias, nullptr, nullptr, dResidual, N, act, dY,
                                   (hipStream_t)stream);
     if (block_takes_two_pass(type, M, K, N, dX, rn.gain, dBias, dY, false)) {
         void *ws = nullptr;
@@ -638,6 +638,23 @@ int gq_qdense_block_f32(int type, const float *dX, int64_t M, int64_t K, const g
     return GQ_OK;
 }
 
+namespace {
+// Whether a list of projections behind one normalisation is one launch of the K-sliced GEMV: every problem a projection of one
+// type, one K and one (small) batch size that kernel takes (dX may point at fp32 or bf16 data: only its alignment matters),
+// unless the shared split-K pass takes them at that batch size.  Fills items[0 .. count).
+bool merges_into_gemv(int count, const gq_dense_desc *descs, const gq_rmsnorm *norm, bool shared_pass, XsBatchItem *items) {
+    const int64_t rows = descs[0].M;
+    bool merged = count >= 2 && count <= 8 && rows >= 1 && rows <= batch_rows_max() && !(shared_pass && rows >= kSharedPassFromRows);
+    for (int i = 0; i < count && merged; i++) {
+        const gq_dense_desc &d = descs[i];
+        merged = d.type == descs[0].type && d.K == descs[0].K && d.M == rows && d.N > 0 && gemv_ks_ext_supported(d.type, rows, d.K, d.N, d.dX, norm->dGain) &&
+                 (rows == 1 || weight_bytes_of(d.type, d.K, d.N) < kLargeWeightBytes);
+        if (merged) items[i] = XsBatchItem{d.dX, (const uint8_t *)d.dW, d.dBias, d.dY, d.K, d.N, d.act};
+    }
+    return merged;
+}
+}  // namespace
+
 int gq_qdense_norm_f32_batch(int count, const gq_dense_desc *descs, const gq_rmsnorm *norm, void *stream) {
     if (!norm) return gq_qdense_f32_batch(count, descs, stream);
     if (count < 0 || (count > 0 && !descs)) return fail(GQ_ERR_INVALID, "gq_qdense_norm_f32_batch: bad descriptor list");
@@ -655,16 +672,8 @@ int gq_qdense_norm_f32_batch(int count, const gq_dense_desc *descs, const gq_rms
     // would convert the activations three times and pay nine launches).
     MmqSetItem set[4];
     const bool shared_pass = takes_shared_pass(count, descs, norm->dGain, set);
-    // one launch when every problem is a projection of one type, one K and one (small) batch size that the K-sliced GEMV takes
-    bool merged = count >= 2 && count <= 8 && rows >= 1 && rows <= batch_rows_max() && !(shared_pass && rows >= kSharedPassFromRows);
     XsBatchItem items[8];
-    for (int i = 0; i < count && merged; i++) {
-        const gq_dense_desc &d = descs[i];
-        merged = d.type == descs[0].type && d.K == descs[0].K && d.M == rows && d.N > 0 && gemv_ks_ext_supported(d.type, rows, d.K, d.N, d.dX, norm->dGain) &&
-                 (rows == 1 || weight_bytes_of(d.type, d.K, d.N) < kLargeWeightBytes);
-        if (merged) items[i] = XsBatchItem{d.dX, (const uint8_t *)d.dW, d.dBias, d.dY, d.K, d.N, d.act};
-    }
-    if (merged) {
+    if (merges_into_gemv(count, descs, norm, shared_pass, items)) {
         const RmsNorm rn{norm->dGain, norm->eps, norm->gain_offset};
         return launch_gemv_ks_batch_norm(descs[0].type, count, items, &rn, (hipStream_t)stream, (int)rows);
     }
@@ -691,7 +700,7 @@ int gq_qdense_gated_f32(int type, const float *dX, int64_t M, int64_t K, const g
     RmsNorm rn{nullptr, 0.f, 0.f};
     if (norm) rn = RmsNorm{norm->dGain, norm->eps, norm->gain_offset};
     if (fold_into_gemv(type, M, K, N, dX, rn.gain, dBiasGate, dY, true))
-        return launch_gemv_ks_ext(type, dX, M, K, norm ? &rn : nullptr, (const uint8_t *)dWgate, dBiasGate, (const uint8_t *)dWup, dBiasUp,
+        return launch_gemv_ks_ext(type, dX, false, M, K, norm ? &rn : nullptr, (const uint8_t *)dWgate, dBiasGate, (const uint8_t *)dWup, dBiasUp,
                                   nullptr, N, act, dY, (hipStream_t)stream);
     if (block_takes_two_pass(type, M, K, N, dX, rn.gain, dBiasGate, dY, true)) {
         void *ws = nullptr;
@@ -725,7 +734,8 @@ int gq_qdense_gated_f32(int type, const float *dX, int64_t M, int64_t K, const g
     return launch_mul_inplace(dY, gate, M * N, (hipStream_t)stream);
 }
 
-// ---- the same callers with bf16 activations: widened exactly to fp32 in the stream's third workspace, then the fp32 routes ----
+// ---- the same callers with bf16 activations: the decode GEMV reads them as they are (widened in registers: exact); the other
+// routes get them widened to fp32 in the stream's third workspace ----
 namespace {
 // fp32 copy of a bf16 [M, K] matrix at `offset` bytes into the widening workspace, whose size the caller has fixed
 int widen_into(void *ws, size_t offset, const uint16_t *x, int64_t M, int64_t K, hipStream_t s, const float **out) {
@@ -741,9 +751,26 @@ int gq_qdense_block_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, con
                          const float *dBias, int act, const float *dResidual, float *dY, void *stream) {
     if (!norm && !dResidual) return gq_qdense_bf16(type, dX, M, K, dW, N, dBias, act, dY, stream);
     if (int rc = check_dense_args("gq_qdense_block_bf16", type, dX, M, K, dW, N, dBias, act, dY, 16)) return rc;
+    if (norm && !(norm->eps >= 0.f)) return fail(GQ_ERR_INVALID, "gq_qdense_block_bf16: epsilon must be >= 0");
+    if (norm && norm->dGain && !aligned_to(norm->dGain, 4)) return fail(GQ_ERR_INVALID, "gq_qdense_block_bf16: gain must be 4-byte aligned");
+    if (dResidual && !aligned_to(dResidual, 4)) return fail(GQ_ERR_INVALID, "gq_qdense_block_bf16: residual must be 4-byte aligned");
     if (M == 0 || N == 0) return GQ_OK;
     if (int rc = use_device()) return rc;
     CallScope scope;
+    if (fold_into_gemv(type, M, K, N, reinterpret_cast<const float *>(dX), norm ? norm->dGain : nullptr, dBias, dY, false)) {
+        const RmsNorm rn = norm ? RmsNorm{norm->dGain, norm->eps, norm->gain_offset} : RmsNorm{nullptr, 0.f, 0.f};
+        return launch_gemv_ks_ext(type, dX, true, M, K, norm ? &rn : nullptr, (const uint8_t *)dW, dBias, nullptr, nullptr, dResidual, N, act, dY,
+                                  (hipStream_t)stream);
+    }
+    {   // the split-K kernels' pre-pass reads bf16 as well (where the fp32 call would take them too)
+        const float *xa = reinterpret_cast<const float *>(dX), *gain = norm ? norm->dGain : nullptr;  // (only their alignment is looked at)
+        if (!block_takes_two_pass(type, M, K, N, xa, gain, dBias, dY, false) && block_takes_split_k(type, M, K, N, xa, dBias, dY, false) &&
+            (!dResidual || aligned_to(dResidual, 16)) && (!gain || aligned_to(gain, 16))) {
+            const RmsNorm rn = norm ? RmsNorm{norm->dGain, norm->eps, norm->gain_offset} : RmsNorm{nullptr, 0.f, 0.f};
+            const MmqExtra ex{nullptr, nullptr, dResidual, norm ? &rn : nullptr};
+            return launch_mmq(type, dX, true, M, K, (const uint8_t *)dW, N, dBias, act, dY, (hipStream_t)stream, &ex);
+        }
+    }
     void *ws = nullptr;
     if (int rc = stream_workspace((hipStream_t)stream, widened_bytes(M, K), &ws, kWsWidenSlot)) return rc;
     const float *x32 = nullptr;
@@ -754,9 +781,26 @@ int gq_qdense_block_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, con
 int gq_qdense_gated_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, const gq_rmsnorm *norm, const void *dWgate,
                          const float *dBiasGate, const void *dWup, const float *dBiasUp, int64_t N, int act, float *dY, void *stream) {
     if (int rc = check_dense_args("gq_qdense_gated_bf16", type, dX, M, K, dWgate, N, dBiasGate, act, dY, 16)) return rc;
+    if (int rc = check_dense_args("gq_qdense_gated_bf16", type, dX, M, K, dWup, N, dBiasUp, act, dY, 16)) return rc;
+    if (norm && !(norm->eps >= 0.f)) return fail(GQ_ERR_INVALID, "gq_qdense_gated_bf16: epsilon must be >= 0");
+    if (norm && norm->dGain && !aligned_to(norm->dGain, 4)) return fail(GQ_ERR_INVALID, "gq_qdense_gated_bf16: gain must be 4-byte aligned");
     if (M == 0 || N == 0) return GQ_OK;
     if (int rc = use_device()) return rc;
     CallScope scope;
+    if (fold_into_gemv(type, M, K, N, reinterpret_cast<const float *>(dX), norm ? norm->dGain : nullptr, dBiasGate, dY, true)) {
+        const RmsNorm rn = norm ? RmsNorm{norm->dGain, norm->eps, norm->gain_offset} : RmsNorm{nullptr, 0.f, 0.f};
+        return launch_gemv_ks_ext(type, dX, true, M, K, norm ? &rn : nullptr, (const uint8_t *)dWgate, dBiasGate, (const uint8_t *)dWup, dBiasUp, nullptr,
+                                  N, act, dY, (hipStream_t)stream);
+    }
+    {
+        const float *xa = reinterpret_cast<const float *>(dX), *gain = norm ? norm->dGain : nullptr;  // (only their alignment is looked at)
+        if (!block_takes_two_pass(type, M, K, N, xa, gain, dBiasGate, dY, true) && block_takes_split_k(type, M, K, N, xa, dBiasGate, dY, true) &&
+            (!dBiasUp || aligned_to(dBiasUp, 16)) && (!gain || aligned_to(gain, 16))) {
+            const RmsNorm rn = norm ? RmsNorm{norm->dGain, norm->eps, norm->gain_offset} : RmsNorm{nullptr, 0.f, 0.f};
+            const MmqExtra ex{(const uint8_t *)dWup, dBiasUp, nullptr, norm ? &rn : nullptr};
+            return launch_mmq(type, dX, true, M, K, (const uint8_t *)dWgate, N, dBiasGate, act, dY, (hipStream_t)stream, &ex);
+        }
+    }
     void *ws = nullptr;
     if (int rc = stream_workspace((hipStream_t)stream, widened_bytes(M, K), &ws, kWsWidenSlot)) return rc;
     const float *x32 = nullptr;
@@ -771,9 +815,23 @@ int gq_qdense_norm_bf16_batch(int count, const gq_dense_desc *descs, const gq_rm
         const gq_dense_desc &d = descs[i];
         if (int rc = check_dense_args("gq_qdense_norm_bf16_batch", d.type, d.dX, d.M, d.K, d.dW, d.N, d.dBias, d.act, d.dY, 16)) return rc;
     }
+    if (norm && !(norm->eps >= 0.f)) return fail(GQ_ERR_INVALID, "gq_qdense_norm_bf16_batch: epsilon must be >= 0");
     if (count == 0) return GQ_OK;
     if (int rc = use_device()) return rc;
     CallScope scope;
+    if (norm && count <= 8) {  // the list as one launch of the decode GEMV, on the bf16 data as it is
+        MmqSetItem set[4];
+        const bool shared_pass = takes_shared_pass(count, descs, norm->dGain, set);
+        XsBatchItem items[8];
+        if (merges_into_gemv(count, descs, norm, shared_pass, items)) {
+            const RmsNorm rn{norm->dGain, norm->eps, norm->gain_offset};
+            return launch_gemv_ks_batch_norm(descs[0].type, count, items, &rn, (hipStream_t)stream, (int)descs[0].M, true);
+        }
+        if (shared_pass) {
+            const RmsNorm rn{norm->dGain, norm->eps, norm->gain_offset};
+            return launch_mmq_set(descs[0].type, descs[0].dX, true, descs[0].M, descs[0].K, count, set, &rn, (hipStream_t)stream);
+        }
+    }
     // every distinct activation matrix (q / k / v share theirs) is widened once
     gq_dense_desc wide[64];
     size_t offset[64], total = 0;

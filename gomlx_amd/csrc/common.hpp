@@ -93,9 +93,9 @@ bool mmq_set_supported(int type, int count, const MmqSetItem *items, int64_t M, 
 int launch_mmq_set(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, int count, const MmqSetItem *items, const RmsNorm *norm,
                    hipStream_t s);
 // The K-sliced GEMV with the normalisation folded in and, when W2 is given, the gated product
-// act(x.W + bias) * (x.W2 + bias2); fp32 activations, at most 16 rows (the entry points use it below 8 rows, where a pass per row still wins).
+// act(x.W + bias) * (x.W2 + bias2); fp32 or bf16 activations, at most 16 rows (the entry points use it below 8 rows, where a pass per row still wins).
 bool gemv_ks_ext_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, const void *gain);
-int launch_gemv_ks_ext(int type, const float *x, int64_t M, int64_t K, const RmsNorm *norm, const uint8_t *W, const float *bias,
+int launch_gemv_ks_ext(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, const RmsNorm *norm, const uint8_t *W, const float *bias,
                        const uint8_t *W2, const float *bias2, const float *residual, int64_t N, int act, float *y, hipStream_t s);
 int launch_add(const float *a, const float *r, float *y, int64_t n, hipStream_t s);
 int launch_rmsnorm(const float *x, int64_t M, int64_t K, const float *gain, float gain_offset, float eps, float *y, hipStream_t s);
@@ -106,7 +106,7 @@ int launch_gemv_xs_batch(int type, int count, const XsBatchItem *items, hipStrea
 // (K-sliced: `rows` activation rows per problem, the same count for all: x and y are [rows, K] and [rows, N])
 int launch_gemv_ks_batch(int type, int count, const XsBatchItem *items, hipStream_t s, int rows = 1);
 // the same with one RMS normalisation applied to every problem's activations (all of one K)
-int launch_gemv_ks_batch_norm(int type, int count, const XsBatchItem *items, const RmsNorm *norm, hipStream_t s, int rows = 1);
+int launch_gemv_ks_batch_norm(int type, int count, const XsBatchItem *items, const RmsNorm *norm, hipStream_t s, int rows = 1, bool x_is_bf16 = false);
 // Large batches: dequantise W once into a 16-bit image (in `workspace`, gemm_two_pass_workspace()
 // bytes), then a plain 16-bit MFMA GEMM.
 bool gemm_two_pass_supported(int type, bool x_is_bf16, int64_t M, int64_t K, int64_t N, const void *x);

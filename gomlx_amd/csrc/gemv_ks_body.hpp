@@ -499,7 +499,10 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8
             if constexpr (XBF16) r.a[i] = KS<T>::x_fetch_bf16(reinterpret_cast<const uint16_t *>(xrow) + sl * kSliceValues, xl);
             else KS<T>::x_fetch(reinterpret_cast<const float *>(xrow) + sl * kSliceValues, xl, r.a[i], r.b[i]);
         }
-        if constexpr (EXT) KS<T>::x_fetch(gsrc + sl * kSliceValues, xl, r.ga, r.gb);
+        if constexpr (EXT) {
+            // (bf16 activations are half as long as the gain: they cannot stand in for it)
+            if (!XBF16 || ext.gain) KS<T>::x_fetch(gsrc + sl * kSliceValues, xl, r.ga, r.gb);
+        }
         return r;
     };
     auto as_f4 = [](const uint4 &u) {

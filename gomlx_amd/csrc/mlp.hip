@@ -12,8 +12,9 @@ namespace gq {
 
 namespace {
 
-template <int T, int PF, int WIN, int R>
-__global__ __launch_bounds__(512) void gemv_ks_ext_kernel(const float *__restrict__ X, const uint8_t *__restrict__ W,
+// X: fp32, or bf16 with XBF16 (widened while a slice is converted: exact)
+template <int T, int PF, int WIN, int R, bool XBF16>
+__global__ __launch_bounds__(512) void gemv_ks_ext_kernel(const void *__restrict__ X, const uint8_t *__restrict__ W,
                                                           const float *__restrict__ bias, float *__restrict__ Y, int M, int K, int N,
                                                           int64_t row_bytes, int iters, int nslices, int half_tail, int act,
                                                           const KsExt ext) {
@@ -21,53 +22,59 @@ __global__ __launch_bounds__(512) void gemv_ks_ext_kernel(const float *__restric
     const int r0 = (int)blockIdx.y * R;
     KsExt e = ext;
     if (e.residual) e.residual += (int64_t)r0 * N;
-    ks_body<T, PF, WIN, true, false, R>(X + (int64_t)r0 * K, W, bias, Y + (int64_t)r0 * N, N, row_bytes, iters, nslices, half_tail, act,
-                                        (int)(blockDim.x >> 6), (int)blockIdx.x, lds, &e, min(R, M - r0), (int64_t)K * 4);
+    const int64_t x_stride = (int64_t)K * (XBF16 ? 2 : 4);
+    ks_body<T, PF, WIN, true, XBF16, R>(reinterpret_cast<const uint8_t *>(X) + r0 * x_stride, W, bias, Y + (int64_t)r0 * N, N, row_bytes, iters, nslices,
+                                        half_tail, act, (int)(blockDim.x >> 6), (int)blockIdx.x, lds, &e, min(R, M - r0), x_stride);
 }
 
 // Batched submission (several batch-1 projections of one format in one launch) with one RMS
 // normalisation shared by all of them: the q/k/v projections behind a layer's input norm.
-template <int T>
+template <int T, bool XBF16>
 __global__ __launch_bounds__(512) void gemv_ks_batch_ext_kernel(const KsBatch b, const KsExt ext) {
     extern __shared__ uint32_t lds[];
     const KsProblem &q = b.p[ks_batch_problem(b, (int)blockIdx.x)];
     const int64_t row = blockIdx.y;  // activation row of every problem
-    ks_body<T, kBatchPF, kBatchPF, true>(q.x + row * q.K, q.W, q.bias, q.y + row * q.N, q.N, q.row_bytes, q.iters, q.nslices, q.half_tail, q.act, q.waves,
-                                         (int)blockIdx.x - q.wg_begin, lds, &ext);
+    const uint8_t *x = reinterpret_cast<const uint8_t *>(q.x) + row * q.K * (XBF16 ? 2 : 4);  // (q.x points at bf16 data with XBF16)
+    ks_body<T, kBatchPF, kBatchPF, true, XBF16>(x, q.W, q.bias, q.y + row * q.N, q.N, q.row_bytes, q.iters, q.nslices, q.half_tail, q.act, q.waves,
+                                                (int)blockIdx.x - q.wg_begin, lds, &ext);
 }
 
 template <int T>
-int launch_batch_ext(int count, const XsBatchItem *items, const KsExt &ext, int rows, hipStream_t s) {
+int launch_batch_ext(int count, const XsBatchItem *items, const KsExt &ext, int rows, bool x_is_bf16, hipStream_t s) {
     KsBatch b;
     size_t shmem;
     int wgs;
     if (int rc = plan_ks_batch<T>(count, items, b, shmem, wgs)) return rc;
-    return launch(gemv_ks_batch_ext_kernel<T>, dim3((unsigned)wgs, (unsigned)rows), dim3(512), shmem, s, b, ext);
+    if (x_is_bf16) return launch(gemv_ks_batch_ext_kernel<T, true>, dim3((unsigned)wgs, (unsigned)rows), dim3(512), shmem, s, b, ext);
+    return launch(gemv_ks_batch_ext_kernel<T, false>, dim3((unsigned)wgs, (unsigned)rows), dim3(512), shmem, s, b, ext);
 }
 
 template <int T, int PF, int R = 1>
-int launch_ext_pf(const KsPlan &p, const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y,
+int launch_ext_pf(const KsPlan &p, const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y,
                   const KsExt &ext, hipStream_t s) {
     const int64_t row_bytes = (K / Geom<T>::vpb) * Geom<T>::bpb;
     const dim3 grid((unsigned)p.wgs, (unsigned)((M + R - 1) / R)), block((unsigned)p.waves * 64);
     constexpr int WIN = PF < 3 ? PF : 3;
-    return launch(gemv_ks_ext_kernel<T, PF, WIN, R>, grid, block, ks_lds_bytes(p.waves, p.iters, R), s, x, W, bias, y, (int)M, (int)K, (int)N,
+    if (x_is_bf16)
+        return launch(gemv_ks_ext_kernel<T, PF, WIN, R, true>, grid, block, ks_lds_bytes(p.waves, p.iters, R), s, x, W, bias, y, (int)M, (int)K, (int)N,
+                      row_bytes, p.iters, p.nslices, p.half_tail, act, ext);
+    return launch(gemv_ks_ext_kernel<T, PF, WIN, R, false>, grid, block, ks_lds_bytes(p.waves, p.iters, R), s, x, W, bias, y, (int)M, (int)K, (int)N,
                   row_bytes, p.iters, p.nslices, p.half_tail, act, ext);
 }
 
 template <int T, int R>
-int launch_ext_rows(KsPlan p, bool dual, const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y,
+int launch_ext_rows(KsPlan p, bool dual, const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y,
                     const KsExt &ext, hipStream_t s) {
     ks_regroup(p, N, dual, 4);  // (two alternating matrices: 2 or 4, both even)
     switch (p.pf) {
-    case 1: return launch_ext_pf<T, 1, R>(p, x, M, K, W, N, bias, act, y, ext, s);
-    case 2: return launch_ext_pf<T, 2, R>(p, x, M, K, W, N, bias, act, y, ext, s);
-    default: return launch_ext_pf<T, 4, R>(p, x, M, K, W, N, bias, act, y, ext, s);
+    case 1: return launch_ext_pf<T, 1, R>(p, x, x_is_bf16, M, K, W, N, bias, act, y, ext, s);
+    case 2: return launch_ext_pf<T, 2, R>(p, x, x_is_bf16, M, K, W, N, bias, act, y, ext, s);
+    default: return launch_ext_pf<T, 4, R>(p, x, x_is_bf16, M, K, W, N, bias, act, y, ext, s);
     }
 }
 
 template <int T>
-int launch_ext(const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y, const KsExt &ext,
+int launch_ext(const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y, const KsExt &ext,
                hipStream_t s) {
     // With two matrices the row-steps alternate between them: plan for 2 N rows and an even count.
     const bool dual = ext.W2 != nullptr;
@@ -76,16 +83,16 @@ int launch_ext(const float *x, int64_t M, int64_t K, const uint8_t *W, int64_t N
     if (dual) p.wgs = (int)((N + p.iters * 4 - 1) / (p.iters * 4));
     // batches over a large matrix run as passes of two rows (the extras leave no registers for the planes of four)
     if (M >= 2 && (int64_t)gq_row_bytes(T, K) * N * (dual ? 2 : 1) >= kLargeWeightBytes)
-        return launch_ext_rows<T, 2>(p, dual, x, M, K, W, N, bias, act, y, ext, s);
+        return launch_ext_rows<T, 2>(p, dual, x, x_is_bf16, M, K, W, N, bias, act, y, ext, s);
     switch (p.pf) {
-    case 1: return launch_ext_pf<T, 1>(p, x, M, K, W, N, bias, act, y, ext, s);
-    case 2: return launch_ext_pf<T, 2>(p, x, M, K, W, N, bias, act, y, ext, s);
-    case 3: return launch_ext_pf<T, 3>(p, x, M, K, W, N, bias, act, y, ext, s);
-    case 4: return launch_ext_pf<T, 4>(p, x, M, K, W, N, bias, act, y, ext, s);
-    case 5: return launch_ext_pf<T, 5>(p, x, M, K, W, N, bias, act, y, ext, s);
-    case 6: return launch_ext_pf<T, 6>(p, x, M, K, W, N, bias, act, y, ext, s);
-    case 7: return launch_ext_pf<T, 7>(p, x, M, K, W, N, bias, act, y, ext, s);
-    default: return launch_ext_pf<T, 8>(p, x, M, K, W, N, bias, act, y, ext, s);
+    case 1: return launch_ext_pf<T, 1>(p, x, x_is_bf16, M, K, W, N, bias, act, y, ext, s);
+    case 2: return launch_ext_pf<T, 2>(p, x, x_is_bf16, M, K, W, N, bias, act, y, ext, s);
+    case 3: return launch_ext_pf<T, 3>(p, x, x_is_bf16, M, K, W, N, bias, act, y, ext, s);
+    case 4: return launch_ext_pf<T, 4>(p, x, x_is_bf16, M, K, W, N, bias, act, y, ext, s);
+    case 5: return launch_ext_pf<T, 5>(p, x, x_is_bf16, M, K, W, N, bias, act, y, ext, s);
+    case 6: return launch_ext_pf<T, 6>(p, x, x_is_bf16, M, K, W, N, bias, act, y, ext, s);
+    case 7: return launch_ext_pf<T, 7>(p, x, x_is_bf16, M, K, W, N, bias, act, y, ext, s);
+    default: return launch_ext_pf<T, 8>(p, x, x_is_bf16, M, K, W, N, bias, act, y, ext, s);
     }
 }
 
@@ -161,29 +168,29 @@ KsExt make_ext(const RmsNorm *norm, int64_t K, const uint8_t *W2, const float *b
 }
 }  // namespace
 
-int launch_gemv_ks_ext(int type, const float *x, int64_t M, int64_t K, const RmsNorm *norm, const uint8_t *W, const float *bias,
+int launch_gemv_ks_ext(int type, const void *x, bool x_is_bf16, int64_t M, int64_t K, const RmsNorm *norm, const uint8_t *W, const float *bias,
                        const uint8_t *W2, const float *bias2, const float *residual, int64_t N, int act, float *y, hipStream_t s) {
     const KsExt ext = make_ext(norm, K, W2, bias2, residual);
     switch (type) {
-    case kQ4_0: return launch_ext<kQ4_0>(x, M, K, W, N, bias, act, y, ext, s);
-    case kQ8_0: return launch_ext<kQ8_0>(x, M, K, W, N, bias, act, y, ext, s);
-    case kQ4_K: return launch_ext<kQ4_K>(x, M, K, W, N, bias, act, y, ext, s);
-    case kQ6_K: return launch_ext<kQ6_K>(x, M, K, W, N, bias, act, y, ext, s);
-    case kIQ4_NL: return launch_ext<kIQ4_NL>(x, M, K, W, N, bias, act, y, ext, s);
+    case kQ4_0: return launch_ext<kQ4_0>(x, x_is_bf16, M, K, W, N, bias, act, y, ext, s);
+    case kQ8_0: return launch_ext<kQ8_0>(x, x_is_bf16, M, K, W, N, bias, act, y, ext, s);
+    case kQ4_K: return launch_ext<kQ4_K>(x, x_is_bf16, M, K, W, N, bias, act, y, ext, s);
+    case kQ6_K: return launch_ext<kQ6_K>(x, x_is_bf16, M, K, W, N, bias, act, y, ext, s);
+    case kIQ4_NL: return launch_ext<kIQ4_NL>(x, x_is_bf16, M, K, W, N, bias, act, y, ext, s);
     default: return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv_ks: ggml type %d is not implemented", type);
     }
 }
 
 // all problems share K (one normalised input feeds them)
-int launch_gemv_ks_batch_norm(int type, int count, const XsBatchItem *items, const RmsNorm *norm, hipStream_t s, int rows) {
+int launch_gemv_ks_batch_norm(int type, int count, const XsBatchItem *items, const RmsNorm *norm, hipStream_t s, int rows, bool x_is_bf16) {
     if (count < 1 || count > kMaxBatchKs) return fail(GQ_ERR_INVALID, "gemv batch: %d problems (1..%d supported per launch)", count, kMaxBatchKs);
     const KsExt ext = make_ext(norm, items[0].K, nullptr, nullptr, nullptr);
     switch (type) {
-    case kQ4_0: return launch_batch_ext<kQ4_0>(count, items, ext, rows, s);
-    case kQ8_0: return launch_batch_ext<kQ8_0>(count, items, ext, rows, s);
-    case kQ4_K: return launch_batch_ext<kQ4_K>(count, items, ext, rows, s);
-    case kQ6_K: return launch_batch_ext<kQ6_K>(count, items, ext, rows, s);
-    case kIQ4_NL: return launch_batch_ext<kIQ4_NL>(count, items, ext, rows, s);
+    case kQ4_0: return launch_batch_ext<kQ4_0>(count, items, ext, rows, x_is_bf16, s);
+    case kQ8_0: return launch_batch_ext<kQ8_0>(count, items, ext, rows, x_is_bf16, s);
+    case kQ4_K: return launch_batch_ext<kQ4_K>(count, items, ext, rows, x_is_bf16, s);
+    case kQ6_K: return launch_batch_ext<kQ6_K>(count, items, ext, rows, x_is_bf16, s);
+    case kIQ4_NL: return launch_batch_ext<kIQ4_NL>(count, items, ext, rows, x_is_bf16, s);
     default: return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv batch: ggml type %d is not implemented", type);
     }
 }

@@ -828,10 +828,11 @@ int launch_mmq_b32(const void *x, bool x_is_bf16, int64_t M, int64_t K, const ui
     float *partial = reinterpret_cast<float *>(ximg + img_bytes + mmq_scale_bytes(nslices, M));
     const int64_t row_bytes = (K / 32) * B32<T>::kBlockBytes;
     const dim3 xgrid((unsigned)(mtiles * nslices * 4));
-    if (int rc = x_is_bf16 ? launch(mmq_b32_xprep_kernel<true>, xgrid, dim3(256), 0, s, x, ximg, xscale, (int)M, (int)K, S, nslices, nullptr, 0.f, nullptr)
-                           : launch(mmq_b32_xprep_kernel<false>, xgrid, dim3(256), 0, s, x, ximg, xscale, (int)M, (int)K, S, nslices, norm ? norm->gain : nullptr,
-                                    norm ? norm->gain_offset : 0.f, norm ? mmq_xss(xscale, nslices, M) : nullptr))
-        return rc;
+    auto prep = [&](auto kernel) {
+        return launch(kernel, xgrid, dim3(256), 0, s, x, ximg, xscale, (int)M, (int)K, S, nslices, norm ? norm->gain : nullptr, norm ? norm->gain_offset : 0.f,
+                      norm ? mmq_xss(xscale, nslices, M) : nullptr);
+    };
+    if (int rc = x_is_bf16 ? prep(mmq_b32_xprep_kernel<true>) : prep(mmq_b32_xprep_kernel<false>)) return rc;
     const dim3 grid((unsigned)rowwgs, (unsigned)nslices, (unsigned)mtiles * (W2 ? 2u : 1u));  // (both matrices of a gated pair in one launch)
     float *partial2 = W2 ? partial + (size_t)nslices * M * N : nullptr;
     if (int rc = launch(mmq_b32_kernel<T, RT>, grid, dim3(RT * 128), lds_bytes, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N, row_bytes, S,
@@ -1023,10 +1024,11 @@ int launch_mmq_q6k_rt(const MmqExtra *ex, const void *x, bool x_is_bf16, int64_t
     float *partial = reinterpret_cast<float *>(ximg + img_bytes + mmq_scale_bytes(nslices, M));
     const int64_t row_bytes = (K / 256) * 210;
     const dim3 xgrid((unsigned)(mtiles * nslices * 4));
-    if (int rc = x_is_bf16 ? launch(mmq_b32_xprep_kernel<true>, xgrid, dim3(256), 0, s, x, ximg, xscale, (int)M, (int)K, kQ6Slice, nslices, nullptr, 0.f, nullptr)
-                           : launch(mmq_b32_xprep_kernel<false>, xgrid, dim3(256), 0, s, x, ximg, xscale, (int)M, (int)K, kQ6Slice, nslices, norm ? norm->gain : nullptr,
-                                    norm ? norm->gain_offset : 0.f, norm ? mmq_xss(xscale, nslices, M) : nullptr))
-        return rc;
+    auto prep = [&](auto kernel) {
+        return launch(kernel, xgrid, dim3(256), 0, s, x, ximg, xscale, (int)M, (int)K, kQ6Slice, nslices, norm ? norm->gain : nullptr,
+                      norm ? norm->gain_offset : 0.f, norm ? mmq_xss(xscale, nslices, M) : nullptr);
+    };
+    if (int rc = x_is_bf16 ? prep(mmq_b32_xprep_kernel<true>) : prep(mmq_b32_xprep_kernel<false>)) return rc;
     const dim3 grid((unsigned)((N + 32 * RT - 1) / (32 * RT)), (unsigned)nslices, (unsigned)mtiles * (W2 ? 2u : 1u));  // (a gated pair: one launch)
     float *partial2 = W2 ? partial + (size_t)nslices * M * N : nullptr;
     if (int rc = launch(mmq_q6k_kernel<RT>, grid, dim3(RT * 128), (size_t)kLds, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N,
@@ -1108,8 +1110,8 @@ int run_q4k_set(const void *x, bool x_is_bf16, int64_t M, int64_t K, int count, 
     const dim3 pgrid((unsigned)nslices, (unsigned)mtiles, fine ? 16u : 8u);
     const float *gain = norm ? norm->gain : nullptr;
     const float goff = norm ? norm->gain_offset : 0.f;
-    float *xss = norm && !x_is_bf16 ? mmq_xss(xscale, nslices, M) : nullptr;
-    auto prep = [&](auto kernel) { return launch(kernel, pgrid, dim3(512), 0, s, x, ximg, xscale, (int)M, (int)K, slice_sb, x_is_bf16 ? nullptr : gain, x_is_bf16 ? 0.f : goff, xss); };
+    float *xss = norm ? mmq_xss(xscale, nslices, M) : nullptr;
+    auto prep = [&](auto kernel) { return launch(kernel, pgrid, dim3(512), 0, s, x, ximg, xscale, (int)M, (int)K, slice_sb, gain, goff, xss); };
     if (int rc = x_is_bf16 ? (fine ? prep(mmq_xprep_kernel<true, 1>) : prep(mmq_xprep_kernel<true, 2>))
                            : (fine ? prep(mmq_xprep_kernel<false, 1>) : prep(mmq_xprep_kernel<false, 2>)))
         return rc;
@@ -1124,7 +1126,7 @@ int run_q4k_set(const void *x, bool x_is_bf16, int64_t M, int64_t K, int count, 
     const int64_t quads = M * N / 4;
     const int threads = quads / 256 >= 2 * device_cu_count() ? 256 : 64;
     return launch(mmq_reduce_set_kernel, dim3((unsigned)((quads + threads - 1) / threads)), dim3(threads), 0, s, (const float *)partial, nslices, (int)M,
-                  out, (const float *)xscale, (const float *)(norm && !x_is_bf16 ? mmq_xss(xscale, nslices, M) : nullptr), norm ? norm->eps : 0.f,
+                  out, (const float *)xscale, (const float *)xss, norm ? norm->eps : 0.f,
                   1.0f / (float)K);
 }
 }  // namespace

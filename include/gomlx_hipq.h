@@ -193,9 +193,11 @@ int gq_qdense_gated_f32(int type, const float *dX, int64_t M, int64_t K, const g
 
 /* The three calls above for bf16 activations (raw 16-bit patterns, 16-byte aligned; in the batched form every
  * descriptor's dX points at bf16 data): what the same layer code (transformer.go:1099-1101, 1276-1294) builds when the
- * model runs in bfloat16.  Gain, bias and residual stay fp32 and the result is fp32, as for gq_qdense_bf16.  The
- * activations are widened to fp32 (exact) in a per-stream workspace - activation matrices shared by several problems of
- * a batch once - and then take the fp32 routes, so results equal those of the fp32 entry points on the widened inputs. */
+ * model runs in bfloat16.  Gain, bias and residual stay fp32 and the result is fp32, as for gq_qdense_bf16.  Results
+ * equal those of the fp32 entry points on the widened inputs bit for bit: the decode kernel and the split-K pre-pass read
+ * the bf16 rows as they are and widen them in registers (exact), so a decode call costs what its fp32 twin costs; on the
+ * other routes the activations are widened to fp32 in a per-stream workspace first - activation matrices shared by
+ * several problems of a batch once - and then take the fp32 routes. */
 int gq_qdense_block_bf16(int type, const uint16_t *dX, int64_t M, int64_t K, const gq_rmsnorm *norm,
                          const void *dW, int64_t N, const float *dBias, int act,
                          const float *dResidual, float *dY, void *stream);

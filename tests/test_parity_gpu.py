@@ -770,8 +770,25 @@ def test_callers_around_a_projection_with_bf16_activations(gpu, oracle, t):
         if M <= 8:
             probs = [(xb, dev(gpu, W), q, None, None), (xb, dev(gpu, W2), q, dev(gpu, bias), None), (xb, dev(gpu, W[: N // 2]), q, None, None)]
             outs = nn.quantized_dense_batch(probs, norm=norm)
-            for out, (Wm, b) in zip(outs, ((W, None), (W2, bias), (W[: N // 2], None))):
+            x32d = dev(gpu, x32)
+            same = nn.quantized_dense_batch([(x32d,) + p[1:] for p in probs], norm=norm)
+            for out, ref, (Wm, b) in zip(outs, same, ((W, None), (W2, bias), (W[: N // 2], None))):
+                assert gpu.equal(out, ref), ("batch", ggml.name(t), M, K, N)
                 assert rel_err(out.cpu().numpy(), oracle.c_qdense(t, xn, Wm, b, 0)) < TOL_F32
+            # a normalisation without a learned scale, and a residual without a normalisation: the decode kernel reads
+            # the bf16 rows as they are (no gain to fetch beside them)
+            plain = nn.RMSNorm(None, 1e-5, 0.0)
+            for kw in (dict(norm=plain), dict(residual=dev(gpu, res)), dict(norm=plain, residual=dev(gpu, res))):
+                got = nn.quantized_dense(xb, dev(gpu, W), q, None, BACKEND_ACT[act], **kw)
+                ref = nn.quantized_dense(x32d, dev(gpu, W), q, None, BACKEND_ACT[act], **kw)
+                assert gpu.equal(got, ref), (sorted(kw), ggml.name(t), M, K, N)
+            xp = oracle.c_rmsnorm(x32, np.ones(K, np.float32), 1e-5, 0.0)
+            got = nn.quantized_dense(xb, dev(gpu, W), q, None, norm=plain, residual=dev(gpu, res)).cpu().numpy()
+            dense = oracle.c_qdense(t, xp, W, None, 0)
+            assert float(np.max(np.abs(got.astype(np.float64) - (dense + res)))) / float(np.max(np.abs(dense))) < TOL_F32, (ggml.name(t), M, K, N)
+            got = nn.gated_feed_forward(xb, dev(gpu, W), dev(gpu, W2), q, Activation.SILU, None, None, norm=plain)
+            ref = nn.gated_feed_forward(x32d, dev(gpu, W), dev(gpu, W2), q, Activation.SILU, None, None, norm=plain)
+            assert gpu.equal(got, ref), ("gated, no scale", ggml.name(t), M, K, N)
 
 
 def test_residual_in_place_on_the_composed_path(gpu, oracle):
@@ -944,13 +961,16 @@ def test_projections_of_one_input_share_a_split_k_pass(gpu, oracle, rows, K):
     gpu.cuda.synchronize()
     for W, b, a, y in zip(Ws, bs, acts, outs):
         assert rel_err(y.cpu().numpy(), oracle.c_qdense(t, x, W, b, a)) < TOL_F32, (rows, K, W.shape, "no norm")
-    # bf16 activations behind the normalisation: widened exactly, then the same pass
+    # bf16 activations behind the normalisation: the pre-pass widens them (exact), the same pass
     xb = bf16_round(x)
     xbd = dev(gpu, xb).to(gpu.bfloat16)
     outs = nn.quantized_dense_batch([(xbd, dev(gpu, W), q, None, None) for W in Ws], norm=cfg)
     gpu.cuda.synchronize()
     xbn = oracle.c_rmsnorm(xb, gain, 1e-5, 0.0)
-    for W, y in zip(Ws, outs):
+    xb32 = dev(gpu, xb)  # (one buffer: the list shares a pass only as projections of the same activations)
+    same = nn.quantized_dense_batch([(xb32, dev(gpu, W), q, None, None) for W in Ws], norm=cfg)
+    for W, y, ref in zip(Ws, outs, same):
+        assert gpu.equal(y, ref), (rows, K, "bf16 against the widened input")
         assert rel_err(y.cpu().numpy(), oracle.c_qdense(t, xbn, W, None)) < TOL_F32, (rows, K, "bf16")
 
 
