@@ -791,6 +791,32 @@ def test_callers_around_a_projection_with_bf16_activations(gpu, oracle, t):
             assert gpu.equal(got, ref), ("gated, no scale", ggml.name(t), M, K, N)
 
 
+@pytest.mark.parametrize("t,M,K,N", [(Q4_K, 2, 4096, 14336), (Q4_K, 3, 4096, 14336), (Q8_0, 2, 4096, 8192), (Q4_0, 1, 1280, 300),
+                                     (Q6_K, 2, 1280, 264), (IQ4_NL, 5, 2304, 128), (Q4_K, 16, 1024, 64)])
+def test_bf16_rows_in_the_decode_kernel_with_its_extras(gpu, oracle, t, M, K, N):
+    """bf16 activations read by the decode kernel itself, with normalisation, gated product and residual: passes of two rows
+    over a large matrix, a K that ends in a half slice, several rows over a small matrix.  Bit-identical to the fp32 entry
+    points on the widened inputs and within the fp32 bound of the oracle."""
+    q = Quantization(ggml_type=t)
+    x32 = bf16_round((synth.activations(8400 + M, M, K) * 1.5).astype(np.float32))
+    xb, xw = dev(gpu, x32).to(gpu.bfloat16), dev(gpu, x32)
+    gain = (synth.normal(8410, 0, K) * 0.5 + 1.0).astype(np.float32)
+    res = synth.activations(8420, M, N)
+    W, W2 = synth.weights(t, 8430, N, K), synth.weights(t, 8431, N, K)
+    Wd, W2d, resd = dev(gpu, W), dev(gpu, W2), dev(gpu, res)
+    for norm, gain_h in ((nn.RMSNorm(dev(gpu, gain), 1e-6, 1.0), gain + 1.0), (nn.RMSNorm(None, 1e-6, 0.0), np.ones(K, np.float32))):
+        got = nn.quantized_dense(xb, Wd, q, None, norm=norm, residual=resd)
+        assert gpu.equal(got, nn.quantized_dense(xw, Wd, q, None, norm=norm, residual=resd)), (ggml.name(t), M, K, N)
+        xn = oracle.c_rmsnorm(x32, gain_h, 1e-6, 0.0)
+        dense = oracle.c_qdense(t, xn, W, None, 0)
+        assert float(np.max(np.abs(got.cpu().numpy().astype(np.float64) - (dense + res)))) / float(np.max(np.abs(dense))) < TOL_F32
+        got = nn.gated_feed_forward(xb, Wd, W2d, q, Activation.SILU, None, None, norm=norm)
+        assert gpu.equal(got, nn.gated_feed_forward(xw, Wd, W2d, q, Activation.SILU, None, None, norm=norm)), ("gated", ggml.name(t), M, K, N)
+        gate, up = oracle.c_qdense(t, xn, W, None, 0), oracle.c_qdense(t, xn, W2, None, 0)
+        want = oracle.c_qdense(t, xn, W, None, 3).astype(np.float64) * up
+        assert float(np.max(np.abs(got.cpu().numpy() - want))) / (float(np.max(np.abs(gate))) * float(np.max(np.abs(up)))) < 2 * TOL_F32
+
+
 def test_residual_in_place_on_the_composed_path(gpu, oracle):
     """y == residual on shapes that none of the fused routes take (K not a multiple of 256; N not a multiple of 4
     beyond 16 rows): the dense result must not overwrite the residual before it is added."""
