@@ -459,11 +459,11 @@ struct KsExt {
 // rows stay in registers and every weight load is contracted against each of them, so a batch of
 // two to four rows costs one pass over W, not one per row (the arithmetic stays well below the
 // memory time up to four rows).
-template <int T, int PF, int WIN, bool EXT = false, bool XBF16 = false, int R = 1>
+template <int T, int PF, int WIN, bool EXT = false, bool XBF16 = false, int R = 1, bool PADDED = false>
 __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8_t *__restrict__ W,
                                         const float *__restrict__ bias, float *__restrict__ y, int N, int64_t row_bytes, int iters,
                                         int nslices, int half_tail, int act, int waves, int wg, uint32_t *lds, const KsExt *extp = nullptr,
-                                        int xrows = 1, int64_t x_stride = 0) {
+                                        int xrows = 1, int64_t x_stride = 0, int live_iters = 0) {
     typedef typename KS<T>::Raw Raw;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int rg = lane >> 3, c = lane & 7;
@@ -471,7 +471,11 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8
     KsExt ext = {};
     if constexpr (EXT) ext = *extp;
     const bool dual = EXT && ext.W2 != nullptr;
-    const int row0 = wg * (dual ? rows_wg >> 1 : rows_wg);
+    // PADDED (batched launches, one matrix per problem): the workgroup owns live_iters row-steps of rows; the row-steps from
+    // there to `iters` (which the group size divides) read the last of them again - from the caches - and their sums go
+    // to slots that are not written out.  So rows per workgroup need not be a multiple of the group size.
+    const int live = PADDED ? live_iters : iters;
+    const int row0 = wg * (dual ? rows_wg >> 1 : live * 8);
     float *all = reinterpret_cast<float *>(lds + waves * kWaveLdsDwords);  // partial sums [waves][R][rows_wg]
     float *ssq_w = all + waves * R * rows_wg;                              // EXT: sum of squares [waves][R]
     float ssq[R];
@@ -540,7 +544,7 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8
         // (finite scales; their activations are zero).
         auto lane_c = [&](int j) { return (half_tail && wave + j * waves == nslices - 1) ? (c & 3) : c; };
         auto addr = [&](int j, int it) -> const uint8_t * {
-            const int row = min(row0 + (dual ? it >> 1 : it) * 8 + rg, last_row);
+            const int row = min(row0 + (dual ? it >> 1 : (PADDED ? min(it, live - 1) : it)) * 8 + rg, last_row);
             const uint8_t *base = (dual && (it & 1)) ? ext.W2 : W;
             return base + (int64_t)row * row_bytes + (int64_t)(wave + j * waves) * KS<T>::kSliceBytes + KS<T>::lane_offset(lane_c(j));
         };
@@ -626,7 +630,7 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8
     }
     __syncthreads();
     // output row r of activation row q: the wavefronts' partial sums meet here
-    const int rows_out = dual ? rows_wg >> 1 : rows_wg;
+    const int rows_out = dual ? rows_wg >> 1 : live * 8;
     for (int e = tid; e < rows_out * R; e += blockDim.x) {
         int q = 0, r = e;
         if constexpr (R > 1) { q = e / rows_out; r = e - q * rows_out; }
@@ -742,7 +746,7 @@ struct KsProblem {
     const float *bias;
     float *y;
     int64_t row_bytes;
-    int N, K, iters, nslices, half_tail, waves, act, wg_begin;
+    int N, K, iters, live, nslices, half_tail, waves, act, wg_begin;  // live <= iters row-steps of rows per workgroup (see ks_body)
 };
 struct KsBatch {
     int count;
@@ -769,10 +773,11 @@ int plan_ks_batch(int count, const XsBatchItem *items, KsBatch &b, size_t &shmem
         if (!ks_split(it.K, q.waves, q.nslices, q.half_tail)) return fail(GQ_ERR_NOT_IMPLEMENTED, "gemv_ks batch: unsupported K");
         spw[i] = (q.nslices + q.waves - 1) / q.waves;
     }
+    // (row-steps of rows per workgroup: any count; the kernel runs them in whole groups of kBatchPF, see live_iters)
     auto iters_for = [&](int i, int budget) {
-        int64_t iters = budget / spw[i] / kBatchPF * kBatchPF;
-        if (iters < kBatchPF) iters = kBatchPF;
-        if (iters > kMaxItersKs) iters = kMaxItersKs;
+        int64_t iters = budget / spw[i];
+        if (iters < 1) iters = 1;
+        if (iters > kMaxItersKs / kBatchPF * kBatchPF) iters = kMaxItersKs / kBatchPF * kBatchPF;
         return iters;
     };
     auto wgs_for = [&](int budget) {
@@ -780,15 +785,16 @@ int plan_ks_batch(int count, const XsBatchItem *items, KsBatch &b, size_t &shmem
         for (int i = 0; i < count; i++) n += (items[i].N + iters_for(i, budget) * 8 - 1) / (iters_for(i, budget) * 8);
         return n;
     };
-    int budget = kBatchPF;
+    int budget = 1;
     const int budget_max = kMaxItersKs * 64;
-    while (budget < budget_max && wgs_for(budget) > cus) budget += kBatchPF;
+    while (budget < budget_max && wgs_for(budget) > cus) budget++;
     shmem = 0;
     int wg = 0;
     for (int i = 0; i < count; i++) {
         KsProblem &q = b.p[i];
         const int64_t iters = iters_for(i, budget);
-        q.iters = (int)iters;
+        q.live = (int)iters;
+        q.iters = (int)((iters + kBatchPF - 1) / kBatchPF * kBatchPF);
         q.wg_begin = wg;
         wg += (int)((items[i].N + iters * 8 - 1) / (iters * 8));
         const size_t need = ks_lds_bytes(q.waves, q.iters);
