@@ -25,7 +25,7 @@ __global__ __launch_bounds__(512) void gemv_ks_batch_kernel(const KsBatch b) {
     extern __shared__ uint32_t lds[];
     const KsProblem &q = b.p[ks_batch_problem(b, (int)blockIdx.x)];
     const int64_t row = blockIdx.y;  // activation row of every problem
-    ks_body<T, kBatchPF, kBatchPF, false, false, 1, true>(q.x + row * q.K, q.W, q.bias, q.y + row * q.N, q.N, q.row_bytes, q.iters, q.nslices, q.half_tail, q.act, q.waves,
+    ks_body<T, kBatchPF, kBatchWin, false, false, 1, true>(q.x + row * q.K, q.W, q.bias, q.y + row * q.N, q.N, q.row_bytes, q.iters, q.nslices, q.half_tail, q.act, q.waves,
                      (int)blockIdx.x - q.wg_begin, lds, nullptr, 1, 0, q.live);
 }
 

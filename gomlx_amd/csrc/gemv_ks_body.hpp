@@ -737,9 +737,10 @@ void ks_regroup(KsPlan &p, int64_t N, bool dual, int max_pf) {
 // groups of two row-steps, both in flight (its iters is a multiple of 2): measured on the seven
 // projections of a Llama-3-8B layer, groups of 2 take 23.8 us, 3 / 2 in flight 24.1, 4 / 3 24.7 .. 25.4,
 // 8 / 4 25.6 - the finer rounding of rows per workgroup balances the problems better than a deeper
-// window helps.
+// window helps.  (Measured again with rows per workgroup free of the group size, see PADDED: groups of 4 with 3 in flight
+// take 25.0 against 22.8 us: the deeper window itself loses.)
 constexpr int kMaxBatchKs = 8;
-constexpr int kBatchPF = 2;
+constexpr int kBatchPF = 2, kBatchWin = 2;
 struct KsProblem {
     const float *x;
     const uint8_t *W;

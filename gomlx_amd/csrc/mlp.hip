@@ -35,7 +35,7 @@ __global__ __launch_bounds__(512) void gemv_ks_batch_ext_kernel(const KsBatch b,
     const KsProblem &q = b.p[ks_batch_problem(b, (int)blockIdx.x)];
     const int64_t row = blockIdx.y;  // activation row of every problem
     const uint8_t *x = reinterpret_cast<const uint8_t *>(q.x) + row * q.K * (XBF16 ? 2 : 4);  // (q.x points at bf16 data with XBF16)
-    ks_body<T, kBatchPF, kBatchPF, true, XBF16, 1, true>(x, q.W, q.bias, q.y + row * q.N, q.N, q.row_bytes, q.iters, q.nslices, q.half_tail, q.act, q.waves,
+    ks_body<T, kBatchPF, kBatchWin, true, XBF16, 1, true>(x, q.W, q.bias, q.y + row * q.N, q.N, q.row_bytes, q.iters, q.nslices, q.half_tail, q.act, q.waves,
                                                 (int)blockIdx.x - q.wg_begin, lds, &ext, 1, 0, q.live);
 }
 
