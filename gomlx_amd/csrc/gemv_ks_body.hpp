@@ -688,7 +688,9 @@ size_t ks_lds_bytes(int waves, int iters, int xrows = 1) {  // xrows: activation
 // Row-steps per workgroup and per group: up to 8 row-steps form one group (an even count when two
 // matrices alternate); deeper problems run in groups of 4.  (Counts that split into larger equal
 // groups, 14 = 2 x 7 instead of 16 = 4 x 4, spread the rows over all workgroups instead of 7/8 of
-// them; measured on the gated feed-forward of 2 x 14336 rows it made no difference.)
+// them; measured on the gated feed-forward of 2 x 14336 rows it made no difference.  Nor does padding: 14 row-steps per
+// workgroup on 256 workgroups, the last group of 4 filled up with re-reads as in the batched launches, took 15.8 against
+// 14.8 us for 16 on 224.)
 void ks_group(int64_t want, bool even, int &iters, int &pf) {
     if (want < 1) want = 1;
     if (even && (want & 1)) want++;
