@@ -1000,6 +1000,46 @@ def test_projections_of_one_input_share_a_split_k_pass(gpu, oracle, rows, K):
         assert rel_err(y.cpu().numpy(), oracle.c_qdense(t, xbn, W, None)) < TOL_F32, (rows, K, "bf16")
 
 
+def test_batched_submissions_randomized(gpu, oracle):
+    """Seeded random lists of two to eight projections of one format and one to three rows, through gq_qdense_f32_batch and
+    (one K, fp32 or bf16 activations) behind a shared normalisation: widths from a single row to a few thousand, K with and
+    without a half slice and with more slices than wavefronts, so that the workgroups of one launch own anything from one
+    row-step (padded to the kernel's group of two) to dozens."""
+    rng = np.random.default_rng(20240611)
+    for case in range(24):
+        t = ALL_TYPES[int(rng.integers(len(ALL_TYPES)))]
+        q = Quantization(ggml_type=t)
+        count, rows = int(rng.integers(2, 9)), int(rng.choice([1, 1, 1, 2, 3]))
+        use_norm = bool(rng.integers(2))
+        bf16 = use_norm and bool(rng.integers(2))
+        same_k = int(rng.choice([256, 768, 1024, 1280, 2048, 3584, 4608, 5120, 6144, 8192, 14336]))
+        gain = (synth.normal(9100 + case, 0, same_k) * 0.5 + 1.0).astype(np.float32)
+        norm = nn.RMSNorm(dev(gpu, gain), 1e-5, 0.0) if use_norm else None
+        hosts, probs = [], []
+        for i in range(count):
+            K = same_k if use_norm else int(rng.choice([256, 512, 1024, 1280, 2048, 4096, 5120, 14336]))
+            N = int(rng.choice([1, 3, 8, 9, 40, 64, 100, 256, 300, 1000, 1024, 2048]))
+            N = max(1, min(N, 6_000_000 // K))
+            W = synth.weights(t, 9200 + 10 * case + i, N, K)
+            x = synth.activations(9500 + 10 * case + i, rows, K)
+            x = bf16_round(x) if bf16 else x
+            b = synth.normal(9800 + 10 * case + i, 0, N).astype(np.float32) * 0.1 if rng.integers(2) else None
+            act = int(rng.choice([0, 1, 2, 3]))
+            hosts.append((x, W, b, act))
+            xd = dev(gpu, x).to(gpu.bfloat16) if bf16 else dev(gpu, x)
+            probs.append((xd, dev(gpu, W), q, None if b is None else dev(gpu, b), BACKEND_ACT[act]))
+        outs = nn.quantized_dense_batch(probs, norm=norm)
+        gpu.cuda.synchronize()
+        for (x, W, b, act), y in zip(hosts, outs):
+            xn = oracle.c_rmsnorm(x, gain, 1e-5, 0.0) if use_norm else x
+            want, pre = oracle.c_qdense(t, xn, W, b, act), oracle.c_qdense(t, xn, W, b, 0)
+            scale = max(float(np.max(np.abs(want))), float(np.max(np.abs(pre))))
+            if not np.isfinite(scale) or scale == 0.0:
+                continue
+            err = float(np.max(np.abs(y.cpu().numpy().astype(np.float64) - want))) / scale
+            assert err < TOL_F32, (case, ggml.name(t), rows, use_norm, bf16, W.shape, act, err)
+
+
 def test_shared_split_k_pass_randomized(gpu, oracle):
     """Seeded random lists of two to four Q4_K projections of one input, 6 to 99 rows, any widths that are multiples of 4
     (most not multiples of the 128-row workgroup), with and without normalisation, gain, bias; activations without tanh
