@@ -17,7 +17,7 @@ __global__ __launch_bounds__(512) void gemv_ks_kernel(const void *__restrict__ X
     const int r0 = (int)blockIdx.y * R;
     const uint8_t *x = reinterpret_cast<const uint8_t *>(X) + r0 * x_stride;
     ks_body<T, PF, WIN, false, XBF16, R>(x, W, bias, Y + (int64_t)r0 * N, N, row_bytes, iters, nslices, half_tail, act, (int)(blockDim.x >> 6),
-                                         (int)blockIdx.x, lds, nullptr, min(R, M - r0), x_stride);
+                                         (int)blockIdx.x, lds, nullptr, min(R, M - r0), x_stride, 0, (int)gridDim.x);
 }
 
 template <int T>
@@ -26,7 +26,7 @@ __global__ __launch_bounds__(512) void gemv_ks_batch_kernel(const KsBatch b) {
     const KsProblem &q = b.p[ks_batch_problem(b, (int)blockIdx.x)];
     const int64_t row = blockIdx.y;  // activation row of every problem
     ks_body<T, kBatchPF, kBatchWin, false, false, 1, true>(q.x + row * q.K, q.W, q.bias, q.y + row * q.N, q.N, q.row_bytes, q.iters, q.nslices, q.half_tail, q.act, q.waves,
-                     (int)blockIdx.x - q.wg_begin, lds, nullptr, 1, 0, q.live);
+                     (int)blockIdx.x - q.wg_begin, lds, nullptr, 1, 0, q.live, q.nwg);
 }
 
 

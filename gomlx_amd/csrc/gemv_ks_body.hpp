@@ -422,8 +422,11 @@ __device__ __forceinline__ void ks_load(typename KS<T>::Raw &r, const uint8_t *p
 constexpr int kWaveLdsDwords = 76 * 4;  // per wavefront: 64 uint4 of planes, 16 scales, up to 32 sums
 
 // Workgroup `wg` of a problem: `waves` wavefronts work (threads beyond them only join the final
-// barrier); wavefront w handles slices w, w + waves, ... below nslices of the 8 * iters rows
-// starting at wg * 8 * iters.  PF divides iters: rows are consumed in groups of PF, buffer j of a
+// barrier); wavefront w handles slices w, w + waves, ... below nslices of the workgroup's 8 * iters rows.
+// Those rows are row-steps wg, wg + nwg, wg + 2 nwg, ... of the matrix (nwg: the workgroups of the launch that share it),
+// not one block: at any moment the workgroups together read one window of consecutive rows that moves through the
+// matrix, as a plain read of the bytes would, instead of nwg streams half a megabyte apart (the seven projections of a
+// Llama-3-8B layer in one launch: 22.6 against 23.4 us).  PF divides iters: rows are consumed in groups of PF, buffer j of a
 // group always holding the row-step with (it % PF == j).
 // WIN <= PF row-steps are kept in flight: WIN go out before the activations are converted, and
 // each consumed step is followed by the load of the step WIN ahead, so that load issue (which
@@ -463,7 +466,7 @@ template <int T, int PF, int WIN, bool EXT = false, bool XBF16 = false, int R = 
 __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8_t *__restrict__ W,
                                         const float *__restrict__ bias, float *__restrict__ y, int N, int64_t row_bytes, int iters,
                                         int nslices, int half_tail, int act, int waves, int wg, uint32_t *lds, const KsExt *extp = nullptr,
-                                        int xrows = 1, int64_t x_stride = 0, int live_iters = 0) {
+                                        int xrows = 1, int64_t x_stride = 0, int live_iters = 0, int nwg = 1) {
     typedef typename KS<T>::Raw Raw;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int rg = lane >> 3, c = lane & 7;
@@ -475,7 +478,6 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8
     // there to `iters` (which the group size divides) read the last of them again - from the caches - and their sums go
     // to slots that are not written out.  So rows per workgroup need not be a multiple of the group size.
     const int live = PADDED ? live_iters : iters;
-    const int row0 = wg * (dual ? rows_wg >> 1 : live * 8);
     float *all = reinterpret_cast<float *>(lds + waves * kWaveLdsDwords);  // partial sums [waves][R][rows_wg]
     float *ssq_w = all + waves * R * rows_wg;                              // EXT: sum of squares [waves][R]
     float ssq[R];
@@ -544,7 +546,8 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8
         // (finite scales; their activations are zero).
         auto lane_c = [&](int j) { return (half_tail && wave + j * waves == nslices - 1) ? (c & 3) : c; };
         auto addr = [&](int j, int it) -> const uint8_t * {
-            const int row = min(row0 + (dual ? it >> 1 : (PADDED ? min(it, live - 1) : it)) * 8 + rg, last_row);
+            const int step = dual ? it >> 1 : (PADDED ? min(it, live - 1) : it);  // of this workgroup; wg + step * nwg of the matrix
+            const int row = min((wg + step * nwg) * 8 + rg, last_row);
             const uint8_t *base = (dual && (it & 1)) ? ext.W2 : W;
             return base + (int64_t)row * row_bytes + (int64_t)(wave + j * waves) * KS<T>::kSliceBytes + KS<T>::lane_offset(lane_c(j));
         };
@@ -634,7 +637,7 @@ __device__ __forceinline__ void ks_body(const void *__restrict__ xv, const uint8
     for (int e = tid; e < rows_out * R; e += blockDim.x) {
         int q = 0, r = e;
         if constexpr (R > 1) { q = e / rows_out; r = e - q * rows_out; }
-        const int row = row0 + r;
+        const int row = (wg + (r >> 3) * nwg) * 8 + (r & 7);
         if (row >= N) continue;
         if constexpr (R > 1) { if (q >= xrows) continue; }
         const int64_t at = (int64_t)q * N + row;
@@ -749,7 +752,7 @@ struct KsProblem {
     const float *bias;
     float *y;
     int64_t row_bytes;
-    int N, K, iters, live, nslices, half_tail, waves, act, wg_begin;  // live <= iters row-steps of rows per workgroup (see ks_body)
+    int N, K, iters, live, nslices, half_tail, waves, act, wg_begin, nwg;  // live <= iters row-steps of rows per workgroup, nwg workgroups (see ks_body)
 };
 struct KsBatch {
     int count;
@@ -800,6 +803,7 @@ int plan_ks_batch(int count, const XsBatchItem *items, KsBatch &b, size_t &shmem
         q.iters = (int)((iters + kBatchPF - 1) / kBatchPF * kBatchPF);
         q.wg_begin = wg;
         wg += (int)((items[i].N + iters * 8 - 1) / (iters * 8));
+        q.nwg = wg - q.wg_begin;
         const size_t need = ks_lds_bytes(q.waves, q.iters);
         if (need > shmem) shmem = need;
     }

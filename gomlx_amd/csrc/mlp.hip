@@ -24,7 +24,7 @@ __global__ __launch_bounds__(512) void gemv_ks_ext_kernel(const void *__restrict
     if (e.residual) e.residual += (int64_t)r0 * N;
     const int64_t x_stride = (int64_t)K * (XBF16 ? 2 : 4);
     ks_body<T, PF, WIN, true, XBF16, R>(reinterpret_cast<const uint8_t *>(X) + r0 * x_stride, W, bias, Y + (int64_t)r0 * N, N, row_bytes, iters, nslices,
-                                        half_tail, act, (int)(blockDim.x >> 6), (int)blockIdx.x, lds, &e, min(R, M - r0), x_stride);
+                                        half_tail, act, (int)(blockDim.x >> 6), (int)blockIdx.x, lds, &e, min(R, M - r0), x_stride, 0, (int)gridDim.x);
 }
 
 // Batched submission (several batch-1 projections of one format in one launch) with one RMS
@@ -36,7 +36,7 @@ __global__ __launch_bounds__(512) void gemv_ks_batch_ext_kernel(const KsBatch b,
     const int64_t row = blockIdx.y;  // activation row of every problem
     const uint8_t *x = reinterpret_cast<const uint8_t *>(q.x) + row * q.K * (XBF16 ? 2 : 4);  // (q.x points at bf16 data with XBF16)
     ks_body<T, kBatchPF, kBatchWin, true, XBF16, 1, true>(x, q.W, q.bias, q.y + row * q.N, q.N, q.row_bytes, q.iters, q.nslices, q.half_tail, q.act, q.waves,
-                                                (int)blockIdx.x - q.wg_begin, lds, &ext, 1, 0, q.live);
+                                                (int)blockIdx.x - q.wg_begin, lds, &ext, 1, 0, q.live, q.nwg);
 }
 
 template <int T>
