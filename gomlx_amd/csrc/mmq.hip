@@ -7,7 +7,8 @@
 //
 //  * Activation traffic.  Every row tile of W needs all of x.  Fetching x per tile through
 //    the CU's vector-memory path would move several times more bytes than the weights themselves, so the
-//    work is split along K instead: a workgroup owns a K-slice of up to 7 super-blocks (1792 values),
+//    work is split along K instead: a workgroup owns a K-slice of up to 7 super-blocks (1792 values; every n-th
+//    super-block of a row for n slices, so that the slices' workgroups together read consecutive bytes),
 //    keeps the slice of x for 32 batch columns resident in LDS (fp16 in MFMA fragment order, written
 //    once by a pre-pass and copied global -> LDS without passing registers) and streams
 //    128 rows of W past it.  Slices are summed by a second, tiny kernel that also applies
@@ -129,11 +130,11 @@ __device__ __forceinline__ float wave_sum(float v) {
 // With xss (normalisation folded in): x is multiplied by gain + gain_offset (gain may be null) and xss[m0 + m] receives
 // the slice's sum of squares of the raw x.
 template <int ROUNDS, bool BF16X>
-__device__ __forceinline__ void stage_x(const void *__restrict__ X, int M, int K, int m0, int k0, uint8_t *__restrict__ lds, int tid,
+__device__ __forceinline__ void stage_x(const void *__restrict__ X, int M, int K, int m0, int sb_first, int sb_stride, uint8_t *__restrict__ lds, int tid,
                                         int round0, bool active, float *red, float *__restrict__ inv_scale, const float *__restrict__ gain,
                                         float gain_offset, float *__restrict__ xss) {
     const int oct = tid & 255;  // fixed per thread; its items are columns (tid >> 8) + 2 r
-    const int k = k0 + 8 * oct;
+    const int k = ((oct >> 5) * sb_stride + sb_first) * 256 + 8 * (oct & 31);  // super-block sbl of the slice is sb_first + sbl * sb_stride of the row
     const int sbl = oct >> 5, v8 = oct & 31;
     const int gp = v8 >> 3, w8 = v8 & 7, high = w8 >> 2, idx8 = w8 & 3;
     const int q = high * 2 + (idx8 & 1), c = 2 * gp + (idx8 >> 1);
@@ -213,7 +214,7 @@ __global__ __launch_bounds__(512) void mmq_xprep_kernel(const void *__restrict__
     __shared__ float red[2 * 2 * ROUNDS * 4];
     const int slice = blockIdx.x, mt = blockIdx.y;
     const bool active = (((int)threadIdx.x & 255) >> 5) < slice_sb;
-    stage_x<ROUNDS, BF16X>(X, M, K, mt * kMT, slice * slice_sb * 256, ximg + ((size_t)mt * gridDim.x + slice) * kLdsBytes, threadIdx.x,
+    stage_x<ROUNDS, BF16X>(X, M, K, mt * kMT, slice, (int)gridDim.x, ximg + ((size_t)mt * gridDim.x + slice) * kLdsBytes, threadIdx.x,
                       ROUNDS * blockIdx.z, active, red, xscale + (size_t)slice * M, gain, gain_offset, xss ? xss + (size_t)slice * M : nullptr);
 }
 
@@ -251,8 +252,10 @@ __global__ __launch_bounds__(64 * RT * kParts) void mmq_q4k_kernel(const uint8_t
     const int kg = lane >> 5, col = lane & 31;
     const int rt = wave % RT, par = wave / RT;  // par = 0 .. kParts-1
     const int slice = blockIdx.y;
-    const int k0 = slice * slice_sb * 256;
-    const int nsb = min(slice_sb, (K - k0) >> 8);
+    // Slice s holds super-blocks s, s + nslices, s + 2 nslices, ... of every row: the workgroups of a row range, which
+    // run side by side, then read one stretch of consecutive bytes of each row at a time and move along the rows together.
+    const int nslices = gridDim.y;
+    const int nsb = ((K >> 8) - slice + nslices - 1) / nslices;
     const int n = xblk * (32 * RT) + rt * 32 + col;  // this lane's weight row
 
     // the slice's activation image goes straight from global memory into LDS (no registers)
@@ -273,7 +276,7 @@ __global__ __launch_bounds__(64 * RT * kParts) void mmq_q4k_kernel(const uint8_t
     // instruction writes 64 lanes x 16 bytes to consecutive LDS addresses, which is the tile's own layout.
     // (byte offsets from the first row of the tile: 32 rows of a matrix the index range admits stay far below 2^32)
     const int row0 = xblk * (32 * RT) + rt * 32;
-    const uint8_t *wtile = W + (int64_t)min(row0, N - 1) * row_bytes + (int64_t)(k0 >> 8) * 144;
+    const uint8_t *wtile = W + (int64_t)min(row0, N - 1) * row_bytes + slice * 144;
     uint32_t csrc[kParkLoads];
 #pragma unroll
     for (int l = 0; l < kParkLoads; l++) {
@@ -282,7 +285,7 @@ __global__ __launch_bounds__(64 * RT * kParts) void mmq_q4k_kernel(const uint8_t
     }
     uint8_t *park = lds + xs_off + kXSBytes + wave * kParkBytes;
     auto fetch = [&](int sb) __attribute__((always_inline)) {
-        const uint8_t *base = wtile + sb * 144;
+        const uint8_t *base = wtile + sb * nslices * 144;
 #pragma unroll
         for (int l = 0; l < kParkLoads; l++)
             if (64 * l + 64 <= 32 * 9 || lane < 32 * 9 - 64 * l)  // (the last instruction carries 32 chunks)
