@@ -52,6 +52,7 @@ SIGNATURES = [
     ("gq_graph_destroy", _int, [_vp]),
     ("gq_profile_begin", _int, []),
     ("gq_profile_end", _int, [_pint, ctypes.POINTER(ctypes.c_double)]),
+    ("gq_workspace_stats", _int, [ctypes.POINTER(_sz), _pint]),
     ("gq_last_error", ctypes.c_char_p, []),
 ]
 

@@ -126,7 +126,40 @@ def build_host_test(verbose: bool = True) -> str:
         sys.stderr.write(r.stderr)
     if verbose:
         print(f"built {WORKSPACE_TEST}")
+    build_sanitized(verbose)
     return HOST_TEST
+
+
+SANITIZED = {
+    # binary: (source, sanitizer flags, links the library)
+    "workspace_test_tsan": ("workspace_test.cpp", ["-fsanitize=thread"], False),
+    "workspace_test_asan": ("workspace_test.cpp", ["-fsanitize=address,undefined", "-fno-sanitize-recover=all"], False),
+    "hipq_backend_test_asan": ("hipq_backend_test.cpp", ["-fsanitize=address,undefined", "-fno-sanitize-recover=all"], True),
+}
+
+
+def sanitized_path(name: str) -> str:
+    return os.path.join(HOST, "build", name)
+
+
+def build_sanitized(verbose: bool = True) -> dict:
+    """The host-only test programs again under ThreadSanitizer (the two-threads-on-one-stream bookkeeping of the scratch
+    pool) and under AddressSanitizer + UndefinedBehaviorSanitizer (pool bookkeeping; the host layer's graph-build rules).
+    Host code only: the device library they link is the ordinary build."""
+    os.makedirs(os.path.join(HOST, "build"), exist_ok=True)
+    out = {}
+    for name, (src, flags, links) in SANITIZED.items():
+        cmd = ["g++", "-O1", "-g", "-fno-omit-frame-pointer", "-std=c++17", "-Wall", "-Wextra", "-pthread", *flags,
+               os.path.join(HOST, src), "-o", sanitized_path(name)]
+        if links:
+            cmd += ["-L" + HERE, "-lgomlx_hipq", "-Wl,-rpath,$ORIGIN/../..", "-Wl,-rpath,/opt/rocm/lib"]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"{name} build failed:\n{r.stdout}\n{r.stderr}")
+        out[name] = sanitized_path(name)
+        if verbose:
+            print(f"built {out[name]}")
+    return out
 
 
 if __name__ == "__main__":

@@ -837,9 +837,11 @@ int gq_qdense_norm_bf16_batch(int count, const gq_dense_desc *descs, const gq_rm
     size_t offset[64], total = 0;
     int first[64];
     for (int i = 0; i < count; i++) {
+        first[i] = -1;  // an empty problem (no rows or no columns) reads no activations: it neither gets nor lends a widened copy
+        if (descs[i].M == 0 || descs[i].N == 0) continue;
         first[i] = i;
         for (int j = 0; j < i; j++)
-            if (descs[j].dX == descs[i].dX && descs[j].M == descs[i].M && descs[j].K == descs[i].K) { first[i] = first[j]; break; }
+            if (first[j] >= 0 && descs[j].dX == descs[i].dX && descs[j].M == descs[i].M && descs[j].K == descs[i].K) { first[i] = first[j]; break; }
         if (first[i] == i) { offset[i] = total; total += widened_bytes(descs[i].M, descs[i].K); }
     }
     void *ws = nullptr;
@@ -847,7 +849,7 @@ int gq_qdense_norm_bf16_batch(int count, const gq_dense_desc *descs, const gq_rm
         if (int rc = stream_workspace((hipStream_t)stream, total, &ws, kWsWidenSlot)) return rc;
     for (int i = 0; i < count; i++) {
         wide[i] = descs[i];
-        if (descs[i].M == 0 || descs[i].N == 0) continue;
+        if (first[i] < 0) continue;
         if (first[i] == i) {
             const float *x32 = nullptr;
             if (int rc = widen_into(ws, offset[i], reinterpret_cast<const uint16_t *>(descs[i].dX), descs[i].M, descs[i].K, (hipStream_t)stream, &x32)) return rc;
@@ -963,6 +965,12 @@ int gq_profile_end(int *launches, double *total_us) {
     if (launches) *launches = n;
     if (total_us) *total_us = total;
     return rc;
+}
+
+int gq_workspace_stats(size_t *live_bytes, int *streams) {
+    if (live_bytes) *live_bytes = pool().live_bytes();
+    if (streams) *streams = (int)pool().stream_count();
+    return GQ_OK;
 }
 
 const char *gq_last_error(void) { return g_error; }

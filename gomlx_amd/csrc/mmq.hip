@@ -274,7 +274,7 @@ __global__ __launch_bounds__(64 * RT * kParts) void mmq_q4k_kernel(const uint8_t
     // Chunk c = lane + 64 l of a (32 rows x 144 bytes) tile is piece c % 9 of row c / 9.  The chunks go from global
     // memory straight into the wavefront's piece of LDS (no registers held while they are in flight): each load
     // instruction writes 64 lanes x 16 bytes to consecutive LDS addresses, which is the tile's own layout.
-    // (byte offsets from the first row of the tile: 32 rows of a matrix the index range admits stay far below 2^32)
+    // (byte offsets from the first row of the tile: mmq_supported keeps 31 rows below 2^32 bytes)
     const int row0 = xblk * (32 * RT) + rt * 32;
     const uint8_t *wtile = W + (int64_t)min(row0, N - 1) * row_bytes + slice * 144;
     uint32_t csrc[kParkLoads];
@@ -294,6 +294,9 @@ __global__ __launch_bounds__(64 * RT * kParts) void mmq_q4k_kernel(const uint8_t
     };
     if (par < nsb) fetch(par);
     const uint8_t *myrow = park + col * 144;
+    // a barrier does not wait for loads in flight: every wavefront's share of the image copy must have landed in LDS
+    // before it arrives (the wait also covers the wavefront's own first tile, which the loop would wait for next anyway)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
     f16v acc;
@@ -736,6 +739,9 @@ __global__ __launch_bounds__(RT * 128) void mmq_b32_kernel(const uint8_t *__rest
         for (int l = 0; l < G::kLoads; l++) buf[l] = *reinterpret_cast<const ChunkA4 *>(base + coff[l]);
     };
     fetch(0);
+    // a barrier does not wait for loads in flight: every wavefront's share of the image copy must have landed in LDS
+    // before it arrives (loads complete in order, so this also waits for the first stretch, which is needed next anyway)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
     f16v acc;
@@ -923,6 +929,8 @@ __global__ __launch_bounds__(512) void mmq_q6k_kernel(const uint8_t *__restrict_
             if (lane + 64 * i < 32 * kQ6HalfDwords) reinterpret_cast<uint32_t *>(park)[lane + 64 * i] = v[i];
     };
     park_half(0);
+    // a barrier does not wait for loads in flight: every wavefront's share of the image copy must have landed first
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();  // image landed; the parked half is this wavefront's own
 
     f16v acc;
@@ -1051,7 +1059,9 @@ int launch_mmq_q6k(const MmqExtra *ex, const void *x, bool x_is_bf16, int64_t M,
 }  // namespace
 
 bool mmq_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, const void *bias, const void *y) {
-    const bool shape_ok = M >= 2 && M <= 256 && N % 4 == 0 && N <= (int64_t)INT32_MAX / 2 && K <= INT32_MAX / 2 &&
+    // K <= 2^26: the kernels address the 32 rows of a tile by 32-bit byte offsets from its first row (31 rows of at most
+    // 2^26 * 34 / 32 bytes stay below 2^32)
+    const bool shape_ok = M >= 2 && M <= 256 && N % 4 == 0 && N <= (int64_t)INT32_MAX / 2 && K <= ((int64_t)1 << 26) &&
                           ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(bias) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
     if (type == kQ4_K) return shape_ok && K % 256 == 0;
     if (type == kQ8_0 || type == kQ4_0 || type == kIQ4_NL) return shape_ok && K % 256 == 0;  // whole stretches of 8 blocks

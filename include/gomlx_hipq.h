@@ -233,6 +233,11 @@ int gq_graph_destroy(void *graph_exec);
 int gq_profile_begin(void);
 int gq_profile_end(int *launches, double *total_us);
 
+/* Bookkeeping of the per-stream workspaces (no counterpart in the reference; for tests and for callers that
+ * watch device memory): the bytes the library currently holds for them and the number of streams that own one.
+ * Either pointer may be null.  The fixed array of gq_qdense_f32_static is not counted. */
+int gq_workspace_stats(size_t *live_bytes, int *streams);
+
 /* Message of the last error on this thread; valid until the next failing call. */
 const char *gq_last_error(void);
 

@@ -43,6 +43,46 @@ def test_workspace_bookkeeping():
     assert "0 failed" in r.stdout and "FAIL" not in r.stdout
 
 
+def _sanitized(name):
+    path = build.sanitized_path(name)
+    if not os.path.exists(path):
+        if not os.path.exists(build.LIB):
+            build.build(verbose=False)
+        else:
+            build.build_sanitized(verbose=False)
+    return path
+
+
+def _clean(r):
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "0 failed" in r.stdout and "FAIL" not in r.stdout
+    for word in ("ThreadSanitizer", "AddressSanitizer", "LeakSanitizer", "runtime error"):
+        assert word not in r.stderr, r.stderr
+
+
+def test_workspace_bookkeeping_under_thread_sanitizer():
+    """Two host threads on one stream, recordings, growth and destruction with every access to the pool's shared state
+    watched for data races (the executor may compile and run from many goroutines, core/graph/exec.go:121-125)."""
+    _clean(_run(binary=_sanitized("workspace_test_tsan")))
+
+
+def test_workspace_bookkeeping_under_address_sanitizer():
+    _clean(_run(binary=_sanitized("workspace_test_asan")))
+
+
+def test_host_layer_build_time_rules_under_address_sanitizer():
+    """The C++ host layer's graph-build validation and fallback rules with address and undefined-behaviour checks on."""
+    _clean(_run("--build-only", binary=_sanitized("hipq_backend_test_asan")))
+
+
+def test_oracle_under_address_sanitizer():
+    """The oracle's C code on exactly-sized buffers with random bytes in every packed field (oracle/oracle_selftest.c)."""
+    odir = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle")
+    r = subprocess.run(["make", "-C", odir, "oracle_selftest_asan"], capture_output=True, text=True, timeout=200)
+    assert r.returncode == 0, r.stdout + r.stderr
+    _clean(_run(binary=os.path.join(odir, "oracle_selftest_asan")))
+
+
 @pytest.mark.gpu
 def test_host_layer_reference_cases_on_gpu():
     r = _run()

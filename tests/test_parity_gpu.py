@@ -1201,6 +1201,94 @@ def test_config4_llama_layer_projections(gpu, oracle):
         assert rel_err(run_dense(gpu, Q4_K, x, W), oracle.c_qdense(Q4_K, x, W)) < TOL_F32, (K, N)
 
 
+C4_SHAPES = [(4096, 4096), (4096, 1024), (4096, 1024), (4096, 4096), (4096, 14336), (4096, 14336), (14336, 4096)]
+
+
+@pytest.mark.parametrize("rows", [1, 2, 3])
+def test_config4_seven_projections_as_one_batched_submission(gpu, oracle, rows):
+    """Configuration 4 the way the benchmark times it: the seven full-size Q4_K matrices handed over in ONE
+    gq_qdense_f32_batch (one launch of the batched decode GEMV, whose plan deals every matrix's rows over a common grid),
+    against the oracle and, bit for bit, against seven separate calls.  Two and three rows per problem as well."""
+    torch = gpu
+    q = Quantization(ggml_type=Q4_K)
+    hosts, probs = [], []
+    for i, (K, N) in enumerate(C4_SHAPES):
+        W = synth.weights(Q4_K, 1004 + i, N, K)
+        x = synth.activations(1104 + i, rows, K)
+        hosts.append((x, W))
+        probs.append((dev(torch, x), dev(torch, W), q, None, Activation.NONE))
+    outs = nn.quantized_dense_batch(probs)
+    torch.cuda.synchronize()
+    for (x, W), p, y in zip(hosts, probs, outs):
+        assert rel_err(y.cpu().numpy(), oracle.c_qdense(Q4_K, x, W)) < TOL_F32, (rows, W.shape)
+        assert torch.equal(nn.quantized_dense(p[0], p[1], q), y), (rows, W.shape)
+
+
+@pytest.mark.parametrize("rows", [1, 2])
+def test_decoder_layer_sequence_full_size(gpu, oracle, rows):
+    """Configuration 4's matrices in the order and with the dependencies of a decoder layer, at full size, as four calls:
+    q / k / v behind one RMSNorm (one submission), o + residual, RMSNorm + act(gate) * up, down + residual in place.
+    Every call is judged against the oracle on the inputs that call received (so each keeps the 1e-3 bound of a single
+    contraction, 2e-3 for the product of two), and the end of the chain against the oracle's own chain."""
+    import ctypes
+    from gomlx_amd import _lib
+    torch = gpu
+    L = _lib.lib()
+    t = Q4_K
+    Ws = [synth.weights(t, 1004 + i, N, K) for i, (K, N) in enumerate(C4_SHAPES)]
+    Wq, Wk, Wv, Wo, Wg, Wu, Wd = (dev(torch, W) for W in Ws)
+    H, KV, F = 4096, 1024, 14336
+    x0 = synth.activations(1104, rows, H)
+    # The rows of these synthetic weights all have the same positive mean, so every output of a projection carries the sum
+    # of its input: an attention output with a positive mean keeps the gates on the rising side of SiLU (with a negative
+    # one act(gate) * up collapses to ~1e-5 and the last call would only test the residual), and a small gain keeps the
+    # down projection at the magnitude of the residual it is added to, so that both show in the result.
+    attn0 = synth.activations(1107, rows, H) + np.float32(0.25)
+    gain = ((synth.normal(1200, 0, H) * 0.5 + 1.0) * 3e-4).astype(np.float32)
+    eps = 1e-5
+    x, attn, gd = dev(torch, x0), dev(torch, attn0), dev(torch, gain)
+    q, k, v = (torch.full((rows, n), float("nan"), device="cuda") for n in (H, KV, KV))
+    h, ff = torch.full((rows, H), float("nan"), device="cuda"), torch.full((rows, F), float("nan"), device="cuda")
+    norm = _lib.RmsNormDesc(gd.data_ptr(), eps, 0.0)
+    sp = torch.cuda.current_stream().cuda_stream
+    d = (_lib.DenseDesc * 3)()
+    for dd, (W, y, n) in zip(d, ((Wq, q, H), (Wk, k, KV), (Wv, v, KV))):
+        dd.type, dd.act, dd.dX, dd.M, dd.K, dd.dW, dd.N, dd.dBias, dd.dY = t, 0, x.data_ptr(), rows, H, W.data_ptr(), n, None, y.data_ptr()
+    _lib.check(L.gq_qdense_norm_f32_batch(3, d, ctypes.byref(norm), sp))
+    _lib.check(L.gq_qdense_block_f32(t, attn.data_ptr(), rows, H, None, Wo.data_ptr(), H, None, 0, x.data_ptr(), h.data_ptr(), sp))
+    _lib.check(L.gq_qdense_gated_f32(t, h.data_ptr(), rows, H, ctypes.byref(norm), Wg.data_ptr(), None, Wu.data_ptr(), None, F, 3,
+                                     ff.data_ptr(), sp))
+    torch.cuda.synchronize()
+    h_mid = h.cpu().numpy()
+    _lib.check(L.gq_qdense_block_f32(t, ff.data_ptr(), rows, F, None, Wd.data_ptr(), H, None, 0, h.data_ptr(), h.data_ptr(), sp))
+    torch.cuda.synchronize()
+
+    def close(got, dense, res, tol, what):  # the bound is on the contraction; a residual only shifts both sides
+        want = dense if res is None else dense + res
+        err = float(np.max(np.abs(got.astype(np.float64) - want)))
+        rel_err(got, want)  # (records the margins)
+        # (the addition of the residual is one more fp32 rounding, of the sum)
+        assert err < tol * float(np.max(np.abs(dense))) + 2.0 ** -23 * float(np.max(np.abs(want))), (what, rows, err)
+
+    xn = oracle.c_rmsnorm(x0, gain, eps, 0.0)
+    for got, W, what in ((q, Ws[0], "q"), (k, Ws[1], "k"), (v, Ws[2], "v")):
+        close(got.cpu().numpy(), oracle.c_qdense(t, xn, W), None, TOL_F32, what)
+    close(h_mid, oracle.c_qdense(t, attn0, Ws[3]), x0.astype(np.float64), TOL_F32, "o + residual")
+    ff_got = ff.cpu().numpy()
+    hn = oracle.c_rmsnorm(h_mid, gain, eps, 0.0)
+    g_pre, u_pre = oracle.c_qdense(t, hn, Ws[4]), oracle.c_qdense(t, hn, Ws[5])
+    ff_want = oracle.c_gated_ffn(t, h_mid, Ws[4], Ws[5], None, None, 3, (gain, eps, 0.0))
+    assert np.max(np.abs(ff_got.astype(np.float64) - ff_want)) / (float(np.max(np.abs(g_pre))) * float(np.max(np.abs(u_pre)))) < 2 * TOL_F32
+    out = h.cpu().numpy()
+    close(out, oracle.c_qdense(t, ff_got, Ws[6]), h_mid.astype(np.float64), TOL_F32, "down + residual")
+    # the oracle's own chain from the layer's inputs (the errors of three contractions in a row add up)
+    h_o = (oracle.c_qdense(t, attn0, Ws[3]) + x0).astype(np.float32)
+    ff_o = oracle.c_gated_ffn(t, h_o, Ws[4], Ws[5], None, None, 3, (gain, eps, 0.0)).astype(np.float32)
+    dense_o = oracle.c_qdense(t, ff_o, Ws[6])
+    assert float(np.max(np.abs(ff_got))) > 0.05 and float(np.max(np.abs(dense_o))) > 0.1 * float(np.max(np.abs(h_o)))  # (not degenerate)
+    assert float(np.max(np.abs(out.astype(np.float64) - (dense_o + h_o)))) / float(np.max(np.abs(dense_o))) < 4 * TOL_F32
+
+
 def test_batched_submission_equals_separate_calls(gpu, oracle):
     """gq_qdense_f32_batch: the seven projections of a decoder layer (scaled down), mixed with a
     batch-5 problem and another format, against one call each and against the oracle."""

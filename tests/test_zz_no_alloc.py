@@ -45,6 +45,55 @@ def test_static_scratch_entry_matches_the_allocating_one(gpu, oracle):
     _both(gpu, oracle, ggml.Q4_K, 1, 4096, 512, 9300)
 
 
+def _ws_stats(L):
+    import ctypes
+    live, streams = ctypes.c_size_t(0), ctypes.c_int(0)
+    _lib.check(L.gq_workspace_stats(ctypes.byref(live), ctypes.byref(streams)))
+    return live.value, streams.value
+
+
+def test_static_scratch_entry_allocates_nothing(gpu, oracle):
+    """The property the entry point exists for.  On a stream the library has never seen (no workspace exists for it, so a
+    call that fell through to the per-stream pool would have to create one), split-K calls go through the static entry
+    first: the pool's books (bytes held, streams known) and the device's free memory must not move, and the results must
+    be right.  The first call loads the kernels' code (the runtime may take device memory for that), so free memory is
+    compared across the second, larger call."""
+    import ctypes
+    torch = gpu
+    L = _lib.lib()
+    sp = ctypes.c_void_p()
+    _lib.check(L.gq_stream_create(ctypes.byref(sp)))
+    try:
+        t = ggml.Q4_K
+        cases = []
+        for M, K, N, seed in ((9, 2048, 512, 9400), (32, 4096, 2048, 9410)):
+            W, x = synth.weights(t, seed, N, K), synth.activations(seed + 1, M, K)
+            cases.append((M, K, N, x, W, _dev(torch, x), _dev(torch, W), torch.full((M, N), float("nan"), device="cuda")))
+        torch.cuda.synchronize()
+        books = _ws_stats(L)
+        free_before = None
+        for i, (M, K, N, x, W, xd, Wd, y) in enumerate(cases):
+            if i == 1:
+                free_before = torch.cuda.mem_get_info()[0]
+            _lib.check(L.gq_qdense_f32_static(t, xd.data_ptr(), M, K, Wd.data_ptr(), N, None, 0, y.data_ptr(), sp))
+            _lib.check(L.gq_sync(sp))
+            assert _ws_stats(L) == books, "the static entry point touched the workspace pool"
+        assert torch.cuda.mem_get_info()[0] == free_before, "device memory was allocated during the call"
+        for M, K, N, x, W, xd, Wd, y in cases:
+            want = oracle.c_qdense(t, x, W)
+            assert float(np.max(np.abs(y.cpu().numpy().astype(np.float64) - want))) / float(np.max(np.abs(want))) < 1e-3
+        # the allocating entry point on the same stream does create a workspace: the books do see what they are meant to see
+        M, K, N, x, W, xd, Wd, y = cases[1]
+        y2 = torch.full((M, N), float("nan"), device="cuda")
+        _lib.check(L.gq_qdense_f32(t, xd.data_ptr(), M, K, Wd.data_ptr(), N, None, 0, y2.data_ptr(), sp))
+        _lib.check(L.gq_sync(sp))
+        after = _ws_stats(L)
+        assert after[0] > books[0] and after[1] == books[1] + 1
+        assert torch.equal(y, y2)
+    finally:
+        _lib.check(L.gq_stream_destroy(sp))
+
+
 def test_static_scratch_entry_rejects_what_does_not_fit(gpu):
     L = _lib.lib()
     t, M, K, N = ggml.Q8_0, 512, 4096, 4096  # two-pass GEMM: a 32 MiB weight image
