@@ -102,9 +102,17 @@ def parse_args():
                         "workload that hardware counter readings (FETCH_SIZE / WRITE_SIZE) are scaled by")
     p.add_argument("--yardstick", action="store_true",
                    help="instead of the benchmark, time the plain read-only kernel on 17.8 / 33.0 / 122.7 MB of cold weights")
+    p.add_argument("--yardstick-size", choices=["c0", "c1", "c2", "c4"], default=None,
+                   help="with --yardstick: only this workload's byte count, with ONE grid shape (--yardstick-shape), so that a "
+                        "kernel trace of the run holds a single kind of launch")
+    p.add_argument("--yardstick-shape", default=None,
+                   help="workgroups,threads,depth of the read-only kernel for --yardstick-size (depth 100 + d: d non-temporal loads in "
+                        "flight); default: the shape that usually reads that size fastest")
     p.add_argument("--matmul-yardstick", action="store_true",
                    help="instead of the benchmark, time the vendor library's plain bf16 GEMM (torch.matmul) on C3's shape, 2048 x 4096 x 4096: "
                         "what a 16-bit GEMM with no dequantisation reaches on this chip")
+    p.add_argument("--mfma-valu-yardstick", action="store_true",
+                   help="only measure how many vector-ALU instructions fit into the shadow of matrix instructions (cycles per group)")
     p.add_argument("--mfma-yardstick", action="store_true",
                    help="instead of the benchmark, time matrix instructions alone (the prefill GEMM's count and occupancy, no data movement) "
                         "with random and with zero operands and on a quarter of the CUs, with the shader clock the kernel measured itself")
@@ -203,12 +211,12 @@ class Yardstick:
     # (depth 100 + d: the same d loads in flight, issued as non-temporal loads)
     SHAPES = ((2048, 256, 2), (1024, 256, 4), (512, 256, 8), (256, 512, 8), (1024, 256, 104), (512, 256, 108))
 
-    def time_buffers(self, torch, bufs, stream, tstream, steps):
-        """Best mean time (us) per launch over SHAPES: one recorded graph of `steps` launches rotating over `bufs`."""
+    def time_buffers(self, torch, bufs, stream, tstream, steps, shapes=None):
+        """Best mean time (us) per launch over SHAPES (or `shapes`): one recorded graph of `steps` launches rotating over `bufs`."""
         nbytes = bufs[0].numel() * bufs[0].element_size()
-        out = torch.zeros(2048 * 256 + 16, dtype=torch.int32, device="cuda")
+        out = torch.zeros(2048 * 512 + 16, dtype=torch.int32, device="cuda")
         best = None
-        for wgs, threads, depth in self.SHAPES:
+        for wgs, threads, depth in shapes or self.SHAPES:
             def launch(i):
                 rc = self.lib.gqy_read(bufs[i % len(bufs)].data_ptr(), nbytes, 0, wgs, threads, depth, 0, 0, 0, out.data_ptr(), stream)
                 if rc:
@@ -493,10 +501,45 @@ def host_threads():
     return max(1, min(n, cap) if cap > 0 else n)
 
 
-def cpu_baseline(name):
+def reference_toolchain():
+    """Whether the reference's own CPU backend could be timed on this host: a Go toolchain and a module cache that holds
+    github.com/gomlx/compute v0.1.2 (go.mod:10 of the reference).  Looked for, never fetched or built."""
+    import shutil
+    go = shutil.which("go")
+    info = {"go": go, "go_version": None, "gomlx_compute_v0.1.2_in_module_cache": False}
+    if go:
+        try:
+            import subprocess
+            info["go_version"] = subprocess.run([go, "version"], capture_output=True, text=True, timeout=20).stdout.strip() or None
+        except (OSError, subprocess.SubprocessError):
+            pass
+    roots = [os.environ.get("GOMODCACHE")]
+    roots += [os.path.join(g, "pkg", "mod") for g in (os.environ.get("GOPATH") or os.path.join(os.path.expanduser("~"), "go")).split(os.pathsep) if g]
+    for r in roots:
+        if r and os.path.isdir(os.path.join(r, "github.com", "gomlx", "compute@v0.1.2")):
+            info["gomlx_compute_v0.1.2_in_module_cache"] = True
+    info["usable"] = bool(go) and info["gomlx_compute_v0.1.2_in_module_cache"]
+    if not info["usable"]:
+        info["consequence"] = "the reference's Go backend cannot be run here: the baseline is this repository's C restatement of its algorithm (kind: port)"
+    return info
+
+
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return None
+
+
+def cpu_baseline(name, min_runs=5, min_seconds=3.0, max_seconds=25.0):
     """The CPU oracle's fused fp32 restatement on the host cores (checker code used as a reported baseline only), on the
     inputs the GPU leg uses (same seeds): >= 2 warm-ups, then >= 5 runs and >= 3 s, like the reference's own timing
-    protocol (internal/perf/dotgeneral_perf_test.go:366-381), capped at ~25 s."""
+    protocol (internal/perf/dotgeneral_perf_test.go:366-381), capped at ~25 s (the side workloads: 1 warm-up, >= 3 runs and
+    >= 1.5 s, so that the default run stays within minutes)."""
     from gomlx_amd import ggml, synth
     from oracle import ggml_oracle as oracle
     cores = host_threads()
@@ -530,16 +573,18 @@ def cpu_baseline(name):
         for t, x, W in probs:
             oracle.c_qdense(t, x, W, None, 0, f32acc_threads=cores)
 
-    once(); once()
+    once()
+    if min_runs >= 5:
+        once()
     runs, t0 = 0, time.perf_counter()
     while True:
         once()
         runs += 1
         el = time.perf_counter() - t0
-        if (runs >= 5 and el >= 3.0) or el >= 25.0:
+        if (runs >= min_runs and el >= min_seconds) or el >= max_seconds:
             break
     per = el / runs
-    common = {"cores": cores, "host_cpus": os.cpu_count(), "kind": "port",
+    common = {"cores": cores, "host_cpus": os.cpu_count(), "cpu_model": cpu_model(), "kind": "port",
               "sample": f"{sample}, same seeded inputs as the GPU leg; {runs} runs, {per * 1e3:.2f} ms each; OpenMP over output rows"}
     if name in ("c3", "prefill"):
         return {"value": flops / per / 1e12, "unit": "TFLOP/s", **common}
@@ -559,18 +604,31 @@ def copy_calibration(torch, steps):
     print(json.dumps({"copy_calibration": True, "launches": steps, "read_bytes_per_launch": n * 4, "write_bytes_per_launch": n * 4}))
 
 
-def yardstick_only(torch, steps):
-    """The plain read-only kernel on cold buffers of the three decode workloads' sizes."""
+YARDSTICK_BYTES = {"c0": 17825792, "c1": 33030144, "c2": 33030144, "c4": 122683392}
+YARDSTICK_DEFAULT_SHAPE = {"c0": (512, 256, 108), "c1": (1024, 256, 104), "c2": (1024, 256, 104), "c4": (256, 512, 8)}
+
+
+def yardstick_only(torch, steps, size=None, shape=None):
+    """The plain read-only kernel on cold buffers of the decode workloads' sizes (best of several grid shapes), or, with
+    `size`, on that one size with one grid shape (for a kernel trace that holds a single kind of launch)."""
     ys = yardstick()
     if ys is None:
         print("bench.py: gomlx_amd/libgq_yardstick.so is missing (python -m gomlx_amd.build)", file=sys.stderr)
         sys.exit(4)
     tstream = torch.cuda.Stream()
     out = {"yardstick": "read-only kernel, every byte loaded once, no arithmetic; cold: rotation over > 512 MB of distinct buffers", "sizes": {}}
-    for name, nbytes in (("c0", 17825792), ("c1", 33030144), ("c2", 33030144), ("c4", 122683392)):
+    shapes = None
+    if size is not None:
+        shapes = (tuple(int(v) for v in shape.split(",")) if shape else YARDSTICK_DEFAULT_SHAPE[size],)
+        if len(shapes[0]) != 3:
+            print("bench.py: --yardstick-shape wants workgroups,threads,depth", file=sys.stderr)
+            sys.exit(2)
+    for name, nbytes in YARDSTICK_BYTES.items():
+        if size is not None and name != size:
+            continue
         copies = max(2, -(-(512 << 20) // nbytes) + 1)
         bufs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device="cuda") for _ in range(copies)]
-        us, wgs, threads, depth = ys.time_buffers(torch, bufs, tstream.cuda_stream, tstream, steps)
+        us, wgs, threads, depth = ys.time_buffers(torch, bufs, tstream.cuda_stream, tstream, steps, shapes)
         out["sizes"][name] = {"bytes": nbytes, "us": us, "gbps": nbytes / us / 1e3, "frac_of_peak": nbytes / us / 1e3 / HBM_PEAK_GBS,
                               "grid": f"{wgs} x {threads}, depth {depth}", "copies": copies}
         del bufs
@@ -652,6 +710,54 @@ def mfma_yardstick(torch, steps, only_first=False):
     return out
 
 
+def mfma_valu_yardstick(torch, groups=512):
+    """Vector-ALU instructions in the shadow of matrix instructions (gomlx_amd/csrc/yardstick.hip, gqy_mfma_valu): shader cycles
+    per group of four independent v_mfma_f32_32x32x16_bf16 per wavefront plus NV independent vector-ALU instructions, placed
+    behind the group or NV / 4 behind each matrix instruction, accumulators in ordinary or in accumulation registers, for one
+    and two wavefronts per SIMD (128 resp. 256 cycles of matrix work per group), on one workgroup (no power limit in play) and on
+    one workgroup per CU.  Cycles: shader clock counter, from the first wavefront's start to the last one's end, per workgroup,
+    mean over workgroups.  A figure that stays at the matrix cycles means the vector-ALU work is free; 4 more cycles per
+    instruction and wavefront mean that nothing overlaps."""
+    ys = yardstick()
+    if ys is None:
+        return None
+    vp = ctypes.c_void_p
+    ys.lib.gqy_mfma_valu.argtypes = [vp] + [ctypes.c_int] * 7 + [vp, vp, vp]
+    ys.lib.gqy_mfma_valu.restype = ctypes.c_int
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    st = torch.cuda.Stream()
+    frags = torch.randn(8 * 4 * 64 * 8, device="cuda").to(torch.bfloat16)
+    sink = torch.zeros(cus * 512, device="cuda")
+    kinds = {0: "v_fma_f32", 1: "v_xor_b32", 2: "v_cvt_pk_bf16_f32"}
+    out = {"mfma_valu_yardstick": "shader cycles per group of 4 x v_mfma_f32_32x32x16_bf16 + NV independent vector-ALU instructions per wavefront",
+           "groups_per_wavefront": groups, "rows": []}
+    for wgs in (1, cus):
+        for threads in (256, 512):
+            for acc in (0, 1):
+                for kind in (0, 1, 2):
+                    for place in (0, 1):
+                        waves = threads // 64
+                        row = {"workgroups": wgs, "wavefronts_per_simd": threads // 256, "matrix_cycles_per_group": 128 * (threads // 256),
+                               "accumulators": "accumulation registers" if acc else "ordinary registers", "instruction": kinds[kind],
+                               "placement": "interleaved" if place else "behind the group", "cycles_per_group": {}, "shader_mhz": {}}
+                        for nv in (0, 8, 16, 32, 48):
+                            clocks = torch.zeros(32 * wgs, dtype=torch.int64, device="cuda")
+                            with torch.cuda.stream(st):
+                                for _ in range(3):  # (the last launch's stamps are the ones read)
+                                    rc = ys.lib.gqy_mfma_valu(frags.data_ptr(), groups, wgs, threads, nv, place, kind, acc, clocks.data_ptr(),
+                                                              sink.data_ptr(), st.cuda_stream)
+                                    if rc:
+                                        raise RuntimeError(f"gqy_mfma_valu failed ({rc})")
+                                torch.cuda.synchronize()
+                            c = clocks.cpu().view(wgs, 8, 4)[:, :waves, :].double()
+                            span = c[:, :, 2].max(dim=1).values - c[:, :, 0].min(dim=1).values
+                            wall = (c[:, :, 3].max(dim=1).values - c[:, :, 1].min(dim=1).values) / 100.0
+                            row["cycles_per_group"][str(nv)] = round(float((span / groups).mean()), 1)
+                            row["shader_mhz"][str(nv)] = round(float((span / wall).mean()))
+                        out["rows"].append(row)
+    return out
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -667,10 +773,17 @@ def main():
         copy_calibration(torch, args.steps)
         return
     if args.yardstick:
-        yardstick_only(torch, min(args.steps, 50))
+        yardstick_only(torch, min(args.steps, 50), args.yardstick_size, args.yardstick_shape)
         return
     if args.matmul_yardstick:
         print(json.dumps(matmul_yardstick(torch, min(args.steps, 50))))
+        return
+    if args.mfma_valu_yardstick:
+        out = mfma_valu_yardstick(torch)
+        if out is None:
+            print("bench.py: gomlx_amd/libgq_yardstick.so is missing (python -m gomlx_amd.build)", file=sys.stderr)
+            sys.exit(4)
+        print(json.dumps(out))
         return
     if args.mfma_yardstick:
         out = mfma_yardstick(torch, min(args.steps, 200))
@@ -736,6 +849,7 @@ def main():
     }
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(args.config)
+        line["cpu_baseline"]["reference_toolchain"] = reference_toolchain()
     if not args.no_others:
         names = ["c0", "c1", "c2", "c3", "c4"] + (["prefill", "ffn", "layer"] if args.all else [])
         others = {}
@@ -749,6 +863,8 @@ def main():
             others[name] = {"workload": WORKLOAD_TEXT[name], "dtype": DTYPE[name], "arithmetic": ARITHMETIC[name], "metric": r["metric"],
                             "value": r["value"], "unit": r["unit"], "ms_per_step": r["ms_per_step"], "roofline": r["roofline"],
                             "clock_state": r.get("clock_state"), "steps": steps, "launches_per_step": r["launches_per_step"]}
+            if not args.no_cpu and name in ("c0", "c1", "c2", "c3", "c4"):  # the five benchmark configurations each carry their CPU baseline
+                others[name]["cpu_baseline"] = cpu_baseline(name, min_runs=3, min_seconds=1.5, max_seconds=12.0)
         line["others"] = others
     print(json.dumps(line))
 

@@ -60,6 +60,10 @@ void *g_scratch_ptr[kMaxDevices] = {};
 
 int ws_alloc(void **p, size_t bytes) {
     GQ_HIP(hipMalloc(p, bytes));
+    // the flag words at the head of a buffer start at zero (allocation never happens inside a recording)
+    hipError_t e = hipMemsetAsync(*p, 0, bytes < kWsSyncBytes ? bytes : kWsSyncBytes, nullptr);
+    if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
+    if (e != hipSuccess) { (void)hipFree(*p); *p = nullptr; return hip_fail(e, "hipMemsetAsync(workspace flags)"); }
     return GQ_OK;
 }
 void ws_release(void *p) { (void)hipFree(p); }
@@ -93,23 +97,28 @@ struct CallScope {
 
 }  // namespace
 
-int stream_workspace(hipStream_t s, size_t bytes, void **out, int slot) {
+int stream_workspace(hipStream_t s, size_t bytes, void **out, int slot, uint32_t **sync) {
     CallScope *sc = t_scope;
     if (!sc) return fail(GQ_ERR_INVALID, "internal: scratch memory requested outside an entry point");
+    void *base = nullptr;
     if (sc->static_ptr) {
-        if (slot != 0 || bytes > kStaticScratchBytes)
+        // (the static array is zero when the library is loaded: its first kWsSyncBytes are the flag words)
+        if (slot != 0 || bytes > kStaticScratchBytes - kWsSyncBytes)
             return fail(GQ_ERR_INVALID, "gq_qdense_f32_static: this call needs %zu bytes of scratch memory, the static buffer holds %zu; use gq_qdense_f32",
-                        bytes, kStaticScratchBytes);
-        *out = sc->static_ptr;
-        return GQ_OK;
+                        bytes, kStaticScratchBytes - kWsSyncBytes);
+        base = sc->static_ptr;
+    } else {
+        if (slot < 0 || slot >= kWsSlots) return fail(GQ_ERR_INVALID, "internal: workspace slot %d", slot);
+        if (!sc->lock.held()) sc->lock.lock(pool().stream(s));
+        const int rc = pool().acquire(*sc->lock.held(), s, slot, bytes + kWsSyncBytes, &base);
+        if (rc == kWsWouldAllocateInRecording)
+            return fail(GQ_ERR_INVALID, "qdense: the %zu-byte workspace of this stream must exist before a graph is recorded; run the "
+                        "same call once outside the recording first", bytes);
+        if (rc) return rc;
     }
-    if (slot < 0 || slot >= kWsSlots) return fail(GQ_ERR_INVALID, "internal: workspace slot %d", slot);
-    if (!sc->lock.held()) sc->lock.lock(pool().stream(s));
-    const int rc = pool().acquire(*sc->lock.held(), s, slot, bytes, out);
-    if (rc == kWsWouldAllocateInRecording)
-        return fail(GQ_ERR_INVALID, "qdense: the %zu-byte workspace of this stream must exist before a graph is recorded; run the "
-                    "same call once outside the recording first", bytes);
-    return rc;
+    *out = static_cast<unsigned char *>(base) + kWsSyncBytes;
+    if (sync) *sync = static_cast<uint32_t *>(base);
+    return GQ_OK;
 }
 
 ProfileState &profile_state() {

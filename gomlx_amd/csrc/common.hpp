@@ -33,7 +33,10 @@ int device_cu_count();
 
 // ---- per-stream scratch memory (grows on demand; must exist before a graph recording uses it) ----
 // Slot 0 belongs to the dense kernels, slot 1 to the operations composed of several dense calls.
-int stream_workspace(hipStream_t s, size_t bytes, void **out, int slot = 0);
+// Every buffer is preceded by kWsSyncBytes of flag words (`sync`, if asked for) that are zero when the buffer is
+// created; kernels that use them leave them zero again.
+constexpr size_t kWsSyncBytes = 4096;
+int stream_workspace(hipStream_t s, size_t bytes, void **out, int slot = 0, uint32_t **sync = nullptr);
 
 // ---- launch ---------------------------------------------------------------------------
 struct ProfileState {

@@ -27,6 +27,8 @@
 #include "blocks.hpp"
 #include "common.hpp"
 
+#include <cstdlib>
+
 namespace gq {
 
 namespace {
@@ -200,6 +202,92 @@ struct RawSB { uint4 hd, c[4]; };  // header + this lane's four chunks (steps 0.
 
 
 
+// One super-block of a 32-row tile against the staged activations: `cur` is lane (row col, k-group kg)'s header and code
+// bytes, `lds` the fragment image (slot-major, see stage_x), `sums` the sub-block sums of the super-block's 32 columns
+// (16 bytes each).  SBSCALE: the activations of this super-block carry their own power-of-two scale per column, whose
+// inverses (`inv`, 32 floats) multiply the block's contribution; otherwise the caller's slice-wide scale is applied later.
+template <bool SBSCALE>
+__device__ __forceinline__ void q4k_contract_sb(const RawSB &cur, const uint8_t *lds, const uint8_t *sums, const float *inv, int sbl, int kg, int col,
+                                                uint32_t magic, f16v &acc) {
+    const float d = half_bits_to_float(cur.hd.x & 0xFFFFu), dmin = half_bits_to_float(cur.hd.x >> 16);
+    // all eight 6-bit scales / minima as bytes: sc0..3, sc4..7, m0..3, m4..7
+    const uint32_t a = cur.hd.y, b = cur.hd.z, c = cur.hd.w;
+    const uint32_t sc_lo = a & 0x3F3F3F3Fu, mn_lo = b & 0x3F3F3F3Fu;
+    const uint32_t sc_hi = (c & 0x0F0F0F0Fu) | ((a >> 2) & 0x30303030u);
+    const uint32_t mn_hi = ((c >> 4) & 0x0F0F0F0Fu) | ((b >> 2) & 0x30303030u);
+    f16v p1;
+#pragma unroll
+    for (int r = 0; r < 16; r++) p1[r] = 0.f;
+    // all sixteen activation fragments of this super-block are requested up front so that the
+    // LDS latency hides behind the code conversion below
+    h8 xfr[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const int slot = (sbl * 8 + 2 * (i >> 2) + kg) * 4 + (i & 3);
+        xfr[i] = *reinterpret_cast<const h8 *>(lds + (slot * kMT + (col ^ (slot & 15))) * 16);
+    }
+#pragma unroll
+    for (int st = 0; st < 4; st++) {
+        // chunk 2 st + kg lies in group st: sub-block 2 st in the low nibbles, 2 st + 1 in the high ones
+        const uint32_t scw = (st < 2 ? sc_lo : sc_hi) >> (16 * (st & 1));
+        const float s0f = (float)(scw & 0xFFu), s1f = (float)((scw >> 8) & 0xFFu);
+        const h2 s0 = as_h2(pack_h2(s0f, s0f));
+        const h2 s1 = as_h2(pack_h2(s1f * 0.0625f, s1f * 0.0625f));  // high-nibble pairs arrive as 1024 + 16 n
+        const h2 k0h = as_h2(pack_h2(-1024.f * s0f, -1024.f * s0f));
+        const h2 k1h = as_h2(pack_h2(-64.f * s1f, -64.f * s1f));
+        const uint32_t dw[4] = {cur.c[st].x, cur.c[st].y, cur.c[st].z, cur.c[st].w};
+        uint32_t wl[8], wh[8];
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const uint32_t u = dw[w], v = dw[w] >> 8;
+            wl[2 * w] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(u, 0x000F000Fu, magic), s0, k0h));
+            wl[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(v, 0x000F000Fu, magic), s0, k0h));
+            wh[2 * w] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(u, 0x00F000F0u, magic), s1, k1h));
+            wh[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(v, 0x00F000F0u, magic), s1, k1h));
+        }
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const uint32_t *src = (q < 2 ? wl : wh) + 4 * (q & 1);
+            const h8 wfrag = __builtin_bit_cast(h8, make_uint4(src[0], src[1], src[2], src[3]));
+            p1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xfr[4 * st + q], wfrag, p1, 0, 0, 0);
+        }
+    }
+    // minima: k-group 0 carries the exact integers (m0, m2, m1, m3, m4, m6, m5, m7) against the sub-block sums of x in
+    // the same order; dmin multiplies the finished fp32 sums below, as d multiplies p1 (in an fp16 operand dmin * m
+    // would be rounded to 11 bits, and overflow from dmin = 1040 on)
+    f16v p2, zero16;
+#pragma unroll
+    for (int r = 0; r < 16; r++) zero16[r] = 0.f;
+    {
+        uint4 mv = make_uint4(0u, 0u, 0u, 0u), sv = make_uint4(0u, 0u, 0u, 0u);
+        if (kg == 0) {
+            const h2 off = as_h2(0xE400E400u);  // (-1024, -1024)
+            mv.x = __builtin_bit_cast(uint32_t, magic_pair(mn_lo, 0x00FF00FFu, magic) + off);
+            mv.y = __builtin_bit_cast(uint32_t, magic_pair(mn_lo >> 8, 0x00FF00FFu, magic) + off);
+            mv.z = __builtin_bit_cast(uint32_t, magic_pair(mn_hi, 0x00FF00FFu, magic) + off);
+            mv.w = __builtin_bit_cast(uint32_t, magic_pair(mn_hi >> 8, 0x00FF00FFu, magic) + off);
+            sv = *reinterpret_cast<const uint4 *>(sums + col * 16);
+        }
+        p2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, sv), __builtin_bit_cast(h8, mv), zero16, 0, 0, 0);
+    }
+    if constexpr (SBSCALE) {
+        // lane holds columns m = 8 (r / 4) + 4 kg + r % 4
+        float4 iv[4];
+#pragma unroll
+        for (int g = 0; g < 4; g++) iv[g] = reinterpret_cast<const float4 *>(inv)[2 * g + kg];
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const float f = (r & 3) == 0 ? iv[r >> 2].x : (r & 3) == 1 ? iv[r >> 2].y : (r & 3) == 2 ? iv[r >> 2].z : iv[r >> 2].w;
+            acc[r] = fmaf(f, fmaf(-dmin, p2[r], d * p1[r]), acc[r]);
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = fmaf(d, p1[r], acc[r]);
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = fmaf(-dmin, p2[r], acc[r]);
+    }
+}
+
 // Activation pre-pass: writes each (K-slice, column tile)'s LDS image (fragment-ordered fp16
 // activations + sub-block sums) to global memory once; the row-range workgroups of the main
 // kernel then only copy 132 KiB each instead of converting it again.  grid = (slices, column
@@ -321,71 +409,7 @@ __global__ __launch_bounds__(64 * RT * kParts) void mmq_q4k_kernel(const uint8_t
         for (int st = 0; st < 4; st++) cur.c[st] = make_uint4(rc[st].x, rc[st].y, rc[st].z, rc[st].w);
         __builtin_amdgcn_wave_barrier();
         if (sbl + kParts < nsb) fetch(sbl + kParts);
-        const float d = half_bits_to_float(cur.hd.x & 0xFFFFu), dmin = half_bits_to_float(cur.hd.x >> 16);
-        // all eight 6-bit scales / minima as bytes: sc0..3, sc4..7, m0..3, m4..7
-        const uint32_t a = cur.hd.y, b = cur.hd.z, c = cur.hd.w;
-        const uint32_t sc_lo = a & 0x3F3F3F3Fu, mn_lo = b & 0x3F3F3F3Fu;
-        const uint32_t sc_hi = (c & 0x0F0F0F0Fu) | ((a >> 2) & 0x30303030u);
-        const uint32_t mn_hi = ((c >> 4) & 0x0F0F0F0Fu) | ((b >> 2) & 0x30303030u);
-        f16v p1;
-#pragma unroll
-        for (int r = 0; r < 16; r++) p1[r] = 0.f;
-        // all sixteen activation fragments of this super-block are requested up front so that the
-        // LDS latency hides behind the code conversion below
-        h8 xfr[16];
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int slot = (sbl * 8 + 2 * (i >> 2) + kg) * 4 + (i & 3);
-            xfr[i] = *reinterpret_cast<const h8 *>(lds + (slot * kMT + (col ^ (slot & 15))) * 16);
-        }
-#pragma unroll
-        for (int st = 0; st < 4; st++) {
-            // chunk 2 st + kg lies in group st: sub-block 2 st in the low nibbles, 2 st + 1 in the high ones
-            const uint32_t scw = (st < 2 ? sc_lo : sc_hi) >> (16 * (st & 1));
-            const float s0f = (float)(scw & 0xFFu), s1f = (float)((scw >> 8) & 0xFFu);
-            const h2 s0 = as_h2(pack_h2(s0f, s0f));
-            const h2 s1 = as_h2(pack_h2(s1f * 0.0625f, s1f * 0.0625f));  // high-nibble pairs arrive as 1024 + 16 n
-            const h2 k0h = as_h2(pack_h2(-1024.f * s0f, -1024.f * s0f));
-            const h2 k1h = as_h2(pack_h2(-64.f * s1f, -64.f * s1f));
-            const uint32_t dw[4] = {cur.c[st].x, cur.c[st].y, cur.c[st].z, cur.c[st].w};
-            uint32_t wl[8], wh[8];
-#pragma unroll
-            for (int w = 0; w < 4; w++) {
-                const uint32_t u = dw[w], v = dw[w] >> 8;
-                wl[2 * w] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(u, 0x000F000Fu, magic), s0, k0h));
-                wl[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(v, 0x000F000Fu, magic), s0, k0h));
-                wh[2 * w] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(u, 0x00F000F0u, magic), s1, k1h));
-                wh[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(v, 0x00F000F0u, magic), s1, k1h));
-            }
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const uint32_t *src = (q < 2 ? wl : wh) + 4 * (q & 1);
-                const h8 wfrag = __builtin_bit_cast(h8, make_uint4(src[0], src[1], src[2], src[3]));
-                p1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(xfr[4 * st + q], wfrag, p1, 0, 0, 0);
-            }
-        }
-        // minima: k-group 0 carries the exact integers (m0, m2, m1, m3, m4, m6, m5, m7) against the sub-block sums of x in
-        // the same order; dmin multiplies the finished fp32 sums below, as d multiplies p1 (in an fp16 operand dmin * m
-        // would be rounded to 11 bits, and overflow from dmin = 1040 on)
-        f16v p2, zero16;
-#pragma unroll
-        for (int r = 0; r < 16; r++) zero16[r] = 0.f;
-        {
-            uint4 mv = make_uint4(0u, 0u, 0u, 0u), sv = make_uint4(0u, 0u, 0u, 0u);
-            if (kg == 0) {
-                const h2 off = as_h2(0xE400E400u);  // (-1024, -1024)
-                mv.x = __builtin_bit_cast(uint32_t, magic_pair(mn_lo, 0x00FF00FFu, magic) + off);
-                mv.y = __builtin_bit_cast(uint32_t, magic_pair(mn_lo >> 8, 0x00FF00FFu, magic) + off);
-                mv.z = __builtin_bit_cast(uint32_t, magic_pair(mn_hi, 0x00FF00FFu, magic) + off);
-                mv.w = __builtin_bit_cast(uint32_t, magic_pair(mn_hi >> 8, 0x00FF00FFu, magic) + off);
-                sv = *reinterpret_cast<const uint4 *>(lds + xs_off + (sbl * kMT + col) * 16);
-            }
-            p2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, sv), __builtin_bit_cast(h8, mv), zero16, 0, 0, 0);
-        }
-#pragma unroll
-        for (int r = 0; r < 16; r++) acc[r] = fmaf(d, p1[r], acc[r]);
-#pragma unroll
-        for (int r = 0; r < 16; r++) acc[r] = fmaf(-dmin, p2[r], acc[r]);
+        q4k_contract_sb<false>(cur, lds, lds + xs_off + sbl * (kMT * 16), nullptr, sbl, kg, col, magic, acc);
     }
 
     // wavefronts 1..kParts-1 of a row tile hand their 32 x 32 partial tiles to wavefront 0 through LDS
@@ -409,6 +433,239 @@ __global__ __launch_bounds__(64 * RT * kParts) void mmq_q4k_kernel(const uint8_t
     }
 }
 
+// ---- the activation pre-pass folded into the main kernel --------------------------------------------------------
+//
+// mmq_q4k_kernel needs two helper launches around it; each costs about four microseconds of which almost nothing is work.
+// mmq_q4k_coop_kernel does without the first: the workgroups of a K-slice stage the slice's activations together.
+// The unit is one super-block of the image (32 columns x 256 values: 16 KiB of fragments, the sub-block sums and, new,
+// one power-of-two scale per column OF THAT SUPER-BLOCK, so that a unit depends on nothing outside itself): a record
+// of kRecBytes, kRecStride apart in memory (whole 128-byte lines: a record is written by exactly one workgroup).
+//   * Every workgroup converts ONE super-block straight into its LDS: the one it contracts first, j0 = blockIdx.x % nsb.
+//     The workgroups blockIdx.x < nsb also publish theirs: record -> memory with write-through stores, then, once
+//     those stores are acknowledged, a flag word (agent-scope atomic).
+//   * While half of the wavefronts contract super-block j0, the other half (which would otherwise have nothing to
+//     do until its first tile) waits for the flags of the slice's other super-blocks and copies their records global ->
+//     LDS.  One workgroup barrier later the whole image is in LDS and the loop runs as in mmq_q4k_kernel.
+// The flags are never waited for with the data path behind them in doubt: a reader has not touched a record's lines
+// before it sees the flag (caches are invalidated where a kernel starts), and the writer's lines have reached memory.
+// Nothing here needs the workgroups to be resident together: publishers wait for nobody, and workgroups are dispatched
+// in blockIdx order, so a waiting workgroup's publishers are running or done.  Should a flag not appear within
+// `spin_ticks` (100 MHz ticks) all the same, the workgroup converts the missing super-blocks itself (same bits).
+// The reduction launch that follows clears the flags (mmq_reduce_kernel), so replays of a recorded graph work.
+constexpr int kRecTail = kMT * 16 + kMT * 4;       // 640: sub-block sums (16 B per column), inverse scales (fp32 per column)
+constexpr int kRecBytes = 16384 + kRecTail;        // 17024
+constexpr int kRecStride = 17408;                  // 136 lines of 128 bytes
+constexpr int kFlagsPerSlice = 8;
+template <int RT> struct Q4KCoopTile {
+    static_assert(RT == 4, "LDS budget below is for four row tiles");
+    static constexpr int kWaves = RT * kParts, kRows = 32 * RT;
+    static constexpr int kMaxSliceSB = 7;
+    static constexpr int kLds = kMaxSliceSB * kRecBytes + kWaves * kParkBytes;
+    static_assert(kLds <= 160 * 1024, "image + parked tiles exceed LDS");
+};
+
+__device__ __forceinline__ float half_wave_max(float v) {  // over the 32 lanes of a wavefront's half
+#define GQ_DPP_MAX(ctrl) v = fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xF, 0xF, true)))
+    GQ_DPP_MAX(0xB1);   // quad_perm [1,0,3,2]
+    GQ_DPP_MAX(0x4E);   // quad_perm [2,3,0,1]
+    GQ_DPP_MAX(0x141);  // row_half_mirror
+    GQ_DPP_MAX(0x140);  // row_mirror
+#undef GQ_DPP_MAX
+    return fmaxf(v, __shfl_xor(v, 16, 64));
+}
+
+// Super-block `sb` of x (columns m0 .. m0 + 31, values 256 sb .. 256 sb + 255) as one image record in LDS: fragments at
+// `frag` (32 slots x 32 columns x 16 bytes, slot and octet order as in stage_x), sums and inverse scales at `tail`.
+// All 512 threads: thread = (octet tid % 32, columns tid / 32 and tid / 32 + 16); a column's 32 octets sit in one half
+// of a wavefront, so its largest magnitude needs no barrier.
+template <bool BF16X>
+__device__ __forceinline__ void convert_sb(const void *__restrict__ X, int M, int K, int m0, int sb, uint8_t *frag, uint8_t *tail, int tid) {
+    const int oct = tid & 31;
+    const int gp = oct >> 3, w8 = oct & 7, high = w8 >> 2, idx8 = w8 & 3;
+    const int q = high * 2 + (idx8 & 1), c = 2 * gp + (idx8 >> 1);
+    const int slot = c * 4 + q, swz = slot & 15;  // (a super-block is 32 slots: the slice-wide slot index has the same low bits)
+    const int j = 2 * gp + high;
+    const int jpos = (j & 4) | ((j & 1) << 1) | ((j >> 1) & 1);
+    const int64_t k = (int64_t)sb * 256 + 8 * oct;
+    float4 lo[2], hi[2];
+#pragma unroll
+    for (int r = 0; r < 2; r++) load_x8<BF16X>(X, (int64_t)min(m0 + (tid >> 5) + 16 * r, M - 1) * K + k, lo[r], hi[r]);
+#pragma unroll
+    for (int r = 0; r < 2; r++) {
+        const int m = (tid >> 5) + 16 * r;
+        const bool ok = m0 + m < M;
+        float sc, inv;
+        pow2_scale(half_wave_max(ok ? amax8(lo[r], hi[r]) : 0.f), sc, inv);
+        if (oct == 0) reinterpret_cast<float *>(tail + kMT * 16)[m] = inv;
+        const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+        float4 a = ok ? lo[r] : z, b = ok ? hi[r] : z;
+        a.x *= sc; a.y *= sc; a.z *= sc; a.w *= sc; b.x *= sc; b.y *= sc; b.z *= sc; b.w *= sc;
+        uint4 o;  // bytes (0,2,1,3,4,6,5,7)
+        o.x = pack_h2(a.x, a.z);
+        o.y = pack_h2(a.y, a.w);
+        o.z = pack_h2(b.x, b.z);
+        o.w = pack_h2(b.y, b.w);
+        *reinterpret_cast<uint4 *>(frag + slot * (kMT * 16) + (m ^ swz) * 16) = o;
+        float sum = ((a.x + a.y) + (a.z + a.w)) + ((b.x + b.y) + (b.z + b.w));
+        sum = dpp_quad_sum(sum);  // the four octets of one 32-value sub-block sit in one quad
+        if (idx8 == 0) *reinterpret_cast<_Float16 *>(tail + m * 16 + jpos * 2) = (_Float16)sum;
+    }
+}
+
+// 16 bytes to memory, written through the caches (visible to every other workgroup of the chip once acknowledged)
+__device__ __forceinline__ void store_through(void *p, const uint4 &v) {
+    typedef uint32_t Chunk __attribute__((ext_vector_type(4)));
+    const Chunk c = {v.x, v.y, v.z, v.w};
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(c) : "memory");
+}
+
+template <int RT, bool BF16X>
+__global__ __launch_bounds__(64 * RT * kParts) void mmq_q4k_coop_kernel(const void *__restrict__ X, uint8_t *ximg, uint32_t *flags, Q4KSet set,
+                                                                        float *__restrict__ partial0, int M, int K, int64_t row_bytes, int m0,
+                                                                        int slice_sb, const uint8_t *__restrict__ W2, float *__restrict__ partial2,
+                                                                        int spin_ticks) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    __shared__ uint32_t ctl[2];  // [0] wavefronts that have written their part of the published record, [1] super-blocks that did not arrive
+    int prob = 0;
+#pragma unroll
+    for (int j = 1; j < kMaxSet; j++)
+        if (j < set.count && (int)blockIdx.x >= set.wg0[j]) prob = j;
+    const uint8_t *__restrict__ W = blockIdx.z ? W2 : set.W[prob];
+    float *__restrict__ partial = blockIdx.z ? partial2 : partial0;
+    const int N = set.N[prob], xblk = (int)blockIdx.x - set.wg0[prob];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kg = lane >> 5, col = lane & 31;
+    const int rt = wave % RT, par = wave / RT;
+    const int slice = blockIdx.y, nslices = gridDim.y;
+    const int nsb = ((K >> 8) - slice + nslices - 1) / nslices;  // slice s holds super-blocks s, s + nslices, ... of every row
+    const int n = xblk * (32 * RT) + rt * 32 + col;
+    const int mt = m0 / kMT;
+    uint8_t *img = ximg + ((size_t)mt * nslices + slice) * ((size_t)Q4KCoopTile<RT>::kMaxSliceSB * kRecStride);
+    uint32_t *flg = flags + ((size_t)mt * nslices + slice) * kFlagsPerSlice;
+    // the super-block this workgroup stages itself and contracts first; position p of its sequence is super-block (j0 + p) % nsb
+    const int j0 = (int)blockIdx.x % nsb;
+    const bool publisher = blockIdx.z == 0 && (int)blockIdx.x < nsb;
+    auto sb_at = [&](int p) { const int sbl = j0 + p; return sbl >= nsb ? sbl - nsb : sbl; };
+
+    const int xs_off = slice_sb * 16384;  // tails follow the fragments
+    const int row0 = xblk * (32 * RT) + rt * 32;
+    const uint8_t *wtile = W + (int64_t)min(row0, N - 1) * row_bytes + slice * 144;
+    uint32_t csrc[kParkLoads];  // (byte offsets from the first row of the tile: mmq_supported keeps 31 rows below 2^32 bytes)
+#pragma unroll
+    for (int l = 0; l < kParkLoads; l++) {
+        const int c = min(lane + 64 * l, 32 * 9 - 1);
+        csrc[l] = (uint32_t)(min(row0 + c / 9, N - 1) - min(row0, N - 1)) * (uint32_t)row_bytes + (uint32_t)((c % 9) * 16);
+    }
+    uint8_t *park = lds + xs_off + slice_sb * kRecTail + wave * kParkBytes;
+    auto fetch = [&](int sbl) __attribute__((always_inline)) {
+        const uint8_t *base = wtile + sbl * nslices * 144;
+#pragma unroll
+        for (int l = 0; l < kParkLoads; l++)
+            if (64 * l + 64 <= 32 * 9 || lane < 32 * 9 - 64 * l)  // (the last instruction carries 32 chunks)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(base + csrc[l]),
+                                                 (__attribute__((address_space(3))) void *)(park + l * 1024), 16, 0, 0);
+    };
+    if (par < nsb) fetch(sb_at(par));  // the weights of the first tile travel while the activations are staged
+    const uint8_t *myrow = park + col * 144;
+    if (tid == 0) { ctl[0] = 0u; ctl[1] = 0u; }
+    convert_sb<BF16X>(X, M, K, m0, slice + j0 * nslices, lds + j0 * 16384, lds + xs_off + j0 * kRecTail, tid);
+    __syncthreads();  // this workgroup's own super-block is staged
+
+    f16v acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+    uint32_t magic;
+    asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));
+    // position p: wait for the parked tile, pick out this lane's part, request the tile two positions on, contract
+    auto contract_at = [&](int p) __attribute__((always_inline)) {
+        const int sbl = sb_at(p);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+        typedef uint32_t Chunk __attribute__((ext_vector_type(4)));
+        Chunk rhd = *reinterpret_cast<const Chunk *>(myrow), rc[4];
+#pragma unroll
+        for (int st = 0; st < 4; st++) rc[st] = *reinterpret_cast<const Chunk *>(myrow + 16 + 32 * st + 16 * kg);
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(rhd), "+v"(rc[0]), "+v"(rc[1]), "+v"(rc[2]), "+v"(rc[3])::"memory");
+        RawSB cur;
+        cur.hd = make_uint4(rhd.x, rhd.y, rhd.z, rhd.w);
+#pragma unroll
+        for (int st = 0; st < 4; st++) cur.c[st] = make_uint4(rc[st].x, rc[st].y, rc[st].z, rc[st].w);
+        __builtin_amdgcn_wave_barrier();
+        if (p + kParts < nsb) fetch(sb_at(p + kParts));
+        const uint8_t *tail = lds + xs_off + sbl * kRecTail;
+        q4k_contract_sb<true>(cur, lds, tail, reinterpret_cast<const float *>(tail + kMT * 16), sbl, kg, col, magic, acc);
+    };
+
+    if (par == 0) {
+        contract_at(0);
+    } else {
+        if (publisher) {  // the record of super-block j0 goes to memory, a quarter per wavefront
+            for (int c = rt * 64 + lane; c < kRecBytes / 16; c += RT * 64) {
+                const uint8_t *src = c < 1024 ? lds + j0 * 16384 + c * 16 : lds + xs_off + j0 * kRecTail + (c - 1024) * 16;
+                store_through(img + (size_t)j0 * kRecStride + (size_t)c * 16, *reinterpret_cast<const uint4 *>(src));
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stores have been acknowledged
+            if (lane == 0 && atomicAdd(&ctl[0], 1u) == (uint32_t)(RT - 1))  // the last of the four wavefronts raises the flag
+                __hip_atomic_store(flg + j0, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        // the slice's other super-blocks: wait until they are published (bounded), then copy them in
+        const uint32_t want = (1u << nsb) - 1u;
+        uint32_t have;
+        {
+            const unsigned long long t0 = wall_clock64();
+            for (;;) {
+                uint32_t v = 1u;
+                if (lane < nsb && lane != j0) v = __hip_atomic_load(flg + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                have = (uint32_t)__ballot(v != 0u) & want;
+                if (have == want || wall_clock64() - t0 >= (unsigned long long)spin_ticks) break;
+                __builtin_amdgcn_s_sleep(1);
+            }
+        }
+        if (have != want && lane == 0) atomicOr(&ctl[1], want & ~have);
+        asm volatile("" ::: "memory");
+        for (int sbl = 0; sbl < nsb; sbl++) {
+            if (sbl == j0 || !((have >> sbl) & 1u)) continue;
+            const uint8_t *rec = img + (size_t)sbl * kRecStride;
+#pragma unroll
+            for (int i = 0; i < 16 / RT; i++) {  // fragments: 16 KiB, 1 KiB per instruction
+                const int kib = rt + RT * i;
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(rec + kib * 1024 + lane * 16),
+                                                 (__attribute__((address_space(3))) void *)(lds + sbl * 16384 + kib * 1024), 16, 0, 0);
+            }
+            if (rt == 0 && lane < kRecTail / 16)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(rec + 16384 + lane * 16),
+                                                 (__attribute__((address_space(3))) void *)(lds + xs_off + sbl * kRecTail), 16, 0, 0);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (a barrier does not wait for loads in flight)
+    }
+    __syncthreads();  // the image is complete
+    if (const uint32_t missing = ctl[1]) {  // (only after a wait ran out) the workgroup stages what did not arrive itself
+        for (int sbl = 0; sbl < nsb; sbl++)
+            if ((missing >> sbl) & 1u) convert_sb<BF16X>(X, M, K, m0, slice + sbl * nslices, lds + sbl * 16384, lds + xs_off + sbl * kRecTail, tid);
+        __syncthreads();
+    }
+    for (int p = par == 0 ? kParts : par; p < nsb; p += kParts) contract_at(p);
+
+    // wavefronts 1..kParts-1 of a row tile hand their 32 x 32 partial tiles to wavefront 0 through LDS
+    __syncthreads();
+    float *xch = reinterpret_cast<float *>(lds) + rt * ((kParts - 1) * 16 * 64);
+    if (par > 0) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) xch[((par - 1) * 16 + r) * 64 + lane] = acc[r];
+    }
+    __syncthreads();
+    if (par == 0 && n < N) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int m = m0 + 8 * (r >> 2) + 4 * kg + (r & 3);
+            float v = acc[r];
+#pragma unroll
+            for (int p = 0; p < kParts - 1; p++) v += xch[(p * 16 + r) * 64 + lane];
+            if (m < M) partial[((int64_t)slice * M + m) * set.ntot + set.n0[prob] + n] = v;
+        }
+    }
+}
+
 // y[m][n] = act(sum_s partial[s][m][n] + bias[n]); N % 4 == 0 is guaranteed by the caller.  With a second
 // set of partial sums (the other matrix of a gated pair) the result is multiplied by
 // sum_s partial2[s][m][n] + bias2[n]; a residual (which may be Y itself) is added last.
@@ -416,7 +673,10 @@ __global__ __launch_bounds__(64 * RT * kParts) void mmq_q4k_kernel(const uint8_t
 __global__ __launch_bounds__(256) void mmq_reduce_kernel(const float *__restrict__ partial, const float *__restrict__ partial2, int nslices,
                                                          int64_t MN, int N, const float *__restrict__ bias, const float *__restrict__ bias2,
                                                          int act, const float *residual, float *Y, const float *__restrict__ xscale,
-                                                         const float *__restrict__ xss, float eps, float inv_k) {
+                                                         const float *__restrict__ xss, float eps, float inv_k, uint32_t *flags, int nflags) {
+    // (the main kernel that stages the activations itself raised these flags; the stream orders this kernel behind it)
+    if (blockIdx.x == 0)
+        for (int f = threadIdx.x; f < nflags; f += blockDim.x) flags[f] = 0u;
     const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
     if (i >= MN) return;
     const bool small = MN <= (int64_t)INT32_MAX;  // (32-bit divisions are a fraction of the cost of 64-bit ones)
@@ -435,7 +695,7 @@ __global__ __launch_bounds__(256) void mmq_reduce_kernel(const float *__restrict
             for (int j = 0; j < 8; j++) {
                 const int k = min(k0 + j, nslices - 1);
                 v[j] = *reinterpret_cast<const float4 *>(p + (int64_t)k * MN + i);
-                f[j] = xscale[(int64_t)k * M + m];
+                f[j] = xscale ? xscale[(int64_t)k * M + m] : 1.f;  // (no slice scales: the main kernel has applied its own)
                 q[j] = xss ? xss[(int64_t)k * M + m] : 0.f;
             }
 #pragma unroll
@@ -474,14 +734,14 @@ size_t mmq_scale_bytes(int nslices, int64_t M) { return ((size_t)2 * nslices * M
 float *mmq_xss(const float *xscale, int nslices, int64_t M) { return const_cast<float *>(xscale) + (size_t)nslices * M; }
 
 int launch_mmq_reduce(const float *partial, const float *partial2, const float *xscale, int nslices, int64_t M, int64_t K, int64_t N,
-                      const float *bias, int act, float *y, const MmqExtra *ex, hipStream_t s) {
+                      const float *bias, int act, float *y, const MmqExtra *ex, hipStream_t s, uint32_t *flags = nullptr, int nflags = 0) {
     const int64_t MN = M * N;
     const RmsNorm *norm = ex ? ex->norm : nullptr;
     // (workgroups of 64 threads while 256 would leave CUs without one: the kernel is one round trip to memory long)
     const int threads = MN / 4 / 256 >= 2 * device_cu_count() ? 256 : 64;
     return launch(mmq_reduce_kernel, dim3((unsigned)((MN / 4 + threads - 1) / threads)), dim3(threads), 0, s, partial, partial2, nslices, MN, (int)N, bias,
                   ex ? ex->bias2 : nullptr, act, ex ? ex->residual : nullptr, y, xscale, norm ? mmq_xss(xscale, nslices, M) : nullptr,
-                  norm ? norm->eps : 0.f, 1.0f / (float)K);
+                  norm ? norm->eps : 0.f, 1.0f / (float)K, flags, nflags);
 }
 
 
@@ -495,7 +755,9 @@ struct MmqSetOut {
 };
 __global__ __launch_bounds__(256) void mmq_reduce_set_kernel(const float *__restrict__ partial, int nslices, int M, MmqSetOut out,
                                                              const float *__restrict__ xscale, const float *__restrict__ xss, float eps,
-                                                             float inv_k) {
+                                                             float inv_k, uint32_t *flags, int nflags) {
+    if (blockIdx.x == 0)
+        for (int f = threadIdx.x; f < nflags; f += blockDim.x) flags[f] = 0u;
     const int64_t total = (int64_t)M * out.ntot;
     const int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
     if (i >= total) return;
@@ -514,7 +776,7 @@ __global__ __launch_bounds__(256) void mmq_reduce_set_kernel(const float *__rest
         for (int j = 0; j < 8; j++) {
             const int k = min(k0 + j, nslices - 1);
             v[j] = *reinterpret_cast<const float4 *>(partial + (int64_t)k * total + i);
-            f[j] = xscale[(int64_t)k * M + m];
+            f[j] = xscale ? xscale[(int64_t)k * M + m] : 1.f;
             q[j] = xss ? xss[(int64_t)k * M + m] : 0.f;
         }
 #pragma unroll
@@ -1070,6 +1332,22 @@ bool mmq_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, con
 }
 
 namespace {
+// GOMLX_HIPQ_COOP=1 sends the Q4_K split-K route through the kernel that stages the activations itself (two launches
+// instead of three).  It is correct and tested, and it is slower: 24.0 against 20.5 us on a 14336 -> 4096 matrix at 32 rows,
+// because a record travels workgroup -> memory -> flag -> other workgroups in four dependent trips to memory, longer than
+// the pre-pass launch they replace; it stays selectable so that the comparison can be repeated.
+// GOMLX_HIPQ_COOP_SPIN_TICKS=n bounds the wait for published activation records (100 MHz ticks; 0 makes every wait run
+// out at once, which is how the tests reach the path that stages the missing records locally).  Both are read at every call.
+bool coop_enabled() {
+    const char *e = std::getenv("GOMLX_HIPQ_COOP");
+    return e && e[0] == '1';
+}
+int coop_spin_ticks() {
+    const char *e = std::getenv("GOMLX_HIPQ_COOP_SPIN_TICKS");
+    const long v = e ? std::atol(e) : 20000;  // 200 us: a record is published a few microseconds into the kernel
+    return v < 0 ? 0 : v > 100000000 ? 100000000 : (int)v;
+}
+
 // `count` Q4_K matrices against one activation image: the pre-pass once, every matrix's row ranges in one launch of the
 // main kernel, one reduction.  A single matrix may carry the extras (gated pair, residual); a set carries a normalisation only.
 int run_q4k_set(const void *x, bool x_is_bf16, int64_t M, int64_t K, int count, const MmqSetItem *items, const MmqExtra *ex, hipStream_t s) {
@@ -1107,6 +1385,46 @@ int run_q4k_set(const void *x, bool x_is_bf16, int64_t M, int64_t K, int count, 
         }
     }
     const int nslices = (int)((sbs + slice_sb - 1) / slice_sb);
+    const int64_t row_bytes = (K / 256) * 144;
+    const RmsNorm *norm = ex ? ex->norm : nullptr;
+    float *partial2 = nullptr;
+    const dim3 grid((unsigned)rowwgs, (unsigned)nslices, W2 ? 2u : 1u);  // (both matrices of a gated pair in one launch)
+    // Without a normalisation the main kernel stages the activations itself (mmq_q4k_coop_kernel): no pre-pass launch.  It
+    // needs a publisher per super-block of a slice among the row workgroups, and its flags in the workspace's flag words.
+    const int nflags = mtiles * nslices * kFlagsPerSlice;
+    if (!norm && rowwgs >= slice_sb && (size_t)nflags * sizeof(uint32_t) <= kWsSyncBytes && coop_enabled()) {
+        typedef Q4KCoopTile<kQ4KRowTiles> CTile;
+        static const bool coop_lds_ok = [] {
+            return hipFuncSetAttribute(reinterpret_cast<const void *>(mmq_q4k_coop_kernel<kQ4KRowTiles, false>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, CTile::kLds) == hipSuccess &&
+                   hipFuncSetAttribute(reinterpret_cast<const void *>(mmq_q4k_coop_kernel<kQ4KRowTiles, true>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, CTile::kLds) == hipSuccess;
+        }();
+        if (!coop_lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", CTile::kLds);
+        // workspace: [activation records: mtiles x nslices x 7 x kRecStride][partial sums: nslices x M x N fp32, twice for a gated pair]
+        const size_t rec_bytes = (size_t)mtiles * nslices * CTile::kMaxSliceSB * kRecStride;
+        const size_t part_bytes = (size_t)nslices * M * N * sizeof(float);
+        void *ws = nullptr;
+        uint32_t *flags = nullptr;
+        if (int rc = stream_workspace(s, rec_bytes + part_bytes * (W2 ? 2 : 1), &ws, 0, &flags)) return rc;
+        uint8_t *ximg = reinterpret_cast<uint8_t *>(ws);
+        float *partial = reinterpret_cast<float *>(ximg + rec_bytes);
+        partial2 = W2 ? partial + (size_t)nslices * M * N : nullptr;
+        const int spin = coop_spin_ticks();
+        for (int64_t m0 = 0; m0 < M; m0 += kMT) {
+            const int rc = x_is_bf16 ? launch(mmq_q4k_coop_kernel<kQ4KRowTiles, true>, grid, dim3(64 * CTile::kWaves), (size_t)CTile::kLds, s, x, ximg,
+                                              flags, set, partial, (int)M, (int)K, row_bytes, (int)m0, slice_sb, W2, partial2, spin)
+                                     : launch(mmq_q4k_coop_kernel<kQ4KRowTiles, false>, grid, dim3(64 * CTile::kWaves), (size_t)CTile::kLds, s, x, ximg,
+                                              flags, set, partial, (int)M, (int)K, row_bytes, (int)m0, slice_sb, W2, partial2, spin);
+            if (rc) return rc;
+        }
+        if (count == 1)
+            return launch_mmq_reduce(partial, partial2, nullptr, nslices, M, K, N, items[0].bias, items[0].act, items[0].y, ex, s, flags, nflags);
+        const int64_t quads = M * N / 4;
+        const int threads = quads / 256 >= 2 * device_cu_count() ? 256 : 64;
+        return launch(mmq_reduce_set_kernel, dim3((unsigned)((quads + threads - 1) / threads)), dim3(threads), 0, s, (const float *)partial, nslices,
+                      (int)M, out, (const float *)nullptr, (const float *)nullptr, 0.f, 1.0f / (float)K, flags, nflags);
+    }
     // workspace: [activation images: mtiles x nslices x kLdsBytes][slice scales: nslices x M][partial sums: nslices x M x N fp32,
     // twice for a gated pair]
     const size_t img_bytes = (size_t)mtiles * nslices * kLdsBytes;
@@ -1116,8 +1434,6 @@ int run_q4k_set(const void *x, bool x_is_bf16, int64_t M, int64_t K, int count, 
     uint8_t *ximg = reinterpret_cast<uint8_t *>(ws);
     float *xscale = reinterpret_cast<float *>(ximg + img_bytes);
     float *partial = reinterpret_cast<float *>(ximg + img_bytes + mmq_scale_bytes(nslices, M));
-    const int64_t row_bytes = (K / 256) * 144;
-    const RmsNorm *norm = ex ? ex->norm : nullptr;
     // (each workgroup of the pre-pass converts 2 or 4 of a tile's 32 columns: the finer split while it still leaves CUs idle)
     const bool fine = (int64_t)nslices * mtiles * 8 * 2 <= device_cu_count();
     const dim3 pgrid((unsigned)nslices, (unsigned)mtiles, fine ? 16u : 8u);
@@ -1128,8 +1444,7 @@ int run_q4k_set(const void *x, bool x_is_bf16, int64_t M, int64_t K, int count, 
     if (int rc = x_is_bf16 ? (fine ? prep(mmq_xprep_kernel<true, 1>) : prep(mmq_xprep_kernel<true, 2>))
                            : (fine ? prep(mmq_xprep_kernel<false, 1>) : prep(mmq_xprep_kernel<false, 2>)))
         return rc;
-    const dim3 grid((unsigned)rowwgs, (unsigned)nslices, W2 ? 2u : 1u);  // (both matrices of a gated pair in one launch)
-    float *partial2 = W2 ? partial + (size_t)nslices * M * N : nullptr;
+    partial2 = W2 ? partial + (size_t)nslices * M * N : nullptr;
     for (int64_t m0 = 0; m0 < M; m0 += kMT) {
         if (int rc = launch(mmq_q4k_kernel<kQ4KRowTiles>, grid, dim3(64 * Tile::kWaves), (size_t)Tile::kLds, s, (const uint8_t *)ximg, set, partial,
                             (int)M, (int)K, row_bytes, (int)m0, slice_sb, W2, partial2))
@@ -1140,7 +1455,7 @@ int run_q4k_set(const void *x, bool x_is_bf16, int64_t M, int64_t K, int count, 
     const int threads = quads / 256 >= 2 * device_cu_count() ? 256 : 64;
     return launch(mmq_reduce_set_kernel, dim3((unsigned)((quads + threads - 1) / threads)), dim3(threads), 0, s, (const float *)partial, nslices, (int)M,
                   out, (const float *)xscale, (const float *)xss, norm ? norm->eps : 0.f,
-                  1.0f / (float)K);
+                  1.0f / (float)K, (uint32_t *)nullptr, 0);
 }
 }  // namespace
 

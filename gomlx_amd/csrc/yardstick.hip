@@ -124,9 +124,116 @@ __global__ __launch_bounds__(512) void mfma_only_kernel(const uint4 *__restrict_
     if (t == 12345.678f) sink[blockIdx.x * 512 + threadIdx.x] = t;  // (practically never: keeps the instructions alive)
 }
 
+// gqy_mfma_valu: does vector-ALU work fit into the shadow of matrix instructions?  Every wavefront runs `groups` groups of
+// four independent v_mfma_f32_32x32x16_bf16 (4 x 8 passes = 128 cycles of matrix work) plus NV independent vector-ALU
+// instructions per group, either all behind the four matrix instructions (PLACE 0) or NV / 4 behind each of them
+// (PLACE 1).  KIND picks the instruction: 0 v_fma_f32 (three register sources), 1 v_xor_b32 (two), 2 v_cvt_pk_bf16_f32.
+// ACC: the accumulators live in 0 ordinary, 1 accumulation registers (AGPRs).
+// The instruction order is pinned by volatile asm statements.  Every wavefront stamps the shader clock counter and the
+// constant 100 MHz counter around its loop (clocks[(8 wg + wave) * 4 ..]): the span from a workgroup's first start to its
+// last end, in shader cycles per group, is the figure of interest.  Workgroups of 256 threads put one wavefront on each SIMD
+// (128 cycles of matrix work per group), of 512 two (256 cycles; the two do not share a SIMD evenly - the older one
+// finishes first - which is why the span over all wavefronts is taken).  Free vector-ALU work leaves the figure at the
+// matrix cycles; 4 more cycles per instruction mean that nothing overlaps.
+template <int NV, int PLACE, int KIND, int ACC>
+__global__ __launch_bounds__(512) void mfma_valu_kernel(const uint4 *__restrict__ frags, int groups, unsigned long long *__restrict__ clocks,
+                                                        float *__restrict__ sink) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    bf16x8 a[2], b[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        a[i] = __builtin_bit_cast(bf16x8, frags[(wave * 4 + i) * 64 + lane]);
+        b[i] = __builtin_bit_cast(bf16x8, frags[(wave * 4 + 2 + i) * 64 + lane]);
+    }
+    f32x16 acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[i][r] = 0.f;
+    constexpr int NT = 12;  // independent vector-ALU chains (an instruction depends on the one NT before it)
+    float t[NT];
+#pragma unroll
+    for (int i = 0; i < NT; i++) t[i] = 1.0f + (float)(lane + i) * 1e-3f;
+    float c1 = 1.0000001f, c2 = 1e-9f;
+    asm volatile("" : "+v"(c1), "+v"(c2));
+    unsigned long long *stamp = clocks + ((size_t)blockIdx.x * 8 + wave) * 4;
+    if (lane == 0) {
+        stamp[0] = clock64();
+        stamp[1] = wall_clock64();
+    }
+    auto valu = [&](int n) __attribute__((always_inline)) {
+        float &x = t[n % NT];
+        if constexpr (KIND == 0) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(x) : "v"(c1), "v"(c2));
+        else if constexpr (KIND == 1) asm volatile("v_xor_b32 %0, %0, %1" : "+v"(x) : "v"(c2));
+        else asm volatile("v_cvt_pk_bf16_f32 %0, %0, %1" : "+v"(x) : "v"(c1));
+    };
+    for (int g = 0; g < groups; g++) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            if constexpr (ACC == 1) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc[i]) : "v"(a[i & 1]), "v"(b[i >> 1]));
+            else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc[i]) : "v"(a[i & 1]), "v"(b[i >> 1]));
+            if constexpr (PLACE == 1) {
+#pragma unroll
+                for (int n = 0; n < NV / 4; n++) valu(i * (NV / 4) + n);
+            }
+        }
+        if constexpr (PLACE == 0) {
+#pragma unroll
+            for (int n = 0; n < NV; n++) valu(n);
+        }
+    }
+    float r = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int k = 0; k < 16; k++) r += acc[i][k];
+#pragma unroll
+    for (int i = 0; i < NT; i++) r += t[i];
+    if (lane == 0) {
+        stamp[2] = clock64() + (r == 12345.678f ? 1 : 0);
+        stamp[3] = wall_clock64();
+    }
+    if (r == 12345.678f) sink[blockIdx.x * 512 + threadIdx.x] = r;
+}
+
+template <int NV, int PLACE, int ACC>
+int launch_mfma_valu(int kind, const uint4 *frags, int groups, int wgs, int threads, unsigned long long *clocks, float *sink, hipStream_t s) {
+    switch (kind) {
+    case 0: hipLaunchKernelGGL((mfma_valu_kernel<NV, PLACE, 0, ACC>), dim3(wgs), dim3(threads), 0, s, frags, groups, clocks, sink); break;
+    case 1: hipLaunchKernelGGL((mfma_valu_kernel<NV, PLACE, 1, ACC>), dim3(wgs), dim3(threads), 0, s, frags, groups, clocks, sink); break;
+    default: hipLaunchKernelGGL((mfma_valu_kernel<NV, PLACE, 2, ACC>), dim3(wgs), dim3(threads), 0, s, frags, groups, clocks, sink); break;
+    }
+    return (int)hipGetLastError();
+}
+
 }  // namespace
 
 extern "C" {
+
+// nv in {0, 8, 16, 32, 48}; place 0 (behind the group) or 1 (interleaved); kind 0 / 1 / 2 (fma / xor / pack to bf16);
+// acc 0 (accumulators in ordinary registers) or 1 (in accumulation registers); threads 256 (one wavefront per SIMD) or
+// 512 (two).  frags and sink as for gqy_mfma; clocks: 32 x wgs uint64 (four stamps per wavefront).  Returns 0, -1 for bad
+// arguments, or a hipError_t.
+int gqy_mfma_valu(const void *frags, int groups, int wgs, int threads, int nv, int place, int kind, int acc, void *clocks, void *sink, void *stream) {
+    const uint4 *f = static_cast<const uint4 *>(frags);
+    unsigned long long *c = static_cast<unsigned long long *>(clocks);
+    float *k = static_cast<float *>(sink);
+    hipStream_t s = (hipStream_t)stream;
+    if ((threads != 256 && threads != 512) || (place != 0 && place != 1) || kind < 0 || kind > 2 || (acc != 0 && acc != 1)) return -1;
+#define GQY_CASE(NV)                                                                                                              \
+    case NV:                                                                                                                      \
+        if (acc) return place ? launch_mfma_valu<NV, 1, 1>(kind, f, groups, wgs, threads, c, k, s) : launch_mfma_valu<NV, 0, 1>(kind, f, groups, wgs, threads, c, k, s); \
+        return place ? launch_mfma_valu<NV, 1, 0>(kind, f, groups, wgs, threads, c, k, s) : launch_mfma_valu<NV, 0, 0>(kind, f, groups, wgs, threads, c, k, s);
+    switch (nv) {
+        GQY_CASE(0)
+        GQY_CASE(8)
+        GQY_CASE(16)
+        GQY_CASE(32)
+        GQY_CASE(48)
+    default: return -1;
+    }
+#undef GQY_CASE
+}
 
 // frags: 8 wavefronts x 4 fragments x 64 lanes x 16 bytes (32 KiB) of bf16 operands; clocks: 4 x wgs uint64; sink: wgs x 512 floats.
 // Each wavefront issues 4 * groups matrix instructions (2 * 32 * 32 * 16 flop each).  Returns 0 or a hipError_t.

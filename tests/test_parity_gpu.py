@@ -1177,6 +1177,33 @@ def test_config2_q4_k_batch32(gpu, oracle):
     assert rel_err(run_dense(gpu, Q4_K, x, W), oracle.c_qdense(Q4_K, x, W)) < TOL_F32
 
 
+@pytest.mark.parametrize("M,K,N", [(32, 14336, 4096), (9, 4096, 1024), (70, 2048, 896)])
+def test_q4_k_split_k_stages_missing_activation_records_itself(gpu, oracle, M, K, N, monkeypatch):
+    """The Q4_K split-K kernel's workgroups share the staging of the activations through memory and flag words.  With the
+    bound on the wait for those flags at zero every wait runs out at once (forced from the host; the kernel exits normally)
+    and each workgroup stages what it misses itself: the results must be the same bits as with the default bound, and within
+    the bound of the oracle.  bf16 rows as well (widened exactly)."""
+    torch = gpu
+    W = synth.weights(Q4_K, 1302, N, K)
+    x = synth.activations(1303, M, K)
+    want = oracle.c_qdense(Q4_K, x, W)
+    monkeypatch.setenv("GOMLX_HIPQ_COOP", "1")  # (the route is not the default: it measured slower than the three launches)
+    monkeypatch.delenv("GOMLX_HIPQ_COOP_SPIN_TICKS", raising=False)
+    ref = run_dense(torch, Q4_K, x, W)
+    assert rel_err(ref, want) < TOL_F32
+    monkeypatch.setenv("GOMLX_HIPQ_COOP_SPIN_TICKS", "0")
+    for _ in range(2):
+        assert np.array_equal(run_dense(torch, Q4_K, x, W).view(np.uint32), ref.view(np.uint32))
+    xb = bf16_round(x)
+    got_b = run_dense(torch, Q4_K, xb, W, bf16=True)
+    monkeypatch.delenv("GOMLX_HIPQ_COOP_SPIN_TICKS")
+    assert np.array_equal(run_dense(torch, Q4_K, xb, W, bf16=True).view(np.uint32), got_b.view(np.uint32))
+    assert rel_err(got_b, oracle.c_qdense(Q4_K, xb, W)) < TOL_F32
+    # the three-launch route (separate pre-pass) agrees to rounding: its activations carry one scale per slice, not per super-block
+    monkeypatch.delenv("GOMLX_HIPQ_COOP")
+    assert rel_err(run_dense(torch, Q4_K, x, W), want) < TOL_F32
+
+
 def test_config3_q8_0_prefill_bf16(gpu, oracle):
     W = synth.weights(Q8_0, 1000, 4096, 4096)
     x = bf16_round(synth.activations(1003, 2048, 4096))
