@@ -111,6 +111,8 @@ def parse_args():
     p.add_argument("--matmul-yardstick", action="store_true",
                    help="instead of the benchmark, time the vendor library's plain bf16 GEMM (torch.matmul) on C3's shape, 2048 x 4096 x 4096: "
                         "what a 16-bit GEMM with no dequantisation reaches on this chip")
+    p.add_argument("--l2-yardstick", action="store_true",
+                   help="only measure how fast the L2 caches hand one small shared buffer to every workgroup (three access patterns)")
     p.add_argument("--mfma-valu-yardstick", action="store_true",
                    help="only measure how many vector-ALU instructions fit into the shadow of matrix instructions (cycles per group)")
     p.add_argument("--mfma-yardstick", action="store_true",
@@ -710,6 +712,56 @@ def mfma_yardstick(torch, steps, only_first=False):
     return out
 
 
+def l2_yardstick(torch, steps=50):
+    """How fast the L2 caches hand ONE small buffer to every workgroup at once (gomlx_amd/csrc/yardstick.hip, gqy_read_shared /
+    gqy_read_streams): what a small-batch kernel pays that streams the whole activation image (0.9 MB of fp16 fragments for 32
+    columns at K = 14336) past every workgroup instead of splitting K.  Three ways to read 56 records of 16 KiB in each of 256
+    workgroups of 512 threads: the workgroup walks the buffer together; every wavefront walks its own records (w, w + 8, ...) with
+    ordinary loads, 16 KiB in flight per wavefront; the same by LDS DMA through a ring of four 4 KiB slots per wavefront (12 KiB
+    in flight).  HIP events around `steps` launches."""
+    ys = yardstick()
+    if ys is None:
+        return None
+    vp = ctypes.c_void_p
+    ys.lib.gqy_read_streams.argtypes = [vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp]
+    ys.lib.gqy_read_streams.restype = ctypes.c_int
+    ys.lib.gqy_read_shared.argtypes = [vp, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp]
+    ys.lib.gqy_read_shared.restype = ctypes.c_int
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    st = torch.cuda.Stream()
+    sink = torch.zeros(2048 * 1024, dtype=torch.int32, device="cuda")
+    records, rec = 56, 16384
+    buf = torch.randint(0, 255, (records * rec,), dtype=torch.uint8, device="cuda")
+    cases = {
+        "workgroup walks the buffer together (ordinary loads, 8 per thread in flight)":
+            lambda: ys.lib.gqy_read_shared(buf.data_ptr(), records * rec, cus, 512, 1, sink.data_ptr(), st.cuda_stream),
+        "one stream of records per wavefront, ordinary loads (16 KiB in flight per wavefront)":
+            lambda: ys.lib.gqy_read_streams(buf.data_ptr(), records, rec, cus, 0, sink.data_ptr(), st.cuda_stream),
+        "one stream of records per wavefront, LDS DMA ring (12 KiB in flight per wavefront)":
+            lambda: ys.lib.gqy_read_streams(buf.data_ptr(), records, rec, cus, 1, sink.data_ptr(), st.cuda_stream),
+    }
+    out = {"l2_yardstick": f"{cus} workgroups x 512 threads each read the same {records * rec} bytes", "cases": {}}
+    total = records * rec * cus
+    for label, fn in cases.items():
+        with torch.cuda.stream(st):
+            for _ in range(3):
+                if fn():
+                    raise RuntimeError("yardstick launch failed")
+            torch.cuda.synchronize()
+            best = None
+            for _ in range(3):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(st)
+                for _ in range(steps):
+                    fn()
+                e1.record(st)
+                torch.cuda.synchronize()
+                us = e0.elapsed_time(e1) * 1e3 / steps
+                best = us if best is None else min(best, us)
+        out["cases"][label] = {"us_per_launch": best, "tb_per_s_out_of_l2": total / best / 1e6, "bytes_per_clock_per_cu_at_2400mhz": total / cus / best / 2400.0}
+    return out
+
+
 def mfma_valu_yardstick(torch, groups=512):
     """Vector-ALU instructions in the shadow of matrix instructions (gomlx_amd/csrc/yardstick.hip, gqy_mfma_valu): shader cycles
     per group of four independent v_mfma_f32_32x32x16_bf16 per wavefront plus NV independent vector-ALU instructions, placed
@@ -777,6 +829,13 @@ def main():
         return
     if args.matmul_yardstick:
         print(json.dumps(matmul_yardstick(torch, min(args.steps, 50))))
+        return
+    if args.l2_yardstick:
+        out = l2_yardstick(torch)
+        if out is None:
+            print("bench.py: gomlx_amd/libgq_yardstick.so is missing (python -m gomlx_amd.build)", file=sys.stderr)
+            sys.exit(4)
+        print(json.dumps(out))
         return
     if args.mfma_valu_yardstick:
         out = mfma_valu_yardstick(torch)

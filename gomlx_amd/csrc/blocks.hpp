@@ -217,6 +217,14 @@ __device__ __forceinline__ float wave_max(float v) {
     return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
 }
 
+// 16 bytes to memory, written through the caches: once the store is acknowledged (s_waitcnt vmcnt) every other workgroup
+// of the chip that has not read the line before in this kernel reads the new bytes.
+__device__ __forceinline__ void store_through(void *p, const uint4 &v) {
+    typedef uint32_t Chunk __attribute__((ext_vector_type(4)));
+    const Chunk c = {v.x, v.y, v.z, v.w};
+    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(c) : "memory");
+}
+
 __device__ __forceinline__ float apply_act(int act, float v) {
     switch (act) {
     case kActRelu: return fmaxf(v, 0.0f);

@@ -28,6 +28,7 @@
 #include "common.hpp"
 
 #include <cstdlib>
+#include <type_traits>
 
 namespace gq {
 
@@ -510,13 +511,6 @@ __device__ __forceinline__ void convert_sb(const void *__restrict__ X, int M, in
         sum = dpp_quad_sum(sum);  // the four octets of one 32-value sub-block sit in one quad
         if (idx8 == 0) *reinterpret_cast<_Float16 *>(tail + m * 16 + jpos * 2) = (_Float16)sum;
     }
-}
-
-// 16 bytes to memory, written through the caches (visible to every other workgroup of the chip once acknowledged)
-__device__ __forceinline__ void store_through(void *p, const uint4 &v) {
-    typedef uint32_t Chunk __attribute__((ext_vector_type(4)));
-    const Chunk c = {v.x, v.y, v.z, v.w};
-    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(c) : "memory");
 }
 
 template <int RT, bool BF16X>
@@ -1332,6 +1326,12 @@ bool mmq_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, con
 }
 
 namespace {
+// GOMLX_HIPQ_COOP=1 sends the Q4_K split-K route through the kernel that stages the activations itself (two launches
+// instead of three).  It is correct and tested, and it is slower: 24.0 against 20.5 us on a 14336 -> 4096 matrix at 32 rows,
+// because a record travels workgroup -> memory -> flag -> other workgroups in four dependent trips to memory, longer than
+// the pre-pass launch they replace; it stays selectable so that the comparison can be repeated.
+// GOMLX_HIPQ_COOP_SPIN_TICKS=n bounds the wait for published activation records (100 MHz ticks; 0 makes every wait run
+// out at once, which is how the tests reach the path that stages the missing records locally).  Both are read at every call.
 // GOMLX_HIPQ_COOP=1 sends the Q4_K split-K route through the kernel that stages the activations itself (two launches
 // instead of three).  It is correct and tested, and it is slower: 24.0 against 20.5 us on a 14336 -> 4096 matrix at 32 rows,
 // because a record travels workgroup -> memory -> flag -> other workgroups in four dependent trips to memory, longer than

@@ -45,6 +45,80 @@ __global__ __launch_bounds__(1024) void read_linear_kernel(const uint4 *__restri
     if (acc == 0x9E3779B9u) out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = acc;  // (practically never: keeps the loads alive)
 }
 
+// Every workgroup reads ALL of a (small, cache-resident) buffer: the rate at which the L2 caches hand the same lines to all
+// CUs at once, which is what a kernel pays that streams a shared operand past every workgroup.  DEPTH loads in flight per thread.
+template <int DEPTH>
+__global__ __launch_bounds__(1024) void read_shared_kernel(const uint4 *__restrict__ p, size_t chunks, int passes, uint32_t *__restrict__ out) {
+    uint32_t acc = 0;
+    for (int pass = 0; pass < passes; pass++) {
+        size_t i = threadIdx.x;
+        for (; i + (DEPTH - 1) * blockDim.x < chunks; i += DEPTH * blockDim.x) {
+            uint4 v[DEPTH];
+#pragma unroll
+            for (int j = 0; j < DEPTH; j++) v[j] = p[i + j * blockDim.x];
+#pragma unroll
+            for (int j = 0; j < DEPTH; j++) acc ^= v[j].x ^ v[j].y ^ v[j].z ^ v[j].w;
+        }
+        asm volatile("" : "+v"(acc));
+    }
+    if (acc == 0x9E3779B9u) out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = acc;
+}
+
+// The same shared buffer read the way a kernel with one stream per wavefront reads it: wavefront w of each workgroup takes
+// the records w, w + 8, ... (`rec_bytes` each, a multiple of 4 KiB) and walks through them in 4 KiB pieces, three pieces in flight.
+// DMA = false: ordinary 16-byte loads into registers; DMA = true: the same bytes by LDS DMA into a ring of four 4 KiB slots
+// per wavefront (the way the small-batch kernels stage their activation image).  What differs between the two is the price
+// of the LDS path alone.
+template <bool DMA>
+__global__ __launch_bounds__(512) void read_streams_kernel(const uint8_t *__restrict__ p, int records, int rec_bytes, uint32_t *__restrict__ out) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t ring_lds[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int pieces_per_rec = rec_bytes / 4096;
+    const int my_recs = (records - wave + 7) / 8;
+    const int total = my_recs * pieces_per_rec;  // pieces of this wavefront
+    uint32_t acc = 0;
+    auto piece_ptr = [&](int i) { return p + (size_t)(wave + 8 * (i / pieces_per_rec)) * rec_bytes + (size_t)(i % pieces_per_rec) * 4096 + lane * 16; };
+    if constexpr (DMA) {
+        uint8_t *ring = ring_lds + wave * 16384;
+        auto issue = [&](int i) {
+            const uint8_t *src = piece_ptr(i);
+#pragma unroll
+            for (int k = 0; k < 4; k++)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(src + k * 1024),
+                                                 (__attribute__((address_space(3))) void *)(ring + (i & 3) * 4096 + k * 1024), 16, 0, 0);
+        };
+        for (int i = 0; i < 3 && i < total; i++) issue(i);
+        for (int i = 0; i < total; i++) {
+            if (i + 3 < total) {
+                issue(i + 3);
+                asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+            } else {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            }
+            const uint4 v = *reinterpret_cast<const uint4 *>(ring + (i & 3) * 4096 + lane * 16);
+            acc ^= v.x ^ v.y ^ v.z ^ v.w;
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        }
+    } else {
+        uint4 v[4][4];
+        auto issue = [&](int i, int slot) {
+            const uint8_t *src = piece_ptr(i);
+#pragma unroll
+            for (int k = 0; k < 4; k++) v[slot][k] = *reinterpret_cast<const uint4 *>(src + k * 1024);
+        };
+        // (whole groups of four pieces keep the slots compile-time: records are 4 or 16 KiB multiples in the uses here)
+        for (int i0 = 0; i0 < total; i0 += 4) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) issue(min(i0 + j, total - 1), j);
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int k = 0; k < 4; k++) acc ^= v[j][k].x ^ v[j][k].y ^ v[j][k].z ^ v[j][k].w;
+        }
+    }
+    if (acc == 0x9E3779B9u) out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = acc;
+}
+
 // grid (N / 128, slices); 512 threads: wavefront = (row tile of 32, half of the slice's super-blocks), all loads up front
 template <bool COALESCED>
 __global__ __launch_bounds__(512) void read_q4k_tiles_kernel(const uint8_t *__restrict__ W, int N, int64_t row_bytes, int slice_sb, int sbs,
@@ -240,6 +314,28 @@ int gqy_mfma_valu(const void *frags, int groups, int wgs, int threads, int nv, i
 int gqy_mfma(const void *frags, int groups, int wgs, void *clocks, void *sink, void *stream) {
     hipLaunchKernelGGL(mfma_only_kernel, dim3(wgs), dim3(512), 0, (hipStream_t)stream, static_cast<const uint4 *>(frags), groups,
                        static_cast<unsigned long long *>(clocks), static_cast<float *>(sink));
+    return (int)hipGetLastError();
+}
+
+// Every one of `wgs` workgroups of `threads` threads reads the whole buffer `passes` times, 8 loads in flight per thread.
+int gqy_read_shared(const void *p, size_t bytes, int wgs, int threads, int passes, void *out, void *stream) {
+    hipLaunchKernelGGL(read_shared_kernel<8>, dim3(wgs), dim3(threads), 0, (hipStream_t)stream, static_cast<const uint4 *>(p), bytes / 16, passes,
+                       static_cast<uint32_t *>(out));
+    return (int)hipGetLastError();
+}
+
+// Every one of `wgs` workgroups (512 threads) reads `records` records of rec_bytes, one stream per wavefront; dma 0 / 1.
+int gqy_read_streams(const void *p, int records, int rec_bytes, int wgs, int dma, void *out, void *stream) {
+    if (rec_bytes % 4096 != 0 || records < 8) return -1;
+    if (dma) {
+        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(read_streams_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, 8 * 16384);
+        if (attr != hipSuccess) return (int)attr;
+        hipLaunchKernelGGL(read_streams_kernel<true>, dim3(wgs), dim3(512), 8 * 16384, (hipStream_t)stream, static_cast<const uint8_t *>(p), records, rec_bytes,
+                           static_cast<uint32_t *>(out));
+    } else {
+        hipLaunchKernelGGL(read_streams_kernel<false>, dim3(wgs), dim3(512), 0, (hipStream_t)stream, static_cast<const uint8_t *>(p), records, rec_bytes,
+                           static_cast<uint32_t *>(out));
+    }
     return (int)hipGetLastError();
 }
 
