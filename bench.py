@@ -96,6 +96,9 @@ def parse_args():
     p.add_argument("--no-graph", action="store_true", help="submit the timed steps one call at a time")
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     p.add_argument("--no-extras", action="store_true", help="skip the cache-resident pass, the plain-read yardstick and the clock sampling")
+    p.add_argument("--ablation", default=None,
+                   help="time a TIMING-ONLY variant of the fused GEMM (python -m gomlx_amd.ablate build NAME first) instead of the product "
+                        "library: its results are wrong on purpose, the line says so, and only --config c3 --no-cpu makes sense with it")
     p.add_argument("--hot", action="store_true", help="single weight buffer (Infinity-Cache resident) for the main measurement as well")
     p.add_argument("--copy-calibration", action="store_true",
                    help="instead of the benchmark, run a plain 64 MiB device-to-device copy kernel --steps times: the known-size "
@@ -852,6 +855,12 @@ def main():
         print(json.dumps(out))
         return
     from gomlx_amd import _lib
+    if args.ablation:
+        from gomlx_amd import ablate
+        if args.ablation not in ablate.VARIANTS or not os.path.exists(ablate.lib_path(args.ablation)):
+            print(f"bench.py: no built ablation {args.ablation!r}: python -m gomlx_amd.ablate build [{' | '.join(ablate.VARIANTS)}]", file=sys.stderr)
+            sys.exit(4)
+        _lib.use_library(ablate.lib_path(args.ablation))
     _lib.init(0)
 
     def measure(name, steps):
@@ -906,6 +915,11 @@ def main():
         "roofline": rep["roofline"],
         "clock_state": rep.get("clock_state"),
     }
+    if args.ablation:
+        from gomlx_amd import ablate
+        line["ablation"] = {"name": args.ablation, "taken_out": ablate.VARIANTS[args.ablation][0],
+                            "note": "TIMING ONLY: this library computes wrong results on purpose; the line is not a benchmark result"}
+        line["metric"] = "ablation timing (not a result): " + line["metric"]
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(args.config)
         line["cpu_baseline"]["reference_toolchain"] = reference_toolchain()

@@ -11,6 +11,15 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libgomlx_hipq.so")
 
+
+def use_library(path: str) -> None:
+    """Loads `path` instead of the in-tree product library; only before the first call of lib().  For the benchmark's
+    timing-only ablation builds, which export the same symbols."""
+    global LIB_PATH
+    if _lib is not None:
+        raise RuntimeError("the library is already loaded")
+    LIB_PATH = path
+
 OK, ERR_INVALID, ERR_NOT_IMPLEMENTED, ERR_HIP, ERR_NO_DEVICE, ERR_OOM = range(6)
 F32, BF16 = 0, 1
 
