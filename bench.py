@@ -97,8 +97,9 @@ def parse_args():
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     p.add_argument("--no-extras", action="store_true", help="skip the cache-resident pass, the plain-read yardstick and the clock sampling")
     p.add_argument("--ablation", default=None,
-                   help="time a TIMING-ONLY variant of the fused GEMM (python -m gomlx_amd.ablate build NAME first) instead of the product "
-                        "library: its results are wrong on purpose, the line says so, and only --config c3 --no-cpu makes sense with it")
+                   help="time a TIMING-ONLY variant of the fused GEMM (gemm_*: --config c3) or of the Q4_K split-K route (q4k_*: --config c2) "
+                        "instead of the product library (python -m gomlx_amd.ablate build NAME first): its results are wrong on purpose and the "
+                        "line says so")
     p.add_argument("--hot", action="store_true", help="single weight buffer (Infinity-Cache resident) for the main measurement as well")
     p.add_argument("--copy-calibration", action="store_true",
                    help="instead of the benchmark, run a plain 64 MiB device-to-device copy kernel --steps times: the known-size "
@@ -917,7 +918,7 @@ def main():
     }
     if args.ablation:
         from gomlx_amd import ablate
-        line["ablation"] = {"name": args.ablation, "taken_out": ablate.VARIANTS[args.ablation][0],
+        line["ablation"] = {"name": args.ablation, "taken_out": ablate.VARIANTS[args.ablation][1],
                             "note": "TIMING ONLY: this library computes wrong results on purpose; the line is not a benchmark result"}
         line["metric"] = "ablation timing (not a result): " + line["metric"]
     if not args.no_cpu:

@@ -1,10 +1,12 @@
-"""Timing-only ablations of the fused dequantise-in-LDS GEMM (csrc/gemm.hip).
+"""Timing-only ablations of the fused dequantise-in-LDS GEMM (csrc/gemm.hip; names gemm_*, timed on --config c3)
+and of the Q4_K split-K route (csrc/mmq.hip; names q4k_*, timed on --config c2) and of the decode GEMV (csrc/gemv_ks_body.hpp; names ks_*, timed on
+--config c0 / c1: single calls only, the batched and extended kernels live in other units).
 
-Each variant is the shipped source with one part of a K step taken out by exact text substitution (the
-substitution fails loudly when the source has moved on), compiled and linked with the product's other
-objects into ``gomlx_amd/libgomlx_hipq_ablate_<name>.so``.  The variants compute WRONG results on purpose:
-they exist to show, by the time that disappears with a part, what that part costs inside the running
-kernel.  ``bench.py --ablation <name> --config c3`` times one; nothing else loads them.
+Each variant is the shipped source with one part taken out by exact text substitution (the substitution
+fails loudly when the source has moved on), compiled and linked with the product's other objects into
+``gomlx_amd/libgomlx_hipq_ablate_<name>.so``.  The variants compute WRONG results on purpose: they exist
+to show, by the time that disappears with a part, what that part costs inside the running kernel.
+``bench.py --ablation <name> --config c3|c2`` times one; nothing else loads them.
 
     python -m gomlx_amd.ablate build [name ...]     # default: all
     python -m gomlx_amd.ablate clean
@@ -57,17 +59,61 @@ def _block(store_x=True, part_w=True, load_x=True):
     return (_BLOCK, (_STORE_X if store_x else "") + (_PART_W if part_w else "") + (_LOAD_X if load_x else ""))
 
 
-# name: (what is taken out of the K loop, [(old, new), ...])
+_Q4K_IMAGE = """            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(img + i * 1024 + lane * 16),
+                                             (__attribute__((address_space(3))) void *)(lds + i0 * 1024), 16, 0, 0);
+"""
+_Q4K_FETCH0 = "    if (par < nsb) fetch(par);\n"
+_Q4K_FETCH = "        if (sbl + kParts < nsb) fetch(sbl + kParts);\n"
+_Q4K_CONTRACT = "        q4k_contract_sb<false>(cur, lds, lds + xs_off + sbl * (kMT * 16), nullptr, sbl, kg, col, magic, acc);\n"
+_Q4K_KEEP = '        asm volatile("" ::"v"(cur.hd.x), "v"(cur.c[0].x), "v"(cur.c[1].x), "v"(cur.c[2].x), "v"(cur.c[3].x), "v"(magic));\n'
+_Q4K_XPREP = """    if (int rc = x_is_bf16 ? (fine ? prep(mmq_xprep_kernel<true, 1>) : prep(mmq_xprep_kernel<true, 2>))
+                           : (fine ? prep(mmq_xprep_kernel<false, 1>) : prep(mmq_xprep_kernel<false, 2>)))
+        return rc;
+"""
+_Q4K_REDUCE = "    if (count == 1) return launch_mmq_reduce(partial, partial2, xscale, nslices, M, K, N, items[0].bias, items[0].act, items[0].y, ex, s);\n"
+
+_KS_STAGE = "                const Staged st = KS<T>::stage(p);\n"
+_KS_NO_STAGE = """                Staged st;
+                st.planes = make_uint4(__builtin_bit_cast(uint32_t, p.lo.x), __builtin_bit_cast(uint32_t, p.lo.y), __builtin_bit_cast(uint32_t, p.hi.x), __builtin_bit_cast(uint32_t, p.hi.y));
+                st.scale = p.lo.z;
+                st.sum = p.hi.z;
+"""
+_KS_DOT = "                for (int q = 0; q < R; q++) d[q] = KS<T>::dot(buf[jj], xq[q], xsc[q], xsm[q], c);\n"
+_KS_NO_DOT = """                for (int q = 0; q < R; q++) {
+                    const uint32_t *raw = reinterpret_cast<const uint32_t *>(&buf[jj]);
+                    for (unsigned i = 0; i < sizeof(Raw) / 4; i++) asm volatile("" ::"v"(raw[i]));
+                    d[q] = __builtin_bit_cast(float, xq[q][0].x ^ xq[q][7].w) + xsc[q][0] + xsm[q][0];
+                }
+"""
+_KS_EPILOGUE = "    const int rows_out = dual ? rows_wg >> 1 : live * 8;\n"
+_KS_NO_EPILOGUE = "    const int rows_out = (dual ? rows_wg >> 1 : live * 8) * (N < 0 ? 1 : 0);\n"
+_KS_XFETCH = "            else KS<T>::x_fetch(reinterpret_cast<const float *>(xrow) + sl * kSliceValues, xl, r.a[i], r.b[i]);\n"
+_KS_NO_XFETCH = "            else { r.a[i] = make_uint4(lane, sl, 3, 4); r.b[i] = make_uint4(5, 6, 7, xl); }\n"
+
+# name: (source file, what is taken out, [(old, new), ...]) - or (unit, what, subs, edited header) when the text
+# lives in a header that the unit includes
 VARIANTS = {
-    "no_convert": ("the int8 -> float arithmetic of the Q8_0 weights (bytes are passed on as bit patterns)", [(_CONVERT, _NO_CONVERT)]),
-    "no_x_staging": ("activation loads and LDS stores", [_block(store_x=False, load_x=False)]),
-    "no_x_stores": ("activation LDS stores (loads kept)", [_block(store_x=False)]),
-    "no_x_loads": ("activation global loads (stores kept)", [_block(load_x=False)]),
-    "no_w_staging": ("weight loads, conversion and LDS stores", [_block(part_w=False), (_STORE_W, ""), (_LOAD_W, _NO_LOAD_W)]),
-    "no_w_loads": ("weight global loads (conversion and stores kept)", [(_LOAD_W, _NO_LOAD_W)]),
-    "no_w_stores": ("weight LDS stores (loads and conversion kept)", [(_STORE_W, _KEEP_W)]),
-    "no_staging": ("all staging: the loop is LDS fragment reads, MFMAs and barriers",
-                   [_block(False, False, False), (_STORE_W, ""), (_LOAD_W, _NO_LOAD_W)]),
+    "gemm_no_convert": ("gemm.hip", "the int8 -> float arithmetic of the Q8_0 weights (bytes are passed on as bit patterns)", [(_CONVERT, _NO_CONVERT)]),
+    "gemm_no_x_staging": ("gemm.hip", "activation loads and LDS stores", [_block(store_x=False, load_x=False)]),
+    "gemm_no_x_stores": ("gemm.hip", "activation LDS stores (their loads are then dead code and go too)", [_block(store_x=False)]),
+    "gemm_no_x_loads": ("gemm.hip", "activation global loads (stores kept)", [_block(load_x=False)]),
+    "gemm_no_w_staging": ("gemm.hip", "weight loads, conversion and LDS stores", [_block(part_w=False), (_STORE_W, ""), (_LOAD_W, _NO_LOAD_W)]),
+    "gemm_no_w_loads": ("gemm.hip", "weight global loads (conversion and stores kept)", [(_LOAD_W, _NO_LOAD_W)]),
+    "gemm_no_w_stores": ("gemm.hip", "weight LDS stores (loads and conversion kept)", [(_STORE_W, _KEEP_W)]),
+    "gemm_no_staging": ("gemm.hip", "all staging: the loop is LDS fragment reads, MFMAs and barriers",
+                        [_block(False, False, False), (_STORE_W, ""), (_LOAD_W, _NO_LOAD_W)]),
+    "ks_no_convert": ("gemv_ks.hip", "the conversion of the activations to fixed-point planes (loads and the LDS exchange kept)",
+                      [(_KS_STAGE, _KS_NO_STAGE)], "gemv_ks_body.hpp"),
+    "ks_no_x": ("gemv_ks.hip", "activation loads and their conversion (the LDS exchange of constants kept)",
+                [(_KS_STAGE, _KS_NO_STAGE), (_KS_XFETCH, _KS_NO_XFETCH)], "gemv_ks_body.hpp"),
+    "ks_no_dot": ("gemv_ks.hip", "the integer dot products (weight loads kept)", [(_KS_DOT, _KS_NO_DOT)], "gemv_ks_body.hpp"),
+    "ks_no_epilogue": ("gemv_ks.hip", "the sum over the workgroup's wavefronts and the stores of y (the barrier stays)",
+                       [(_KS_EPILOGUE, _KS_NO_EPILOGUE)], "gemv_ks_body.hpp"),
+    "q4k_no_image": ("mmq.hip", "the copy of the slice's activation image into LDS (main kernel)", [(_Q4K_IMAGE, "            (void)img;\n")]),
+    "q4k_no_weights": ("mmq.hip", "the weight loads of the main kernel (it contracts whatever LDS holds)", [(_Q4K_FETCH0, ""), (_Q4K_FETCH, "")]),
+    "q4k_no_contract": ("mmq.hip", "unpacking and MFMAs of the main kernel (loads and LDS reads kept)", [(_Q4K_CONTRACT, _Q4K_KEEP)]),
+    "q4k_no_xprep": ("mmq.hip", "the activation pre-pass launch", [(_Q4K_XPREP, "    (void)prep;\n")]),
+    "q4k_no_reduce": ("mmq.hip", "the reduction launch", [(_Q4K_REDUCE, "    if (count == 1) return GQ_OK;\n")]),
 }
 
 
@@ -76,10 +122,13 @@ def lib_path(name: str) -> str:
 
 
 def variant_source(name: str) -> str:
-    text = open(os.path.join(B.CSRC, "gemm.hip")).read()
-    for old, new in VARIANTS[name][1]:
+    """The edited text of the variant's file (the unit itself, or the header named as fourth entry)."""
+    v = VARIANTS[name]
+    src = v[3] if len(v) > 3 else v[0]
+    text = open(os.path.join(B.CSRC, src)).read()
+    for old, new in VARIANTS[name][2]:
         if text.count(old) != 1:
-            raise RuntimeError(f"ablation {name}: expected exactly one occurrence in gemm.hip of:\n{old}")
+            raise RuntimeError(f"ablation {name}: expected exactly one occurrence in {src} of:\n{old}")
         text = text.replace(old, new)
     return text
 
@@ -87,17 +136,29 @@ def variant_source(name: str) -> str:
 def build_variant(name: str) -> str:
     out_dir = os.path.join(B.OBJ, "ablate")
     os.makedirs(out_dir, exist_ok=True)
-    src = os.path.join(out_dir, f"gemm_{name}.hip")
-    with open(src, "w") as f:
-        f.write(variant_source(name))
-    obj = os.path.join(out_dir, f"gemm_{name}.o")
+    v = VARIANTS[name]
+    src = os.path.join(out_dir, f"{name}.hip")
+    if len(v) > 3:
+        # the edited header goes into a directory of its own beside a copy of the unit: an #include "..." looks beside
+        # the including file first
+        out_dir = os.path.join(out_dir, name)
+        os.makedirs(out_dir, exist_ok=True)
+        src = os.path.join(out_dir, v[0])
+        with open(os.path.join(out_dir, v[3]), "w") as f:
+            f.write(variant_source(name))
+        with open(src, "w") as f:
+            f.write(open(os.path.join(B.CSRC, v[0])).read())
+    else:
+        with open(src, "w") as f:
+            f.write(variant_source(name))
+    obj = os.path.join(out_dir, f"{name}.o")
     flags = [f for f in B.HIPCC_FLAGS if not f.startswith("-Rpass")]
     r = subprocess.run([B.hipcc(), *flags, "-I", B.CSRC, "-c", src, "-o", obj], capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed for ablation {name}:\n{r.stderr}")
     others = []
     for s in B.SOURCES:
-        if s == "gemm.hip":
+        if s == VARIANTS[name][0]:
             continue
         o = os.path.join(B.OBJ, os.path.splitext(s)[0] + ".o")
         if not os.path.exists(o):
@@ -118,7 +179,7 @@ def main(argv):
         sys.stderr.write(__doc__)
         return 2
     for name in argv[1:] or list(VARIANTS):
-        print("built", build_variant(name), "--", "without", VARIANTS[name][0])
+        print("built", build_variant(name), "--", "without", VARIANTS[name][1])
     return 0
 
 
