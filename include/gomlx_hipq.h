@@ -110,7 +110,8 @@ int gq_qdense_f32(int type, const float *dX, int64_t M, int64_t K, const void *d
  * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same
  * arguments, same kernels and bit-identical results; the scratch memory that batches of 5 rows and
  * more use (activation image, split-K partial sums) is a fixed 16 MiB device array inside the library
- * instead of a per-stream workspace, and the call makes no hipMalloc / hipFree at all.  A problem
+ * instead of a per-stream workspace (its first 4 KiB are the flag words every workspace starts with:
+ * 16 MiB - 4 KiB serve the call), and the call makes no hipMalloc / hipFree at all.  A problem
  * that needs more scratch than that (the two-pass GEMM's 16-bit weight image of a large matrix, or
  * about M * N * K / 2048 > 3.5 Mi for the split-K kernels) fails with GQ_ERR_INVALID and a message
  * naming the size; nothing is launched then.  Every call on a GPU shares that GPU's array: calls
