@@ -157,6 +157,42 @@ func (f *Function) FusedQuantizedDense(x, weights, bias compute.Value, wq *compu
 	return f.register(n), nil
 }
 
+// QuantizedEmbeddingLookup validates at graph-build time and records the node
+// (core/graph/fused_ops.go:295-296; shapes as in ml/ggml/gather.go:21-49: table Uint8 [vocab, bytesPerRow],
+// indices an integer tensor whose last dimension is 1, output Float32 [batch..., K]).
+func (f *Function) QuantizedEmbeddingLookup(table, indices compute.Value, tq *compute.Quantization) (compute.Value, error) {
+	if tq == nil {
+		return nil, errors.New("hipq: QuantizedEmbeddingLookup: tq must not be nil")
+	}
+	if tq.Scheme != compute.QuantGGML {
+		return nil, errors.Wrap(compute.ErrNotImplemented, "hipq: only the GGML scheme runs on the GPU")
+	}
+	tn, in := f.node(table), f.node(indices)
+	if tn.shape.DType != dtypes.Uint8 || tn.shape.Rank() != 2 {
+		return nil, errors.Errorf("hipq: GGML table must be Uint8 [vocab, bytesPerRow], got %s", tn.shape)
+	}
+	if in.shape.DType != dtypes.Int32 { // other integer types are converted by a node in front (fallback backend)
+		return nil, errors.Wrapf(compute.ErrNotImplemented, "hipq: indices of dtype %s", in.shape.DType)
+	}
+	if in.shape.Rank() < 1 || in.shape.Dimensions[in.shape.Rank()-1] != 1 {
+		return nil, errors.Errorf("hipq: indices must end in a dimension of 1, got %s", in.shape)
+	}
+	typeID := C.int(tq.GGMLType.TypeID())
+	bpb, vpb := int(C.gq_bytes_per_block(typeID)), int(C.gq_values_per_block(typeID))
+	if bpb == 0 {
+		return nil, errors.Wrapf(compute.ErrNotImplemented, "hipq: GGML type %d", int(typeID))
+	}
+	if tn.shape.Dimensions[1]%bpb != 0 {
+		return nil, errors.Errorf("hipq: %d bytes per row is not a whole number of %d-byte blocks", tn.shape.Dimensions[1], bpb)
+	}
+	k := tn.shape.Dimensions[1] / bpb * vpb
+	outDims := append([]int(nil), in.shape.Dimensions[:in.shape.Rank()-1]...)
+	outDims = append(outDims, k)
+	n := &node{kind: opQuantizedEmbeddingLookup, shape: shapes.Make(dtypes.Float32, outDims...),
+		inputs: f.nodes(table, indices), ggmlType: typeID, k: int64(k)}
+	return f.register(n), nil
+}
+
 // ---- Executable.Execute: one FusedQuantizedDense node ---------------------------------------------
 
 func (e *Executable) runQuantizedDense(n *node, x, w, bias, y *Buffer, stream unsafe.Pointer) error {
@@ -172,6 +208,17 @@ func (e *Executable) runQuantizedDense(n *node, x, w, bias, y *Buffer, stream un
 		}
 		return C.gq_qdense_f32(n.ggmlType, (*C.float)(x.dptr), C.int64_t(m), C.int64_t(n.k), w.dptr,
 			C.int64_t(w.shape.Dimensions[0]), b, n.act, (*C.float)(y.dptr), stream)
+	})
+}
+
+// runEmbeddingLookup gathers and dequantises rows.  errFlag is a device int32 the Executable clears before the
+// call and reads back with the outputs: 1 means an index was outside [0, vocab) (its row is NaN), which Execute
+// reports as an error like the reference's bounds check.
+func (e *Executable) runEmbeddingLookup(n *node, table, indices, out, errFlag *Buffer, stream unsafe.Pointer) error {
+	count := int64(indices.shape.Size())
+	return call(func() C.int {
+		return C.gq_embedding_lookup(n.ggmlType, table.dptr, C.int64_t(table.shape.Dimensions[0]), C.int64_t(n.k),
+			(*C.int32_t)(indices.dptr), C.int64_t(count), (*C.float)(out.dptr), (*C.int32_t)(errFlag.dptr), stream)
 	})
 }
 

@@ -28,6 +28,30 @@ def test_header_symbols_are_all_exported_and_bound():
     assert bound == set(syms)
 
 
+def test_go_binding_source_names_only_what_the_header_declares():
+    """The cgo source under go/hipbackend cannot be compiled here (no Go toolchain): at least every C name it uses
+    must exist in the header - functions, the two structs and the constants."""
+    text = open(os.path.join(ROOT, "include", "gomlx_hipq.h")).read()
+    header_names = set(re.findall(r"\b(gq_[a-z0-9_]+|GQ_[A-Z0-9_]+)\b", re.sub(r"/\*.*?\*/", "", text, flags=re.S)))
+    used = set()
+    godir = os.path.join(ROOT, "go", "hipbackend")
+    for fn in os.listdir(godir):
+        if fn.endswith(".go"):
+            used |= set(re.findall(r"\bC\.(gq_[a-z0-9_]+|GQ_[A-Z0-9_]+)\b", open(os.path.join(godir, fn)).read()))
+    assert len(used) >= 15
+    assert used <= header_names, sorted(used - header_names)
+    # both fused ops of the path are bound
+    assert {"gq_qdense_f32", "gq_qdense_bf16", "gq_embedding_lookup", "gq_qdense_check"} <= used
+
+
+def test_ablation_variants_still_apply_to_the_sources():
+    """The timing-only builds of the benchmark are made by exact text substitution on the kernel sources: every
+    substitution must still find its text (a kernel edit that moves it has to move the variant too)."""
+    from gomlx_amd import ablate
+    for name in ablate.VARIANTS:
+        assert ablate.variant_source(name)
+
+
 def test_no_oracle_or_torch_linked_into_the_library():
     import subprocess
     out = subprocess.run(["ldd", _lib.LIB_PATH], capture_output=True, text=True).stdout
