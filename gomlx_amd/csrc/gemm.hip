@@ -339,20 +339,42 @@ __global__ __launch_bounds__(512) void gemm_kernel(const void *Xv, const uint8_t
     if (SKEW) mfma_group(1);  // group 3 of the last step
 
     // ---- epilogue: acc[i][j][r] is Y[m, n] with n = lane % 32, m = 8*(r/4) + 4*(lane/32) + r%4
+    // Per element: one add, the activation, one store; the address is a per-lane base plus an offset that is the same for
+    // the whole wavefront, and what does not depend on the element - which activation, whether the tile reaches over the
+    // edge of the matrix - is decided once, outside the 64 stores.  (Written as one loop with those tests inside, the
+    // compiler spent some twenty vector-ALU instructions per element: C3 took 84.4 us against 79.3.)
+    const int m0 = bm + wm + 4 * (lane >> 5);
+    auto store_all = [&](auto bounded, auto activate) __attribute__((always_inline)) {
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const int n = bn + wn + j * 32 + (lane & 31);
-        if (n >= N) continue;
-        const float bv = bias ? bias[n] : 0.f;
+        for (int j = 0; j < 2; j++) {
+            const int n = bn + wn + j * 32 + (lane & 31);
+            if constexpr (decltype(bounded)::value) { if (n >= N) continue; }
+            const float bv = bias ? bias[n] : 0.f;
+            float *__restrict__ yp = Y + (int64_t)m0 * N + n;
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
+            for (int i = 0; i < 2; i++) {
+                // a block of 32 rows is inside the matrix as a whole, outside as a whole, or (one block per tile column at most) cut by its edge
+                const int rows_left = decltype(bounded)::value ? M - (bm + wm + i * 32) : 32;
+                if (rows_left <= 0) continue;
+                auto store16 = [&](auto checked) __attribute__((always_inline)) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int m = bm + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (m < M) Y[(int64_t)m * N + n] = apply_act(act, acc[i][j][r] + bv);
+                    for (int r = 0; r < 16; r++) {
+                        const int dm = i * 32 + 8 * (r >> 2) + (r & 3);
+                        if constexpr (decltype(checked)::value) { if (m0 + dm >= M) continue; }
+                        yp[(int64_t)dm * N] = activate(acc[i][j][r] + bv);
+                    }
+                };
+                if (rows_left >= 32) store16(std::false_type());
+                else store16(std::true_type());
             }
         }
-    }
+    };
+    auto by_act = [&](auto bounded) __attribute__((always_inline)) {
+        if (act == kActNone) store_all(bounded, [](float v) { return v; });
+        else store_all(bounded, [act](float v) { return apply_act(act, v); });
+    };
+    if (bm + BM <= M && bn + BN <= N) by_act(std::false_type());
+    else by_act(std::true_type());
 }
 
 template <int T, bool BF16, bool KTAIL>

@@ -21,6 +21,8 @@
 #include "blocks.hpp"
 #include "common.hpp"
 
+#include <type_traits>
+
 #include <cstdlib>
 
 namespace gq {
@@ -388,48 +390,101 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the re-read DMAs of the last steps
 
     // ---- epilogue: acc[i][j][r] is Y[m, n] with n = lane % 32, m = 8*(r/4) + 4*(lane/32) + r%4
+    // Per element: an add (or a multiply-add with the row's scale), the activation, a store; the address is a per-lane base
+    // plus an offset that is the same for the whole wavefront, and everything that does not depend on the element - which
+    // activation, row scales or not, residual or not, whether the tile reaches over the edge of the matrix - is decided
+    // once, outside the 64 stores.  (Written as one loop with those tests inside, the compiler spent some twenty vector-ALU
+    // instructions per element: C3 through the two passes took 83.3 us against 75.9, fp32 prefill 98.3 against 87.3.)
+    const int m0 = bm + wm + 4 * (lane >> 5);
     if constexpr (GATED) {
         static_assert(TN == 2, "a gated tile pairs two 32-column blocks");
+        // (the image of a gated pair may have more rows than 2 n_out: the bound is on the output columns)
         const int n = ((bn + wn) >> 1) + (lane & 31);
-        if (n < n_out) {
-            const float bg = bias ? bias[n] : 0.f, bu = bias2 ? bias2[n] : 0.f;
+        if (n >= n_out) return;
+        const float bg = bias ? bias[n] : 0.f, bu = bias2 ? bias2[n] : 0.f;
+        const int64_t at0 = (int64_t)m0 * n_out + n;
+        auto store_all = [&](auto bounded, auto scaled, auto with_residual, auto activate) __attribute__((always_inline)) {
 #pragma unroll
             for (int i = 0; i < TM; i++) {
+                const int rows_left = decltype(bounded)::value ? M - (bm + wm + i * 32) : 32;  // (see the plain form below)
+                if (rows_left <= 0) continue;
+                auto store16 = [&](auto checked) __attribute__((always_inline)) {
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int m = bm + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                    if (m < M) {
-                        const int64_t at = (int64_t)m * n_out + n;
-                        const float rs = rowscale ? rowscale[m] : 1.f;
-                        float v = apply_act(act, fmaf(acc[i][0][r], rs, bg)) * fmaf(acc[i][1][r], rs, bu);
-                        if (residual) v += residual[at];
-                        Y[at] = v;
+                    for (int r = 0; r < 16; r++) {
+                        const int dm = i * 32 + 8 * (r >> 2) + (r & 3);
+                        if constexpr (decltype(checked)::value) { if (m0 + dm >= M) continue; }
+                        float rs = 1.f;
+                        if constexpr (decltype(scaled)::value) rs = rowscale[m0 + dm];
+                        float v = activate(fmaf(acc[i][0][r], rs, bg)) * fmaf(acc[i][1][r], rs, bu);
+                        if constexpr (decltype(with_residual)::value) v += residual[at0 + (int64_t)dm * n_out];
+                        Y[at0 + (int64_t)dm * n_out] = v;
                     }
-                }
+                };
+                if (rows_left >= 32) store16(std::false_type());
+                else store16(std::true_type());
             }
-        }
+        };
+        auto by_act = [&](auto bounded, auto scaled, auto with_residual) __attribute__((always_inline)) {
+            if (act == kActSilu) store_all(bounded, scaled, with_residual, [](float v) { return v / (1.0f + __expf(-v)); });
+            else store_all(bounded, scaled, with_residual, [act](float v) { return apply_act(act, v); });
+        };
+        auto by_scale = [&](auto bounded, auto with_residual) __attribute__((always_inline)) {
+            if (rowscale) by_act(bounded, std::true_type(), with_residual);
+            else by_act(bounded, std::false_type(), with_residual);
+        };
+        auto by_edge = [&](auto with_residual) __attribute__((always_inline)) {
+            if (bm + G::DM <= M) by_scale(std::false_type(), with_residual);
+            else by_scale(std::true_type(), with_residual);
+        };
+        if (residual) by_edge(std::true_type());
+        else by_edge(std::false_type());
         return;
     }
+    auto store_all = [&](auto bounded, auto scaled, auto with_residual, auto activate) __attribute__((always_inline)) {
 #pragma unroll
-    for (int j = 0; j < TN; j++) {
-        const int n = bn + wn + j * 32 + (lane & 31);
-        if (n >= N) continue;
-        const float bv = bias ? bias[n] : 0.f;
+        for (int j = 0; j < TN; j++) {
+            const int n = bn + wn + j * 32 + (lane & 31);
+            if constexpr (decltype(bounded)::value) { if (n >= N) continue; }
+            const float bv = bias ? bias[n] : 0.f;
+            const int64_t at0 = (int64_t)m0 * N + n;
 #pragma unroll
-        for (int i = 0; i < TM; i++) {
+            for (int i = 0; i < TM; i++) {
+                // a block of 32 rows is inside the matrix as a whole, outside as a whole, or (one block per tile column at most) cut by its edge
+                const int rows_left = decltype(bounded)::value ? M - (bm + wm + i * 32) : 32;
+                if (rows_left <= 0) continue;
+                auto store16 = [&](auto checked) __attribute__((always_inline)) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int m = bm + wm + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (m < M) {
-                    // act(x.W + bias) plus a residual (which may be Y itself: one thread reads and writes an element)
-                    const int64_t at = (int64_t)m * N + n;
-                    float v = apply_act(act, rowscale ? fmaf(acc[i][j][r], rowscale[m], bv) : acc[i][j][r] + bv);
-                    if (residual) v += residual[at];
-                    Y[at] = v;
-                }
+                    for (int r = 0; r < 16; r++) {
+                        const int dm = i * 32 + 8 * (r >> 2) + (r & 3);
+                        if constexpr (decltype(checked)::value) { if (m0 + dm >= M) continue; }
+                        float v = acc[i][j][r];
+                        if constexpr (decltype(scaled)::value) v = fmaf(v, rowscale[m0 + dm], bv);
+                        else v += bv;
+                        v = activate(v);
+                        // (a residual may be Y itself: one thread reads and writes an element)
+                        if constexpr (decltype(with_residual)::value) v += residual[at0 + (int64_t)dm * N];
+                        Y[at0 + (int64_t)dm * N] = v;
+                    }
+                };
+                if (rows_left >= 32) store16(std::false_type());
+                else store16(std::true_type());
             }
         }
-    }
+    };
+    auto by_act = [&](auto bounded, auto scaled, auto with_residual) __attribute__((always_inline)) {
+        if (act == kActNone) store_all(bounded, scaled, with_residual, [](float v) { return v; });
+        else store_all(bounded, scaled, with_residual, [act](float v) { return apply_act(act, v); });
+    };
+    auto by_scale = [&](auto bounded, auto with_residual) __attribute__((always_inline)) {
+        if (rowscale) by_act(bounded, std::true_type(), with_residual);
+        else by_act(bounded, std::false_type(), with_residual);
+    };
+    auto by_edge = [&](auto with_residual) __attribute__((always_inline)) {
+        if (bm + G::DM <= M && bn + G::DN <= N) by_scale(std::false_type(), with_residual);
+        else by_scale(std::true_type(), with_residual);
+    };
+    if (residual) by_edge(std::true_type());
+    else by_edge(std::false_type());
 }
 
 template <int T, bool BF16>
@@ -474,13 +529,30 @@ int tile_env() {
     return v;
 }
 
-// The largest tile that still gives the chip about one workgroup per CU.
+// Which tile: 0 = 256 x 128, 1 = 128 x 128 (one workgroup per CU each), 2 = 128 x 64 (two per CU).  The workgroups run in
+// rounds of one per CU; a round of 128 x 128 tiles takes about 0.61 of a round of 256 x 128 tiles, and a last round that is
+// only partly filled still costs a good half of a full one (the chip clocks higher and the memory system is less
+// crowded, but every workgroup walks all of K).  Estimated that way, the choice matches the faster tile in 22 of 24
+// measured cases (K = 4096 and 14336, N = 4096 and 14336, 640 .. 1536 rows) - e.g. 1280 rows on 4096 x 4096 are 160
+// large tiles in one round (57 us) or 320 small ones in two (70 us), where a rule by tile count alone took the small ones.
+int pick_tile(int64_t M, int64_t N) {
+    const int64_t cus = device_cu_count();
+    auto tiles = [&](int64_t dm, int64_t dn) { return ((M + dm - 1) / dm) * ((N + dn - 1) / dn); };
+    if (tiles(128, 64) <= cus) return 2;  // small problems: as long as the smallest tiles run in one round they win (512 rows on 4096 x 4096: 35 against 38 us; 640 rows: 48 against 39)
+    if (M <= 128) return 1;                       // (no half-empty 256-row tiles)
+    auto rounds = [&](int64_t wgs, double empty_round) {
+        const int64_t full = wgs / cus;
+        const double frac = (double)(wgs % cus) / (double)cus;
+        return (double)full + (frac > 0.0 ? empty_round + (1.0 - empty_round) * frac : 0.0);
+    };
+    const double t0 = rounds(tiles(256, 128), 0.6), t1 = 0.61 * rounds(tiles(128, 128), 0.5);
+    return t0 <= t1 ? 0 : 1;
+}
+
 template <bool BF16>
 int launch_gemm16(const uint16_t *x, int64_t M, int64_t K, const uint16_t *Wh, int64_t N, const float *bias, int act, float *y, hipStream_t s,
                   const float *residual = nullptr, const float *rowscale = nullptr) {
-    const int64_t want = (int64_t)device_cu_count() * 3 / 4;
-    auto tiles = [&](int64_t dm, int64_t dn) { return ((M + dm - 1) / dm) * ((N + dn - 1) / dn); };
-    int choice = (tiles(256, 128) >= want && M > 128) ? 0 : tiles(128, 128) >= want ? 1 : 2;  // (no half-empty 256-row tiles)
+    int choice = pick_tile(M, N);
     if (tile_env() >= 0 && tile_env() <= 2) choice = tile_env();
     switch (choice) {
     case 0: return launch_gemm16_tile<BF16, 2, 2>(x, M, K, Wh, N, bias, act, y, nullptr, N, residual, rowscale, s);
@@ -494,19 +566,17 @@ int64_t gated_image_rows(int64_t N) { return (N + 31) / 32 * 64; }
 int launch_gemm16_gated(const uint16_t *x, int64_t M, int64_t K, const uint16_t *Wh, int64_t N, const float *bias, const float *bias2, int act,
                         float *y, const float *residual, const float *rowscale, hipStream_t s) {
     const int64_t rows = gated_image_rows(N);
-    const int64_t want = (int64_t)device_cu_count() * 3 / 4;
-    const bool big = M > 128 && ((M + 255) / 256) * ((rows + 127) / 128) >= want;
+    const bool big = pick_tile(M, rows) == 0;  // (the gated kernel exists for the two 128-column tiles)
     if (big && tile_env() != 1) return launch_gemm16_tile<false, 2, 2, true>(x, M, K, Wh, rows, bias, act, y, bias2, N, residual, rowscale, s);
     return launch_gemm16_tile<false, 1, 2, true>(x, M, K, Wh, rows, bias, act, y, bias2, N, residual, rowscale, s);
 }
 
 // Measured against the fused kernel (K = 4096, N = 4096 .. 14336): the two passes win from the
 // first batch size the GEMV passes do not take (17 rows: 33 against 60 us for Q8_0 at 64 rows, 37
-// against 66 .. 102 us at 512 rows) up to the largest; the fused kernel is within 5 % only for
-// Q8_0 with bf16 activations, whose conversion is the cheapest: there it stays ahead between
-// about 1300 and 4000 rows (2048 rows: 85 .. 88 us against 81 .. 95 us for the two passes).
+// against 66 .. 102 us at 512 rows) up to the largest.  The fused kernel comes within 5 % only for Q8_0 with bf16
+// activations, whose conversion is the cheapest (2048 rows on 4096 x 4096: 79 us against 76 for the two passes; 1536 rows on
+// 14336 -> 4096: 226 against 194); it serves the shapes the two passes do not take.
 constexpr int64_t kMinRowsTwoPass = 17;
-constexpr int64_t kFusedQ8Bf16From = 1281, kFusedQ8Bf16Below = 4096;
 constexpr uint64_t kMaxImageBytes = (uint64_t)4 << 30;   // largest 16-bit weight image kept in a workspace
 
 // GOMLX_HIPQ_TWO_PASS_MIN_ROWS=<rows> overrides the threshold (tuning runs only).
@@ -522,7 +592,6 @@ int64_t two_pass_env_rows() {
 // fp32 activations are rewritten anyway and get rows padded to that.
 bool gemm_two_pass_supported(int type, bool x_is_bf16, int64_t M, int64_t K, int64_t N, const void *x) {
     if (type != kQ4_0 && type != kQ8_0 && type != kIQ4_NL && type != kQ4_K && type != kQ6_K) return false;
-    if (type == kQ8_0 && x_is_bf16 && M >= kFusedQ8Bf16From && M < kFusedQ8Bf16Below && two_pass_env_rows() <= 0) return false;
     const int64_t min_rows = two_pass_env_rows() > 0 ? two_pass_env_rows() : kMinRowsTwoPass;
     if (M < min_rows || K % (x_is_bf16 ? 64 : 32) != 0) return false;
     if (K > (1 << 22) || N > INT32_MAX || M > INT32_MAX || (M + 127) / 128 > 65535) return false;

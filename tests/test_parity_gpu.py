@@ -655,6 +655,44 @@ def gated_case(gpu, oracle, t, M, K, N, act, norm_kind, with_bias, seed):
     return err
 
 
+def test_gemm_epilogues_stay_inside_their_output(gpu, oracle):
+    """The GEMM kernels write whole interior tiles without per-element bounds checks.  Outputs placed in the middle of a
+    larger buffer filled with a sentinel: shapes that are exact multiples of the tiles, one row / column over and under,
+    and a gated pair whose interleaved weight image is longer than twice its outputs - the sentinel on both sides must
+    survive and the result must be right."""
+    import ctypes
+    from gomlx_amd import _lib
+    L = _lib.lib()
+    stream = gpu.cuda.current_stream().cuda_stream
+    pad = 4096
+    t = Q8_0
+    for M, K, N, bf16 in [(256, 512, 128, True), (512, 512, 256, False), (257, 512, 129, True), (255, 512, 127, False), (1408, 256, 192, True),
+                          (384, 512, 320, False)]:
+        W, x = synth.weights(t, 9500 + M, N, K), synth.activations(9501 + N, M, K)
+        xin = bf16_round(x) if bf16 else x
+        buf = gpu.full((pad + M * N + pad,), 12345.0, device="cuda")
+        xd = dev(gpu, xin).to(gpu.bfloat16) if bf16 else dev(gpu, xin)
+        Wd = dev(gpu, W)  # (kept alive until the call has run)
+        fn = L.gq_qdense_bf16 if bf16 else L.gq_qdense_f32
+        _lib.check(fn(t, xd.data_ptr(), M, K, Wd.data_ptr(), N, None, 0, buf.data_ptr() + 4 * pad, stream))
+        gpu.cuda.synchronize()
+        h = buf.cpu().numpy()
+        assert np.all(h[:pad] == 12345.0) and np.all(h[pad + M * N:] == 12345.0), (M, K, N, bf16)
+        assert rel_err(h[pad:pad + M * N].reshape(M, N), oracle.c_qdense(t, xin, W)) < (TOL_BF16 if bf16 else TOL_F32)
+    for M, K, N in [(256, 512, 1000), (512, 256, 64), (300, 512, 96)]:
+        Wg, Wu, x = synth.weights(t, 9600 + N, N, K), synth.weights(t, 9601 + N, N, K), synth.activations(9602 + M, M, K)
+        buf = gpu.full((pad + M * N + pad,), 12345.0, device="cuda")
+        xd, Wgd, Wud = dev(gpu, x), dev(gpu, Wg), dev(gpu, Wu)
+        _lib.check(L.gq_qdense_gated_f32(t, xd.data_ptr(), M, K, None, Wgd.data_ptr(), None, Wud.data_ptr(), None, N, 3,
+                                         buf.data_ptr() + 4 * pad, stream))
+        gpu.cuda.synchronize()
+        h = buf.cpu().numpy()
+        assert np.all(h[:pad] == 12345.0) and np.all(h[pad + M * N:] == 12345.0), ("gated", M, K, N)
+        want = oracle.c_gated_ffn(t, x, Wg, Wu, None, None, 3, None)
+        scale = float(np.max(np.abs(oracle.c_qdense(t, x, Wg)))) * float(np.max(np.abs(oracle.c_qdense(t, x, Wu))))
+        assert float(np.max(np.abs(h[pad:pad + M * N].reshape(M, N).astype(np.float64) - want))) / scale < 2 * TOL_F32
+
+
 @pytest.mark.parametrize("t", ALL_TYPES)
 def test_gated_feed_forward_decode(gpu, oracle, t):
     """Fused path: up to 16 rows, K a multiple of 256 (one launch over both matrices)."""
