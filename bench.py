@@ -73,7 +73,7 @@ ARITHMETIC = {
     "c0": "f32 in/out; x -> 16-bit block fixed point (two int8 limbs per 32 values), v_dot4_i32_i8 against the int8 codes, i32 sums scaled and added in f32",
     "c1": "f32 in/out; x -> 16-bit block fixed point (four int4 digits per 32 values), v_dot8_i32_i4 against the 4-bit codes, i32 sums scaled and added in f32",
     "c2": "f32 in/out; x -> f16 (each row and K-slice scaled by a power of two), 4-bit codes x 6-bit scales as exact f16 integers, f16 MFMA with f32 accumulation, d / dmin and the K-slice sums in f32",
-    "c3": "bf16 activations, weights dequantised (exact f32 value, one rounding) to bf16 operands in LDS, bf16 MFMA with f32 accumulation, f32 out",
+    "c3": "bf16 activations, weights dequantised (exact f32 value, one rounding) to a bf16 image by one pass, then a bf16 MFMA GEMM with f32 accumulation, f32 out",
     "c4": "f32 in/out; x -> 16-bit block fixed point (two int8 limbs per 32 values), v_dot4_i32_i8 against the 4-bit codes, i32 sums scaled (d * 6-bit scale, dmin * 6-bit minimum) and added in f32",
     "prefill": "f32 in/out; x and dequantised W rounded to f16 operands (x rows scaled by a power of two), f16 MFMA with f32 accumulation",
 }
@@ -97,7 +97,8 @@ def parse_args():
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     p.add_argument("--no-extras", action="store_true", help="skip the cache-resident pass, the plain-read yardstick and the clock sampling")
     p.add_argument("--ablation", default=None,
-                   help="time a TIMING-ONLY variant of the fused GEMM (gemm_*: --config c3) or of the Q4_K split-K route (q4k_*: --config c2) "
+                   help="time a TIMING-ONLY variant of the fused GEMM (gemm_*: --config c3 with GOMLX_HIPQ_TWO_PASS_MIN_ROWS=100000, which sends C3 through that kernel), "
+                        "of the Q4_K split-K route (q4k_*: --config c2) or of the decode GEMV (ks_*: --config c0) "
                         "instead of the product library (python -m gomlx_amd.ablate build NAME first): its results are wrong on purpose and the "
                         "line says so")
     p.add_argument("--hot", action="store_true", help="single weight buffer (Infinity-Cache resident) for the main measurement as well")

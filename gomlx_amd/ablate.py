@@ -1,4 +1,5 @@
-"""Timing-only ablations of the fused dequantise-in-LDS GEMM (csrc/gemm.hip; names gemm_*, timed on --config c3)
+"""Timing-only ablations of the fused dequantise-in-LDS GEMM (csrc/gemm.hip; names gemm_*, timed on --config c3 with
+GOMLX_HIPQ_TWO_PASS_MIN_ROWS=100000 in the environment, which sends that shape through the fused kernel)
 and of the Q4_K split-K route (csrc/mmq.hip; names q4k_*, timed on --config c2) and of the decode GEMV (csrc/gemv_ks_body.hpp; names ks_*, timed on
 --config c0 / c1: single calls only, the batched and extended kernels live in other units).
 
@@ -66,6 +67,18 @@ _Q4K_FETCH0 = "    if (par < nsb) fetch(par);\n"
 _Q4K_FETCH = "        if (sbl + kParts < nsb) fetch(sbl + kParts);\n"
 _Q4K_CONTRACT = "        q4k_contract_sb<false>(cur, lds, lds + xs_off + sbl * (kMT * 16), nullptr, sbl, kg, col, magic, acc);\n"
 _Q4K_KEEP = '        asm volatile("" ::"v"(cur.hd.x), "v"(cur.c[0].x), "v"(cur.c[1].x), "v"(cur.c[2].x), "v"(cur.c[3].x), "v"(magic));\n'
+_Q4K_PARTIAL = """            if (m < M) partial[((int64_t)slice * M + m) * set.ntot + set.n0[prob] + n] = v;
+        }
+    }
+}
+
+// ---- the activation pre-pass folded into the main kernel"""
+_Q4K_NO_PARTIAL = """            asm volatile("" ::"v"(v));
+        }
+    }
+}
+
+// ---- the activation pre-pass folded into the main kernel"""
 _Q4K_XPREP = """    if (int rc = x_is_bf16 ? (fine ? prep(mmq_xprep_kernel<true, 1>) : prep(mmq_xprep_kernel<true, 2>))
                            : (fine ? prep(mmq_xprep_kernel<false, 1>) : prep(mmq_xprep_kernel<false, 2>)))
         return rc;
@@ -112,6 +125,9 @@ VARIANTS = {
     "q4k_no_image": ("mmq.hip", "the copy of the slice's activation image into LDS (main kernel)", [(_Q4K_IMAGE, "            (void)img;\n")]),
     "q4k_no_weights": ("mmq.hip", "the weight loads of the main kernel (it contracts whatever LDS holds)", [(_Q4K_FETCH0, ""), (_Q4K_FETCH, "")]),
     "q4k_no_contract": ("mmq.hip", "unpacking and MFMAs of the main kernel (loads and LDS reads kept)", [(_Q4K_CONTRACT, _Q4K_KEEP)]),
+    "q4k_main_empty": ("mmq.hip", "image copy, weight loads and contraction of the main kernel together (launch, barriers, LDS hand-over and partial stores remain)",
+                       [(_Q4K_IMAGE, "            (void)img;\n"), (_Q4K_FETCH0, ""), (_Q4K_FETCH, ""), (_Q4K_CONTRACT, _Q4K_KEEP)]),
+    "q4k_no_partials": ("mmq.hip", "the main kernel's stores of its partial sums", [(_Q4K_PARTIAL, _Q4K_NO_PARTIAL)]),
     "q4k_no_xprep": ("mmq.hip", "the activation pre-pass launch", [(_Q4K_XPREP, "    (void)prep;\n")]),
     "q4k_no_reduce": ("mmq.hip", "the reduction launch", [(_Q4K_REDUCE, "    if (count == 1) return GQ_OK;\n")]),
 }
