@@ -52,6 +52,39 @@ def test_ablation_variants_still_apply_to_the_sources():
         assert ablate.variant_source(name)
 
 
+def test_written_out_memory_instructions_keep_their_wait_states(tmp_path):
+    """A vector-memory instruction that reads a scalar register needs five wait states after a vector instruction wrote
+    that register (v_readfirstlane and friends).  The compiler inserts them for its own loads; for instructions written
+    out as text it cannot, and a load that runs too early takes the register's previous contents as its address.  The
+    GEMM's LDS-DMA copies are such text: its assembly must show no vector-ALU write to their scalar operands within the
+    five instructions in front of them."""
+    import subprocess
+    from gomlx_amd import build as B
+    asm = tmp_path / "gemm_dma.s"
+    flags = [f for f in B.HIPCC_FLAGS if not f.startswith("-Rpass")]
+    r = subprocess.run([B.hipcc(), *flags, "-S", "--cuda-device-only", "-I", B.CSRC, os.path.join(B.CSRC, "gemm_dma.hip"), "-o", str(asm)],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    lines = asm.read_text().split("\n")
+    checked = 0
+    for i, l in enumerate(lines):
+        m = re.search(r"buffer_load_dwordx4 v\d+, s\[(\d+):(\d+)\], (s\d+) offen lds", l)
+        if not m:
+            continue
+        checked += 1
+        sregs = {f"s{k}" for k in range(int(m.group(1)), int(m.group(2)) + 1)} | {m.group(3)}
+        k, seen = i - 1, 0
+        while k > 0 and seen < 5:
+            t = lines[k].strip()
+            k -= 1
+            if not t or t.startswith((";", ".")):
+                continue
+            seen += 1
+            if t.startswith("v_") and t.split()[1].rstrip(",") in sregs:
+                raise AssertionError(f"line {k + 2}: {t!r} writes a scalar operand of the copy at line {i + 1} {seen - 1} instructions before it")
+    assert checked > 100  # every instance of the kernel carries its copies
+
+
 def test_no_oracle_or_torch_linked_into_the_library():
     import subprocess
     out = subprocess.run(["ldd", _lib.LIB_PATH], capture_output=True, text=True).stdout
