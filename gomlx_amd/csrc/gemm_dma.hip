@@ -73,13 +73,13 @@ __host__ __device__ inline int64_t padded_k(int64_t K) { return (K + 63) / 64 * 
 // The image's rows hold runs_per_row runs, of which the first `runs` come from W and the rest (padding
 // of K to the GEMM's step of 64) are zero.
 template <int T, bool BF16>
-__global__ __launch_bounds__(256) void dequant16bit_kernel(const uint8_t *__restrict__ W, uint16_t *__restrict__ out, uint32_t runs_per_row,
-                                                          uint32_t total_runs, int64_t row_bytes, int half, uint32_t runs) {
+__device__ __forceinline__ void dequant16bit_body(const uint8_t *__restrict__ W, uint16_t *__restrict__ out, uint32_t runs_per_row,
+                                                  uint32_t total_runs, int64_t row_bytes, int half, uint32_t runs, uint32_t block) {
     // The 16-byte halves of the runs meet in LDS so that consecutive lanes store consecutive 16 bytes
     // (whole cache lines per store instruction; a lane storing its own 32 bytes in two instructions
     // half-fills twice as many).  An image holds at most 2^27 runs: 32-bit index arithmetic.
     __shared__ uint4 halves[512];
-    const uint32_t tid = threadIdx.x, g0 = blockIdx.x * 256u, g = g0 + tid;
+    const uint32_t tid = threadIdx.x, g0 = block * 256u, g = g0 + tid;
     if (g < total_runs) {
         const uint32_t row = g / runs_per_row, run = g % runs_per_row;
         float w[16];
@@ -103,6 +103,12 @@ __global__ __launch_bounds__(256) void dequant16bit_kernel(const uint8_t *__rest
         const int64_t out_row = half == 0 ? (int64_t)row : (int64_t)(row >> 5) * 64 + (half - 1) * 32 + (row & 31);
         *reinterpret_cast<uint4 *>(out + (out_row * runs_per_row + run) * 16 + (c & 1u) * 8u) = halves[c];
     }
+}
+
+template <int T, bool BF16>
+__global__ __launch_bounds__(256) void dequant16bit_kernel(const uint8_t *__restrict__ W, uint16_t *__restrict__ out, uint32_t runs_per_row,
+                                                          uint32_t total_runs, int64_t row_bytes, int half, uint32_t runs) {
+    dequant16bit_body<T, BF16>(W, out, runs_per_row, total_runs, row_bytes, half, runs, blockIdx.x);
 }
 
 // fp32 activations -> fp16 [M, K], one workgroup per row: the row is scaled by a power of two
@@ -163,10 +169,10 @@ __global__ __launch_bounds__(256) void x_rmsnorm_to_f16_kernel(const float *__re
 // Both activation passes for rows of at most 2048 IT values: the row stays in registers between the reduction and
 // the conversion, so it is read once.  NORM: the RMS normalisation variant.
 template <int IT, bool NORM>
-__global__ __launch_bounds__(256) void x_row_to_f16_kernel(const float *__restrict__ X, const float *__restrict__ gain, float gain_offset, float eps,
-                                                           int K, uint16_t *__restrict__ out, float *__restrict__ rowscale) {
+__device__ __forceinline__ void x_row_to_f16_body(const float *__restrict__ X, const float *__restrict__ gain, float gain_offset, float eps,
+                                                  int K, uint16_t *__restrict__ out, float *__restrict__ rowscale, uint32_t row) {
     __shared__ float part[4];
-    const float4 *x = reinterpret_cast<const float4 *>(X + (int64_t)blockIdx.x * K);
+    const float4 *x = reinterpret_cast<const float4 *>(X + (int64_t)row * K);
     const int k8 = K / 8, kp8 = (int)(padded_k(K) / 8);
     float4 a[IT], b[IT];
 #pragma unroll
@@ -195,13 +201,13 @@ __global__ __launch_bounds__(256) void x_row_to_f16_kernel(const float *__restri
     float sc = 1.f, r = 1.f;
     if constexpr (NORM) {
         r = sqrtf(((part[0] + part[1]) + (part[2] + part[3])) / (float)K + eps);
-        if (threadIdx.x == 0) rowscale[blockIdx.x] = 1.f;  // normalised rows are O(gain): no scaling
+        if (threadIdx.x == 0) rowscale[row] = 1.f;  // normalised rows are O(gain): no scaling
     } else {
         float inv;
         pow2_scale(fmaxf(fmaxf(part[0], part[1]), fmaxf(part[2], part[3])), sc, inv);
-        if (threadIdx.x == 0) rowscale[blockIdx.x] = inv;
+        if (threadIdx.x == 0) rowscale[row] = inv;
     }
-    uint4 *o = reinterpret_cast<uint4 *>(out + (int64_t)blockIdx.x * (kp8 * 8));
+    uint4 *o = reinterpret_cast<uint4 *>(out + (int64_t)row * (kp8 * 8));
 #pragma unroll
     for (int i = 0; i < IT; i++) {
         const int g = (int)threadIdx.x + 256 * i;
@@ -220,6 +226,12 @@ __global__ __launch_bounds__(256) void x_row_to_f16_kernel(const float *__restri
         }
         o[g] = make_uint4(Op16<false>::pack(p.x, p.y), Op16<false>::pack(p.z, p.w), Op16<false>::pack(q.x, q.y), Op16<false>::pack(q.z, q.w));
     }
+}
+
+template <int IT, bool NORM>
+__global__ __launch_bounds__(256) void x_row_to_f16_kernel(const float *__restrict__ X, const float *__restrict__ gain, float gain_offset, float eps,
+                                                           int K, uint16_t *__restrict__ out, float *__restrict__ rowscale) {
+    x_row_to_f16_body<IT, NORM>(X, gain, gain_offset, eps, K, out, rowscale, blockIdx.x);
 }
 
 // x -> fp16 rows (+ row scales), with the normalisation when norm is given
@@ -508,6 +520,61 @@ int launch_dequant16bit_type(int type, const uint8_t *W, int64_t N, int64_t K, u
     }
 }
 
+// Both pre-passes of the fp32-activation route in ONE launch (they do not depend on each other): the first M workgroups
+// convert an activation row each (x_row_to_f16_body), the others 256 runs of weights each (dequant16bit_body), of W and -
+// for a gated pair, whose images interleave - of W2.  Rows of up to 8192 values (longer ones keep their own two-read kernel).
+template <int T, int IT, bool NORM>
+__global__ __launch_bounds__(256) void prep_f32_kernel(const float *__restrict__ X, const float *__restrict__ gain, float gain_offset, float eps, int K,
+                                                       uint16_t *__restrict__ xh, float *__restrict__ rowscale, uint32_t xblocks,
+                                                       const uint8_t *__restrict__ W, const uint8_t *__restrict__ W2, uint16_t *__restrict__ wh,
+                                                       uint32_t runs_per_row, uint32_t total_runs, int64_t row_bytes, uint32_t runs, uint32_t wblocks) {
+    const uint32_t b = blockIdx.x;
+    if (b < xblocks) {
+        x_row_to_f16_body<IT, NORM>(X, gain, gain_offset, eps, K, xh, rowscale, b);
+    } else if (b - xblocks < wblocks) {
+        dequant16bit_body<T, false>(W, wh, runs_per_row, total_runs, row_bytes, W2 ? 1 : 0, runs, b - xblocks);
+    } else {
+        dequant16bit_body<T, false>(W2, wh, runs_per_row, total_runs, row_bytes, 2, runs, b - xblocks - wblocks);
+    }
+}
+
+template <int T>
+int launch_prep_f32_t(const float *x, int64_t M, int64_t K, const RmsNorm *norm, uint16_t *xh, float *rowscale, const uint8_t *W, const uint8_t *W2,
+                      int64_t N, uint16_t *wh, hipStream_t s) {
+    const int64_t runs = K / 16, runs_per_row = padded_k(K) / 16, total = N * runs_per_row;
+    const int64_t row_bytes = (K / Geom<T>::vpb) * Geom<T>::bpb;
+    if (total > ((int64_t)1 << 27)) return fail(GQ_ERR_INVALID, "gemm: a 16-bit image of %lld x %lld values is too large", (long long)N, (long long)K);
+    const int64_t wblocks = (total + 255) / 256, blocks = M + wblocks * (W2 ? 2 : 1);
+    if (blocks > INT32_MAX) return fail(GQ_ERR_INVALID, "gemm: too many workgroups in the pre-pass");
+    const float *gain = norm ? norm->gain : nullptr;
+    const float off = norm ? norm->gain_offset : 0.f, eps = norm ? norm->eps : 0.f;
+    const dim3 grid((unsigned)blocks), block(256);
+    auto go = [&](auto kernel) {
+        return launch(kernel, grid, block, 0, s, x, gain, off, eps, (int)K, xh, rowscale, (uint32_t)M, W, W2, wh, (uint32_t)runs_per_row, (uint32_t)total,
+                      row_bytes, (uint32_t)runs, (uint32_t)wblocks);
+    };
+    if (padded_k(K) <= 4096) return norm ? go(prep_f32_kernel<T, 2, true>) : go(prep_f32_kernel<T, 2, false>);
+    return norm ? go(prep_f32_kernel<T, 4, true>) : go(prep_f32_kernel<T, 4, false>);
+}
+
+// x -> fp16 rows and W (and W2) -> fp16 image: one launch for rows of up to 8192 values, else one per operand
+int launch_prep_f32(int type, const float *x, int64_t M, int64_t K, const RmsNorm *norm, uint16_t *xh, float *rowscale, const uint8_t *W,
+                    const uint8_t *W2, int64_t N, uint16_t *wh, hipStream_t s) {
+    if (padded_k(K) > 8192) {
+        if (int rc = launch_x_to_f16(x, M, K, norm, xh, rowscale, s)) return rc;
+        if (int rc = launch_dequant16bit_type<false>(type, W, N, K, wh, s, W2 ? 1 : 0)) return rc;
+        return W2 ? launch_dequant16bit_type<false>(type, W2, N, K, wh, s, 2) : GQ_OK;
+    }
+    switch (type) {
+    case kQ4_0: return launch_prep_f32_t<kQ4_0>(x, M, K, norm, xh, rowscale, W, W2, N, wh, s);
+    case kQ8_0: return launch_prep_f32_t<kQ8_0>(x, M, K, norm, xh, rowscale, W, W2, N, wh, s);
+    case kIQ4_NL: return launch_prep_f32_t<kIQ4_NL>(x, M, K, norm, xh, rowscale, W, W2, N, wh, s);
+    case kQ4_K: return launch_prep_f32_t<kQ4_K>(x, M, K, norm, xh, rowscale, W, W2, N, wh, s);
+    case kQ6_K: return launch_prep_f32_t<kQ6_K>(x, M, K, norm, xh, rowscale, W, W2, N, wh, s);
+    default: return fail(GQ_ERR_NOT_IMPLEMENTED, "qdense: ggml type %d is not implemented", type);
+    }
+}
+
 // N counts the rows of the weight image (for a gated pair: both halves, 64 per 32 outputs)
 template <bool BF16, int TM, int TN, bool GATED = false>
 int launch_gemm16_tile(const uint16_t *x, int64_t M, int64_t K, const uint16_t *Wh, int64_t N, const float *bias, int act, float *y,
@@ -616,8 +683,7 @@ int launch_gemm_two_pass(int type, bool x_is_bf16, const void *x, int64_t M, int
     const int64_t Kp = padded_k(K);
     uint16_t *xh = wh + (((size_t)N * Kp * 2 + 255) & ~(size_t)255) / 2;
     float *rowscale = reinterpret_cast<float *>(xh + (((size_t)M * Kp * 2 + 255) & ~(size_t)255) / 2);
-    if (int rc = launch_dequant16bit_type<false>(type, W, N, K, wh, s)) return rc;
-    if (int rc = launch_x_to_f16(static_cast<const float *>(x), M, K, nullptr, xh, rowscale, s)) return rc;
+    if (int rc = launch_prep_f32(type, static_cast<const float *>(x), M, K, nullptr, xh, rowscale, W, nullptr, N, wh, s)) return rc;
     return launch_gemm16<false>(xh, M, Kp, wh, N, bias, act, y, s, nullptr, rowscale);
 }
 
@@ -644,13 +710,8 @@ int launch_gemm_two_pass_block(int type, const float *x, int64_t M, int64_t K, c
     const int64_t Kp = padded_k(K);
     uint16_t *xh = wh + (((size_t)rows * Kp * 2 + 255) & ~(size_t)255) / 2;
     float *rowscale = reinterpret_cast<float *>(xh + (((size_t)M * Kp * 2 + 255) & ~(size_t)255) / 2);
-    if (int rc = launch_x_to_f16(x, M, K, norm, xh, rowscale, s)) return rc;
-    if (!W2) {
-        if (int rc = launch_dequant16bit_type<false>(type, W, N, K, wh, s)) return rc;
-        return launch_gemm16<false>(xh, M, Kp, wh, N, bias, act, y, s, residual, rowscale);
-    }
-    if (int rc = launch_dequant16bit_type<false>(type, W, N, K, wh, s, 1)) return rc;
-    if (int rc = launch_dequant16bit_type<false>(type, W2, N, K, wh, s, 2)) return rc;
+    if (int rc = launch_prep_f32(type, x, M, K, norm, xh, rowscale, W, W2, N, wh, s)) return rc;
+    if (!W2) return launch_gemm16<false>(xh, M, Kp, wh, N, bias, act, y, s, residual, rowscale);
     return launch_gemm16_gated(xh, M, Kp, wh, N, bias, bias2, act, y, residual, rowscale, s);
 }
 
