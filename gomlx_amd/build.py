@@ -22,7 +22,8 @@ HOST = os.path.join(HERE, "host")
 HOST_TEST = os.path.join(HOST, "build", "hipq_backend_test")
 WORKSPACE_TEST = os.path.join(HOST, "build", "workspace_test")
 
-SOURCES = ["api.hip", "dequant.hip", "gemv.hip", "gemv_xs.hip", "gemv_ks.hip", "mlp.hip", "mmq.hip", "gemm.hip", "gemm_dma.hip"]
+# (the units that take longest to compile come first: they are the critical path of the parallel build)
+SOURCES = ["gemm.hip", "gemm_dma.hip", "mlp.hip", "gemv_ks.hip", "api.hip", "dequant.hip", "gemv.hip", "gemv_xs.hip", "mmq.hip"]
 
 # -packed-fp32-ops (note the minus): keep hipcc from forming v_pk_*_f32 instructions.
 # -ffp-contract=off: dequantisation must round every fp32 operation on its own; fused

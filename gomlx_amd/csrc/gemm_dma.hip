@@ -37,6 +37,12 @@ typedef int i32x4 __attribute__((ext_vector_type(4)));
 constexpr int DK = 64;
 constexpr int ROWB = 128;  // bytes per LDS row
 
+// a compile-time switch (std::true_type / std::false_type) or a run-time one (bool) behind one spelling
+template <class F> __device__ __forceinline__ constexpr bool is_on(F f) {
+    if constexpr (std::is_same_v<F, bool>) return f;
+    else return F::value;
+}
+
 template <bool BF16> struct Op16;
 template <> struct Op16<true> {
     typedef bf16x8 vec8;
@@ -426,9 +432,9 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const 
                         const int dm = i * 32 + 8 * (r >> 2) + (r & 3);
                         if constexpr (decltype(checked)::value) { if (m0 + dm >= M) continue; }
                         float rs = 1.f;
-                        if constexpr (decltype(scaled)::value) rs = rowscale[m0 + dm];
+                        if (is_on(scaled)) rs = rowscale[m0 + dm];
                         float v = activate(fmaf(acc[i][0][r], rs, bg)) * fmaf(acc[i][1][r], rs, bu);
-                        if constexpr (decltype(with_residual)::value) v += residual[at0 + (int64_t)dm * n_out];
+                        if (is_on(with_residual)) v += residual[at0 + (int64_t)dm * n_out];
                         Y[at0 + (int64_t)dm * n_out] = v;
                     }
                 };
@@ -436,20 +442,18 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const 
                 else store16(std::true_type());
             }
         };
-        auto by_act = [&](auto bounded, auto scaled, auto with_residual) __attribute__((always_inline)) {
-            if (act == kActSilu) store_all(bounded, scaled, with_residual, [](float v) { return v / (1.0f + __expf(-v)); });
-            else store_all(bounded, scaled, with_residual, [act](float v) { return apply_act(act, v); });
+        // (SiLU, the activation of the feed-forward blocks this form exists for, gets the compile-time switches; the
+        // others take row scales and residual as run-time tests, uniform over the wavefront: a quarter of the code)
+        auto by_edge = [&](auto bounded) __attribute__((always_inline)) {
+            auto silu = [](float v) { return v / (1.0f + __expf(-v)); };
+            if (act != kActSilu) store_all(bounded, rowscale != nullptr, residual != nullptr, [act](float v) { return apply_act(act, v); });
+            else if (rowscale && residual) store_all(bounded, std::true_type(), std::true_type(), silu);
+            else if (rowscale) store_all(bounded, std::true_type(), std::false_type(), silu);
+            else if (residual) store_all(bounded, std::false_type(), std::true_type(), silu);
+            else store_all(bounded, std::false_type(), std::false_type(), silu);
         };
-        auto by_scale = [&](auto bounded, auto with_residual) __attribute__((always_inline)) {
-            if (rowscale) by_act(bounded, std::true_type(), with_residual);
-            else by_act(bounded, std::false_type(), with_residual);
-        };
-        auto by_edge = [&](auto with_residual) __attribute__((always_inline)) {
-            if (bm + G::DM <= M) by_scale(std::false_type(), with_residual);
-            else by_scale(std::true_type(), with_residual);
-        };
-        if (residual) by_edge(std::true_type());
-        else by_edge(std::false_type());
+        if (bm + G::DM <= M) by_edge(std::false_type());
+        else by_edge(std::true_type());
         return;
     }
     auto store_all = [&](auto bounded, auto scaled, auto with_residual, auto activate) __attribute__((always_inline)) {
@@ -470,11 +474,11 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const 
                         const int dm = i * 32 + 8 * (r >> 2) + (r & 3);
                         if constexpr (decltype(checked)::value) { if (m0 + dm >= M) continue; }
                         float v = acc[i][j][r];
-                        if constexpr (decltype(scaled)::value) v = fmaf(v, rowscale[m0 + dm], bv);
+                        if (is_on(scaled)) v = fmaf(v, rowscale[m0 + dm], bv);
                         else v += bv;
                         v = activate(v);
                         // (a residual may be Y itself: one thread reads and writes an element)
-                        if constexpr (decltype(with_residual)::value) v += residual[at0 + (int64_t)dm * N];
+                        if (is_on(with_residual)) v += residual[at0 + (int64_t)dm * N];
                         Y[at0 + (int64_t)dm * N] = v;
                     }
                 };
@@ -483,20 +487,18 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const 
             }
         }
     };
-    auto by_act = [&](auto bounded, auto scaled, auto with_residual) __attribute__((always_inline)) {
-        if (act == kActNone) store_all(bounded, scaled, with_residual, [](float v) { return v; });
-        else store_all(bounded, scaled, with_residual, [act](float v) { return apply_act(act, v); });
+    // (no activation - the projections of a decoder - gets the compile-time switches; with an activation, row scales and
+    // residual are run-time tests, uniform over the wavefront: a quarter of the code)
+    auto by_edge = [&](auto bounded) __attribute__((always_inline)) {
+        auto none = [](float v) { return v; };
+        if (act != kActNone) store_all(bounded, rowscale != nullptr, residual != nullptr, [act](float v) { return apply_act(act, v); });
+        else if (rowscale && residual) store_all(bounded, std::true_type(), std::true_type(), none);
+        else if (rowscale) store_all(bounded, std::true_type(), std::false_type(), none);
+        else if (residual) store_all(bounded, std::false_type(), std::true_type(), none);
+        else store_all(bounded, std::false_type(), std::false_type(), none);
     };
-    auto by_scale = [&](auto bounded, auto with_residual) __attribute__((always_inline)) {
-        if (rowscale) by_act(bounded, std::true_type(), with_residual);
-        else by_act(bounded, std::false_type(), with_residual);
-    };
-    auto by_edge = [&](auto with_residual) __attribute__((always_inline)) {
-        if (bm + G::DM <= M && bn + G::DN <= N) by_scale(std::false_type(), with_residual);
-        else by_scale(std::true_type(), with_residual);
-    };
-    if (residual) by_edge(std::true_type());
-    else by_edge(std::false_type());
+    if (bm + G::DM <= M && bn + G::DN <= N) by_edge(std::false_type());
+    else by_edge(std::true_type());
 }
 
 template <int T, bool BF16>
