@@ -122,6 +122,9 @@ VARIANTS = {
     "ks_no_dot": ("gemv_ks.hip", "the integer dot products (weight loads kept)", [(_KS_DOT, _KS_NO_DOT)], "gemv_ks_body.hpp"),
     "ks_no_epilogue": ("gemv_ks.hip", "the sum over the workgroup's wavefronts and the stores of y (the barrier stays)",
                        [(_KS_EPILOGUE, _KS_NO_EPILOGUE)], "gemv_ks_body.hpp"),
+    "ks_no_store": ("gemv_ks.hip", "the global stores of y only (the sum over the wavefronts and the barrier stay)",
+                    [("            y[at] = apply_act(act, t + (bias ? bias[row] : 0.f));\n",
+                      '            asm volatile("" ::"v"(apply_act(act, t + (bias ? bias[row] : 0.f))), "v"(at));\n')], "gemv_ks_body.hpp"),
     "q4k_no_image": ("mmq.hip", "the copy of the slice's activation image into LDS (main kernel)", [(_Q4K_IMAGE, "            (void)img;\n")]),
     "q4k_no_weights": ("mmq.hip", "the weight loads of the main kernel (it contracts whatever LDS holds)", [(_Q4K_FETCH0, ""), (_Q4K_FETCH, "")]),
     "q4k_no_contract": ("mmq.hip", "unpacking and MFMAs of the main kernel (loads and LDS reads kept)", [(_Q4K_CONTRACT, _Q4K_KEEP)]),
