@@ -202,20 +202,51 @@ int64_t weight_bytes_of(int type, int64_t K, int64_t N) { return (int64_t)gq_row
 // Last batch size of the split-K kernels before the two-pass GEMM takes over.  The split-K route streams W once per 32
 // batch rows; the two passes pay the 16-bit image (in proportion to N K) and a GEMM that, below a few hundred rows, has
 // only N / 64 workgroups walking all of K: cheap for a small matrix, costly for a long-K one (the down projection).
-// Measured (us per call in a replayed graph; rows 32 64 96 128 160 192 256; split-K | two passes, flat up to 128 rows):
-//   Q8_0   4096x4096  17 22 27 29 35 37 44 | 38-40    4096x14336  33 52  71  85 102 119 148 | 62-65, 80 from 160    14336x4096  33 52  72  85 104 124 153 |  95-109
-//   Q4_0   4096x4096  15 19 25 27 33 34 41 | 38-41    4096x14336  27 42  56  66  81  94 120 | 60-64, 80 from 160    14336x4096  28 43  57  69  83  97 122 |  92-103
-//   Q4_K   4096x4096  15 23 31 39 46 50 64 | 38-41    4096x14336  21 34  47  58  71  85 108 | 65-70, 85 from 160    14336x4096  22 35  49  61  74  87 113 |  98-108
-//   Q6_K   4096x4096  19 22 30 33 41 41  - | 37-41    4096x14336  36 56  78  92 111 133   - | 64-67, 84 from 160    14336x4096  37 57  79  94 114 136   - |  96-109
-//   IQ4_NL 4096x4096  16 21 27 29 36 38 45 | 40-42    4096x14336  30 47  64  75  92 108 137 | 68-75, 89 from 160    14336x4096  30 47  64  78  94 110 141 | 100-111
+// Measured (python -m gomlx_amd.tune.crossover with GOMLX_HIPQ_SPLIT_K_TO=100000 and =16: us per call in a replayed graph of 20
+// calls on rotating weights, fp32 activations; rows 32 64 96 128 160 192; split-K | two passes at the same rows):
+//   Q8_0   4096x4096  16 22 27 29 35 36 | 32 32 33 33 33 33    4096x14336  33 52  71  84 100 118 | 57 59 59 61 70 71    14336x4096  33 52 72 85 104 121 |  92  93  96  99  99  99
+//   Q4_0   4096x4096  15 20 25 26 32 33 | 33 33 33 33 33 33    4096x14336  27 42  56  66  80  94 | 55 55 56 56 71 70    14336x4096  28 43 57 68  83  97 |  91  92  94  97  97  97
+//   Q4_K   4096x4096  14 23 32 39 46 52 | 33 33 33 34 33 33    4096x14336  27 44  61  79  96 113 | 61 60 62 63 75 76    14336x4096  22 36 49 63  77  92 |  95  97 100 102 102 102
+//   Q6_K   4096x4096  19 22 30 32 39 40 | 33 33 34 34 34 34    4096x14336  36 56  76  89 109 130 | 59 58 60 61 75 75    14336x4096  36 56 77 90 111 132 |  93  93  96  99  99 100
+//   IQ4_NL 4096x4096  16 21 28 29 37 37 | 35 34 35 35 34 34    4096x14336  30 48  65  78  95 112 | 65 63 66 66 79 80    14336x4096  31 49 66 80  97 114 |  97  98 101 104 103 104
+// GOMLX_HIPQ_SPLIT_K_TO=rows overrides the table (tuning runs only).
+int64_t split_k_to_env() {
+    static const int64_t v = [] { const char *e = std::getenv("GOMLX_HIPQ_SPLIT_K_TO"); return e ? (int64_t)std::atoll(e) : (int64_t)-1; }();
+    return v;
+}
 int64_t split_k_to(int type, int64_t K, int64_t N) {
+    if (split_k_to_env() >= 0) return split_k_to_env();
     const bool large = weight_bytes_of(type, K, N) >= kLargeWeightBytes, long_k = K > N;
     switch (type) {
-    case GQ_Q8_0: return !large ? 192 : long_k ? 160 : 64;
-    case GQ_Q4_0: return !large ? 192 : long_k ? 192 : 96;
-    case GQ_Q4_K: return !large ? 128 : long_k ? 192 : 160;
+    case GQ_Q8_0: return !large ? 128 : long_k ? 128 : 64;
+    case GQ_Q4_0: return !large ? 160 : long_k ? 192 : 96;
+    case GQ_Q4_K: return !large ? 96 : long_k ? 192 : 96;
     case GQ_Q6_K: return !large ? 128 : long_k ? 128 : 64;
-    case GQ_IQ4_NL: return !large ? 192 : long_k ? 160 : 96;
+    case GQ_IQ4_NL: return !large ? 128 : long_k ? 160 : 96;
+    default: return 96;
+    }
+}
+
+// The same point for a gated pair act(x.Wgate) * (x.Wup): both matrices are contracted against one activation image by the
+// split-K kernels, or dequantised into one interleaved image for ONE GEMM by the two passes.  Measured (same tool, mode
+// `gated`, SiLU; rows 32 64 96 128 160 192 256; split-K | two passes):
+//   Q8_0   4096x4096  24 35 39 45 52 58 73 | 46 45 46 46 47 46 46    4096x14336  50 79 110 136 165 193 247 | 112 117 123 129 142 145 151
+//   Q4_0   4096x4096  20 27 34 41 47 52 66 | 45 44 44 45 45 45 45    4096x14336  42 62  86 107 132 153 199 | 107 114 121 118 138 133 141
+//   Q4_K   4096x4096  17 28 37 45 53 61 78 | 46 45 45 45 46 46 45    4096x14336  37 65  93 120 149 178 233 | 118 125 131 128 147 142 151
+//   Q6_K   4096x4096  28 33 43 51 59 67 85 | 46 46 46 46 47 46 46    4096x14336  57 89 129 161 200 231 302 | 112 117 124 127 138 137 146
+//   IQ4_NL 4096x4096  22 29 39 47 54 61 77 | 49 48 48 47 48 48 48    4096x14336  48 73 103 129 160 186 244 | 120 125 131 128 147 144 150
+// (The pair composed of two dense calls and a multiplication is never ahead of the one GEMM: 127 - 159 against 118 - 143 us
+// for Q4_K 4096 -> 2 x 14336 at 64 - 256 rows.)
+int64_t gated_split_k_to(int type, int64_t K, int64_t N) {
+    if (split_k_to_env() >= 0) return split_k_to_env();
+    const bool large = weight_bytes_of(type, K, N) >= kLargeWeightBytes, long_k = K > N;
+    if (large && long_k) return split_k_to(type, K, N);
+    switch (type) {
+    case GQ_Q8_0: return large ? 96 : 128;
+    case GQ_Q4_0: return large ? 160 : 128;
+    case GQ_Q4_K: return 128;
+    case GQ_Q6_K: return large ? 64 : 96;
+    case GQ_IQ4_NL: return 128;
     default: return 96;
     }
 }
@@ -550,9 +581,9 @@ bool fold_into_gemv(int type, int64_t M, int64_t K, int64_t N, const float *x, c
 
 // Whether a projection with its neighbours runs on the split-K kernels (after fold_into_gemv() has declined).
 bool block_takes_split_k(int type, int64_t M, int64_t K, int64_t N, const float *x, const float *bias, const float *y, bool gated) {
-    const bool tp = gemm_two_pass_supported(type, false, M, K, N, x);
-    return M >= block_split_k_from(type, weight_bytes_of(type, K, N), gated) && mmq_supported(type, M, K, N, x, bias, y) &&
-           (M <= split_k_to(type, K, N) || !tp);
+    const bool tp = gated ? gemm_two_pass_block_supported(type, M, K, N, x, true) : gemm_two_pass_supported(type, false, M, K, N, x);
+    const int64_t to = gated ? gated_split_k_to(type, K, N) : split_k_to(type, K, N);
+    return M >= block_split_k_from(type, weight_bytes_of(type, K, N), gated) && mmq_supported(type, M, K, N, x, bias, y) && (M <= to || !tp);
 }
 
 // Whether a plain dense call on these operands runs on the split-K kernels (the dispatch of gq_qdense_f32).
@@ -561,31 +592,42 @@ bool dense_takes_split_k(int type, int64_t M, int64_t K, int64_t N, const float 
     return M >= split_k_from(type, weight_bytes_of(type, K, N)) && mmq_supported(type, M, K, N, x, bias, y) && (M <= split_k_to(type, K, N) || !tp);
 }
 
+// First batch size of the gated pair as one GEMM (wherever the split-K kernels have handed over: the composed form is never
+// ahead); GOMLX_HIPQ_GATED_TWO_PASS_FROM=rows overrides it (tuning runs only).
+int64_t gated_two_pass_from() {
+    static const int64_t v = [] { const char *e = std::getenv("GOMLX_HIPQ_GATED_TWO_PASS_FROM"); return e ? (int64_t)std::atoll(e) : (int64_t)(kGemvMaxRows + 1); }();
+    return v;
+}
+
 // Batches that a plain dense call would hand to the two-pass GEMM take its block form: the
 // normalisation rides on the activation pass, the residual and the gated product on the epilogue.
 bool block_takes_two_pass(int type, int64_t M, int64_t K, int64_t N, const float *x, const float *gain, const float *bias, const float *y,
                           bool gated) {
     if (M <= kGemvMaxRows || !gemm_two_pass_block_supported(type, M, K, N, x, gated)) return false;
-    // A gated pair as one GEMM pays off from a few hundred rows (4096 -> 2 x 14336 in Q4_K: 237 against 255 us at 512 rows,
-    // 660 against 743 us at 2048; at 128 rows, where dequantising the two matrices dominates, 147 against 132 us).
-    if (gated && M < 256) return false;
+    if (gated && M < gated_two_pass_from()) return false;
     if (gain && !aligned_to(gain, 16)) return false;
-    const bool sk = M >= split_k_from(type, weight_bytes_of(type, K, N)) && mmq_supported(type, M, K, N, x, bias, y) && M <= split_k_to(type, K, N);
+    const int64_t to = gated ? gated_split_k_to(type, K, N) : split_k_to(type, K, N);
+    const bool sk = M >= split_k_from(type, weight_bytes_of(type, K, N)) && mmq_supported(type, M, K, N, x, bias, y) && M <= to;
     return !sk;
 }
 // Whether a list of projections is one input contracted with two to four matrices that the shared split-K pass takes
 // (launch_mmq_set): equal type, activations, rows and K, the matrices taken together in the split-K kernels' range.
+// Whether a list of two to four projections reads one input: equal type, activations, rows and K (fills `set`).
+bool same_input_set(int count, const gq_dense_desc *descs, MmqSetItem *set) {
+    if (count < 2 || count > 4) return false;
+    for (int i = 0; i < count; i++) {
+        const gq_dense_desc &d = descs[i];
+        if (d.type != descs[0].type || d.dX != descs[0].dX || d.M != descs[0].M || d.K != descs[0].K || d.N <= 0) return false;
+        set[i] = MmqSetItem{(const uint8_t *)d.dW, d.N, d.dBias, d.act, d.dY};
+    }
+    return true;
+}
 bool takes_shared_pass(int count, const gq_dense_desc *descs, const float *gain, MmqSetItem *set) {
-    if (count < 2 || count > 4 || (gain && !aligned_to(gain, 16))) return false;
+    if ((gain && !aligned_to(gain, 16)) || !same_input_set(count, descs, set)) return false;
     const int type = descs[0].type;
     const int64_t rows = descs[0].M, K = descs[0].K;
     int64_t ntot = 0;
-    for (int i = 0; i < count; i++) {
-        const gq_dense_desc &d = descs[i];
-        if (d.type != type || d.dX != descs[0].dX || d.M != rows || d.K != K || d.N <= 0) return false;
-        set[i] = MmqSetItem{(const uint8_t *)d.dW, d.N, d.dBias, d.act, d.dY};
-        ntot += d.N;
-    }
+    for (int i = 0; i < count; i++) ntot += descs[i].N;
     return mmq_set_supported(type, count, set, rows, K, descs[0].dX) &&
            rows >= block_split_k_from(type, weight_bytes_of(type, K, ntot), false) &&
            (rows <= split_k_to(type, K, ntot) || !gemm_two_pass_supported(type, false, rows, K, ntot, descs[0].dX));
@@ -689,6 +731,15 @@ int gq_qdense_norm_f32_batch(int count, const gq_dense_desc *descs, const gq_rms
     if (shared_pass) {
         const RmsNorm rn{norm->dGain, norm->eps, norm->gain_offset};
         return launch_mmq_set(descs[0].type, descs[0].dX, false, rows, descs[0].K, count, set, &rn, (hipStream_t)stream);
+    }
+    // Past the split-K range the same projections share the two passes: one activation conversion, one image of all the
+    // matrices, one GEMM (a decoder layer's q / k / v at 128 rows: two launches instead of six).
+    if (same_input_set(count, descs, set) && rows > kGemvMaxRows && (!norm->dGain || aligned_to(norm->dGain, 16)) &&
+        gemm_two_pass_set_supported(descs[0].type, count, set, rows, descs[0].K, descs[0].dX)) {
+        void *ws = nullptr;
+        if (int rc = stream_workspace((hipStream_t)stream, gemm_two_pass_set_workspace(count, set, rows, descs[0].K), &ws)) return rc;
+        const RmsNorm rn{norm->dGain, norm->eps, norm->gain_offset};
+        return launch_gemm_two_pass_set(descs[0].type, descs[0].dX, rows, descs[0].K, &rn, count, set, ws, (hipStream_t)stream);
     }
     for (int i = 0; i < count; i++) {
         const gq_dense_desc &d = descs[i];

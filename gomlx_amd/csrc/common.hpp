@@ -124,6 +124,12 @@ bool gemm_two_pass_block_supported(int type, int64_t M, int64_t K, int64_t N, co
 int launch_gemm_two_pass_block(int type, const float *x, int64_t M, int64_t K, const RmsNorm *norm, const uint8_t *W, const float *bias,
                                const uint8_t *W2, const float *bias2, const float *residual, int64_t N, int act, float *y, void *workspace,
                                hipStream_t s);
+// Two to four matrices against the same fp32 activations through the two passes: one activation conversion, one image, one
+// GEMM that writes each matrix's columns to its own output (every N a multiple of 32, one activation for all).
+bool gemm_two_pass_set_supported(int type, int count, const MmqSetItem *items, int64_t M, int64_t K, const void *x);
+size_t gemm_two_pass_set_workspace(int count, const MmqSetItem *items, int64_t M, int64_t K);
+int launch_gemm_two_pass_set(int type, const float *x, int64_t M, int64_t K, const RmsNorm *norm, int count, const MmqSetItem *items, void *workspace,
+                             hipStream_t s);
 int launch_gemm(int type, bool x_is_bf16, const void *x, int64_t M, int64_t K, const uint8_t *W, int64_t N,
                 const float *bias, int act, float *y, hipStream_t s);
 

@@ -296,10 +296,20 @@ template <int TM, int TN> struct DmaTile {
 // GATED (TN == 2): Wh is the interleaved image of a gated pair (N counts its rows); column block j = 0
 // of a wavefront's tile is the first projection, j = 1 the second, of the same 32 outputs, and the
 // result is act(first + bias) * (second + bias2) in a [M, n_out] matrix.
-template <bool BF16, int TM, int TN, bool GATED = false>
+// SEGS: the image is several matrices one after the other (N counts all their rows) and the columns of the result go to
+// one output matrix per segment: columns n0[i] .. n0[i + 1] - 1 to y[i] (row length n0[i + 1] - n0[i]) with bias[i]; the
+// boundaries are multiples of 32, so a wavefront's block of 32 columns lies in one segment.
+struct GemmSegs {
+    float *y[4];
+    const float *bias[4];
+    int n0[5];
+    int count;
+};
+
+template <bool BF16, int TM, int TN, bool GATED = false, bool SEGS = false>
 __global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const uint16_t *Wh, const float *__restrict__ bias,
                                                        float *Y, int M, int K, int N, int act, const float *__restrict__ bias2, int n_out,
-                                                       const float *residual, const float *__restrict__ rowscale) {
+                                                       const float *residual, const float *__restrict__ rowscale, GemmSegs segs) {
     typedef Op16<BF16> Op;
     typedef DmaTile<TM, TN> G;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -456,11 +466,27 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const 
         else by_edge(std::true_type());
         return;
     }
+    float *const Yall = Y;
+    const float *const bias_all = bias;
+    const int Nall = N;
     auto store_all = [&](auto bounded, auto scaled, auto with_residual, auto activate) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < TN; j++) {
-            const int n = bn + wn + j * 32 + (lane & 31);
+            int n = bn + wn + j * 32 + (lane & 31);
             if constexpr (decltype(bounded)::value) { if (n >= N) continue; }
+            float *Y = Yall;               // (shadow the kernel's arguments: a segment brings its own output, row length and bias)
+            const float *bias = bias_all;
+            int N = Nall;
+            if constexpr (SEGS) {
+                int sg = 0;
+#pragma unroll
+                for (int q = 1; q < 4; q++)
+                    if (q < segs.count && n >= segs.n0[q]) sg = q;
+                Y = segs.y[sg];
+                bias = segs.bias[sg];
+                N = segs.n0[sg + 1] - segs.n0[sg];
+                n -= segs.n0[sg];
+            }
             const float bv = bias ? bias[n] : 0.f;
             const int64_t at0 = (int64_t)m0 * N + n;
 #pragma unroll
@@ -525,71 +551,100 @@ int launch_dequant16bit_type(int type, const uint8_t *W, int64_t N, int64_t K, u
 // Both pre-passes of the fp32-activation route in ONE launch (they do not depend on each other): the first M workgroups
 // convert an activation row each (x_row_to_f16_body), the others 256 runs of weights each (dequant16bit_body), of W and -
 // for a gated pair, whose images interleave - of W2.  Rows of up to 8192 values (longer ones keep their own two-read kernel).
+// The matrices of one pre-pass: matrix i is W[i] with rows[i] rows, written from image row row0[i] on with the interleaving
+// `half[i]` of dequant16bit_body (a gated pair: both matrices at row 0 with halves 1 and 2; a set: halves 0, one after the other).
+struct PrepMatrices {
+    const uint8_t *W[4];
+    uint32_t rows[4], row0[4], blocks_end[4];  // blocks_end[i]: workgroups of matrices 0 .. i
+    int half[4], count;
+};
+
 template <int T, int IT, bool NORM>
 __global__ __launch_bounds__(256) void prep_f32_kernel(const float *__restrict__ X, const float *__restrict__ gain, float gain_offset, float eps, int K,
-                                                       uint16_t *__restrict__ xh, float *__restrict__ rowscale, uint32_t xblocks,
-                                                       const uint8_t *__restrict__ W, const uint8_t *__restrict__ W2, uint16_t *__restrict__ wh,
-                                                       uint32_t runs_per_row, uint32_t total_runs, int64_t row_bytes, uint32_t runs, uint32_t wblocks) {
+                                                       uint16_t *__restrict__ xh, float *__restrict__ rowscale, uint32_t xblocks, PrepMatrices pm,
+                                                       uint16_t *__restrict__ wh, uint32_t runs_per_row, int64_t row_bytes, uint32_t runs) {
     const uint32_t b = blockIdx.x;
     if (b < xblocks) {
         x_row_to_f16_body<IT, NORM>(X, gain, gain_offset, eps, K, xh, rowscale, b);
-    } else if (b - xblocks < wblocks) {
-        dequant16bit_body<T, false>(W, wh, runs_per_row, total_runs, row_bytes, W2 ? 1 : 0, runs, b - xblocks);
-    } else {
-        dequant16bit_body<T, false>(W2, wh, runs_per_row, total_runs, row_bytes, 2, runs, b - xblocks - wblocks);
+        return;
     }
+    const uint32_t wb = b - xblocks;
+    int i = 0;
+#pragma unroll
+    for (int q = 1; q < 4; q++)
+        if (q < pm.count && wb >= pm.blocks_end[q - 1]) i = q;
+    const uint32_t first = i ? pm.blocks_end[i - 1] : 0u;
+    dequant16bit_body<T, false>(pm.W[i], wh + (size_t)pm.row0[i] * runs_per_row * 16, runs_per_row, pm.rows[i] * runs_per_row, row_bytes, pm.half[i], runs,
+                                wb - first);
 }
 
 template <int T>
-int launch_prep_f32_t(const float *x, int64_t M, int64_t K, const RmsNorm *norm, uint16_t *xh, float *rowscale, const uint8_t *W, const uint8_t *W2,
-                      int64_t N, uint16_t *wh, hipStream_t s) {
-    const int64_t runs = K / 16, runs_per_row = padded_k(K) / 16, total = N * runs_per_row;
+int launch_prep_f32_t(const float *x, int64_t M, int64_t K, const RmsNorm *norm, uint16_t *xh, float *rowscale, PrepMatrices pm, uint16_t *wh,
+                      hipStream_t s) {
+    const int64_t runs = K / 16, runs_per_row = padded_k(K) / 16;
     const int64_t row_bytes = (K / Geom<T>::vpb) * Geom<T>::bpb;
-    if (total > ((int64_t)1 << 27)) return fail(GQ_ERR_INVALID, "gemm: a 16-bit image of %lld x %lld values is too large", (long long)N, (long long)K);
-    const int64_t wblocks = (total + 255) / 256, blocks = M + wblocks * (W2 ? 2 : 1);
+    int64_t wblocks = 0;
+    for (int i = 0; i < pm.count; i++) {
+        const int64_t total = (int64_t)pm.rows[i] * runs_per_row;
+        if (total > ((int64_t)1 << 27)) return fail(GQ_ERR_INVALID, "gemm: a 16-bit image of %u x %lld values is too large", pm.rows[i], (long long)K);
+        wblocks += (total + 255) / 256;
+        if (wblocks > INT32_MAX) return fail(GQ_ERR_INVALID, "gemm: too many workgroups in the pre-pass");
+        pm.blocks_end[i] = (uint32_t)wblocks;
+    }
+    const int64_t blocks = M + wblocks;
     if (blocks > INT32_MAX) return fail(GQ_ERR_INVALID, "gemm: too many workgroups in the pre-pass");
     const float *gain = norm ? norm->gain : nullptr;
     const float off = norm ? norm->gain_offset : 0.f, eps = norm ? norm->eps : 0.f;
     const dim3 grid((unsigned)blocks), block(256);
     auto go = [&](auto kernel) {
-        return launch(kernel, grid, block, 0, s, x, gain, off, eps, (int)K, xh, rowscale, (uint32_t)M, W, W2, wh, (uint32_t)runs_per_row, (uint32_t)total,
-                      row_bytes, (uint32_t)runs, (uint32_t)wblocks);
+        return launch(kernel, grid, block, 0, s, x, gain, off, eps, (int)K, xh, rowscale, (uint32_t)M, pm, wh, (uint32_t)runs_per_row, row_bytes, (uint32_t)runs);
     };
     if (padded_k(K) <= 4096) return norm ? go(prep_f32_kernel<T, 2, true>) : go(prep_f32_kernel<T, 2, false>);
     return norm ? go(prep_f32_kernel<T, 4, true>) : go(prep_f32_kernel<T, 4, false>);
 }
 
-// x -> fp16 rows and W (and W2) -> fp16 image: one launch for rows of up to 8192 values, else one per operand
-int launch_prep_f32(int type, const float *x, int64_t M, int64_t K, const RmsNorm *norm, uint16_t *xh, float *rowscale, const uint8_t *W,
-                    const uint8_t *W2, int64_t N, uint16_t *wh, hipStream_t s) {
+// x -> fp16 rows and the matrices -> fp16 image: one launch for rows of up to 8192 values, else one per operand
+int launch_prep_f32(int type, const float *x, int64_t M, int64_t K, const RmsNorm *norm, uint16_t *xh, float *rowscale, const PrepMatrices &pm,
+                    uint16_t *wh, hipStream_t s) {
     if (padded_k(K) > 8192) {
         if (int rc = launch_x_to_f16(x, M, K, norm, xh, rowscale, s)) return rc;
-        if (int rc = launch_dequant16bit_type<false>(type, W, N, K, wh, s, W2 ? 1 : 0)) return rc;
-        return W2 ? launch_dequant16bit_type<false>(type, W2, N, K, wh, s, 2) : GQ_OK;
+        for (int i = 0; i < pm.count; i++)
+            if (int rc = launch_dequant16bit_type<false>(type, pm.W[i], pm.rows[i], K, wh + (size_t)pm.row0[i] * padded_k(K), s, pm.half[i])) return rc;
+        return GQ_OK;
     }
     switch (type) {
-    case kQ4_0: return launch_prep_f32_t<kQ4_0>(x, M, K, norm, xh, rowscale, W, W2, N, wh, s);
-    case kQ8_0: return launch_prep_f32_t<kQ8_0>(x, M, K, norm, xh, rowscale, W, W2, N, wh, s);
-    case kIQ4_NL: return launch_prep_f32_t<kIQ4_NL>(x, M, K, norm, xh, rowscale, W, W2, N, wh, s);
-    case kQ4_K: return launch_prep_f32_t<kQ4_K>(x, M, K, norm, xh, rowscale, W, W2, N, wh, s);
-    case kQ6_K: return launch_prep_f32_t<kQ6_K>(x, M, K, norm, xh, rowscale, W, W2, N, wh, s);
+    case kQ4_0: return launch_prep_f32_t<kQ4_0>(x, M, K, norm, xh, rowscale, pm, wh, s);
+    case kQ8_0: return launch_prep_f32_t<kQ8_0>(x, M, K, norm, xh, rowscale, pm, wh, s);
+    case kIQ4_NL: return launch_prep_f32_t<kIQ4_NL>(x, M, K, norm, xh, rowscale, pm, wh, s);
+    case kQ4_K: return launch_prep_f32_t<kQ4_K>(x, M, K, norm, xh, rowscale, pm, wh, s);
+    case kQ6_K: return launch_prep_f32_t<kQ6_K>(x, M, K, norm, xh, rowscale, pm, wh, s);
     default: return fail(GQ_ERR_NOT_IMPLEMENTED, "qdense: ggml type %d is not implemented", type);
     }
 }
 
+// one matrix, or the two of a gated pair
+PrepMatrices prep_one_or_pair(const uint8_t *W, const uint8_t *W2, int64_t N) {
+    PrepMatrices pm{};
+    pm.count = W2 ? 2 : 1;
+    pm.W[0] = W; pm.rows[0] = (uint32_t)N; pm.row0[0] = 0; pm.half[0] = W2 ? 1 : 0;
+    pm.W[1] = W2; pm.rows[1] = (uint32_t)N; pm.row0[1] = 0; pm.half[1] = 2;
+    return pm;
+}
+
 // N counts the rows of the weight image (for a gated pair: both halves, 64 per 32 outputs)
-template <bool BF16, int TM, int TN, bool GATED = false>
+template <bool BF16, int TM, int TN, bool GATED = false, bool SEGS = false>
 int launch_gemm16_tile(const uint16_t *x, int64_t M, int64_t K, const uint16_t *Wh, int64_t N, const float *bias, int act, float *y,
-                       const float *bias2, int64_t n_out, const float *residual, const float *rowscale, hipStream_t s) {
+                       const float *bias2, int64_t n_out, const float *residual, const float *rowscale, hipStream_t s,
+                       const GemmSegs *segs = nullptr) {
     typedef DmaTile<TM, TN> G;
     static const bool lds_ok = [] {
-        return hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_dma_kernel<BF16, TM, TN, GATED>),
+        return hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_dma_kernel<BF16, TM, TN, GATED, SEGS>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, G::kLdsBytes) == hipSuccess;
     }();
     if (!lds_ok) return fail(GQ_ERR_HIP, "gemm: cannot reserve %d bytes of LDS", G::kLdsBytes);
     const dim3 grid((unsigned)((N + G::DN - 1) / G::DN), (unsigned)((M + G::DM - 1) / G::DM));
-    return launch(gemm_dma_kernel<BF16, TM, TN, GATED>, grid, dim3(512), (size_t)G::kLdsBytes, s, x, Wh, bias, y, (int)M, (int)K, (int)N, act,
-                  bias2, (int)n_out, residual, rowscale);
+    return launch(gemm_dma_kernel<BF16, TM, TN, GATED, SEGS>, grid, dim3(512), (size_t)G::kLdsBytes, s, x, Wh, bias, y, (int)M, (int)K, (int)N, act,
+                  bias2, (int)n_out, residual, rowscale, segs ? *segs : GemmSegs{});
 }
 
 // GOMLX_HIPQ_GEMM_TILE=0|1|2 forces the 256x128 / 128x128 / 128x64 tile (tuning runs only).
@@ -627,6 +682,18 @@ int launch_gemm16(const uint16_t *x, int64_t M, int64_t K, const uint16_t *Wh, i
     case 0: return launch_gemm16_tile<BF16, 2, 2>(x, M, K, Wh, N, bias, act, y, nullptr, N, residual, rowscale, s);
     case 1: return launch_gemm16_tile<BF16, 1, 2>(x, M, K, Wh, N, bias, act, y, nullptr, N, residual, rowscale, s);
     default: return launch_gemm16_tile<BF16, 1, 1>(x, M, K, Wh, N, bias, act, y, nullptr, N, residual, rowscale, s);
+    }
+}
+
+// Several matrices' images one after the other, one GEMM, each segment's columns to its own output (fp16 operands).
+int launch_gemm16_set(const uint16_t *x, int64_t M, int64_t K, const uint16_t *Wh, const GemmSegs &segs, int act, const float *rowscale, hipStream_t s) {
+    const int64_t N = segs.n0[segs.count];
+    int choice = pick_tile(M, N);
+    if (tile_env() >= 0 && tile_env() <= 2) choice = tile_env();
+    switch (choice) {
+    case 0: return launch_gemm16_tile<false, 2, 2, false, true>(x, M, K, Wh, N, nullptr, act, nullptr, nullptr, N, nullptr, rowscale, s, &segs);
+    case 1: return launch_gemm16_tile<false, 1, 2, false, true>(x, M, K, Wh, N, nullptr, act, nullptr, nullptr, N, nullptr, rowscale, s, &segs);
+    default: return launch_gemm16_tile<false, 1, 1, false, true>(x, M, K, Wh, N, nullptr, act, nullptr, nullptr, N, nullptr, rowscale, s, &segs);
     }
 }
 
@@ -685,7 +752,7 @@ int launch_gemm_two_pass(int type, bool x_is_bf16, const void *x, int64_t M, int
     const int64_t Kp = padded_k(K);
     uint16_t *xh = wh + (((size_t)N * Kp * 2 + 255) & ~(size_t)255) / 2;
     float *rowscale = reinterpret_cast<float *>(xh + (((size_t)M * Kp * 2 + 255) & ~(size_t)255) / 2);
-    if (int rc = launch_prep_f32(type, static_cast<const float *>(x), M, K, nullptr, xh, rowscale, W, nullptr, N, wh, s)) return rc;
+    if (int rc = launch_prep_f32(type, static_cast<const float *>(x), M, K, nullptr, xh, rowscale, prep_one_or_pair(W, nullptr, N), wh, s)) return rc;
     return launch_gemm16<false>(xh, M, Kp, wh, N, bias, act, y, s, nullptr, rowscale);
 }
 
@@ -712,9 +779,49 @@ int launch_gemm_two_pass_block(int type, const float *x, int64_t M, int64_t K, c
     const int64_t Kp = padded_k(K);
     uint16_t *xh = wh + (((size_t)rows * Kp * 2 + 255) & ~(size_t)255) / 2;
     float *rowscale = reinterpret_cast<float *>(xh + (((size_t)M * Kp * 2 + 255) & ~(size_t)255) / 2);
-    if (int rc = launch_prep_f32(type, x, M, K, norm, xh, rowscale, W, W2, N, wh, s)) return rc;
+    if (int rc = launch_prep_f32(type, x, M, K, norm, xh, rowscale, prep_one_or_pair(W, W2, N), wh, s)) return rc;
     if (!W2) return launch_gemm16<false>(xh, M, Kp, wh, N, bias, act, y, s, residual, rowscale);
     return launch_gemm16_gated(xh, M, Kp, wh, N, bias, bias2, act, y, residual, rowscale, s);
+}
+
+// Two to four matrices of one K against the same fp32 activations (the q / k / v projections behind one normalisation) at
+// the batch sizes of the two-pass GEMM: the activations are converted ONCE, the matrices' images follow each other in
+// one image, and ONE GEMM writes each matrix's columns to its own output - two launches where separate calls take six and
+// convert the activations three times.  Every N a multiple of 32, one activation for all.
+bool gemm_two_pass_set_supported(int type, int count, const MmqSetItem *items, int64_t M, int64_t K, const void *x) {
+    if (count < 2 || count > 4) return false;
+    int64_t ntot = 0;
+    for (int i = 0; i < count; i++) {
+        if (items[i].N <= 0 || items[i].N % 32 != 0 || items[i].act != items[0].act) return false;
+        ntot += items[i].N;
+    }
+    return gemm_two_pass_supported(type, false, M, K, ntot, x);
+}
+
+size_t gemm_two_pass_set_workspace(int count, const MmqSetItem *items, int64_t M, int64_t K) {
+    int64_t ntot = 0;
+    for (int i = 0; i < count; i++) ntot += items[i].N;
+    return gemm_two_pass_block_workspace(M, K, ntot, false);
+}
+
+int launch_gemm_two_pass_set(int type, const float *x, int64_t M, int64_t K, const RmsNorm *norm, int count, const MmqSetItem *items, void *workspace,
+                             hipStream_t s) {
+    PrepMatrices pm{};
+    GemmSegs segs{};
+    pm.count = segs.count = count;
+    int64_t ntot = 0;
+    for (int i = 0; i < count; i++) {
+        pm.W[i] = items[i].W; pm.rows[i] = (uint32_t)items[i].N; pm.row0[i] = (uint32_t)ntot; pm.half[i] = 0;
+        segs.y[i] = items[i].y; segs.bias[i] = items[i].bias; segs.n0[i] = (int)ntot;
+        ntot += items[i].N;
+    }
+    segs.n0[count] = (int)ntot;
+    uint16_t *wh = static_cast<uint16_t *>(workspace);
+    const int64_t Kp = padded_k(K);
+    uint16_t *xh = wh + (((size_t)ntot * Kp * 2 + 255) & ~(size_t)255) / 2;
+    float *rowscale = reinterpret_cast<float *>(xh + (((size_t)M * Kp * 2 + 255) & ~(size_t)255) / 2);
+    if (int rc = launch_prep_f32(type, x, M, K, norm, xh, rowscale, pm, wh, s)) return rc;
+    return launch_gemm16_set(xh, M, Kp, wh, segs, items[0].act, rowscale, s);
 }
 
 }  // namespace gq

@@ -499,6 +499,21 @@ def test_small_batches_on_large_matrices(gpu, oracle, t, N):
         assert rel_err(run_dense(gpu, t, xb, W, bias, 3, bf16=True), oracle.c_qdense(t, xb, W, bias, 3)) < TOL_BF16, (t, M)
 
 
+@pytest.mark.parametrize("t", ALL_TYPES)
+def test_hand_over_from_split_k_to_the_two_passes(gpu, oracle, t):
+    """A 4096 x 2048 matrix (between 6 and 24 MB in every format): the split-K kernels hand over to the two-pass GEMM after
+    96, 128 or 160 rows depending on the format; both sides of each of those points, fp32 and bf16 activations."""
+    K, N = 4096, 2048 if t != Q4_0 and t != IQ4_NL and t != Q4_K else 3072
+    assert 6 << 20 <= N * ggml.row_bytes(t, K) < 24 << 20
+    W = synth.weights(t, 350 + t, N, K)
+    for M in (96, 97, 128, 129, 160, 161):
+        x = synth.activations(351 + M, M, K)
+        assert rel_err(run_dense(gpu, t, x, W), oracle.c_qdense(t, x, W)) < TOL_F32, (t, M)
+    for M in (97, 129):
+        xb = bf16_round(synth.activations(360 + M, M, K))
+        assert rel_err(run_dense(gpu, t, xb, W, bf16=True), oracle.c_qdense(t, xb, W)) < TOL_BF16, (t, M)
+
+
 @pytest.mark.parametrize("t,N", [(Q8_0, 3328), (Q4_K, 5632), (Q6_K, 4096)])
 def test_small_batches_with_neighbours_on_large_matrices(gpu, oracle, t, N):
     """The same batches through the calls around a projection: passes of two rows inside the decode GEMV up to the
@@ -1040,6 +1055,46 @@ def test_batched_projections_behind_one_norm(gpu, oracle, t):
         gpu.cuda.synchronize()
         for x, W, b, y in zip(xs, Ws, bs, plain):
             assert rel_err(y.cpu().numpy(), oracle.c_qdense(t, x, W, b)) < TOL_F32
+
+
+@pytest.mark.parametrize("t", ALL_TYPES)
+def test_projections_of_one_input_share_the_two_passes(gpu, oracle, t):
+    """q / k / v past the split-K range: the activations are normalised and converted once, the matrices' 16-bit images
+    follow each other and ONE GEMM writes each matrix's columns to its own output (widths that are multiples of 32, one
+    activation for all, each with or without bias).  Checked against the oracle; row counts on and off the tiles, two to
+    four matrices; a width that is not a multiple of 32 and mixed activations take the separate calls."""
+    K = 1024
+    gain = (synth.normal(1770, 0, K) * 0.5 + 1.0).astype(np.float32)
+    cfg = nn.RMSNorm(dev(gpu, gain), 1e-5, 0.0)
+    q = Quantization(ggml_type=t)
+    widths = (512, 128, 96, 64)
+    Ws = [synth.weights(t, 1772 + j, n, K) for j, n in enumerate(widths)]
+    bs = [None, synth.normal(1775, 0, 128).astype(np.float32) * 0.1, None, synth.normal(1776, 0, 64).astype(np.float32) * 0.1]
+    for rows in (130, 256, 300):
+        x = synth.activations(1771 + rows, rows, K)
+        xd = dev(gpu, x)
+        xn = oracle.c_rmsnorm(x, gain, 1e-5, 0.0)
+        for count in (3, 2, 4):
+            outs = nn.quantized_dense_batch([(xd, dev(gpu, W), q, None if b is None else dev(gpu, b), None) for W, b in zip(Ws[:count], bs)], norm=cfg)
+            gpu.cuda.synchronize()
+            for W, b, y in zip(Ws, bs, outs):
+                assert rel_err(y.cpu().numpy(), oracle.c_qdense(t, xn, W, b)) < TOL_F32, (ggml.name(t), rows, count, W.shape)
+    # one activation for all: SiLU
+    outs = nn.quantized_dense_batch([(xd, dev(gpu, W), q, None, BACKEND_ACT[3]) for W in Ws[:3]], norm=cfg)
+    for W, y in zip(Ws, outs):
+        assert rel_err(y.cpu().numpy(), oracle.c_qdense(t, xn, W, None, 3)) < TOL_F32
+    # outside the shared form: a width of 100, and mixed activations
+    odd = synth.weights(t, 1790, 100, K)
+    outs = nn.quantized_dense_batch([(xd, dev(gpu, Ws[0]), q, None, None), (xd, dev(gpu, odd), q, None, None)], norm=cfg)
+    assert rel_err(outs[1].cpu().numpy(), oracle.c_qdense(t, xn, odd, None)) < TOL_F32
+    outs = nn.quantized_dense_batch([(xd, dev(gpu, Ws[0]), q, None, None), (xd, dev(gpu, Ws[1]), q, None, BACKEND_ACT[2])], norm=cfg)
+    assert rel_err(outs[1].cpu().numpy(), oracle.c_qdense(t, xn, Ws[1], None, 2)) < TOL_F32
+    # bf16 activations behind the normalisation: widened exactly, then the same route
+    xb = bf16_round(x)
+    outs = nn.quantized_dense_batch([(dev(gpu, xb).to(gpu.bfloat16), dev(gpu, W), q, None, None) for W in Ws[:3]], norm=cfg)
+    same = nn.quantized_dense_batch([(dev(gpu, xb), dev(gpu, W), q, None, None) for W in Ws[:3]], norm=cfg)
+    for y, ref in zip(outs, same):
+        assert gpu.equal(y, ref)
 
 
 @pytest.mark.parametrize("rows,K", [(6, 2048), (8, 4096), (12, 2048), (32, 4096), (70, 2048), (33, 1536)])
