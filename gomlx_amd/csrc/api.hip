@@ -200,15 +200,16 @@ int64_t split_k_from(int type, int64_t weight_bytes) {
 }
 int64_t weight_bytes_of(int type, int64_t K, int64_t N) { return (int64_t)gq_row_bytes(type, K) * N; }
 // Last batch size of the split-K kernels before the two-pass GEMM takes over.  The split-K route streams W once per 32
-// batch rows; the two passes pay the 16-bit image (in proportion to N K) and a GEMM that, below a few hundred rows, has
-// only N / 64 workgroups walking all of K: cheap for a small matrix, costly for a long-K one (the down projection).
+// batch rows; the two passes pay the 16-bit image (written once and read once, in proportion to N K) and a GEMM that splits
+// K itself while its tiles are fewer than the CUs.
 // Measured (python -m gomlx_amd.tune.crossover with GOMLX_HIPQ_SPLIT_K_TO=100000 and =16: us per call in a replayed graph of 20
 // calls on rotating weights, fp32 activations; rows 32 64 96 128 160 192; split-K | two passes at the same rows):
-//   Q8_0   4096x4096  16 22 27 29 35 36 | 32 32 33 33 33 33    4096x14336  33 52  71  84 100 118 | 57 59 59 61 70 71    14336x4096  33 52 72 85 104 121 |  92  93  96  99  99  99
-//   Q4_0   4096x4096  15 20 25 26 32 33 | 33 33 33 33 33 33    4096x14336  27 42  56  66  80  94 | 55 55 56 56 71 70    14336x4096  28 43 57 68  83  97 |  91  92  94  97  97  97
-//   Q4_K   4096x4096  14 23 32 39 46 52 | 33 33 33 34 33 33    4096x14336  27 44  61  79  96 113 | 61 60 62 63 75 76    14336x4096  22 36 49 63  77  92 |  95  97 100 102 102 102
-//   Q6_K   4096x4096  19 22 30 32 39 40 | 33 33 34 34 34 34    4096x14336  36 56  76  89 109 130 | 59 58 60 61 75 75    14336x4096  36 56 77 90 111 132 |  93  93  96  99  99 100
-//   IQ4_NL 4096x4096  16 21 28 29 37 37 | 35 34 35 35 34 34    4096x14336  30 48  65  78  95 112 | 65 63 66 66 79 80    14336x4096  31 49 66 80  97 114 |  97  98 101 104 103 104
+//   Q8_0   4096x4096  16 22 27 29 35 36 | 27 28 29 30 31 31    4096x14336  33 52  71  84 100 118 | 56 56 55 58 69 69    14336x4096  33 52 72 85 104 121 | 63 70 72 73 81 82
+//   Q4_0   4096x4096  15 20 25 26 32 33 | 25 26 26 27 29 29    4096x14336  27 42  56  66  80  94 | 57 55 55 56 67 69    14336x4096  28 43 57 68  83  97 | 62 63 69 68 79 79
+//   Q4_K   4096x4096  14 23 32 39 46 52 | 26 26 27 29 30 30    4096x14336  27 44  61  79  96 113 | 61 59 60 60 73 72    14336x4096  22 36 49 63  77  92 | 69 73 72 71 85 85
+//   Q6_K   4096x4096  19 22 30 32 39 40 | 26 28 29 30 31 32    4096x14336  36 56  76  89 109 130 | 61 57 58 59 70 71    14336x4096  36 56 77 90 111 132 | 68 68 74 74 82 83
+//   IQ4_NL 4096x4096  16 21 28 29 37 37 | 27 28 29 30 31 32    4096x14336  30 48  65  78  95 112 | 63 62 62 64 76 77    14336x4096  31 49 66 80  97 114 | 70 75 78 78 87 88
+// (Before the GEMM split K on narrow problems the two passes took 33 us on 4096x4096 and 92 .. 102 us on 14336x4096 at these rows.)
 // GOMLX_HIPQ_SPLIT_K_TO=rows overrides the table (tuning runs only).
 int64_t split_k_to_env() {
     static const int64_t v = [] { const char *e = std::getenv("GOMLX_HIPQ_SPLIT_K_TO"); return e ? (int64_t)std::atoll(e) : (int64_t)-1; }();
@@ -218,11 +219,11 @@ int64_t split_k_to(int type, int64_t K, int64_t N) {
     if (split_k_to_env() >= 0) return split_k_to_env();
     const bool large = weight_bytes_of(type, K, N) >= kLargeWeightBytes, long_k = K > N;
     switch (type) {
-    case GQ_Q8_0: return !large ? 128 : long_k ? 128 : 64;
-    case GQ_Q4_0: return !large ? 160 : long_k ? 192 : 96;
-    case GQ_Q4_K: return !large ? 96 : long_k ? 192 : 96;
-    case GQ_Q6_K: return !large ? 128 : long_k ? 128 : 64;
-    case GQ_IQ4_NL: return !large ? 128 : long_k ? 160 : 96;
+    case GQ_Q8_0: return !large ? 128 : long_k ? 96 : 64;
+    case GQ_Q4_0: return !large ? 128 : long_k ? 128 : 96;
+    case GQ_Q4_K: return !large ? 64 : long_k ? 160 : 96;
+    case GQ_Q6_K: return !large ? 96 : 64;
+    case GQ_IQ4_NL: return !large ? 128 : long_k ? 128 : 64;
     default: return 96;
     }
 }

@@ -21,6 +21,7 @@
 #include "blocks.hpp"
 #include "common.hpp"
 
+#include <algorithm>
 #include <type_traits>
 
 #include <cstdlib>
@@ -299,6 +300,8 @@ template <int TM, int TN> struct DmaTile {
 // SEGS: the image is several matrices one after the other (N counts all their rows) and the columns of the result go to
 // one output matrix per segment: columns n0[i] .. n0[i + 1] - 1 to y[i] (row length n0[i + 1] - n0[i]) with bias[i]; the
 // boundaries are multiples of 32, so a wavefront's block of 32 columns lies in one segment.
+// gridDim.z > 1 (not GATED): K is split into that many slices of whole steps; slice z contracts its steps only and writes
+// its [M, N] sums behind those of the slices before it (Y + z M N), for gemm_slices_reduce_kernel to add up and finish.
 struct GemmSegs {
     float *y[4];
     const float *bias[4];
@@ -317,7 +320,9 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int bm = blockIdx.y * G::DM, bn = blockIdx.x * G::DN;
     const int wm = (wave >> 1) * (32 * TM), wn = (wave & 1) * (32 * TN);
-    const int nk = K / DK;
+    const int nk_all = K / DK, nk_slice = (nk_all + (int)gridDim.z - 1) / (int)gridDim.z;
+    const int k0 = (int)blockIdx.z * nk_slice;       // (the host gives every slice at least one step)
+    const int nk = min(nk_slice, nk_all - k0);
 
     // ---- DMA roles: per step a wavefront moves XI row blocks (8 rows each) of X and WI of W
     const i32x4 xrsrc = make_rsrc(X + (int64_t)bm * K, (uint64_t)(M - bm) * (uint64_t)K * 2);
@@ -339,7 +344,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const 
     const uint32_t xdst = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)(G::XI * wave) * 1024u);
     const uint32_t wdst = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t)(G::DM * ROWB) + (uint32_t)(G::WI * wave) * 1024u);
     auto issue = [&](int kt, int stage) __attribute__((always_inline)) {  // steps past the end re-read the last one (the data is never used)
-        const uint32_t soff = (uint32_t)min(kt, nk - 1) * (uint32_t)(DK * 2);
+        const uint32_t soff = (uint32_t)(k0 + min(kt, nk - 1)) * (uint32_t)(DK * 2);
         const uint32_t sb = (uint32_t)stage * (uint32_t)G::kStageBytes;
 #pragma unroll
         for (int j = 0; j < G::XI; j++) dma16(xdst + sb + (uint32_t)j * 1024u, xrsrc, xvoff[j], soff);
@@ -466,7 +471,7 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const 
         else by_edge(std::true_type());
         return;
     }
-    float *const Yall = Y;
+    float *const Yall = Y + (int64_t)blockIdx.z * (int64_t)M * (int64_t)N;
     const float *const bias_all = bias;
     const int Nall = N;
     auto store_all = [&](auto bounded, auto scaled, auto with_residual, auto activate) __attribute__((always_inline)) {
@@ -525,6 +530,42 @@ __global__ __launch_bounds__(512) void gemm_dma_kernel(const uint16_t *X, const 
     };
     if (bm + G::DM <= M && bn + G::DN <= N) by_edge(std::false_type());
     else by_edge(std::true_type());
+}
+
+// The sums of a GEMM whose K was split into slices: partial[z][m][n] added in slice order, then what the GEMM's own
+// epilogue does for an unsplit one - row scale, bias, activation, residual (which may be Y itself), and with segments
+// each column to its matrix's output.  N and the segment boundaries are multiples of 4: a thread owns four columns of a row.
+__global__ __launch_bounds__(256) void gemm_slices_reduce_kernel(const float *__restrict__ partial, int slices, int M, int N,
+                                                                 const float *__restrict__ rowscale, const float *__restrict__ bias, int act,
+                                                                 const float *residual, float *Y, GemmSegs segs, int use_segs) {
+    const int64_t MN = (int64_t)M * N;
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= MN) return;
+    const int m = MN <= (int64_t)INT32_MAX ? (int)((uint32_t)i / (uint32_t)N) : (int)(i / N);
+    int n = (int)(i - (int64_t)m * N);
+    float4 v[8];  // (eight slices at most: all loads issued before the first sum)
+#pragma unroll
+    for (int z = 0; z < 8; z++) v[z] = *reinterpret_cast<const float4 *>(partial + (int64_t)min(z, slices - 1) * MN + i);
+    float4 t = v[0];
+#pragma unroll
+    for (int z = 1; z < 8; z++)
+        if (z < slices) { t.x += v[z].x; t.y += v[z].y; t.z += v[z].z; t.w += v[z].w; }
+    int64_t at = i;
+    if (use_segs) {
+        int sg = 0;
+#pragma unroll
+        for (int q = 1; q < 4; q++)
+            if (q < segs.count && n >= segs.n0[q]) sg = q;
+        Y = segs.y[sg];
+        bias = segs.bias[sg];
+        n -= segs.n0[sg];
+        at = (int64_t)m * (segs.n0[sg + 1] - segs.n0[sg]) + n;
+    }
+    if (rowscale) { const float rs = rowscale[m]; t.x *= rs; t.y *= rs; t.z *= rs; t.w *= rs; }
+    if (bias) { const float4 b = *reinterpret_cast<const float4 *>(bias + n); t.x += b.x; t.y += b.y; t.z += b.z; t.w += b.w; }
+    t = make_float4(apply_act(act, t.x), apply_act(act, t.y), apply_act(act, t.z), apply_act(act, t.w));
+    if (residual) { const float4 r = *reinterpret_cast<const float4 *>(residual + at); t.x += r.x; t.y += r.y; t.z += r.z; t.w += r.w; }
+    *reinterpret_cast<float4 *>(Y + at) = t;
 }
 
 template <int T, bool BF16>
@@ -635,14 +676,17 @@ PrepMatrices prep_one_or_pair(const uint8_t *W, const uint8_t *W2, int64_t N) {
 template <bool BF16, int TM, int TN, bool GATED = false, bool SEGS = false>
 int launch_gemm16_tile(const uint16_t *x, int64_t M, int64_t K, const uint16_t *Wh, int64_t N, const float *bias, int act, float *y,
                        const float *bias2, int64_t n_out, const float *residual, const float *rowscale, hipStream_t s,
-                       const GemmSegs *segs = nullptr) {
+                       const GemmSegs *segs = nullptr, int slices = 1) {
     typedef DmaTile<TM, TN> G;
     static const bool lds_ok = [] {
         return hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_dma_kernel<BF16, TM, TN, GATED, SEGS>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, G::kLdsBytes) == hipSuccess;
     }();
     if (!lds_ok) return fail(GQ_ERR_HIP, "gemm: cannot reserve %d bytes of LDS", G::kLdsBytes);
-    const dim3 grid((unsigned)((N + G::DN - 1) / G::DN), (unsigned)((M + G::DM - 1) / G::DM));
+    static_assert(!GATED || !SEGS, "a gated pair has one output");
+    if (slices < 1 || (GATED && slices != 1) || (int64_t)(slices - 1) * ((K / DK + slices - 1) / slices) >= K / DK)
+        return fail(GQ_ERR_INVALID, "gemm: %d slices of K = %lld", slices, (long long)K);
+    const dim3 grid((unsigned)((N + G::DN - 1) / G::DN), (unsigned)((M + G::DM - 1) / G::DM), (unsigned)slices);
     return launch(gemm_dma_kernel<BF16, TM, TN, GATED, SEGS>, grid, dim3(512), (size_t)G::kLdsBytes, s, x, Wh, bias, y, (int)M, (int)K, (int)N, act,
                   bias2, (int)n_out, residual, rowscale, segs ? *segs : GemmSegs{});
 }
@@ -673,9 +717,42 @@ int pick_tile(int64_t M, int64_t N) {
     return t0 <= t1 ? 0 : 1;
 }
 
+// Few rows on a matrix with few columns leave most of the chip without a workgroup, each of the few walking all of K
+// (128 rows on 14336 -> 4096: 64 tiles of 128 x 64 on 256 CUs).  Then K is split into slices, as many as fill the chip
+// with at least 16 steps (1024 values) each, eight at most; the slices' sums go to `partial` ([slices][M][N] fp32) and a
+// small kernel adds them up and finishes them.  GOMLX_HIPQ_GEMM_K_SLICES=n forces n where it applies (1: never split).
+int k_slices_env() {
+    static const int v = [] { const char *e = std::getenv("GOMLX_HIPQ_GEMM_K_SLICES"); return e ? std::atoi(e) : 0; }();
+    return v;
+}
+int gemm_k_slices(int64_t M, int64_t K, int64_t N) {
+    if (N % 4 != 0) return 1;
+    const int64_t steps = K / DK, tiles = ((M + 127) / 128) * ((N + 63) / 64);
+    int64_t ns = std::min<int64_t>(std::min<int64_t>(device_cu_count() / tiles, steps / 16), 8);
+    if (k_slices_env() > 0) ns = std::min<int64_t>(std::min<int64_t>(k_slices_env(), steps), 8);
+    while (ns > 1 && (ns - 1) * ((steps + ns - 1) / ns) >= steps) ns--;  // no empty slice
+    return ns < 2 ? 1 : (int)ns;
+}
+size_t gemm_partial_bytes(int64_t M, int64_t K, int64_t N) {
+    const int ns = gemm_k_slices(M, K, N);
+    return ns > 1 ? (size_t)ns * (size_t)M * (size_t)N * sizeof(float) : 0;
+}
+template <class... P> bool aligned16(P... p) { return (((reinterpret_cast<uintptr_t>(p)) | ...) & 15) == 0; }  // (the reduction's float4 accesses)
+int launch_slices_reduce(const float *partial, int slices, int64_t M, int64_t N, const float *rowscale, const float *bias, int act,
+                         const float *residual, float *y, const GemmSegs *segs, hipStream_t s) {
+    const int64_t quads = M * N / 4;
+    return launch(gemm_slices_reduce_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, partial, slices, (int)M, (int)N, rowscale, bias, act,
+                  residual, y, segs ? *segs : GemmSegs{}, segs ? 1 : 0);
+}
+
+// partial: room for gemm_partial_bytes(M, K, N), or null (then K is never split)
 template <bool BF16>
 int launch_gemm16(const uint16_t *x, int64_t M, int64_t K, const uint16_t *Wh, int64_t N, const float *bias, int act, float *y, hipStream_t s,
-                  const float *residual = nullptr, const float *rowscale = nullptr) {
+                  const float *residual = nullptr, const float *rowscale = nullptr, float *partial = nullptr) {
+    if (const int ns = partial && aligned16(bias, residual, y) ? gemm_k_slices(M, K, N) : 1; ns > 1) {
+        if (int rc = launch_gemm16_tile<BF16, 1, 1>(x, M, K, Wh, N, nullptr, kActNone, partial, nullptr, N, nullptr, nullptr, s, nullptr, ns)) return rc;
+        return launch_slices_reduce(partial, ns, M, N, rowscale, bias, act, residual, y, nullptr, s);
+    }
     int choice = pick_tile(M, N);
     if (tile_env() >= 0 && tile_env() <= 2) choice = tile_env();
     switch (choice) {
@@ -686,8 +763,15 @@ int launch_gemm16(const uint16_t *x, int64_t M, int64_t K, const uint16_t *Wh, i
 }
 
 // Several matrices' images one after the other, one GEMM, each segment's columns to its own output (fp16 operands).
-int launch_gemm16_set(const uint16_t *x, int64_t M, int64_t K, const uint16_t *Wh, const GemmSegs &segs, int act, const float *rowscale, hipStream_t s) {
+int launch_gemm16_set(const uint16_t *x, int64_t M, int64_t K, const uint16_t *Wh, const GemmSegs &segs, int act, const float *rowscale, hipStream_t s,
+                      float *partial) {
     const int64_t N = segs.n0[segs.count];
+    bool aligned = true;
+    for (int i = 0; i < segs.count; i++) aligned = aligned && aligned16(segs.bias[i], segs.y[i]);
+    if (const int ns = partial && aligned ? gemm_k_slices(M, K, N) : 1; ns > 1) {
+        if (int rc = launch_gemm16_tile<false, 1, 1>(x, M, K, Wh, N, nullptr, kActNone, partial, nullptr, N, nullptr, nullptr, s, nullptr, ns)) return rc;
+        return launch_slices_reduce(partial, ns, M, N, rowscale, nullptr, act, nullptr, nullptr, &segs, s);
+    }
     int choice = pick_tile(M, N);
     if (tile_env() >= 0 && tile_env() <= 2) choice = tile_env();
     switch (choice) {
@@ -735,25 +819,31 @@ bool gemm_two_pass_supported(int type, bool x_is_bf16, int64_t M, int64_t K, int
     return (reinterpret_cast<uintptr_t>(x) & 15) == 0;
 }
 
-// [16-bit weight image][fp32 activations only: fp16 activation image, M row scales]
+// [16-bit weight image][fp32 activations only: fp16 activation image, M row scales][sums of the K slices, where K is split]
+namespace {
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+size_t two_pass_front_bytes(bool x_is_bf16, int64_t M, int64_t Kp, int64_t rows) {
+    return align256((size_t)rows * Kp * 2) + (x_is_bf16 ? 0 : align256((size_t)M * Kp * 2) + align256((size_t)M * sizeof(float)));
+}
+}  // namespace
 size_t gemm_two_pass_workspace(bool x_is_bf16, int64_t M, int64_t K, int64_t N) {
     K = padded_k(K);
-    const size_t w = ((size_t)N * K * 2 + 255) & ~(size_t)255;
-    return w + (x_is_bf16 ? 0 : (((size_t)M * K * 2 + 255) & ~(size_t)255) + (size_t)M * sizeof(float));
+    return two_pass_front_bytes(x_is_bf16, M, K, N) + gemm_partial_bytes(M, K, N);
 }
 
 int launch_gemm_two_pass(int type, bool x_is_bf16, const void *x, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias,
                          int act, float *y, void *workspace, hipStream_t s) {
     uint16_t *wh = static_cast<uint16_t *>(workspace);
+    const int64_t Kp = padded_k(K);
+    float *partial = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + two_pass_front_bytes(x_is_bf16, M, Kp, N));
     if (x_is_bf16) {
         if (int rc = launch_dequant16bit_type<true>(type, W, N, K, wh, s)) return rc;
-        return launch_gemm16<true>(static_cast<const uint16_t *>(x), M, K, wh, N, bias, act, y, s);
+        return launch_gemm16<true>(static_cast<const uint16_t *>(x), M, K, wh, N, bias, act, y, s, nullptr, nullptr, partial);
     }
-    const int64_t Kp = padded_k(K);
-    uint16_t *xh = wh + (((size_t)N * Kp * 2 + 255) & ~(size_t)255) / 2;
-    float *rowscale = reinterpret_cast<float *>(xh + (((size_t)M * Kp * 2 + 255) & ~(size_t)255) / 2);
+    uint16_t *xh = wh + align256((size_t)N * Kp * 2) / 2;
+    float *rowscale = reinterpret_cast<float *>(xh + align256((size_t)M * Kp * 2) / 2);
     if (int rc = launch_prep_f32(type, static_cast<const float *>(x), M, K, nullptr, xh, rowscale, prep_one_or_pair(W, nullptr, N), wh, s)) return rc;
-    return launch_gemm16<false>(xh, M, Kp, wh, N, bias, act, y, s, nullptr, rowscale);
+    return launch_gemm16<false>(xh, M, Kp, wh, N, bias, act, y, s, nullptr, rowscale, partial);
 }
 
 // The two passes for a projection with its neighbours (fp32 activations): the RMS normalisation
@@ -763,7 +853,7 @@ int launch_gemm_two_pass(int type, bool x_is_bf16, const void *x, int64_t M, int
 size_t gemm_two_pass_block_workspace(int64_t M, int64_t K, int64_t N, bool gated) {
     const int64_t rows = gated ? gated_image_rows(N) : N;
     K = padded_k(K);
-    return (((size_t)rows * K * 2 + 255) & ~(size_t)255) + (((size_t)M * K * 2 + 255) & ~(size_t)255) + (size_t)M * sizeof(float);
+    return two_pass_front_bytes(false, M, K, rows) + (gated ? 0 : gemm_partial_bytes(M, K, N));
 }
 
 bool gemm_two_pass_block_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, bool gated) {
@@ -777,10 +867,11 @@ int launch_gemm_two_pass_block(int type, const float *x, int64_t M, int64_t K, c
     const int64_t rows = W2 ? gated_image_rows(N) : N;
     uint16_t *wh = static_cast<uint16_t *>(workspace);
     const int64_t Kp = padded_k(K);
-    uint16_t *xh = wh + (((size_t)rows * Kp * 2 + 255) & ~(size_t)255) / 2;
-    float *rowscale = reinterpret_cast<float *>(xh + (((size_t)M * Kp * 2 + 255) & ~(size_t)255) / 2);
+    uint16_t *xh = wh + align256((size_t)rows * Kp * 2) / 2;
+    float *rowscale = reinterpret_cast<float *>(xh + align256((size_t)M * Kp * 2) / 2);
+    float *partial = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + two_pass_front_bytes(false, M, Kp, rows));
     if (int rc = launch_prep_f32(type, x, M, K, norm, xh, rowscale, prep_one_or_pair(W, W2, N), wh, s)) return rc;
-    if (!W2) return launch_gemm16<false>(xh, M, Kp, wh, N, bias, act, y, s, residual, rowscale);
+    if (!W2) return launch_gemm16<false>(xh, M, Kp, wh, N, bias, act, y, s, residual, rowscale, partial);
     return launch_gemm16_gated(xh, M, Kp, wh, N, bias, bias2, act, y, residual, rowscale, s);
 }
 
@@ -818,10 +909,11 @@ int launch_gemm_two_pass_set(int type, const float *x, int64_t M, int64_t K, con
     segs.n0[count] = (int)ntot;
     uint16_t *wh = static_cast<uint16_t *>(workspace);
     const int64_t Kp = padded_k(K);
-    uint16_t *xh = wh + (((size_t)ntot * Kp * 2 + 255) & ~(size_t)255) / 2;
-    float *rowscale = reinterpret_cast<float *>(xh + (((size_t)M * Kp * 2 + 255) & ~(size_t)255) / 2);
+    uint16_t *xh = wh + align256((size_t)ntot * Kp * 2) / 2;
+    float *rowscale = reinterpret_cast<float *>(xh + align256((size_t)M * Kp * 2) / 2);
+    float *partial = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + two_pass_front_bytes(false, M, Kp, ntot));
     if (int rc = launch_prep_f32(type, x, M, K, norm, xh, rowscale, pm, wh, s)) return rc;
-    return launch_gemm16_set(xh, M, Kp, wh, segs, items[0].act, rowscale, s);
+    return launch_gemm16_set(xh, M, Kp, wh, segs, items[0].act, rowscale, s, partial);
 }
 
 }  // namespace gq

@@ -176,7 +176,10 @@ int gq_qdense_block_f32(int type, const float *dX, int64_t M, int64_t K, const g
  * when all are problems of one type, one K and one batch size of at most 8 rows.  Two to four
  * Q4_K projections of the SAME activation buffer (equal dX, M, K) with more rows than that share
  * one split-K pass (activations converted once, one main launch, one reduction; uses the
- * per-stream workspace); anything else runs as separate gq_qdense_block_f32 calls. */
+ * per-stream workspace); past the split-K kernels' range such projections of any one type, with
+ * widths that are multiples of 32 and one activation function, share the two-pass GEMM (one activation
+ * conversion, one 16-bit image of all the matrices, one GEMM that writes each matrix's columns to its
+ * own output); anything else runs as separate gq_qdense_block_f32 calls. */
 int gq_qdense_norm_f32_batch(int count, const gq_dense_desc *descs, const gq_rmsnorm *norm,
                              void *stream);
 /* The gated feed-forward front (transformer.go:1279-1287, after the pre_feedforward_norm of

@@ -250,7 +250,7 @@ def test_split_k_small_batches_k_quants(gpu, oracle, t, M, K, N):
     bias = synth.normal(77, 0, N).astype(np.float32) * 0.1
     assert rel_err(run_dense(gpu, t, x, W, bias, 3), oracle.c_qdense(t, x, W, bias, 3)) < TOL_F32, (t, M, K, N, "f32")
     xb = bf16_round(x)
-    tol = TOL_F32 if (t == Q4_K or M <= 32) else TOL_BF16  # Q6_K beyond 32 rows takes the bf16 MFMA GEMM
+    tol = TOL_F32 if M <= (64 if t == Q4_K else 32) else TOL_BF16  # beyond 64 (Q6_K: 32) rows these matrices take the bf16 MFMA GEMM
     assert rel_err(run_dense(gpu, t, xb, W, bias, 3, bf16=True), oracle.c_qdense(t, xb, W, bias, 3)) < tol, (t, M, K, N, "bf16")
 
 
@@ -502,16 +502,48 @@ def test_small_batches_on_large_matrices(gpu, oracle, t, N):
 @pytest.mark.parametrize("t", ALL_TYPES)
 def test_hand_over_from_split_k_to_the_two_passes(gpu, oracle, t):
     """A 4096 x 2048 matrix (between 6 and 24 MB in every format): the split-K kernels hand over to the two-pass GEMM after
-    96, 128 or 160 rows depending on the format; both sides of each of those points, fp32 and bf16 activations."""
+    64, 96 or 128 rows depending on the format; both sides of each of those points and of 160, fp32 and bf16 activations."""
     K, N = 4096, 2048 if t != Q4_0 and t != IQ4_NL and t != Q4_K else 3072
     assert 6 << 20 <= N * ggml.row_bytes(t, K) < 24 << 20
     W = synth.weights(t, 350 + t, N, K)
-    for M in (96, 97, 128, 129, 160, 161):
+    for M in (64, 65, 96, 97, 128, 129, 160, 161):
         x = synth.activations(351 + M, M, K)
         assert rel_err(run_dense(gpu, t, x, W), oracle.c_qdense(t, x, W)) < TOL_F32, (t, M)
-    for M in (97, 129):
+    for M in (65, 97, 129):
         xb = bf16_round(synth.activations(360 + M, M, K))
         assert rel_err(run_dense(gpu, t, xb, W, bf16=True), oracle.c_qdense(t, xb, W)) < TOL_BF16, (t, M)
+
+
+@pytest.mark.parametrize("t", ALL_TYPES)
+def test_few_rows_on_few_columns_split_k_inside_the_gemm(gpu, oracle, t):
+    """Past the split-K kernels' range a narrow matrix gives the GEMM fewer tiles than the chip has CUs; K is then cut into up
+    to eight slices whose sums a small kernel adds up and finishes (row scales, bias, activation, residual).  Dense calls
+    with fp32 and bf16 activations, a projection with normalisation and residual, q / k / v behind one normalisation;
+    slices of equal and unequal length; a width that is not a multiple of 4 keeps the unsplit GEMM."""
+    q = Quantization(ggml_type=t)
+    for M, K, N, act in ((200, 4096, 512, 3), (130, 2304, 1024, 0), (300, 3328, 256, 2), (200, 4096, 510, 1), (17, 8192, 64, 0)):
+        W = synth.weights(t, 1400 + t, N, K)
+        bias = synth.normal(1401, 0, N).astype(np.float32) * 0.1
+        x = synth.activations(1402 + M, M, K)
+        assert rel_err(run_dense(gpu, t, x, W, bias, act), oracle.c_qdense(t, x, W, bias, act)) < TOL_F32, (ggml.name(t), M, K, N)
+        xb = bf16_round(x)
+        assert rel_err(run_dense(gpu, t, xb, W, None, act, bf16=True), oracle.c_qdense(t, xb, W, None, act)) < TOL_BF16, (ggml.name(t), M, K, N)
+    M, K, N = 200, 4096, 512
+    W = synth.weights(t, 1410 + t, N, K)
+    gain = (synth.normal(1411, 0, K) * 0.5 + 1.0).astype(np.float32)
+    cfg = nn.RMSNorm(dev(gpu, gain), 1e-6, 0.0)
+    x = (synth.activations(1412, M, K) * 2.0).astype(np.float32)
+    xn = oracle.c_rmsnorm(x, gain, 1e-6, 0.0)
+    res = synth.activations(1413, M, N)
+    got = nn.quantized_dense(dev(gpu, x), dev(gpu, W), q, None, BACKEND_ACT[0], norm=cfg, residual=dev(gpu, res)).cpu().numpy()
+    dense = oracle.c_qdense(t, xn, W)
+    assert float(np.max(np.abs(got.astype(np.float64) - (dense + res)))) / float(np.max(np.abs(dense))) < TOL_F32, ggml.name(t)
+    Ws = [synth.weights(t, 1420 + j, n, K) for j, n in enumerate((512, 128, 128))]
+    bs = [synth.normal(1425, 0, 512).astype(np.float32) * 0.1, None, None]
+    outs = nn.quantized_dense_batch([(dev(gpu, x), dev(gpu, Wj), q, None if b is None else dev(gpu, b), None) for Wj, b in zip(Ws, bs)], norm=cfg)
+    gpu.cuda.synchronize()
+    for Wj, b, y in zip(Ws, bs, outs):
+        assert rel_err(y.cpu().numpy(), oracle.c_qdense(t, xn, Wj, b)) < TOL_F32, (ggml.name(t), Wj.shape)
 
 
 @pytest.mark.parametrize("t,N", [(Q8_0, 3328), (Q4_K, 5632), (Q6_K, 4096)])
@@ -1320,7 +1352,7 @@ def test_config2_q4_k_batch32(gpu, oracle):
     assert rel_err(run_dense(gpu, Q4_K, x, W), oracle.c_qdense(Q4_K, x, W)) < TOL_F32
 
 
-@pytest.mark.parametrize("M,K,N", [(32, 14336, 4096), (9, 4096, 1024), (70, 2048, 896)])
+@pytest.mark.parametrize("M,K,N", [(32, 14336, 4096), (9, 4096, 1024), (40, 2048, 896)])
 def test_q4_k_split_k_stages_missing_activation_records_itself(gpu, oracle, M, K, N, monkeypatch):
     """The Q4_K split-K kernel's workgroups share the staging of the activations through memory and flag words.  With the
     bound on the wait for those flags at zero every wait runs out at once (forced from the host; the kernel exits normally)
