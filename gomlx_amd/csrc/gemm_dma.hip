@@ -253,6 +253,9 @@ int launch_x_to_f16(const float *x, int64_t M, int64_t K, const RmsNorm *norm, u
     if (kp <= 8192)
         return norm ? launch(x_row_to_f16_kernel<4, true>, grid, block, 0, s, x, gain, off, eps, (int)K, xh, rowscale)
                     : launch(x_row_to_f16_kernel<4, false>, grid, block, 0, s, x, gain, off, eps, (int)K, xh, rowscale);
+    if (kp <= 16384)
+        return norm ? launch(x_row_to_f16_kernel<8, true>, grid, block, 0, s, x, gain, off, eps, (int)K, xh, rowscale)
+                    : launch(x_row_to_f16_kernel<8, false>, grid, block, 0, s, x, gain, off, eps, (int)K, xh, rowscale);
     return norm ? launch(x_rmsnorm_to_f16_kernel, grid, block, 0, s, x, gain, off, eps, (int)K, xh, rowscale)
                 : launch(x_to_f16_kernel, grid, block, 0, s, x, (int)K, xh, rowscale);
 }
@@ -591,7 +594,7 @@ int launch_dequant16bit_type(int type, const uint8_t *W, int64_t N, int64_t K, u
 
 // Both pre-passes of the fp32-activation route in ONE launch (they do not depend on each other): the first M workgroups
 // convert an activation row each (x_row_to_f16_body), the others 256 runs of weights each (dequant16bit_body), of W and -
-// for a gated pair, whose images interleave - of W2.  Rows of up to 8192 values (longer ones keep their own two-read kernel).
+// for a gated pair, whose images interleave - of W2.  Rows of up to 16384 values (longer ones keep their own two-read kernel).
 // The matrices of one pre-pass: matrix i is W[i] with rows[i] rows, written from image row row0[i] on with the interleaving
 // `half[i]` of dequant16bit_body (a gated pair: both matrices at row 0 with halves 1 and 2; a set: halves 0, one after the other).
 struct PrepMatrices {
@@ -641,13 +644,15 @@ int launch_prep_f32_t(const float *x, int64_t M, int64_t K, const RmsNorm *norm,
         return launch(kernel, grid, block, 0, s, x, gain, off, eps, (int)K, xh, rowscale, (uint32_t)M, pm, wh, (uint32_t)runs_per_row, row_bytes, (uint32_t)runs);
     };
     if (padded_k(K) <= 4096) return norm ? go(prep_f32_kernel<T, 2, true>) : go(prep_f32_kernel<T, 2, false>);
-    return norm ? go(prep_f32_kernel<T, 4, true>) : go(prep_f32_kernel<T, 4, false>);
+    if (padded_k(K) <= 8192) return norm ? go(prep_f32_kernel<T, 4, true>) : go(prep_f32_kernel<T, 4, false>);
+    return norm ? go(prep_f32_kernel<T, 8, true>) : go(prep_f32_kernel<T, 8, false>);
 }
 
-// x -> fp16 rows and the matrices -> fp16 image: one launch for rows of up to 8192 values, else one per operand
+// x -> fp16 rows and the matrices -> fp16 image: one launch for rows of up to 16384 values (64 per thread in registers; on its
+// own the activation pass of 128 rows of 14336 values took 6 us, a workgroup per row with nothing beside it), else one per operand
 int launch_prep_f32(int type, const float *x, int64_t M, int64_t K, const RmsNorm *norm, uint16_t *xh, float *rowscale, const PrepMatrices &pm,
                     uint16_t *wh, hipStream_t s) {
-    if (padded_k(K) > 8192) {
+    if (padded_k(K) > 16384) {
         if (int rc = launch_x_to_f16(x, M, K, norm, xh, rowscale, s)) return rc;
         for (int i = 0; i < pm.count; i++)
             if (int rc = launch_dequant16bit_type<false>(type, pm.W[i], pm.rows[i], K, wh + (size_t)pm.row0[i] * padded_k(K), s, pm.half[i])) return rc;

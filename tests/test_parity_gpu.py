@@ -521,23 +521,23 @@ def test_few_rows_on_few_columns_split_k_inside_the_gemm(gpu, oracle, t):
     with fp32 and bf16 activations, a projection with normalisation and residual, q / k / v behind one normalisation;
     slices of equal and unequal length; a width that is not a multiple of 4 keeps the unsplit GEMM."""
     q = Quantization(ggml_type=t)
-    for M, K, N, act in ((200, 4096, 512, 3), (130, 2304, 1024, 0), (300, 3328, 256, 2), (200, 4096, 510, 1), (17, 8192, 64, 0)):
+    for M, K, N, act in ((200, 4096, 512, 3), (130, 2304, 1024, 0), (300, 3328, 256, 2), (200, 4096, 510, 1), (17, 8192, 64, 0), (130, 14336, 256, 0)):
         W = synth.weights(t, 1400 + t, N, K)
         bias = synth.normal(1401, 0, N).astype(np.float32) * 0.1
         x = synth.activations(1402 + M, M, K)
         assert rel_err(run_dense(gpu, t, x, W, bias, act), oracle.c_qdense(t, x, W, bias, act)) < TOL_F32, (ggml.name(t), M, K, N)
         xb = bf16_round(x)
         assert rel_err(run_dense(gpu, t, xb, W, None, act, bf16=True), oracle.c_qdense(t, xb, W, None, act)) < TOL_BF16, (ggml.name(t), M, K, N)
-    M, K, N = 200, 4096, 512
-    W = synth.weights(t, 1410 + t, N, K)
-    gain = (synth.normal(1411, 0, K) * 0.5 + 1.0).astype(np.float32)
-    cfg = nn.RMSNorm(dev(gpu, gain), 1e-6, 0.0)
-    x = (synth.activations(1412, M, K) * 2.0).astype(np.float32)
-    xn = oracle.c_rmsnorm(x, gain, 1e-6, 0.0)
-    res = synth.activations(1413, M, N)
-    got = nn.quantized_dense(dev(gpu, x), dev(gpu, W), q, None, BACKEND_ACT[0], norm=cfg, residual=dev(gpu, res)).cpu().numpy()
-    dense = oracle.c_qdense(t, xn, W)
-    assert float(np.max(np.abs(got.astype(np.float64) - (dense + res)))) / float(np.max(np.abs(dense))) < TOL_F32, ggml.name(t)
+    for M, K, N in ((130, 10240, 256), (200, 4096, 512)):  # (rows of more than 8192 values: 64 per thread in the activation pass)
+        W = synth.weights(t, 1410 + t, N, K)
+        gain = (synth.normal(1411, 0, K) * 0.5 + 1.0).astype(np.float32)
+        cfg = nn.RMSNorm(dev(gpu, gain), 1e-6, 0.0)
+        x = (synth.activations(1412, M, K) * 2.0).astype(np.float32)
+        xn = oracle.c_rmsnorm(x, gain, 1e-6, 0.0)
+        res = synth.activations(1413, M, N)
+        got = nn.quantized_dense(dev(gpu, x), dev(gpu, W), q, None, BACKEND_ACT[0], norm=cfg, residual=dev(gpu, res)).cpu().numpy()
+        dense = oracle.c_qdense(t, xn, W)
+        assert float(np.max(np.abs(got.astype(np.float64) - (dense + res)))) / float(np.max(np.abs(dense))) < TOL_F32, (ggml.name(t), K)
     Ws = [synth.weights(t, 1420 + j, n, K) for j, n in enumerate((512, 128, 128))]
     bs = [synth.normal(1425, 0, 512).astype(np.float32) * 0.1, None, None]
     outs = nn.quantized_dense_batch([(dev(gpu, x), dev(gpu, Wj), q, None if b is None else dev(gpu, b), None) for Wj, b in zip(Ws, bs)], norm=cfg)
