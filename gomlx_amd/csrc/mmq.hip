@@ -27,6 +27,7 @@
 #include "blocks.hpp"
 #include "common.hpp"
 
+#include <algorithm>
 #include <cstdlib>
 #include <type_traits>
 
@@ -289,6 +290,80 @@ __device__ __forceinline__ void q4k_contract_sb(const RawSB &cur, const uint8_t 
     }
 }
 
+// The same super-block against the images of RM tiles of 32 batch columns (tile t: fragments at img + 16384 t,
+// sub-block sums at sums + 512 t): the codes are turned into operand fragments ONCE and every
+// fragment meets each tile's activations, so the conversion, the parked tile and the header are shared by up to 128
+// batch rows.  Per tile the arithmetic and its order are those of q4k_contract_sb<false>.
+template <int RM>
+__device__ __forceinline__ void q4k_contract_sb_tiles(const RawSB &cur, const uint8_t *img, const uint8_t *sums, int kg, int col, uint32_t magic,
+                                                      f16v (&acc)[RM]) {
+    const float d = half_bits_to_float(cur.hd.x & 0xFFFFu), dmin = half_bits_to_float(cur.hd.x >> 16);
+    const uint32_t a = cur.hd.y, b = cur.hd.z, c = cur.hd.w;
+    const uint32_t sc_lo = a & 0x3F3F3F3Fu, mn_lo = b & 0x3F3F3F3Fu;
+    const uint32_t sc_hi = (c & 0x0F0F0F0Fu) | ((a >> 2) & 0x30303030u);
+    const uint32_t mn_hi = ((c >> 4) & 0x0F0F0F0Fu) | ((b >> 2) & 0x30303030u);
+    f16v p1[RM];
+#pragma unroll
+    for (int t = 0; t < RM; t++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) p1[t][r] = 0.f;
+#pragma unroll
+    for (int st = 0; st < 4; st++) {
+        const uint32_t scw = (st < 2 ? sc_lo : sc_hi) >> (16 * (st & 1));
+        const float s0f = (float)(scw & 0xFFu), s1f = (float)((scw >> 8) & 0xFFu);
+        const h2 s0 = as_h2(pack_h2(s0f, s0f));
+        const h2 s1 = as_h2(pack_h2(s1f * 0.0625f, s1f * 0.0625f));
+        const h2 k0h = as_h2(pack_h2(-1024.f * s0f, -1024.f * s0f));
+        const h2 k1h = as_h2(pack_h2(-64.f * s1f, -64.f * s1f));
+        const uint32_t dw[4] = {cur.c[st].x, cur.c[st].y, cur.c[st].z, cur.c[st].w};
+        uint32_t wl[8], wh[8];
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const uint32_t u = dw[w], v = dw[w] >> 8;
+            wl[2 * w] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(u, 0x000F000Fu, magic), s0, k0h));
+            wl[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(v, 0x000F000Fu, magic), s0, k0h));
+            wh[2 * w] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(u, 0x00F000F0u, magic), s1, k1h));
+            wh[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(v, 0x00F000F0u, magic), s1, k1h));
+        }
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const uint32_t *src = (q < 2 ? wl : wh) + 4 * (q & 1);
+            const h8 wfrag = __builtin_bit_cast(h8, make_uint4(src[0], src[1], src[2], src[3]));
+            const int slot = (2 * st + kg) * 4 + q;  // (slot of fragment 4 st + q in a one-super-block image, see stage_x)
+#pragma unroll
+            for (int t = 0; t < RM; t++) {
+                const h8 xf = *reinterpret_cast<const h8 *>(img + t * 16384 + (slot * kMT + (col ^ (slot & 15))) * 16);
+                p1[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xf, wfrag, p1[t], 0, 0, 0);
+            }
+        }
+    }
+    // minima against the sub-block sums, as in q4k_contract_sb: only k-group 0 carries operands (the sums are read by every
+    // lane and cleared by a select in k-group 1: no branch around an LDS read)
+    f16v zero16;
+#pragma unroll
+    for (int r = 0; r < 16; r++) zero16[r] = 0.f;
+    uint4 mv = make_uint4(0u, 0u, 0u, 0u);
+    {
+        const h2 off = as_h2(0xE400E400u);  // (-1024, -1024)
+        const uint32_t keep = kg == 0 ? 0xFFFFFFFFu : 0u;
+        mv.x = __builtin_bit_cast(uint32_t, magic_pair(mn_lo, 0x00FF00FFu, magic) + off) & keep;
+        mv.y = __builtin_bit_cast(uint32_t, magic_pair(mn_lo >> 8, 0x00FF00FFu, magic) + off) & keep;
+        mv.z = __builtin_bit_cast(uint32_t, magic_pair(mn_hi, 0x00FF00FFu, magic) + off) & keep;
+        mv.w = __builtin_bit_cast(uint32_t, magic_pair(mn_hi >> 8, 0x00FF00FFu, magic) + off) & keep;
+    }
+#pragma unroll
+    for (int t = 0; t < RM; t++) {
+        uint4 sv = *reinterpret_cast<const uint4 *>(sums + t * 512 + col * 16);
+        const uint32_t keep = kg == 0 ? 0xFFFFFFFFu : 0u;
+        sv.x &= keep; sv.y &= keep; sv.z &= keep; sv.w &= keep;
+        const f16v p2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, sv), __builtin_bit_cast(h8, mv), zero16, 0, 0, 0);
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[t][r] = fmaf(d, p1[t][r], acc[t][r]);
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[t][r] = fmaf(-dmin, p2[r], acc[t][r]);
+    }
+}
+
 // Activation pre-pass: writes each (K-slice, column tile)'s LDS image (fragment-ordered fp16
 // activations + sub-block sums) to global memory once; the row-range workgroups of the main
 // kernel then only copy 132 KiB each instead of converting it again.  grid = (slices, column
@@ -430,6 +505,115 @@ __global__ __launch_bounds__(64 * RT * kParts) void mmq_q4k_kernel(const uint8_t
 #pragma unroll
             for (int p = 0; p < kParts - 1; p++) v += xch[(p * 16 + r) * 64 + lane];
             if (m < M) partial[((int64_t)slice * M + m) * set.ntot + set.n0[prob] + n] = v;
+        }
+    }
+}
+
+// ---- several tiles of 32 batch rows per weight tile ---------------------------------------------------------------
+//
+// mmq_q4k_kernel serves one tile of 32 batch rows per launch: 128 rows stream W four times and convert every code four
+// times.  mmq_q4k_tiles_kernel walks up to four such tiles together: eight wavefronts, each with its own row tile of 32 rows
+// of W (256 per workgroup) and all of the slice's super-blocks; the activation images of the tiles no longer fit LDS for
+// a whole slice, so the workgroup moves along K one super-block at a time - the images of that super-block for every
+// tile (16.5 KiB each, global -> LDS by DMA from the pre-pass's image), a barrier, then every wavefront's super-block
+// against all of them (q4k_contract_sb_tiles) while its next weight tile is on its way into its parked piece of LDS.
+// Same grid roles, same image and partial-sum layouts as mmq_q4k_kernel (m0 = first batch row, NT = tiles of 32 from there).
+struct Q4KTiles {
+    static constexpr int kMaxTiles = 4, kWaves = 8, kRows = 32 * kWaves;
+    static constexpr int kImgBytes = kMaxTiles * 16384, kSumBytes = kMaxTiles * kMT * 16;
+    static constexpr int kLds = kImgBytes + kSumBytes + kWaves * kParkBytes;
+    static_assert(kLds <= 160 * 1024, "images + parked tiles exceed LDS");
+};
+
+template <int NT>
+__global__ __launch_bounds__(64 * Q4KTiles::kWaves) void mmq_q4k_tiles_kernel(const uint8_t *__restrict__ ximg, Q4KSet set, float *__restrict__ partial0,
+                                                                               int M, int K, int64_t row_bytes, int m0,
+                                                                               const uint8_t *__restrict__ W2, float *__restrict__ partial2) {
+    typedef Q4KTiles G;
+    static_assert(NT >= 1 && NT <= G::kMaxTiles, "one to four tiles of 32 batch rows");
+    constexpr int ntile = NT;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    int prob = 0;
+#pragma unroll
+    for (int j = 1; j < kMaxSet; j++)
+        if (j < set.count && (int)blockIdx.x >= set.wg0[j]) prob = j;
+    const uint8_t *__restrict__ W = blockIdx.z ? W2 : set.W[prob];
+    float *__restrict__ partial = blockIdx.z ? partial2 : partial0;
+    const int N = set.N[prob], xblk = (int)blockIdx.x - set.wg0[prob];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kg = lane >> 5, col = lane & 31;
+    const int slice = blockIdx.y, nslices = gridDim.y;
+    const int nsb = ((K >> 8) - slice + nslices - 1) / nslices;  // slice s holds super-blocks s, s + nslices, ... of every row
+    const int row0 = xblk * G::kRows + wave * 32;
+    const int n = row0 + col;  // this lane's weight row
+
+    const uint8_t *wtile = W + (int64_t)min(row0, N - 1) * row_bytes + slice * 144;
+    uint32_t csrc[kParkLoads];
+#pragma unroll
+    for (int l = 0; l < kParkLoads; l++) {
+        const int c = min(lane + 64 * l, 32 * 9 - 1);
+        csrc[l] = (uint32_t)(min(row0 + c / 9, N - 1) - min(row0, N - 1)) * (uint32_t)row_bytes + (uint32_t)((c % 9) * 16);
+    }
+    uint8_t *park = lds + G::kImgBytes + G::kSumBytes + wave * kParkBytes;
+    auto fetch = [&](int sb) __attribute__((always_inline)) {
+        const uint8_t *base = wtile + sb * nslices * 144;
+#pragma unroll
+        for (int l = 0; l < kParkLoads; l++)
+            if (64 * l + 64 <= 32 * 9 || lane < 32 * 9 - 64 * l)  // (the last instruction carries 32 chunks)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(base + csrc[l]),
+                                                 (__attribute__((address_space(3))) void *)(park + l * 1024), 16, 0, 0);
+    };
+    fetch(0);  // (every slice holds at least one super-block)
+    const uint8_t *myrow = park + col * 144;
+    // tile t's image of this slice: fragments of super-block j at 16384 j, its sub-block sums at kXFBytes + 512 j
+    const uint8_t *img0 = ximg + ((size_t)(m0 / kMT) * nslices + slice) * kLdsBytes;
+    const size_t tile_stride = (size_t)nslices * kLdsBytes;
+
+    f16v acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[t][r] = 0.f;
+    uint32_t magic;
+    asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));
+
+    for (int sbl = 0; sbl < nsb; sbl++) {
+        __syncthreads();  // every wavefront has finished with the images of the super-block before
+        for (int i = wave; i < ntile * 16; i += G::kWaves) {
+            const int t = i >> 4, ck = i & 15;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(img0 + t * tile_stride + sbl * 16384 + ck * 1024 + lane * 16),
+                                             (__attribute__((address_space(3))) void *)(lds + t * 16384 + ck * 1024), 16, 0, 0);
+        }
+        if (wave < ntile && lane < 32)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(img0 + wave * tile_stride + kXFBytes + sbl * 512 + lane * 16),
+                                             (__attribute__((address_space(3))) void *)(lds + G::kImgBytes + wave * 512), 16, 0, 0);
+        // a barrier does not wait for loads in flight: this wavefront's share of the images (and its weight tile) must
+        // have landed before it arrives
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        typedef uint32_t Chunk __attribute__((ext_vector_type(4)));
+        Chunk rhd = *reinterpret_cast<const Chunk *>(myrow), rc[4];
+#pragma unroll
+        for (int st = 0; st < 4; st++) rc[st] = *reinterpret_cast<const Chunk *>(myrow + 16 + 32 * st + 16 * kg);
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(rhd), "+v"(rc[0]), "+v"(rc[1]), "+v"(rc[2]), "+v"(rc[3])::"memory");
+        RawSB cur;
+        cur.hd = make_uint4(rhd.x, rhd.y, rhd.z, rhd.w);
+#pragma unroll
+        for (int st = 0; st < 4; st++) cur.c[st] = make_uint4(rc[st].x, rc[st].y, rc[st].z, rc[st].w);
+        __builtin_amdgcn_wave_barrier();
+        if (sbl + 1 < nsb) fetch(sbl + 1);
+        q4k_contract_sb_tiles<NT>(cur, lds, lds + G::kImgBytes, kg, col, magic, acc);
+    }
+
+    if (n < N) {
+        // lane holds y[m = 32 t + 8 (r / 4) + 4 kg + r % 4][n] for its K-slice
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = m0 + 32 * t + 8 * (r >> 2) + 4 * kg + (r & 3);
+                if (m < M) partial[((int64_t)slice * M + m) * set.ntot + set.n0[prob] + n] = acc[t][r];
+            }
         }
     }
 }
@@ -1332,12 +1516,6 @@ namespace {
 // the pre-pass launch they replace; it stays selectable so that the comparison can be repeated.
 // GOMLX_HIPQ_COOP_SPIN_TICKS=n bounds the wait for published activation records (100 MHz ticks; 0 makes every wait run
 // out at once, which is how the tests reach the path that stages the missing records locally).  Both are read at every call.
-// GOMLX_HIPQ_COOP=1 sends the Q4_K split-K route through the kernel that stages the activations itself (two launches
-// instead of three).  It is correct and tested, and it is slower: 24.0 against 20.5 us on a 14336 -> 4096 matrix at 32 rows,
-// because a record travels workgroup -> memory -> flag -> other workgroups in four dependent trips to memory, longer than
-// the pre-pass launch they replace; it stays selectable so that the comparison can be repeated.
-// GOMLX_HIPQ_COOP_SPIN_TICKS=n bounds the wait for published activation records (100 MHz ticks; 0 makes every wait run
-// out at once, which is how the tests reach the path that stages the missing records locally).  Both are read at every call.
 bool coop_enabled() {
     const char *e = std::getenv("GOMLX_HIPQ_COOP");
     return e && e[0] == '1';
@@ -1346,6 +1524,13 @@ int coop_spin_ticks() {
     const char *e = std::getenv("GOMLX_HIPQ_COOP_SPIN_TICKS");
     const long v = e ? std::atol(e) : 20000;  // 200 us: a record is published a few microseconds into the kernel
     return v < 0 ? 0 : v > 100000000 ? 100000000 : (int)v;
+}
+
+// GOMLX_HIPQ_Q4K_TILES_TOGETHER=0: batches of more than 32 rows as one launch of mmq_q4k_kernel per 32 rows (tuning runs and
+// comparisons only).  Read at every call.
+bool tiles_together_enabled() {
+    const char *e = std::getenv("GOMLX_HIPQ_Q4K_TILES_TOGETHER");
+    return !(e && e[0] == '0');
 }
 
 // `count` Q4_K matrices against one activation image: the pre-pass once, every matrix's row ranges in one launch of the
@@ -1360,13 +1545,23 @@ int run_q4k_set(const void *x, bool x_is_bf16, int64_t M, int64_t K, int count, 
     if (!lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", Tile::kLds);
     const int mtiles = (int)((M + kMT - 1) / kMT);
     const int64_t sbs = K / 256;
+    // more than 32 batch rows: the kernel that walks up to four tiles of 32 together (256 rows of W per workgroup)
+    const bool together = mtiles >= 2 && !coop_enabled() && tiles_together_enabled();
+    static const bool tiles_lds_ok = [] {
+        auto room = [](auto kernel) {
+            return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, Q4KTiles::kLds) == hipSuccess;
+        };
+        return room(mmq_q4k_tiles_kernel<1>) && room(mmq_q4k_tiles_kernel<2>) && room(mmq_q4k_tiles_kernel<3>) && room(mmq_q4k_tiles_kernel<4>);
+    }();
+    if (together && !tiles_lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", Q4KTiles::kLds);
+    const int wg_rows = together ? Q4KTiles::kRows : Tile::kRows;
     Q4KSet set = {};
     MmqSetOut out = {};
     int64_t rowwgs = 0, N = 0;  // workgroups along the rows of all matrices; their columns side by side
     for (int i = 0; i < count; i++) {
         set.W[i] = items[i].W; set.N[i] = (int)items[i].N; set.wg0[i] = (int)rowwgs; set.n0[i] = (int)N;
         out.bias[i] = items[i].bias; out.y[i] = items[i].y; out.N[i] = (int)items[i].N; out.n0[i] = (int)N; out.act[i] = items[i].act;
-        rowwgs += (items[i].N + Tile::kRows - 1) / Tile::kRows;
+        rowwgs += (items[i].N + wg_rows - 1) / wg_rows;
         N += items[i].N;
     }
     set.count = out.count = count;
@@ -1383,6 +1578,10 @@ int run_q4k_set(const void *x, bool x_is_bf16, int64_t M, int64_t K, int count, 
             const int64_t cost = ((wgs + cus - 1) / cus) * (ssb + 3);
             if (cost < best_cost) { best_cost = cost; slice_sb = ssb; }
         }
+    }
+    if (const char *e = std::getenv("GOMLX_HIPQ_Q4K_SLICE_SB")) {  // (tuning runs only)
+        const int v = std::atoi(e);
+        if (v >= 1 && v <= Tile::kMaxSliceSB) slice_sb = v;
     }
     const int nslices = (int)((sbs + slice_sb - 1) / slice_sb);
     const int64_t row_bytes = (K / 256) * 144;
@@ -1445,7 +1644,21 @@ int run_q4k_set(const void *x, bool x_is_bf16, int64_t M, int64_t K, int count, 
                            : (fine ? prep(mmq_xprep_kernel<false, 1>) : prep(mmq_xprep_kernel<false, 2>)))
         return rc;
     partial2 = W2 ? partial + (size_t)nslices * M * N : nullptr;
-    for (int64_t m0 = 0; m0 < M; m0 += kMT) {
+    // (the tiles are dealt evenly over the fewest launches: five tiles go as 3 + 2, not as 4 + 1 - every launch streams all of W)
+    const int nlaunch = (mtiles + Q4KTiles::kMaxTiles - 1) / Q4KTiles::kMaxTiles;
+    for (int l = 0, tile0 = 0; together && l < nlaunch; l++) {
+        const int ntile = (mtiles - tile0 + (nlaunch - l) - 1) / (nlaunch - l);
+        const int64_t m0 = (int64_t)tile0 * kMT;
+        tile0 += ntile;
+        auto go = [&](auto kernel) {
+            return launch(kernel, grid, dim3(64 * Q4KTiles::kWaves), (size_t)Q4KTiles::kLds, s, (const uint8_t *)ximg, set, partial, (int)M, (int)K,
+                          row_bytes, (int)m0, W2, partial2);
+        };
+        if (int rc = ntile == 4 ? go(mmq_q4k_tiles_kernel<4>) : ntile == 3 ? go(mmq_q4k_tiles_kernel<3>) : ntile == 2 ? go(mmq_q4k_tiles_kernel<2>)
+                                                                                                                     : go(mmq_q4k_tiles_kernel<1>))
+            return rc;
+    }
+    for (int64_t m0 = 0; !together && m0 < M; m0 += kMT) {
         if (int rc = launch(mmq_q4k_kernel<kQ4KRowTiles>, grid, dim3(64 * Tile::kWaves), (size_t)Tile::kLds, s, (const uint8_t *)ximg, set, partial,
                             (int)M, (int)K, row_bytes, (int)m0, slice_sb, W2, partial2))
             return rc;

@@ -250,8 +250,46 @@ def test_split_k_small_batches_k_quants(gpu, oracle, t, M, K, N):
     bias = synth.normal(77, 0, N).astype(np.float32) * 0.1
     assert rel_err(run_dense(gpu, t, x, W, bias, 3), oracle.c_qdense(t, x, W, bias, 3)) < TOL_F32, (t, M, K, N, "f32")
     xb = bf16_round(x)
-    tol = TOL_F32 if M <= (64 if t == Q4_K else 32) else TOL_BF16  # beyond 64 (Q6_K: 32) rows these matrices take the bf16 MFMA GEMM
+    tol = TOL_F32 if (t == Q4_K or M <= 32) else TOL_BF16  # Q6_K beyond 32 rows takes the bf16 MFMA GEMM on these matrices
     assert rel_err(run_dense(gpu, t, xb, W, bias, 3, bf16=True), oracle.c_qdense(t, xb, W, bias, 3)) < tol, (t, M, K, N, "bf16")
+
+
+def test_q4_k_split_k_walks_several_batch_tiles_together(gpu, oracle):
+    """More than 32 batch rows on the Q4_K split-K route: one launch contracts up to four tiles of 32 rows against every weight
+    tile (codes converted once).  A long-K matrix of 25.6 MB, which keeps the route up to 256 rows: every tile count, a second
+    launch for the rows past 128 (tiles dealt evenly: 3 + 2, 4 + 4), a last tile that is partly filled, a width that is not a multiple of the workgroup's 256
+    rows; fp32 and bf16 activations; the gated pair, the projection with normalisation and residual, and q / k / v."""
+    t, K, N = Q4_K, 14336, 3172
+    assert N * ggml.row_bytes(t, K) >= 24 << 20
+    q = Quantization(ggml_type=t)
+    W = synth.weights(t, 1500, N, K)
+    bias = synth.normal(1501, 0, N).astype(np.float32) * 0.1
+    Wd = dev(gpu, W)
+    for M in (33, 64, 70, 96, 128, 129, 160, 250):
+        x = synth.activations(1502 + M, M, K)
+        got = nn.quantized_dense(dev(gpu, x), Wd, q, dev(gpu, bias), BACKEND_ACT[3]).cpu().numpy()
+        assert rel_err(got, oracle.c_qdense(t, x, W, bias, 3)) < TOL_F32, M
+    xb = bf16_round(synth.activations(1510, 100, K))
+    assert rel_err(run_dense(gpu, t, xb, W, bias, 0, bf16=True), oracle.c_qdense(t, xb, W, bias, 0)) < TOL_F32
+    # projection with normalisation and residual
+    M = 100
+    gain = (synth.normal(1511, 0, K) * 0.5 + 1.0).astype(np.float32)
+    cfg = nn.RMSNorm(dev(gpu, gain), 1e-6, 0.0)
+    x = (synth.activations(1512, M, K) * 2.0).astype(np.float32)
+    xn = oracle.c_rmsnorm(x, gain, 1e-6, 0.0)
+    res = synth.activations(1513, M, N)
+    got = nn.quantized_dense(dev(gpu, x), Wd, q, None, BACKEND_ACT[0], norm=cfg, residual=dev(gpu, res)).cpu().numpy()
+    dense = oracle.c_qdense(t, xn, W)
+    assert float(np.max(np.abs(got.astype(np.float64) - (dense + res)))) / float(np.max(np.abs(dense))) < TOL_F32
+    # q / k / v of one normalised input: 2048 + 512 + 612 rows side by side
+    parts = [(0, 2048), (2048, 2560), (2560, 3172)]
+    outs = nn.quantized_dense_batch([(dev(gpu, x), dev(gpu, np.ascontiguousarray(W[a:b])), q, None, None) for a, b in parts], norm=cfg)
+    gpu.cuda.synchronize()
+    for (a, b), y in zip(parts, outs):
+        assert rel_err(y.cpu().numpy(), dense[:, a:b]) < TOL_F32, (a, b)
+    # gated pair
+    assert gated_case(gpu, oracle, t, 96, K, 3140, 3, 1, True, 1520) < 2 * TOL_F32
+    assert gated_case(gpu, oracle, t, 130, K, 3140, 3, 0, False, 1530) < 2 * TOL_F32
 
 
 def test_q4_k_large_minima_through_the_split_k_kernel(gpu, oracle):
