@@ -72,13 +72,13 @@ _Q4K_PARTIAL = """            if (m < M) partial[((int64_t)slice * M + m) * set.
     }
 }
 
-// ---- the activation pre-pass folded into the main kernel"""
+// ---- several tiles of 32 batch rows per weight tile"""
 _Q4K_NO_PARTIAL = """            asm volatile("" ::"v"(v));
         }
     }
 }
 
-// ---- the activation pre-pass folded into the main kernel"""
+// ---- several tiles of 32 batch rows per weight tile"""
 _Q4K_XPREP = """    if (int rc = x_is_bf16 ? (fine ? prep(mmq_xprep_kernel<true, 1>) : prep(mmq_xprep_kernel<true, 2>))
                            : (fine ? prep(mmq_xprep_kernel<false, 1>) : prep(mmq_xprep_kernel<false, 2>)))
         return rc;
