@@ -79,6 +79,9 @@ _Q4K_NO_PARTIAL = """            asm volatile("" ::"v"(v));
 }
 
 // ---- several tiles of 32 batch rows per weight tile"""
+_Q4K_TILES_IMAGE = "        for (int i = wave; i < NT * 8; i += G::kWaves) {\n"
+_Q4K_TILES_NO_IMAGE = "        for (int i = wave; i < (sb == 0 ? NT * 8 : 0); i += G::kWaves) {\n"
+_Q4K_TILES_CONTRACT = "        q4k_tiles_half<NT, 0>(cur, lds, kg, col, magic, p1);\n"
 _Q4K_XPREP = """    if (int rc = x_is_bf16 ? (fine ? prep(mmq_xprep_kernel<true, 1>) : prep(mmq_xprep_kernel<true, 2>))
                            : (fine ? prep(mmq_xprep_kernel<false, 1>) : prep(mmq_xprep_kernel<false, 2>)))
         return rc;
@@ -131,6 +134,11 @@ VARIANTS = {
     "q4k_main_empty": ("mmq.hip", "image copy, weight loads and contraction of the main kernel together (launch, barriers, LDS hand-over and partial stores remain)",
                        [(_Q4K_IMAGE, "            (void)img;\n"), (_Q4K_FETCH0, ""), (_Q4K_FETCH, ""), (_Q4K_CONTRACT, _Q4K_KEEP)]),
     "q4k_no_partials": ("mmq.hip", "the main kernel's stores of its partial sums", [(_Q4K_PARTIAL, _Q4K_NO_PARTIAL)]),
+    "q4k_tiles_no_image": ("mmq.hip", "the image copies of the kernel for several batch tiles after its first super-block (barriers kept)",
+                           [(_Q4K_TILES_IMAGE, _Q4K_TILES_NO_IMAGE)]),
+    "q4k_tiles_no_contract": ("mmq.hip", "unpacking and MFMAs of the kernel for several batch tiles (loads, image copies and barriers kept)",
+                              [(_Q4K_TILES_CONTRACT, _Q4K_KEEP),
+                               ("        q4k_tiles_half<NT, 1>(cur, lds + G::kMaxTiles * G::kHalfBytes, kg, col, magic, p1);\n", "")]),
     "q4k_no_xprep": ("mmq.hip", "the activation pre-pass launch", [(_Q4K_XPREP, "    (void)prep;\n")]),
     "q4k_no_reduce": ("mmq.hip", "the reduction launch", [(_Q4K_REDUCE, "    if (count == 1) return GQ_OK;\n")]),
 }

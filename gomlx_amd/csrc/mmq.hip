@@ -290,77 +290,90 @@ __device__ __forceinline__ void q4k_contract_sb(const RawSB &cur, const uint8_t 
     }
 }
 
-// The same super-block against the images of RM tiles of 32 batch columns (tile t: fragments at img + 16384 t,
-// sub-block sums at sums + 512 t): the codes are turned into operand fragments ONCE and every
-// fragment meets each tile's activations, so the conversion, the parked tile and the header are shared by up to 128
-// batch rows.  Per tile the arithmetic and its order are those of q4k_contract_sb<false>.
-template <int RM>
-__device__ __forceinline__ void q4k_contract_sb_tiles(const RawSB &cur, const uint8_t *img, const uint8_t *sums, int kg, int col, uint32_t magic,
-                                                      f16v (&acc)[RM]) {
-    const float d = half_bits_to_float(cur.hd.x & 0xFFFFu), dmin = half_bits_to_float(cur.hd.x >> 16);
-    const uint32_t a = cur.hd.y, b = cur.hd.z, c = cur.hd.w;
-    const uint32_t sc_lo = a & 0x3F3F3F3Fu, mn_lo = b & 0x3F3F3F3Fu;
-    const uint32_t sc_hi = (c & 0x0F0F0F0Fu) | ((a >> 2) & 0x30303030u);
-    const uint32_t mn_hi = ((c >> 4) & 0x0F0F0F0Fu) | ((b >> 2) & 0x30303030u);
-    f16v p1[RM];
+// One super-block against the images of RM tiles of 32 batch columns at once: the codes are turned into operand fragments
+// ONCE and every fragment meets each tile's activations, so the conversion, the parked tile and the header are shared by
+// up to 128 batch rows.  Per tile the arithmetic and its order are those of q4k_contract_sb<false>.  The work comes in two
+// halves (steps 2 H and 2 H + 1 of the super-block's four), so that the images can be staged half a super-block at a time:
+// `img` holds tile t's half at 8192 t - 16 slots of (32 columns x 16 bytes) in the order of stage_x, whose slot index
+// modulo 16 is the position inside the half.
+template <int RM, int H>
+__device__ __forceinline__ void q4k_tiles_half(const RawSB &cur, const uint8_t *img, int kg, int col, uint32_t magic, f16v (&p1)[RM]) {
+    const uint32_t a = cur.hd.y, c = cur.hd.w;
+    const uint32_t sc = H == 0 ? (a & 0x3F3F3F3Fu) : ((c & 0x0F0F0F0Fu) | ((a >> 2) & 0x30303030u));  // scales 0..3 / 4..7 as bytes
+    // Eight groups (step s2, fragment q) of RM MFMAs each; the activations of group g + 1 are requested from LDS before the
+    // MFMAs of group g are issued and nothing moves across the group boundaries, so that two groups' fragments are all the
+    // registers the reads take (left to itself the compiler hoists sixteen reads and more, and four tiles spill).
+    h8 xf[2][RM];
+    auto request = [&](int g) __attribute__((always_inline)) {
+        const int slot = (2 * (g >> 2) + kg) * 4 + (g & 3);  // fragment 4 st + q sits in slot 32 sb + 8 st + 4 kg + q of the image: this is that modulo 16
 #pragma unroll
-    for (int t = 0; t < RM; t++)
+        for (int t = 0; t < RM; t++) xf[g & 1][t] = *reinterpret_cast<const h8 *>(img + t * 8192 + (slot * kMT + (col ^ slot)) * 16);
+    };
+    request(0);
+    uint32_t wl[8], wh[8];
 #pragma unroll
-        for (int r = 0; r < 16; r++) p1[t][r] = 0.f;
+    for (int g = 0; g < 8; g++) {
+        const int s2 = g >> 2, q = g & 3;
+        if (q == 0) {
+            const int st = 2 * H + s2;
+            const uint32_t scw = sc >> (16 * s2);
+            const float s0f = (float)(scw & 0xFFu), s1f = (float)((scw >> 8) & 0xFFu);
+            const h2 s0 = as_h2(pack_h2(s0f, s0f));
+            const h2 s1 = as_h2(pack_h2(s1f * 0.0625f, s1f * 0.0625f));  // high-nibble pairs arrive as 1024 + 16 n
+            const h2 k0h = as_h2(pack_h2(-1024.f * s0f, -1024.f * s0f));
+            const h2 k1h = as_h2(pack_h2(-64.f * s1f, -64.f * s1f));
+            const uint32_t dw[4] = {cur.c[st].x, cur.c[st].y, cur.c[st].z, cur.c[st].w};
 #pragma unroll
-    for (int st = 0; st < 4; st++) {
-        const uint32_t scw = (st < 2 ? sc_lo : sc_hi) >> (16 * (st & 1));
-        const float s0f = (float)(scw & 0xFFu), s1f = (float)((scw >> 8) & 0xFFu);
-        const h2 s0 = as_h2(pack_h2(s0f, s0f));
-        const h2 s1 = as_h2(pack_h2(s1f * 0.0625f, s1f * 0.0625f));
-        const h2 k0h = as_h2(pack_h2(-1024.f * s0f, -1024.f * s0f));
-        const h2 k1h = as_h2(pack_h2(-64.f * s1f, -64.f * s1f));
-        const uint32_t dw[4] = {cur.c[st].x, cur.c[st].y, cur.c[st].z, cur.c[st].w};
-        uint32_t wl[8], wh[8];
-#pragma unroll
-        for (int w = 0; w < 4; w++) {
-            const uint32_t u = dw[w], v = dw[w] >> 8;
-            wl[2 * w] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(u, 0x000F000Fu, magic), s0, k0h));
-            wl[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(v, 0x000F000Fu, magic), s0, k0h));
-            wh[2 * w] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(u, 0x00F000F0u, magic), s1, k1h));
-            wh[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(v, 0x00F000F0u, magic), s1, k1h));
-        }
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const uint32_t *src = (q < 2 ? wl : wh) + 4 * (q & 1);
-            const h8 wfrag = __builtin_bit_cast(h8, make_uint4(src[0], src[1], src[2], src[3]));
-            const int slot = (2 * st + kg) * 4 + q;  // (slot of fragment 4 st + q in a one-super-block image, see stage_x)
-#pragma unroll
-            for (int t = 0; t < RM; t++) {
-                const h8 xf = *reinterpret_cast<const h8 *>(img + t * 16384 + (slot * kMT + (col ^ (slot & 15))) * 16);
-                p1[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xf, wfrag, p1[t], 0, 0, 0);
+            for (int w = 0; w < 4; w++) {
+                const uint32_t u = dw[w], v = dw[w] >> 8;
+                wl[2 * w] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(u, 0x000F000Fu, magic), s0, k0h));
+                wl[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(v, 0x000F000Fu, magic), s0, k0h));
+                wh[2 * w] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(u, 0x00F000F0u, magic), s1, k1h));
+                wh[2 * w + 1] = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(magic_pair(v, 0x00F000F0u, magic), s1, k1h));
             }
         }
+        if (g + 1 < 8) request(g + 1);
+        const uint32_t *src = (q < 2 ? wl : wh) + 4 * (q & 1);
+        const h8 wfrag = __builtin_bit_cast(h8, make_uint4(src[0], src[1], src[2], src[3]));
+#pragma unroll
+        for (int t = 0; t < RM; t++) p1[t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xf[g & 1][t], wfrag, p1[t], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
     }
-    // minima against the sub-block sums, as in q4k_contract_sb: only k-group 0 carries operands (the sums are read by every
-    // lane and cleared by a select in k-group 1: no branch around an LDS read)
+}
+
+// The end of a super-block: the minima against the tiles' sub-block sums (tile t's at sums + 1024 t), then d and dmin in fp32;
+// p1 starts the next super-block at zero.  Only k-group 0 carries operands of the minima's MFMA (the sums are read by
+// every lane and cleared by a mask in k-group 1: no branch around an LDS read).
+template <int RM>
+__device__ __forceinline__ void q4k_tiles_finish(const RawSB &cur, const uint8_t *sums, int kg, int col, uint32_t magic, f16v (&p1)[RM], f16v (&acc)[RM]) {
+    const float d = half_bits_to_float(cur.hd.x & 0xFFFFu), dmin = half_bits_to_float(cur.hd.x >> 16);
+    const uint32_t a = cur.hd.y, b = cur.hd.z, c = cur.hd.w;
+    (void)a;
+    const uint32_t mn_lo = b & 0x3F3F3F3Fu, mn_hi = ((c >> 4) & 0x0F0F0F0Fu) | ((b >> 2) & 0x30303030u);
     f16v zero16;
 #pragma unroll
     for (int r = 0; r < 16; r++) zero16[r] = 0.f;
-    uint4 mv = make_uint4(0u, 0u, 0u, 0u);
-    {
-        const h2 off = as_h2(0xE400E400u);  // (-1024, -1024)
-        const uint32_t keep = kg == 0 ? 0xFFFFFFFFu : 0u;
-        mv.x = __builtin_bit_cast(uint32_t, magic_pair(mn_lo, 0x00FF00FFu, magic) + off) & keep;
-        mv.y = __builtin_bit_cast(uint32_t, magic_pair(mn_lo >> 8, 0x00FF00FFu, magic) + off) & keep;
-        mv.z = __builtin_bit_cast(uint32_t, magic_pair(mn_hi, 0x00FF00FFu, magic) + off) & keep;
-        mv.w = __builtin_bit_cast(uint32_t, magic_pair(mn_hi >> 8, 0x00FF00FFu, magic) + off) & keep;
-    }
+    const uint32_t keep = kg == 0 ? 0xFFFFFFFFu : 0u;
+    const h2 off = as_h2(0xE400E400u);  // (-1024, -1024)
+    uint4 mv;
+    mv.x = __builtin_bit_cast(uint32_t, magic_pair(mn_lo, 0x00FF00FFu, magic) + off) & keep;
+    mv.y = __builtin_bit_cast(uint32_t, magic_pair(mn_lo >> 8, 0x00FF00FFu, magic) + off) & keep;
+    mv.z = __builtin_bit_cast(uint32_t, magic_pair(mn_hi, 0x00FF00FFu, magic) + off) & keep;
+    mv.w = __builtin_bit_cast(uint32_t, magic_pair(mn_hi >> 8, 0x00FF00FFu, magic) + off) & keep;
 #pragma unroll
     for (int t = 0; t < RM; t++) {
-        uint4 sv = *reinterpret_cast<const uint4 *>(sums + t * 512 + col * 16);
-        const uint32_t keep = kg == 0 ? 0xFFFFFFFFu : 0u;
-        sv.x &= keep; sv.y &= keep; sv.z &= keep; sv.w &= keep;
+        // (a native vector type: read as HIP's uint4 struct the load loses what tells the compiler that it cannot touch the
+        // destination of a load into LDS, and it then waits for every such load in flight before this read)
+        typedef uint32_t Quad __attribute__((ext_vector_type(4)));
+        Quad sv = *reinterpret_cast<const Quad *>(sums + t * 1024 + col * 16);
+        sv &= keep;
         const f16v p2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8, sv), __builtin_bit_cast(h8, mv), zero16, 0, 0, 0);
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[t][r] = fmaf(d, p1[t][r], acc[t][r]);
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[t][r] = fmaf(-dmin, p2[r], acc[t][r]);
+#pragma unroll
+        for (int r = 0; r < 16; r++) p1[t][r] = 0.f;
     }
 }
 
@@ -513,15 +526,21 @@ __global__ __launch_bounds__(64 * RT * kParts) void mmq_q4k_kernel(const uint8_t
 //
 // mmq_q4k_kernel serves one tile of 32 batch rows per launch: 128 rows stream W four times and convert every code four
 // times.  mmq_q4k_tiles_kernel walks up to four such tiles together: eight wavefronts, each with its own row tile of 32 rows
-// of W (256 per workgroup) and all of the slice's super-blocks; the activation images of the tiles no longer fit LDS for
-// a whole slice, so the workgroup moves along K one super-block at a time - the images of that super-block for every
-// tile (16.5 KiB each, global -> LDS by DMA from the pre-pass's image), a barrier, then every wavefront's super-block
-// against all of them (q4k_contract_sb_tiles) while its next weight tile is on its way into its parked piece of LDS.
+// of W (256 per workgroup) and all of the slice's super-blocks.  The activation images of four tiles do not fit LDS for a
+// whole slice, so the workgroup moves along K half a super-block at a time: the halves of every tile's image (8 KiB each,
+// global -> LDS by DMA from the pre-pass's image) go through a ring of two stages - while the wavefronts contract one
+// half (q4k_tiles_half: every converted fragment against all tiles), the next is on its way - with one barrier per half.
+// A wavefront's weight tiles are parked two super-blocks ahead.  The waits are counted: a wavefront's loads complete in
+// the order they were issued, so "at most five outstanding" after a request of a weight tile (five load instructions)
+// means that everything older has landed, the image half among it.
 // Same grid roles, same image and partial-sum layouts as mmq_q4k_kernel (m0 = first batch row, NT = tiles of 32 from there).
 struct Q4KTiles {
     static constexpr int kMaxTiles = 4, kWaves = 8, kRows = 32 * kWaves;
-    static constexpr int kImgBytes = kMaxTiles * 16384, kSumBytes = kMaxTiles * kMT * 16;
-    static constexpr int kLds = kImgBytes + kSumBytes + kWaves * kParkBytes;
+    static constexpr int kHalfBytes = 8192;                                    // half a super-block of one tile's image
+    static constexpr int kRingBytes = 2 * kMaxTiles * kHalfBytes;              // two stages
+    static constexpr int kSumBytes = kMaxTiles * 1024;                         // sub-block sums of one super-block: 512 bytes per tile, 1 KiB apart
+    static constexpr int kParks = 2;                                           // weight tiles on their way per wavefront
+    static constexpr int kLds = kRingBytes + kSumBytes + kParks * kWaves * kParkBytes;
     static_assert(kLds <= 160 * 1024, "images + parked tiles exceed LDS");
 };
 
@@ -531,7 +550,7 @@ __global__ __launch_bounds__(64 * Q4KTiles::kWaves) void mmq_q4k_tiles_kernel(co
                                                                                const uint8_t *__restrict__ W2, float *__restrict__ partial2) {
     typedef Q4KTiles G;
     static_assert(NT >= 1 && NT <= G::kMaxTiles, "one to four tiles of 32 batch rows");
-    constexpr int ntile = NT;
+    static_assert(kParkLoads == 5, "the counted waits below assume five load instructions per weight tile");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     int prob = 0;
 #pragma unroll
@@ -543,7 +562,7 @@ __global__ __launch_bounds__(64 * Q4KTiles::kWaves) void mmq_q4k_tiles_kernel(co
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int kg = lane >> 5, col = lane & 31;
     const int slice = blockIdx.y, nslices = gridDim.y;
-    const int nsb = ((K >> 8) - slice + nslices - 1) / nslices;  // slice s holds super-blocks s, s + nslices, ... of every row
+    const int nsb = ((K >> 8) - slice + nslices - 1) / nslices;  // slice s holds super-blocks s, s + nslices, ... of every row (at least one)
     const int row0 = xblk * G::kRows + wave * 32;
     const int n = row0 + col;  // this lane's weight row
 
@@ -554,43 +573,69 @@ __global__ __launch_bounds__(64 * Q4KTiles::kWaves) void mmq_q4k_tiles_kernel(co
         const int c = min(lane + 64 * l, 32 * 9 - 1);
         csrc[l] = (uint32_t)(min(row0 + c / 9, N - 1) - min(row0, N - 1)) * (uint32_t)row_bytes + (uint32_t)((c % 9) * 16);
     }
-    uint8_t *park = lds + G::kImgBytes + G::kSumBytes + wave * kParkBytes;
+    uint8_t *const park0 = lds + G::kRingBytes + G::kSumBytes + wave * (G::kParks * kParkBytes);
+    // super-block j of this wavefront's row tile -> park j % 2: exactly kParkLoads load instructions
     auto fetch = [&](int sb) __attribute__((always_inline)) {
         const uint8_t *base = wtile + sb * nslices * 144;
+        uint8_t *park = park0 + (sb & 1) * kParkBytes;
 #pragma unroll
         for (int l = 0; l < kParkLoads; l++)
             if (64 * l + 64 <= 32 * 9 || lane < 32 * 9 - 64 * l)  // (the last instruction carries 32 chunks)
                 __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(base + csrc[l]),
                                                  (__attribute__((address_space(3))) void *)(park + l * 1024), 16, 0, 0);
     };
-    fetch(0);  // (every slice holds at least one super-block)
-    const uint8_t *myrow = park + col * 144;
-    // tile t's image of this slice: fragments of super-block j at 16384 j, its sub-block sums at kXFBytes + 512 j
+    // tile t's image of this slice: fragments of super-block j at 16384 j (its second half 8192 further), sums at kXFBytes + 512 j
     const uint8_t *img0 = ximg + ((size_t)(m0 / kMT) * nslices + slice) * kLdsBytes;
     const size_t tile_stride = (size_t)nslices * kLdsBytes;
+    // half `h` of super-block `sb` of every tile -> ring stage h; with the second half come the super-block's sub-block sums, which
+    // are read at its end and not again (one buffer, at a fixed address: the compiler's own wait insertion can tell it from the ring)
+    auto stage = [&](int sb, int h) __attribute__((always_inline)) {
+        uint8_t *dst = lds + h * (G::kMaxTiles * G::kHalfBytes);
+        for (int i = wave; i < NT * 8; i += G::kWaves) {
+            const int t = i >> 3, ck = i & 7;
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void *)(img0 + t * tile_stride + sb * 16384 + h * G::kHalfBytes + ck * 1024 + lane * 16),
+                (__attribute__((address_space(3))) void *)(dst + t * G::kHalfBytes + ck * 1024), 16, 0, 0);
+        }
+        // (every wavefront copies the 512 bytes of one tile's sums, with all 64 lanes - the upper half lands behind them, unused -
+        // and several wavefronts may copy the same tile's: no branch around a load into LDS, behind which the compiler would wait
+        // for every load in flight in front of the next LDS read)
+        if (h == 1)
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void *)(img0 + (wave % NT) * tile_stride + kXFBytes + sb * 512 + (lane & 31) * 16),
+                (__attribute__((address_space(3))) void *)(lds + G::kRingBytes + (wave % NT) * 1024), 16, 0, 0);
+    };
+    // (no fence: the loads that must have landed are waited for by count, and LDS reads have been consumed before a wavefront arrives)
+    auto meet = [&](bool all) __attribute__((always_inline)) {
+        // (the builtin, not written-out text: the compiler keeps its own count of loads into LDS and would otherwise wait for
+        // all of them in front of the first LDS read it cannot tell apart from their destinations)
+        if (all) __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+        else __builtin_amdgcn_s_waitcnt(0x0F75);       // vmcnt(5)
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
 
-    f16v acc[NT];
+    f16v acc[NT], p1[NT];
 #pragma unroll
     for (int t = 0; t < NT; t++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) acc[t][r] = 0.f;
+        for (int r = 0; r < 16; r++) acc[t][r] = p1[t][r] = 0.f;
     uint32_t magic;
     asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));
 
-    for (int sbl = 0; sbl < nsb; sbl++) {
-        __syncthreads();  // every wavefront has finished with the images of the super-block before
-        for (int i = wave; i < ntile * 16; i += G::kWaves) {
-            const int t = i >> 4, ck = i & 15;
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(img0 + t * tile_stride + sbl * 16384 + ck * 1024 + lane * 16),
-                                             (__attribute__((address_space(3))) void *)(lds + t * 16384 + ck * 1024), 16, 0, 0);
-        }
-        if (wave < ntile && lane < 32)
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(img0 + wave * tile_stride + kXFBytes + sbl * 512 + lane * 16),
-                                             (__attribute__((address_space(3))) void *)(lds + G::kImgBytes + wave * 512), 16, 0, 0);
-        // a barrier does not wait for loads in flight: this wavefront's share of the images (and its weight tile) must
-        // have landed before it arrives
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
+    // issue order: stage(0,0) fetch(0) fetch(1) | per super-block j: stage(j,1) fetch(j+2) | stage(j+1,0)
+    stage(0, 0);
+    asm volatile("" ::: "memory");  // (the counted waits rely on this order of the requests)
+    fetch(0);
+    asm volatile("" ::: "memory");
+    if (nsb > 1) fetch(1);
+    for (int sb = 0; sb < nsb; sb++) {
+        // first half: its image (requested one step ago) and this wavefront's weight tile must be there; every wavefront has
+        // finished with stage 1, which the second half's image now overwrites
+        meet(sb > 0 || nsb == 1);  // (super-block 0: only the request of tile 1 may still be out)
+        stage(sb, 1);
+        const uint8_t *myrow = park0 + (sb & 1) * kParkBytes + col * 144;
         typedef uint32_t Chunk __attribute__((ext_vector_type(4)));
         Chunk rhd = *reinterpret_cast<const Chunk *>(myrow), rc[4];
 #pragma unroll
@@ -601,8 +646,14 @@ __global__ __launch_bounds__(64 * Q4KTiles::kWaves) void mmq_q4k_tiles_kernel(co
 #pragma unroll
         for (int st = 0; st < 4; st++) cur.c[st] = make_uint4(rc[st].x, rc[st].y, rc[st].z, rc[st].w);
         __builtin_amdgcn_wave_barrier();
-        if (sbl + 1 < nsb) fetch(sbl + 1);
-        q4k_contract_sb_tiles<NT>(cur, lds, lds + G::kImgBytes, kg, col, magic, acc);
+        const bool more = sb + 2 < nsb;
+        if (more) fetch(sb + 2);
+        q4k_tiles_half<NT, 0>(cur, lds, kg, col, magic, p1);
+        // second half: the image requested above must be there (the request of tile sb + 2, issued after it, may still be out)
+        meet(!more);
+        if (sb + 1 < nsb) stage(sb + 1, 0);
+        q4k_tiles_half<NT, 1>(cur, lds + G::kMaxTiles * G::kHalfBytes, kg, col, magic, p1);
+        q4k_tiles_finish<NT>(cur, lds + G::kRingBytes, kg, col, magic, p1, acc);
     }
 
     if (n < N) {
