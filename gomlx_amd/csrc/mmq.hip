@@ -1552,7 +1552,8 @@ int launch_mmq_q6k(const MmqExtra *ex, const void *x, bool x_is_bf16, int64_t M,
 bool mmq_supported(int type, int64_t M, int64_t K, int64_t N, const void *x, const void *bias, const void *y) {
     // K <= 2^26: the kernels address the 32 rows of a tile by 32-bit byte offsets from its first row (31 rows of at most
     // 2^26 * 34 / 32 bytes stay below 2^32)
-    const bool shape_ok = M >= 2 && M <= 256 && N % 4 == 0 && N <= (int64_t)INT32_MAX / 2 && K <= ((int64_t)1 << 26) &&
+    // (Q4_K walks four tiles of 32 rows per launch and stays ahead of the two-pass GEMM for longer than the others)
+    const bool shape_ok = M >= 2 && M <= (type == kQ4_K ? 512 : 256) && N % 4 == 0 && N <= (int64_t)INT32_MAX / 2 && K <= ((int64_t)1 << 26) &&
                           ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(bias) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
     if (type == kQ4_K) return shape_ok && K % 256 == 0;
     if (type == kQ8_0 || type == kQ4_0 || type == kIQ4_NL) return shape_ok && K % 256 == 0;  // whole stretches of 8 blocks

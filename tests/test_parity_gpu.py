@@ -256,8 +256,8 @@ def test_split_k_small_batches_k_quants(gpu, oracle, t, M, K, N):
 
 def test_q4_k_split_k_walks_several_batch_tiles_together(gpu, oracle):
     """More than 32 batch rows on the Q4_K split-K route: one launch contracts up to four tiles of 32 rows against every weight
-    tile (codes converted once).  A long-K matrix of 25.6 MB, which keeps the route up to 256 rows: every tile count, a second
-    launch for the rows past 128 (tiles dealt evenly: 3 + 2, 4 + 4), a last tile that is partly filled, a width that is not a multiple of the workgroup's 256
+    tile (codes converted once).  A long-K matrix of 25.6 MB, which keeps the route up to 320 rows: every tile count, further
+    launches for the rows past 128 (tiles dealt evenly: 3 + 2, 4 + 4, 4 + 3 + 3), a last tile that is partly filled, a width that is not a multiple of the workgroup's 256
     rows; fp32 and bf16 activations; the gated pair, the projection with normalisation and residual, and q / k / v."""
     t, K, N = Q4_K, 14336, 3172
     assert N * ggml.row_bytes(t, K) >= 24 << 20
@@ -265,7 +265,7 @@ def test_q4_k_split_k_walks_several_batch_tiles_together(gpu, oracle):
     W = synth.weights(t, 1500, N, K)
     bias = synth.normal(1501, 0, N).astype(np.float32) * 0.1
     Wd = dev(gpu, W)
-    for M in (33, 64, 70, 96, 128, 129, 160, 250):
+    for M in (33, 64, 70, 96, 128, 129, 160, 250, 320):
         x = synth.activations(1502 + M, M, K)
         got = nn.quantized_dense(dev(gpu, x), Wd, q, dev(gpu, bias), BACKEND_ACT[3]).cpu().numpy()
         assert rel_err(got, oracle.c_qdense(t, x, W, bias, 3)) < TOL_F32, M
@@ -290,6 +290,7 @@ def test_q4_k_split_k_walks_several_batch_tiles_together(gpu, oracle):
     # gated pair
     assert gated_case(gpu, oracle, t, 96, K, 3140, 3, 1, True, 1520) < 2 * TOL_F32
     assert gated_case(gpu, oracle, t, 130, K, 3140, 3, 0, False, 1530) < 2 * TOL_F32
+    assert gated_case(gpu, oracle, t, 300, 4096, 11008, 3, 1, True, 1540) < 2 * TOL_F32  # (a wide pair of 25 MB each keeps the route up to 384 rows)
 
 
 def test_q4_k_large_minima_through_the_split_k_kernel(gpu, oracle):
