@@ -1578,11 +1578,11 @@ int coop_spin_ticks() {
     return v < 0 ? 0 : v > 100000000 ? 100000000 : (int)v;
 }
 
-// GOMLX_HIPQ_Q4K_TILES_TOGETHER=0: batches of more than 32 rows as one launch of mmq_q4k_kernel per 32 rows (tuning runs and
-// comparisons only).  Read at every call.
-bool tiles_together_enabled() {
+// GOMLX_HIPQ_Q4K_TILES_TOGETHER=0: batches of more than 32 rows as one launch of mmq_q4k_kernel per 32 rows; =2: batches of up
+// to 32 rows through mmq_q4k_tiles_kernel<1> as well (tuning runs and comparisons only).  Read at every call.
+int tiles_together_mode() {
     const char *e = std::getenv("GOMLX_HIPQ_Q4K_TILES_TOGETHER");
-    return !(e && e[0] == '0');
+    return e && e[0] >= '0' && e[0] <= '2' ? e[0] - '0' : 1;
 }
 
 // `count` Q4_K matrices against one activation image: the pre-pass once, every matrix's row ranges in one launch of the
@@ -1598,7 +1598,12 @@ int run_q4k_set(const void *x, bool x_is_bf16, int64_t M, int64_t K, int count, 
     const int mtiles = (int)((M + kMT - 1) / kMT);
     const int64_t sbs = K / 256;
     // more than 32 batch rows: the kernel that walks up to four tiles of 32 together (256 rows of W per workgroup)
-    const bool together = mtiles >= 2 && !coop_enabled() && tiles_together_enabled();
+    // (a single tile of up to 32 rows as well where the matrix is wide and large - 4096 -> 14336 at 32 rows 22.7 against 25.3 us,
+    // the gated pair 35.8 against 37.5, a 128k-vocabulary head 134 against 143 - but not on long-K ones: 14336 -> 4096 23.7 against 20.5)
+    int64_t all_rows = 0;
+    for (int i = 0; i < count; i++) all_rows += items[i].N;
+    const bool wide = all_rows >= 2 * K && all_rows * (K / 256) * 144 >= ((int64_t)24 << 20);
+    const bool together = !coop_enabled() && (tiles_together_mode() == 2 || (tiles_together_mode() == 1 && (mtiles >= 2 || wide)));
     static const bool tiles_lds_ok = [] {
         auto room = [](auto kernel) {
             return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, Q4KTiles::kLds) == hipSuccess;
