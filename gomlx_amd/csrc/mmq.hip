@@ -537,10 +537,16 @@ __global__ __launch_bounds__(64 * RT * kParts) void mmq_q4k_kernel(const uint8_t
 struct Q4KTiles {
     static constexpr int kMaxTiles = 4, kWaves = 8, kRows = 32 * kWaves;
     static constexpr int kHalfBytes = 8192;                                    // half a super-block of one tile's image
-    static constexpr int kRingBytes = 2 * kMaxTiles * kHalfBytes;              // two stages
-    static constexpr int kSumBytes = kMaxTiles * 1024;                         // sub-block sums of one super-block: 512 bytes per tile, 1 KiB apart
-    static constexpr int kParks = 2;                                           // weight tiles on their way per wavefront
-    static constexpr int kLds = kRingBytes + kSumBytes + kParks * kWaves * kParkBytes;
+};
+// LDS of the kernel for NT tiles: [ring: 2 stages x NT halves][sums][parked weight tiles].  A single tile keeps one parked
+// tile per wavefront, which lets two workgroups share a CU (53 KiB each); more tiles are bound to one workgroup by their
+// registers anyway and park two.
+template <int NT> struct Q4KTilesOf {
+    static constexpr int kStageBytes = NT * Q4KTiles::kHalfBytes;
+    static constexpr int kRingBytes = 2 * kStageBytes;
+    static constexpr int kSumBytes = NT * 1024;                                // sub-block sums of one super-block: 512 bytes per tile, 1 KiB apart
+    static constexpr int kParks = NT == 1 ? 1 : 2;                             // weight tiles on their way per wavefront
+    static constexpr int kLds = kRingBytes + kSumBytes + kParks * Q4KTiles::kWaves * kParkBytes;
     static_assert(kLds <= 160 * 1024, "images + parked tiles exceed LDS");
 };
 
@@ -549,6 +555,7 @@ __global__ __launch_bounds__(64 * Q4KTiles::kWaves) void mmq_q4k_tiles_kernel(co
                                                                                int M, int K, int64_t row_bytes, int m0,
                                                                                const uint8_t *__restrict__ W2, float *__restrict__ partial2) {
     typedef Q4KTiles G;
+    typedef Q4KTilesOf<NT> L;
     static_assert(NT >= 1 && NT <= G::kMaxTiles, "one to four tiles of 32 batch rows");
     static_assert(kParkLoads == 5, "the counted waits below assume five load instructions per weight tile");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -573,11 +580,11 @@ __global__ __launch_bounds__(64 * Q4KTiles::kWaves) void mmq_q4k_tiles_kernel(co
         const int c = min(lane + 64 * l, 32 * 9 - 1);
         csrc[l] = (uint32_t)(min(row0 + c / 9, N - 1) - min(row0, N - 1)) * (uint32_t)row_bytes + (uint32_t)((c % 9) * 16);
     }
-    uint8_t *const park0 = lds + G::kRingBytes + G::kSumBytes + wave * (G::kParks * kParkBytes);
-    // super-block j of this wavefront's row tile -> park j % 2: exactly kParkLoads load instructions
+    uint8_t *const park0 = lds + L::kRingBytes + L::kSumBytes + wave * (L::kParks * kParkBytes);
+    // super-block j of this wavefront's row tile -> park j % kParks: exactly kParkLoads load instructions
     auto fetch = [&](int sb) __attribute__((always_inline)) {
         const uint8_t *base = wtile + sb * nslices * 144;
-        uint8_t *park = park0 + (sb & 1) * kParkBytes;
+        uint8_t *park = park0 + (sb % L::kParks) * kParkBytes;
 #pragma unroll
         for (int l = 0; l < kParkLoads; l++)
             if (64 * l + 64 <= 32 * 9 || lane < 32 * 9 - 64 * l)  // (the last instruction carries 32 chunks)
@@ -590,7 +597,7 @@ __global__ __launch_bounds__(64 * Q4KTiles::kWaves) void mmq_q4k_tiles_kernel(co
     // half `h` of super-block `sb` of every tile -> ring stage h; with the second half come the super-block's sub-block sums, which
     // are read at its end and not again (one buffer, at a fixed address: the compiler's own wait insertion can tell it from the ring)
     auto stage = [&](int sb, int h) __attribute__((always_inline)) {
-        uint8_t *dst = lds + h * (G::kMaxTiles * G::kHalfBytes);
+        uint8_t *dst = lds + h * L::kStageBytes;
         for (int i = wave; i < NT * 8; i += G::kWaves) {
             const int t = i >> 3, ck = i & 7;
             __builtin_amdgcn_global_load_lds(
@@ -603,7 +610,7 @@ __global__ __launch_bounds__(64 * Q4KTiles::kWaves) void mmq_q4k_tiles_kernel(co
         if (h == 1)
             __builtin_amdgcn_global_load_lds(
                 (const __attribute__((address_space(1))) void *)(img0 + (wave % NT) * tile_stride + kXFBytes + sb * 512 + (lane & 31) * 16),
-                (__attribute__((address_space(3))) void *)(lds + G::kRingBytes + (wave % NT) * 1024), 16, 0, 0);
+                (__attribute__((address_space(3))) void *)(lds + L::kRingBytes + (wave % NT) * 1024), 16, 0, 0);
     };
     // (no fence: the loads that must have landed are waited for by count, and LDS reads have been consumed before a wavefront arrives)
     auto meet = [&](bool all) __attribute__((always_inline)) {
@@ -624,18 +631,19 @@ __global__ __launch_bounds__(64 * Q4KTiles::kWaves) void mmq_q4k_tiles_kernel(co
     uint32_t magic;
     asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));
 
-    // issue order: stage(0,0) fetch(0) fetch(1) | per super-block j: stage(j,1) fetch(j+2) | stage(j+1,0)
+    // issue order (two parks): stage(0,0) fetch(0) fetch(1) | per super-block j: stage(j,1) fetch(j+2) | stage(j+1,0);
+    // with one park the weight tiles are requested one super-block ahead: stage(0,0) fetch(0) | stage(j,1) fetch(j+1) | stage(j+1,0)
     stage(0, 0);
     asm volatile("" ::: "memory");  // (the counted waits rely on this order of the requests)
     fetch(0);
     asm volatile("" ::: "memory");
-    if (nsb > 1) fetch(1);
+    if (L::kParks == 2 && nsb > 1) fetch(1);
     for (int sb = 0; sb < nsb; sb++) {
         // first half: its image (requested one step ago) and this wavefront's weight tile must be there; every wavefront has
         // finished with stage 1, which the second half's image now overwrites
-        meet(sb > 0 || nsb == 1);  // (super-block 0: only the request of tile 1 may still be out)
+        meet(sb > 0 || nsb == 1 || L::kParks == 1);  // (two parks, super-block 0: only the request of tile 1 may still be out)
         stage(sb, 1);
-        const uint8_t *myrow = park0 + (sb & 1) * kParkBytes + col * 144;
+        const uint8_t *myrow = park0 + (sb % L::kParks) * kParkBytes + col * 144;
         typedef uint32_t Chunk __attribute__((ext_vector_type(4)));
         Chunk rhd = *reinterpret_cast<const Chunk *>(myrow), rc[4];
 #pragma unroll
@@ -646,14 +654,14 @@ __global__ __launch_bounds__(64 * Q4KTiles::kWaves) void mmq_q4k_tiles_kernel(co
 #pragma unroll
         for (int st = 0; st < 4; st++) cur.c[st] = make_uint4(rc[st].x, rc[st].y, rc[st].z, rc[st].w);
         __builtin_amdgcn_wave_barrier();
-        const bool more = sb + 2 < nsb;
-        if (more) fetch(sb + 2);
+        const bool more = sb + L::kParks < nsb;
+        if (more) fetch(sb + L::kParks);
         q4k_tiles_half<NT, 0>(cur, lds, kg, col, magic, p1);
-        // second half: the image requested above must be there (the request of tile sb + 2, issued after it, may still be out)
+        // second half: the image requested above must be there (the request of a weight tile, issued after it, may still be out)
         meet(!more);
         if (sb + 1 < nsb) stage(sb + 1, 0);
-        q4k_tiles_half<NT, 1>(cur, lds + G::kMaxTiles * G::kHalfBytes, kg, col, magic, p1);
-        q4k_tiles_finish<NT>(cur, lds + G::kRingBytes, kg, col, magic, p1, acc);
+        q4k_tiles_half<NT, 1>(cur, lds + L::kStageBytes, kg, col, magic, p1);
+        q4k_tiles_finish<NT>(cur, lds + L::kRingBytes, kg, col, magic, p1, acc);
     }
 
     if (n < N) {
@@ -1605,12 +1613,13 @@ int run_q4k_set(const void *x, bool x_is_bf16, int64_t M, int64_t K, int count, 
     const bool wide = all_rows >= 2 * K && all_rows * (K / 256) * 144 >= ((int64_t)24 << 20);
     const bool together = !coop_enabled() && (tiles_together_mode() == 2 || (tiles_together_mode() == 1 && (mtiles >= 2 || wide)));
     static const bool tiles_lds_ok = [] {
-        auto room = [](auto kernel) {
-            return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, Q4KTiles::kLds) == hipSuccess;
+        auto room = [](auto kernel, int bytes) {
+            return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess;
         };
-        return room(mmq_q4k_tiles_kernel<1>) && room(mmq_q4k_tiles_kernel<2>) && room(mmq_q4k_tiles_kernel<3>) && room(mmq_q4k_tiles_kernel<4>);
+        return room(mmq_q4k_tiles_kernel<1>, Q4KTilesOf<1>::kLds) && room(mmq_q4k_tiles_kernel<2>, Q4KTilesOf<2>::kLds) &&
+               room(mmq_q4k_tiles_kernel<3>, Q4KTilesOf<3>::kLds) && room(mmq_q4k_tiles_kernel<4>, Q4KTilesOf<4>::kLds);
     }();
-    if (together && !tiles_lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", Q4KTiles::kLds);
+    if (together && !tiles_lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", Q4KTilesOf<4>::kLds);
     const int wg_rows = together ? Q4KTiles::kRows : Tile::kRows;
     Q4KSet set = {};
     MmqSetOut out = {};
@@ -1707,12 +1716,14 @@ int run_q4k_set(const void *x, bool x_is_bf16, int64_t M, int64_t K, int count, 
         const int ntile = (mtiles - tile0 + (nlaunch - l) - 1) / (nlaunch - l);
         const int64_t m0 = (int64_t)tile0 * kMT;
         tile0 += ntile;
-        auto go = [&](auto kernel) {
-            return launch(kernel, grid, dim3(64 * Q4KTiles::kWaves), (size_t)Q4KTiles::kLds, s, (const uint8_t *)ximg, set, partial, (int)M, (int)K,
-                          row_bytes, (int)m0, W2, partial2);
+        auto go = [&](auto kernel, int lds_bytes) {
+            return launch(kernel, grid, dim3(64 * Q4KTiles::kWaves), (size_t)lds_bytes, s, (const uint8_t *)ximg, set, partial, (int)M, (int)K, row_bytes,
+                          (int)m0, W2, partial2);
         };
-        if (int rc = ntile == 4 ? go(mmq_q4k_tiles_kernel<4>) : ntile == 3 ? go(mmq_q4k_tiles_kernel<3>) : ntile == 2 ? go(mmq_q4k_tiles_kernel<2>)
-                                                                                                                     : go(mmq_q4k_tiles_kernel<1>))
+        if (int rc = ntile == 4   ? go(mmq_q4k_tiles_kernel<4>, Q4KTilesOf<4>::kLds)
+                     : ntile == 3 ? go(mmq_q4k_tiles_kernel<3>, Q4KTilesOf<3>::kLds)
+                     : ntile == 2 ? go(mmq_q4k_tiles_kernel<2>, Q4KTilesOf<2>::kLds)
+                                  : go(mmq_q4k_tiles_kernel<1>, Q4KTilesOf<1>::kLds))
             return rc;
     }
     for (int64_t m0 = 0; !together && m0 < M; m0 += kMT) {
