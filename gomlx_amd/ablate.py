@@ -138,7 +138,7 @@ VARIANTS = {
                            [(_Q4K_TILES_IMAGE, _Q4K_TILES_NO_IMAGE)]),
     "q4k_tiles_no_contract": ("mmq.hip", "unpacking and MFMAs of the kernel for several batch tiles (loads, image copies and barriers kept)",
                               [(_Q4K_TILES_CONTRACT, _Q4K_KEEP),
-                               ("        q4k_tiles_half<NT, 1>(cur, lds + G::kMaxTiles * G::kHalfBytes, kg, col, magic, p1);\n", "")]),
+                               ("        q4k_tiles_half<NT, 1>(cur, lds + L::kStageBytes, kg, col, magic, p1);\n", "")]),
     "q4k_no_xprep": ("mmq.hip", "the activation pre-pass launch", [(_Q4K_XPREP, "    (void)prep;\n")]),
     "q4k_no_reduce": ("mmq.hip", "the reduction launch", [(_Q4K_REDUCE, "    if (count == 1) return GQ_OK;\n")]),
 }
