@@ -99,7 +99,7 @@ int gq_dequantize(int type, const void *dW, int64_t N, int64_t K, float *dOut, v
  * (ml/nn/quantized_dense.go:31-57) and ggml.DenseDecomposed (ml/ggml/dense.go:23-62).
  * dBias may be NULL.  fp32 activations, fp32 accumulation.  The first few rows (4 to 6, depending
  * on format and matrix size; 16 for matrices of a few megabytes) run as bandwidth-bound GEMV
- * passes; larger batches contract on the matrix cores with the activations (and, from 65 to 193
+ * passes; larger batches contract on the matrix cores with the activations (and, from 65 to 385
  * rows on, depending on format and shape, the dequantised weights) rounded to fp16 operands (each batch row scaled by a power of two first, so the magnitude of x does not
  * matter).  Batches of 5 rows and more may use a
  * per-stream workspace that is created on the first such call on the stream: make
