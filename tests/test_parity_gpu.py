@@ -1254,6 +1254,32 @@ def test_batched_submissions_randomized(gpu, oracle):
             assert err < TOL_F32, (case, ggml.name(t), rows, use_norm, bf16, W.shape, act, err)
 
 
+@pytest.mark.parametrize("t", ALL_TYPES)
+def test_batches_between_decode_and_prefill_randomized(gpu, oracle, t):
+    """Seeded random dense problems at 17 to 400 rows: the range in which the routes change hands (split-K kernels with one or
+    several tiles of 32 rows per launch, the two-pass GEMM with and without its own split of K).  Widths that are and are not
+    multiples of 4, 32 and 256, K from one to forty 256-value stretches, fp32 and bf16 activations scaled over six decades."""
+    rng = np.random.default_rng(9000 + t)
+    for case in range(10):
+        M = int(rng.integers(17, 401))
+        K = 256 * int(rng.integers(1, 41)) * (2 if t == Q6_K and rng.integers(0, 2) else 1)
+        N = int(rng.choice([4 * int(rng.integers(1, 300)), 32 * int(rng.integers(1, 80)), int(rng.integers(1, 900)), 256 * int(rng.integers(1, 9))]))
+        act = int(rng.choice([0, 1, 2, 3, 4]))
+        W = synth.weights(t, 9100 + case, N, K)
+        bias = synth.normal(9200 + case, 0, N).astype(np.float32) * 0.1 if rng.integers(0, 2) else None
+        x = (synth.activations(9300 + case, M, K) * float(10.0 ** rng.uniform(-3, 3))).astype(np.float32)
+        got = run_dense(gpu, t, x, W, bias, act)
+        want = oracle.c_qdense(t, x, W, bias, act)
+        pre = oracle.c_qdense(t, x, W, bias, 0)  # (an activation that saturates hides the contraction: judge on the larger scale)
+        scale = max(float(np.max(np.abs(want))), float(np.max(np.abs(pre)))) or 1.0
+        err = float(np.max(np.abs(got.astype(np.float64) - want))) / scale
+        assert err < TOL_F32, (ggml.name(t), case, M, K, N, act, err)
+        if case % 3 == 0:
+            xb = bf16_round(x)
+            got = run_dense(gpu, t, xb, W, bias, 0, bf16=True)
+            assert rel_err(got, oracle.c_qdense(t, xb, W, bias, 0)) < TOL_BF16, (ggml.name(t), case, M, K, N, "bf16")
+
+
 def test_shared_split_k_pass_randomized(gpu, oracle):
     """Seeded random lists of two to four Q4_K projections of one input, 6 to 99 rows, any widths that are multiples of 4
     (most not multiples of the 128-row workgroup), with and without normalisation, gain, bias; activations without tanh
