@@ -1,4 +1,4 @@
-// Small-batch (decode batch 5..~128) quantised Dense on the gfx950 matrix cores: Q4_K, and further
+// Small-batch (decode batch 5..~128; Q4_K up to 512 rows) quantised Dense on the gfx950 matrix cores: Q4_K, and further
 // down Q8_0 / Q4_0 / IQ4_NL and Q6_K.
 //
 // At batch 32 the contraction is 228 flop per weight byte: far beyond the vector ALUs, still
