@@ -265,10 +265,11 @@ def test_q4_k_split_k_walks_several_batch_tiles_together(gpu, oracle):
     W = synth.weights(t, 1500, N, K)
     bias = synth.normal(1501, 0, N).astype(np.float32) * 0.1
     Wd = dev(gpu, W)
+    x_all = synth.activations(1502, 320, K)
+    want_all = oracle.c_qdense(t, x_all, W, bias, 3)  # (rows are independent: one oracle pass serves every batch size)
     for M in (33, 64, 70, 96, 128, 129, 160, 250, 320):
-        x = synth.activations(1502 + M, M, K)
-        got = nn.quantized_dense(dev(gpu, x), Wd, q, dev(gpu, bias), BACKEND_ACT[3]).cpu().numpy()
-        assert rel_err(got, oracle.c_qdense(t, x, W, bias, 3)) < TOL_F32, M
+        got = nn.quantized_dense(dev(gpu, np.ascontiguousarray(x_all[320 - M:])), Wd, q, dev(gpu, bias), BACKEND_ACT[3]).cpu().numpy()
+        assert rel_err(got, want_all[320 - M:]) < TOL_F32, M
     xb = bf16_round(synth.activations(1510, 100, K))
     assert rel_err(run_dense(gpu, t, xb, W, bias, 0, bf16=True), oracle.c_qdense(t, xb, W, bias, 0)) < TOL_F32
     # projection with normalisation and residual
@@ -288,9 +289,9 @@ def test_q4_k_split_k_walks_several_batch_tiles_together(gpu, oracle):
     for (a, b), y in zip(parts, outs):
         assert rel_err(y.cpu().numpy(), dense[:, a:b]) < TOL_F32, (a, b)
     # gated pair
-    assert gated_case(gpu, oracle, t, 96, K, 3140, 3, 1, True, 1520) < 2 * TOL_F32
-    assert gated_case(gpu, oracle, t, 130, K, 3140, 3, 0, False, 1530) < 2 * TOL_F32
-    assert gated_case(gpu, oracle, t, 300, 4096, 11008, 3, 1, True, 1540) < 2 * TOL_F32  # (a wide pair of 25 MB each keeps the route up to 384 rows)
+    assert gated_case(gpu, oracle, t, 96, K, 1028, 3, 1, True, 1520) < 2 * TOL_F32
+    assert gated_case(gpu, oracle, t, 130, 4096, 2052, 3, 0, False, 1530) < 2 * TOL_F32
+    assert gated_case(gpu, oracle, t, 170, 4096, 11008, 3, 1, True, 1540) < 2 * TOL_F32  # (a wide pair of 25 MB each keeps the route past 160 rows, up to 384)
 
 
 def test_q4_k_large_minima_through_the_split_k_kernel(gpu, oracle):
