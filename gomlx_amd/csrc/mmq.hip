@@ -1307,6 +1307,175 @@ __global__ __launch_bounds__(RT * 128) void mmq_b32_kernel(const uint8_t *__rest
     }
 }
 
+// ---- the 18-byte-block formats at more than 32 batch rows -------------------------------------------------------
+//
+// A 256-value stretch of Q4_0 or IQ4_NL is 144 bytes of a row, like a Q4_K super-block, and rows are 16-byte aligned when K
+// is a multiple of 256: mmq_q4k_tiles_kernel's plan carries over as it stands - eight wavefronts with a row tile of 32 rows
+// each, weight tiles parked in LDS by DMA two stretches ahead, the images of up to four tiles of 32 batch rows staged half
+// a stretch (four blocks) at a time through a ring of two stages with counted waits - and only the arithmetic differs:
+// per block two MFMAs per tile against fragments converted ONCE for all tiles, and the block's d applied to each tile's
+// sums in fp32.  Slices are S consecutive values (512 or 1024), the image is mmq_b32_xprep_kernel's.
+int tiles_together_mode();
+
+template <int NT> struct B32TilesOf {  // LDS: [ring: 2 stages x NT halves of 8 KiB][two parked stretches per wavefront]
+    static constexpr int kStageBytes = NT * Q4KTiles::kHalfBytes;
+    static constexpr int kRingBytes = 2 * kStageBytes;
+    static constexpr int kParks = 2;
+    static constexpr int kLds = kRingBytes + kParks * Q4KTiles::kWaves * kParkBytes + 16;  // (+ slack: a code window may end past the last row)
+    static_assert(kLds <= 160 * 1024, "images + parked tiles exceed LDS");
+};
+
+template <int T, int NT>
+__global__ __launch_bounds__(64 * Q4KTiles::kWaves) void mmq_b32_tiles_kernel(const uint8_t *__restrict__ ximg, const uint8_t *__restrict__ W0,
+                                                                               float *__restrict__ partial0, int M, int K, int N, int64_t row_bytes, int S,
+                                                                               int m0, const uint8_t *__restrict__ W2, float *__restrict__ partial2) {
+    typedef B32<T> F;
+    typedef Q4KTiles G;
+    typedef B32TilesOf<NT> L;
+    static_assert(F::kBlockBytes == 18 && kB32Stretch * F::kBlockBytes * 32 == kParkBytes, "a stretch of 32 rows is a parked tile of 32 x 144 bytes");
+    static_assert(kParkLoads == 5, "the counted waits below assume five load instructions per weight tile");
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const uint8_t *__restrict__ W = blockIdx.z ? W2 : W0;
+    float *__restrict__ partial = blockIdx.z ? partial2 : partial0;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kg = lane >> 5, col = lane & 31;
+    const int slice = blockIdx.y, nslices = gridDim.y;
+    const int per_slice = S >> 8, first = slice * per_slice;
+    const int nst = min(per_slice, (K >> 8) - first);  // stretches of this slice (at least one)
+    const int row0 = (int)blockIdx.x * G::kRows + wave * 32;
+    const int n = row0 + col;  // this lane's weight row
+
+    const uint8_t *wtile = W + (int64_t)min(row0, N - 1) * row_bytes + (int64_t)first * 144;
+    uint32_t csrc[kParkLoads];
+#pragma unroll
+    for (int l = 0; l < kParkLoads; l++) {
+        const int c = min(lane + 64 * l, 32 * 9 - 1);
+        csrc[l] = (uint32_t)(min(row0 + c / 9, N - 1) - min(row0, N - 1)) * (uint32_t)row_bytes + (uint32_t)((c % 9) * 16);
+    }
+    uint8_t *const park0 = lds + L::kRingBytes + wave * (L::kParks * kParkBytes);
+    auto fetch = [&](int j) __attribute__((always_inline)) {  // stretch j of the slice -> park j % 2: exactly kParkLoads load instructions
+        const uint8_t *base = wtile + j * 144;
+        uint8_t *park = park0 + (j & 1) * kParkBytes;
+#pragma unroll
+        for (int l = 0; l < kParkLoads; l++)
+            if (64 * l + 64 <= 32 * 9 || lane < 32 * 9 - 64 * l)  // (the last instruction carries 32 chunks)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(base + csrc[l]),
+                                                 (__attribute__((address_space(3))) void *)(park + l * 1024), 16, 0, 0);
+    };
+    // tile t's image of this slice: [octet][32 columns][16 bytes], 32 octets (16 KiB) per stretch
+    const size_t img_bytes = (size_t)S * 64;
+    const uint8_t *img0 = ximg + ((size_t)(m0 / kMT) * nslices + slice) * img_bytes;
+    const size_t tile_stride = (size_t)nslices * img_bytes;
+    auto stage = [&](int j, int h) __attribute__((always_inline)) {  // half h (four blocks) of stretch j of every tile -> ring stage h
+        uint8_t *dst = lds + h * L::kStageBytes;
+        for (int i = wave; i < NT * 8; i += G::kWaves) {
+            const int t = i >> 3, ck = i & 7;
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void *)(img0 + t * tile_stride + j * 16384 + h * G::kHalfBytes + ck * 1024 + lane * 16),
+                (__attribute__((address_space(3))) void *)(dst + t * G::kHalfBytes + ck * 1024), 16, 0, 0);
+        }
+    };
+    auto meet = [&](bool all) __attribute__((always_inline)) {  // (see mmq_q4k_tiles_kernel)
+        if (all) __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+        else __builtin_amdgcn_s_waitcnt(0x0F75);       // vmcnt(5)
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
+
+    f16v acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[t][r] = 0.f;
+    uint32_t magic;
+    asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));
+
+    // four blocks of the parked stretch (read in place: the park is not requested again before the stretch is done) against
+    // ring stage H: block b's codes are lane (col, kg)'s eight bytes, a dword window from the dword at or below them,
+    // funnel-shifted when the block starts 2 bytes off a dword (every even block)
+    auto half = [&](auto hc, const uint8_t *myrow) __attribute__((always_inline)) {
+        constexpr int H = decltype(hc)::value;
+        const uint8_t *img = lds + H * L::kStageBytes;
+#pragma unroll
+        for (int bb = 0; bb < 4; bb++) {
+            const int b = 4 * H + bb;
+            const int at = b * F::kBlockBytes + F::code_byte(kg);
+            const uint32_t *wp = reinterpret_cast<const uint32_t *>(myrow + (at & ~3));
+            uint32_t w[F::kWin], c[F::kWin - 1];
+#pragma unroll
+            for (int q = 0; q < F::kWin; q++) w[q] = wp[q];
+#pragma unroll
+            for (int q = 0; q < F::kWin - 1; q++) c[q] = (b & 1) ? w[q] : __builtin_amdgcn_alignbit(w[q + 1], w[q], 16);
+            const float d = half_bits_to_float(*reinterpret_cast<const uint16_t *>(myrow + b * F::kBlockBytes));
+            const h8 f0 = F::frag(c, 0, magic), f1 = F::frag(c, 1, magic);
+            const int o0 = F::octet(bb, kg, 0), o1 = F::octet(bb, kg, 1);  // octets of the half: 0 .. 15
+            // (two tiles at a time and nothing moved across the pairs: with all four tiles' products in flight the kernel spills)
+#pragma unroll
+            for (int t0 = 0; t0 < NT; t0 += 2) {
+                f16v p[2];
+#pragma unroll
+                for (int u = 0; u < 2; u++) {
+                    const int t = t0 + u;
+                    if (t >= NT) continue;
+                    const h8 x0 = *reinterpret_cast<const h8 *>(img + t * G::kHalfBytes + (o0 * kMT + col) * 16);
+                    const h8 x1 = *reinterpret_cast<const h8 *>(img + t * G::kHalfBytes + (o1 * kMT + col) * 16);
+#pragma unroll
+                    for (int r = 0; r < 16; r++) p[u][r] = 0.f;
+                    p[u] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x0, f0, p[u], 0, 0, 0);
+                    p[u] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x1, f1, p[u], 0, 0, 0);
+                }
+#pragma unroll
+                for (int u = 0; u < 2; u++) {
+                    const int t = t0 + u;
+                    if (t >= NT) continue;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[t][r] = fmaf(d, p[u][r], acc[t][r]);
+                    // (the sums are pinned here: left free, the multiply-adds drift to the end of the stretch and every block's
+                    // products stay in registers until then - 192 registers for one tile, spills from two)
+                    asm volatile("" : "+v"(acc[t]));
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+
+    // issue order: stage(0,0) fetch(0) fetch(1) | per stretch j: stage(j,1) | stage(j+1,0) fetch(j+2)
+    stage(0, 0);
+    asm volatile("" ::: "memory");  // (the counted waits rely on this order of the requests)
+    fetch(0);
+    asm volatile("" ::: "memory");
+    if (nst > 1) fetch(1);
+    for (int j = 0; j < nst; j++) {
+        // first half: its image and this wavefront's stretch must be there (the request of the next stretch, issued after both, may
+        // still be out); every wavefront has finished with stage 1, which the second half's image now overwrites
+        meet(j + 1 >= nst);
+        stage(j, 1);
+        const uint8_t *myrow = park0 + (j & 1) * kParkBytes + col * 144;
+        half(std::integral_constant<int, 0>(), myrow);
+        // second half: the image requested above is the youngest request
+        meet(true);
+        if (j + 1 < nst) stage(j + 1, 0);
+        half(std::integral_constant<int, 1>(), myrow);
+        // the stretch has been read out: its park takes the stretch after the next
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+        if (j + 2 < nst) fetch(j + 2);
+    }
+
+    if (n < N) {
+        // lane holds y[m = 32 t + 8 (r / 4) + 4 kg + r % 4][n] for its K-slice
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = m0 + 32 * t + 8 * (r >> 2) + 4 * kg + (r & 3);
+                if (m < M) partial[((int64_t)slice * M + m) * N + n] = acc[t][r];
+            }
+        }
+    }
+}
+
 template <int T, int RT>
 int launch_mmq_b32(const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y, hipStream_t s,
                    const MmqExtra *ex) {
@@ -1314,10 +1483,18 @@ int launch_mmq_b32(const void *x, bool x_is_bf16, int64_t M, int64_t K, const ui
     const RmsNorm *norm = ex ? ex->norm : nullptr;
     const int cus = device_cu_count();
     const int mtiles = (int)((M + kMT - 1) / kMT);
-    const int64_t rowwgs = (N + 32 * RT - 1) / (32 * RT);
+    // more than 32 batch rows of an 18-byte-block format: the kernel that walks up to four tiles of 32 rows per launch
+    constexpr bool kHasTiles = B32<T>::kBlockBytes == 18;
+    // (where its 256-row workgroups with the shortest slices still cover three quarters of the CUs: on 4096 x 4096 they are 128, and
+    // the kernel below it stays ahead from 128 rows on, 26 against 32 us)
+    const bool together = kHasTiles && mtiles >= 2 && tiles_together_mode() != 0 &&
+                          ((N + Q4KTiles::kRows - 1) / Q4KTiles::kRows) * ((K + 511) / 512) * (W2 ? 2 : 1) >= (int64_t)cus * 3 / 4;
+    const int64_t rowwgs = together ? (N + Q4KTiles::kRows - 1) / Q4KTiles::kRows : (N + 32 * RT - 1) / (32 * RT);
     // slices of 1024 when that still leaves every CU a workgroup and a half (LDS holds a 1024-value image
-    // next to the parked stretches, not a 2048-value one)
-    const int S = rowwgs * ((K + 1023) / 1024) * mtiles >= (int64_t)cus * 3 / 2 ? 1024 : 512;
+    // next to the parked stretches, not a 2048-value one); the kernel for several tiles has one workgroup per CU at a time
+    // and takes the long slices from three quarters of the CUs on
+    const int S = together ? (rowwgs * ((K + 1023) / 1024) * (W2 ? 2 : 1) >= (int64_t)cus * 3 / 4 ? 1024 : 512)
+                           : (rowwgs * ((K + 1023) / 1024) * mtiles >= (int64_t)cus * 3 / 2 ? 1024 : 512);
     const int nslices = (int)((K + S - 1) / S);
     const size_t lds_bytes = (size_t)S * 64 + (size_t)2 * RT * B32Geom<T>::kWaveLds;  // image (later the handed-over tiles) + parked stretches
     static const bool lds_ok = [] {
@@ -1341,8 +1518,38 @@ int launch_mmq_b32(const void *x, bool x_is_bf16, int64_t M, int64_t K, const ui
                       norm ? mmq_xss(xscale, nslices, M) : nullptr);
     };
     if (int rc = x_is_bf16 ? prep(mmq_b32_xprep_kernel<true>) : prep(mmq_b32_xprep_kernel<false>)) return rc;
-    const dim3 grid((unsigned)rowwgs, (unsigned)nslices, (unsigned)mtiles * (W2 ? 2u : 1u));  // (both matrices of a gated pair in one launch)
     float *partial2 = W2 ? partial + (size_t)nslices * M * N : nullptr;
+    if constexpr (kHasTiles) {
+        if (together) {
+            static const bool tiles_lds_ok = [] {
+                auto room = [](auto kernel, int bytes) {
+                    return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess;
+                };
+                return room(mmq_b32_tiles_kernel<T, 1>, B32TilesOf<1>::kLds) && room(mmq_b32_tiles_kernel<T, 2>, B32TilesOf<2>::kLds) &&
+                       room(mmq_b32_tiles_kernel<T, 3>, B32TilesOf<3>::kLds) && room(mmq_b32_tiles_kernel<T, 4>, B32TilesOf<4>::kLds);
+            }();
+            if (!tiles_lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", B32TilesOf<4>::kLds);
+            const dim3 tgrid((unsigned)rowwgs, (unsigned)nslices, W2 ? 2u : 1u);
+            // (the tiles are dealt evenly over the fewest launches, as for Q4_K)
+            const int nlaunch = (mtiles + Q4KTiles::kMaxTiles - 1) / Q4KTiles::kMaxTiles;
+            for (int l = 0, tile0 = 0; l < nlaunch; l++) {
+                const int ntile = (mtiles - tile0 + (nlaunch - l) - 1) / (nlaunch - l);
+                const int64_t m0 = (int64_t)tile0 * kMT;
+                tile0 += ntile;
+                auto go = [&](auto kernel, int lds) {
+                    return launch(kernel, tgrid, dim3(64 * Q4KTiles::kWaves), (size_t)lds, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N,
+                                  row_bytes, S, (int)m0, W2, partial2);
+                };
+                if (int rc = ntile == 4   ? go(mmq_b32_tiles_kernel<T, 4>, B32TilesOf<4>::kLds)
+                             : ntile == 3 ? go(mmq_b32_tiles_kernel<T, 3>, B32TilesOf<3>::kLds)
+                             : ntile == 2 ? go(mmq_b32_tiles_kernel<T, 2>, B32TilesOf<2>::kLds)
+                                          : go(mmq_b32_tiles_kernel<T, 1>, B32TilesOf<1>::kLds))
+                    return rc;
+            }
+            return launch_mmq_reduce(partial, partial2, xscale, nslices, M, K, N, bias, act, y, ex, s);
+        }
+    }
+    const dim3 grid((unsigned)rowwgs, (unsigned)nslices, (unsigned)mtiles * (W2 ? 2u : 1u));  // (both matrices of a gated pair in one launch)
     if (int rc = launch(mmq_b32_kernel<T, RT>, grid, dim3(RT * 128), lds_bytes, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N, row_bytes, S,
                         mtiles, W2, partial2))
         return rc;

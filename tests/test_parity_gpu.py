@@ -294,6 +294,37 @@ def test_q4_k_split_k_walks_several_batch_tiles_together(gpu, oracle):
     assert gated_case(gpu, oracle, t, 170, 4096, 11008, 3, 1, True, 1540) < 2 * TOL_F32  # (a wide pair of 25 MB each keeps the route past 160 rows, up to 384)
 
 
+@pytest.mark.parametrize("t", [Q4_0, IQ4_NL])
+def test_18_byte_block_formats_walk_several_batch_tiles_together(gpu, oracle, t):
+    """Q4_0 and IQ4_NL at more than 32 batch rows on the split-K route (up to 128 rows): one launch contracts two to four tiles
+    of 32 rows against every parked stretch of weights.  A width that is not a multiple of the workgroup's 256 rows, a last
+    tile that is partly filled, slices of 512 and of 1024 values with a shorter last one, a long-K matrix; fp32 and bf16
+    activations, a projection with normalisation and residual, a gated pair."""
+    q = Quantization(ggml_type=t)
+    # (the kernel serves matrices whose 256-row workgroups times 512-value slices cover three quarters of the CUs)
+    for K, N in ((4096, 6148), (4096 + 768, 5124), (14336, 1796)):
+        W = synth.weights(t, 1600 + t, N, K)
+        bias = synth.normal(1601, 0, N).astype(np.float32) * 0.1
+        x_all = synth.activations(1602 + K, 128, K)
+        want_all = oracle.c_qdense(t, x_all, W, bias, 3)  # (rows are independent: one oracle pass serves every batch size)
+        for M in (33, 64, 70, 97, 128):
+            got = nn.quantized_dense(dev(gpu, np.ascontiguousarray(x_all[128 - M:])), dev(gpu, W), q, dev(gpu, bias), BACKEND_ACT[3]).cpu().numpy()
+            assert rel_err(got, want_all[128 - M:]) < TOL_F32, (ggml.name(t), K, N, M)
+        xb = bf16_round(x_all[:100])
+        assert rel_err(run_dense(gpu, t, xb, W, bias, 0, bf16=True), oracle.c_qdense(t, xb, W, bias, 0)) < TOL_F32, (ggml.name(t), K, N, "bf16")
+    K, N, M = 4096, 6148, 100
+    W = synth.weights(t, 1610 + t, N, K)
+    gain = (synth.normal(1611, 0, K) * 0.5 + 1.0).astype(np.float32)
+    x = (synth.activations(1612, M, K) * 2.0).astype(np.float32)
+    res = synth.activations(1613, M, N)
+    got = nn.quantized_dense(dev(gpu, x), dev(gpu, W), q, None, BACKEND_ACT[0], norm=nn.RMSNorm(dev(gpu, gain), 1e-6, 0.0),
+                             residual=dev(gpu, res)).cpu().numpy()
+    dense = oracle.c_qdense(t, oracle.c_rmsnorm(x, gain, 1e-6, 0.0), W)
+    assert float(np.max(np.abs(got.astype(np.float64) - (dense + res)))) / float(np.max(np.abs(dense))) < TOL_F32, ggml.name(t)
+    assert gated_case(gpu, oracle, t, 100, 4096, 3076, 3, 1, True, 1620) < 2 * TOL_F32
+    assert gated_case(gpu, oracle, t, 70, 2048, 516, 3, 0, False, 1630) < 2 * TOL_F32  # (a small pair: one launch per 32 rows)
+
+
 def test_q4_k_large_minima_through_the_split_k_kernel(gpu, oracle):
     """Q4_K super-blocks whose minimum term is as large as the format allows to matter: dmin = 2048 with every 6-bit minimum at
     63 (dmin * m = 129 024 lies beyond the largest fp16, 65 504, and has 17 significant bits).  The small-batch kernel must
