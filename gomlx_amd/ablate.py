@@ -79,8 +79,8 @@ _Q4K_NO_PARTIAL = """            asm volatile("" ::"v"(v));
 }
 
 // ---- several tiles of 32 batch rows per weight tile"""
-_Q4K_TILES_IMAGE = "        for (int i = wave; i < NT * 8; i += G::kWaves) {\n"
-_Q4K_TILES_NO_IMAGE = "        for (int i = wave; i < (sb == 0 ? NT * 8 : 0); i += G::kWaves) {\n"
+_Q4K_TILES_IMAGE = "    auto stage = [&](int sb, int h) __attribute__((always_inline)) {\n        uint8_t *dst = lds + h * L::kStageBytes;\n        for (int i = wave; i < NT * 8; i += G::kWaves) {\n"
+_Q4K_TILES_NO_IMAGE = "    auto stage = [&](int sb, int h) __attribute__((always_inline)) {\n        uint8_t *dst = lds + h * L::kStageBytes;\n        for (int i = wave; i < (sb == 0 ? NT * 8 : 0); i += G::kWaves) {\n"
 _Q4K_TILES_CONTRACT = "        q4k_tiles_half<NT, 0>(cur, lds, kg, col, magic, p1);\n"
 _Q4K_XPREP = """    if (int rc = x_is_bf16 ? (fine ? prep(mmq_xprep_kernel<true, 1>) : prep(mmq_xprep_kernel<true, 2>))
                            : (fine ? prep(mmq_xprep_kernel<false, 1>) : prep(mmq_xprep_kernel<false, 2>)))
