@@ -1761,12 +1761,12 @@ def test_operator_rejects_bad_arguments(gpu):
     assert gpu.equal(y0, y1)
 
 
-@pytest.mark.parametrize("rows", [1, 3, 24, 300])
+@pytest.mark.parametrize("rows", [1, 3, 24, 100, 300])
 def test_decoder_layer_calls_replay_as_a_graph(gpu, rows):
     """The calls of a decoder layer (q/k/v behind a norm, o + residual, norm + gate/up product, down +
     residual in place) recorded once and replayed four times, with eager work between the replays:
     every replay must reproduce the eager results exactly.  Batch sizes of all three kernel
-    families; one eager pass first creates the workspaces the larger ones need."""
+    families (100 rows: the split-K kernel that walks four tiles of 32 rows); one eager pass first creates the workspaces the larger ones need."""
     import ctypes
     from gomlx_amd import _lib
     torch = gpu
