@@ -204,15 +204,16 @@ int64_t weight_bytes_of(int type, int64_t K, int64_t N) { return (int64_t)gq_row
 // K itself while its tiles are fewer than the CUs.
 // Measured (python -m gomlx_amd.tune.crossover with GOMLX_HIPQ_SPLIT_K_TO=100000 and =16: us per call in a replayed graph of 20
 // calls on rotating weights, fp32 activations; rows 32 64 96 128 160 192; split-K | two passes at the same rows):
-//   Q8_0   4096x4096  16 22 27 29 35 36 | 27 28 29 30 31 31    4096x14336  33 52  71  84 100 118 | 56 56 55 58 69 69    14336x4096  33 52 72 85 104 121 | 63 70 72 73 81 82
+//   Q8_0   4096x4096  16 22 27 29 35 36 | 27 28 29 30 31 31    4096x14336  32 37  43  49  69  76 | 56 56 55 58 69 69    14336x4096  32 38 44 49  70  77 | 63 70 72 73 81 82
 //   Q4_0   4096x4096  15 20 25 26 32 33 | 25 26 26 27 29 29    4096x14336  27 33  40  45  61  67 | 57 55 55 56 67 69    14336x4096  28 34 40 45  62  69 | 62 63 69 68 79 79
 //   Q4_K   4096x4096  15 17 21 29 36 38 | 26 26 27 29 30 30    4096x14336  25 28  34  38  53  57 | 61 59 60 60 73 72    14336x4096  21 30 36 41  55  59 | 69 73 72 71 85 85
 //          (at 256 320 384 rows: 4096x14336 74 96 108 | 74 94 95; 14336x4096 77 99 112 | 87 108 109.  Q4_K walks up to four tiles of 32 batch rows per
 //          launch; with one launch per 32 rows, as the other formats' kernels still work, it took 14 23 32 39 46 52, 27 44 61 79 96 113 and 22 36 49 63 77 92)
 //   Q6_K   4096x4096  19 22 30 32 39 40 | 26 28 29 30 31 32    4096x14336  36 56  76  89 109 130 | 61 57 58 59 70 71    14336x4096  36 56 77 90 111 132 | 68 68 74 74 82 83
 //   IQ4_NL 4096x4096  16 21 28 29 37 37 | 27 28 29 30 31 32    4096x14336  30 36  43  48  66  72 | 63 62 62 64 76 77    14336x4096  31 37 43 48  67  74 | 70 75 78 78 87 88
-//          (Q4_0 and IQ4_NL walk up to four tiles of 32 batch rows per launch on the large matrices, like Q4_K; one launch per 32 rows took
-//          27 42 56 66 80 94 / 28 43 57 68 83 97 and 30 48 65 78 95 112 / 31 49 66 80 97 114; at 256 rows the tiles take 79 - 86 against 70 - 90)
+//          (Q8_0, Q4_0 and IQ4_NL walk up to four tiles of 32 batch rows per launch on the large matrices, like Q4_K; one pass per 32 rows took
+//          33 52 71 84 100 118 / 33 52 72 85 104 121, 27 42 56 66 80 94 / 28 43 57 68 83 97 and 30 48 65 78 95 112 / 31 49 66 80 97 114; at 256
+//          rows the tiles take 79 - 90 against 70 - 90)
 // (Before the GEMM split K on narrow problems the two passes took 33 us on 4096x4096 and 92 .. 102 us on 14336x4096 at these rows.)
 // GOMLX_HIPQ_SPLIT_K_TO=rows overrides the table (tuning runs only).
 int64_t split_k_to_env() {
@@ -223,7 +224,7 @@ int64_t split_k_to(int type, int64_t K, int64_t N) {
     if (split_k_to_env() >= 0) return split_k_to_env();
     const bool large = weight_bytes_of(type, K, N) >= kLargeWeightBytes, long_k = K > N;
     switch (type) {
-    case GQ_Q8_0: return !large ? 128 : long_k ? 96 : 64;
+    case GQ_Q8_0: return !large ? 128 : long_k ? 192 : 160;
     case GQ_Q4_0: return !large ? 128 : 192;
     case GQ_Q4_K: return !large ? 128 : long_k ? 320 : 256;
     case GQ_Q6_K: return !large ? 96 : 64;
@@ -235,7 +236,7 @@ int64_t split_k_to(int type, int64_t K, int64_t N) {
 // The same point for a gated pair act(x.Wgate) * (x.Wup): both matrices are contracted against one activation image by the
 // split-K kernels, or dequantised into one interleaved image for ONE GEMM by the two passes.  Measured (same tool, mode
 // `gated`, SiLU; rows 32 64 96 128 160 192 256; split-K | two passes):
-//   Q8_0   4096x4096  24 35 39 45 52 58 73 | 46 45 46 46 47 46 46    4096x14336  50 79 110 136 165 193 247 | 112 117 123 129 142 145 151
+//   Q8_0   4096x4096  24 35 39 45 52 58 73 | 46 45 46 46 47 46 46    4096x14336  50 60  72  86 122 136 161 | 112 117 123 129 142 145 151
 //   Q4_0   4096x4096  20 27 34 41 47 52 66 | 45 44 44 45 45 45 45    4096x14336  42 53  65  75 107 119 141 | 107 114 121 118 138 133 141
 //   Q4_K   4096x4096  17 22 27 32 44 48 60 | 46 45 45 45 46 46 45    4096x14336  37 46  55  65  92 101 121 | 118 125 131 128 147 142 151
 //          (one launch per 32 rows: 17 28 37 45 53 61 78 and 37 65 93 120 149 178 233; at 320 384 448 rows the large pair takes 173 198 243 | 203 205 209)
@@ -248,7 +249,7 @@ int64_t gated_split_k_to(int type, int64_t K, int64_t N) {
     const bool large = weight_bytes_of(type, K, N) >= kLargeWeightBytes, long_k = K > N;
     if (large && long_k) return split_k_to(type, K, N);
     switch (type) {
-    case GQ_Q8_0: return large ? 96 : 128;
+    case GQ_Q8_0: return large ? 192 : 128;
     case GQ_Q4_0: return large ? 192 : 128;
     case GQ_Q4_K: return large ? 384 : 160;
     case GQ_Q6_K: return large ? 64 : 96;

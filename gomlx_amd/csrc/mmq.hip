@@ -1476,6 +1476,171 @@ __global__ __launch_bounds__(64 * Q4KTiles::kWaves) void mmq_b32_tiles_kernel(co
     }
 }
 
+// ---- Q8_0 at more than 32 batch rows -------------------------------------------------------------------------------
+//
+// The same ring of half images and the same contraction as mmq_b32_tiles_kernel.  A Q8_0 stretch is 272 bytes of a row
+// (8.5 KiB per tile of 32 rows): two parked tiles per wavefront do not fit beside the ring, so a wavefront has ONE park and
+// the next stretch travels through registers, as in mmq_b32_kernel - requested when the stretch before it has been stored to
+// the park, stored when that one has been read out.  Request order per stretch j: stage(j,1), loads(j+1) | stage(j+1,0); the
+// wait in front of the second half leaves the nine register loads of the next stretch in flight.
+template <int NT> struct Q8TilesOf {
+    typedef B32Geom<kQ8_0> G;
+    static constexpr int kStageBytes = NT * Q4KTiles::kHalfBytes;
+    static constexpr int kRingBytes = 2 * kStageBytes;
+    static constexpr int kLds = kRingBytes + Q4KTiles::kWaves * G::kWaveLds;  // (kWaveLds carries the slack for a code window that ends past the last row)
+    static_assert(kLds <= 160 * 1024, "images + parked tiles exceed LDS");
+};
+
+template <int NT>
+__global__ __launch_bounds__(64 * Q4KTiles::kWaves) void mmq_q8_tiles_kernel(const uint8_t *__restrict__ ximg, const uint8_t *__restrict__ W0,
+                                                                              float *__restrict__ partial0, int M, int K, int N, int64_t row_bytes, int S,
+                                                                              int m0, const uint8_t *__restrict__ W2, float *__restrict__ partial2) {
+    typedef B32<kQ8_0> F;
+    typedef B32Geom<kQ8_0> G;
+    typedef Q4KTiles Q;
+    typedef Q8TilesOf<NT> L;
+    static_assert(G::kLoads == 9, "the counted wait below assumes nine load instructions per stretch");
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const uint8_t *__restrict__ W = blockIdx.z ? W2 : W0;
+    float *__restrict__ partial = blockIdx.z ? partial2 : partial0;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kg = lane >> 5, col = lane & 31;
+    const int slice = blockIdx.y, nslices = gridDim.y;
+    const int per_slice = S >> 8, first = slice * per_slice;
+    const int nst = min(per_slice, (K >> 8) - first);  // stretches of this slice (at least one)
+    const int row0 = (int)blockIdx.x * Q::kRows + wave * 32;
+    const int n = row0 + col;  // this lane's weight row
+
+    // chunk c = lane + 64 i of a stretch is chunk c % kCPR of row c / kCPR of the tile (rows past N re-read the last one)
+    uint32_t coff[G::kLoads];
+#pragma unroll
+    for (int i = 0; i < G::kLoads; i++) {
+        const int c = min(lane + 64 * i, G::kChunks - 1);
+        coff[i] = (uint32_t)min(c / G::kCPR, max(N - 1 - row0, 0)) * (uint32_t)row_bytes + (uint32_t)(c % G::kCPR) * 16u;
+    }
+    const uint8_t *wtile = W + (int64_t)min(row0, N - 1) * row_bytes + (int64_t)first * G::kStretchBytes;
+    typedef uint32_t Chunk __attribute__((ext_vector_type(4)));
+    typedef Chunk ChunkA4 __attribute__((aligned(4)));  // (rows are 4-byte aligned in general)
+    Chunk buf[G::kLoads];
+    auto load = [&](int j) __attribute__((always_inline)) {  // stretch j of the slice -> registers: exactly kLoads load instructions
+        const uint8_t *base = wtile + (int64_t)j * G::kStretchBytes;
+#pragma unroll
+        for (int l = 0; l < G::kLoads; l++) buf[l] = *reinterpret_cast<const ChunkA4 *>(base + coff[l]);
+    };
+    uint8_t *const park = lds + L::kRingBytes + wave * G::kWaveLds;
+    const uint8_t *const myrow = park + col * G::kStretchBytes;
+
+    const size_t img_bytes = (size_t)S * 64;
+    const uint8_t *img0 = ximg + ((size_t)(m0 / kMT) * nslices + slice) * img_bytes;
+    const size_t tile_stride = (size_t)nslices * img_bytes;
+    auto stage = [&](int j, int h) __attribute__((always_inline)) {  // half h (four blocks) of stretch j of every tile -> ring stage h
+        uint8_t *dst = lds + h * L::kStageBytes;
+        for (int i = wave; i < NT * 8; i += Q::kWaves) {
+            const int t = i >> 3, ck = i & 7;
+            __builtin_amdgcn_global_load_lds(
+                (const __attribute__((address_space(1))) void *)(img0 + t * tile_stride + j * 16384 + h * Q::kHalfBytes + ck * 1024 + lane * 16),
+                (__attribute__((address_space(3))) void *)(dst + t * Q::kHalfBytes + ck * 1024), 16, 0, 0);
+        }
+    };
+    auto meet = [&](bool all) __attribute__((always_inline)) {  // (see mmq_q4k_tiles_kernel)
+        if (all) __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+        else __builtin_amdgcn_s_waitcnt(0x0F79);       // vmcnt(9)
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
+
+    f16v acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[t][r] = 0.f;
+    uint32_t magic;
+    asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));
+
+    auto half = [&](auto hc) __attribute__((always_inline)) {  // four blocks of the parked stretch against ring stage H (as in mmq_b32_tiles_kernel)
+        constexpr int H = decltype(hc)::value;
+        const uint8_t *img = lds + H * L::kStageBytes;
+#pragma unroll
+        for (int bb = 0; bb < 4; bb++) {
+            const int b = 4 * H + bb;
+            const int at = b * F::kBlockBytes + F::code_byte(kg);
+            const uint32_t *wp = reinterpret_cast<const uint32_t *>(myrow + (at & ~3));
+            uint32_t w[F::kWin], c[F::kWin - 1];
+#pragma unroll
+            for (int q = 0; q < F::kWin; q++) w[q] = wp[q];
+#pragma unroll
+            for (int q = 0; q < F::kWin - 1; q++) c[q] = (b & 1) ? w[q] : __builtin_amdgcn_alignbit(w[q + 1], w[q], 16);
+            const float d = half_bits_to_float(*reinterpret_cast<const uint16_t *>(myrow + b * F::kBlockBytes));
+            const h8 f0 = F::frag(c, 0, magic), f1 = F::frag(c, 1, magic);
+            const int o0 = F::octet(bb, kg, 0), o1 = F::octet(bb, kg, 1);  // octets of the half: 0 .. 15
+#pragma unroll
+            for (int t0 = 0; t0 < NT; t0 += 2) {
+                f16v p[2];
+#pragma unroll
+                for (int u = 0; u < 2; u++) {
+                    const int t = t0 + u;
+                    if (t >= NT) continue;
+                    const h8 x0 = *reinterpret_cast<const h8 *>(img + t * Q::kHalfBytes + (o0 * kMT + col) * 16);
+                    const h8 x1 = *reinterpret_cast<const h8 *>(img + t * Q::kHalfBytes + (o1 * kMT + col) * 16);
+#pragma unroll
+                    for (int r = 0; r < 16; r++) p[u][r] = 0.f;
+                    p[u] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x0, f0, p[u], 0, 0, 0);
+                    p[u] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x1, f1, p[u], 0, 0, 0);
+                }
+#pragma unroll
+                for (int u = 0; u < 2; u++) {
+                    const int t = t0 + u;
+                    if (t >= NT) continue;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[t][r] = fmaf(d, p[u][r], acc[t][r]);
+                    asm volatile("" : "+v"(acc[t]));  // (pinned: see mmq_b32_tiles_kernel)
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+
+    stage(0, 0);
+    asm volatile("" ::: "memory");  // (the counted wait relies on the order of the requests)
+    load(0);
+    for (int j = 0; j < nst; j++) {
+        // first half: its image and this wavefront's stretch (in registers) must be there; every wavefront has finished with stage 1
+        meet(true);
+        stage(j, 1);
+        asm volatile("" ::: "memory");
+        // park the stretch (LDS operations of one wavefront execute in order; no other wavefront reads it)
+#pragma unroll
+        for (int l = 0; l < G::kLoads; l++)
+            if (lane + 64 * l < G::kChunks) *reinterpret_cast<Chunk *>(park + (lane + 64 * l) * 16) = buf[l];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const bool more = j + 1 < nst;
+        if (more) load(j + 1);
+        asm volatile("" ::: "memory");
+        half(std::integral_constant<int, 0>());
+        // second half: the image requested above must be there; the register loads of the next stretch, issued after it, may still be out
+        meet(!more);
+        if (more) stage(j + 1, 0);
+        half(std::integral_constant<int, 1>());
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");  // the reads above are done before the next stretch is parked
+        __builtin_amdgcn_wave_barrier();
+    }
+
+    if (n < N) {
+        // lane holds y[m = 32 t + 8 (r / 4) + 4 kg + r % 4][n] for its K-slice
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = m0 + 32 * t + 8 * (r >> 2) + 4 * kg + (r & 3);
+                if (m < M) partial[((int64_t)slice * M + m) * N + n] = acc[t][r];
+            }
+        }
+    }
+}
+
 template <int T, int RT>
 int launch_mmq_b32(const void *x, bool x_is_bf16, int64_t M, int64_t K, const uint8_t *W, int64_t N, const float *bias, int act, float *y, hipStream_t s,
                    const MmqExtra *ex) {
@@ -1483,8 +1648,9 @@ int launch_mmq_b32(const void *x, bool x_is_bf16, int64_t M, int64_t K, const ui
     const RmsNorm *norm = ex ? ex->norm : nullptr;
     const int cus = device_cu_count();
     const int mtiles = (int)((M + kMT - 1) / kMT);
-    // more than 32 batch rows of an 18-byte-block format: the kernel that walks up to four tiles of 32 rows per launch
-    constexpr bool kHasTiles = B32<T>::kBlockBytes == 18;
+    // more than 32 batch rows: the kernels that walk up to four tiles of 32 rows per launch (Q8_0 has its own, with one parked tile)
+    constexpr bool kHasTiles = true;
+    constexpr bool kDmaTiles = B32<T>::kBlockBytes == 18;
     // (where its 256-row workgroups with the shortest slices still cover three quarters of the CUs: on 4096 x 4096 they are 128, and
     // the kernel below it stays ahead from 128 rows on, 26 against 32 us)
     const bool together = kHasTiles && mtiles >= 2 && tiles_together_mode() != 0 &&
@@ -1525,10 +1691,14 @@ int launch_mmq_b32(const void *x, bool x_is_bf16, int64_t M, int64_t K, const ui
                 auto room = [](auto kernel, int bytes) {
                     return hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess;
                 };
-                return room(mmq_b32_tiles_kernel<T, 1>, B32TilesOf<1>::kLds) && room(mmq_b32_tiles_kernel<T, 2>, B32TilesOf<2>::kLds) &&
-                       room(mmq_b32_tiles_kernel<T, 3>, B32TilesOf<3>::kLds) && room(mmq_b32_tiles_kernel<T, 4>, B32TilesOf<4>::kLds);
+                if constexpr (kDmaTiles)
+                    return room(mmq_b32_tiles_kernel<T, 1>, B32TilesOf<1>::kLds) && room(mmq_b32_tiles_kernel<T, 2>, B32TilesOf<2>::kLds) &&
+                           room(mmq_b32_tiles_kernel<T, 3>, B32TilesOf<3>::kLds) && room(mmq_b32_tiles_kernel<T, 4>, B32TilesOf<4>::kLds);
+                else
+                    return room(mmq_q8_tiles_kernel<1>, Q8TilesOf<1>::kLds) && room(mmq_q8_tiles_kernel<2>, Q8TilesOf<2>::kLds) &&
+                           room(mmq_q8_tiles_kernel<3>, Q8TilesOf<3>::kLds) && room(mmq_q8_tiles_kernel<4>, Q8TilesOf<4>::kLds);
             }();
-            if (!tiles_lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", B32TilesOf<4>::kLds);
+            if (!tiles_lds_ok) return fail(GQ_ERR_HIP, "mmq: cannot reserve %d bytes of LDS", kDmaTiles ? B32TilesOf<4>::kLds : Q8TilesOf<4>::kLds);
             const dim3 tgrid((unsigned)rowwgs, (unsigned)nslices, W2 ? 2u : 1u);
             // (the tiles are dealt evenly over the fewest launches, as for Q4_K)
             const int nlaunch = (mtiles + Q4KTiles::kMaxTiles - 1) / Q4KTiles::kMaxTiles;
@@ -1540,11 +1710,18 @@ int launch_mmq_b32(const void *x, bool x_is_bf16, int64_t M, int64_t K, const ui
                     return launch(kernel, tgrid, dim3(64 * Q4KTiles::kWaves), (size_t)lds, s, (const uint8_t *)ximg, W, partial, (int)M, (int)K, (int)N,
                                   row_bytes, S, (int)m0, W2, partial2);
                 };
-                if (int rc = ntile == 4   ? go(mmq_b32_tiles_kernel<T, 4>, B32TilesOf<4>::kLds)
-                             : ntile == 3 ? go(mmq_b32_tiles_kernel<T, 3>, B32TilesOf<3>::kLds)
-                             : ntile == 2 ? go(mmq_b32_tiles_kernel<T, 2>, B32TilesOf<2>::kLds)
-                                          : go(mmq_b32_tiles_kernel<T, 1>, B32TilesOf<1>::kLds))
-                    return rc;
+                int rc;
+                if constexpr (kDmaTiles)
+                    rc = ntile == 4   ? go(mmq_b32_tiles_kernel<T, 4>, B32TilesOf<4>::kLds)
+                         : ntile == 3 ? go(mmq_b32_tiles_kernel<T, 3>, B32TilesOf<3>::kLds)
+                         : ntile == 2 ? go(mmq_b32_tiles_kernel<T, 2>, B32TilesOf<2>::kLds)
+                                      : go(mmq_b32_tiles_kernel<T, 1>, B32TilesOf<1>::kLds);
+                else
+                    rc = ntile == 4   ? go(mmq_q8_tiles_kernel<4>, Q8TilesOf<4>::kLds)
+                         : ntile == 3 ? go(mmq_q8_tiles_kernel<3>, Q8TilesOf<3>::kLds)
+                         : ntile == 2 ? go(mmq_q8_tiles_kernel<2>, Q8TilesOf<2>::kLds)
+                                      : go(mmq_q8_tiles_kernel<1>, Q8TilesOf<1>::kLds);
+                if (rc) return rc;
             }
             return launch_mmq_reduce(partial, partial2, xscale, nslices, M, K, N, bias, act, y, ex, s);
         }

@@ -294,10 +294,10 @@ def test_q4_k_split_k_walks_several_batch_tiles_together(gpu, oracle):
     assert gated_case(gpu, oracle, t, 170, 4096, 11008, 3, 1, True, 1540) < 2 * TOL_F32  # (a wide pair of 25 MB each keeps the route past 160 rows, up to 384)
 
 
-@pytest.mark.parametrize("t", [Q4_0, IQ4_NL])
-def test_18_byte_block_formats_walk_several_batch_tiles_together(gpu, oracle, t):
-    """Q4_0 and IQ4_NL at more than 32 batch rows on the split-K route (up to 128 rows): one launch contracts two to four tiles
-    of 32 rows against every parked stretch of weights.  A width that is not a multiple of the workgroup's 256 rows, a last
+@pytest.mark.parametrize("t", [Q4_0, IQ4_NL, Q8_0])
+def test_32_value_block_formats_walk_several_batch_tiles_together(gpu, oracle, t):
+    """Q4_0, IQ4_NL and Q8_0 at more than 32 batch rows on the split-K route (up to 128 rows and more): one launch contracts two
+    to four tiles of 32 rows against every parked stretch of weights (Q8_0: one parked stretch, the next one through registers).  A width that is not a multiple of the workgroup's 256 rows, a last
     tile that is partly filled, slices of 512 and of 1024 values with a shorter last one, a long-K matrix; fp32 and bf16
     activations, a projection with normalisation and residual, a gated pair."""
     q = Quantization(ggml_type=t)
