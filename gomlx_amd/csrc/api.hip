@@ -224,7 +224,7 @@ int64_t split_k_to(int type, int64_t K, int64_t N) {
     if (split_k_to_env() >= 0) return split_k_to_env();
     const bool large = weight_bytes_of(type, K, N) >= kLargeWeightBytes, long_k = K > N;
     switch (type) {
-    case GQ_Q8_0: return !large ? 128 : long_k ? 192 : 160;
+    case GQ_Q8_0: return !large ? 128 : long_k ? 192 : 128;  // (4096x6144, 27 MB: 34 46 | 34 39 at 128 and 160 rows)
     case GQ_Q4_0: return !large ? 128 : 192;
     case GQ_Q4_K: return !large ? 128 : long_k ? 320 : 256;
     case GQ_Q6_K: return !large ? 96 : 64;
